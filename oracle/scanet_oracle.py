@@ -1,0 +1,869 @@
+"""CPU oracle for scanet's compiled training/inference step (TEST INFRASTRUCTURE ONLY).
+
+This module is a numpy restatement, op for op and in the reference's evaluation
+order, of the graph that scanet3 lowers to TensorFlow for one training step:
+layers, losses, hand-derived backward passes that follow the reference's
+``localGrad`` rules, the eight optimizer algorithms, the per-partition step
+loop and the parameter averaging.  It is the checker for the HIP library and
+nothing else: only tests, the smoke entry and the benchmark's CPU-baseline leg
+import it.  The shipped package never does.
+
+Every function works in the dtype of its inputs (float32 on the hot path,
+float64 when a test wants a high-precision check of the mathematics).
+
+What pins each part (see tests/test_oracle_golden.py):
+  * dense / bias / sigmoid forward, BinaryCrossentropy gradients ... reference goldens
+  * softmax rows, tanh, relu, exp, log, sigmoid points ........... reference goldens
+  * conv2d (same/valid/explicit, stride 1/2), both conv grads ..... reference goldens + brute force + torch
+  * max pool (same/valid, stride 1/2), max-pool grad with ties .... reference goldens + brute force
+  * SimpleRNN and LSTM forward ................................... reference goldens
+  * LSTM / conv / pool / softmax+CCE backward .................... float64 numerical gradients + torch autograd
+  * decayingAvg / boost / sqrtZeroSafe ........................... reference goldens
+  * optimizer trajectories ....................................... reference convergence thresholds + closed forms
+Parity unpinned (only running TensorFlow-CPU could pin them): last-ulp
+behaviour of TF's Exp/Tanh/Sigmoid/Log/Pow, summation order inside TF's
+MatMul/Conv2D/Sum, averaging of more than one replica and the multi-partition
+iteration counter (no reference test runs with more than one partition).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+F32 = np.float32
+
+# --------------------------------------------------------------------------- #
+# scalar helpers (src/main/scala/scanet/math/alg/AllKernels.scala:491-549)
+# --------------------------------------------------------------------------- #
+
+
+def _c(x, like):
+    """A constant cast to the dtype of `like` (reference: `x.const.cast[T]`)."""
+    return np.asarray(like).dtype.type(x)
+
+
+def pow_scalar(base, exponent, dtype=F32):
+    """`Pow(rate, iter.cast[Float])` on scalars, rounded once to `dtype`.
+
+    AllKernels.scala:546-549 (`boost`).  Evaluated in float64 and rounded, which
+    is the correctly rounded float32 power.
+    """
+    return np.dtype(dtype).type(float(np.dtype(dtype).type(base)) ** float(exponent))
+
+
+def sqr(x):
+    """`sqr = Pow(x, 2)` (AllKernels.scala:648); x*x is the correctly rounded value."""
+    return x * x
+
+
+def decaying_avg(avg, nxt, decay):
+    """`decay * avg + (1 - decay) * next` (AllKernels.scala:541-544)."""
+    d = _c(decay, avg)
+    one = _c(1.0, avg)
+    return d * avg + (one - d) * nxt
+
+
+def boost(x, rate, it):
+    """`x / (1 - rate^iter)` (AllKernels.scala:546-549)."""
+    dt = np.asarray(x).dtype
+    return x / (dt.type(1.0) - pow_scalar(rate, it, dt))
+
+
+def sqrt_zero_safe(x, eps):
+    """`sqrt(x + eps)` (AllKernels.scala:491-492)."""
+    return np.sqrt(x + _c(eps, x))
+
+
+def rint(x):
+    """TF `Rint`: round half to even (AllKernels.scala:339-345)."""
+    return np.rint(x)
+
+
+# --------------------------------------------------------------------------- #
+# activations (models/Activation.scala:32-83; grads math/alg/AllKernels.scala)
+# --------------------------------------------------------------------------- #
+
+
+def sigmoid(x):
+    one = _c(1.0, x)
+    return one / (one + np.exp(-x))
+
+
+def sigmoid_grad(x, dy):
+    """AllKernels.scala:397-404: recomputes s, grad = s*(1-s), then * parent."""
+    s = sigmoid(x)
+    return (s * (_c(1.0, x) - s)) * dy
+
+
+def tanh_grad(x, dy):
+    """AllKernels.scala:414-420: (1 - tanh(x)^2) * parent."""
+    return (_c(1.0, x) - sqr(np.tanh(x))) * dy
+
+
+def relu(x, threshold=0.0):
+    """Activation.scala:79-82: Maximum(threshold, x)."""
+    return np.maximum(_c(threshold, x), x)
+
+
+def relu_grad(x, dy, threshold=0.0):
+    """Maximum's grad to its right input: (left < right) strict (AllKernels.scala:297-302)."""
+    return (_c(threshold, x) < x).astype(x.dtype) * dy
+
+
+def softmax(x):
+    """Activation.scala:63-69: e = exp(x); e / sum(e, axis 1).  No max subtraction."""
+    e = np.exp(x)
+    s = e.sum(axis=1, dtype=x.dtype)
+    return e / s[:, None]
+
+
+def softmax_grad(x, dp):
+    """Chain of Div / Sum / Exp local gradients (AllKernels.scala:196-201,214-227,237-244)."""
+    e = np.exp(x)
+    s = e.sum(axis=1, dtype=x.dtype)[:, None]
+    de_div = dp / s
+    ds = ((-e * dp) / sqr(s)).sum(axis=1, dtype=x.dtype)[:, None]
+    de = de_div + ds            # Sum's grad broadcasts ds over the row
+    return e * de
+
+
+ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = 0, 1, 2, 3, 4
+
+
+def activate(kind, x, param=0.0):
+    if kind == ACT_IDENTITY:
+        return x
+    if kind == ACT_SIGMOID:
+        return sigmoid(x)
+    if kind == ACT_TANH:
+        return np.tanh(x)
+    if kind == ACT_RELU:
+        return relu(x, param)
+    if kind == ACT_SOFTMAX:
+        return softmax(x)
+    raise ValueError(f"unknown activation {kind}")
+
+
+def activate_grad(kind, x, dy, param=0.0):
+    if kind == ACT_IDENTITY:
+        return dy
+    if kind == ACT_SIGMOID:
+        return sigmoid_grad(x, dy)
+    if kind == ACT_TANH:
+        return tanh_grad(x, dy)
+    if kind == ACT_RELU:
+        return relu_grad(x, dy, param)
+    if kind == ACT_SOFTMAX:
+        return softmax_grad(x, dy)
+    raise ValueError(f"unknown activation {kind}")
+
+
+# --------------------------------------------------------------------------- #
+# losses (models/Loss.scala:18-57)
+# --------------------------------------------------------------------------- #
+
+LOSS_IDENTITY, LOSS_MSE, LOSS_BCE, LOSS_CCE = 0, 1, 2, 3
+
+
+def loss_value(kind, p, y):
+    dt = p.dtype
+    if kind == LOSS_IDENTITY:
+        return p
+    if kind == LOSS_MSE:                      # Loss.scala:18-24
+        return sqr(p - y).mean(dtype=dt)
+    if kind == LOSS_BCE:                      # Loss.scala:26-42
+        one, eps = dt.type(1.0), dt.type(1e-8)
+        left = y * np.log(p + eps)
+        right = (one - y) * np.log(one - (p - eps))
+        return (-left - right).mean(dtype=dt)
+    if kind == LOSS_CCE:                      # Loss.scala:44-57
+        eps = dt.type(1e-8)
+        num = dt.type(y.shape[0])
+        return -((y * np.log(p + eps)).sum(dtype=dt)) / num
+    raise ValueError(f"unknown loss {kind}")
+
+
+def loss_grad(kind, p, y):
+    """d loss / d predicted, following the reference's localGrad chain."""
+    dt = p.dtype
+    if kind == LOSS_MSE:
+        # Mean: ones/size ; Pow: (d^(2-1) * 2) * parent ; Minus: +parent
+        size = dt.type(p.size)
+        g = np.ones_like(p) * dt.type(1.0) / size
+        d = p - y
+        return (d * dt.type(2.0)) * g
+    if kind == LOSS_BCE:
+        one, eps = dt.type(1.0), dt.type(1e-8)
+        size = dt.type(p.size)
+        g = np.ones_like(p) * dt.type(1.0) / size
+        # (left.negate - right): d left = -g ; d right = -g
+        # left = y * log(p+eps): d log = y * (-g); d p = that / (p+eps)
+        dp_left = (y * (-g)) / (p + eps)
+        # right = (1-y) * log(1 - (p-eps)): d log = (1-y)*(-g); d(1-(p-eps)) = that/(1-(p-eps)); d p = -that
+        dp_right = -(((one - y) * (-g)) / (one - (p - eps)))
+        return dp_left + dp_right
+    if kind == LOSS_CCE:
+        eps = dt.type(1e-8)
+        num = dt.type(y.shape[0])
+        g = -(dt.type(1.0) / num)             # Div then Negate
+        return (y * g) / (p + eps)
+    raise ValueError(f"no gradient for loss {kind}")
+
+
+# --------------------------------------------------------------------------- #
+# convolution / pooling (math/nn/AllKernels.scala)
+# --------------------------------------------------------------------------- #
+
+PAD_VALID, PAD_SAME, PAD_EXPLICIT = 0, 1, 2
+
+
+def out_size(padding, inp, window, stride, explicit=(0, 0)):
+    """Padding.size (nn/AllKernels.scala:39-89)."""
+    if padding == PAD_SAME:
+        return int(math.ceil(inp / stride))
+    if padding == PAD_VALID:
+        return int(math.ceil((inp - window + 1) / stride))
+    return int(math.ceil((inp + explicit[0] + explicit[1] - window) / stride)) + 1
+
+
+def pads_for(padding, inp, window, stride, explicit=(0, 0)):
+    """(before, after) zero padding TensorFlow applies along one spatial axis."""
+    if padding == PAD_VALID:
+        return 0, 0
+    if padding == PAD_EXPLICIT:
+        return explicit
+    out = out_size(PAD_SAME, inp, window, stride)
+    total = max((out - 1) * stride + window - inp, 0)
+    return total // 2, total - total // 2
+
+
+def _geometry(xshape, kh, kw, strides, padding, explicit):
+    n, h, w, c = xshape
+    sh, sw = strides
+    eh, ew = (explicit[0], explicit[1]), (explicit[2], explicit[3])
+    ho = out_size(padding, h, kh, sh, eh)
+    wo = out_size(padding, w, kw, sw, ew)
+    pt, pb = pads_for(padding, h, kh, sh, eh)
+    pl, pr = pads_for(padding, w, kw, sw, ew)
+    # make the padded plane large enough for every window that is read
+    need_h = (ho - 1) * sh + kh
+    need_w = (wo - 1) * sw + kw
+    pb = max(pb, need_h - h - pt)
+    pr = max(pr, need_w - w - pl)
+    return ho, wo, pt, pb, pl, pr
+
+
+def _patches(xp, kh, kw, sh, sw, ho, wo):
+    """[N, Ho, Wo, kh, kw, C] view-copy of the sliding windows of a padded input."""
+    win = np.lib.stride_tricks.sliding_window_view(xp, (kh, kw), axis=(1, 2))
+    win = win[:, ::sh, ::sw][:, :ho, :wo]           # [N, Ho, Wo, C, kh, kw]
+    return win.transpose(0, 1, 2, 4, 5, 3)
+
+
+def conv2d(x, w, strides=(1, 1), padding=PAD_VALID, explicit=(0, 0, 0, 0)):
+    """TF `Conv2D`, NHWC, filter [kh, kw, Cin, Cout], cross-correlation (nn/AllKernels.scala:143-209)."""
+    kh, kw, cin, cout = w.shape
+    ho, wo, pt, pb, pl, pr = _geometry(x.shape, kh, kw, strides, padding, explicit)
+    xp = np.pad(x, ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+    p = _patches(xp, kh, kw, strides[0], strides[1], ho, wo)
+    out = p.reshape(-1, kh * kw * cin) @ w.reshape(kh * kw * cin, cout)
+    return out.reshape(x.shape[0], ho, wo, cout)
+
+
+def conv2d_grad_filter(x, wshape, dy, strides=(1, 1), padding=PAD_VALID, explicit=(0, 0, 0, 0)):
+    """TF `Conv2DBackpropFilter` (nn/AllKernels.scala:211-235)."""
+    kh, kw, cin, cout = wshape
+    ho, wo, pt, pb, pl, pr = _geometry(x.shape, kh, kw, strides, padding, explicit)
+    xp = np.pad(x, ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+    p = _patches(xp, kh, kw, strides[0], strides[1], ho, wo)
+    g = p.reshape(-1, kh * kw * cin).T @ dy.reshape(-1, cout)
+    return g.reshape(kh, kw, cin, cout)
+
+
+def conv2d_grad_input(xshape, w, dy, strides=(1, 1), padding=PAD_VALID, explicit=(0, 0, 0, 0)):
+    """TF `Conv2DBackpropInput` (nn/AllKernels.scala:237-261)."""
+    kh, kw, cin, cout = w.shape
+    n, h, wd, _ = xshape
+    sh, sw = strides
+    ho, wo, pt, pb, pl, pr = _geometry(xshape, kh, kw, strides, padding, explicit)
+    dp = dy.reshape(-1, cout) @ w.reshape(kh * kw * cin, cout).T
+    dp = dp.reshape(n, ho, wo, kh, kw, cin)
+    dxp = np.zeros((n, h + pt + pb, wd + pl + pr, cin), dtype=dy.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            dxp[:, r:r + sh * ho:sh, q:q + sw * wo:sw, :] += dp[:, :, :, r, q, :]
+    return dxp[:, pt:pt + h, pl:pl + wd, :]
+
+
+def max_pool(x, window=(2, 2), strides=(1, 1), padding=PAD_VALID, return_arg=False):
+    """TF `MaxPoolV2`, NHWC (nn/AllKernels.scala:270-303). Padding cells never win."""
+    kh, kw = window
+    ho, wo, pt, pb, pl, pr = _geometry(x.shape, kh, kw, strides, padding, (0, 0, 0, 0))
+    xp = np.pad(x, ((0, 0), (pt, pb), (pl, pr), (0, 0)), constant_values=-np.inf)
+    p = _patches(xp, kh, kw, strides[0], strides[1], ho, wo)       # [N,Ho,Wo,kh,kw,C]
+    flat = p.reshape(p.shape[0], ho, wo, kh * kw, p.shape[-1])
+    arg = flat.argmax(axis=3)                                      # first max, row-major window order
+    out = np.take_along_axis(flat, arg[:, :, :, None, :], axis=3)[:, :, :, 0, :]
+    if return_arg:
+        return out, arg
+    return out
+
+
+def max_pool_grad(x, dy, window=(2, 2), strides=(1, 1), padding=PAD_VALID):
+    """TF `MaxPoolGradV2`: each window's gradient goes to its first maximum (nn/AllKernels.scala:305-324)."""
+    kh, kw = window
+    sh, sw = strides
+    n, h, wd, c = x.shape
+    ho, wo, pt, pb, pl, pr = _geometry(x.shape, kh, kw, strides, padding, (0, 0, 0, 0))
+    _, arg = max_pool(x, window, strides, padding, return_arg=True)
+    dxp = np.zeros((n, h + pt + pb, wd + pl + pr, c), dtype=dy.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            dxp[:, r:r + sh * ho:sh, q:q + sw * wo:sw, :] += dy * (arg == r * kw + q)
+    return dxp[:, pt:pt + h, pl:pl + wd, :]
+
+
+# --------------------------------------------------------------------------- #
+# layers (models/layer/*.scala) -- the flattened `Composed` list
+# --------------------------------------------------------------------------- #
+
+REG_NONE, REG_L1, REG_L2 = 0, 1, 2
+
+
+@dataclass
+class Layer:
+    """One entry of the flattened layer list of `Composed` (layer/Composed.scala:89-99)."""
+    kind: str                       # dense | bias | activate | flatten | conv2d | pool2d | lstm | simple_rnn
+    units: int = 0
+    activation: int = ACT_IDENTITY
+    act_param: float = 0.0
+    kernel: Tuple[int, int] = (3, 3)
+    strides: Tuple[int, int] = (1, 1)
+    padding: int = PAD_VALID
+    reg: int = REG_NONE
+    reg_lambda: float = 0.0
+    bias: bool = True               # lstm / simple_rnn only
+    rnn_activation: int = ACT_TANH  # simple_rnn cell activation / lstm `activation`
+
+    # ---- parameter definitions, in flat-buffer order ---------------------- #
+    def params(self, in_shape) -> List[Tuple[str, Tuple[int, ...]]]:
+        if self.kind == "dense":        # Dense.scala:50-55
+            return [("weights", (in_shape[1], self.units))]
+        if self.kind == "bias":         # Bias.scala:29-30
+            return [("weights", (self.units,))]
+        if self.kind == "conv2d":       # Conv2D.scala:84-90
+            return [("weights", (self.kernel[0], self.kernel[1], in_shape[3], self.units))]
+        if self.kind == "lstm":         # RNN.scala:285-305 (gate order forget,input,gate,output)
+            f, h = in_shape[2], self.units
+            out = []
+            for gate in ("forget", "input", "gate", "output"):
+                out.append((f"{gate}/0/kernel_weights", (f, h)))
+                out.append((f"{gate}/0/recurrent_weights", (h, h)))
+                if self.bias:
+                    out.append((f"{gate}/1/weights", (h,)))
+            return out
+        if self.kind == "simple_rnn":   # RNN.scala:170-206
+            f, h = in_shape[2], self.units
+            out = [("0/kernel_weights", (f, h)), ("0/recurrent_weights", (h, h))]
+            if self.bias:
+                out.append(("1/weights", (h,)))
+            return out
+        return []
+
+    def out_shape(self, s):
+        if self.kind == "dense":
+            return (s[0], self.units)
+        if self.kind in ("bias", "activate"):
+            return tuple(s)
+        if self.kind == "flatten":      # Flatten.scala:12-18
+            return (s[0], int(np.prod(s[1:])))
+        if self.kind == "conv2d":
+            return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0]),
+                    out_size(self.padding, s[2], self.kernel[1], self.strides[1]), self.units)
+        if self.kind == "pool2d":
+            return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0]),
+                    out_size(self.padding, s[2], self.kernel[1], self.strides[1]), s[3])
+        if self.kind in ("lstm", "simple_rnn"):
+            return (s[0], self.units)
+        raise ValueError(self.kind)
+
+
+def Dense(units, activation=ACT_IDENTITY, act_param=0.0, reg=REG_NONE, reg_lambda=0.0, bias=True):
+    """`Dense(..)` expands to Dense ?>> Bias ?>> Activate (Dense.scala:30-40)."""
+    out = [Layer("dense", units=units, reg=reg, reg_lambda=reg_lambda)]
+    if bias:
+        out.append(Layer("bias", units=units, reg=reg, reg_lambda=reg_lambda))
+    if activation != ACT_IDENTITY:
+        out.append(Layer("activate", activation=activation, act_param=act_param))
+    return out
+
+
+def Conv2D(filters, kernel=(3, 3), strides=(1, 1), padding=PAD_VALID, activation=ACT_IDENTITY,
+           act_param=0.0, bias=False):
+    """Conv2D.scala:54-68: defaults Valid, stride 1, no bias."""
+    out = [Layer("conv2d", units=filters, kernel=kernel, strides=strides, padding=padding)]
+    if bias:
+        out.append(Layer("bias", units=filters))
+    if activation != ACT_IDENTITY:
+        out.append(Layer("activate", activation=activation, act_param=act_param))
+    return out
+
+
+def Pool2D(window=(2, 2), strides=(1, 1), padding=PAD_VALID):
+    """Pool2D.scala:28-42: the layer always max-pools."""
+    return [Layer("pool2d", kernel=window, strides=strides, padding=padding)]
+
+
+def Flatten():
+    return [Layer("flatten")]
+
+
+def LSTM(units, bias=True):
+    return [Layer("lstm", units=units, bias=bias)]
+
+
+def SimpleRNN(units, activation=ACT_TANH, bias=True):
+    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation)]
+
+
+class Model:
+    """A `Composed` model: flattened layers, index-prefixed parameter paths (Composed.scala:22-31)."""
+
+    def __init__(self, layers: Sequence, loss: int = LOSS_MSE):
+        flat: List[Layer] = []
+        for l in layers:
+            flat.extend(l if isinstance(l, (list, tuple)) else [l])
+        self.layers = flat
+        self.loss = loss
+
+    def _prefix(self, idx):
+        return "" if len(self.layers) == 1 else f"{idx}/"
+
+    def param_defs(self, in_shape) -> List[Tuple[str, Tuple[int, ...]]]:
+        out, s = [], tuple(in_shape)
+        for i, l in enumerate(self.layers):
+            for name, shape in l.params(s):
+                out.append((self._prefix(i) + name, shape))
+            s = l.out_shape(s)
+        return out
+
+    def out_shape(self, in_shape):
+        s = tuple(in_shape)
+        for l in self.layers:
+            s = l.out_shape(s)
+        return s
+
+    # ---- forward ---------------------------------------------------------- #
+    def forward(self, x, params: Dict[str, np.ndarray], cache: Optional[list] = None):
+        for i, l in enumerate(self.layers):
+            pre = self._prefix(i)
+            k = l.kind
+            if k == "dense":
+                w = params[pre + "weights"]
+                y = x @ w                                     # Dense.scala:57-61
+                c = (x, w)
+            elif k == "bias":
+                y = x + params[pre + "weights"]               # Bias.scala:32-33
+                c = None
+            elif k == "activate":
+                y = activate(l.activation, x, l.act_param)
+                c = x
+            elif k == "flatten":
+                y = x.reshape(x.shape[0], -1)
+                c = x.shape
+            elif k == "conv2d":
+                w = params[pre + "weights"]
+                y = conv2d(x, w, l.strides, l.padding)
+                c = (x, w)
+            elif k == "pool2d":
+                y = max_pool(x, l.kernel, l.strides, l.padding)
+                c = x
+            elif k == "lstm":
+                y, c = lstm_forward(x, params, pre, l)
+            elif k == "simple_rnn":
+                y, c = simple_rnn_forward(x, params, pre, l)
+            else:
+                raise ValueError(k)
+            if cache is not None:
+                cache.append(c)
+            x = y
+        return x
+
+    # ---- penalty (Regularization.scala:30-44; Composed.scala:66-75) -------- #
+    def penalty(self, params):
+        dt = next(iter(params.values())).dtype if params else np.dtype(F32)
+        total = dt.type(0.0)
+        for i, l in enumerate(self.layers):
+            if l.kind in ("dense", "bias") and l.reg != REG_NONE:
+                w = params[self._prefix(i) + "weights"]
+                if l.reg == REG_L2:
+                    total = total + dt.type(l.reg_lambda) * sqr(w).sum(dtype=dt) / dt.type(2.0)
+                else:
+                    total = total + dt.type(l.reg_lambda) * np.abs(w).sum(dtype=dt) / dt.type(2.0)
+        return total
+
+    def loss_of(self, x, y, params):
+        """LossModel.buildStateful (Model.scala:92-99): loss(model(x), y) + penalty."""
+        p = self.forward(x, params)
+        return loss_value(self.loss, p, y) + self.penalty(params)
+
+    # ---- backward: gradients w.r.t. every weight -------------------------- #
+    def grad(self, x, y, params):
+        """LossModel.grad (Model.scala:107-119): returns (loss, {path: gradient})."""
+        cache: list = []
+        p = self.forward(x, params, cache)
+        loss = loss_value(self.loss, p, y) + self.penalty(params)
+        dy = np.ones_like(p) if self.loss == LOSS_IDENTITY else loss_grad(self.loss, p, y)
+        grads: Dict[str, np.ndarray] = {}
+        for i in range(len(self.layers) - 1, -1, -1):
+            l, c, pre = self.layers[i], cache[i], self._prefix(i)
+            k = l.kind
+            if k == "dense":
+                xi, w = c
+                grads[pre + "weights"] = xi.T @ dy            # AllKernels.scala:382-388
+                dy = dy @ w.T
+            elif k == "bias":
+                axes = tuple(range(dy.ndim - 1))
+                grads[pre + "weights"] = dy.sum(axis=axes, dtype=dy.dtype)   # Plus grad: Sum over broadcast axes
+            elif k == "activate":
+                dy = activate_grad(l.activation, c, dy, l.act_param)
+            elif k == "flatten":
+                dy = dy.reshape(c)
+            elif k == "conv2d":
+                xi, w = c
+                grads[pre + "weights"] = conv2d_grad_filter(xi, w.shape, dy, l.strides, l.padding)
+                dy = conv2d_grad_input(xi.shape, w, dy, l.strides, l.padding) if i > 0 else None
+            elif k == "pool2d":
+                dy = max_pool_grad(c, dy, l.kernel, l.strides, l.padding)
+            elif k == "lstm":
+                dy = lstm_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
+            elif k == "simple_rnn":
+                dy = simple_rnn_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
+            if l.kind in ("dense", "bias") and l.reg != REG_NONE:
+                w = params[pre + "weights"]
+                lam = w.dtype.type(l.reg_lambda)
+                if l.reg == REG_L2:       # d/dw lambda * sum(w^2) / 2 through Pow's grad: (w^1 * 2) * (lambda/2)
+                    grads[pre + "weights"] = grads[pre + "weights"] + (w * w.dtype.type(2.0)) * (lam / w.dtype.type(2.0))
+                else:                     # Abs grad in the reference is |parent| (AllKernels.scala:330-335)
+                    grads[pre + "weights"] = grads[pre + "weights"] + np.abs(np.ones_like(w) * (lam / w.dtype.type(2.0)))
+        return loss, grads
+
+
+# --------------------------------------------------------------------------- #
+# recurrent layers (models/layer/RNN.scala)
+# --------------------------------------------------------------------------- #
+
+GATES = ("forget", "input", "gate", "output")
+
+
+def lstm_forward(x, params, pre, l: Layer):
+    """RNN.build + LSTMCell.build (RNN.scala:40-72, 320-338); returns the last hidden state."""
+    b, t_steps, _ = x.shape
+    h_units = l.units
+    dt = x.dtype
+    c = np.zeros((b, h_units), dt)
+    h = np.zeros((b, h_units), dt)
+    steps = []
+    for t in range(t_steps):
+        xt = x[:, t, :]
+        z = {}
+        for gate in GATES:
+            zz = (xt @ params[f"{pre}{gate}/0/kernel_weights"]) + (h @ params[f"{pre}{gate}/0/recurrent_weights"])
+            if l.bias:
+                zz = zz + params[f"{pre}{gate}/1/weights"]
+            z[gate] = zz
+        f = sigmoid(z["forget"])
+        i = sigmoid(z["input"])
+        g = activate(l.rnn_activation, z["gate"])
+        o = sigmoid(z["output"])
+        c_new = c * f + i * g                     # RNN.scala:336
+        h_new = o * activate(l.rnn_activation, c_new)   # RNN.scala:337
+        steps.append((xt, h, c, z, f, i, g, o, c_new))
+        c, h = c_new, h_new
+    return h, (x.shape, steps)
+
+
+def lstm_backward(dh_last, cache, params, pre, l: Layer, grads, need_dx=False):
+    xshape, steps = cache
+    dt = dh_last.dtype
+    b = xshape[0]
+    dh = dh_last
+    dc = np.zeros_like(dh_last)
+    acc = {}
+    dx = np.zeros(xshape, dt) if need_dx else None
+    for t in range(len(steps) - 1, -1, -1):
+        xt, h_prev, c_prev, z, f, i, g, o, c_new = steps[t]
+        a = activate(l.rnn_activation, c_new)
+        do = dh * a
+        dc = dc + activate_grad(l.rnn_activation, c_new, dh * o)
+        df = dc * c_prev
+        di = dc * g
+        dg = dc * i
+        dc_prev = dc * f
+        dz = {
+            "forget": sigmoid_grad(z["forget"], df),
+            "input": sigmoid_grad(z["input"], di),
+            "gate": activate_grad(l.rnn_activation, z["gate"], dg),
+            "output": sigmoid_grad(z["output"], do),
+        }
+        dh_prev = np.zeros_like(dh)
+        for gate in GATES:
+            kk, rr, bb = f"{pre}{gate}/0/kernel_weights", f"{pre}{gate}/0/recurrent_weights", f"{pre}{gate}/1/weights"
+            acc[kk] = acc.get(kk, 0) + xt.T @ dz[gate]
+            acc[rr] = acc.get(rr, 0) + h_prev.T @ dz[gate]
+            if l.bias:
+                acc[bb] = acc.get(bb, 0) + dz[gate].sum(axis=0, dtype=dt)
+            dh_prev = dh_prev + dz[gate] @ params[rr].T
+            if need_dx:
+                dx[:, t, :] += dz[gate] @ params[kk].T
+        dh, dc = dh_prev, dc_prev
+    grads.update(acc)
+    return dx
+
+
+def simple_rnn_forward(x, params, pre, l: Layer):
+    """RNN over `SimpleRNNCell ?>> Bias ?>> act` (RNN.scala:170-206).
+
+    The cell's carried state is its own pre-bias, pre-activation output
+    (`Params(State -> result)`, RNN.scala:195-196)."""
+    b, t_steps, _ = x.shape
+    dt = x.dtype
+    wk, wr = params[pre + "0/kernel_weights"], params[pre + "0/recurrent_weights"]
+    s = np.zeros((b, l.units), dt)
+    steps = []
+    out = None
+    for t in range(t_steps):
+        xt = x[:, t, :]
+        r = (xt @ wk) + (s @ wr)
+        zz = r + params[pre + "1/weights"] if l.bias else r
+        out = activate(l.rnn_activation, zz)
+        steps.append((xt, s, zz))
+        s = r
+    return out, (x.shape, steps)
+
+
+def simple_rnn_backward(dout, cache, params, pre, l: Layer, grads, need_dx=False):
+    xshape, steps = cache
+    dt = dout.dtype
+    wk, wr = params[pre + "0/kernel_weights"], params[pre + "0/recurrent_weights"]
+    dx = np.zeros(xshape, dt) if need_dx else None
+    gk = np.zeros_like(wk)
+    gr = np.zeros_like(wr)
+    gb = np.zeros((l.units,), dt)
+    # only the last step's output feeds the loss; earlier steps act through the state
+    t_last = len(steps) - 1
+    xt, s_prev, zz = steps[t_last]
+    dz = activate_grad(l.rnn_activation, zz, dout)
+    gb += dz.sum(axis=0, dtype=dt)
+    dr = dz
+    for t in range(t_last, -1, -1):
+        xt, s_prev, _ = steps[t]
+        gk += xt.T @ dr
+        gr += s_prev.T @ dr
+        if need_dx:
+            dx[:, t, :] = dr @ wk.T
+        dr = dr @ wr.T
+    grads[pre + "0/kernel_weights"] = gk
+    grads[pre + "0/recurrent_weights"] = gr
+    if l.bias:
+        grads[pre + "1/weights"] = gb
+    return dx
+
+
+# --------------------------------------------------------------------------- #
+# optimizer algorithms (optimizers/*.scala)
+# --------------------------------------------------------------------------- #
+
+OPT_SGD, OPT_ADAGRAD, OPT_ADADELTA, OPT_RMSPROP, OPT_ADAM, OPT_NADAM, OPT_ADAMAX, OPT_AMSGRAD = range(8)
+
+
+@dataclass
+class Algorithm:
+    kind: int
+    rate: float = 0.001
+    beta1: float = 0.9          # momentum (SGD) / rho (AdaDelta, RMSProp) / beta1
+    beta2: float = 0.999
+    epsilon: float = 1e-7
+    init_acc: float = 0.0
+    nesterov: bool = False
+
+    @property
+    def state_names(self) -> List[str]:
+        return {
+            OPT_SGD: ["velocity"], OPT_ADAGRAD: ["grad_acc"], OPT_ADADELTA: ["avg_grad", "avg_delta"],
+            OPT_RMSPROP: ["avg_grad"], OPT_ADAM: ["momentum", "velocity"], OPT_NADAM: ["momentum", "velocity"],
+            OPT_ADAMAX: ["momentum_1", "momentum_2"], OPT_AMSGRAD: ["momentum", "velocity", "corrected_velocity"],
+        }[self.kind]
+
+    def init_state(self, shape, dtype=F32) -> List[np.ndarray]:
+        return [np.full(shape, self.init_acc, dtype) for _ in self.state_names]
+
+    def build(self, g, state: List[np.ndarray], it: int):
+        """`Algorithm.build(grad, params, iter): Delta` -> (delta, new_state)."""
+        dt = g.dtype
+        r, b1, b2, eps = dt.type(self.rate), dt.type(self.beta1), dt.type(self.beta2), dt.type(self.epsilon)
+        one = dt.type(1.0)
+        k = self.kind
+        if k == OPT_SGD:                                  # SGD.scala:15-25
+            v = (r * g) - (b1 * state[0])
+            delta = (r * g) - (b1 * v) if self.nesterov else v
+            return delta, [v]
+        if k == OPT_ADAGRAD:                              # AdaGrad.scala:21-32
+            acc = state[0] + sqr(g)
+            rates = r / sqrt_zero_safe(acc, eps)
+            return rates * g, [acc]
+        if k == OPT_ADADELTA:                             # AdaDelta.scala:33-44
+            avg_grad = decaying_avg(state[0], sqr(g), b1)
+            delta = r * ((sqrt_zero_safe(state[1], eps) / sqrt_zero_safe(avg_grad, eps)) * g)
+            avg_delta = decaying_avg(state[1], sqr(delta), b1)
+            return delta, [avg_grad, avg_delta]
+        if k == OPT_RMSPROP:                              # RMSProp.scala:24-32
+            avg_grad = decaying_avg(state[0], sqr(g), b1)
+            delta = (r / sqrt_zero_safe(avg_grad, eps)) * g
+            return delta, [avg_grad]
+        if k == OPT_ADAM:                                 # Adam.scala:29-41
+            m = decaying_avg(state[0], g, b1)
+            v = decaying_avg(state[1], sqr(g), b2)
+            delta = (r / np.sqrt(boost(v, b2, it) + eps)) * boost(m, b1, it)
+            return delta, [m, v]
+        if k == OPT_NADAM:                                # Nadam.scala:37-49
+            m = decaying_avg(state[0], g, b1)
+            v = decaying_avg(state[1], sqr(g), b2)
+            m_nest = (b1 * boost(m, b1, it)) + ((one - b1) * boost(g, b1, it))
+            delta = m_nest / (np.sqrt(boost(v, b2, it)) + eps)
+            return delta, [m, v]
+        if k == OPT_ADAMAX:                               # Adamax.scala:41-52
+            m1 = decaying_avg(state[0], g, b1)
+            m2 = np.maximum(b2 * state[1], (one - b2) * np.abs(g))
+            delta = r * boost(m1, b1, it) / (m2 + eps)
+            return delta, [m1, m2]
+        if k == OPT_AMSGRAD:                              # AMSGrad.scala:34-46
+            m = decaying_avg(state[0], g, b1)
+            v_cur = decaying_avg(state[1], sqr(g), b2)
+            v = np.maximum(state[2], v_cur)
+            delta = r * m / (np.sqrt(v) + eps)
+            return delta, [m, v_cur, v]
+        raise ValueError(k)
+
+
+def SGD(rate=0.01, momentum=0.0, nesterov=False):
+    return Algorithm(OPT_SGD, rate=rate, beta1=momentum, nesterov=nesterov)
+
+
+def AdaGrad(rate=0.001, epsilon=1e-7):
+    return Algorithm(OPT_ADAGRAD, rate=rate, epsilon=epsilon)
+
+
+def AdaDelta(rate=1.0, rho=0.9, epsilon=1e-7):
+    return Algorithm(OPT_ADADELTA, rate=rate, beta1=rho, epsilon=epsilon)
+
+
+def RMSProp(rate=0.001, rho=0.9, epsilon=1e-7):
+    return Algorithm(OPT_RMSPROP, rate=rate, beta1=rho, epsilon=epsilon)
+
+
+def Adam(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7):
+    return Algorithm(OPT_ADAM, rate=rate, beta1=beta1, beta2=beta2, epsilon=epsilon)
+
+
+def Nadam(beta1=0.9, beta2=0.999, epsilon=1e-7, init_acc=0.001):
+    return Algorithm(OPT_NADAM, rate=0.0, beta1=beta1, beta2=beta2, epsilon=epsilon, init_acc=init_acc)
+
+
+def Adamax(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7, init_acc=0.001):
+    return Algorithm(OPT_ADAMAX, rate=rate, beta1=beta1, beta2=beta2, epsilon=epsilon, init_acc=init_acc)
+
+
+def AMSGrad(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7):
+    return Algorithm(OPT_AMSGRAD, rate=rate, beta1=beta1, beta2=beta2, epsilon=epsilon)
+
+
+# --------------------------------------------------------------------------- #
+# the step, the per-partition loop and the averaging (optimizers/Optimizer.scala)
+# --------------------------------------------------------------------------- #
+
+
+def train_step(model: Model, alg: Algorithm, x, y, params, opt_state, it: int, minimizing=True):
+    """`compileBackprop`'s function (Optimizer.scala:169-194): one update of every weight.
+
+    Returns (new_params, new_opt_state, loss_before_update, grads)."""
+    loss, grads = model.grad(x, y, params)
+    new_params, new_state = {}, {}
+    for path, w in params.items():
+        delta, st = alg.build(grads[path], opt_state[path], it)
+        new_params[path] = w - delta if minimizing else w + delta    # Optimizer.scala:186
+        new_state[path] = st
+    return new_params, new_state, loss, grads
+
+
+def init_opt_state(alg: Algorithm, params):
+    return {p: alg.init_state(w.shape, w.dtype) for p, w in params.items()}
+
+
+def optimize_on_partition(model, alg, X, Y, batch, global_iter, params, opt_state):
+    """`optimizeOnPartition` (Optimizer.scala:106-161).
+
+    Full batches only (Iterators.scala:90, `Skip`); iteration numbers are
+    `global_iter + i + 1`; after the last batch the loss of that batch is
+    evaluated once more with the updated parameters (Optimizer.scala:148).
+    Returns (iterations, params, opt_state, loss)."""
+    n_batches = X.shape[0] // batch
+    if n_batches == 0:
+        raise StopIteration("empty partition")          # batches.next() throws (Iterators.scala:80-81)
+    for i in range(n_batches):
+        xb, yb = X[i * batch:(i + 1) * batch], Y[i * batch:(i + 1) * batch]
+        params, opt_state, _, _ = train_step(model, alg, xb, yb, params, opt_state, global_iter + i + 1)
+    loss = model.loss_of(xb, yb, params)
+    return n_batches, params, opt_state, loss
+
+
+def average_uniform(replicas: Sequence[np.ndarray]):
+    """`Aggregation.Avg` over K inputs: AddN(inputs) / K (Aggregation.scala:16-19).
+
+    AddN accumulates left to right in the element type."""
+    acc = replicas[0].copy()
+    for r in replicas[1:]:
+        acc = acc + r
+    return acc / acc.dtype.type(len(replicas))
+
+
+def avg2(l, r):
+    """The pairwise form `aggregateParams` applies (Optimizer.scala:205-210)."""
+    return (l + r) / l.dtype.type(2.0)
+
+
+def train(model, alg, partitions, batch, epochs, init_params, avg="uniform"):
+    """`Optimizer.run` (Optimizer.scala:59-104) with the Spark partitions given explicitly.
+
+    `partitions` is a list of (X, Y).  Every epoch each partition starts from
+    the same broadcast parameters; results are averaged (parameters and
+    optimizer state), losses averaged, iterations summed."""
+    params = {k: v.copy() for k, v in init_params.items()}
+    opt_state = init_opt_state(alg, params)
+    global_iter = 0
+    history = []
+    for _ in range(epochs):
+        results = [optimize_on_partition(model, alg, X, Y, batch, global_iter, params, opt_state)
+                   for X, Y in partitions]
+        if len(results) == 1:
+            iters, params, opt_state, loss = results[0]
+        else:
+            iters = sum(r[0] for r in results)
+            params = {p: average_uniform([r[1][p] for r in results]) for p in params}
+            opt_state = {p: [average_uniform([r[2][p][s] for r in results])
+                             for s in range(len(alg.state_names))] for p in params}
+            loss = float(np.mean([r[3] for r in results]))
+        global_iter += iters
+        history.append(float(loss))
+    return params, opt_state, history
+
+
+def count_correct(model, x, y, params):
+    """`estimators.accuracy`'s per-batch count (estimators/package.scala:28-32):
+    rows whose every rounded output equals the label."""
+    p = rint(model.forward(x, params))
+    matched = (y == p).astype(np.int32).sum(axis=1)
+    return int((matched == model.out_shape(x.shape)[-1]).astype(np.int32).sum())

@@ -1,0 +1,493 @@
+"""Pins the CPU oracle: reference known-answer vectors, brute force, an independent
+library (torch CPU) and float64 numerical gradients.  Nothing here touches a GPU."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as TF
+
+from oracle import scanet_oracle as O
+
+f32 = np.float32
+
+
+def A(v, dt=f32):
+    return np.asarray(v, dtype=dt)
+
+
+def round_at(x, p):
+    """`roundAt(p)` of the reference: Rint(x * 10^p) / 10^p (AllKernels.scala:528-531)."""
+    s = x.dtype.type(10.0 ** p)
+    return np.rint(x * s) / s
+
+
+# ----------------------------------------------------------------- conv / pool goldens
+@pytest.mark.parametrize("key,strides,padding,explicit", [
+    ("same_s1", (1, 1), O.PAD_SAME, (0, 0, 0, 0)),
+    ("same_s2", (2, 2), O.PAD_SAME, (0, 0, 0, 0)),
+    ("valid_s1", (1, 1), O.PAD_VALID, (0, 0, 0, 0)),
+    ("valid_s2", (2, 2), O.PAD_VALID, (0, 0, 0, 0)),
+    ("explicit_1010_s2", (2, 2), O.PAD_EXPLICIT, (1, 0, 1, 0)),
+])
+def test_conv2d_golden(golden, key, strides, padding, explicit):
+    x = A(golden["image_5x5"], np.float64).reshape(1, 5, 5, 1)
+    w = A(golden["filter_2x2"], np.float64).reshape(2, 2, 1, 1)
+    out = O.conv2d(x, w, strides, padding, explicit)
+    exp = A(golden["conv2d"][key], np.float64)
+    assert out.shape == (1,) + exp.shape + (1,)
+    np.testing.assert_array_equal(round_at(out, 2).reshape(exp.shape), exp)
+
+
+def test_conv2d_grads_golden(golden):
+    x = A(golden["image_5x5"], np.float64).reshape(1, 5, 5, 1)
+    w = A(golden["filter_2x2"], np.float64).reshape(2, 2, 1, 1)
+    dy = np.ones((1, 4, 4, 1))
+    gf = O.conv2d_grad_filter(x, w.shape, dy)
+    gi = O.conv2d_grad_input(x.shape, w, dy)
+    np.testing.assert_array_equal(gf.reshape(2, 2), A(golden["conv2d"]["valid_s1_grad_filter_of_sum"], np.float64))
+    np.testing.assert_array_equal(gi.reshape(5, 5), A(golden["conv2d"]["valid_s1_grad_input_of_sum"], np.float64))
+
+
+@pytest.mark.parametrize("key,strides,padding", [
+    ("same_s1", (1, 1), O.PAD_SAME), ("same_s2", (2, 2), O.PAD_SAME),
+    ("valid_s1", (1, 1), O.PAD_VALID), ("valid_s2", (2, 2), O.PAD_VALID),
+])
+def test_max_pool_golden(golden, key, strides, padding):
+    x = A(golden["image_5x5"], np.float64).reshape(1, 5, 5, 1)
+    out = O.max_pool(x, (2, 2), strides, padding)
+    exp = A(golden["max_pool_2x2"][key], np.float64)
+    np.testing.assert_array_equal(out.reshape(exp.shape), exp)
+
+
+def test_max_pool_grad_ties_golden(golden):
+    x = A(golden["image_5x5"], np.float64).reshape(1, 5, 5, 1)
+    g = O.max_pool_grad(x, np.ones((1, 5, 5, 1)), (2, 2), (1, 1), O.PAD_SAME)
+    np.testing.assert_array_equal(g.reshape(5, 5), A(golden["max_pool_2x2"]["same_s1_grad_input_of_sum"], np.float64))
+
+
+# ----------------------------------------------------------------- brute force + torch
+def _brute_conv(x, w, strides, padding):
+    n, h, wd, c = x.shape
+    kh, kw, _, f = w.shape
+    ho = O.out_size(padding, h, kh, strides[0])
+    wo = O.out_size(padding, wd, kw, strides[1])
+    pt, _ = O.pads_for(padding, h, kh, strides[0])
+    pl, _ = O.pads_for(padding, wd, kw, strides[1])
+    out = np.zeros((n, ho, wo, f))
+    for b, i, j, o in itertools.product(range(n), range(ho), range(wo), range(f)):
+        s = 0.0
+        for r, q, ci in itertools.product(range(kh), range(kw), range(c)):
+            y, xx = i * strides[0] + r - pt, j * strides[1] + q - pl
+            if 0 <= y < h and 0 <= xx < wd:
+                s += x[b, y, xx, ci] * w[r, q, ci, o]
+        out[b, i, j, o] = s
+    return out
+
+
+@pytest.mark.parametrize("strides", [(1, 1), (2, 2), (2, 1)])
+@pytest.mark.parametrize("padding", [O.PAD_VALID, O.PAD_SAME])
+def test_conv2d_brute_and_torch(strides, padding):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 7, 6, 3))
+    w = rng.standard_normal((3, 2, 3, 4))
+    out = O.conv2d(x, w, strides, padding)
+    np.testing.assert_allclose(out, _brute_conv(x, w, strides, padding), rtol=1e-12, atol=1e-12)
+    # gradients against torch autograd (independent library), explicit padding reproduced by F.pad
+    pt, pb = O.pads_for(padding, 7, 3, strides[0])
+    pl, pr = O.pads_for(padding, 6, 2, strides[1])
+    xt = torch.tensor(x.transpose(0, 3, 1, 2), requires_grad=True)
+    wt = torch.tensor(w.transpose(3, 2, 0, 1), requires_grad=True)
+    yt = TF.conv2d(TF.pad(xt, (pl, pr, pt, pb)), wt, stride=strides)
+    np.testing.assert_allclose(out, yt.detach().numpy().transpose(0, 2, 3, 1), rtol=1e-12, atol=1e-12)
+    dy = rng.standard_normal(out.shape)
+    yt.backward(torch.tensor(dy.transpose(0, 3, 1, 2)))
+    np.testing.assert_allclose(O.conv2d_grad_input(x.shape, w, dy, strides, padding),
+                               xt.grad.numpy().transpose(0, 2, 3, 1), rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(O.conv2d_grad_filter(x, w.shape, dy, strides, padding),
+                               wt.grad.numpy().transpose(2, 3, 1, 0), rtol=1e-11, atol=1e-11)
+
+
+@pytest.mark.parametrize("strides", [(1, 1), (2, 2)])
+@pytest.mark.parametrize("padding", [O.PAD_VALID, O.PAD_SAME])
+def test_max_pool_brute_first_max(strides, padding):
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 3, size=(2, 6, 5, 3)).astype(np.float64)      # many ties
+    kh = kw = 2
+    n, h, wd, c = x.shape
+    ho, wo = O.out_size(padding, h, kh, strides[0]), O.out_size(padding, wd, kw, strides[1])
+    pt, _ = O.pads_for(padding, h, kh, strides[0])
+    pl, _ = O.pads_for(padding, wd, kw, strides[1])
+    dy = rng.standard_normal((n, ho, wo, c))
+    out = np.zeros((n, ho, wo, c))
+    dx = np.zeros_like(x)
+    for b, i, j, ch in itertools.product(range(n), range(ho), range(wo), range(c)):
+        best, at = -np.inf, None
+        for r, q in itertools.product(range(kh), range(kw)):
+            y, xx = i * strides[0] + r - pt, j * strides[1] + q - pl
+            if 0 <= y < h and 0 <= xx < wd and x[b, y, xx, ch] > best:     # strict: first max wins
+                best, at = x[b, y, xx, ch], (y, xx)
+        out[b, i, j, ch] = best
+        dx[b, at[0], at[1], ch] += dy[b, i, j, ch]
+    np.testing.assert_array_equal(O.max_pool(x, (2, 2), strides, padding), out)
+    np.testing.assert_allclose(O.max_pool_grad(x, dy, (2, 2), strides, padding), dx, rtol=0, atol=1e-15)
+
+
+# ----------------------------------------------------------------- layer goldens
+def test_dense_sigmoid_forward_golden(golden):
+    g = golden["dense_sigmoid"]
+    m = O.Model([O.Dense(4, O.ACT_SIGMOID)])
+    assert [p for p, _ in m.param_defs((4, 3))] == ["0/weights", "1/weights"]
+    y = m.forward(A(g["x"]), {"0/weights": A(g["w"]), "1/weights": A(g["b"])})
+    np.testing.assert_array_equal(round_at(y, 6), A(g["y_6dp"]))
+
+
+def test_dense_bce_gradient_golden(golden):
+    g = golden["dense_sigmoid"]
+    m = O.Model([O.Dense(4, O.ACT_SIGMOID)], O.LOSS_BCE)
+    p = {"0/weights": np.zeros((3, 4), f32), "1/weights": np.zeros(4, f32)}
+    _, grads = m.grad(A(g["x"]), A(g["bce_y"]), p)
+    # the reference asserts exact float equality against TF; the restatement agrees to the last ulp or two
+    np.testing.assert_allclose(grads["0/weights"], A(g["bce_grad_w"]), rtol=3e-7, atol=0)
+    np.testing.assert_allclose(grads["1/weights"], A(g["bce_grad_b"]), rtol=3e-7, atol=0)
+
+
+def test_mlp_forward_and_loss_golden(golden):
+    g = golden["mlp_4_1"]
+    m = O.Model([O.Dense(4, O.ACT_SIGMOID), O.Dense(1, O.ACT_SIGMOID)])
+    assert [p for p, _ in m.param_defs((4, 3))] == ["0/weights", "1/weights", "3/weights", "4/weights"]
+    y = m.forward(A(g["x"]), {"0/weights": A(g["w1"]), "1/weights": A(g["b1"]),
+                              "3/weights": A(g["w2"]), "4/weights": A(g["b2"])})
+    # the last row is 0.80188651..: one float32 ulp decides which way the reference's 6-digit rounding falls,
+    # so this vector is compared as "equal before rounding, to within one ulp"
+    np.testing.assert_allclose(y, A(g["y_6dp"]), rtol=0, atol=0.5e-6 + 1.2e-7)
+    g = golden["mlp_3_1_loss"]
+    params = {"0/weights": A(g["w1"]), "1/weights": A(g["b1"]), "3/weights": A(g["w2"]), "4/weights": A(g["b2"])}
+    m = O.Model([O.Dense(3, O.ACT_SIGMOID), O.Dense(1, O.ACT_SIGMOID)], O.LOSS_MSE)
+    assert round_at(np.asarray(m.loss_of(A(g["x"]), A(g["y"]), params)), 6) == f32(g["mse_6dp"])
+    m2 = O.Model([O.Dense(3, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=1.0),
+                  O.Dense(1, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=1.0)], O.LOSS_MSE)
+    np.testing.assert_allclose(m2.loss_of(A(g["x"]), A(g["y"]), params), f32(g["mse_plus_l2"]), rtol=2e-7)
+
+
+def test_penalty_golden(golden):
+    g = golden["penalty_l2"]
+    m = O.Model([O.Dense(4, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=1.0)])
+    np.testing.assert_allclose(m.penalty({"0/weights": A(g["dense_w"]), "1/weights": np.zeros(2, f32)}),
+                               f32(g["dense_penalty"]), rtol=2e-7)
+    m = O.Model([O.Dense(4, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=1.0),
+                 O.Dense(1, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=1.0)])
+    p = {"0/weights": A(g["mlp_w1"]), "1/weights": np.zeros(4, f32), "3/weights": A(g["mlp_w2"]),
+         "4/weights": np.zeros(1, f32)}
+    np.testing.assert_allclose(m.penalty(p), f32(g["mlp_penalty"]), rtol=2e-7)
+
+
+def test_regression_goldens(golden):
+    g = golden["linear_regression"]
+    m = O.Model([O.Dense(1)], O.LOSS_MSE)
+    p = {"0/weights": A(g["w"]), "1/weights": A(g["b"])}
+    assert m.loss_of(A(g["x"]), A(g["y"]), p) == f32(g["mse"])
+    np.testing.assert_array_equal(m.forward(A(g["x"]), p), A(g["result"]))
+    _, grads = m.grad(A(g["x"]), A(g["y"]), {"0/weights": np.zeros((2, 1), f32), "1/weights": np.zeros(1, f32)})
+    np.testing.assert_array_equal(grads["0/weights"], A(g["grad_at_zero_w"]))
+    np.testing.assert_array_equal(grads["1/weights"], A(g["grad_at_zero_b"]))
+    g = golden["logistic_regression"]
+    m = O.Model([O.Dense(1, O.ACT_SIGMOID)], O.LOSS_BCE)
+    p = {"0/weights": A(g["w"]), "1/weights": A(g["b"])}
+    assert abs(float(m.loss_of(A(g["x"]), A(g["y"]), p)) - g["bce"]) <= 1e-6
+    np.testing.assert_array_equal(round_at(m.forward(A(g["x"]), p), 6), A(g["result_6dp"]))
+    _, grads = m.grad(A(g["x"]), A(g["y"]), p)
+    np.testing.assert_array_equal(round_at(grads["0/weights"], 6), A(g["grad_w_6dp"]))
+    np.testing.assert_array_equal(round_at(grads["1/weights"], 6), A(g["grad_b_6dp"]))
+
+
+def test_activation_goldens(golden):
+    g = golden["activations"]
+    np.testing.assert_allclose(np.tanh(f32(0.5)), f32(g["tanh_0.5"]), rtol=1.3e-7)     # one ulp
+    np.testing.assert_allclose(O.tanh_grad(A([-0.5, 0.0, 0.5]), np.ones(3, f32)),
+                               A([g["tanh_grad_at_pm0.5"], 1.0, g["tanh_grad_at_pm0.5"]]), rtol=1.2e-7)
+    np.testing.assert_array_equal(round_at(O.softmax(A(g["softmax_in"])), 5), A(g["softmax_5dp"]))
+    for k, v in g["relu"].items():
+        assert O.relu(f32(k)) == f32(v)
+    np.testing.assert_array_equal(round_at(O.sigmoid(A(g["sigmoid_in"])), 6), A(g["sigmoid_6dp"]))
+    np.testing.assert_allclose(np.exp(A(g["exp_in"])), A(g["exp"]), rtol=1.2e-7)
+    np.testing.assert_allclose(np.log(A(g["log_in"])), A(g["log"]), rtol=1.2e-7)
+    np.testing.assert_array_equal(O.rint(A(g["round_in"])), A(g["round"]))
+    assert O.relu_grad(f32(0.0), f32(1.0)) == 0.0       # strict comparison: no gradient at the threshold
+
+
+def test_matmul_and_helpers_golden(golden):
+    g = golden["matmul"]
+    np.testing.assert_array_equal(A(g["a"]) @ A(g["b"]), A(g["c"]))
+    ones = np.ones((2, 2), f32)
+    np.testing.assert_array_equal(A(g["a"]).T @ ones, A(g["grad_right_of_sum"]))          # left^T . parent
+    np.testing.assert_array_equal(ones @ A(g["x_right"]).T, A(g["grad_left_of_sum"]))     # parent . right^T
+    h = golden["helpers"]
+    d = h["decaying_avg"]
+    assert O.decaying_avg(np.float64(d["avg"]), np.float64(d["next"]), d["decay"]) == pytest.approx(d["out"], abs=1e-12)
+    s = h["sqrt_zero_safe"]
+    assert O.sqrt_zero_safe(f32(s["x"]), s["eps"]) == f32(s["out"])
+    for k in ("boost_t2", "boost_t1e6"):
+        b = h[k]
+        assert O.boost(f32(b["x"]), b["rate"], b["iter"]) == f32(b["out"])
+
+
+def test_simple_rnn_golden(golden):
+    g = golden["simple_rnn"]
+    m = O.Model([O.SimpleRNN(2, activation=O.ACT_IDENTITY)])
+    p = {"0/kernel_weights": A(g["wx"]), "0/recurrent_weights": A(g["wh"]), "1/weights": A(g["b"])}
+    y = m.forward(A(g["x"]).reshape(1, 3, 1), p)
+    np.testing.assert_array_equal(round_at(y, 6), A(g["y_6dp"]))
+
+
+def _lstm_params(g, pre=""):
+    p = {}
+    for gate in O.GATES:
+        p[f"{pre}{gate}/0/kernel_weights"] = A(g[gate]["k"])
+        p[f"{pre}{gate}/0/recurrent_weights"] = A(g[gate]["r"])
+        p[f"{pre}{gate}/1/weights"] = A(g[gate]["b"])
+    return p
+
+
+def test_lstm_forward_golden(golden):
+    g = golden["lstm"]
+    m = O.Model([O.LSTM(2)])
+    y = m.forward(A(g["x"]).reshape(1, 3, 1), _lstm_params(g))
+    np.testing.assert_array_equal(round_at(y, 6), A(g["y_6dp"]))
+
+
+def test_cnn_shape_table_golden(golden):
+    g = golden["cnn_shapes"]
+    m = O.Model([O.Conv2D(32, activation=O.ACT_RELU), O.Pool2D(), O.Conv2D(64, activation=O.ACT_RELU), O.Pool2D(),
+                 O.Flatten(), O.Dense(10, O.ACT_SOFTMAX)])
+    defs = dict(m.param_defs((1, 24, 24, 1)))
+    assert {k: list(v) for k, v in defs.items()} == g["weights"]
+    assert sum(int(np.prod(v)) for v in defs.values()) == g["total_params"]
+    s, outs = (1, 24, 24, 1), []
+    for l in m.layers:
+        s = l.out_shape(s)
+        outs.append(list(s[1:]))
+    assert outs == g["outputs"]
+
+
+# ----------------------------------------------------------------- gradients: float64 numerics + torch
+def _numeric_grad(m, x, y, params, path, eps=1e-6):
+    w = params[path]
+    g = np.zeros_like(w)
+    it = np.nditer(w, flags=["multi_index"])
+    for _ in it:
+        idx = it.multi_index
+        old = w[idx]
+        w[idx] = old + eps
+        lp = float(m.loss_of(x, y, params))
+        w[idx] = old - eps
+        lm = float(m.loss_of(x, y, params))
+        w[idx] = old
+        g[idx] = (lp - lm) / (2 * eps)
+    return g
+
+
+def _rand_params(m, in_shape, rng, dt=np.float64, scale=0.4):
+    return {p: (rng.standard_normal(s) * scale).astype(dt) for p, s in m.param_defs(in_shape)}
+
+
+@pytest.mark.parametrize("name", ["mlp_cce", "cnn_cce", "lstm_mse", "rnn_mse", "mlp_bce_l2"])
+def test_model_gradients_match_numeric_float64(name):
+    rng = np.random.default_rng(11)
+    if name == "mlp_cce":
+        m = O.Model([O.Dense(5, O.ACT_SIGMOID), O.Dense(6, O.ACT_TANH), O.Dense(4, O.ACT_SOFTMAX)], O.LOSS_CCE)
+        x = rng.random((3, 7))
+        y = np.eye(4)[rng.integers(0, 4, 3)]
+    elif name == "cnn_cce":
+        m = O.Model([O.Conv2D(3, activation=O.ACT_RELU), O.Pool2D(), O.Conv2D(2, (2, 2), (2, 2), O.PAD_SAME, O.ACT_RELU, bias=True),
+                     O.Pool2D(strides=(2, 2)), O.Flatten(), O.Dense(3, O.ACT_SOFTMAX)], O.LOSS_CCE)
+        x = rng.random((2, 9, 8, 2))
+        y = np.eye(3)[rng.integers(0, 3, 2)]
+    elif name == "lstm_mse":
+        m = O.Model([O.LSTM(4), O.Dense(1, O.ACT_TANH)], O.LOSS_MSE)
+        x = rng.standard_normal((3, 5, 2))
+        y = rng.uniform(-1, 1, (3, 1))
+    elif name == "rnn_mse":
+        m = O.Model([O.SimpleRNN(3), O.Dense(2)], O.LOSS_MSE)
+        x = rng.standard_normal((2, 4, 3))
+        y = rng.uniform(-1, 1, (2, 2))
+    else:
+        m = O.Model([O.Dense(3, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=0.3), O.Dense(2, O.ACT_SIGMOID)], O.LOSS_BCE)
+        x = rng.random((4, 3))
+        y = rng.integers(0, 2, (4, 2)).astype(np.float64)
+    params = _rand_params(m, x.shape, rng)
+    _, grads = m.grad(x, y, params)
+    for path in params:
+        num = _numeric_grad(m, x, y, params, path)
+        np.testing.assert_allclose(grads[path], num, rtol=2e-5, atol=2e-8, err_msg=path)
+
+
+def test_lstm_matches_torch_lstm_cell():
+    """Independent library check: torch.nn.LSTM (gate order i,f,g,o) with the reference's weights mapped in."""
+    rng = np.random.default_rng(2)
+    b, t, f, h = 3, 6, 4, 5
+    m = O.Model([O.LSTM(h)], O.LOSS_MSE)
+    params = _rand_params(m, (b, t, f), rng)
+    x = rng.standard_normal((b, t, f))
+    y = rng.standard_normal((b, h))
+    lstm = torch.nn.LSTM(f, h, batch_first=True).double()
+    order = ["input", "forget", "gate", "output"]
+    with torch.no_grad():
+        lstm.weight_ih_l0.copy_(torch.tensor(np.concatenate([params[f"{g}/0/kernel_weights"].T for g in order])))
+        lstm.weight_hh_l0.copy_(torch.tensor(np.concatenate([params[f"{g}/0/recurrent_weights"].T for g in order])))
+        lstm.bias_ih_l0.copy_(torch.tensor(np.concatenate([params[f"{g}/1/weights"] for g in order])))
+        lstm.bias_hh_l0.zero_()
+    out, _ = lstm(torch.tensor(x))
+    last = out[:, -1, :]
+    np.testing.assert_allclose(m.forward(x, params), last.detach().numpy(), rtol=1e-10, atol=1e-12)
+    loss = ((last - torch.tensor(y)) ** 2).mean()
+    loss.backward()
+    lo, grads = m.grad(x, y, params)
+    assert float(lo) == pytest.approx(float(loss.detach()), rel=1e-12)
+    gk = np.concatenate([grads[f"{g}/0/kernel_weights"].T for g in order])
+    gr = np.concatenate([grads[f"{g}/0/recurrent_weights"].T for g in order])
+    gb = np.concatenate([grads[f"{g}/1/weights"] for g in order])
+    np.testing.assert_allclose(gk, lstm.weight_ih_l0.grad.numpy(), rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(gr, lstm.weight_hh_l0.grad.numpy(), rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(gb, lstm.bias_ih_l0.grad.numpy(), rtol=1e-9, atol=1e-12)
+
+
+def test_softmax_cce_general_form_vs_textbook():
+    """With one-hot rows and eps negligible the chain reduces to (p - y) / B."""
+    rng = np.random.default_rng(4)
+    z = rng.standard_normal((6, 5))
+    y = np.eye(5)[rng.integers(0, 5, 6)]
+    p = O.softmax(z)
+    dz = O.softmax_grad(z, O.loss_grad(O.LOSS_CCE, p, y))
+    np.testing.assert_allclose(dz, (p - y) / 6, rtol=1e-6, atol=1e-9)
+
+
+# ----------------------------------------------------------------- optimizers
+ALGS = {"SGD": O.SGD, "Adam": O.Adam, "AdaGrad": O.AdaGrad, "AdaDelta": O.AdaDelta, "RMSProp": O.RMSProp,
+        "Nadam": O.Nadam, "Adamax": O.Adamax, "AMSGrad": O.AMSGrad}
+
+
+def test_state_names_and_inits():
+    assert O.SGD().state_names == ["velocity"]                                   # SGD.scala:29
+    assert O.AdaGrad().state_names == ["grad_acc"]                               # AdaGrad.scala:36
+    assert O.AdaDelta().state_names == ["avg_grad", "avg_delta"]                 # AdaDelta.scala:48-49
+    assert O.RMSProp().state_names == ["avg_grad"]
+    assert O.Adam().state_names == ["momentum", "velocity"]
+    assert O.Adamax().state_names == ["momentum_1", "momentum_2"]
+    assert O.AMSGrad().state_names == ["momentum", "velocity", "corrected_velocity"]
+    assert float(O.Nadam().init_state((1,))[0][0]) == f32(0.001)                 # Nadam.scala:26-35
+    assert float(O.Adamax().init_state((1,))[1][0]) == f32(0.001)                # Adamax.scala:30-39
+    assert float(O.Adam().init_state((1,))[0][0]) == 0.0
+
+
+def test_convergence_thresholds(golden, linear_function):
+    X, Y = linear_function
+    assert X.shape == (97, 1)
+    m = O.Model([O.Dense(1)], O.LOSS_MSE)
+    init = {"0/weights": np.zeros((1, 1), f32), "1/weights": np.zeros(1, f32)}
+    for case in golden["convergence"]["cases"]:
+        alg = ALGS[case["alg"]](**case["args"])
+        params, _, _ = O.train(m, alg, [(X, Y)], 97, case["epochs"], init)
+        final = float(m.loss_of(X, Y, params))
+        assert final <= case["max_loss"], (case, final)
+        assert final > 4.0            # the data's least-squares optimum is about 4.48; nothing can beat it
+
+
+def test_logistic_adam_golden(golden, logistic_data):
+    g = golden["convergence"]["logistic_adam"]
+    X, Y = logistic_data
+    m = O.Model([O.Dense(1, O.ACT_SIGMOID)], O.LOSS_BCE)
+    init = {"0/weights": np.zeros((2, 1), f32), "1/weights": np.zeros(1, f32)}
+    params, _, _ = O.train(m, O.Adam(g["rate"]), [(X, Y)], g["batch"], g["epochs"], init)
+    assert float(m.loss_of(X, Y, params)) <= g["max_loss"]
+    assert O.count_correct(m, X, Y, params) / X.shape[0] >= g["min_accuracy"]
+    np.testing.assert_array_equal(O.rint(m.forward(A(g["predict_in"]), params)), A(g["predict_rounded"]))
+
+
+def test_sgd_x2_closed_form(golden):
+    g = golden["convergence"]["sgd_x2"]
+    alg = O.SGD(g["rate"])
+    w, st = np.array(g["w0"], np.float64), alg.init_state((), np.float64)
+    for t in range(1, g["epochs"] + 1):
+        delta, st = alg.build(2 * w, st, t)        # d/dw w^2
+        w = w - delta
+    assert float(w) == pytest.approx(g["w0"] * 0.8 ** g["epochs"], rel=1e-9)
+    assert float(w * w) <= g["max_loss"]
+
+
+def test_optimizer_closed_forms_constant_gradient():
+    """With a constant gradient and zero state the bias-corrected moments equal g and g^2 at every step,
+    so each rule collapses to a closed form that a dropped (1-beta), a wrong exponent or a misplaced
+    epsilon would break."""
+    g = np.array([0.3, -1.7, 2.5e-3], np.float64)
+    w0 = np.array([1.0, -2.0, 0.5], np.float64)
+    lr, eps = 0.01, 1e-7
+    a = O.Adam(lr)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 8):
+        d, st = a.build(g, st, t)
+        np.testing.assert_allclose(d, lr * g / np.sqrt(g * g + eps), rtol=1e-10)
+    a = O.AdaGrad(lr)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)
+        np.testing.assert_allclose(d, lr * g / np.sqrt(t * g * g + eps), rtol=1e-12)
+    a = O.RMSProp(lr)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)
+        np.testing.assert_allclose(d, lr * g / np.sqrt((1 - 0.9 ** t) * g * g + eps), rtol=1e-10)
+    a = O.AMSGrad(lr)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)
+        np.testing.assert_allclose(d, lr * (1 - 0.9 ** t) * g / (np.sqrt((1 - 0.999 ** t) * g * g) + eps), rtol=1e-10)
+    a = O.Adamax(lr, init_acc=0.0)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)      # m2 = max(beta2*m2, (1-beta2)|g|) stays (1-beta2)|g|
+        np.testing.assert_allclose(d, lr * g / (0.001 * np.abs(g) + eps), rtol=1e-9)
+    a = O.Nadam(init_acc=0.0)
+    st = a.init_state(g.shape, np.float64)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)      # m_hat = g, g_hat = g/(1-b1^t)
+        np.testing.assert_allclose(d, (0.9 * g + 0.1 * g / (1 - 0.9 ** t)) / (np.abs(g) + eps), rtol=1e-9)
+    a = O.SGD(lr, momentum=0.5)
+    st = a.init_state(g.shape, np.float64)
+    v = np.zeros_like(g)
+    for t in range(1, 6):
+        d, st = a.build(g, st, t)      # v_t = lr g - mu v_{t-1} = lr g (1 - (-mu)^t) / (1 + mu)
+        np.testing.assert_allclose(d, lr * g * (1 - (-0.5) ** t) / 1.5, rtol=1e-12)
+    a = O.AdaDelta()
+    st = a.init_state(g.shape, np.float64)
+    d, st = a.build(g, st, 1)
+    np.testing.assert_allclose(d, np.sqrt(eps) / np.sqrt(0.1 * g * g + eps) * g, rtol=1e-12)
+    np.testing.assert_allclose(st[1], 0.1 * d * d, rtol=1e-12)
+
+
+def test_average_uniform_and_pairwise():
+    rng = np.random.default_rng(0)
+    reps = [rng.standard_normal(1000).astype(f32) for _ in range(8)]
+    ref = np.mean(np.stack(reps).astype(np.float64), axis=0)
+    np.testing.assert_allclose(O.average_uniform(reps), ref, rtol=1e-6, atol=1e-7)
+    np.testing.assert_array_equal(O.avg2(reps[0], reps[1]), (reps[0] + reps[1]) / f32(2))
+    # one replica: identity
+    np.testing.assert_array_equal(O.average_uniform(reps[:1]), reps[0])
+
+
+def test_partition_loop_semantics(linear_function):
+    """1-based iteration numbers, partial batch dropped, final loss evaluated after the last update."""
+    X, Y = linear_function
+    m = O.Model([O.Dense(1)], O.LOSS_MSE)
+    init = {"0/weights": np.zeros((1, 1), f32), "1/weights": np.zeros(1, f32)}
+    alg = O.Adam(0.1)
+    it, p, st, loss = O.optimize_on_partition(m, alg, X, Y, 40, 0, init, O.init_opt_state(alg, init))
+    assert it == 2                                   # 97 rows, batch 40: 2 full batches, 17 rows skipped
+    # replay by hand
+    q, s = init, O.init_opt_state(alg, init)
+    for i in range(2):
+        q, s, _, _ = O.train_step(m, alg, X[i * 40:(i + 1) * 40], Y[i * 40:(i + 1) * 40], q, s, i + 1)
+    np.testing.assert_array_equal(p["0/weights"], q["0/weights"])
+    assert loss == m.loss_of(X[40:80], Y[40:80], q)
+    with pytest.raises(StopIteration):
+        O.optimize_on_partition(m, alg, X[:10], Y[:10], 40, 0, init, O.init_opt_state(alg, init))
