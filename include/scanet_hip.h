@@ -1,0 +1,236 @@
+/*
+ * scanet_hip.h -- C ABI of the MI355X (gfx950) execution backend for scanet's
+ * compiled training / inference step.
+ *
+ * The library replaces what scanet3 reaches through TensorFlow-Java: graph
+ * construction + Session.run for the step that `Optimizer.compileBackprop`
+ * builds, the forward/loss functions, and the parameter averaging of
+ * `Optimizer.aggregateParams`.  Every entry point notes the reference
+ * interface it stands in for (paths under src/main/scala/scanet/).
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative SN_E_* code on failure;
+ *     sn_last_error() gives the message of the calling thread's last failure
+ *     (the reference turns a TF status into an exception, native/package.scala:6-10);
+ *   - handles are owned by the caller and must be destroyed by it;
+ *   - a context, and everything created from it, is used by one host thread at
+ *     a time (the reference hands a Session to one thread at a time,
+ *     core/Session.scala:147-166); different contexts may run concurrently;
+ *   - all work of a context is issued on that context's HIP stream; calls that
+ *     return host values (a loss, a count, a d2h copy) wait for the stream,
+ *     the others are asynchronous and ordered;
+ *   - pointers named *_dev are device addresses (from sn_buffer_alloc or any
+ *     other HIP allocation on the context's device), pointers named *_host are
+ *     ordinary host memory;
+ *   - tensors are dense, row-major float32; images are NHWC
+ *     (core/TensorType.scala:170-174, math/nn/AllKernels.scala:129-133).
+ */
+#ifndef SCANET_HIP_H
+#define SCANET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct sn_ctx sn_ctx;
+typedef struct sn_model sn_model;
+typedef struct sn_replica sn_replica;
+
+enum {
+  SN_OK = 0,
+  SN_E_INVALID = -1,     /* bad argument / unsupported combination (reference: require(..) failures) */
+  SN_E_HIP = -2,         /* a HIP runtime call failed */
+  SN_E_OOM = -3,         /* device or host allocation failed */
+  SN_E_STATE = -4        /* object used after destroy / wrong context */
+};
+
+/* ---- layer list (models/layer/*.scala, flattened as layer/Composed.scala:89-99 does) ---- */
+enum { SN_LAYER_DENSE = 0, SN_LAYER_BIAS = 1, SN_LAYER_ACTIVATE = 2, SN_LAYER_FLATTEN = 3,
+       SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6 };
+/* models/Activation.scala:32-83 */
+enum { SN_ACT_IDENTITY = 0, SN_ACT_SIGMOID = 1, SN_ACT_TANH = 2, SN_ACT_RELU = 3, SN_ACT_SOFTMAX = 4 };
+/* models/Loss.scala:18-57 */
+enum { SN_LOSS_IDENTITY = 0, SN_LOSS_MSE = 1, SN_LOSS_BINARY_CROSSENTROPY = 2, SN_LOSS_CATEGORICAL_CROSSENTROPY = 3 };
+/* math/nn/AllKernels.scala:25-103 */
+enum { SN_PAD_VALID = 0, SN_PAD_SAME = 1 };
+/* models/Regularization.scala:16-44 */
+enum { SN_REG_NONE = 0, SN_REG_L1 = 1, SN_REG_L2 = 2 };
+/* optimizers/{SGD,AdaGrad,AdaDelta,RMSProp,Adam,Nadam,Adamax,AMSGrad}.scala */
+enum { SN_OPT_SGD = 0, SN_OPT_ADAGRAD = 1, SN_OPT_ADADELTA = 2, SN_OPT_RMSPROP = 3,
+       SN_OPT_ADAM = 4, SN_OPT_NADAM = 5, SN_OPT_ADAMAX = 6, SN_OPT_AMSGRAD = 7 };
+/* model flags */
+enum {
+  SN_FLAG_GEMM_BF16 = 1,       /* Dense GEMMs take bf16 inputs (fp32 accumulate, fp32 master weights) */
+  SN_FLAG_STABLE_SOFTMAX = 2   /* subtract the row maximum before exp (the reference does not, Activation.scala:63-69) */
+};
+
+/* One entry of the flattened layer list.  `Dense(n, act)` of the reference is the
+ * three entries DENSE, BIAS, ACTIVATE (layer/Dense.scala:30-40), `Conv2D(..)` is
+ * CONV2D [, BIAS] [, ACTIVATE] (layer/Conv2D.scala:54-68); parameter paths are
+ * "<index in this list>/weights" exactly as Composed.params builds them. */
+typedef struct sn_layer_desc {
+  int32_t kind;          /* SN_LAYER_* */
+  int32_t units;         /* Dense outputs / Bias features / Conv2D filters / LSTM units */
+  int32_t activation;    /* ACTIVATE: SN_ACT_*  (LSTM: cell activation, must be SN_ACT_TANH) */
+  float act_param;       /* ReLU threshold (Activation.scala:79-82) */
+  int32_t kernel_h, kernel_w;   /* Conv2D kernel / Pool2D window */
+  int32_t stride_h, stride_w;
+  int32_t padding;       /* SN_PAD_* */
+  int32_t reg_kind;      /* Dense/Bias: SN_REG_* */
+  float reg_lambda;
+  int32_t use_bias;      /* LSTM only: per-gate bias vectors (layer/RNN.scala:215) */
+} sn_layer_desc;
+
+/* An `Algorithm` case class (optimizers/Algorithm.scala:6-11).  Field use per kind:
+ *   SGD      rate, beta1 = momentum, nesterov
+ *   AdaGrad  rate, epsilon
+ *   AdaDelta rate, beta1 = rho, epsilon
+ *   RMSProp  rate, beta1 = rho, epsilon
+ *   Adam / AMSGrad  rate, beta1, beta2, epsilon
+ *   Nadam    beta1, beta2, epsilon, init_acc
+ *   Adamax   rate, beta1, beta2, epsilon, init_acc                              */
+typedef struct sn_optimizer_desc {
+  int32_t kind;          /* SN_OPT_* */
+  float rate;
+  float beta1;
+  float beta2;
+  float epsilon;
+  float init_acc;        /* initial value of every state tensor (Nadam.scala:26-35, Adamax.scala:30-39) */
+  int32_t nesterov;
+} sn_optimizer_desc;
+
+#define SN_MAX_RANK 8
+#define SN_MAX_OPT_STATES 3
+#define SN_MAX_AVG_INPUTS 32
+
+/* One parameter tensor of a model, in flat-buffer order. */
+typedef struct sn_param_info {
+  char path[96];                 /* reference path, e.g. "0/weights", "0/forget/0/kernel_weights" */
+  int64_t offset;                /* first element inside the replica's flat parameter buffer */
+  int64_t size;                  /* number of elements */
+  int32_t rank;
+  int64_t dims[SN_MAX_RANK];
+} sn_param_info;
+
+/* ---------------------------------------------------------------- context / errors */
+
+/* Replaces `new Session()` = Graph + TF Session (core/Session.scala:57-63).
+ * `stream` is a hipStream_t to issue all work on, or NULL to let the context
+ * create (and own) one. */
+int sn_ctx_create(int device, void* stream, sn_ctx** out);
+/* Replaces Session.close (core/Session.scala:106). Waits for outstanding work. */
+int sn_ctx_destroy(sn_ctx* ctx);
+/* Message of the calling thread's most recent failing call (never NULL). */
+const char* sn_last_error(void);
+/* Blocks until everything issued on the context's stream has finished. */
+int sn_sync(sn_ctx* ctx);
+/* Name, HBM bytes and compute-unit count of the context's device
+ * (reference: core/Devices.scala:23-37 lists TF devices). */
+int sn_device_info(sn_ctx* ctx, char* name, int name_cap, int64_t* hbm_bytes, int32_t* compute_units);
+
+/* ---------------------------------------------------------------- tensors / memory */
+
+/* Replaces TF_AllocateTensor / TF_DeleteTensor (native/RawTensors.scala:81-88,106-115)
+ * for device-resident tensors. */
+int sn_buffer_alloc(sn_ctx* ctx, size_t bytes, void** out_dev);
+int sn_buffer_free(sn_ctx* ctx, void* dev);
+/* Pinned host memory a JVM can wrap as a read-only DirectBuffer
+ * (native/RawTensors.scala:24-30, core/TensorCodec.scala:12-22). */
+int sn_host_alloc(sn_ctx* ctx, size_t bytes, void** out_host);
+int sn_host_free(sn_ctx* ctx, void* host);
+/* Replaces the feed / fetch halves of Session.Runner (core/Session.scala:83-95).
+ * h2d is asynchronous when src is pinned; d2h returns after the data has arrived. */
+int sn_copy_h2d(sn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int sn_copy_d2h(sn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+int sn_fill(sn_ctx* ctx, float* dst_dev, float value, int64_t n);
+
+/* ---------------------------------------------------------------- model = compiled step */
+
+/* Replaces building `model.withLoss(loss)` and compiling its functions
+ * (models/Model.scala:84-119, optimizers/Optimizer.scala:163-194, core/TF.scala:391-438).
+ * `input_dims` is the shape of ONE sample (e.g. {784}, {28,28,1}, {64,32}); `batch`
+ * is the largest number of rows any call will pass. */
+int sn_model_create(sn_ctx* ctx, const sn_layer_desc* layers, int32_t n_layers, int32_t loss,
+                    const int64_t* input_dims, int32_t input_rank, int32_t batch, uint32_t flags,
+                    sn_model** out);
+int sn_model_destroy(sn_model* model);
+/* `model.params(input)` restricted to trainable weights (models/Model.scala:18;
+ * optimizers/Optimizer.scala:117-122), in flat-buffer order. */
+int sn_model_param_count(sn_model* model, int32_t* n_tensors, int64_t* flat_elems);
+int sn_model_param_info(sn_model* model, int32_t index, sn_param_info* out);
+/* `model.outputShape(input)` for one sample (models/Model.scala:41). */
+int sn_model_output_shape(sn_model* model, int32_t* rank, int64_t* dims);
+
+/* ---------------------------------------------------------------- replica = params + optimizer state */
+
+/* One partition's training state: the flat weight, gradient and optimizer-state
+ * buffers that optimizeOnPartition threads through its loop
+ * (optimizers/Optimizer.scala:117-131). Weights start at zero, optimizer state at
+ * `opt->init_acc` (ParamDef.initialize). `opt` may be NULL for inference only. */
+int sn_replica_create(sn_model* model, const sn_optimizer_desc* opt, sn_replica** out);
+int sn_replica_destroy(sn_replica* rep);
+/* `.initParams(Params)` / reading `TrainedModel.params` (optimizers/Optimizer.scala:276-277,103). */
+int sn_params_set(sn_replica* rep, int32_t index, const float* src_host, int64_t n);
+int sn_params_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
+/* Optimizer state tensor `<path>/<state name>` (optimizers/Optimizer.scala:118-121); slot order is
+ * the order of the algorithm's `params` (e.g. Adam: 0 momentum, 1 velocity). */
+int sn_optstate_set(sn_replica* rep, int32_t index, int32_t slot, const float* src_host, int64_t n);
+int sn_optstate_get(sn_replica* rep, int32_t index, int32_t slot, float* dst_host, int64_t n);
+/* Gradient of the last sn_step / sn_grad for one tensor (`LossModel.grad`, models/Model.scala:107-111). */
+int sn_grads_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
+/* Device views of the flat buffers: slot -2 weights, -1 gradients, 0.. optimizer state tensors. */
+int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n);
+
+/* One call of the compiled backprop function (optimizers/Optimizer.scala:142-143, 169-194):
+ * forward, loss, gradients of every weight, optimizer update w' = w - delta with iteration
+ * number `iter` (1-based). `rows` <= batch. If `loss_host` is not NULL the loss of this batch
+ * (before the update) is written there and the call waits for the device. */
+int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host);
+/* `LossModel.grad` (models/Model.scala:107-111): gradients only, no update. */
+int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
+/* `model.result` (models/Model.scala:35-36): out_dev receives rows x output elements. */
+int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
+/* `LossModel.loss` (models/Model.scala:101-102). */
+int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
+/* Per-batch body of `estimators.accuracy` (estimators/package.scala:28-32): rows whose every
+ * rounded (half to even) output equals the label. */
+int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int64_t* count_host);
+/* `optimizeOnPartition` (optimizers/Optimizer.scala:106-161) over a device-resident partition of
+ * `total_rows` samples: every full batch in order with iter = global_iter + i + 1, partial batch
+ * skipped (optimizers/Iterators.scala:90), then the loss of the last batch under the updated
+ * weights. Fails with SN_E_INVALID when the partition holds no full batch. */
+int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch,
+                   int32_t global_iter, int32_t* iterations_host, float* loss_host);
+
+/* `aggregateParams` (optimizers/Optimizer.scala:196-230) for K replicas of one model: weights and
+ * every optimizer-state tensor become the uniform mean AddN(..)/K (models/Aggregation.scala:16-19)
+ * and are written back to all K replicas (the next epoch's broadcast, Optimizer.scala:72-73). */
+int sn_replicas_average(sn_replica* const* reps, int32_t k);
+
+/* ---------------------------------------------------------------- flat kernels (the memory-bound pair) */
+
+/* One fused `Algorithm.build` + `w - delta` over a flat vector (optimizers/Optimizer.scala:181-188):
+ * w[i], state*[i] updated in place from g[i]. Unused state pointers may be NULL. */
+int sn_optimizer_update(sn_ctx* ctx, const sn_optimizer_desc* opt, float* w_dev, const float* g_dev,
+                        float* s0_dev, float* s1_dev, float* s2_dev, int64_t n, int32_t iter);
+/* `Aggregation.Avg` over k inputs (models/Aggregation.scala:16-19): out = (in[0] + .. + in[k-1]) / k,
+ * accumulated left to right. `inputs_host` is a host array of k device pointers; out may alias in[0]. */
+int sn_average(sn_ctx* ctx, const float* const* inputs_host, int32_t k, int64_t n, float* out_dev);
+
+/* ---------------------------------------------------------------- per-kernel timing */
+
+/* When enabled every kernel launch of the context is bracketed by HIP events on the context's
+ * stream (the reference only has wall-clock per epoch, optimizers/Optimizer.scala:74,87-89). */
+int sn_profile_enable(sn_ctx* ctx, int32_t on);
+int sn_profile_reset(sn_ctx* ctx);
+/* Number of distinct kernel names seen since the last reset (waits for the stream). */
+int sn_profile_count(sn_ctx* ctx, int32_t* n);
+int sn_profile_get(sn_ctx* ctx, int32_t index, char* name, int32_t name_cap, double* total_ms, int64_t* launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCANET_HIP_H */

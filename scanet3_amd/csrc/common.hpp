@@ -1,0 +1,190 @@
+// Internal declarations shared by the HIP translation units of libscanet_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/scanet_hip.h"
+
+namespace sn {
+
+// ---- error handling -------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+
+#define SN_HIP(expr)                                                                         \
+  do {                                                                                       \
+    hipError_t e__ = (expr);                                                                 \
+    if (e__ != hipSuccess)                                                                   \
+      return sn::fail(e__ == hipErrorOutOfMemory ? SN_E_OOM : SN_E_HIP, "%s failed: %s (%s:%d)", #expr, \
+                      hipGetErrorString(e__), __FILE__, __LINE__);                           \
+  } while (0)
+
+#define SN_TRY(expr)           \
+  do {                         \
+    int r__ = (expr);          \
+    if (r__ != SN_OK) return r__; \
+  } while (0)
+
+#define SN_REQUIRE(cond, ...)                                \
+  do {                                                       \
+    if (!(cond)) return sn::fail(SN_E_INVALID, __VA_ARGS__); \
+  } while (0)
+
+// ---- per-kernel timing ----------------------------------------------------------------
+struct ProfileEntry {
+  double total_ms = 0.0;
+  int64_t launches = 0;
+};
+
+struct PendingEvent {
+  hipEvent_t start, stop;
+  const char* name;
+};
+
+}  // namespace sn
+
+struct sn_ctx {
+  uint32_t magic;
+  int device;
+  hipStream_t stream;
+  bool owns_stream;
+  int compute_units;
+  // timing
+  bool profiling;
+  std::vector<sn::PendingEvent> pending;
+  std::vector<hipEvent_t> event_pool;
+  std::map<std::string, sn::ProfileEntry> profile;
+  std::vector<std::string> profile_names;  // stable order for sn_profile_get
+};
+
+namespace sn {
+
+constexpr uint32_t CTX_MAGIC = 0x534e4358u;  // "SNCX"
+constexpr uint32_t MODEL_MAGIC = 0x534e4d44u;
+constexpr uint32_t REPLICA_MAGIC = 0x534e5250u;
+
+// Brackets one kernel launch with events when the context is profiling.
+struct LaunchScope {
+  sn_ctx* ctx;
+  hipEvent_t start = nullptr, stop = nullptr;
+  const char* name;
+  LaunchScope(sn_ctx* c, const char* n);
+  ~LaunchScope();
+};
+int profile_drain(sn_ctx* ctx);
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int64_t align_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// ---- optimizer / averaging kernels (optim_kernels.hip) ---------------------------------
+// Scalars every algorithm needs, evaluated once per step on the host in float32.
+struct OptScalars {
+  float rate, b1, b2, eps;
+  float one_minus_b1, one_minus_b2;  // `1f.const - beta` evaluated in float32
+  float bc1, bc2;                    // 1 - beta^iter, the divisor of `boost`
+  int nesterov;
+};
+OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter);
+int opt_state_count(int kind);
+int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
+                     int64_t n, int iter);
+struct AvgInputs {
+  const float* p[SN_MAX_AVG_INPUTS];
+};
+int launch_average(sn_ctx* ctx, const AvgInputs& in, int k, int64_t n, float* out, float* const* extra_out, int n_extra);
+int launch_fill(sn_ctx* ctx, float* dst, float v, int64_t n);
+
+// ---- elementwise / row kernels (elementwise_kernels.hip) -------------------------------
+int launch_bias_act(sn_ctx* ctx, const float* x, const float* bias, float* y, int64_t rows, int cols, int act, float act_param);
+int launch_act_bwd(sn_ctx* ctx, const float* y, const float* dy, float* dx, int64_t n, int act, float act_param);
+int launch_softmax_fwd(sn_ctx* ctx, const float* z, float* p, int rows, int cols, bool stable);
+int launch_softmax_bwd(sn_ctx* ctx, const float* p, const float* dp, float* dz, int rows, int cols);
+// loss value (sum of per-element terms / divisor) into *loss_dev and d loss / d p into dp (dp may be null)
+int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp, float* loss_dev, float* partials,
+                int rows, int cols);
+// out[c] = sum over rows of dy[r*ld + c]; `ws` (optional) lets many rows be summed in parallel slices
+int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems);
+int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev);
+int launch_penalty_grad(sn_ctx* ctx, const float* w, float* g, int64_t n, int reg_kind, float lambda);
+int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, int cols, unsigned long long* count_dev);
+int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo,
+                       int kh, int kw, int sh, int sw, int pt, int pl);
+int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho,
+                       int wo, int kh, int kw, int sh, int sw, int pt, int pl);
+struct LstmGateArgs {
+  const float* z;       // [rows, 4H] pre-activations incl. bias, gate order forget,input,gate,output
+  const float* c_prev;  // [rows, H] or null (zeros)
+  float* gates;         // [rows, 4H] activated f,i,g,o
+  float* c;             // [rows, H]
+  float* h;             // [rows, H]
+};
+int launch_lstm_gates_fwd(sn_ctx* ctx, const LstmGateArgs& a, int rows, int hidden);
+struct LstmGateBwdArgs {
+  const float* gates;   // activated f,i,g,o of this step
+  const float* c;       // c_t
+  const float* c_prev;  // c_{t-1} or null
+  const float* dh;      // [rows,H]
+  float* dc;            // [rows,H] in: dc_t carried from t+1 (or zeros), out: dc_{t-1}
+  float* dz;            // [rows,4H]
+  int dc_is_zero;       // first backward step: treat dc as zeros on input
+};
+int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
+
+// ---- GEMM family (gemm_kernels.hip) ----------------------------------------------------
+struct Epilogue {
+  float* out = nullptr;
+  int64_t ldo = 0;
+  const float* bias = nullptr;  // per output column, may be null
+  int act = SN_ACT_IDENTITY;    // identity / sigmoid / tanh / relu (softmax is a row kernel)
+  float act_param = 0.f;
+};
+// C[M,N] = A[M,K] * B[K,N] with arbitrary element strides (covers NN, NT, TN).
+struct GemmDesc {
+  const float* a; int64_t a_sm, a_sk;   // A(m,k) = a[m*a_sm + k*a_sk]
+  const float* b; int64_t b_sk, b_sn;   // B(k,n) = b[k*b_sk + n*b_sn]
+  int m, n, k;
+};
+int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* workspace, int64_t workspace_elems, bool bf16);
+
+struct ConvGeom {
+  int n, h, w, cin;      // input
+  int ho, wo, cout;      // output
+  int kh, kw, sh, sw, pt, pl;
+};
+int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& ep, float* ws, int64_t ws_elems);
+int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems);
+int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems);
+
+struct LstmWeights {
+  const float* wk[4];  // [F,H] forget,input,gate,output
+  const float* wr[4];  // [H,H]
+  const float* b[4];   // [H] or null
+};
+struct LstmGrads {
+  float* wk[4];
+  float* wr[4];
+  float* b[4];
+};
+// z[rows,4H] = [x_t, h_prev] * [Wk; Wr] + b   (x_t = x[:, t, :] of a [rows,T,F] tensor)
+int launch_lstm_z(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, int rows, int H, const LstmWeights& w,
+                  float* z, float* ws, int64_t ws_elems);
+// dh_prev[rows,H] = dz[rows,4H] * Wr^T
+int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems);
+// dx[:, t, :] = dz * Wk^T
+int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, int T, const LstmWeights& w, float* dx, float* ws,
+                   int64_t ws_elems);
+// dWk = X^T dZ, dWr = Hprev^T dZ over all steps (dz_all, h_all time-major [T,rows,*]; h_all[t] = h_{t-1})
+int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
+                      const LstmGrads& g, float* ws, int64_t ws_elems);
+
+int64_t gemm_workspace_elems(int m, int n, int k, int cu);
+
+}  // namespace sn

@@ -1,0 +1,515 @@
+// Memory-bound layer kernels: bias + activation, activation backward, softmax rows,
+// losses, column sums (bias gradients), regularisation, max pooling, LSTM gate maths
+// and the accuracy count.  All arithmetic is float32 in the reference's operation
+// order (no fused multiply-add; the file is compiled with -ffp-contract=off).
+#include "common.hpp"
+
+namespace sn {
+
+// ---------------------------------------------------------------------------- helpers
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ float act_fwd(int act, float x, float param) {
+  switch (act) {
+    case SN_ACT_SIGMOID: return sigmoidf_(x);
+    case SN_ACT_TANH: return tanhf(x);
+    case SN_ACT_RELU: return fmaxf(param, x);  // Maximum(threshold, x), Activation.scala:79-82
+    default: return x;
+  }
+}
+
+// Gradient through an activation given its OUTPUT y (each rule below is the reference's
+// localGrad with the recomputed forward value replaced by the stored one, which is the
+// same float):
+//   sigmoid: s*(1-s)*dy (AllKernels.scala:397-404)   tanh: (1 - y^2)*dy (:414-420)
+//   relu: (threshold < x) * dy with x > threshold <=> y > threshold (:297-302)
+__device__ __forceinline__ float act_bwd(int act, float y, float dy, float param) {
+  switch (act) {
+    case SN_ACT_SIGMOID: return (y * (1.0f - y)) * dy;
+    case SN_ACT_TANH: return (1.0f - y * y) * dy;
+    case SN_ACT_RELU: return (param < y ? 1.0f : 0.0f) * dy;
+    default: return dy;
+  }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Sum over a 256-thread block; result valid in every thread.
+__device__ __forceinline__ float block_sum(float v, float* smem /* >= 4 floats */) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  const int nw = (blockDim.x + 63) >> 6;
+  for (int i = 0; i < nw; ++i) t += smem[i];
+  return t;
+}
+__device__ __forceinline__ float block_max(float v, float* smem) {
+  v = wave_max(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) smem[wave] = v;
+  __syncthreads();
+  float t = smem[0];
+  const int nw = (blockDim.x + 63) >> 6;
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, smem[i]);
+  return t;
+}
+
+static inline unsigned grid_for(sn_ctx* ctx, int64_t n, int per_block) {
+  int64_t blocks = ceil_div(n, per_block);
+  const int64_t cap = (int64_t)ctx->compute_units * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+// ---------------------------------------------------------------------------- bias + activation
+__global__ __launch_bounds__(256) void bias_act_kernel(const float* __restrict__ x, const float* __restrict__ bias,
+                                                        float* __restrict__ y, int64_t n, int cols, int act, float param) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    float v = x[i];
+    if (bias) v = v + bias[i % cols];  // Bias.scala:32-33
+    y[i] = act_fwd(act, v, param);
+  }
+}
+
+int launch_bias_act(sn_ctx* ctx, const float* x, const float* bias, float* y, int64_t rows, int cols, int act, float act_param) {
+  const int64_t n = rows * cols;
+  if (n <= 0) return SN_OK;
+  LaunchScope scope(ctx, "bias_activation");
+  hipLaunchKernelGGL(bias_act_kernel, dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, bias, y, n, cols, act, act_param);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+__global__ __launch_bounds__(256) void act_bwd_kernel(const float* __restrict__ y, const float* __restrict__ dy,
+                                                       float* __restrict__ dx, int64_t n, int act, float param) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dx[i] = act_bwd(act, y[i], dy[i], param);
+}
+
+int launch_act_bwd(sn_ctx* ctx, const float* y, const float* dy, float* dx, int64_t n, int act, float act_param) {
+  if (n <= 0) return SN_OK;
+  LaunchScope scope(ctx, "activation_backward");
+  hipLaunchKernelGGL(act_bwd_kernel, dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, y, dy, dx, n, act, act_param);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- softmax
+// One 256-thread block per row. p = exp(z) / sum(exp(z)) (Activation.scala:63-69); with
+// `stable` the row maximum is subtracted first (same value in exact arithmetic).
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float* __restrict__ z, float* __restrict__ p, int cols, int stable) {
+  __shared__ float smem[4];
+  const float* zr = z + (int64_t)blockIdx.x * cols;
+  float* pr = p + (int64_t)blockIdx.x * cols;
+  float mx = 0.f;
+  if (stable) {
+    float m = -INFINITY;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) m = fmaxf(m, zr[c]);
+    mx = block_max(m, smem);
+  }
+  float s = 0.f;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float e = expf(zr[c] - mx);
+    pr[c] = e;
+    s += e;
+  }
+  const float total = block_sum(s, smem);
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) pr[c] = pr[c] / total;
+}
+
+int launch_softmax_fwd(sn_ctx* ctx, const float* z, float* p, int rows, int cols, bool stable) {
+  if (rows <= 0) return SN_OK;
+  LaunchScope scope(ctx, "softmax_forward");
+  const int threads = cols <= 64 ? 64 : 256;
+  hipLaunchKernelGGL(softmax_fwd_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, p, cols, stable ? 1 : 0);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// dz_i = p_i * dp_i - p_i * sum_j(p_j * dp_j): the Div/Sum/Exp chain of the reference
+// (AllKernels.scala:196-201,214-227,237-244) with e/S written as p.
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const float* __restrict__ p, const float* __restrict__ dp,
+                                                           float* __restrict__ dz, int cols) {
+  __shared__ float smem[4];
+  const int64_t base = (int64_t)blockIdx.x * cols;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) s += p[base + c] * dp[base + c];
+  const float dot = block_sum(s, smem);
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float pi = p[base + c];
+    dz[base + c] = pi * dp[base + c] - pi * dot;
+  }
+}
+
+int launch_softmax_bwd(sn_ctx* ctx, const float* p, const float* dp, float* dz, int rows, int cols) {
+  if (rows <= 0) return SN_OK;
+  LaunchScope scope(ctx, "softmax_backward");
+  const int threads = cols <= 64 ? 64 : 256;
+  hipLaunchKernelGGL(softmax_bwd_kernel, dim3(rows), dim3(threads), 0, ctx->stream, p, dp, dz, cols);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- losses
+// Stage 1: per-block partial sums of the per-element loss terms and, when dp != null,
+// d loss / d p.  Stage 2 (one block) adds the partials in order and scales.
+//   MSE  (Loss.scala:18-24):  mean((p-y)^2);        dp = ((p-y)*2) * (1/size)
+//   BCE  (Loss.scala:26-42):  mean(-y log(p+e) - (1-y) log(1-(p-e)))
+//   CCE  (Loss.scala:44-57):  -sum(y log(p+e)) / rows;  dp = (y * -(1/rows)) / (p+e)
+constexpr int LOSS_BLOCKS_MAX = 1024;
+
+__global__ __launch_bounds__(256) void loss_stage1_kernel(int kind, const float* __restrict__ p, const float* __restrict__ y,
+                                                           float* __restrict__ dp, float* __restrict__ partials, int64_t n,
+                                                           float inv_size, float neg_inv_rows) {
+  __shared__ float smem[4];
+  const float eps = 1e-8f;
+  float s = 0.f;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const float pi = p[i], yi = y[i];
+    if (kind == SN_LOSS_MSE) {
+      const float d = pi - yi;
+      s += d * d;
+      if (dp) dp[i] = (d * 2.0f) * inv_size;
+    } else if (kind == SN_LOSS_BINARY_CROSSENTROPY) {
+      const float left = yi * logf(pi + eps);
+      const float right = (1.0f - yi) * logf(1.0f - (pi - eps));
+      s += (-left - right);
+      if (dp) {
+        const float g = inv_size;
+        const float dl = (yi * (-g)) / (pi + eps);
+        const float dr = -(((1.0f - yi) * (-g)) / (1.0f - (pi - eps)));
+        dp[i] = dl + dr;
+      }
+    } else if (kind == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
+      s += yi * logf(pi + eps);
+      if (dp) dp[i] = (yi * neg_inv_rows) / (pi + eps);
+    } else {  // identity: the prediction is the loss (Loss.scala:10-14); callers guarantee n == 1
+      s += pi;
+      if (dp) dp[i] = 1.0f;
+    }
+  }
+  const float t = block_sum(s, smem);
+  if (threadIdx.x == 0) partials[blockIdx.x] = t;
+}
+
+__global__ __launch_bounds__(256) void loss_stage2_kernel(int kind, const float* __restrict__ partials, int n_partials,
+                                                           float* __restrict__ loss, float inv_size, float rows) {
+  __shared__ float smem[4];
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n_partials; i += blockDim.x) s += partials[i];
+  const float t = block_sum(s, smem);
+  if (threadIdx.x == 0) {
+    if (kind == SN_LOSS_CATEGORICAL_CROSSENTROPY) *loss = (-t) / rows;
+    else if (kind == SN_LOSS_IDENTITY) *loss = t;
+    else *loss = t * inv_size;
+  }
+}
+
+int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp, float* loss_dev, float* partials, int rows,
+                int cols) {
+  const int64_t n = (int64_t)rows * cols;
+  SN_REQUIRE(n > 0, "loss over an empty batch");
+  const unsigned blocks = (unsigned)std::min<int64_t>(LOSS_BLOCKS_MAX, std::max<int64_t>(1, ceil_div(n, 2048)));
+  const float inv_size = 1.0f / (float)n;
+  const float neg_inv_rows = -(1.0f / (float)rows);
+  {
+    LaunchScope scope(ctx, "loss_stage1");
+    hipLaunchKernelGGL(loss_stage1_kernel, dim3(blocks), dim3(256), 0, ctx->stream, kind, p, y, dp, partials, n, inv_size,
+                       neg_inv_rows);
+  }
+  {
+    LaunchScope scope(ctx, "loss_stage2");
+    hipLaunchKernelGGL(loss_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, kind, partials, (int)blocks, loss_dev, inv_size,
+                       (float)rows);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- column sums (bias gradient)
+// out[c] = sum_r dy[r, c] (Plus's gradient: Sum over the broadcast axes, AllKernels.scala:21-31).
+// A block owns 64 columns; its 4 waves stride over the rows; partial sums meet in LDS.
+__global__ __launch_bounds__(256) void col_sum_kernel(const float* __restrict__ dy, int64_t ld, float* __restrict__ out, int64_t rows,
+                                                       int cols) {
+  __shared__ float smem[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  float s = 0.f;
+  if (c < cols)
+    for (int64_t r = wave; r < rows; r += 4) s += dy[r * ld + c];
+  smem[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < cols) out[c] = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
+}
+
+// Many rows: the rows are cut into gridDim.y slices that write partial sums, which a second
+// launch of col_sum_kernel adds up in slice order (deterministic, no atomics).
+__global__ __launch_bounds__(256) void col_sum_split_kernel(const float* __restrict__ dy, int64_t ld, float* __restrict__ part,
+                                                             int64_t rows, int cols, int64_t rows_per_slice) {
+  __shared__ float smem[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
+  const int64_t r1 = r0 + rows_per_slice < rows ? r0 + rows_per_slice : rows;
+  float s = 0.f;
+  if (c < cols)
+    for (int64_t r = r0 + wave; r < r1; r += 4) s += dy[r * ld + c];
+  smem[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < cols) part[(int64_t)blockIdx.y * cols + c] = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
+}
+
+int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems) {
+  if (cols <= 0) return SN_OK;
+  const unsigned col_blocks = (unsigned)ceil_div(cols, 64);
+  int64_t slices = 1;
+  if (rows >= 512 && ws) {
+    slices = std::min<int64_t>(ceil_div(rows, 128), ceil_div((int64_t)ctx->compute_units * 4, col_blocks));
+    slices = std::min<int64_t>(slices, ws_elems / cols);
+    if (slices < 1) slices = 1;
+  }
+  LaunchScope scope(ctx, "bias_gradient");
+  if (slices <= 1) {
+    hipLaunchKernelGGL(col_sum_kernel, dim3(col_blocks), dim3(256), 0, ctx->stream, dy, ld, out, rows, cols);
+  } else {
+    const int64_t per = ceil_div(rows, slices);
+    slices = ceil_div(rows, per);
+    hipLaunchKernelGGL(col_sum_split_kernel, dim3(col_blocks, (unsigned)slices), dim3(256), 0, ctx->stream, dy, ld, ws, rows, cols, per);
+    hipLaunchKernelGGL(col_sum_kernel, dim3(col_blocks), dim3(256), 0, ctx->stream, (const float*)ws, (int64_t)cols, out, slices, cols);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- regularisation
+// L2: lambda * sum(w^2) / 2 ; L1: lambda * sum(|w|) / 2 (Regularization.scala:30-44); added to *loss.
+__global__ __launch_bounds__(256) void penalty_kernel(const float* __restrict__ w, int64_t n, int reg, float lambda, float* loss) {
+  __shared__ float smem[4];
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += reg == SN_REG_L2 ? w[i] * w[i] : fabsf(w[i]);
+  const float t = block_sum(s, smem);
+  if (threadIdx.x == 0) *loss = *loss + (lambda * t) / 2.0f;
+}
+
+int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev) {
+  LaunchScope scope(ctx, "penalty");
+  hipLaunchKernelGGL(penalty_kernel, dim3(1), dim3(256), 0, ctx->stream, w, n, reg_kind, lambda, loss_dev);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// d penalty / d w: L2 through Pow's gradient (w*2)*(lambda/2); L1 through Abs's gradient, which in
+// the reference is |parent| = lambda/2 for every element (AllKernels.scala:330-335).
+__global__ __launch_bounds__(256) void penalty_grad_kernel(const float* __restrict__ w, float* __restrict__ g, int64_t n, int reg,
+                                                            float lambda) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const float half = lambda / 2.0f;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    g[i] = g[i] + (reg == SN_REG_L2 ? (w[i] * 2.0f) * half : fabsf(half));
+}
+
+int launch_penalty_grad(sn_ctx* ctx, const float* w, float* g, int64_t n, int reg_kind, float lambda) {
+  if (n <= 0) return SN_OK;
+  LaunchScope scope(ctx, "penalty_gradient");
+  hipLaunchKernelGGL(penalty_grad_kernel, dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, w, g, n, reg_kind, lambda);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- accuracy count
+// rows where every rint(p) equals y (estimators/package.scala:28-32); rintf rounds half to even.
+__global__ __launch_bounds__(256) void count_correct_kernel(const float* __restrict__ p, const float* __restrict__ y, int rows,
+                                                             int cols, unsigned long long* count) {
+  __shared__ float smem[4];
+  float local = 0.f;
+  for (int r = blockIdx.x * blockDim.x + threadIdx.x; r < rows; r += gridDim.x * blockDim.x) {
+    int matched = 0;
+    for (int c = 0; c < cols; ++c) matched += (y[(int64_t)r * cols + c] == rintf(p[(int64_t)r * cols + c])) ? 1 : 0;
+    local += matched == cols ? 1.f : 0.f;
+  }
+  const float t = block_sum(local, smem);  // exact: at most 2^24 rows per block
+  if (threadIdx.x == 0 && t > 0.f) atomicAdd(count, (unsigned long long)t);
+}
+
+int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, int cols, unsigned long long* count_dev) {
+  if (rows <= 0) return SN_OK;
+  LaunchScope scope(ctx, "count_correct");
+  hipLaunchKernelGGL(count_correct_kernel, dim3(grid_for(ctx, rows, 256)), dim3(256), 0, ctx->stream, p, y, rows, cols, count_dev);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- max pooling (NHWC)
+// Forward keeps, per output element, the window offset (r*kw + q) of the first maximum in
+// row-major window order; padding cells never win (TF MaxPoolV2, math/nn/AllKernels.scala:270-303).
+__global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
+                                                           int n, int h, int w, int c, int ho, int wo, int kh, int kw, int sh,
+                                                           int sw, int pt, int pl) {
+  const int64_t total = (int64_t)n * ho * wo * c;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int ch = (int)(i % c);
+    int64_t t = i / c;
+    const int ow = (int)(t % wo); t /= wo;
+    const int oh = (int)(t % ho);
+    const int b = (int)(t / ho);
+    float best = -INFINITY;
+    int at = 0;
+    for (int r = 0; r < kh; ++r) {
+      const int iy = oh * sh - pt + r;
+      if (iy < 0 || iy >= h) continue;
+      for (int q = 0; q < kw; ++q) {
+        const int ix = ow * sw - pl + q;
+        if (ix < 0 || ix >= w) continue;
+        const float v = x[(((int64_t)b * h + iy) * w + ix) * c + ch];
+        if (v > best) { best = v; at = r * kw + q; }
+      }
+    }
+    y[i] = best;
+    arg[i] = (uint8_t)at;
+  }
+}
+
+int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo, int kh,
+                       int kw, int sh, int sw, int pt, int pl) {
+  const int64_t total = (int64_t)n * ho * wo * c;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "maxpool_forward");
+  hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(ctx, total, 512)), dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo,
+                     kh, kw, sh, sw, pt, pl);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// Backward as a gather: each input element adds the gradients of the windows whose recorded
+// first maximum is this element (TF MaxPoolGradV2, math/nn/AllKernels.scala:305-324). No atomics.
+__global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
+                                                           float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo,
+                                                           int kh, int kw, int sh, int sw, int pt, int pl) {
+  const int64_t total = (int64_t)n * h * w * c;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int ch = (int)(i % c);
+    int64_t t = i / c;
+    const int ix = (int)(t % w); t /= w;
+    const int iy = (int)(t % h);
+    const int b = (int)(t / h);
+    float s = 0.f;
+    // windows (oh, ow) with oh*sh - pt <= iy < oh*sh - pt + kh
+    int oh_lo = iy + pt - kh + 1;
+    oh_lo = oh_lo <= 0 ? 0 : (oh_lo + sh - 1) / sh;
+    int oh_hi = (iy + pt) / sh;
+    if (oh_hi > ho - 1) oh_hi = ho - 1;
+    int ow_lo = ix + pl - kw + 1;
+    ow_lo = ow_lo <= 0 ? 0 : (ow_lo + sw - 1) / sw;
+    int ow_hi = (ix + pl) / sw;
+    if (ow_hi > wo - 1) ow_hi = wo - 1;
+    for (int oh = oh_lo; oh <= oh_hi; ++oh) {
+      const int r = iy - (oh * sh - pt);
+      for (int ow = ow_lo; ow <= ow_hi; ++ow) {
+        const int q = ix - (ow * sw - pl);
+        const int64_t o = (((int64_t)b * ho + oh) * wo + ow) * c + ch;
+        if (arg[o] == (uint8_t)(r * kw + q)) s += dy[o];
+      }
+    }
+    dx[i] = s;
+  }
+}
+
+int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho, int wo,
+                       int kh, int kw, int sh, int sw, int pt, int pl) {
+  const int64_t total = (int64_t)n * h * w * c;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "maxpool_backward");
+  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(ctx, total, 512)), dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho,
+                     wo, kh, kw, sh, sw, pt, pl);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- LSTM gate maths
+// c = c_prev * f + i * g ; h = o * tanh(c) (layer/RNN.scala:336-337), gates f,i,o = sigmoid, g = tanh.
+__global__ __launch_bounds__(256) void lstm_gates_fwd_kernel(LstmGateArgs a, int rows, int hidden) {
+  const int64_t total = (int64_t)rows * hidden;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / hidden;
+    const int u = (int)(i % hidden);
+    const int64_t zb = r * 4 * hidden + u;
+    const float f = sigmoidf_(a.z[zb]);
+    const float in = sigmoidf_(a.z[zb + hidden]);
+    const float g = tanhf(a.z[zb + 2 * hidden]);
+    const float o = sigmoidf_(a.z[zb + 3 * hidden]);
+    const float cp = a.c_prev ? a.c_prev[i] : 0.f;
+    const float c = cp * f + in * g;
+    a.gates[zb] = f;
+    a.gates[zb + hidden] = in;
+    a.gates[zb + 2 * hidden] = g;
+    a.gates[zb + 3 * hidden] = o;
+    a.c[i] = c;
+    a.h[i] = o * tanhf(c);
+  }
+}
+
+int launch_lstm_gates_fwd(sn_ctx* ctx, const LstmGateArgs& a, int rows, int hidden) {
+  const int64_t total = (int64_t)rows * hidden;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "lstm_gates_forward");
+  hipLaunchKernelGGL(lstm_gates_fwd_kernel, dim3(grid_for(ctx, total, 256)), dim3(256), 0, ctx->stream, a, rows, hidden);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// Reverse of the step above, by the reference's local gradient rules:
+//   do = dh * tanh(c);  dc += (1 - tanh(c)^2) * (dh * o)
+//   df = dc * c_prev;   di = dc * g;   dg = dc * i;   dc_prev = dc * f
+//   dz_gate = act'(z_gate) * d_gate  (sigmoid: s(1-s), tanh: 1 - g^2)
+__global__ __launch_bounds__(256) void lstm_gates_bwd_kernel(LstmGateBwdArgs a, int rows, int hidden) {
+  const int64_t total = (int64_t)rows * hidden;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / hidden;
+    const int u = (int)(i % hidden);
+    const int64_t zb = r * 4 * hidden + u;
+    const float f = a.gates[zb], in = a.gates[zb + hidden], g = a.gates[zb + 2 * hidden], o = a.gates[zb + 3 * hidden];
+    const float tc = tanhf(a.c[i]);
+    const float dh = a.dh[i];
+    const float d_o = dh * tc;
+    float dc = a.dc_is_zero ? 0.f : a.dc[i];
+    dc = dc + (1.0f - tc * tc) * (dh * o);
+    const float cp = a.c_prev ? a.c_prev[i] : 0.f;
+    const float df = dc * cp, di = dc * g, dg = dc * in;
+    a.dc[i] = dc * f;
+    a.dz[zb] = (f * (1.0f - f)) * df;
+    a.dz[zb + hidden] = (in * (1.0f - in)) * di;
+    a.dz[zb + 2 * hidden] = (1.0f - g * g) * dg;
+    a.dz[zb + 3 * hidden] = (o * (1.0f - o)) * d_o;
+  }
+}
+
+int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden) {
+  const int64_t total = (int64_t)rows * hidden;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "lstm_gates_backward");
+  hipLaunchKernelGGL(lstm_gates_bwd_kernel, dim3(grid_for(ctx, total, 256)), dim3(256), 0, ctx->stream, a, rows, hidden);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+}  // namespace sn

@@ -1,0 +1,617 @@
+// MFMA GEMM family for gfx950: one LDS-tiled kernel template whose operand tiles are
+// gathered by small "loader" functors, so the same matrix-core inner loop serves
+//   - Dense forward / dX / dW (strided operands: NN, NT, TN),
+//   - Conv2D forward, input gradient and filter gradient as implicit GEMMs over NHWC,
+//   - the LSTM step (4-gate GEMM over [x_t, h_{t-1}]), its dh/dx and its weight gradients.
+// fp32 path: v_mfma_f32_32x32x2_f32.  bf16 path (Dense, on request): operands are rounded to
+// bf16 while they are staged into LDS and multiplied with v_mfma_f32_32x32x16_bf16, fp32 accumulate.
+//
+// Block = 256 threads = 4 wavefronts in a 2x2 arrangement; block tile BM x BN (64 or 128 each),
+// K step 16; each wavefront owns (BM/2) x (BN/2) as 32x32 MFMA tiles.  Small-output problems
+// are split along K over gridDim.z; partial tiles go to a workspace and a second kernel adds
+// them in split order (deterministic) and applies the epilogue.
+#include "common.hpp"
+
+namespace sn {
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int BK = 16;
+constexpr int THREADS = 256;
+
+// ============================================================================ loaders
+// A loader describes one operand as a function (outer index, k) -> value, where the outer
+// index is the row m of A or the column n of B.  K_CONTIG tells the tile copy which index
+// should run fastest across lanes so that global loads coalesce.
+//   Cursor   per-element state
+//   init     position a cursor at (outer, k)
+//   load     value at the cursor (0 outside the matrix or past k_end)
+//   advance  move the cursor dk along k
+
+template <bool KC>
+struct StridedLoader {
+  static constexpr bool K_CONTIG = KC;
+  const float* p;
+  int64_t s_outer, s_k;
+  int outer_n;
+  struct Cursor {
+    const float* ptr;
+    int k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int outer, int k) const {
+    c.ptr = outer < outer_n ? p + (int64_t)outer * s_outer : nullptr;
+    c.k = k;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    return (c.ptr && c.k < k_end) ? c.ptr[(int64_t)c.k * s_k] : 0.f;
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+};
+
+// ---- Conv2D forward: A(m,k) = x[b, oh*sh-pt+r, ow*sw-pl+q, ci], m=(b,oh,ow), k=(r,q,ci)
+struct ConvFwdA {
+  static constexpr bool K_CONTIG = true;
+  const float* x;
+  ConvGeom g;
+  int M;
+  struct Cursor {
+    const float* img;  // x + b*h*w*cin, null when the row is outside the matrix
+    int iy0, ix0, r, q, ci, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int m, int k) const {
+    c.k = k;
+    if (m >= M) { c.img = nullptr; c.iy0 = c.ix0 = c.r = c.q = c.ci = 0; return; }
+    const int ow = m % g.wo;
+    const int t = m / g.wo;
+    const int oh = t % g.ho;
+    const int b = t / g.ho;
+    c.img = x + (int64_t)b * g.h * g.w * g.cin;
+    c.iy0 = oh * g.sh - g.pt;
+    c.ix0 = ow * g.sw - g.pl;
+    c.ci = k % g.cin;
+    const int rq = k / g.cin;
+    c.q = rq % g.kw;
+    c.r = rq / g.kw;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (!c.img || c.k >= k_end) return 0.f;
+    const int iy = c.iy0 + c.r, ix = c.ix0 + c.q;
+    if (iy < 0 || iy >= g.h || ix < 0 || ix >= g.w) return 0.f;
+    return c.img[((int64_t)iy * g.w + ix) * g.cin + c.ci];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const {
+    c.k += dk;
+    c.ci += dk;
+    while (c.ci >= g.cin) {
+      c.ci -= g.cin;
+      if (++c.q == g.kw) { c.q = 0; ++c.r; }
+    }
+  }
+};
+
+// ---- Conv2D input gradient: dx[b,iy,ix,ci] = sum_{r,q,co} dy[b,(iy+pt-r)/sh,(ix+pl-q)/sw,co] * w[r,q,ci,co]
+struct ConvDgradA {  // m=(b,iy,ix), k=(r,q,co)
+  static constexpr bool K_CONTIG = true;
+  const float* dy;
+  ConvGeom g;
+  int M;
+  struct Cursor {
+    const float* img;  // dy + b*ho*wo*cout
+    int ty, tx, r, q, co, k;  // ty = iy + pt, tx = ix + pl
+  };
+  __device__ __forceinline__ void init(Cursor& c, int m, int k) const {
+    c.k = k;
+    if (m >= M) { c.img = nullptr; c.ty = c.tx = c.r = c.q = c.co = 0; return; }
+    const int ix = m % g.w;
+    const int t = m / g.w;
+    const int iy = t % g.h;
+    const int b = t / g.h;
+    c.img = dy + (int64_t)b * g.ho * g.wo * g.cout;
+    c.ty = iy + g.pt;
+    c.tx = ix + g.pl;
+    c.co = k % g.cout;
+    const int rq = k / g.cout;
+    c.q = rq % g.kw;
+    c.r = rq / g.kw;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (!c.img || c.k >= k_end) return 0.f;
+    const int ny = c.ty - c.r, nx = c.tx - c.q;
+    if (ny < 0 || nx < 0) return 0.f;
+    const int oy = ny / g.sh, ox = nx / g.sw;
+    if (oy * g.sh != ny || ox * g.sw != nx || oy >= g.ho || ox >= g.wo) return 0.f;
+    return c.img[((int64_t)oy * g.wo + ox) * g.cout + c.co];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const {
+    c.k += dk;
+    c.co += dk;
+    while (c.co >= g.cout) {
+      c.co -= g.cout;
+      if (++c.q == g.kw) { c.q = 0; ++c.r; }
+    }
+  }
+};
+
+struct ConvDgradB {  // outer n = ci, k=(r,q,co): w[((r*kw+q)*cin + ci)*cout + co]
+  static constexpr bool K_CONTIG = true;
+  const float* w;
+  ConvGeom g;
+  struct Cursor {
+    int ci, rq, co, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int n, int k) const {
+    c.k = k;
+    c.ci = n < g.cin ? n : -1;
+    c.co = k % g.cout;
+    c.rq = k / g.cout;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.ci < 0 || c.k >= k_end) return 0.f;
+    return w[((int64_t)c.rq * g.cin + c.ci) * g.cout + c.co];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const {
+    c.k += dk;
+    c.co += dk;
+    while (c.co >= g.cout) { c.co -= g.cout; ++c.rq; }
+  }
+};
+
+// ---- Conv2D filter gradient: dw[r,q,ci,co] = sum_{b,oh,ow} x[b,oh*sh-pt+r,ow*sw-pl+q,ci] * dy[b,oh,ow,co]
+struct ConvWgradA {  // m=(r,q,ci) (ci fastest -> contiguous), k=(b,oh,ow)
+  static constexpr bool K_CONTIG = false;
+  const float* x;
+  ConvGeom g;
+  int M;
+  struct Cursor {
+    int r, q, ci;  // ci < 0: row outside the matrix
+    int b, oh, ow, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int m, int k) const {
+    c.k = k;
+    if (m >= M) { c.ci = -1; c.r = c.q = 0; }
+    else {
+      c.ci = m % g.cin;
+      const int rq = m / g.cin;
+      c.q = rq % g.kw;
+      c.r = rq / g.kw;
+    }
+    c.ow = k % g.wo;
+    const int t = k / g.wo;
+    c.oh = t % g.ho;
+    c.b = t / g.ho;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.ci < 0 || c.k >= k_end) return 0.f;
+    const int iy = c.oh * g.sh - g.pt + c.r, ix = c.ow * g.sw - g.pl + c.q;
+    if (iy < 0 || iy >= g.h || ix < 0 || ix >= g.w) return 0.f;
+    return x[(((int64_t)c.b * g.h + iy) * g.w + ix) * g.cin + c.ci];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const {
+    c.k += dk;
+    c.ow += dk;
+    while (c.ow >= g.wo) {
+      c.ow -= g.wo;
+      if (++c.oh == g.ho) { c.oh = 0; ++c.b; }
+    }
+  }
+};
+
+// ---- LSTM step: A(m,k) = k < F ? x[m, t, k] : h_prev[m, k-F]
+struct LstmZA {
+  static constexpr bool K_CONTIG = true;
+  const float* x;       // [rows, T, F]
+  const float* h_prev;  // [rows, H] or null (zeros)
+  int rows, T, F, H, t;
+  struct Cursor {
+    int m, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int m, int k) const { c.m = m < rows ? m : -1; c.k = k; }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.m < 0 || c.k >= k_end) return 0.f;
+    if (c.k < F) return x[((int64_t)c.m * T + t) * F + c.k];
+    return h_prev ? h_prev[(int64_t)c.m * H + (c.k - F)] : 0.f;
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+};
+
+// B(k,n) with n = gate*H + u: k < F ? Wk_gate[k, u] : Wr_gate[k-F, u]
+struct LstmZB {
+  static constexpr bool K_CONTIG = false;
+  LstmWeights w;
+  int F, H;
+  struct Cursor {
+    const float* wk;  // column base inside the gate's kernel matrix, null outside
+    const float* wr;
+    int k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int n, int k) const {
+    c.k = k;
+    if (n >= 4 * H) { c.wk = c.wr = nullptr; return; }
+    const int gate = n / H, u = n % H;
+    c.wk = w.wk[gate] + u;
+    c.wr = w.wr[gate] + u;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (!c.wk || c.k >= k_end) return 0.f;
+    return c.k < F ? c.wk[(int64_t)c.k * H] : c.wr[(int64_t)(c.k - F) * H];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+};
+
+// B(k,n) = W_gate[n, u], k = gate*H + u (transposed gate weights: dh = dz Wr^T, dx = dz Wk^T)
+struct LstmWT {
+  static constexpr bool K_CONTIG = true;
+  const float* w[4];
+  int n_rows, H;  // W_gate is [n_rows, H]
+  struct Cursor {
+    int n, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int n, int k) const { c.n = n < n_rows ? n : -1; c.k = k; }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.n < 0 || c.k >= k_end) return 0.f;
+    const int gate = c.k / H, u = c.k - gate * H;
+    return w[gate][(int64_t)c.n * H + u];
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+};
+
+// Weight gradients of all steps at once: A(m,k), k = t*rows + b:
+//   m < F: x[b, t, m];  F <= m < F+H: h_{t-1}[b, m-F];  m == F+H: 1 (bias row)
+struct LstmWgradA {
+  static constexpr bool K_CONTIG = false;
+  const float* x;           // [rows, T, F]
+  const float* h_prev_all;  // [T, rows, H], slice t holds h_{t-1}
+  int rows, T, F, H, M;
+  struct Cursor {
+    int m, t, b, k;
+  };
+  __device__ __forceinline__ void init(Cursor& c, int m, int k) const {
+    c.m = m < M ? m : -1;
+    c.k = k;
+    c.t = k / rows;
+    c.b = k - c.t * rows;
+  }
+  __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.m < 0 || c.k >= k_end) return 0.f;
+    if (c.m < F) return x[((int64_t)c.b * T + c.t) * F + c.m];
+    if (c.m < F + H) return h_prev_all[((int64_t)c.t * rows + c.b) * H + (c.m - F)];
+    return 1.0f;
+  }
+  __device__ __forceinline__ void advance(Cursor& c, int dk) const {
+    c.k += dk;
+    c.b += dk;
+    while (c.b >= rows) { c.b -= rows; ++c.t; }
+  }
+};
+
+// ============================================================================ epilogues
+__device__ __forceinline__ float ep_act(int act, float v, float param) {
+  switch (act) {
+    case SN_ACT_SIGMOID: return 1.0f / (1.0f + expf(-v));
+    case SN_ACT_TANH: return tanhf(v);
+    case SN_ACT_RELU: return fmaxf(param, v);
+    default: return v;
+  }
+}
+
+struct StdEpilogue {
+  Epilogue e;
+  __device__ __forceinline__ void store(int m, int n, float acc) const {
+    float v = acc;
+    if (e.bias) v = v + e.bias[n];
+    e.out[(int64_t)m * e.ldo + n] = ep_act(e.act, v, e.act_param);
+  }
+};
+
+struct LstmZEpilogue {  // z[m, n] = acc + b_gate[u]
+  float* z;
+  const float* b[4];
+  int H;
+  __device__ __forceinline__ void store(int m, int n, float acc) const {
+    const int gate = n / H, u = n - gate * H;
+    float v = acc;
+    if (b[gate]) v = v + b[gate][u];
+    z[(int64_t)m * 4 * H + n] = v;
+  }
+};
+
+struct LstmWgradEpilogue {  // rows: F kernel rows, H recurrent rows, 1 bias row; columns gate*H + u
+  LstmGrads g;
+  int F, H;
+  __device__ __forceinline__ void store(int m, int n, float acc) const {
+    const int gate = n / H, u = n - gate * H;
+    if (m < F) g.wk[gate][(int64_t)m * H + u] = acc;
+    else if (m < F + H) g.wr[gate][(int64_t)(m - F) * H + u] = acc;
+    else if (g.b[gate]) g.b[gate][u] = acc;
+  }
+};
+
+struct DxScatterEpilogue {  // dx[m, t, n] of a [rows, T, F] tensor
+  float* dx;
+  int T, F, t;
+  __device__ __forceinline__ void store(int m, int n, float acc) const { dx[((int64_t)m * T + t) * F + n] = acc; }
+};
+
+// ============================================================================ the kernel
+template <bool KC, int BT>
+__device__ __forceinline__ int lds_index(int outer, int k) {
+  // K-contiguous operands are staged as [outer][BK+1], the others as [BK][BT+1]; either way
+  // both the staging writes and the MFMA operand reads are free of systematic bank conflicts.
+  return KC ? outer * (BK + 1) + k : k * (BT + 1) + outer;
+}
+
+template <bool BF16>
+struct LdsElem { typedef float type; };
+template <>
+struct LdsElem<true> { typedef __bf16 type; };
+
+template <int BM, int BN, bool BF16, class AL, class BL, class EP>
+__global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int k_per_split, AL al, BL bl, EP ep, float* ws) {
+  typedef typename LdsElem<BF16>::type lds_t;
+  constexpr int EA = BM * BK / THREADS, EB = BN * BK / THREADS;
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  __shared__ lds_t As[BM * (BK + 1)];
+  __shared__ lds_t Bs[BN * (BK + 1)];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int k_begin = blockIdx.z * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+
+  typename AL::Cursor ca[EA];
+  typename BL::Cursor cb[EB];
+  int ia[EA], ib[EB];  // LDS slots
+#pragma unroll
+  for (int e = 0; e < EA; ++e) {
+    int mm, kk;
+    if (AL::K_CONTIG) { kk = tid % BK; mm = tid / BK + e * (THREADS / BK); }
+    else { mm = tid % BM; kk = tid / BM + e * (THREADS / BM); }
+    al.init(ca[e], m0 + mm, k_begin + kk);
+    ia[e] = lds_index<AL::K_CONTIG, BM>(mm, kk);
+  }
+#pragma unroll
+  for (int e = 0; e < EB; ++e) {
+    int nn, kk;
+    if (BL::K_CONTIG) { kk = tid % BK; nn = tid / BK + e * (THREADS / BK); }
+    else { nn = tid % BN; kk = tid / BN + e * (THREADS / BN); }
+    bl.init(cb[e], n0 + nn, k_begin + kk);
+    ib[e] = lds_index<BL::K_CONTIG, BN>(nn, kk);
+  }
+
+  f16v acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  float ra[EA], rb[EB];
+#pragma unroll
+  for (int e = 0; e < EA; ++e) ra[e] = al.load(ca[e], k_end);
+#pragma unroll
+  for (int e = 0; e < EB; ++e) rb[e] = bl.load(cb[e], k_end);
+
+  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int l32 = lane & 31, lhi = lane >> 5;
+
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+#pragma unroll
+    for (int e = 0; e < EA; ++e) As[ia[e]] = (lds_t)ra[e];
+#pragma unroll
+    for (int e = 0; e < EB; ++e) Bs[ib[e]] = (lds_t)rb[e];
+    __syncthreads();
+    if (k0 + BK < k_end) {  // next tile's global loads fly while this tile is multiplied
+#pragma unroll
+      for (int e = 0; e < EA; ++e) { al.advance(ca[e], BK); ra[e] = al.load(ca[e], k_end); }
+#pragma unroll
+      for (int e = 0; e < EB; ++e) { bl.advance(cb[e], BK); rb[e] = bl.load(cb[e], k_end); }
+    }
+    if constexpr (!BF16) {
+#pragma unroll
+      for (int ks = 0; ks < BK; ks += 2) {
+        const int k = ks + lhi;
+        float av[TM], bv[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[i] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, k)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, k)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+      }
+    } else {
+      // 32x32x16 bf16: lane supplies k = 8*(lane/32) .. +7 of row/col lane%32
+      bf16x8 av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 8; ++v) av[i][v] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 8; ++v) bv[j][v] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // accumulator element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn + j * 32 + l32;
+      if (col >= N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm + i * 32 + (v >> 2) * 8 + lhi * 4 + (v & 3);
+        if (row >= M) continue;
+        if (ws) ws[((int64_t)blockIdx.z * M + row) * N + col] = acc[i][j][v];
+        else ep.store(row, col, acc[i][j][v]);
+      }
+    }
+}
+
+template <class EP>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int M, int N, EP ep) {
+  const int64_t total = (int64_t)M * N;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    float s = ws[i];
+    for (int z = 1; z < splits; ++z) s += ws[(int64_t)z * total + i];
+    ep.store((int)(i / N), (int)(i % N), s);
+  }
+}
+
+// ============================================================================ dispatch
+int64_t gemm_workspace_elems(int m, int n, int k, int cu) {
+  // room for the largest split count the heuristic below may pick
+  const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
+  if (tiles >= cu || k <= 256) return 0;
+  int64_t splits = std::min<int64_t>(ceil_div((int64_t)2 * cu, tiles), std::max<int64_t>(1, k / 128));
+  splits = std::min<int64_t>(splits, 64);
+  return splits * (int64_t)m * n;
+}
+
+template <int BM, int BN, bool BF16, class AL, class BL, class EP>
+static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, const AL& al, const BL& bl, const EP& ep, float* ws,
+                        int64_t ws_elems) {
+  const int64_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
+  int splits = 1;
+  if (tiles < ctx->compute_units && K > 256 && ws) {
+    int64_t s = std::min<int64_t>(ceil_div((int64_t)2 * ctx->compute_units, tiles), std::max<int64_t>(1, K / 128));
+    s = std::min<int64_t>(s, 64);
+    s = std::min<int64_t>(s, ws_elems / ((int64_t)M * N));
+    splits = (int)std::max<int64_t>(1, s);
+  }
+  int k_per_split = (int)align_up(ceil_div(K, splits), BK);
+  splits = (int)ceil_div(K, k_per_split);
+  const dim3 grid((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), (unsigned)splits);
+  {
+    LaunchScope scope(ctx, name);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
+                       splits > 1 ? ws : nullptr);
+  }
+  if (splits > 1) {
+    const int64_t total = (int64_t)M * N;
+    int64_t blocks = std::min<int64_t>(ceil_div(total, 256), (int64_t)ctx->compute_units * 8);
+    LaunchScope scope(ctx, "splitk_reduce");
+    hipLaunchKernelGGL((splitk_reduce_kernel<EP>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, splits, M, N, ep);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+template <bool BF16, class AL, class BL, class EP>
+static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const AL& al, const BL& bl, const EP& ep, float* ws,
+                      int64_t ws_elems) {
+  if (M <= 0 || N <= 0) return SN_OK;
+  SN_REQUIRE(K > 0, "%s: empty reduction dimension", name);
+  const bool big_m = M > 64, big_n = N > 64;
+  if (big_m && big_n) return launch_tiles<128, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
+  if (big_m) return launch_tiles<128, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
+  if (big_n) return launch_tiles<64, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
+  return launch_tiles<64, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
+}
+
+template <bool BF16>
+static int launch_gemm_t(sn_ctx* ctx, const GemmDesc& g, const Epilogue& e, float* ws, int64_t ws_elems) {
+  StdEpilogue ep{e};
+  const char* name = BF16 ? "gemm_bf16" : "gemm_f32";
+  const bool akc = g.a_sk == 1, bkc = g.b_sk == 1 && g.b_sn != 1;
+  if (akc && bkc) {
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
+    return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+  } else if (akc) {
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m};
+    StridedLoader<false> bl{g.b, g.b_sn, g.b_sk, g.n};
+    return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+  } else if (bkc) {
+    StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m};
+    StridedLoader<true> bl{g.b, g.b_sn, g.b_sk, g.n};
+    return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+  }
+  StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
+  return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+}
+
+int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* workspace, int64_t workspace_elems, bool bf16) {
+  SN_REQUIRE(g.a && g.b && ep.out, "gemm: null operand");
+  return bf16 ? launch_gemm_t<true>(ctx, g, ep, workspace, workspace_elems) : launch_gemm_t<false>(ctx, g, ep, workspace, workspace_elems);
+}
+
+// ---------------------------------------------------------------------------- Conv2D
+int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e, float* ws, int64_t ws_elems) {
+  const int M = g.n * g.ho * g.wo, N = g.cout, K = g.kh * g.kw * g.cin;
+  ConvFwdA al{x, g, M};
+  StridedLoader<false> bl{w, 1, (int64_t)g.cout, N};  // filter [kh,kw,cin,cout] is a row-major [K, cout] matrix
+  StdEpilogue ep{e};
+  return launch_any<false>(ctx, "conv2d_forward", M, N, K, al, bl, ep, ws, ws_elems);
+}
+
+int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems) {
+  const int M = g.n * g.h * g.w, N = g.cin, K = g.kh * g.kw * g.cout;
+  ConvDgradA al{dy, g, M};
+  ConvDgradB bl{w, g};
+  Epilogue e;
+  e.out = dx;
+  e.ldo = g.cin;
+  StdEpilogue ep{e};
+  return launch_any<false>(ctx, "conv2d_input_gradient", M, N, K, al, bl, ep, ws, ws_elems);
+}
+
+int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems) {
+  const int M = g.kh * g.kw * g.cin, N = g.cout, K = g.n * g.ho * g.wo;
+  ConvWgradA al{x, g, M};
+  StridedLoader<false> bl{dy, 1, (int64_t)g.cout, N};
+  Epilogue e;
+  e.out = dw;
+  e.ldo = g.cout;
+  StdEpilogue ep{e};
+  return launch_any<false>(ctx, "conv2d_filter_gradient", M, N, K, al, bl, ep, ws, ws_elems);
+}
+
+// ---------------------------------------------------------------------------- LSTM
+int launch_lstm_z(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, int rows, int H, const LstmWeights& w,
+                  float* z, float* ws, int64_t ws_elems) {
+  LstmZA al{x, h_prev, rows, T, F, H, t};
+  LstmZB bl{w, F, H};
+  LstmZEpilogue ep{z, {w.b[0], w.b[1], w.b[2], w.b[3]}, H};
+  return launch_any<false>(ctx, "lstm_gate_gemm", rows, 4 * H, F + H, al, bl, ep, ws, ws_elems);
+}
+
+int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems) {
+  StridedLoader<true> al{dz, (int64_t)4 * H, 1, rows};
+  LstmWT bl{{w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, H, H};
+  Epilogue e;
+  e.out = dh_prev;
+  e.ldo = H;
+  StdEpilogue ep{e};
+  return launch_any<false>(ctx, "lstm_hidden_gradient", rows, H, 4 * H, al, bl, ep, ws, ws_elems);
+}
+
+int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, int T, const LstmWeights& w, float* dx, float* ws,
+                   int64_t ws_elems) {
+  StridedLoader<true> al{dz, (int64_t)4 * H, 1, rows};
+  LstmWT bl{{w.wk[0], w.wk[1], w.wk[2], w.wk[3]}, F, H};
+  DxScatterEpilogue ep{dx, T, F, t};
+  return launch_any<false>(ctx, "lstm_input_gradient", rows, F, 4 * H, al, bl, ep, ws, ws_elems);
+}
+
+int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
+                      const LstmGrads& g, float* ws, int64_t ws_elems) {
+  const bool has_bias = g.b[0] != nullptr;
+  const int M = F + H + (has_bias ? 1 : 0);
+  LstmWgradA al{x, h_prev_all, rows, T, F, H, M};
+  StridedLoader<false> bl{dz_all, 1, (int64_t)4 * H, 4 * H};
+  LstmWgradEpilogue ep{g, F, H};
+  return launch_any<false>(ctx, "lstm_weight_gradient", M, 4 * H, T * rows, al, bl, ep, ws, ws_elems);
+}
+
+}  // namespace sn

@@ -1,0 +1,839 @@
+// Host side of the compiled step: turns the flattened layer list into a plan of fused
+// operations over a flat parameter buffer, and runs forward / loss / backward / update,
+// the per-partition epoch loop and the replica average.
+//
+// Correspondence with the reference (paths under src/main/scala/scanet/):
+//   plan building ........ models/layer/Composed.scala:22-53 (parameter paths, layer order)
+//   sn_step .............. optimizers/Optimizer.scala:169-194 (compileBackprop)
+//   sn_train_epoch ....... optimizers/Optimizer.scala:106-161 (optimizeOnPartition)
+//   sn_replicas_average .. optimizers/Optimizer.scala:196-230 (aggregateParams)
+#include "common.hpp"
+
+#include <algorithm>
+#include <cmath>
+
+namespace sn {
+
+enum OpKind { OP_DENSE, OP_CONV, OP_POOL, OP_FLATTEN, OP_BIASACT, OP_SOFTMAX, OP_LSTM };
+
+struct ParamDef {
+  sn_param_info info;
+  int reg_kind = SN_REG_NONE;
+  float reg_lambda = 0.f;
+};
+
+struct Op {
+  OpKind kind;
+  std::vector<int64_t> in_dims, out_dims;  // per sample
+  int64_t in_elems = 0, out_elems = 0;     // per sample
+  int w = -1, b = -1;                      // parameter indices
+  int act = SN_ACT_IDENTITY;
+  float act_param = 0.f;
+  // conv / pool geometry (per sample: h, w, c)
+  int kh = 0, kw = 0, sh = 1, sw = 1, pt = 0, pl = 0;
+  // lstm
+  int T = 0, F = 0, H = 0;
+  int lstm_p[4][3] = {{-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}};  // gate x {kernel, recurrent, bias}
+  // buffers (indices into replica buffer table), assigned at replica creation
+  int out_buf = -1;
+};
+
+}  // namespace sn
+
+struct sn_model {
+  uint32_t magic;
+  sn_ctx* ctx;
+  int loss;
+  uint32_t flags;
+  int batch;
+  std::vector<int64_t> input_dims;
+  int64_t in_elems;
+  std::vector<sn::Op> ops;
+  std::vector<sn::ParamDef> params;
+  int64_t flat_elems;  // padded length of the flat parameter buffer
+  std::vector<int64_t> out_dims;
+  int64_t out_elems;
+  int64_t max_act_elems;   // per sample, over every op input/output
+  int64_t workspace_elems;
+  int live_replicas;
+};
+
+struct sn_replica {
+  uint32_t magic;
+  sn_model* model;
+  sn_ctx* ctx;
+  bool has_opt;
+  sn_optimizer_desc opt;
+  int n_states;
+  float* w = nullptr;
+  float* g = nullptr;
+  float* s[SN_MAX_OPT_STATES] = {nullptr, nullptr, nullptr};
+  std::vector<float*> act;      // per op output (null for views)
+  std::vector<uint8_t*> arg;    // per op: max-pool argmax
+  float* grad_buf[2] = {nullptr, nullptr};
+  float* ws = nullptr;
+  float* loss_dev = nullptr;
+  float* loss_partials = nullptr;
+  unsigned long long* count_dev = nullptr;
+  // lstm scratch (one set, shared by every LSTM op; sized for the largest)
+  float* lstm_z = nullptr;
+  std::vector<float*> lstm_gates, lstm_c, lstm_h, lstm_dz;  // per op
+  float* lstm_dh[2] = {nullptr, nullptr};
+  float* lstm_dc = nullptr;
+  std::vector<void*> owned;
+};
+
+namespace sn {
+
+static int check_model(sn_model* m) {
+  if (!m || m->magic != MODEL_MAGIC) return fail(SN_E_STATE, "invalid or destroyed model handle");
+  return SN_OK;
+}
+static int check_replica(sn_replica* r) {
+  if (!r || r->magic != REPLICA_MAGIC) return fail(SN_E_STATE, "invalid or destroyed replica handle");
+  return SN_OK;
+}
+
+static int64_t prod(const std::vector<int64_t>& d) {
+  int64_t p = 1;
+  for (auto v : d) p *= v;
+  return p;
+}
+
+// Padding.size / TensorFlow's SAME rule (math/nn/AllKernels.scala:39-65): extra padding goes after.
+static void conv_out(int padding, int in, int k, int s, int* out, int* pad_before) {
+  if (padding == SN_PAD_SAME) {
+    *out = (in + s - 1) / s;
+    const int total = std::max((*out - 1) * s + k - in, 0);
+    *pad_before = total / 2;
+  } else {
+    *out = (in - k + 1 + s - 1) / s;  // ceil((in - k + 1) / s)
+    *pad_before = 0;
+  }
+}
+
+static int add_param(sn_model* m, const std::string& path, const std::vector<int64_t>& dims, int reg_kind, float reg_lambda) {
+  ParamDef p;
+  memset(&p.info, 0, sizeof(p.info));
+  snprintf(p.info.path, sizeof(p.info.path), "%s", path.c_str());
+  p.info.rank = (int32_t)dims.size();
+  p.info.size = 1;
+  for (size_t i = 0; i < dims.size(); ++i) {
+    p.info.dims[i] = dims[i];
+    p.info.size *= dims[i];
+  }
+  p.info.offset = m->flat_elems;
+  p.reg_kind = reg_kind;
+  p.reg_lambda = reg_lambda;
+  m->flat_elems += align_up(p.info.size, 64);  // every tensor starts on a 256-byte boundary
+  m->params.push_back(p);
+  return (int)m->params.size() - 1;
+}
+
+static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
+  std::vector<int64_t> cur = m->input_dims;
+  const bool single = n_layers == 1;  // Composed(single) is the layer itself: no index prefix (Composed.scala:95-98)
+  auto prefix = [&](int i) { return single ? std::string() : std::to_string(i) + "/"; };
+  int64_t max_act = prod(cur);
+  int64_t ws = 0;
+  const int cu = m->ctx->compute_units;
+  const int B = m->batch;
+  int i = 0;
+  while (i < n_layers) {
+    const sn_layer_desc& L = layers[i];
+    Op op;
+    op.in_dims = cur;
+    op.in_elems = prod(cur);
+    switch (L.kind) {
+      case SN_LAYER_DENSE: {
+        SN_REQUIRE(cur.size() == 1, "layer %d: Dense expects a (batch, features) input, got rank %zu (add Flatten)", i, cur.size() + 1);
+        SN_REQUIRE(L.units > 0, "layer %d: Dense needs units > 0", i);
+        op.kind = OP_DENSE;
+        op.w = add_param(m, prefix(i) + "weights", {cur[0], L.units}, L.reg_kind, L.reg_lambda);
+        op.out_dims = {L.units};
+        ++i;
+        if (i < n_layers && layers[i].kind == SN_LAYER_BIAS) {
+          SN_REQUIRE(layers[i].units == L.units, "layer %d: Bias has %d features, input has %d", i, layers[i].units, L.units);
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda);
+          ++i;
+        }
+        if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
+          op.act = layers[i].activation;
+          op.act_param = layers[i].act_param;
+          ++i;
+        }
+        const int in_f = (int)cur[0], out_f = L.units;
+        ws = std::max(ws, gemm_workspace_elems(B, out_f, in_f, cu));
+        ws = std::max(ws, gemm_workspace_elems(in_f, out_f, B, cu));
+        ws = std::max(ws, gemm_workspace_elems(B, in_f, out_f, cu));
+        break;
+      }
+      case SN_LAYER_CONV2D: {
+        SN_REQUIRE(cur.size() == 3, "layer %d: Conv2D input should have a shape (NHWC) but was rank %zu", i, cur.size() + 1);
+        SN_REQUIRE(L.units > 0 && L.kernel_h > 0 && L.kernel_w > 0 && L.stride_h > 0 && L.stride_w > 0,
+                   "layer %d: Conv2D needs positive filters, kernel and strides", i);
+        SN_REQUIRE(L.padding == SN_PAD_VALID || L.padding == SN_PAD_SAME, "layer %d: unknown padding %d", i, L.padding);
+        op.kind = OP_CONV;
+        op.kh = L.kernel_h; op.kw = L.kernel_w; op.sh = L.stride_h; op.sw = L.stride_w;
+        int ho, wo;
+        conv_out(L.padding, (int)cur[0], op.kh, op.sh, &ho, &op.pt);
+        conv_out(L.padding, (int)cur[1], op.kw, op.sw, &wo, &op.pl);
+        SN_REQUIRE(ho > 0 && wo > 0, "layer %d: Conv2D kernel larger than its input", i);
+        op.w = add_param(m, prefix(i) + "weights", {op.kh, op.kw, cur[2], L.units}, SN_REG_NONE, 0.f);
+        op.out_dims = {ho, wo, L.units};
+        ++i;
+        if (i < n_layers && layers[i].kind == SN_LAYER_BIAS) {
+          SN_REQUIRE(layers[i].units == L.units, "layer %d: Bias has %d features, input has %d", i, layers[i].units, L.units);
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda);
+          ++i;
+        }
+        if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
+          op.act = layers[i].activation;
+          op.act_param = layers[i].act_param;
+          ++i;
+        }
+        const int64_t K = (int64_t)op.kh * op.kw * cur[2];
+        ws = std::max(ws, gemm_workspace_elems(B * ho * wo, L.units, (int)K, cu));
+        ws = std::max(ws, gemm_workspace_elems((int)K, L.units, B * ho * wo, cu));
+        ws = std::max(ws, gemm_workspace_elems(B * (int)cur[0] * (int)cur[1], (int)cur[2], op.kh * op.kw * L.units, cu));
+        break;
+      }
+      case SN_LAYER_POOL2D: {
+        SN_REQUIRE(cur.size() == 3, "layer %d: Pool2D input should have a shape (NHWC) but was rank %zu", i, cur.size() + 1);
+        SN_REQUIRE(L.kernel_h > 0 && L.kernel_w > 0 && L.stride_h > 0 && L.stride_w > 0 && L.kernel_h * L.kernel_w <= 255,
+                   "layer %d: Pool2D needs a positive window (at most 255 cells) and strides", i);
+        SN_REQUIRE(L.padding == SN_PAD_VALID || L.padding == SN_PAD_SAME, "layer %d: only [Same, Valid] paddings are supported", i);
+        op.kind = OP_POOL;
+        op.kh = L.kernel_h; op.kw = L.kernel_w; op.sh = L.stride_h; op.sw = L.stride_w;
+        int ho, wo;
+        conv_out(L.padding, (int)cur[0], op.kh, op.sh, &ho, &op.pt);
+        conv_out(L.padding, (int)cur[1], op.kw, op.sw, &wo, &op.pl);
+        SN_REQUIRE(ho > 0 && wo > 0, "layer %d: Pool2D window larger than its input", i);
+        op.out_dims = {ho, wo, cur[2]};
+        ++i;
+        break;
+      }
+      case SN_LAYER_FLATTEN: {
+        SN_REQUIRE(cur.size() >= 1, "layer %d: rank should be >= 2", i);
+        op.kind = OP_FLATTEN;
+        op.out_dims = {prod(cur)};
+        ++i;
+        break;
+      }
+      case SN_LAYER_BIAS:
+      case SN_LAYER_ACTIVATE: {
+        op.out_dims = cur;
+        if (L.kind == SN_LAYER_ACTIVATE && L.activation == SN_ACT_SOFTMAX) {
+          SN_REQUIRE(cur.size() == 1, "layer %d: Softmax expects a (batch, classes) input", i);
+          op.kind = OP_SOFTMAX;
+          ++i;
+          break;
+        }
+        op.kind = OP_BIASACT;
+        if (L.kind == SN_LAYER_BIAS) {
+          SN_REQUIRE(L.units == cur.back(), "layer %d: Bias has %d features, input has %lld", i, L.units, (long long)cur.back());
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, L.reg_kind, L.reg_lambda);
+          ++i;
+          if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
+            op.act = layers[i].activation;
+            op.act_param = layers[i].act_param;
+            ++i;
+          }
+        } else {
+          SN_REQUIRE(L.activation >= SN_ACT_IDENTITY && L.activation <= SN_ACT_RELU, "layer %d: unknown activation %d", i, L.activation);
+          op.act = L.activation;
+          op.act_param = L.act_param;
+          ++i;
+        }
+        break;
+      }
+      case SN_LAYER_LSTM: {
+        SN_REQUIRE(cur.size() == 2, "layer %d: RNN requires input to have Shape(batch, time, features)", i);
+        SN_REQUIRE(L.units > 0, "layer %d: RNN Cell should contain at least one unit", i);
+        SN_REQUIRE(L.activation == SN_ACT_TANH || L.activation == SN_ACT_IDENTITY,
+                   "layer %d: only the default LSTM activations (tanh cell, sigmoid gates) are built", i);
+        op.kind = OP_LSTM;
+        op.T = (int)cur[0]; op.F = (int)cur[1]; op.H = L.units;
+        static const char* gates[4] = {"forget", "input", "gate", "output"};  // layer/RNN.scala:285-289
+        for (int gi = 0; gi < 4; ++gi) {
+          const std::string gp = prefix(i) + gates[gi];
+          op.lstm_p[gi][0] = add_param(m, gp + "/0/kernel_weights", {op.F, op.H}, SN_REG_NONE, 0.f);
+          op.lstm_p[gi][1] = add_param(m, gp + "/0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
+          if (L.use_bias) op.lstm_p[gi][2] = add_param(m, gp + "/1/weights", {op.H}, SN_REG_NONE, 0.f);
+        }
+        op.out_dims = {L.units};
+        ws = std::max(ws, gemm_workspace_elems(B, 4 * op.H, op.F + op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(B, op.H, 4 * op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(B, op.F, 4 * op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(op.F + op.H + 1, 4 * op.H, op.T * B, cu));
+        ++i;
+        break;
+      }
+      default:
+        return fail(SN_E_INVALID, "layer %d: unknown layer kind %d", i, L.kind);
+    }
+    op.out_elems = prod(op.out_dims);
+    max_act = std::max(max_act, op.out_elems);
+    cur = op.out_dims;
+    m->ops.push_back(op);
+  }
+  m->out_dims = cur;
+  m->out_elems = prod(cur);
+  m->max_act_elems = max_act;
+  // column sums over many rows use the workspace too
+  ws = std::max<int64_t>(ws, (int64_t)cu * 4 * 64 * 4);
+  m->workspace_elems = ws;
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- replica memory
+template <class T>
+static int dev_alloc(sn_replica* r, T** out, int64_t elems) {
+  *out = nullptr;
+  if (elems <= 0) return SN_OK;
+  void* p = nullptr;
+  SN_HIP(hipMalloc(&p, (size_t)elems * sizeof(T)));
+  r->owned.push_back(p);
+  *out = (T*)p;
+  return SN_OK;
+}
+
+static float* param_ptr(sn_replica* r, float* base, int idx) { return idx < 0 ? nullptr : base + r->model->params[idx].info.offset; }
+
+static int alloc_replica(sn_replica* r) {
+  sn_model* m = r->model;
+  const int64_t B = m->batch;
+  SN_HIP(hipSetDevice(r->ctx->device));
+  SN_TRY(dev_alloc(r, &r->w, m->flat_elems));
+  SN_TRY(dev_alloc(r, &r->g, m->flat_elems));
+  SN_TRY(launch_fill(r->ctx, r->w, 0.f, m->flat_elems));
+  SN_TRY(launch_fill(r->ctx, r->g, 0.f, m->flat_elems));
+  for (int s = 0; s < r->n_states; ++s) {
+    SN_TRY(dev_alloc(r, &r->s[s], m->flat_elems));
+    SN_TRY(launch_fill(r->ctx, r->s[s], r->opt.init_acc, m->flat_elems));
+  }
+  const size_t n_ops = m->ops.size();
+  r->act.assign(n_ops, nullptr);
+  r->arg.assign(n_ops, nullptr);
+  r->lstm_gates.assign(n_ops, nullptr);
+  r->lstm_c.assign(n_ops, nullptr);
+  r->lstm_h.assign(n_ops, nullptr);
+  r->lstm_dz.assign(n_ops, nullptr);
+  int64_t lstm_z = 0, lstm_h = 0;
+  for (size_t i = 0; i < n_ops; ++i) {
+    const Op& op = m->ops[i];
+    if (op.kind == OP_FLATTEN) continue;  // a view of its input
+    if (op.kind == OP_LSTM) {
+      const int64_t bh = B * op.H;
+      SN_TRY(dev_alloc(r, &r->lstm_gates[i], (int64_t)op.T * bh * 4));
+      SN_TRY(dev_alloc(r, &r->lstm_c[i], (int64_t)op.T * bh));
+      SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = h_{-1}
+      SN_TRY(dev_alloc(r, &r->lstm_dz[i], (int64_t)op.T * bh * 4));
+      SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
+      lstm_z = std::max(lstm_z, bh * 4);
+      lstm_h = std::max(lstm_h, bh);
+      continue;  // output = last slice of lstm_h
+    }
+    SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
+    if (op.kind == OP_POOL) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
+  }
+  SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
+  SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h));
+  SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h));
+  SN_TRY(dev_alloc(r, &r->lstm_dc, lstm_h));
+  SN_TRY(dev_alloc(r, &r->grad_buf[0], B * m->max_act_elems));
+  SN_TRY(dev_alloc(r, &r->grad_buf[1], B * m->max_act_elems));
+  SN_TRY(dev_alloc(r, &r->ws, m->workspace_elems));
+  SN_TRY(dev_alloc(r, &r->loss_dev, 1));
+  SN_TRY(dev_alloc(r, &r->loss_partials, 1024));
+  SN_TRY(dev_alloc(r, &r->count_dev, 1));
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- forward
+static const float* op_output(sn_replica* r, int i, const float* x, int rows) {
+  // output pointer of op i (x for i == -1)
+  if (i < 0) return x;
+  const Op& op = r->model->ops[i];
+  if (op.kind == OP_FLATTEN) return op_output(r, i - 1, x, rows);
+  if (op.kind == OP_LSTM) return r->lstm_h[i] + (int64_t)op.T * r->model->batch * op.H;
+  return r->act[i];
+}
+
+static LstmWeights lstm_weights(sn_replica* r, const Op& op, float* base) {
+  LstmWeights w;
+  for (int gi = 0; gi < 4; ++gi) {
+    w.wk[gi] = param_ptr(r, base, op.lstm_p[gi][0]);
+    w.wr[gi] = param_ptr(r, base, op.lstm_p[gi][1]);
+    w.b[gi] = param_ptr(r, base, op.lstm_p[gi][2]);
+  }
+  return w;
+}
+
+static int forward(sn_replica* r, const float* x, int rows) {
+  sn_model* m = r->model;
+  sn_ctx* ctx = r->ctx;
+  const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
+  for (size_t i = 0; i < m->ops.size(); ++i) {
+    const Op& op = m->ops[i];
+    const float* in = op_output(r, (int)i - 1, x, rows);
+    switch (op.kind) {
+      case OP_DENSE: {
+        const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
+        GemmDesc g{in, in_f, 1, param_ptr(r, r->w, op.w), out_f, 1, rows, out_f, in_f};
+        Epilogue ep;
+        ep.out = r->act[i]; ep.ldo = out_f; ep.bias = param_ptr(r, r->w, op.b); ep.act = op.act; ep.act_param = op.act_param;
+        SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
+        break;
+      }
+      case OP_CONV: {
+        ConvGeom g{rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2], (int)op.out_dims[0], (int)op.out_dims[1],
+                   (int)op.out_dims[2], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl};
+        Epilogue ep;
+        ep.out = r->act[i]; ep.ldo = g.cout; ep.bias = param_ptr(r, r->w, op.b); ep.act = op.act; ep.act_param = op.act_param;
+        SN_TRY(launch_conv_fwd(ctx, g, in, param_ptr(r, r->w, op.w), ep, r->ws, m->workspace_elems));
+        break;
+      }
+      case OP_POOL:
+        SN_TRY(launch_maxpool_fwd(ctx, in, r->act[i], r->arg[i], rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
+                                  (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl));
+        break;
+      case OP_FLATTEN:
+        break;
+      case OP_BIASACT:
+        SN_TRY(launch_bias_act(ctx, in, param_ptr(r, r->w, op.b), r->act[i], (int64_t)rows * (op.out_elems / op.out_dims.back()),
+                               (int)op.out_dims.back(), op.act, op.act_param));
+        break;
+      case OP_SOFTMAX:
+        SN_TRY(launch_softmax_fwd(ctx, in, r->act[i], rows, (int)op.out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+        break;
+      case OP_LSTM: {
+        // time-major slices are laid out with the model's batch capacity so addresses do not depend on `rows`
+        const int64_t bh = (int64_t)m->batch * op.H;
+        const LstmWeights w = lstm_weights(r, op, r->w);
+        for (int t = 0; t < op.T; ++t) {
+          const float* h_prev = r->lstm_h[i] + (int64_t)t * bh;
+          SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, rows, op.H, w, r->lstm_z, r->ws, m->workspace_elems));
+          LstmGateArgs a{r->lstm_z, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, r->lstm_gates[i] + (int64_t)t * bh * 4,
+                         r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
+          SN_TRY(launch_lstm_gates_fwd(ctx, a, rows, op.H));
+        }
+        break;
+      }
+    }
+  }
+  return SN_OK;
+}
+
+// loss (+ penalty) into loss_dev; dp (may be null) receives d loss / d prediction
+static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp) {
+  sn_model* m = r->model;
+  if (m->loss == SN_LOSS_IDENTITY)
+    SN_REQUIRE((int64_t)rows * m->out_elems == 1, "Identity loss needs a scalar model output");
+  SN_TRY(launch_loss(r->ctx, m->loss, pred, y, dp, r->loss_dev, r->loss_partials, rows, (int)m->out_elems));
+  for (auto& p : m->params)
+    if (p.reg_kind != SN_REG_NONE)
+      SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev));
+  return SN_OK;
+}
+
+// ---------------------------------------------------------------------------- backward
+static int backward(sn_replica* r, const float* x, int rows) {
+  sn_model* m = r->model;
+  sn_ctx* ctx = r->ctx;
+  const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
+  int cur = 0;  // grad_buf[cur] holds d loss / d (output of op i)
+  for (int i = (int)m->ops.size() - 1; i >= 0; --i) {
+    const Op& op = m->ops[i];
+    const float* in = op_output(r, i - 1, x, rows);
+    float* dy = r->grad_buf[cur];
+    float* dx = r->grad_buf[cur ^ 1];
+    const bool need_dx = i > 0;
+    switch (op.kind) {
+      case OP_DENSE: {
+        const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
+        if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
+        if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
+        {  // dW = X^T . dY (math/alg/AllKernels.scala:382-388)
+          GemmDesc g{in, 1, in_f, dy, out_f, 1, in_f, out_f, rows};
+          Epilogue ep;
+          ep.out = param_ptr(r, r->g, op.w); ep.ldo = out_f;
+          SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
+        }
+        if (need_dx) {  // dX = dY . W^T
+          GemmDesc g{dy, out_f, 1, param_ptr(r, r->w, op.w), 1, out_f, rows, in_f, out_f};
+          Epilogue ep;
+          ep.out = dx; ep.ldo = in_f;
+          SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
+          cur ^= 1;
+        }
+        break;
+      }
+      case OP_CONV: {
+        ConvGeom g{rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2], (int)op.out_dims[0], (int)op.out_dims[1],
+                   (int)op.out_dims[2], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl};
+        const int64_t n_out = (int64_t)rows * op.out_elems;
+        if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
+        if (op.b >= 0)
+          SN_TRY(launch_col_sum(ctx, dy, g.cout, param_ptr(r, r->g, op.b), (int64_t)rows * g.ho * g.wo, g.cout, r->ws, m->workspace_elems));
+        SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems));
+        if (need_dx) {
+          SN_TRY(launch_conv_dgrad(ctx, g, dy, param_ptr(r, r->w, op.w), dx, r->ws, m->workspace_elems));
+          cur ^= 1;
+        }
+        break;
+      }
+      case OP_POOL:
+        if (need_dx) {
+          SN_TRY(launch_maxpool_bwd(ctx, dy, r->arg[i], dx, rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
+                                    (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl));
+          cur ^= 1;
+        }
+        break;
+      case OP_FLATTEN:
+        break;
+      case OP_BIASACT: {
+        const int cols = (int)op.out_dims.back();
+        const int64_t n_out = (int64_t)rows * op.out_elems;
+        if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
+        if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, cols, param_ptr(r, r->g, op.b), n_out / cols, cols, r->ws, m->workspace_elems));
+        break;
+      }
+      case OP_SOFTMAX:
+        SN_TRY(launch_softmax_bwd(ctx, r->act[i], dy, dx, rows, (int)op.out_elems));
+        cur ^= 1;
+        break;
+      case OP_LSTM: {
+        // the weight-gradient GEMM reads the saved steps as one [T*rows, .] matrix, so the slices must be full
+        SN_REQUIRE(rows == m->batch, "LSTM training needs rows == batch (%d), got %d", m->batch, rows);
+        const int64_t bh = (int64_t)m->batch * op.H;
+        const LstmWeights w = lstm_weights(r, op, r->w);
+        const float* dh = dy;  // gradient of the last hidden state
+        int hb = 0;
+        for (int t = op.T - 1; t >= 0; --t) {
+          LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
+                            t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
+                            r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0};
+          SN_TRY(launch_lstm_gates_bwd(ctx, a, rows, op.H));
+          if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
+          if (t > 0) {
+            SN_TRY(launch_lstm_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], r->ws, m->workspace_elems));
+            dh = r->lstm_dh[hb];
+            hb ^= 1;
+          }
+        }
+        LstmGrads gr;
+        for (int gi = 0; gi < 4; ++gi) {
+          gr.wk[gi] = param_ptr(r, r->g, op.lstm_p[gi][0]);
+          gr.wr[gi] = param_ptr(r, r->g, op.lstm_p[gi][1]);
+          gr.b[gi] = param_ptr(r, r->g, op.lstm_p[gi][2]);
+        }
+        SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems));
+        if (need_dx) cur ^= 1;
+        break;
+      }
+    }
+  }
+  for (auto& p : m->params)
+    if (p.reg_kind != SN_REG_NONE)
+      SN_TRY(launch_penalty_grad(ctx, r->w + p.info.offset, r->g + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda));
+  return SN_OK;
+}
+
+static int check_rows(sn_replica* r, int rows) {
+  SN_REQUIRE(rows >= 1 && rows <= r->model->batch, "rows must be in 1..%d (the model's batch), got %d", r->model->batch, rows);
+  return SN_OK;
+}
+
+static int read_loss(sn_replica* r, float* loss_host) {
+  if (!loss_host) return SN_OK;
+  SN_HIP(hipMemcpyAsync(loss_host, r->loss_dev, sizeof(float), hipMemcpyDeviceToHost, r->ctx->stream));
+  SN_HIP(hipStreamSynchronize(r->ctx->stream));
+  return SN_OK;
+}
+
+static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
+  SN_TRY(forward(r, x, rows));
+  const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);
+  SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0]));
+  SN_TRY(backward(r, x, rows));
+  return SN_OK;
+}
+
+static int update(sn_replica* r, int iter) {
+  SN_REQUIRE(r->has_opt, "replica was created without an optimizer");
+  return launch_optimizer(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], r->model->flat_elems, iter);
+}
+
+static int tensor_io(sn_replica* r, float* base, int index, float* host, const float* src, int64_t n) {
+  sn_model* m = r->model;
+  SN_REQUIRE(index >= 0 && index < (int)m->params.size(), "parameter index %d out of range (model has %zu)", index, m->params.size());
+  const sn_param_info& p = m->params[index].info;
+  SN_REQUIRE(n == p.size, "parameter %s holds %lld elements, caller passed %lld", p.path, (long long)p.size, (long long)n);
+  SN_REQUIRE(base != nullptr, "replica has no such buffer");
+  if (src) {
+    SN_HIP(hipMemcpyAsync(base + p.offset, src, (size_t)n * sizeof(float), hipMemcpyHostToDevice, r->ctx->stream));
+    SN_HIP(hipStreamSynchronize(r->ctx->stream));  // the caller may reuse `src` right away
+  } else {
+    SN_HIP(hipMemcpyAsync(host, base + p.offset, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, r->ctx->stream));
+    SN_HIP(hipStreamSynchronize(r->ctx->stream));
+  }
+  return SN_OK;
+}
+
+}  // namespace sn
+
+using namespace sn;
+
+extern "C" {
+
+int sn_model_create(sn_ctx* ctx, const sn_layer_desc* layers, int32_t n_layers, int32_t loss, const int64_t* input_dims,
+                    int32_t input_rank, int32_t batch, uint32_t flags, sn_model** out) {
+  SN_REQUIRE(out != nullptr, "sn_model_create: out is NULL");
+  *out = nullptr;
+  if (!ctx || ctx->magic != CTX_MAGIC) return fail(SN_E_STATE, "invalid or destroyed context handle");
+  SN_REQUIRE(layers && n_layers >= 1, "at least 1 layer is required");
+  SN_REQUIRE(loss >= SN_LOSS_IDENTITY && loss <= SN_LOSS_CATEGORICAL_CROSSENTROPY, "unknown loss %d", loss);
+  SN_REQUIRE(input_dims && input_rank >= 1 && input_rank < SN_MAX_RANK, "input rank must be in 1..%d", SN_MAX_RANK - 1);
+  SN_REQUIRE(batch >= 1, "batch must be positive");
+  sn_model* m = new sn_model();
+  m->magic = MODEL_MAGIC;
+  m->ctx = ctx;
+  m->loss = loss;
+  m->flags = flags;
+  m->batch = batch;
+  m->flat_elems = 0;
+  m->live_replicas = 0;
+  for (int i = 0; i < input_rank; ++i) {
+    if (input_dims[i] < 1) {
+      delete m;
+      return fail(SN_E_INVALID, "input dimension %d must be positive", i);
+    }
+    m->input_dims.push_back(input_dims[i]);
+  }
+  m->in_elems = prod(m->input_dims);
+  int rc = build_plan(m, layers, n_layers);
+  if (rc == SN_OK && (int64_t)batch * m->max_act_elems > (int64_t)INT32_MAX)
+    rc = fail(SN_E_INVALID, "batch x largest activation exceeds 2^31 elements");
+  if (rc != SN_OK) {
+    delete m;
+    return rc;
+  }
+  *out = m;
+  return SN_OK;
+}
+
+int sn_model_destroy(sn_model* model) {
+  SN_TRY(check_model(model));
+  SN_REQUIRE(model->live_replicas == 0, "model still has %d live replicas", model->live_replicas);
+  model->magic = 0;
+  delete model;
+  return SN_OK;
+}
+
+int sn_model_param_count(sn_model* model, int32_t* n_tensors, int64_t* flat_elems) {
+  SN_TRY(check_model(model));
+  if (n_tensors) *n_tensors = (int32_t)model->params.size();
+  if (flat_elems) *flat_elems = model->flat_elems;
+  return SN_OK;
+}
+
+int sn_model_param_info(sn_model* model, int32_t index, sn_param_info* out) {
+  SN_TRY(check_model(model));
+  SN_REQUIRE(out != nullptr, "sn_model_param_info: out is NULL");
+  SN_REQUIRE(index >= 0 && index < (int32_t)model->params.size(), "parameter index %d out of range", index);
+  *out = model->params[index].info;
+  return SN_OK;
+}
+
+int sn_model_output_shape(sn_model* model, int32_t* rank, int64_t* dims) {
+  SN_TRY(check_model(model));
+  if (rank) *rank = (int32_t)model->out_dims.size();
+  if (dims)
+    for (size_t i = 0; i < model->out_dims.size(); ++i) dims[i] = model->out_dims[i];
+  return SN_OK;
+}
+
+int sn_replica_create(sn_model* model, const sn_optimizer_desc* opt, sn_replica** out) {
+  SN_REQUIRE(out != nullptr, "sn_replica_create: out is NULL");
+  *out = nullptr;
+  SN_TRY(check_model(model));
+  sn_replica* r = new sn_replica();
+  r->magic = REPLICA_MAGIC;
+  r->model = model;
+  r->ctx = model->ctx;
+  r->has_opt = opt != nullptr;
+  r->n_states = 0;
+  if (opt) {
+    r->opt = *opt;
+    r->n_states = opt_state_count(opt->kind);
+    if (r->n_states < 0) {
+      delete r;
+      return fail(SN_E_INVALID, "unknown optimizer kind %d", opt->kind);
+    }
+  }
+  int rc = alloc_replica(r);
+  if (rc != SN_OK) {
+    for (void* p : r->owned) (void)hipFree(p);
+    delete r;
+    return rc;
+  }
+  model->live_replicas++;
+  *out = r;
+  return SN_OK;
+}
+
+int sn_replica_destroy(sn_replica* rep) {
+  SN_TRY(check_replica(rep));
+  (void)hipStreamSynchronize(rep->ctx->stream);
+  for (void* p : rep->owned) (void)hipFree(p);
+  rep->model->live_replicas--;
+  rep->magic = 0;
+  delete rep;
+  return SN_OK;
+}
+
+int sn_params_set(sn_replica* rep, int32_t index, const float* src_host, int64_t n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(src_host != nullptr, "sn_params_set: source is NULL");
+  return tensor_io(rep, rep->w, index, nullptr, src_host, n);
+}
+int sn_params_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(dst_host != nullptr, "sn_params_get: destination is NULL");
+  return tensor_io(rep, rep->w, index, dst_host, nullptr, n);
+}
+int sn_optstate_set(sn_replica* rep, int32_t index, int32_t slot, const float* src_host, int64_t n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(src_host != nullptr, "sn_optstate_set: source is NULL");
+  SN_REQUIRE(slot >= 0 && slot < rep->n_states, "optimizer has %d state tensors per weight, slot %d asked", rep->n_states, slot);
+  return tensor_io(rep, rep->s[slot], index, nullptr, src_host, n);
+}
+int sn_optstate_get(sn_replica* rep, int32_t index, int32_t slot, float* dst_host, int64_t n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(dst_host != nullptr, "sn_optstate_get: destination is NULL");
+  SN_REQUIRE(slot >= 0 && slot < rep->n_states, "optimizer has %d state tensors per weight, slot %d asked", rep->n_states, slot);
+  return tensor_io(rep, rep->s[slot], index, dst_host, nullptr, n);
+}
+int sn_grads_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(dst_host != nullptr, "sn_grads_get: destination is NULL");
+  return tensor_io(rep, rep->g, index, dst_host, nullptr, n);
+}
+
+int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(out_dev != nullptr, "sn_replica_flat: out is NULL");
+  SN_REQUIRE(slot >= -2 && slot < rep->n_states, "slot %d out of range", slot);
+  *out_dev = slot == -2 ? rep->w : (slot == -1 ? rep->g : rep->s[slot]);
+  if (n) *n = rep->model->flat_elems;
+  return SN_OK;
+}
+
+int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev, "sn_step: null batch pointer");
+  SN_TRY(check_rows(rep, rows));
+  SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
+  SN_REQUIRE(rep->has_opt, "replica was created without an optimizer");
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows));
+  SN_TRY(update(rep, iter));
+  return read_loss(rep, loss_host);
+}
+
+int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev, "sn_grad: null batch pointer");
+  SN_TRY(check_rows(rep, rows));
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows));
+  return read_loss(rep, loss_host);
+}
+
+int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && out_dev, "sn_forward: null pointer");
+  SN_TRY(check_rows(rep, rows));
+  SN_TRY(forward(rep, x_dev, rows));
+  const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
+  SN_HIP(hipMemcpyAsync(out_dev, pred, (size_t)rows * rep->model->out_elems * sizeof(float), hipMemcpyDeviceToDevice, rep->ctx->stream));
+  return SN_OK;
+}
+
+int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev && loss_host, "sn_loss: null pointer");
+  SN_TRY(check_rows(rep, rows));
+  SN_TRY(forward(rep, x_dev, rows));
+  const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
+  SN_TRY(loss_of(rep, pred, y_dev, rows, nullptr));
+  return read_loss(rep, loss_host);
+}
+
+int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int64_t* count_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev && count_host, "sn_count_correct: null pointer");
+  SN_TRY(check_rows(rep, rows));
+  SN_TRY(forward(rep, x_dev, rows));
+  const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
+  SN_HIP(hipMemsetAsync(rep->count_dev, 0, sizeof(unsigned long long), rep->ctx->stream));
+  const int cols = (int)rep->model->out_dims.back();
+  SN_TRY(launch_count_correct(rep->ctx, pred, y_dev, (int)((int64_t)rows * rep->model->out_elems / cols), cols, rep->count_dev));
+  unsigned long long c = 0;
+  SN_HIP(hipMemcpyAsync(&c, rep->count_dev, sizeof(c), hipMemcpyDeviceToHost, rep->ctx->stream));
+  SN_HIP(hipStreamSynchronize(rep->ctx->stream));
+  *count_host = (int64_t)c;
+  return SN_OK;
+}
+
+int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch, int32_t global_iter,
+                   int32_t* iterations_host, float* loss_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev, "sn_train_epoch: null partition pointer");
+  SN_REQUIRE(batch >= 1 && batch <= rep->model->batch, "batch must be in 1..%d, got %d", rep->model->batch, batch);
+  SN_REQUIRE(global_iter >= 0, "global_iter must not be negative");
+  const int64_t n_batches = total_rows / batch;  // the partial batch is skipped (optimizers/Iterators.scala:90)
+  SN_REQUIRE(n_batches >= 1, "partition of %lld rows holds no full batch of %d (the reference's iterator throws here)",
+             (long long)total_rows, batch);
+  const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
+  for (int64_t i = 0; i < n_batches; ++i) {
+    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch));
+    SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
+  }
+  if (iterations_host) *iterations_host = (int32_t)n_batches;
+  if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
+    const float* xl = x_dev + (n_batches - 1) * xs;
+    const float* yl = y_dev + (n_batches - 1) * ys;
+    SN_TRY(forward(rep, xl, batch));
+    const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, xl, batch);
+    SN_TRY(loss_of(rep, pred, yl, batch, nullptr));
+    SN_TRY(read_loss(rep, loss_host));
+  }
+  return SN_OK;
+}
+
+int sn_replicas_average(sn_replica* const* reps, int32_t k) {
+  SN_REQUIRE(reps != nullptr, "sn_replicas_average: replica list is NULL");
+  SN_REQUIRE(k >= 1 && k <= SN_MAX_AVG_INPUTS, "sn_replicas_average: k must be in 1..%d, got %d", SN_MAX_AVG_INPUTS, k);
+  for (int i = 0; i < k; ++i) {
+    SN_TRY(check_replica(reps[i]));
+    SN_REQUIRE(reps[i]->model == reps[0]->model, "replica %d belongs to another model", i);
+    SN_REQUIRE(reps[i]->n_states == reps[0]->n_states && (!reps[i]->has_opt || reps[i]->opt.kind == reps[0]->opt.kind),
+               "replica %d uses another optimizer", i);
+  }
+  if (k == 1) return SN_OK;  // treeReduce of one partition never calls aggregateParams
+  sn_ctx* ctx = reps[0]->ctx;
+  const int64_t n = reps[0]->model->flat_elems;
+  for (int slot = -1; slot < reps[0]->n_states; ++slot) {
+    AvgInputs in;
+    float* outs[SN_MAX_AVG_INPUTS];
+    for (int i = 0; i < k; ++i) {
+      float* p = slot < 0 ? reps[i]->w : reps[i]->s[slot];
+      in.p[i] = p;
+      outs[i] = p;
+    }
+    SN_TRY(launch_average(ctx, in, k, n, outs[0], outs + 1, k - 1));
+  }
+  return SN_OK;
+}
+
+}  // extern "C"

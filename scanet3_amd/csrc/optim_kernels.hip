@@ -1,0 +1,316 @@
+// Fused optimizer updates over a flat parameter vector and the K-replica average.
+//
+// Both families are pure streaming kernels: every element is read once and
+// written once, so the bound is HBM bandwidth.  Bytes per element:
+//   update:  4 * (2 + 2 * n_state)   (read w, g, states; write w, states)
+//   average: 4 * (K + n_outputs)
+// The arithmetic follows the reference's operation order exactly (one rounding
+// per TensorFlow op, no fused multiply-add), see optimizers/*.scala.
+#include "common.hpp"
+
+#include <cmath>
+
+namespace sn {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter) {
+  OptScalars s;
+  s.rate = d.rate;
+  s.b1 = d.beta1;
+  s.b2 = d.beta2;
+  s.eps = d.epsilon;
+  s.one_minus_b1 = 1.0f - d.beta1;
+  s.one_minus_b2 = 1.0f - d.beta2;
+  // `Pow(rate, iter.cast[Float])` (math/alg/AllKernels.scala:546-549), correctly rounded to float32
+  s.bc1 = 1.0f - (float)std::pow((double)d.beta1, (double)iter);
+  s.bc2 = 1.0f - (float)std::pow((double)d.beta2, (double)iter);
+  s.nesterov = d.nesterov;
+  return s;
+}
+
+int opt_state_count(int kind) {
+  switch (kind) {
+    case SN_OPT_SGD: case SN_OPT_ADAGRAD: case SN_OPT_RMSPROP: return 1;
+    case SN_OPT_ADADELTA: case SN_OPT_ADAM: case SN_OPT_NADAM: case SN_OPT_ADAMAX: return 2;
+    case SN_OPT_AMSGRAD: return 3;
+  }
+  return -1;
+}
+
+// decayingAvg(avg, next, decay) = decay*avg + (1-decay)*next (math/alg/AllKernels.scala:541-544)
+__device__ __forceinline__ float decaying_avg(float avg, float next, float d, float one_minus_d) {
+  return d * avg + one_minus_d * next;
+}
+
+template <int KIND>
+__device__ __forceinline__ void update_one(float& w, float g, float& s0, float& s1, float& s2, const OptScalars& p) {
+  float delta;
+  if constexpr (KIND == SN_OPT_SGD) {  // SGD.scala:15-25
+    float v = (p.rate * g) - (p.b1 * s0);
+    delta = p.nesterov ? (p.rate * g) - (p.b1 * v) : v;
+    s0 = v;
+  } else if constexpr (KIND == SN_OPT_ADAGRAD) {  // AdaGrad.scala:21-32
+    float acc = s0 + g * g;
+    float rates = p.rate / sqrtf(acc + p.eps);
+    delta = rates * g;
+    s0 = acc;
+  } else if constexpr (KIND == SN_OPT_ADADELTA) {  // AdaDelta.scala:33-44
+    float avg_grad = decaying_avg(s0, g * g, p.b1, p.one_minus_b1);
+    delta = p.rate * ((sqrtf(s1 + p.eps) / sqrtf(avg_grad + p.eps)) * g);
+    s1 = decaying_avg(s1, delta * delta, p.b1, p.one_minus_b1);
+    s0 = avg_grad;
+  } else if constexpr (KIND == SN_OPT_RMSPROP) {  // RMSProp.scala:24-32
+    float avg_grad = decaying_avg(s0, g * g, p.b1, p.one_minus_b1);
+    delta = (p.rate / sqrtf(avg_grad + p.eps)) * g;
+    s0 = avg_grad;
+  } else if constexpr (KIND == SN_OPT_ADAM) {  // Adam.scala:29-41
+    float m = decaying_avg(s0, g, p.b1, p.one_minus_b1);
+    float v = decaying_avg(s1, g * g, p.b2, p.one_minus_b2);
+    delta = (p.rate / sqrtf(v / p.bc2 + p.eps)) * (m / p.bc1);
+    s0 = m;
+    s1 = v;
+  } else if constexpr (KIND == SN_OPT_NADAM) {  // Nadam.scala:37-49
+    float m = decaying_avg(s0, g, p.b1, p.one_minus_b1);
+    float v = decaying_avg(s1, g * g, p.b2, p.one_minus_b2);
+    float m_nesterov = (p.b1 * (m / p.bc1)) + (p.one_minus_b1 * (g / p.bc1));
+    delta = m_nesterov / (sqrtf(v / p.bc2) + p.eps);
+    s0 = m;
+    s1 = v;
+  } else if constexpr (KIND == SN_OPT_ADAMAX) {  // Adamax.scala:41-52
+    float m1 = decaying_avg(s0, g, p.b1, p.one_minus_b1);
+    float m2 = fmaxf(p.b2 * s1, p.one_minus_b2 * fabsf(g));
+    delta = (p.rate * (m1 / p.bc1)) / (m2 + p.eps);
+    s0 = m1;
+    s1 = m2;
+  } else {  // AMSGrad.scala:34-46
+    float m = decaying_avg(s0, g, p.b1, p.one_minus_b1);
+    float v_cur = decaying_avg(s1, g * g, p.b2, p.one_minus_b2);
+    float v = fmaxf(s2, v_cur);
+    delta = (p.rate * m) / (sqrtf(v) + p.eps);
+    s0 = m;
+    s1 = v_cur;
+    s2 = v;
+  }
+  w = w - delta;  // Optimizer.scala:186 (minimizing)
+}
+
+template <int KIND>
+constexpr int n_states() {
+  return (KIND == SN_OPT_SGD || KIND == SN_OPT_ADAGRAD || KIND == SN_OPT_RMSPROP) ? 1 : (KIND == SN_OPT_AMSGRAD ? 3 : 2);
+}
+
+// One float4 per lane per iteration, UNROLL independent iterations in flight.
+template <int KIND, int UNROLL>
+__global__ __launch_bounds__(256) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
+                                                            f4* __restrict__ s1, f4* __restrict__ s2, int64_t n4,
+                                                            OptScalars p) {
+  constexpr int NS = n_states<KIND>();
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
+    f4 vw[UNROLL], vg[UNROLL], a[UNROLL], b[UNROLL], c[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t j = i + u * stride;
+      vw[u] = __builtin_nontemporal_load(w + j);
+      vg[u] = __builtin_nontemporal_load(g + j);
+      a[u] = __builtin_nontemporal_load(s0 + j);
+      if (NS > 1) b[u] = __builtin_nontemporal_load(s1 + j);
+      if (NS > 2) c[u] = __builtin_nontemporal_load(s2 + j);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t j = i + u * stride;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float ww = vw[u][e], aa = a[u][e], bb = NS > 1 ? b[u][e] : 0.f, cc = NS > 2 ? c[u][e] : 0.f;
+        update_one<KIND>(ww, vg[u][e], aa, bb, cc, p);
+        vw[u][e] = ww;
+        a[u][e] = aa;
+        if (NS > 1) b[u][e] = bb;
+        if (NS > 2) c[u][e] = cc;
+      }
+      __builtin_nontemporal_store(vw[u], w + j);
+      __builtin_nontemporal_store(a[u], s0 + j);
+      if (NS > 1) __builtin_nontemporal_store(b[u], s1 + j);
+      if (NS > 2) __builtin_nontemporal_store(c[u], s2 + j);
+    }
+  }
+  for (; i < n4; i += stride) {
+    f4 vw = w[i], vg = g[i], a = s0[i], b = {0, 0, 0, 0}, c = {0, 0, 0, 0};
+    if (NS > 1) b = s1[i];
+    if (NS > 2) c = s2[i];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float ww = vw[e], aa = a[e], bb = b[e], cc = c[e];
+      update_one<KIND>(ww, vg[e], aa, bb, cc, p);
+      vw[e] = ww; a[e] = aa; b[e] = bb; c[e] = cc;
+    }
+    w[i] = vw;
+    s0[i] = a;
+    if (NS > 1) s1[i] = b;
+    if (NS > 2) s2[i] = c;
+  }
+}
+
+// Scalar form for a misaligned buffer or the last n % 4 elements.
+template <int KIND>
+__global__ __launch_bounds__(256) void optimizer_kernel_scalar(float* __restrict__ w, const float* __restrict__ g,
+                                                                float* __restrict__ s0, float* __restrict__ s1,
+                                                                float* __restrict__ s2, int64_t n, OptScalars p) {
+  constexpr int NS = n_states<KIND>();
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    float ww = w[i], aa = s0[i], bb = NS > 1 ? s1[i] : 0.f, cc = NS > 2 ? s2[i] : 0.f;
+    update_one<KIND>(ww, g[i], aa, bb, cc, p);
+    w[i] = ww;
+    s0[i] = aa;
+    if (NS > 1) s1[i] = bb;
+    if (NS > 2) s2[i] = cc;
+  }
+}
+
+static bool aligned16(const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int KIND>
+static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g, float* s0, float* s1, float* s2, int64_t n,
+                        const OptScalars& p) {
+  constexpr int UNROLL = 4;
+  const bool vec = aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2);
+  const int64_t n4 = vec ? n / 4 : 0;
+  if (n4 > 0) {
+    // enough workgroups to cover every CU several times over; each lane keeps UNROLL float4 per array in flight
+    int64_t blocks = ceil_div(n4, (int64_t)256 * UNROLL);
+    const int64_t cap = (int64_t)ctx->compute_units * 16;
+    if (blocks > cap) blocks = cap;
+    LaunchScope scope(ctx, name);
+    hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (f4*)w,
+                       (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p);
+  }
+  const int64_t done = n4 * 4;
+  if (done < n) {
+    const int64_t rest = n - done;
+    int64_t blocks = ceil_div(rest, 256);
+    const int64_t cap = (int64_t)ctx->compute_units * 8;
+    if (blocks > cap) blocks = cap;
+    LaunchScope scope(ctx, name);
+    hipLaunchKernelGGL((optimizer_kernel_scalar<KIND>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w + done, g + done,
+                       s0 + done, s1 ? s1 + done : nullptr, s2 ? s2 + done : nullptr, rest, p);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
+                     int64_t n, int iter) {
+  const int ns = opt_state_count(d.kind);
+  SN_REQUIRE(ns > 0, "unknown optimizer kind %d", d.kind);
+  SN_REQUIRE(w && g && s0 && (ns < 2 || s1) && (ns < 3 || s2), "optimizer kind %d needs %d state buffers", d.kind, ns);
+  SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
+  if (n <= 0) return SN_OK;
+  const OptScalars p = make_opt_scalars(d, iter);
+  switch (d.kind) {
+    case SN_OPT_SGD: return launch_opt_t<SN_OPT_SGD>(ctx, "optimizer_sgd", w, g, s0, s1, s2, n, p);
+    case SN_OPT_ADAGRAD: return launch_opt_t<SN_OPT_ADAGRAD>(ctx, "optimizer_adagrad", w, g, s0, s1, s2, n, p);
+    case SN_OPT_ADADELTA: return launch_opt_t<SN_OPT_ADADELTA>(ctx, "optimizer_adadelta", w, g, s0, s1, s2, n, p);
+    case SN_OPT_RMSPROP: return launch_opt_t<SN_OPT_RMSPROP>(ctx, "optimizer_rmsprop", w, g, s0, s1, s2, n, p);
+    case SN_OPT_ADAM: return launch_opt_t<SN_OPT_ADAM>(ctx, "optimizer_adam", w, g, s0, s1, s2, n, p);
+    case SN_OPT_NADAM: return launch_opt_t<SN_OPT_NADAM>(ctx, "optimizer_nadam", w, g, s0, s1, s2, n, p);
+    case SN_OPT_ADAMAX: return launch_opt_t<SN_OPT_ADAMAX>(ctx, "optimizer_adamax", w, g, s0, s1, s2, n, p);
+    default: return launch_opt_t<SN_OPT_AMSGRAD>(ctx, "optimizer_amsgrad", w, g, s0, s1, s2, n, p);
+  }
+}
+
+// ---- K-replica average --------------------------------------------------------------------
+struct AvgOutputs {
+  float* p[SN_MAX_AVG_INPUTS + 1];
+};
+
+template <int K_STATIC>
+__global__ __launch_bounds__(256) void average_kernel_v4(AvgInputs in, int k, int64_t n4, AvgOutputs out, int n_out, float kf) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+    f4 acc;
+    if constexpr (K_STATIC > 0) {
+      f4 v[K_STATIC];
+#pragma unroll
+      for (int r = 0; r < K_STATIC; ++r) v[r] = __builtin_nontemporal_load((const f4*)in.p[r] + i);
+      acc = v[0];
+#pragma unroll
+      for (int r = 1; r < K_STATIC; ++r) acc = acc + v[r];  // AddN, left to right
+    } else {
+      acc = ((const f4*)in.p[0])[i];
+      for (int r = 1; r < k; ++r) acc = acc + ((const f4*)in.p[r])[i];
+    }
+    acc = acc / kf;  // `plus(inputs) / inputs.size` (models/Aggregation.scala:16-19)
+    for (int o = 0; o < n_out; ++o) __builtin_nontemporal_store(acc, (f4*)out.p[o] + i);
+  }
+}
+
+__global__ __launch_bounds__(256) void average_kernel_scalar(AvgInputs in, int k, int64_t first, int64_t n, AvgOutputs out,
+                                                              int n_out, float kf) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    float acc = in.p[0][i];
+    for (int r = 1; r < k; ++r) acc = acc + in.p[r][i];
+    acc = acc / kf;
+    for (int o = 0; o < n_out; ++o) out.p[o][i] = acc;
+  }
+}
+
+int launch_average(sn_ctx* ctx, const AvgInputs& in, int k, int64_t n, float* out, float* const* extra_out, int n_extra) {
+  SN_REQUIRE(k >= 1 && k <= SN_MAX_AVG_INPUTS, "average takes 1..%d inputs, got %d", SN_MAX_AVG_INPUTS, k);
+  SN_REQUIRE(n_extra >= 0 && n_extra <= SN_MAX_AVG_INPUTS, "too many average outputs");
+  if (n <= 0) return SN_OK;
+  AvgOutputs o;
+  o.p[0] = out;
+  for (int i = 0; i < n_extra; ++i) o.p[i + 1] = extra_out[i];
+  const int n_out = 1 + n_extra;
+  bool vec = aligned16(out);
+  for (int i = 0; i < k; ++i) vec = vec && aligned16(in.p[i]);
+  for (int i = 0; i < n_extra; ++i) vec = vec && aligned16(extra_out[i]);
+  const int64_t n4 = vec ? n / 4 : 0;
+  const float kf = (float)k;
+  if (n4 > 0) {
+    int64_t blocks = ceil_div(n4, 256);
+    const int64_t cap = (int64_t)ctx->compute_units * 16;
+    if (blocks > cap) blocks = cap;
+    LaunchScope scope(ctx, "average_replicas");
+    if (k == 8)
+      hipLaunchKernelGGL((average_kernel_v4<8>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+    else if (k == 4)
+      hipLaunchKernelGGL((average_kernel_v4<4>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+    else if (k == 2)
+      hipLaunchKernelGGL((average_kernel_v4<2>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+    else
+      hipLaunchKernelGGL((average_kernel_v4<0>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+  }
+  if (n4 * 4 < n) {
+    LaunchScope scope(ctx, "average_replicas");
+    int64_t blocks = ceil_div(n - n4 * 4, 256);
+    const int64_t cap = (int64_t)ctx->compute_units * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(average_kernel_scalar, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4 * 4, n, o, n_out, kf);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(float* dst, float v, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = v;
+}
+
+int launch_fill(sn_ctx* ctx, float* dst, float v, int64_t n) {
+  if (n <= 0) return SN_OK;
+  int64_t blocks = ceil_div(n, 256 * 4);
+  const int64_t cap = (int64_t)ctx->compute_units * 8;
+  if (blocks > cap) blocks = cap;
+  LaunchScope scope(ctx, "fill");
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, dst, v, n);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+}  // namespace sn

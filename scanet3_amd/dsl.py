@@ -1,0 +1,530 @@
+"""Host-side mirror of scanet's user-facing training DSL on top of the HIP library.
+
+    model = Dense(50, Sigmoid) >> Dense(10, Softmax)
+    trained = ds.train(model).loss(CategoricalCrossentropy).using(Adam(0.01)).batch(1000).epochs(10).run()
+    accuracy(trained, test_ds)
+
+Names, defaults and semantics follow the reference (paths under src/main/scala/scanet/):
+layers models/layer/*.scala, activations models/Activation.scala, losses models/Loss.scala,
+algorithms optimizers/*.scala, the builder optimizers/Optimizer.scala:267-310, the epoch
+loop optimizers/Optimizer.scala:59-161 and `accuracy` estimators/package.scala:18-47.
+The Spark partitions of the reference become K device-resident replicas that are averaged
+on the GPU after every epoch.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field, replace
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _lib as L
+from .core import CompiledModel, Context, DeviceBuffer, Replica, average_replicas
+
+# --------------------------------------------------------------------------- activations / losses / misc
+
+
+@dataclass(frozen=True)
+class Activation:
+    kind: int
+    param: float = 0.0
+    name: str = ""
+
+    @property
+    def identity(self) -> bool:
+        return self.kind == L.ACT_IDENTITY
+
+    def __repr__(self):
+        return self.name
+
+
+Identity = Activation(L.ACT_IDENTITY, name="Identity")
+Sigmoid = Activation(L.ACT_SIGMOID, name="Sigmoid")
+Tanh = Activation(L.ACT_TANH, name="Tanh")
+Softmax = Activation(L.ACT_SOFTMAX, name="Softmax")
+
+
+def ReLU(threshold: float = 0.0) -> Activation:
+    return Activation(L.ACT_RELU, float(threshold), f"ReLU({float(threshold)})")
+
+
+@dataclass(frozen=True)
+class Loss:
+    kind: int
+    name: str
+
+    def __repr__(self):
+        return self.name
+
+
+MeanSquaredError = Loss(L.LOSS_MSE, "MeanSquaredError")
+BinaryCrossentropy = Loss(L.LOSS_BINARY_CROSSENTROPY, "BinaryCrossentropy")
+CategoricalCrossentropy = Loss(L.LOSS_CATEGORICAL_CROSSENTROPY, "CategoricalCrossentropy")
+IdentityLoss = Loss(L.LOSS_IDENTITY, "Identity")
+
+
+@dataclass(frozen=True)
+class Regularization:
+    kind: int = L.REG_NONE
+    lam: float = 0.0
+
+
+Zero = Regularization()
+
+
+def L1(lam: float = 0.01) -> Regularization:
+    return Regularization(L.REG_L1, lam)
+
+
+def L2(lam: float = 0.01) -> Regularization:
+    return Regularization(L.REG_L2, lam)
+
+
+Valid, Same = L.PAD_VALID, L.PAD_SAME
+_PAD_NAME = {Valid: "Valid", Same: "Same"}
+
+# --------------------------------------------------------------------------- initializers (models/Initializer.scala)
+
+
+def fans(shape: Sequence[int]) -> Tuple[int, int]:
+    """Initializer.fans (Initializer.scala:16-25), including its rank > 2 rule `out :: in :: receptive`."""
+    s = list(shape)
+    if len(s) == 0:
+        return 1, 1
+    if len(s) == 1:
+        return s[0], s[0]
+    if len(s) == 2:
+        return s[0], s[1]
+    size = int(np.prod(s[2:]))
+    return size * s[1], size * s[0]
+
+
+@dataclass(frozen=True)
+class Initializer:
+    """Draws come from numpy, not from TensorFlow's Philox stream: seeded values differ from the
+    reference's; the distributions are the same. Use `.initParams(..)` for bit-identical starts."""
+    name: str
+    value: float = 0.0
+    seed: Optional[int] = None
+
+    def build(self, shape, rng: np.random.Generator) -> np.ndarray:
+        shape = tuple(shape)
+        if self.name == "Zeros":
+            return np.zeros(shape, np.float32)
+        if self.name == "Ones":
+            return np.ones(shape, np.float32)
+        if self.name == "Const":
+            return np.full(shape, self.value, np.float32)
+        r = np.random.default_rng(self.seed) if self.seed is not None else rng
+        if self.name == "GlorotUniform":                      # Initializer.scala:83-90
+            fan_in, fan_out = fans(shape)
+            limit = np.float32(math.sqrt(np.float32(6.0) / (fan_in + fan_out)))
+            return (r.random(shape, np.float32) * (2 * limit) - limit).astype(np.float32)
+        if self.name == "Orthogonal":                         # Initializer.scala:202-219
+            rows, cols = int(np.prod(shape[:-1])), shape[-1]
+            a = r.standard_normal((max(rows, cols), min(rows, cols)))
+            q, rr = np.linalg.qr(a)
+            q = q * np.sign(np.diag(rr))
+            if rows < cols:
+                q = q.T
+            return q.reshape(shape).astype(np.float32)
+        raise ValueError(self.name)
+
+
+Zeros, Ones = Initializer("Zeros"), Initializer("Ones")
+
+
+def Const(v: float) -> Initializer:
+    return Initializer("Const", float(v))
+
+
+def GlorotUniform(seed: Optional[int] = None) -> Initializer:
+    return Initializer("GlorotUniform", seed=seed)
+
+
+def Orthogonal(seed: Optional[int] = None) -> Initializer:
+    return Initializer("Orthogonal", seed=seed)
+
+
+# --------------------------------------------------------------------------- layers
+
+
+@dataclass(frozen=True)
+class Layer:
+    """One primitive layer; `>>` composes (layer/Layer.scala:24-31)."""
+    kind: int
+    text: str
+    units: int = 0
+    activation: Activation = Identity
+    kernel: Tuple[int, int] = (0, 0)
+    strides: Tuple[int, int] = (1, 1)
+    padding: int = Valid
+    reg: Regularization = Zero
+    use_bias: bool = True
+    inits: Tuple[Initializer, ...] = ()
+
+    def __rshift__(self, other):
+        return Composed.of(self, other)
+
+    @property
+    def layers(self) -> List["Layer"]:
+        return [self]
+
+    def desc(self) -> L.LayerDesc:
+        return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
+                           self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0)
+
+    def __repr__(self):
+        return self.text
+
+
+class Composed:
+    """Flattened sequence of layers (layer/Composed.scala:14-103)."""
+
+    def __init__(self, layers: Sequence[Layer]):
+        if not layers:
+            raise ValueError("requirement failed: at least 1 layer is required")
+        self.layers = list(layers)
+
+    @staticmethod
+    def of(left, right):
+        return Composed(list(left.layers) + list(right.layers))
+
+    def __rshift__(self, other):
+        return Composed.of(self, other)
+
+    def __repr__(self):
+        return " >> ".join(repr(l) for l in self.layers)
+
+
+def _chain(first: Layer, *rest: Optional[Layer]):
+    out = [first] + [l for l in rest if l is not None]
+    return out[0] if len(out) == 1 else Composed(out)
+
+
+def Bias(features: int, reg: Regularization = Zero, initializer: Initializer = Zeros) -> Layer:
+    return Layer(L.LAYER_BIAS, f"Bias({features})", units=features, reg=reg, inits=(initializer,))
+
+
+def Activate(activation: Activation) -> Layer:
+    return Layer(L.LAYER_ACTIVATE, repr(activation), activation=activation)
+
+
+def Dense(outputs: int, activation: Activation = Identity, reg: Regularization = Zero, bias: bool = True,
+          kernelInitializer: Initializer = GlorotUniform(), biasInitializer: Initializer = Zeros):
+    """layer/Dense.scala:30-40: Dense ?>> Bias ?>> Activate."""
+    dense = Layer(L.LAYER_DENSE, f"Dense({outputs})", units=outputs, reg=reg, inits=(kernelInitializer,))
+    return _chain(dense, Bias(outputs, reg, biasInitializer) if bias else None,
+                  Activate(activation) if not activation.identity else None)
+
+
+def Conv2D(filters: int, kernel: Tuple[int, int] = (3, 3), strides: Tuple[int, int] = (1, 1), padding: int = Valid,
+           activation: Activation = Identity, bias: bool = False, kernelInitializer: Initializer = GlorotUniform(),
+           biasInitializer: Initializer = Zeros):
+    """layer/Conv2D.scala:54-68."""
+    conv = Layer(L.LAYER_CONV2D, f"Conv2D({filters},{tuple(kernel)},{tuple(strides)},{_PAD_NAME[padding]},NHWC)".replace(" ", ""),
+                 units=filters, kernel=tuple(kernel), strides=tuple(strides), padding=padding, inits=(kernelInitializer,))
+    return _chain(conv, Bias(filters, Zero, biasInitializer) if bias else None,
+                  Activate(activation) if not activation.identity else None)
+
+
+def Pool2D(window: Tuple[int, int] = (2, 2), strides: Tuple[int, int] = (1, 1), padding: int = Valid) -> Layer:
+    """layer/Pool2D.scala:28-42 (always max pooling)."""
+    return Layer(L.LAYER_POOL2D, f"Pool2D({tuple(window)},{tuple(strides)},{_PAD_NAME[padding]},NHWC,Max)".replace(" ", ""),
+                 kernel=tuple(window), strides=tuple(strides), padding=padding)
+
+
+Flatten = Layer(L.LAYER_FLATTEN, "Flatten")
+
+
+def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
+         recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
+         biasForgetInitializer: Initializer = Ones) -> Layer:
+    """layer/RNN.scala:208-258: tanh cell, sigmoid gates, forget bias one."""
+    return Layer(L.LAYER_LSTM, f"RNN(LSTMCell({units},Tanh,Sigmoid,{'true' if bias else 'false'}))", units=units,
+                 activation=Tanh, use_bias=bias,
+                 inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
+
+
+def LinearRegression(reg: Regularization = Zero, bias: bool = True):
+    """models/LinearRegression.scala: Dense(1), zero-initialised."""
+    return Dense(1, Identity, reg, bias, Zeros, Zeros)
+
+
+def LogisticRegression(reg: Regularization = Zero, bias: bool = True):
+    """models/LogisticRegression.scala: Dense(1, Sigmoid), zero-initialised."""
+    return Dense(1, Sigmoid, reg, bias, Zeros, Zeros)
+
+
+# --------------------------------------------------------------------------- algorithms
+
+
+def _alg(kind, rate=0.0, beta1=0.0, beta2=0.0, epsilon=0.0, init_acc=0.0, nesterov=False) -> L.OptimizerDesc:
+    return L.OptimizerDesc(kind, rate, beta1, beta2, epsilon, init_acc, 1 if nesterov else 0)
+
+
+def SGD(rate=0.01, momentum=0.0, nesterov=False):
+    return _alg(L.OPT_SGD, rate, momentum, nesterov=nesterov)
+
+
+def AdaGrad(rate=0.001, epsilon=1e-7):
+    return _alg(L.OPT_ADAGRAD, rate, epsilon=epsilon)
+
+
+def AdaDelta(rate=1.0, rho=0.9, epsilon=1e-7):
+    return _alg(L.OPT_ADADELTA, rate, rho, epsilon=epsilon)
+
+
+def RMSProp(rate=0.001, rho=0.9, epsilon=1e-7):
+    return _alg(L.OPT_RMSPROP, rate, rho, epsilon=epsilon)
+
+
+def Adam(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7):
+    return _alg(L.OPT_ADAM, rate, beta1, beta2, epsilon)
+
+
+def Nadam(beta1=0.9, beta2=0.999, epsilon=1e-7, initAcc=0.001):
+    return _alg(L.OPT_NADAM, 0.0, beta1, beta2, epsilon, initAcc)
+
+
+def Adamax(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7, initAcc=0.001):
+    return _alg(L.OPT_ADAMAX, rate, beta1, beta2, epsilon, initAcc)
+
+
+def AMSGrad(rate=0.001, beta1=0.9, beta2=0.999, epsilon=1e-7):
+    return _alg(L.OPT_AMSGRAD, rate, beta1, beta2, epsilon)
+
+
+STATE_NAMES = {
+    L.OPT_SGD: ["velocity"], L.OPT_ADAGRAD: ["grad_acc"], L.OPT_ADADELTA: ["avg_grad", "avg_delta"],
+    L.OPT_RMSPROP: ["avg_grad"], L.OPT_ADAM: ["momentum", "velocity"], L.OPT_NADAM: ["momentum", "velocity"],
+    L.OPT_ADAMAX: ["momentum_1", "momentum_2"], L.OPT_AMSGRAD: ["momentum", "velocity", "corrected_velocity"],
+}
+
+# --------------------------------------------------------------------------- datasets / training
+
+
+class Dataset:
+    """Rows of (features, labels) with per-sample shapes, cut into `partitions` contiguous parts
+    (the reference keeps shapes in Spark column metadata, optimizers/SparkExt.scala:16-33)."""
+
+    def __init__(self, x, y, partitions: int = 1):
+        self.x = np.ascontiguousarray(x, np.float32)
+        self.y = np.ascontiguousarray(y, np.float32)
+        if self.x.shape[0] != self.y.shape[0]:
+            raise ValueError("features and labels differ in row count")
+        self.partitions = int(partitions)
+
+    @property
+    def shapes(self):
+        return self.x.shape[1:], self.y.shape[1:]
+
+    def __len__(self):
+        return self.x.shape[0]
+
+    def coalesce(self, n: int) -> "Dataset":
+        return Dataset(self.x, self.y, n)
+
+    def split(self) -> List[Tuple[np.ndarray, np.ndarray]]:
+        idx = np.array_split(np.arange(len(self)), self.partitions)
+        return [(self.x[i[0]:i[-1] + 1], self.y[i[0]:i[-1] + 1]) for i in idx if len(i)]
+
+    def train(self, model) -> "Builder":
+        return Builder(model=model, dataset=self)
+
+
+def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndarray]:
+    """ParamDef.initialize for every weight (optimizers/Optimizer.scala:124-128)."""
+    rng = np.random.default_rng(seed)
+    layers = model.layers
+    single = len(layers) == 1
+    out: Dict[str, np.ndarray] = {}
+    shapes = {p: s for p, s, _ in compiled.params}
+    for i, l in enumerate(layers):
+        pre = "" if single else f"{i}/"
+        if l.kind in (L.LAYER_DENSE, L.LAYER_BIAS, L.LAYER_CONV2D):
+            out[pre + "weights"] = l.inits[0].build(shapes[pre + "weights"], rng)
+        elif l.kind == L.LAYER_LSTM:
+            k_init, r_init, b_init, bf_init = l.inits
+            for gate in ("forget", "input", "gate", "output"):
+                out[f"{pre}{gate}/0/kernel_weights"] = k_init.build(shapes[f"{pre}{gate}/0/kernel_weights"], rng)
+                out[f"{pre}{gate}/0/recurrent_weights"] = r_init.build(shapes[f"{pre}{gate}/0/recurrent_weights"], rng)
+                if l.use_bias:
+                    b = bf_init if gate == "forget" else b_init
+                    out[f"{pre}{gate}/1/weights"] = b.build(shapes[f"{pre}{gate}/1/weights"], rng)
+    return out
+
+
+@dataclass
+class TrainedModel:
+    """`TrainedModel` (models/Model.scala:154-187): a model, its loss and the learned parameters."""
+    model: object
+    loss_fn: Loss
+    params: Dict[str, np.ndarray]
+    opt_state: Dict[str, List[np.ndarray]]
+    history: List[float]
+    iterations: int
+    input_shape: Tuple[int, ...]
+    flags: int = 0
+    ctx: Optional[Context] = None
+
+    def _run(self, x, batch, fn):
+        x = np.ascontiguousarray(x, np.float32)
+        ctx = self.ctx or Context()
+        try:
+            cm = CompiledModel(ctx, [l.desc() for l in self.model.layers], self.loss_fn.kind, self.input_shape, batch, self.flags)
+            rep = cm.replica(None)
+            rep.set_params(self.params)
+            try:
+                return fn(ctx, cm, rep)
+            finally:
+                rep.close()
+                cm.close()
+        finally:
+            if self.ctx is None:
+                ctx.close()
+
+    def result(self, x) -> np.ndarray:
+        x = np.ascontiguousarray(x, np.float32)
+
+        def go(ctx, cm, rep):
+            xb = ctx.to_device(x)
+            try:
+                return rep.forward(xb, x.shape[0])
+            finally:
+                xb.free()
+        return self._run(x, x.shape[0], go)
+
+    def loss(self, x, y) -> float:
+        x = np.ascontiguousarray(x, np.float32)
+
+        def go(ctx, cm, rep):
+            xb, yb = ctx.to_device(x), ctx.to_device(y)
+            try:
+                return rep.loss(xb, yb, x.shape[0])
+            finally:
+                xb.free()
+                yb.free()
+        return self._run(x, x.shape[0], go)
+
+
+def accuracy(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
+    """estimators.accuracy (estimators/package.scala:18-47): batches of `batch` rows, the last one partial."""
+    n = len(ds)
+    batch = min(batch, n)
+
+    def go(ctx, cm, rep):
+        positives = 0
+        for s in range(0, n, batch):
+            xs, ys = ds.x[s:s + batch], ds.y[s:s + batch]
+            xb, yb = ctx.to_device(xs), ctx.to_device(ys)
+            try:
+                positives += rep.count_correct(xb, yb, xs.shape[0])
+            finally:
+                xb.free()
+                yb.free()
+        return positives / n
+    return trained._run(ds.x, batch, go)
+
+
+@dataclass
+class Builder:
+    """The type-state builder of the reference without the types (optimizers/Optimizer.scala:267-310)."""
+    model: object
+    dataset: Optional[Dataset] = None
+    loss_fn: Optional[Loss] = None
+    alg: Optional[L.OptimizerDesc] = None
+    batch_size: int = 10000                      # Optimizer.scala:321
+    n_epochs: Optional[int] = None
+    n_iterations: Optional[int] = None
+    init: Optional[Callable[[], Dict[str, np.ndarray]]] = None
+    effects: List[Callable] = field(default_factory=list)
+    flags: int = 0
+    seed: int = 0
+    device: int = 0
+
+    def loss(self, loss: Loss):
+        return replace(self, loss_fn=loss)
+
+    def using(self, alg: L.OptimizerDesc):
+        return replace(self, alg=alg)
+
+    def initParams(self, params):
+        return replace(self, init=(params if callable(params) else (lambda: params)))
+
+    def on(self, dataset: Dataset):
+        return replace(self, dataset=dataset)
+
+    def batch(self, size: int):
+        return replace(self, batch_size=int(size))
+
+    def epochs(self, number: int):
+        return replace(self, n_epochs=int(number))
+
+    stopAfterEpochs = epochs
+
+    def iterations(self, number: int):
+        return replace(self, n_iterations=int(number))
+
+    def each(self, effect: Callable):
+        """effect(epoch, iterations, loss) after every epoch (optimizers/Effect.scala)."""
+        return replace(self, effects=self.effects + [effect])
+
+    def bf16(self, on: bool = True):
+        return replace(self, flags=(self.flags | L.FLAG_GEMM_BF16) if on else (self.flags & ~L.FLAG_GEMM_BF16))
+
+    def run(self) -> TrainedModel:
+        for name, v in (("loss", self.loss_fn), ("using", self.alg), ("on/train", self.dataset)):
+            if v is None:
+                raise ValueError(f"builder is incomplete: call .{name}(..) first")
+        if self.n_epochs is None and self.n_iterations is None:
+            raise ValueError("builder is incomplete: call .epochs(..) or .iterations(..) first")
+        ds = self.dataset
+        in_shape, _ = ds.shapes
+        parts = ds.split()
+        ctx = Context(self.device)
+        bufs: List[DeviceBuffer] = []
+        reps: List[Replica] = []
+        cm = None
+        try:
+            cm = CompiledModel(ctx, [l.desc() for l in self.model.layers], self.loss_fn.kind, in_shape, self.batch_size, self.flags)
+            params = self.init() if self.init else _init_params(self.model, cm, self.seed)
+            data = []
+            for px, py in parts:
+                xb, yb = ctx.to_device(px), ctx.to_device(py)
+                bufs += [xb, yb]
+                data.append((xb, yb, px.shape[0]))
+                rep = cm.replica(self.alg)
+                rep.set_params(params)
+                reps.append(rep)
+            global_iter, epoch, history = 0, 0, []
+            while True:
+                iters, losses = 0, []
+                for rep, (xb, yb, rows) in zip(reps, data):       # one partition after the other on the one GPU
+                    it, lo = rep.train_epoch(xb, yb, rows, self.batch_size, global_iter)
+                    iters += it
+                    losses.append(lo)
+                average_replicas(reps)                              # Optimizer.scala:86,196-230
+                loss = float(np.mean(np.asarray(losses, np.float32)))   # `(l.loss + r.loss) / 2`, uniform over K here
+                global_iter += iters                                # Optimizer.scala:88
+                epoch += 1
+                history.append(loss)
+                for e in self.effects:
+                    e(epoch, global_iter, loss)
+                if (self.n_epochs is not None and epoch >= self.n_epochs) or \
+                        (self.n_iterations is not None and global_iter >= self.n_iterations):
+                    break
+            final = reps[0].get_params()
+            n_states = len(STATE_NAMES[self.alg.kind])
+            slots = [reps[0].get_opt_state(s) for s in range(n_states)]
+            opt_state = {p: [slots[s][p] for s in range(n_states)] for p in final}
+            return TrainedModel(self.model, self.loss_fn, final, opt_state, history, global_iter, tuple(in_shape), self.flags)
+        finally:
+            for r in reps:
+                r.close()
+            if cm is not None:
+                cm.close()
+            for b in bufs:
+                b.free()
+            ctx.close()

@@ -1,0 +1,109 @@
+"""Shared helpers of the parity tests: one model spec builds both the oracle model and the
+HIP-side layer list, so both sides see identical layers, parameters and data."""
+from __future__ import annotations
+
+from typing import Dict, List, Tuple
+
+import numpy as np
+
+from oracle import scanet_oracle as O
+
+f32 = np.float32
+
+
+def build_pair(spec: List[tuple], loss: str):
+    """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
+    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("activate", act) | ("bias", features)
+    Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
+    import scanet3_amd as S
+    acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
+              "softmax": O.ACT_SOFTMAX}
+    acts_s = {"identity": S.Identity, "sigmoid": S.Sigmoid, "tanh": S.Tanh, "relu": S.ReLU(), "softmax": S.Softmax}
+    pads_o = {"valid": O.PAD_VALID, "same": O.PAD_SAME}
+    pads_s = {"valid": S.Valid, "same": S.Same}
+    regs_o = {"none": O.REG_NONE, "l1": O.REG_L1, "l2": O.REG_L2}
+    ol, sl = [], None
+
+    def add(layer):
+        nonlocal sl
+        sl = layer if sl is None else (sl >> layer)
+
+    for e in spec:
+        k = e[0]
+        if k == "dense":
+            units, act = e[1], e[2]
+            reg, lam = (e[3], e[4]) if len(e) > 3 else ("none", 0.0)
+            ol.append(O.Dense(units, acts_o[act], reg=regs_o[reg], reg_lambda=lam))
+            sreg = S.Zero if reg == "none" else (S.L1(lam) if reg == "l1" else S.L2(lam))
+            add(S.Dense(units, acts_s[act], reg=sreg))
+        elif k == "conv":
+            _, filters, kernel, strides, pad, act, bias = e
+            ol.append(O.Conv2D(filters, kernel, strides, pads_o[pad], acts_o[act], bias=bias))
+            add(S.Conv2D(filters, kernel, strides, pads_s[pad], acts_s[act], bias=bias))
+        elif k == "pool":
+            _, window, strides, pad = e
+            ol.append(O.Pool2D(window, strides, pads_o[pad]))
+            add(S.Pool2D(window, strides, pads_s[pad]))
+        elif k == "flatten":
+            ol.append(O.Flatten())
+            add(S.Flatten)
+        elif k == "lstm":
+            bias = e[2] if len(e) > 2 else True
+            ol.append(O.LSTM(e[1], bias=bias))
+            add(S.LSTM(e[1], bias=bias))
+        elif k == "activate":
+            ol.append([O.Layer("activate", activation=acts_o[e[1]])])
+            add(S.Activate(acts_s[e[1]]))
+        elif k == "bias":
+            ol.append([O.Layer("bias", units=e[1])])
+            add(S.Bias(e[1]))
+        else:
+            raise ValueError(k)
+    losses_o = {"mse": O.LOSS_MSE, "bce": O.LOSS_BCE, "cce": O.LOSS_CCE}
+    losses_s = {"mse": S.MeanSquaredError, "bce": S.BinaryCrossentropy, "cce": S.CategoricalCrossentropy}
+    return O.Model(ol, losses_o[loss]), sl, losses_s[loss]
+
+
+def glorot_params(model: O.Model, in_shape, rng: np.random.Generator, scale: float = 1.0) -> Dict[str, np.ndarray]:
+    """Xavier-uniform weights, zero biases (forget-gate bias one), from the harness' own generator."""
+    out = {}
+    for path, shape in model.param_defs(in_shape):
+        if len(shape) == 1:
+            out[path] = np.ones(shape, f32) if "forget/1/" in path else np.zeros(shape, f32)
+        else:
+            fan_in = int(np.prod(shape[:-1]))
+            fan_out = shape[-1]
+            lim = np.sqrt(6.0 / (fan_in + fan_out)) * scale
+            out[path] = rng.uniform(-lim, lim, shape).astype(f32)
+    return out
+
+
+def one_hot(rng, rows, classes):
+    return np.eye(classes, dtype=f32)[rng.integers(0, classes, rows)]
+
+
+def rel_err(a: np.ndarray, b: np.ndarray) -> float:
+    """max |a-b| relative to the largest magnitude of the reference tensor b."""
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    denom = max(float(np.max(np.abs(b))), 1e-30)
+    return float(np.max(np.abs(a - b))) / denom
+
+
+OPT_PAIRS = None
+
+
+def optimizer_pairs():
+    """[(name, oracle Algorithm, HIP optimizer descriptor)] with the reference's defaults."""
+    import scanet3_amd as S
+    return [
+        ("sgd", O.SGD(), S.SGD()),
+        ("sgd_momentum", O.SGD(0.01, 0.9), S.SGD(0.01, 0.9)),
+        ("sgd_nesterov", O.SGD(0.01, 0.9, True), S.SGD(0.01, 0.9, True)),
+        ("adagrad", O.AdaGrad(), S.AdaGrad()),
+        ("adadelta", O.AdaDelta(), S.AdaDelta()),
+        ("rmsprop", O.RMSProp(), S.RMSProp()),
+        ("adam", O.Adam(), S.Adam()),
+        ("nadam", O.Nadam(), S.Nadam()),
+        ("adamax", O.Adamax(), S.Adamax()),
+        ("amsgrad", O.AMSGrad(), S.AMSGrad()),
+    ]

@@ -1,0 +1,511 @@
+"""Parity of the HIP library (through its C ABI) with the CPU oracle on identical seeded inputs,
+and with the reference's own golden vectors.  Needs an MI355X: run with `-m gpu`.
+
+Tolerances (relative to the largest magnitude of the reference tensor):
+  optimizer updates, activations, averaging ... 1e-6
+  GEMM / convolution outputs and gradients ..... 1e-4
+  loss trajectories ............................ 1e-3
+  accuracy counts .............................. exact
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+from oracle import scanet_oracle as O
+from tests.helpers import build_pair, f32, glorot_params, one_hot, optimizer_pairs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL_ELEMENTWISE = 1e-6
+TOL_GEMM = 1e-4
+TOL_TRAJECTORY = 1e-3
+
+
+@pytest.fixture(scope="module")
+def S():
+    import scanet3_amd
+    return scanet3_amd
+
+
+@pytest.fixture(scope="module")
+def ctx(S):
+    c = S.Context(0)
+    yield c
+    c.close()
+
+
+def A(v):
+    return np.asarray(v, dtype=f32)
+
+
+def round_at(x, p):
+    s = f32(10.0 ** p)
+    return np.rint(x * s) / s
+
+
+class Harness:
+    """Compiles a model on the GPU and holds its oracle twin."""
+
+    def __init__(self, S, ctx, spec, loss, in_shape, batch, alg=None, flags=0):
+        self.omodel, layers, sloss = build_pair(spec, loss)
+        self.cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, in_shape, batch, flags)
+        self.rep = self.cm.replica(alg)
+        self.ctx = ctx
+        self.in_shape = tuple(in_shape)
+        self.batch = batch
+
+    def close(self):
+        self.rep.close()
+        self.cm.close()
+
+
+# ----------------------------------------------------------------------------- flat kernels
+@pytest.mark.parametrize("n", [1, 63, 1000, 100003, 1 << 20])
+def test_optimizer_updates_match_oracle(S, ctx, n):
+    rng = np.random.default_rng(100 + n % 97)
+    for name, oalg, desc in optimizer_pairs():
+        w = (rng.standard_normal(n) * 0.02).astype(f32)
+        w0 = w.copy()
+        states = oalg.init_state((n,))
+        wb = ctx.to_device(w)
+        sb = [ctx.to_device(s) for s in states]
+        gb = ctx.alloc(n)
+        for it in range(1, 4):
+            g = (rng.standard_normal(n) * 1e-3).astype(f32)
+            gb.copy_from(g)
+            delta, states = oalg.build(g, states, it)
+            w = w - delta
+            ctx.optimizer_update(desc, wb, gb, sb, it)
+        assert rel_err(wb.numpy(), w) <= TOL_ELEMENTWISE, name
+        for s_gpu, s_ref in zip(sb, states):
+            assert rel_err(s_gpu.numpy(), s_ref) <= TOL_ELEMENTWISE, name
+        assert np.any(wb.numpy() != w0), name            # the kernel did move the weights
+        for b in [wb, gb] + sb:
+            b.free()
+
+
+def test_optimizer_high_iteration_and_unaligned_views(S, ctx):
+    """iteration 10^6 (bias corrections ~ 1) and buffers that start 4 bytes off a 16-byte boundary."""
+    rng = np.random.default_rng(7)
+    n = 4099
+    for name, oalg, desc in optimizer_pairs():
+        w = (rng.standard_normal(n) * 0.02).astype(f32)
+        g = (rng.standard_normal(n) * 1e-3).astype(f32)
+        states = [np.abs(rng.standard_normal(n)).astype(f32) * f32(1e-4) for _ in oalg.state_names]
+        big = [ctx.alloc(n + 1) for _ in range(2 + len(states))]
+        import ctypes as C
+        from scanet3_amd._lib import check, lib
+        views = [b.offset(1) for b in big]
+        for v, arr in zip(views, [w, g] + states):
+            check(lib.sn_copy_h2d(ctx.handle, v, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+        ctx.sync()
+        sv = views[2:] + [None] * (3 - len(states))
+        check(lib.sn_optimizer_update(ctx.handle, C.byref(desc), views[0], views[1], sv[0], sv[1], sv[2], n, 1000000))
+        delta, _ = oalg.build(g, states, 1000000)
+        got = big[0].numpy()[1:]
+        assert rel_err(got, w - delta) <= TOL_ELEMENTWISE, name
+        for b in big:
+            b.free()
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 8])
+@pytest.mark.parametrize("n", [5, 1000, 250001])
+def test_average_matches_oracle(S, ctx, k, n):
+    rng = np.random.default_rng(k * 1000 + n % 13)
+    reps = [(rng.standard_normal(n) * 0.02).astype(f32) for _ in range(k)]
+    bufs = [ctx.to_device(r) for r in reps]
+    out = ctx.alloc(n)
+    ctx.average(bufs, out)
+    ref = O.average_uniform(reps)
+    got = out.numpy()
+    assert rel_err(got, ref) <= TOL_ELEMENTWISE
+    np.testing.assert_array_equal(got, ref)          # same left-to-right float32 sum, so in fact identical
+    for b in bufs + [out]:
+        b.free()
+
+
+def test_average_rejects_bad_arguments(S, ctx):
+    a = ctx.alloc(8)
+    with pytest.raises(S.ScanetError):
+        ctx.average([], a)
+    with pytest.raises(S.ScanetError):
+        ctx.average([a] * 33, a)
+    with pytest.raises(S.ScanetError):
+        ctx.optimizer_update(S.Adam(), a, a, [a], 1)          # Adam needs two state buffers
+    with pytest.raises(S.ScanetError):
+        ctx.optimizer_update(S.Adam(), a, a, [a, a], 0)       # iterations are 1-based
+    a.free()
+
+
+# ----------------------------------------------------------------------------- reference goldens through the C ABI
+def test_golden_dense_and_losses(S, ctx, golden):
+    g = golden["dense_sigmoid"]
+    h = Harness(S, ctx, [("dense", 4, "sigmoid")], "bce", (3,), 4)
+    h.rep.set_params({"0/weights": A(g["w"]), "1/weights": A(g["b"])})
+    x = ctx.to_device(A(g["x"]))
+    np.testing.assert_array_equal(round_at(h.rep.forward(x), 6), A(g["y_6dp"]))
+    h.rep.set_params({"0/weights": np.zeros((3, 4), f32), "1/weights": np.zeros(4, f32)})
+    y = ctx.to_device(A(g["bce_y"]))
+    h.rep.grad(x, y)
+    grads = h.rep.get_grads()
+    np.testing.assert_allclose(grads["0/weights"], A(g["bce_grad_w"]), rtol=1e-6)
+    np.testing.assert_allclose(grads["1/weights"], A(g["bce_grad_b"]), rtol=1e-6)
+    h.close()
+
+    g = golden["mlp_3_1_loss"]
+    params = {"0/weights": A(g["w1"]), "1/weights": A(g["b1"]), "3/weights": A(g["w2"]), "4/weights": A(g["b2"])}
+    h = Harness(S, ctx, [("dense", 3, "sigmoid"), ("dense", 1, "sigmoid")], "mse", (3,), 2)
+    assert [p for p, _, _ in h.cm.params] == ["0/weights", "1/weights", "3/weights", "4/weights"]
+    h.rep.set_params(params)
+    x, y = ctx.to_device(A(g["x"])), ctx.to_device(A(g["y"]))
+    assert round_at(np.asarray(h.rep.loss(x, y), f32), 6) == f32(g["mse_6dp"])
+    h.close()
+    h = Harness(S, ctx, [("dense", 3, "sigmoid", "l2", 1.0), ("dense", 1, "sigmoid", "l2", 1.0)], "mse", (3,), 2)
+    h.rep.set_params(params)
+    np.testing.assert_allclose(h.rep.loss(x, y), g["mse_plus_l2"], rtol=1e-6)
+    h.close()
+
+    g = golden["linear_regression"]
+    h = Harness(S, ctx, [("dense", 1, "identity")], "mse", (2,), 2)
+    h.rep.set_params({"0/weights": A(g["w"]), "1/weights": A(g["b"])})
+    x, y = ctx.to_device(A(g["x"])), ctx.to_device(A(g["y"]))
+    assert h.rep.loss(x, y) == g["mse"]
+    np.testing.assert_array_equal(h.rep.forward(x), A(g["result"]))
+    h.rep.set_params({"0/weights": np.zeros((2, 1), f32), "1/weights": np.zeros(1, f32)})
+    h.rep.grad(x, y)
+    np.testing.assert_array_equal(h.rep.get_grads()["0/weights"], A(g["grad_at_zero_w"]))
+    np.testing.assert_array_equal(h.rep.get_grads()["1/weights"], A(g["grad_at_zero_b"]))
+    h.close()
+
+    g = golden["logistic_regression"]
+    h = Harness(S, ctx, [("dense", 1, "sigmoid")], "bce", (2,), 2)
+    h.rep.set_params({"0/weights": A(g["w"]), "1/weights": A(g["b"])})
+    x, y = ctx.to_device(A(g["x"])), ctx.to_device(A(g["y"]))
+    assert abs(h.rep.loss(x, y) - g["bce"]) <= 1e-6
+    np.testing.assert_array_equal(round_at(h.rep.forward(x), 6), A(g["result_6dp"]))
+    h.rep.grad(x, y)
+    np.testing.assert_array_equal(round_at(h.rep.get_grads()["0/weights"], 6), A(g["grad_w_6dp"]))
+    np.testing.assert_array_equal(round_at(h.rep.get_grads()["1/weights"], 6), A(g["grad_b_6dp"]))
+    h.close()
+
+
+def test_golden_softmax_and_activations(S, ctx, golden):
+    g = golden["activations"]
+    h = Harness(S, ctx, [("activate", "softmax")], "cce", (5,), 2)
+    x = ctx.to_device(A(g["softmax_in"]))
+    np.testing.assert_array_equal(round_at(h.rep.forward(x), 5), A(g["softmax_5dp"]))
+    h.close()
+    for act, xs, ys, tol in [("tanh", [-0.5, 0.0, 0.5], [-g["tanh_0.5"], 0.0, g["tanh_0.5"]], 1.3e-7),
+                             ("sigmoid", g["sigmoid_in"], None, 0), ("relu", [5.0, 0.0, -5.0], [5.0, 0.0, 0.0], 0)]:
+        h = Harness(S, ctx, [("activate", act)], "mse", (3,), 1)
+        out = h.rep.forward(ctx.to_device(A([xs])))[0]
+        if act == "sigmoid":
+            np.testing.assert_array_equal(round_at(out, 6), A(g["sigmoid_6dp"]))
+        else:
+            np.testing.assert_allclose(out, A(ys), rtol=tol, atol=0)
+        h.close()
+
+
+@pytest.mark.parametrize("key,strides,pad", [("same_s1", (1, 1), "same"), ("same_s2", (2, 2), "same"),
+                                             ("valid_s1", (1, 1), "valid"), ("valid_s2", (2, 2), "valid")])
+def test_golden_conv_and_pool(S, ctx, golden, key, strides, pad):
+    img = A(golden["image_5x5"]).reshape(1, 5, 5, 1)
+    x = ctx.to_device(img)
+    h = Harness(S, ctx, [("conv", 1, (2, 2), strides, pad, "identity", False)], "mse", (5, 5, 1), 1)
+    assert [p for p, _, _ in h.cm.params] == ["weights"]          # a single layer carries no index prefix
+    h.rep.set_params({"weights": A(golden["filter_2x2"]).reshape(2, 2, 1, 1)})
+    exp = A(golden["conv2d"][key])
+    np.testing.assert_array_equal(h.rep.forward(x).reshape(exp.shape), exp)
+    h.close()
+    h = Harness(S, ctx, [("pool", (2, 2), strides, pad)], "mse", (5, 5, 1), 1)
+    exp = A(golden["max_pool_2x2"][key])
+    np.testing.assert_array_equal(h.rep.forward(x).reshape(exp.shape), exp)
+    h.close()
+
+
+def test_golden_conv_pool_gradients(S, ctx, golden):
+    """d sum(conv)/d filter and d sum(pool(conv))/.. via a model whose loss gradient is all ones:
+    MSE against y = out - size/2 gives d loss / d out = 1 exactly."""
+    img = A(golden["image_5x5"]).reshape(1, 5, 5, 1)
+    x = ctx.to_device(img)
+    h = Harness(S, ctx, [("conv", 1, (2, 2), (1, 1), "valid", "identity", False)], "mse", (5, 5, 1), 1)
+    w = A(golden["filter_2x2"]).reshape(2, 2, 1, 1)
+    h.rep.set_params({"weights": w})
+    out = h.rep.forward(x)
+    y = ctx.to_device(out - f32(out.size / 2.0))
+    h.rep.grad(x, y)
+    np.testing.assert_allclose(h.rep.get_grads()["weights"].reshape(2, 2), A(golden["conv2d"]["valid_s1_grad_filter_of_sum"]),
+                               rtol=1e-6)
+    h.close()
+    # pool gradient with ties: identity 1x1 convolution in front so that the pool's input gradient lands in a weight-free
+    # path we can read back: d loss / d w of the 1x1 conv = sum(x * dpool_input); compare with the golden mask
+    h = Harness(S, ctx, [("conv", 1, (1, 1), (1, 1), "valid", "identity", False), ("pool", (2, 2), (1, 1), "same")],
+                "mse", (5, 5, 1), 1)
+    h.rep.set_params({"0/weights": np.ones((1, 1, 1, 1), f32)})
+    out = h.rep.forward(x)
+    y = ctx.to_device(out - f32(out.size / 2.0))
+    h.rep.grad(x, y)
+    mask = A(golden["max_pool_2x2"]["same_s1_grad_input_of_sum"])
+    np.testing.assert_allclose(h.rep.get_grads()["0/weights"].ravel()[0], float((img.reshape(5, 5) * mask).sum()), rtol=1e-6)
+    h.close()
+
+
+def test_golden_lstm_forward(S, ctx, golden):
+    g = golden["lstm"]
+    h = Harness(S, ctx, [("lstm", 2)], "mse", (3, 1), 1)
+    params = {}
+    for gate in O.GATES:
+        params[f"{gate}/0/kernel_weights"] = A(g[gate]["k"])
+        params[f"{gate}/0/recurrent_weights"] = A(g[gate]["r"])
+        params[f"{gate}/1/weights"] = A(g[gate]["b"])
+    assert sorted(p for p, _, _ in h.cm.params) == sorted(params)
+    h.rep.set_params(params)
+    out = h.rep.forward(ctx.to_device(A(g["x"]).reshape(1, 3, 1)))
+    np.testing.assert_array_equal(round_at(out, 6), A(g["y_6dp"]))
+    h.close()
+
+
+def test_cnn_shape_table(S, ctx, golden):
+    g = golden["cnn_shapes"]
+    spec = [("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+            ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+            ("flatten",), ("dense", 10, "softmax")]
+    h = Harness(S, ctx, spec, "cce", tuple(g["input"]), 1)
+    assert {p: list(s) for p, s, _ in h.cm.params} == g["weights"]
+    assert sum(int(np.prod(s)) for _, s, _ in h.cm.params) == g["total_params"]
+    assert h.cm.output_shape == (10,)
+    h.close()
+
+
+# ----------------------------------------------------------------------------- model parity against the oracle
+MODELS = {
+    # name: (spec, loss, input shape, batch, data kind)
+    "mlp_cfg1": ([("dense", 50, "sigmoid"), ("dense", 10, "softmax")], "cce", (784,), 1000, "uniform_onehot"),
+    "mlp_tanh_relu": ([("dense", 33, "tanh"), ("dense", 65, "relu"), ("dense", 7, "softmax")], "cce", (19,), 130, "normal_onehot"),
+    "mlp_bce_l2": ([("dense", 12, "sigmoid", "l2", 0.05), ("dense", 3, "sigmoid", "l1", 0.01)], "bce", (9,), 40, "uniform_binary"),
+    "lenet_small": ([("conv", 8, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+                     ("conv", 16, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+                     ("flatten",), ("dense", 10, "softmax")], "cce", (12, 12, 1), 20, "uniform_onehot"),
+    "cnn_same_stride2_bias": ([("conv", 5, (3, 2), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "same"),
+                               ("activate", "relu"), ("flatten",), ("dense", 4, "softmax")], "cce", (9, 10, 3), 7, "uniform_onehot"),
+    "lstm_small": ([("lstm", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
+    "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
+}
+
+
+def make_data(kind, rng, rows, in_shape, out_dim):
+    if kind == "uniform_onehot":
+        return rng.random((rows,) + in_shape, f32), one_hot(rng, rows, out_dim)
+    if kind == "normal_onehot":
+        return rng.standard_normal((rows,) + in_shape).astype(f32), one_hot(rng, rows, out_dim)
+    if kind == "uniform_binary":
+        return rng.random((rows,) + in_shape, f32), rng.integers(0, 2, (rows, out_dim)).astype(f32)
+    x = rng.standard_normal((rows,) + in_shape).astype(f32)
+    return x, rng.uniform(-1, 1, (rows, out_dim)).astype(f32)
+
+
+@pytest.mark.parametrize("name", list(MODELS))
+def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
+    spec, loss, in_shape, batch, kind = MODELS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000 + 20251125)
+    h = Harness(S, ctx, spec, loss, in_shape, batch)
+    om = h.omodel
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    for p in params:                      # non-zero biases so their gradients and use are exercised
+        if params[p].ndim == 1:
+            params[p] = params[p] + rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
+    out_dim = om.out_shape((batch,) + in_shape)[-1]
+    x, y = make_data(kind, rng, batch, in_shape, out_dim)
+    h.rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    pred = h.rep.forward(xb)
+    assert rel_err(pred, om.forward(x, params)) <= TOL_GEMM
+    oloss, ograds = om.grad(x, y, params)
+    gloss = h.rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    assert abs(h.rep.loss(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ggrads = h.rep.get_grads()
+    assert set(ggrads) == set(ograds)
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+    # partial batch (the accuracy estimator feeds one): rows < batch must give the same per-row predictions
+    rows = max(1, batch // 3)
+    np.testing.assert_allclose(h.rep.forward(xb, rows), pred[:rows], rtol=1e-6, atol=1e-7)
+    h.close()
+
+
+@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("mlp_bce_l2", 25)])
+@pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
+def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
+    spec, loss, in_shape, batch, kind = MODELS[name]
+    oalg, desc = {n: (o, d) for n, o, d in optimizer_pairs()}[alg]
+    if name == "mlp_cfg1":
+        oalg, desc = O.Adam(0.01), S.Adam(0.01)
+    rng = np.random.default_rng(20251125 + 1)
+    h = Harness(S, ctx, spec, loss, in_shape, batch, desc)
+    om = h.omodel
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    out_dim = om.out_shape((batch,) + in_shape)[-1]
+    n_batches = 3
+    X, Y = make_data(kind, rng, batch * n_batches, in_shape, out_dim)
+    h.rep.set_params(params)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    ostate = O.init_opt_state(oalg, params)
+    for t in range(1, steps + 1):
+        b = (t - 1) % n_batches
+        xs, ys = X[b * batch:(b + 1) * batch], Y[b * batch:(b + 1) * batch]
+        params, ostate, oloss, _ = O.train_step(om, oalg, xs, ys, params, ostate, t)
+        gloss = h.rep.step(Xb.offset(b * batch * int(np.prod(in_shape))), Yb.offset(b * batch * out_dim), t, want_loss=True)
+        assert abs(gloss - float(oloss)) <= TOL_TRAJECTORY * max(1.0, abs(float(oloss))), (t, gloss, float(oloss))
+    got = h.rep.get_params()
+    for p in params:
+        assert rel_err(got[p], params[p]) <= 2e-3, p
+    h.close()
+
+
+def test_full_config_lenet_and_lstm_one_step(S, ctx):
+    """The LeNet and LSTM benchmark shapes at full size: one gradient against the oracle."""
+    cases = [
+        ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+          ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+          ("flatten",), ("dense", 10, "softmax")], "cce", (28, 28, 1), 100, "uniform_onehot"),
+        ([("lstm", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),
+    ]
+    for spec, loss, in_shape, batch, kind in cases:
+        rng = np.random.default_rng(20251125 + 2)
+        h = Harness(S, ctx, spec, loss, in_shape, batch)
+        om = h.omodel
+        params = glorot_params(om, (batch,) + in_shape, rng)
+        out_dim = om.out_shape((batch,) + in_shape)[-1]
+        x, y = make_data(kind, rng, batch, in_shape, out_dim)
+        h.rep.set_params(params)
+        xb, yb = ctx.to_device(x), ctx.to_device(y)
+        oloss, ograds = om.grad(x, y, params)
+        gloss = h.rep.grad(xb, yb)
+        assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+        ggrads = h.rep.get_grads()
+        for p in ograds:
+            assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        h.close()
+        xb.free()
+        yb.free()
+
+
+# ----------------------------------------------------------------------------- epoch loop, averaging, accuracy
+def test_train_epoch_semantics_and_replica_average(S, ctx, linear_function):
+    X, Y = linear_function
+    spec = [("dense", 1, "identity")]
+    om, layers, sloss = build_pair(spec, "mse")
+    init = {"0/weights": np.zeros((1, 1), f32), "1/weights": np.zeros(1, f32)}
+    oalg, desc = O.Adam(0.1), S.Adam(0.1)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (1,), 40)
+    rep = cm.replica(desc)
+    rep.set_params(init)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    iters, loss = rep.train_epoch(Xb, Yb, X.shape[0], 40, 0)
+    oi, op_, ost, oloss = O.optimize_on_partition(om, oalg, X, Y, 40, 0, init, O.init_opt_state(oalg, init))
+    assert iters == oi == 2                      # 97 rows: two full batches, 17 rows skipped
+    assert abs(loss - float(oloss)) <= TOL_GEMM * abs(float(oloss))
+    got = rep.get_params()
+    for p in op_:
+        assert rel_err(got[p], op_[p]) <= 1e-5
+    with pytest.raises(S.ScanetError):
+        rep.train_epoch(Xb, Yb, 10, 40, 0)       # no full batch: the reference's iterator throws
+    # two replicas on the two halves, then the uniform average of weights and optimizer state
+    rep2 = cm.replica(desc)
+    rep.set_params(init)
+    rep2.set_params(init)
+    for s in range(2):
+        rep.set_opt_state(s, {p: np.zeros_like(v) for p, v in init.items()})
+    half = 48
+    rep.train_epoch(Xb, Yb, half, 40, 0)
+    rep2.train_epoch(Xb.offset(half), Yb.offset(half), X.shape[0] - half, 40, 0)
+    pa, pb = rep.get_params(), rep2.get_params()
+    sa, sb = rep.get_opt_state(1), rep2.get_opt_state(1)
+    S.average_replicas([rep, rep2])
+    for r in (rep, rep2):
+        got = r.get_params()
+        st = r.get_opt_state(1)
+        for p in pa:
+            np.testing.assert_array_equal(got[p], O.average_uniform([pa[p], pb[p]]))
+            np.testing.assert_array_equal(st[p], O.average_uniform([sa[p], sb[p]]))
+    rep.close()
+    rep2.close()
+    cm.close()
+
+
+def test_dsl_training_run_matches_oracle_and_thresholds(S, golden, linear_function, logistic_data):
+    """The reference's own convergence tests, run through the DSL mirror on the GPU."""
+    X, Y = linear_function
+    algs = {"SGD": (S.SGD, O.SGD), "Adam": (S.Adam, O.Adam), "AdaGrad": (S.AdaGrad, O.AdaGrad), "AdaDelta": (S.AdaDelta, O.AdaDelta),
+            "RMSProp": (S.RMSProp, O.RMSProp), "Nadam": (S.Nadam, O.Nadam), "Adamax": (S.Adamax, O.Adamax),
+            "AMSGrad": (S.AMSGrad, O.AMSGrad)}
+    om = O.Model([O.Dense(1)], O.LOSS_MSE)
+    init = {"0/weights": np.zeros((1, 1), f32), "1/weights": np.zeros(1, f32)}
+    for case in golden["convergence"]["cases"]:
+        sa, oa = algs[case["alg"]]
+        trained = S.Dataset(X, Y).train(S.LinearRegression()).loss(S.MeanSquaredError).using(sa(**case["args"])) \
+            .batch(97).epochs(case["epochs"]).run()
+        final = trained.loss(X, Y)
+        assert final <= case["max_loss"], (case, final)
+        oparams, _, ohist = O.train(om, oa(**case["args"]), [(X, Y)], 97, case["epochs"], init)
+        ofinal = float(om.loss_of(X, Y, oparams))
+        assert abs(final - ofinal) <= TOL_TRAJECTORY * ofinal, (case, final, ofinal)
+        assert trained.iterations == case["epochs"]
+        np.testing.assert_allclose(trained.history, ohist, rtol=TOL_TRAJECTORY)
+    g = golden["convergence"]["logistic_adam"]
+    Xl, Yl = logistic_data
+    ds = S.Dataset(Xl, Yl)
+    trained = ds.train(S.LogisticRegression()).loss(S.BinaryCrossentropy).using(S.Adam(g["rate"])).batch(g["batch"]) \
+        .epochs(g["epochs"]).run()
+    assert trained.loss(Xl, Yl) <= g["max_loss"]
+    assert S.accuracy(trained, ds) >= g["min_accuracy"]
+    np.testing.assert_array_equal(np.rint(trained.result(A(g["predict_in"]))), A(g["predict_rounded"]))
+    # accuracy count is exactly the oracle's
+    om2 = O.Model([O.Dense(1, O.ACT_SIGMOID)], O.LOSS_BCE)
+    assert round(S.accuracy(trained, ds, batch=33) * len(ds)) == O.count_correct(om2, Xl, Yl, trained.params)
+
+
+def test_k_replica_training_matches_oracle(S, linear_function):
+    """K = 3 partitions: per-epoch broadcast, independent epochs, uniform average, summed iterations."""
+    X, Y = linear_function
+    X, Y = X[:96], Y[:96]
+    om = O.Model([O.Dense(1)], O.LOSS_MSE)
+    init = {"0/weights": np.zeros((1, 1), f32), "1/weights": np.zeros(1, f32)}
+    parts = [(X[i * 32:(i + 1) * 32], Y[i * 32:(i + 1) * 32]) for i in range(3)]
+    oparams, _, ohist = O.train(om, O.Adam(0.1), parts, 16, 20, init)
+    trained = S.Dataset(X, Y, partitions=3).train(S.LinearRegression()).loss(S.MeanSquaredError).using(S.Adam(0.1)) \
+        .batch(16).epochs(20).run()
+    assert trained.iterations == 20 * 6
+    np.testing.assert_allclose(trained.history, ohist, rtol=TOL_TRAJECTORY)
+    for p in oparams:
+        assert rel_err(trained.params[p], oparams[p]) <= 1e-4
+
+
+def test_error_paths(S, ctx):
+    with pytest.raises(S.ScanetError):
+        S.Context(99)
+    spec_layers = (S.Dense(4, S.Sigmoid)).layers
+    cm = S.CompiledModel(ctx, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3,), 8)
+    rep = cm.replica(None)
+    x = ctx.alloc(24)
+    y = ctx.alloc(32)
+    with pytest.raises(S.ScanetError):
+        rep.step(x, y, 1)                                   # no optimizer
+    with pytest.raises(S.ScanetError):
+        rep.forward(x, rows=9)                              # more rows than the compiled batch
+    with pytest.raises(S.ScanetError):
+        rep.set_params({"0/weights": np.zeros((3, 5), f32)})   # wrong element count
+    with pytest.raises(KeyError):
+        rep.set_params({"7/weights": np.zeros((3, 4), f32)})
+    with pytest.raises(S.ScanetError):
+        cm.close()                                          # replicas still alive
+    rep.close()
+    cm.close()
+    with pytest.raises(S.ScanetError):                      # Dense straight on an image
+        S.CompiledModel(ctx, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3, 3, 1), 8)
+    with pytest.raises(S.ScanetError):                      # kernel larger than the input
+        S.CompiledModel(ctx, [S.Conv2D(2, (5, 5)).desc()], S.MeanSquaredError.kind, (3, 3, 1), 8)
+    x.free()
+    y.free()
