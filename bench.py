@@ -1,0 +1,348 @@
+#!/usr/bin/env python3
+"""Benchmark of the scanet training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload lenet|mlp|lstm|wide_mlp|optim] [--no-extras]
+
+One "step" is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM when the timed region starts.  The headline value is train samples/s of the
+LeNet-style CNN (the second configuration of the baseline list); with extras on (default) the
+same JSON line also carries the other configurations: the small MLP, the LSTM, the wide bf16
+MLP (GEMM roofline) and the 100 M-element optimizer / 8-replica averaging sweep (HBM roofline).
+
+`roofline.achieved` = algorithmic work per launch of the dominant kernel divided by that
+kernel's average launch duration, measured here with HIP events on the stream the kernels are
+launched on (the library brackets every launch when profiling is enabled).
+`cpu_baseline` times the CPU oracle (oracle/) on this box's host cores on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+PEAK_FP32_MFMA = 157.3         # TFLOP/s dense
+PEAK_BF16_MFMA = 2500.0        # TFLOP/s dense
+SEED = 20251125
+
+
+def lenet_layers(S, pool_stride=1):
+    ps = (pool_stride, pool_stride)
+    return (S.Conv2D(32, activation=S.ReLU()) >> S.Pool2D(strides=ps) >> S.Conv2D(64, activation=S.ReLU())
+            >> S.Pool2D(strides=ps) >> S.Flatten >> S.Dense(10, S.Softmax))
+
+
+def glorot(rng, shape):
+    fan_in, fan_out = int(np.prod(shape[:-1])), shape[-1]
+    lim = np.sqrt(6.0 / (fan_in + fan_out))
+    return rng.uniform(-lim, lim, shape).astype(np.float32)
+
+
+def init_params(cm, rng):
+    out = {}
+    for path, shape, _ in cm.params:
+        if len(shape) == 1:
+            out[path] = np.ones(shape, np.float32) if "forget/1/" in path else np.zeros(shape, np.float32)
+        else:
+            out[path] = glorot(rng, shape)
+    return out
+
+
+def one_hot(rng, rows, classes):
+    return np.eye(classes, dtype=np.float32)[rng.integers(0, classes, rows)]
+
+
+def kernel_table(ctx):
+    rep = ctx.profile_report()
+    return {k: {"total_ms": v[0], "launches": v[1], "avg_us": 1e3 * v[0] / max(v[1], 1)} for k, v in rep.items()}
+
+
+def gemm_flops(name):
+    m = re.search(r"\[(\d+)x(\d+)x(\d+)\]", name)
+    if not m:
+        return None
+    M, N, K = (int(v) for v in m.groups())
+    return 2.0 * M * N * K
+
+
+def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy, n_batches, steps, warmup, flags=0):
+    """Times `steps` training steps (forward, loss, backward, update) cycling over n_batches resident batches."""
+    rng = np.random.default_rng(SEED)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], loss.kind, in_shape, batch, flags)
+    rep = cm.replica(alg)
+    rep.set_params(init_params(cm, rng))
+    X, Y = make_xy(rng, batch * n_batches)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    xs, ys = batch * cm.in_elems, batch * cm.out_elems
+    it = 0
+
+    def step():
+        nonlocal it
+        b = it % n_batches
+        it += 1
+        rep.step(Xb.offset(b * xs), Yb.offset(b * ys), it)
+
+    for _ in range(warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    first_loss = None
+    # second, instrumented pass: per-kernel durations from HIP events on the library's stream
+    ctx.profile_reset()
+    ctx.profile(True)
+    prof_steps = max(3, min(steps, 20))
+    for _ in range(prof_steps):
+        step()
+    ctx.profile(False)
+    kernels = kernel_table(ctx)
+    for k in kernels.values():
+        k["per_step_us"] = 1e3 * k["total_ms"] / prof_steps
+    last_loss = rep.loss(Xb.offset(0), Yb.offset(0))
+    n_params = sum(int(np.prod(s)) for _, s, _ in cm.params)
+    rep.close()
+    cm.close()
+    Xb.free()
+    Yb.free()
+    return {"workload": name, "samples_per_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps, "steps": steps,
+            "batch": batch, "params": n_params, "loss_after": last_loss, "kernels": kernels}
+
+
+def dominant_gemm_roofline(kernels, peak_tflops):
+    """Roofline entry for the matrix-core kernel that takes the most time."""
+    best = None
+    for name, k in kernels.items():
+        fl = gemm_flops(name)
+        if fl is None:
+            continue
+        if best is None or k["total_ms"] > best[1]["total_ms"]:
+            best = (name, k, fl)
+    if best is None:
+        return None
+    name, k, fl = best
+    ach = fl / (k["avg_us"] * 1e-6) / 1e12
+    return {"kernel": name, "bound": "mfma", "achieved": ach, "peak": peak_tflops, "unit": "TFLOP/s", "frac": ach / peak_tflops,
+            "avg_launch_us": k["avg_us"], "flops_per_launch": fl, "traffic": None}
+
+
+def bench_lenet(S, ctx, steps, warmup, pool_stride=1):
+    return run_model_workload(
+        S, ctx, f"LeNet-style CNN 28x28x1, batch 100, Adam 1e-3, fp32, pool stride {pool_stride}", lenet_layers(S, pool_stride),
+        S.CategoricalCrossentropy, (28, 28, 1), 100, S.Adam(1e-3),
+        lambda rng, n: (rng.random((n, 28, 28, 1), np.float32), one_hot(rng, n, 10)), 100, steps, warmup)
+
+
+def bench_mlp(S, ctx, steps, warmup):
+    return run_model_workload(
+        S, ctx, "MLP 784->50 sigmoid->10 softmax, batch 1000, Adam 0.01, fp32", S.Dense(50, S.Sigmoid) >> S.Dense(10, S.Softmax),
+        S.CategoricalCrossentropy, (784,), 1000, S.Adam(0.01),
+        lambda rng, n: (rng.random((n, 784), np.float32), one_hot(rng, n, 10)), 30, steps, warmup)
+
+
+def bench_lstm(S, ctx, steps, warmup):
+    return run_model_workload(
+        S, ctx, "LSTM(256)->Dense(1,tanh), batch 512, T 64, F 32, Adam, MSE, fp32", S.LSTM(256) >> S.Dense(1, S.Tanh),
+        S.MeanSquaredError, (64, 32), 512, S.Adam(),
+        lambda rng, n: (rng.standard_normal((n, 64, 32)).astype(np.float32), rng.uniform(-1, 1, (n, 1)).astype(np.float32)),
+        4, steps, warmup)
+
+
+def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
+    from scanet3_amd import _lib as L
+    return run_model_workload(
+        S, ctx, "MLP 4096->4096 relu->4096 relu->1000 softmax, batch 8192, Adam 1e-3, " + ("bf16 MFMA / fp32 acc" if bf16 else "fp32"),
+        S.Dense(4096, S.ReLU()) >> S.Dense(4096, S.ReLU()) >> S.Dense(1000, S.Softmax),
+        S.CategoricalCrossentropy, (4096,), 8192, S.Adam(1e-3),
+        lambda rng, n: (rng.standard_normal((n, 4096)).astype(np.float32), one_hot(rng, n, 1000)), 1, steps, warmup,
+        flags=L.FLAG_GEMM_BF16 if bf16 else 0)
+
+
+OPT_BYTES = {"sgd": 20, "adagrad": 20, "rmsprop": 20, "adadelta": 28, "adam": 28, "nadam": 28, "adamax": 28, "amsgrad": 36}
+
+
+def bench_optim(S, ctx, steps, warmup, n=100_000_000, k=8, n_avg=25_000_000):
+    """One fused update per optimizer over n float32 parameters, then the mean of k replicas of n_avg."""
+    rng = np.random.default_rng(SEED + 5)
+    block = 1 << 20
+    reps = -(-n // block)
+    w = np.tile((rng.standard_normal(block) * 0.02).astype(np.float32), reps)[:n]
+    g = np.tile((rng.standard_normal(block) * 1e-3).astype(np.float32), reps)[:n]
+    wb, gb = ctx.to_device(w), ctx.to_device(g)
+    states = [ctx.alloc(n) for _ in range(3)]
+    algs = [("sgd", S.SGD()), ("adagrad", S.AdaGrad()), ("adadelta", S.AdaDelta()), ("rmsprop", S.RMSProp()), ("adam", S.Adam()),
+            ("nadam", S.Nadam()), ("adamax", S.Adamax()), ("amsgrad", S.AMSGrad())]
+    out = {}
+    ctx.profile_reset()
+    for name, desc in algs:
+        ns = {20: 1, 28: 2, 36: 3}[OPT_BYTES[name]]
+        for s in states[:ns]:
+            s.fill(desc.init_acc)
+        wb.copy_from(w)
+        it = 0
+        for _ in range(warmup):          # warm-up steps also move the state off its degenerate initial value
+            it += 1
+            ctx.optimizer_update(desc, wb, gb, states[:ns], it)
+        ctx.sync()
+        ctx.profile(True)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            it += 1
+            ctx.optimizer_update(desc, wb, gb, states[:ns], it)
+        ctx.sync()
+        dt = time.perf_counter() - t0
+        ctx.profile(False)
+        kern = ctx.profile_report()[f"optimizer_{name}"]
+        avg_s = kern[0] / kern[1] * 1e-3
+        out[name] = {"bytes_per_elem": OPT_BYTES[name], "ms_per_step": 1e3 * dt / steps, "kernel_avg_us": avg_s * 1e6,
+                     "GBps": OPT_BYTES[name] * n / avg_s / 1e9, "frac_of_peak": OPT_BYTES[name] * n / avg_s / 1e9 / PEAK_HBM_GBS,
+                     "elems_per_s": n / avg_s}
+    for b in states + [wb, gb]:
+        b.free()
+    # averaging
+    base = (rng.standard_normal(block) * 0.02).astype(np.float32)
+    reps_bufs = []
+    for r in range(k):
+        reps_bufs.append(ctx.to_device(np.tile(np.roll(base, r * 17), -(-n_avg // block))[:n_avg]))
+    dst = ctx.alloc(n_avg)
+    for _ in range(warmup):
+        ctx.average(reps_bufs, dst)
+    ctx.sync()
+    ctx.profile_reset()
+    ctx.profile(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ctx.average(reps_bufs, dst)
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    ctx.profile(False)
+    kern = ctx.profile_report()["average_replicas"]
+    avg_s = kern[0] / kern[1] * 1e-3
+    bpe = 4 * (k + 1)
+    out["average"] = {"k": k, "n": n_avg, "bytes_per_elem": bpe, "ms_per_step": 1e3 * dt / steps, "kernel_avg_us": avg_s * 1e6,
+                      "GBps": bpe * n_avg / avg_s / 1e9, "frac_of_peak": bpe * n_avg / avg_s / 1e9 / PEAK_HBM_GBS}
+    for b in reps_bufs + [dst]:
+        b.free()
+    return {"workload": f"fused optimizer updates over {n} fp32 params + average of {k} x {n_avg}", "n": n, "results": out}
+
+
+def cpu_baseline_lenet(pool_stride=1, budget_s=15.0):
+    """The oracle's LeNet step on the host cores; bounded to about `budget_s` seconds."""
+    from oracle import scanet_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    ps = (pool_stride, pool_stride)
+    model = O.Model([O.Conv2D(32, activation=O.ACT_RELU), O.Pool2D(strides=ps), O.Conv2D(64, activation=O.ACT_RELU),
+                     O.Pool2D(strides=ps), O.Flatten(), O.Dense(10, O.ACT_SOFTMAX)], O.LOSS_CCE)
+    rng = np.random.default_rng(SEED)
+    batch = 100
+    params = {p: (glorot(rng, s) if len(s) > 1 else np.zeros(s, np.float32)) for p, s in model.param_defs((batch, 28, 28, 1))}
+    alg = O.Adam(1e-3)
+    state = O.init_opt_state(alg, params)
+    x = rng.random((batch, 28, 28, 1), np.float32)
+    y = one_hot(rng, batch, 10)
+    params, state, _, _ = O.train_step(model, alg, x, y, params, state, 1)      # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        n += 1
+        params, state, _, _ = O.train_step(model, alg, x, y, params, state, n + 1)
+        if time.perf_counter() - t0 > budget_s or n >= 200:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": batch * n / dt, "unit": "samples/s", "cores": int(threads), "kind": "port",
+            "sample": f"{n} LeNet training steps of batch {batch} (numpy oracle, BLAS threads = {threads})"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="lenet", choices=["lenet", "mlp", "lstm", "wide_mlp", "optim"])
+    ap.add_argument("--pool-stride", type=int, default=1, help="LeNet pool stride (reference default 1)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import scanet3_amd as S
+    ctx = S.Context(0)
+    dev_name, hbm, cu = ctx.device_info()
+    steps, warmup = args.steps, args.warmup
+
+    def run(which, st, wu):
+        if which == "lenet":
+            return bench_lenet(S, ctx, st, wu, args.pool_stride)
+        if which == "mlp":
+            return bench_mlp(S, ctx, st, wu)
+        if which == "lstm":
+            return bench_lstm(S, ctx, st, wu)
+        if which == "wide_mlp":
+            return bench_wide_mlp(S, ctx, st, wu)
+        return bench_optim(S, ctx, st, wu)
+
+    main_res = run(args.workload, steps, warmup)
+    line = {"metric": "train samples/sec on 1 GPU", "unit": "samples/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "data": "synthetic", "dtype": "f32",
+            "device": dev_name}
+    if args.workload == "optim":
+        adam = main_res["results"]["adam"]
+        line.update({"metric": "fused Adam update, elements/s over 100M fp32 params", "unit": "elements/s",
+                     "value": adam["elems_per_s"], "ms_per_step": adam["ms_per_step"],
+                     "config": {"workload": main_res["workload"]},
+                     "roofline": {"kernel": "optimizer_adam", "bound": "hbm", "achieved": adam["GBps"], "peak": PEAK_HBM_GBS,
+                                  "unit": "GB/s", "frac": adam["frac_of_peak"], "traffic": None},
+                     "optimizers": main_res["results"]})
+    else:
+        peak = PEAK_BF16_MFMA if args.workload == "wide_mlp" else PEAK_FP32_MFMA
+        line.update({"value": main_res["samples_per_s"], "ms_per_step": main_res["ms_per_step"],
+                     "dtype": "bf16" if args.workload == "wide_mlp" else "f32",
+                     "config": {"workload": main_res["workload"], "batch": main_res["batch"], "params": main_res["params"]},
+                     "roofline": dominant_gemm_roofline(main_res["kernels"], peak),
+                     "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
+                                             sorted(main_res["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:12]}})
+    if not args.no_extras:
+        extras = {}
+        for which, st, wu in (("mlp", 100, 10), ("lstm", 10, 2), ("wide_mlp", 5, 2), ("optim", 10, 3), ("lenet", 50, 5)):
+            if which == args.workload:
+                continue
+            try:
+                r = run(which, st, wu)
+            except Exception as e:        # an extra must never hide the headline number
+                extras[which] = {"error": str(e)}
+                continue
+            if which == "optim":
+                extras[which] = r
+            else:
+                peak = PEAK_BF16_MFMA if which == "wide_mlp" else PEAK_FP32_MFMA
+                extras[which] = {"workload": r["workload"], "samples_per_s": r["samples_per_s"], "ms_per_step": r["ms_per_step"],
+                                 "steps": r["steps"], "loss_after": r["loss_after"],
+                                 "roofline": dominant_gemm_roofline(r["kernels"], peak),
+                                 "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
+                                                         sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}
+        line["other_configs"] = extras
+    ctx.close()
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_lenet(args.pool_stride)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

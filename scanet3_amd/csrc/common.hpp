@@ -46,7 +46,7 @@ struct ProfileEntry {
 
 struct PendingEvent {
   hipEvent_t start, stop;
-  const char* name;
+  std::string name;
 };
 
 }  // namespace sn
@@ -75,8 +75,10 @@ constexpr uint32_t REPLICA_MAGIC = 0x534e5250u;
 struct LaunchScope {
   sn_ctx* ctx;
   hipEvent_t start = nullptr, stop = nullptr;
-  const char* name;
+  std::string name;
   LaunchScope(sn_ctx* c, const char* n);
+  LaunchScope(sn_ctx* c, const char* n, int m, int nn, int k);  // name becomes "n[MxNxK]"
+  void begin();
   ~LaunchScope();
 };
 int profile_drain(sn_ctx* ctx);

@@ -494,7 +494,7 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   splits = (int)ceil_div(K, k_per_split);
   const dim3 grid((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), (unsigned)splits);
   {
-    LaunchScope scope(ctx, name);
+    LaunchScope scope(ctx, name, M, N, K);
     hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
                        splits > 1 ? ws : nullptr);
   }

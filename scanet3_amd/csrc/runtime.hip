@@ -20,8 +20,21 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-LaunchScope::LaunchScope(sn_ctx* c, const char* n) : ctx(c), name(n) {
+LaunchScope::LaunchScope(sn_ctx* c, const char* n) : ctx(c) {
   if (!ctx->profiling) return;
+  name = n;
+  begin();
+}
+
+LaunchScope::LaunchScope(sn_ctx* c, const char* n, int m, int nn, int k) : ctx(c) {
+  if (!ctx->profiling) return;
+  char buf[160];
+  snprintf(buf, sizeof(buf), "%s[%dx%dx%d]", n, m, nn, k);
+  name = buf;
+  begin();
+}
+
+void LaunchScope::begin() {
   if (ctx->pending.size() >= 8192) profile_drain(ctx);
   auto take = [&](hipEvent_t& e) {
     if (!ctx->event_pool.empty()) {
