@@ -100,57 +100,63 @@ constexpr int n_states() {
   return (KIND == SN_OPT_SGD || KIND == SN_OPT_ADAGRAD || KIND == SN_OPT_RMSPROP) ? 1 : (KIND == SN_OPT_AMSGRAD ? 3 : 2);
 }
 
-// One float4 per lane per iteration, UNROLL independent iterations in flight.
-template <int KIND, int UNROLL>
+// A block owns 256*U consecutive float4 of every array and touches ONE ARRAY AT A TIME: U loads of w,
+// then U of g, ... then the stores array by array.  Each wavefront so issues U back-to-back 1 KiB rows of
+// the same stream; measured on MI355X this keeps 4 read + 3 write streams at about 6.1 TB/s where the
+// element-interleaved order reaches 5.6 TB/s.  U = 4 is the sweet spot (8 spills registers).
+template <int KIND, int U>
 __global__ __launch_bounds__(256) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
                                                             f4* __restrict__ s1, f4* __restrict__ s2, int64_t n4,
                                                             OptScalars p) {
   constexpr int NS = n_states<KIND>();
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + (UNROLL - 1) * stride < n4; i += UNROLL * stride) {
-    f4 vw[UNROLL], vg[UNROLL], a[UNROLL], b[UNROLL], c[UNROLL];
+  const int64_t base = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  f4 vw[U], vg[U], a[U], b[U], c[U];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t j = i + u * stride;
-      vw[u] = __builtin_nontemporal_load(w + j);
-      vg[u] = __builtin_nontemporal_load(g + j);
-      a[u] = __builtin_nontemporal_load(s0 + j);
-      if (NS > 1) b[u] = __builtin_nontemporal_load(s1 + j);
-      if (NS > 2) c[u] = __builtin_nontemporal_load(s2 + j);
-    }
+  for (int u = 0; u < U; ++u)
+    if (base + u * 256 < n4) vw[u] = __builtin_nontemporal_load(w + base + u * 256);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t j = i + u * stride;
+  for (int u = 0; u < U; ++u)
+    if (base + u * 256 < n4) vg[u] = __builtin_nontemporal_load(g + base + u * 256);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float ww = vw[u][e], aa = a[u][e], bb = NS > 1 ? b[u][e] : 0.f, cc = NS > 2 ? c[u][e] : 0.f;
-        update_one<KIND>(ww, vg[u][e], aa, bb, cc, p);
-        vw[u][e] = ww;
-        a[u][e] = aa;
-        if (NS > 1) b[u][e] = bb;
-        if (NS > 2) c[u][e] = cc;
-      }
-      __builtin_nontemporal_store(vw[u], w + j);
-      __builtin_nontemporal_store(a[u], s0 + j);
-      if (NS > 1) __builtin_nontemporal_store(b[u], s1 + j);
-      if (NS > 2) __builtin_nontemporal_store(c[u], s2 + j);
-    }
+  for (int u = 0; u < U; ++u)
+    if (base + u * 256 < n4) a[u] = __builtin_nontemporal_load(s0 + base + u * 256);
+  if (NS > 1) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) b[u] = __builtin_nontemporal_load(s1 + base + u * 256);
   }
-  for (; i < n4; i += stride) {
-    f4 vw = w[i], vg = g[i], a = s0[i], b = {0, 0, 0, 0}, c = {0, 0, 0, 0};
-    if (NS > 1) b = s1[i];
-    if (NS > 2) c = s2[i];
+  if (NS > 2) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) c[u] = __builtin_nontemporal_load(s2 + base + u * 256);
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      float ww = vw[e], aa = a[e], bb = b[e], cc = c[e];
-      update_one<KIND>(ww, vg[e], aa, bb, cc, p);
-      vw[e] = ww; a[e] = aa; b[e] = bb; c[e] = cc;
+      float ww = vw[u][e], aa = a[u][e], bb = NS > 1 ? b[u][e] : 0.f, cc = NS > 2 ? c[u][e] : 0.f;
+      update_one<KIND>(ww, vg[u][e], aa, bb, cc, p);
+      vw[u][e] = ww;
+      a[u][e] = aa;
+      if (NS > 1) b[u][e] = bb;
+      if (NS > 2) c[u][e] = cc;
     }
-    w[i] = vw;
-    s0[i] = a;
-    if (NS > 1) s1[i] = b;
-    if (NS > 2) s2[i] = c;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (base + u * 256 < n4) __builtin_nontemporal_store(vw[u], w + base + u * 256);
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+    if (base + u * 256 < n4) __builtin_nontemporal_store(a[u], s0 + base + u * 256);
+  if (NS > 1) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) __builtin_nontemporal_store(b[u], s1 + base + u * 256);
+  }
+  if (NS > 2) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) __builtin_nontemporal_store(c[u], s2 + base + u * 256);
   }
 }
 
@@ -180,10 +186,8 @@ static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g,
   const bool vec = aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2);
   const int64_t n4 = vec ? n / 4 : 0;
   if (n4 > 0) {
-    // enough workgroups to cover every CU several times over; each lane keeps UNROLL float4 per array in flight
-    int64_t blocks = ceil_div(n4, (int64_t)256 * UNROLL);
-    const int64_t cap = (int64_t)ctx->compute_units * 16;
-    if (blocks > cap) blocks = cap;
+    const int64_t blocks = ceil_div(n4, (int64_t)256 * UNROLL);  // one pass, no grid-stride loop
+    SN_REQUIRE(blocks <= 0x7fffffff, "optimizer update over %lld elements exceeds one launch", (long long)n);
     LaunchScope scope(ctx, name);
     hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (f4*)w,
                        (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p);
@@ -227,25 +231,39 @@ struct AvgOutputs {
   float* p[SN_MAX_AVG_INPUTS + 1];
 };
 
-template <int K_STATIC>
+// Block-contiguous like the optimizer kernel: a block owns 256*U float4, reads them input by input.
+template <int K_STATIC, int U>
 __global__ __launch_bounds__(256) void average_kernel_v4(AvgInputs in, int k, int64_t n4, AvgOutputs out, int n_out, float kf) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    f4 acc;
-    if constexpr (K_STATIC > 0) {
-      f4 v[K_STATIC];
+  const int64_t base = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  f4 acc[U];
+  if constexpr (K_STATIC > 0) {
+    f4 v[K_STATIC][U];
 #pragma unroll
-      for (int r = 0; r < K_STATIC; ++r) v[r] = __builtin_nontemporal_load((const f4*)in.p[r] + i);
-      acc = v[0];
+    for (int r = 0; r < K_STATIC; ++r)
 #pragma unroll
-      for (int r = 1; r < K_STATIC; ++r) acc = acc + v[r];  // AddN, left to right
-    } else {
-      acc = ((const f4*)in.p[0])[i];
-      for (int r = 1; r < k; ++r) acc = acc + ((const f4*)in.p[r])[i];
+      for (int u = 0; u < U; ++u)
+        if (base + u * 256 < n4) v[r][u] = __builtin_nontemporal_load((const f4*)in.p[r] + base + u * 256);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc[u] = v[0][u];
+#pragma unroll
+      for (int r = 1; r < K_STATIC; ++r) acc[u] = acc[u] + v[r][u];  // AddN, left to right
     }
-    acc = acc / kf;  // `plus(inputs) / inputs.size` (models/Aggregation.scala:16-19)
-    for (int o = 0; o < n_out; ++o) __builtin_nontemporal_store(acc, (f4*)out.p[o] + i);
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) acc[u] = __builtin_nontemporal_load((const f4*)in.p[0] + base + u * 256);
+    for (int r = 1; r < k; ++r)
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (base + u * 256 < n4) acc[u] = acc[u] + __builtin_nontemporal_load((const f4*)in.p[r] + base + u * 256);
   }
+#pragma unroll
+  for (int u = 0; u < U; ++u) acc[u] = acc[u] / kf;  // `plus(inputs) / inputs.size` (models/Aggregation.scala:16-19)
+  for (int o = 0; o < n_out; ++o)
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (base + u * 256 < n4) __builtin_nontemporal_store(acc[u], (f4*)out.p[o] + base + u * 256);
 }
 
 __global__ __launch_bounds__(256) void average_kernel_scalar(AvgInputs in, int k, int64_t first, int64_t n, AvgOutputs out,
@@ -273,18 +291,18 @@ int launch_average(sn_ctx* ctx, const AvgInputs& in, int k, int64_t n, float* ou
   const int64_t n4 = vec ? n / 4 : 0;
   const float kf = (float)k;
   if (n4 > 0) {
-    int64_t blocks = ceil_div(n4, 256);
-    const int64_t cap = (int64_t)ctx->compute_units * 16;
-    if (blocks > cap) blocks = cap;
+    constexpr int U = 2;
+    const int64_t blocks = ceil_div(n4, 256 * U);
+    SN_REQUIRE(blocks <= 0x7fffffff, "average over %lld elements exceeds one launch", (long long)n);
     LaunchScope scope(ctx, "average_replicas");
     if (k == 8)
-      hipLaunchKernelGGL((average_kernel_v4<8>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<8, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else if (k == 4)
-      hipLaunchKernelGGL((average_kernel_v4<4>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<4, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else if (k == 2)
-      hipLaunchKernelGGL((average_kernel_v4<2>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<2, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else
-      hipLaunchKernelGGL((average_kernel_v4<0>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<0, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
   }
   if (n4 * 4 < n) {
     LaunchScope scope(ctx, "average_replicas");
