@@ -77,6 +77,18 @@ def sqrt_zero_safe(x, eps):
     return np.sqrt(x + _c(eps, x))
 
 
+def to_bf16(x):
+    """float32 values rounded to the nearest bfloat16 (ties to even), returned as float32.
+
+    Used only by the bf16 Dense mode, which has no counterpart in the reference (its arithmetic is
+    float32 throughout): the HIP library's bf16 GEMMs are checked against float32 products of
+    operands rounded this way."""
+    a = np.ascontiguousarray(x, dtype=np.float32)
+    u = a.view(np.uint32)
+    r = ((u >> 16) & 1) + np.uint32(0x7FFF)
+    return ((u + r) & np.uint32(0xFFFF0000)).view(np.float32)
+
+
 def rint(x):
     """TF `Rint`: round half to even (AllKernels.scala:339-345)."""
     return np.rint(x)
@@ -432,7 +444,8 @@ def SimpleRNN(units, activation=ACT_TANH, bias=True):
 class Model:
     """A `Composed` model: flattened layers, index-prefixed parameter paths (Composed.scala:22-31)."""
 
-    def __init__(self, layers: Sequence, loss: int = LOSS_MSE):
+    def __init__(self, layers: Sequence, loss: int = LOSS_MSE, bf16_dense: bool = False):
+        self.bf16_dense = bf16_dense
         flat: List[Layer] = []
         for l in layers:
             flat.extend(l if isinstance(l, (list, tuple)) else [l])
@@ -463,6 +476,8 @@ class Model:
             k = l.kind
             if k == "dense":
                 w = params[pre + "weights"]
+                if self.bf16_dense:
+                    x, w = to_bf16(x), to_bf16(w)
                 y = x @ w                                     # Dense.scala:57-61
                 c = (x, w)
             elif k == "bias":
@@ -523,6 +538,8 @@ class Model:
             k = l.kind
             if k == "dense":
                 xi, w = c
+                if self.bf16_dense:
+                    dy = to_bf16(dy)
                 grads[pre + "weights"] = xi.T @ dy            # AllKernels.scala:382-388
                 dy = dy @ w.T
             elif k == "bias":

@@ -156,6 +156,21 @@ struct GemmDesc {
 };
 int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* workspace, int64_t workspace_elems, bool bf16);
 
+// bf16 fast path (gemm_bf16.hip): C[M,N] = A[M,K] * Bt[N,K]^T, operands bf16 with k contiguous.
+// Besides the fp32 result (e.out, may be null) the epilogue can emit bf16 copies in both orientations,
+// which is how a Dense layer hands its output to the next one without a separate cast pass.
+struct EpilogueBf16 {
+  Epilogue e;
+  void* out_bf = nullptr;    // bf16 [M, e.ldo]
+  void* out_bf_t = nullptr;  // bf16 [N, ld_t]
+  int64_t ld_t = 0;
+};
+int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep);
+// bf16 copies out[rows,cols] and out_t[cols,rows] of an fp32 matrix; with y != null the activation gradient
+// act'(y) * src is what gets cast (and is written to dz in fp32 when dz != null)
+int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
+                          int act, float act_param, float* dz);
+
 struct ConvGeom {
   int n, h, w, cin;      // input
   int ho, wo, cout;      // output

@@ -275,8 +275,49 @@ __global__ __launch_bounds__(256) void col_sum_split_kernel(const float* __restr
   if (wave == 0 && c < cols) part[(int64_t)blockIdx.y * cols + c] = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
 }
 
+// Wide matrices: a lane owns 4 consecutive columns (float4), a wavefront 256 columns = 1 KiB of a row, the
+// block's 4 wavefronts take every 4th row of the slice, 4 rows in flight per lane.
+typedef float cs_f4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void col_sum_wide_kernel(const float* __restrict__ dy, int64_t ld, float* __restrict__ part,
+                                                            int64_t rows, int cols, int64_t rows_per_slice) {
+  __shared__ cs_f4 smem[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) * 4;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
+  const int64_t r1 = r0 + rows_per_slice < rows ? r0 + rows_per_slice : rows;
+  cs_f4 s = {0.f, 0.f, 0.f, 0.f};
+  if (c < cols) {
+    int64_t r = r0 + wave;
+    for (; r + 12 < r1; r += 16) {
+      const cs_f4 a = __builtin_nontemporal_load((const cs_f4*)(dy + r * ld + c));
+      const cs_f4 b = __builtin_nontemporal_load((const cs_f4*)(dy + (r + 4) * ld + c));
+      const cs_f4 d = __builtin_nontemporal_load((const cs_f4*)(dy + (r + 8) * ld + c));
+      const cs_f4 e = __builtin_nontemporal_load((const cs_f4*)(dy + (r + 12) * ld + c));
+      s = (((s + a) + b) + d) + e;
+    }
+    for (; r < r1; r += 4) s = s + *(const cs_f4*)(dy + r * ld + c);
+  }
+  smem[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && c < cols) *(cs_f4*)(part + (int64_t)blockIdx.y * cols + c) = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
+}
+
 int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems) {
   if (cols <= 0) return SN_OK;
+  if (cols >= 256 && cols % 4 == 0 && ld % 4 == 0 && rows >= 512 && ws && ws_elems >= 2 * (int64_t)cols &&
+      (reinterpret_cast<uintptr_t>(dy) & 15u) == 0 && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
+    const unsigned cb = (unsigned)ceil_div(cols, 256);
+    int64_t slices = std::min<int64_t>(ceil_div(rows, 64), ceil_div((int64_t)ctx->compute_units * 8, cb));
+    slices = std::max<int64_t>(1, std::min<int64_t>(slices, ws_elems / cols));
+    const int64_t per = ceil_div(rows, slices);
+    slices = ceil_div(rows, per);
+    LaunchScope scope(ctx, "bias_gradient");
+    hipLaunchKernelGGL(col_sum_wide_kernel, dim3(cb, (unsigned)slices), dim3(256), 0, ctx->stream, dy, ld, ws, rows, cols, per);
+    hipLaunchKernelGGL(col_sum_kernel, dim3((unsigned)ceil_div(cols, 64)), dim3(256), 0, ctx->stream, (const float*)ws, (int64_t)cols, out,
+                       slices, cols);
+    SN_HIP(hipGetLastError());
+    return SN_OK;
+  }
   const unsigned col_blocks = (unsigned)ceil_div(cols, 64);
   int64_t slices = 1;
   if (rows >= 512 && ws) {

@@ -80,6 +80,9 @@ struct sn_replica {
   std::vector<float*> lstm_gates, lstm_c, lstm_h, lstm_dz;  // per op
   float* lstm_dh[2] = {nullptr, nullptr};
   float* lstm_dc = nullptr;
+  // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
+  std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
+  bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
   std::vector<void*> owned;
 };
 
@@ -298,6 +301,11 @@ static int dev_alloc(sn_replica* r, T** out, int64_t elems) {
   return SN_OK;
 }
 
+// The 256x256 bf16 kernel needs 16-byte chunks of 8 k-values in every operand row.
+static bool dense_bf16_fast(const sn_model* m, const Op& op) {
+  return (m->flags & SN_FLAG_GEMM_BF16) && op.kind == OP_DENSE && op.in_elems % 8 == 0 && op.out_elems % 8 == 0 && m->batch % 8 == 0;
+}
+
 static float* param_ptr(sn_replica* r, float* base, int idx) { return idx < 0 ? nullptr : base + r->model->params[idx].info.offset; }
 
 static int alloc_replica(sn_replica* r) {
@@ -319,6 +327,8 @@ static int alloc_replica(sn_replica* r) {
   r->lstm_c.assign(n_ops, nullptr);
   r->lstm_h.assign(n_ops, nullptr);
   r->lstm_dz.assign(n_ops, nullptr);
+  r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
+  r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
   int64_t lstm_z = 0, lstm_h = 0;
   for (size_t i = 0; i < n_ops; ++i) {
     const Op& op = m->ops[i];
@@ -336,6 +346,14 @@ static int alloc_replica(sn_replica* r) {
     }
     SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
     if (op.kind == OP_POOL) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
+    if (dense_bf16_fast(m, op)) {
+      SN_TRY(dev_alloc(r, &r->bf_x[i], B * op.in_elems));
+      SN_TRY(dev_alloc(r, &r->bf_xt[i], B * op.in_elems));
+      SN_TRY(dev_alloc(r, &r->bf_dz[i], B * op.out_elems));
+      SN_TRY(dev_alloc(r, &r->bf_dzt[i], B * op.out_elems));
+      SN_TRY(dev_alloc(r, &r->bf_w[i], op.in_elems * op.out_elems));
+      SN_TRY(dev_alloc(r, &r->bf_wt[i], op.in_elems * op.out_elems));
+    }
   }
   SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
   SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h));
@@ -374,16 +392,39 @@ static int forward(sn_replica* r, const float* x, int rows) {
   sn_model* m = r->model;
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
+  if (bf16 && r->bf_weights_stale) {
+    for (size_t i = 0; i < m->ops.size(); ++i)
+      if (dense_bf16_fast(m, m->ops[i]))
+        SN_TRY(launch_cast_transpose(ctx, param_ptr(r, r->w, m->ops[i].w), m->ops[i].out_elems, (int)m->ops[i].in_elems,
+                                     (int)m->ops[i].out_elems, r->bf_w[i], r->bf_wt[i], nullptr, 0, 0.f, nullptr));
+    r->bf_weights_stale = false;
+  }
+  std::vector<char> bf_ready(m->ops.size() + 1, 0);  // op i's bf16 input copies were written by op i-1's epilogue
   for (size_t i = 0; i < m->ops.size(); ++i) {
     const Op& op = m->ops[i];
     const float* in = op_output(r, (int)i - 1, x, rows);
     switch (op.kind) {
       case OP_DENSE: {
         const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
-        GemmDesc g{in, in_f, 1, param_ptr(r, r->w, op.w), out_f, 1, rows, out_f, in_f};
         Epilogue ep;
         ep.out = r->act[i]; ep.ldo = out_f; ep.bias = param_ptr(r, r->w, op.b); ep.act = op.act; ep.act_param = op.act_param;
-        SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
+        if (dense_bf16_fast(m, op) && rows % 8 == 0) {
+          // X in both orientations (X^T feeds dW later) unless the layer below already wrote them from its
+          // epilogue, then Y = X . (W^T)^T on the matrix cores
+          if (!bf_ready[i]) SN_TRY(launch_cast_transpose(ctx, in, in_f, rows, in_f, r->bf_x[i], r->bf_xt[i], nullptr, 0, 0.f, nullptr));
+          EpilogueBf16 eb;
+          eb.e = ep;
+          if (i + 1 < m->ops.size() && dense_bf16_fast(m, m->ops[i + 1])) {
+            eb.out_bf = r->bf_x[i + 1];
+            eb.out_bf_t = r->bf_xt[i + 1];
+            eb.ld_t = rows;
+            bf_ready[i + 1] = true;
+          }
+          SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_x[i], in_f, r->bf_wt[i], in_f, rows, out_f, in_f, eb));
+        } else {
+          GemmDesc g{in, in_f, 1, param_ptr(r, r->w, op.w), out_f, 1, rows, out_f, in_f};
+          SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
+        }
         break;
       }
       case OP_CONV: {
@@ -452,6 +493,23 @@ static int backward(sn_replica* r, const float* x, int rows) {
     switch (op.kind) {
       case OP_DENSE: {
         const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
+        if (dense_bf16_fast(m, op) && rows % 8 == 0) {
+          // one pass: dZ = act'(Y) * dY in fp32 (bias gradient) and as bf16 in both orientations
+          SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
+                                       op.act != SN_ACT_IDENTITY ? r->act[i] : nullptr, op.act, op.act_param,
+                                       op.act != SN_ACT_IDENTITY ? dy : nullptr));
+          if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
+          EpilogueBf16 ew;
+          ew.e.out = param_ptr(r, r->g, op.w); ew.e.ldo = out_f;
+          SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_xt[i], rows, r->bf_dzt[i], rows, in_f, out_f, rows, ew));  // dW = X^T . dZ
+          if (need_dx) {
+            EpilogueBf16 ex;
+            ex.e.out = dx; ex.e.ldo = in_f;
+            SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
+            cur ^= 1;
+          }
+          break;
+        }
         if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
         if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
         {  // dW = X^T . dY (math/alg/AllKernels.scala:382-388)
@@ -562,6 +620,7 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
 
 static int update(sn_replica* r, int iter) {
   SN_REQUIRE(r->has_opt, "replica was created without an optimizer");
+  r->bf_weights_stale = true;
   return launch_optimizer(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], r->model->flat_elems, iter);
 }
 
@@ -696,6 +755,7 @@ int sn_replica_destroy(sn_replica* rep) {
 int sn_params_set(sn_replica* rep, int32_t index, const float* src_host, int64_t n) {
   SN_TRY(check_replica(rep));
   SN_REQUIRE(src_host != nullptr, "sn_params_set: source is NULL");
+  rep->bf_weights_stale = true;
   return tensor_io(rep, rep->w, index, nullptr, src_host, n);
 }
 int sn_params_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n) {
@@ -726,6 +786,7 @@ int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n) 
   SN_REQUIRE(out_dev != nullptr, "sn_replica_flat: out is NULL");
   SN_REQUIRE(slot >= -2 && slot < rep->n_states, "slot %d out of range", slot);
   *out_dev = slot == -2 ? rep->w : (slot == -1 ? rep->g : rep->s[slot]);
+  if (slot == -2) rep->bf_weights_stale = true;  // the caller may write through the view
   if (n) *n = rep->model->flat_elems;
   return SN_OK;
 }
@@ -821,6 +882,7 @@ int sn_replicas_average(sn_replica* const* reps, int32_t k) {
                "replica %d uses another optimizer", i);
   }
   if (k == 1) return SN_OK;  // treeReduce of one partition never calls aggregateParams
+  for (int i = 0; i < k; ++i) reps[i]->bf_weights_stale = true;
   sn_ctx* ctx = reps[0]->ctx;
   const int64_t n = reps[0]->model->flat_elems;
   for (int slot = -1; slot < reps[0]->n_states; ++slot) {

@@ -515,3 +515,39 @@ def test_error_paths(S, ctx):
         S.CompiledModel(ctx, [S.Conv2D(2, (5, 5)).desc()], S.MeanSquaredError.kind, (3, 3, 1), 8)
     x.free()
     y.free()
+
+
+# ----------------------------------------------------------------------------- bf16 Dense mode (no counterpart in the reference)
+TOL_BF16 = 2e-3   # operands are rounded to bf16 on both sides; what is left is accumulation order and the few
+                  # activations whose float32 last bit flips their bf16 rounding
+
+
+@pytest.mark.parametrize("dims,batch", [((64, 4096, 64, 8), 4096), ((256, 512, 104), 512), ((1000, 264, 40), 136)])
+def test_bf16_dense_path_matches_bf16_rounded_oracle(S, ctx, dims, batch):
+    from scanet3_amd import _lib as L
+    acts = ["relu", "tanh", "sigmoid"]
+    spec = [("dense", d, acts[i % 3]) for i, d in enumerate(dims[1:-1])] + [("dense", dims[-1], "softmax")]
+    rng = np.random.default_rng(20251125 + 4)
+    h = Harness(S, ctx, spec, "cce", (dims[0],), batch, flags=L.FLAG_GEMM_BF16)
+    om = O.Model(h.omodel.layers, O.LOSS_CCE, bf16_dense=True)
+    params = glorot_params(om, (batch, dims[0]), rng)
+    for p in params:
+        if params[p].ndim == 1:
+            params[p] = rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
+    x = rng.standard_normal((batch, dims[0])).astype(f32)
+    y = one_hot(rng, batch, dims[-1])
+    h.rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    assert rel_err(h.rep.forward(xb), om.forward(x, params)) <= TOL_BF16
+    oloss, ograds = om.grad(x, y, params)
+    gloss = h.rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_BF16 * max(1.0, abs(float(oloss)))
+    ggrads = h.rep.get_grads()
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= TOL_BF16, p
+    # and the bf16 result stays close to the float32 one (sanity of the mode itself)
+    o32 = O.Model(h.omodel.layers, O.LOSS_CCE)
+    assert abs(gloss - float(o32.loss_of(x, y, params))) <= 2e-2 * max(1.0, abs(gloss))
+    h.close()
+    xb.free()
+    yb.free()
