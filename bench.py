@@ -168,6 +168,10 @@ def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
         flags=L.FLAG_GEMM_BF16 if bf16 else 0)
 
 
+# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` (two runs, scaled by a copy kernel
+# of known size: WRITE_SIZE x 1.0, FETCH_SIZE x 2.0); summary in profiles/optimizer_100M_and_average_8x25M_hbm_traffic_pmc.md
+MEASURED_TRAFFIC_BYTES = {"sgd": 2.000e9, "adagrad": 2.000e9, "rmsprop": 2.000e9, "adadelta": 2.800e9, "adam": 2.800e9,
+                          "nadam": 2.800e9, "adamax": 2.800e9, "amsgrad": 3.600e9, "average": 0.900e9}
 OPT_BYTES = {"sgd": 20, "adagrad": 20, "rmsprop": 20, "adadelta": 28, "adam": 28, "nadam": 28, "adamax": 28, "amsgrad": 36}
 
 
@@ -231,6 +235,17 @@ def bench_optim(S, ctx, steps, warmup, n=100_000_000, k=8, n_avg=25_000_000):
     bpe = 4 * (k + 1)
     out["average"] = {"k": k, "n": n_avg, "bytes_per_elem": bpe, "ms_per_step": 1e3 * dt / steps, "kernel_avg_us": avg_s * 1e6,
                       "GBps": bpe * n_avg / avg_s / 1e9, "frac_of_peak": bpe * n_avg / avg_s / 1e9 / PEAK_HBM_GBS}
+    # mean of ONE input = a plain copy of known size (n_avg floats in, n_avg out): the reference point that
+    # hardware byte counters of the kernels above are scaled by
+    ctx.profile_reset()
+    ctx.profile(True)
+    for _ in range(steps):
+        ctx.average(reps_bufs[:1], dst)
+    ctx.profile(False)
+    kern = ctx.profile_report()["average_replicas"]
+    avg_s = kern[0] / kern[1] * 1e-3
+    out["copy_k1"] = {"k": 1, "n": n_avg, "bytes_per_elem": 8, "kernel_avg_us": avg_s * 1e6, "GBps": 8 * n_avg / avg_s / 1e9,
+                      "frac_of_peak": 8 * n_avg / avg_s / 1e9 / PEAK_HBM_GBS}
     for b in reps_bufs + [dst]:
         b.free()
     return {"workload": f"fused optimizer updates over {n} fp32 params + average of {k} x {n_avg}", "n": n, "results": out}
@@ -306,7 +321,7 @@ def main():
                      "value": adam["elems_per_s"], "ms_per_step": adam["ms_per_step"],
                      "config": {"workload": main_res["workload"]},
                      "roofline": {"kernel": "optimizer_adam", "bound": "hbm", "achieved": adam["GBps"], "peak": PEAK_HBM_GBS,
-                                  "unit": "GB/s", "frac": adam["frac_of_peak"], "traffic": None},
+                                  "unit": "GB/s", "frac": adam["frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["adam"]},
                      "optimizers": main_res["results"]})
     else:
         peak = PEAK_BF16_MFMA if args.workload == "wide_mlp" else PEAK_FP32_MFMA
@@ -336,6 +351,19 @@ def main():
                                  "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                                          sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}
         line["other_configs"] = extras
+        # the two rooflines the memory-bound and the GEMM-bound configurations are judged on
+        rl = {}
+        opt = extras.get("optim") or (main_res if args.workload == "optim" else None)
+        if opt and "results" in opt:
+            for k in ("adam", "average"):
+                v = opt["results"][k]
+                rl["optimizer_adam_100M" if k == "adam" else "average_8x25M"] = {
+                    "bound": "hbm", "achieved": v["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": v["frac_of_peak"],
+                    "traffic": MEASURED_TRAFFIC_BYTES[k]}
+        wide = extras.get("wide_mlp")
+        if wide and wide.get("roofline"):
+            rl["wide_mlp_gemm_bf16"] = wide["roofline"]
+        line["rooflines"] = rl
     ctx.close()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_lenet(args.pool_stride)
