@@ -15,6 +15,7 @@
 namespace sn {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int BK = 16;
@@ -45,6 +46,17 @@ struct StridedLoader {
   }
   __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
     return (c.ptr && c.k < k_end) ? c.ptr[(int64_t)c.k * s_k] : 0.f;
+  }
+  // 4 values along the contiguous index (k when KC, the outer index otherwise); vec4_ok() guarantees that the
+  // four are inside or outside the matrix together and 16-byte aligned
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.ptr && c.k < k_end) r = *(const f4v*)(c.ptr + (int64_t)c.k * s_k);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int K) const {
+    const bool aligned = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+    return KC ? (s_k == 1 && s_outer % 4 == 0 && K % 4 == 0 && aligned) : (s_outer == 1 && s_k % 4 == 0 && outer_n % 4 == 0 && aligned);
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
 };
@@ -80,6 +92,13 @@ struct ConvFwdA {
     if (iy < 0 || iy >= g.h || ix < 0 || ix >= g.w) return 0.f;
     return c.img[((int64_t)iy * g.w + ix) * g.cin + c.ci];
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {  // ci .. ci+3 of one pixel
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    const int iy = c.iy0 + c.r, ix = c.ix0 + c.q;
+    if (c.img && c.k < k_end && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w) r = *(const f4v*)(c.img + ((int64_t)iy * g.w + ix) * g.cin + c.ci);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const { return g.cin % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0; }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const {
     c.k += dk;
     c.ci += dk;
@@ -123,6 +142,16 @@ struct ConvDgradA {  // m=(b,iy,ix), k=(r,q,co)
     if (oy * g.sh != ny || ox * g.sw != nx || oy >= g.ho || ox >= g.wo) return 0.f;
     return c.img[((int64_t)oy * g.wo + ox) * g.cout + c.co];
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {  // co .. co+3 of one output pixel
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    const int ny = c.ty - c.r, nx = c.tx - c.q;
+    if (c.img && c.k < k_end && ny >= 0 && nx >= 0) {
+      const int oy = ny / g.sh, ox = nx / g.sw;
+      if (oy * g.sh == ny && ox * g.sw == nx && oy < g.ho && ox < g.wo) r = *(const f4v*)(c.img + ((int64_t)oy * g.wo + ox) * g.cout + c.co);
+    }
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const { return g.cout % 4 == 0 && (reinterpret_cast<uintptr_t>(dy) & 15u) == 0; }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const {
     c.k += dk;
     c.co += dk;
@@ -150,6 +179,12 @@ struct ConvDgradB {  // outer n = ci, k=(r,q,co): w[((r*kw+q)*cin + ci)*cout + c
     if (c.ci < 0 || c.k >= k_end) return 0.f;
     return w[((int64_t)c.rq * g.cin + c.ci) * g.cout + c.co];
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.ci >= 0 && c.k < k_end) r = *(const f4v*)(w + ((int64_t)c.rq * g.cin + c.ci) * g.cout + c.co);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const { return g.cout % 4 == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0; }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const {
     c.k += dk;
     c.co += dk;
@@ -187,6 +222,14 @@ struct ConvWgradA {  // m=(r,q,ci) (ci fastest -> contiguous), k=(b,oh,ow)
     if (iy < 0 || iy >= g.h || ix < 0 || ix >= g.w) return 0.f;
     return x[(((int64_t)c.b * g.h + iy) * g.w + ix) * g.cin + c.ci];
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {  // rows (r,q,ci..ci+3) at one k
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    const int iy = c.oh * g.sh - g.pt + c.r, ix = c.ow * g.sw - g.pl + c.q;
+    if (c.ci >= 0 && c.k < k_end && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w)
+      r = *(const f4v*)(x + (((int64_t)c.b * g.h + iy) * g.w + ix) * g.cin + c.ci);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const { return g.cin % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0; }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const {
     c.k += dk;
     c.ow += dk;
@@ -212,6 +255,17 @@ struct LstmZA {
     if (c.k < F) return x[((int64_t)c.m * T + t) * F + c.k];
     return h_prev ? h_prev[(int64_t)c.m * H + (c.k - F)] : 0.f;
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.m >= 0 && c.k < k_end) {
+      if (c.k < F) r = *(const f4v*)(x + ((int64_t)c.m * T + t) * F + c.k);
+      else if (h_prev) r = *(const f4v*)(h_prev + (int64_t)c.m * H + (c.k - F));
+    }
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const {
+    return F % 4 == 0 && H % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(h_prev) & 15u) == 0;
+  }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
 };
 
@@ -236,6 +290,16 @@ struct LstmZB {
     if (!c.wk || c.k >= k_end) return 0.f;
     return c.k < F ? c.wk[(int64_t)c.k * H] : c.wr[(int64_t)(c.k - F) * H];
   }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {  // units u..u+3 of one gate
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.wk && c.k < k_end) r = c.k < F ? *(const f4v*)(c.wk + (int64_t)c.k * H) : *(const f4v*)(c.wr + (int64_t)(c.k - F) * H);
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const {
+    bool ok = H % 4 == 0;
+    for (int g = 0; g < 4; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w.wk[g]) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w.wr[g]) & 15u) == 0;
+    return ok;
+  }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
 };
 
@@ -252,6 +316,19 @@ struct LstmWT {
     if (c.n < 0 || c.k >= k_end) return 0.f;
     const int gate = c.k / H, u = c.k - gate * H;
     return w[gate][(int64_t)c.n * H + u];
+  }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.n >= 0 && c.k < k_end) {
+      const int gate = c.k / H, u = c.k - gate * H;
+      r = *(const f4v*)(w[gate] + (int64_t)c.n * H + u);
+    }
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const {
+    bool ok = H % 4 == 0;
+    for (int g = 0; g < 4; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w[g]) & 15u) == 0;
+    return ok;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
 };
@@ -277,6 +354,18 @@ struct LstmWgradA {
     if (c.m < F) return x[((int64_t)c.b * T + c.t) * F + c.m];
     if (c.m < F + H) return h_prev_all[((int64_t)c.t * rows + c.b) * H + (c.m - F)];
     return 1.0f;
+  }
+  __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {  // rows m..m+3 at one k
+    f4v r = {0.f, 0.f, 0.f, 0.f};
+    if (c.m >= 0 && c.k < k_end) {
+      if (c.m < F) r = *(const f4v*)(x + ((int64_t)c.b * T + c.t) * F + c.m);
+      else if (c.m < F + H) r = *(const f4v*)(h_prev_all + ((int64_t)c.t * rows + c.b) * H + (c.m - F));
+      else r[0] = 1.0f;  // the bias row; rows F+H+1.. lie outside the matrix
+    }
+    v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+  }
+  bool vec4_ok(int) const {
+    return F % 4 == 0 && H % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(h_prev_all) & 15u) == 0;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const {
     c.k += dk;
@@ -346,10 +435,12 @@ struct LdsElem { typedef float type; };
 template <>
 struct LdsElem<true> { typedef __bf16 type; };
 
-template <int BM, int BN, bool BF16, class AL, class BL, class EP>
+// VEC = 4: every tile copy moves 4 values per load along the operand's contiguous index (the host checks
+// vec4_ok() of both loaders); VEC = 1 is the general element-wise form.
+template <int BM, int BN, bool BF16, int VEC, class AL, class BL, class EP>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int k_per_split, AL al, BL bl, EP ep, float* ws) {
   typedef typename LdsElem<BF16>::type lds_t;
-  constexpr int EA = BM * BK / THREADS, EB = BN * BK / THREADS;
+  constexpr int EA = BM * BK / (THREADS * VEC), EB = BN * BK / (THREADS * VEC);
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   __shared__ lds_t As[BM * (BK + 1)];
   __shared__ lds_t Bs[BN * (BK + 1)];
@@ -361,20 +452,20 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 
   typename AL::Cursor ca[EA];
   typename BL::Cursor cb[EB];
-  int ia[EA], ib[EB];  // LDS slots
+  int ia[EA], ib[EB];  // LDS slot of the first value of each vector; the others follow one slot apart
 #pragma unroll
   for (int e = 0; e < EA; ++e) {
     int mm, kk;
-    if (AL::K_CONTIG) { kk = tid % BK; mm = tid / BK + e * (THREADS / BK); }
-    else { mm = tid % BM; kk = tid / BM + e * (THREADS / BM); }
+    if (AL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; mm = tid / KV + e * (THREADS / KV); }
+    else { constexpr int OV = BM / VEC; mm = (tid % OV) * VEC; kk = tid / OV + e * (THREADS / OV); }
     al.init(ca[e], m0 + mm, k_begin + kk);
     ia[e] = lds_index<AL::K_CONTIG, BM>(mm, kk);
   }
 #pragma unroll
   for (int e = 0; e < EB; ++e) {
     int nn, kk;
-    if (BL::K_CONTIG) { kk = tid % BK; nn = tid / BK + e * (THREADS / BK); }
-    else { nn = tid % BN; kk = tid / BN + e * (THREADS / BN); }
+    if (BL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; nn = tid / KV + e * (THREADS / KV); }
+    else { constexpr int OV = BN / VEC; nn = (tid % OV) * VEC; kk = tid / OV + e * (THREADS / OV); }
     bl.init(cb[e], n0 + nn, k_begin + kk);
     ib[e] = lds_index<BL::K_CONTIG, BN>(nn, kk);
   }
@@ -387,26 +478,41 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  float ra[EA], rb[EB];
+  // both staging layouts put consecutive values of the contiguous index one LDS slot apart
+  float ra[EA][VEC], rb[EB][VEC];
+  auto fetch = [&]() {
 #pragma unroll
-  for (int e = 0; e < EA; ++e) ra[e] = al.load(ca[e], k_end);
+    for (int e = 0; e < EA; ++e) {
+      if constexpr (VEC == 4) al.load4(ca[e], k_end, ra[e]);
+      else ra[e][0] = al.load(ca[e], k_end);
+    }
 #pragma unroll
-  for (int e = 0; e < EB; ++e) rb[e] = bl.load(cb[e], k_end);
+    for (int e = 0; e < EB; ++e) {
+      if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[e]);
+      else rb[e][0] = bl.load(cb[e], k_end);
+    }
+  };
+  fetch();
 
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
 #pragma unroll
-    for (int e = 0; e < EA; ++e) As[ia[e]] = (lds_t)ra[e];
+    for (int e = 0; e < EA; ++e)
 #pragma unroll
-    for (int e = 0; e < EB; ++e) Bs[ib[e]] = (lds_t)rb[e];
+      for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[e][i];
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
     __syncthreads();
     if (k0 + BK < k_end) {  // next tile's global loads fly while this tile is multiplied
 #pragma unroll
-      for (int e = 0; e < EA; ++e) { al.advance(ca[e], BK); ra[e] = al.load(ca[e], k_end); }
+      for (int e = 0; e < EA; ++e) al.advance(ca[e], BK);
 #pragma unroll
-      for (int e = 0; e < EB; ++e) { bl.advance(cb[e], BK); rb[e] = bl.load(cb[e], k_end); }
+      for (int e = 0; e < EB; ++e) bl.advance(cb[e], BK);
+      fetch();
     }
     if constexpr (!BF16) {
 #pragma unroll
@@ -484,7 +590,7 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
                         int64_t ws_elems) {
   const int64_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
   int splits = 1;
-  if (tiles < ctx->compute_units && K > 256 && ws) {
+  if (tiles * 2 <= ctx->compute_units && K >= 512 && ws) {  // a split costs a second pass over M*N*splits floats
     int64_t s = std::min<int64_t>(ceil_div((int64_t)2 * ctx->compute_units, tiles), std::max<int64_t>(1, K / 128));
     s = std::min<int64_t>(s, 64);
     s = std::min<int64_t>(s, ws_elems / ((int64_t)M * N));
@@ -495,8 +601,12 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   const dim3 grid((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), (unsigned)splits);
   {
     LaunchScope scope(ctx, name, M, N, K);
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
-                       splits > 1 ? ws : nullptr);
+    if (al.vec4_ok(K) && bl.vec4_ok(K))
+      hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 4, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
+                         splits > 1 ? ws : nullptr);
+    else
+      hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 1, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
+                         splits > 1 ? ws : nullptr);
   }
   if (splits > 1) {
     const int64_t total = (int64_t)M * N;
@@ -513,7 +623,9 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
                       int64_t ws_elems) {
   if (M <= 0 || N <= 0) return SN_OK;
   SN_REQUIRE(K > 0, "%s: empty reduction dimension", name);
-  const bool big_m = M > 64, big_n = N > 64;
+  bool big_m = M > 64, big_n = N > 64;
+  // 128-wide tiles only when they still cover every CU at least once; otherwise more, smaller workgroups
+  if (ceil_div(M, big_m ? 128 : 64) * ceil_div(N, big_n ? 128 : 64) < ctx->compute_units) big_m = big_n = false;
   if (big_m && big_n) return launch_tiles<128, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_m) return launch_tiles<128, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_n) return launch_tiles<64, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
