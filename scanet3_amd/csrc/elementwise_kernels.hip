@@ -399,59 +399,91 @@ int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, 
 // ---------------------------------------------------------------------------- max pooling (NHWC)
 // Forward keeps, per output element, the window offset (r*kw + q) of the first maximum in
 // row-major window order; padding cells never win (TF MaxPoolV2, math/nn/AllKernels.scala:270-303).
+// V channels per thread (V = 4 needs c % 4 == 0 and 16-byte aligned tensors); I is the index type.
+template <int V, typename I>
 __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
                                                            int n, int h, int w, int c, int ho, int wo, int kh, int kw, int sh,
                                                            int sw, int pt, int pl) {
-  const int64_t total = (int64_t)n * ho * wo * c;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int ch = (int)(i % c);
-    int64_t t = i / c;
+  const I cv = (I)(c / V);
+  const I total = (I)n * ho * wo * cv;
+  const I stride = (I)gridDim.x * blockDim.x;
+  for (I i = (I)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const I ch = (i % cv) * V;
+    I t = i / cv;
     const int ow = (int)(t % wo); t /= wo;
     const int oh = (int)(t % ho);
-    const int b = (int)(t / ho);
-    float best = -INFINITY;
-    int at = 0;
+    const I b = t / ho;
+    float best[V];
+    int at[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) { best[v] = -INFINITY; at[v] = 0; }
     for (int r = 0; r < kh; ++r) {
       const int iy = oh * sh - pt + r;
       if (iy < 0 || iy >= h) continue;
       for (int q = 0; q < kw; ++q) {
         const int ix = ow * sw - pl + q;
         if (ix < 0 || ix >= w) continue;
-        const float v = x[(((int64_t)b * h + iy) * w + ix) * c + ch];
-        if (v > best) { best = v; at = r * kw + q; }
+        const float* src = x + ((b * h + iy) * w + ix) * c + ch;
+        float val[V];
+        if constexpr (V == 4) { const float4 f = *(const float4*)src; val[0] = f.x; val[1] = f.y; val[2] = f.z; val[3] = f.w; }
+        else val[0] = *src;
+#pragma unroll
+        for (int v = 0; v < V; ++v)
+          if (val[v] > best[v]) { best[v] = val[v]; at[v] = r * kw + q; }
       }
     }
-    y[i] = best;
-    arg[i] = (uint8_t)at;
+    const I o = i * V;
+    if constexpr (V == 4) {
+      *(float4*)(y + o) = make_float4(best[0], best[1], best[2], best[3]);
+      *(uint32_t*)(arg + o) = (uint32_t)at[0] | ((uint32_t)at[1] << 8) | ((uint32_t)at[2] << 16) | ((uint32_t)at[3] << 24);
+    } else {
+      y[o] = best[0];
+      arg[o] = (uint8_t)at[0];
+    }
   }
+}
+
+static bool pool_vec4(const void* a, const void* b, const void* m, int c) {
+  return c % 4 == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0 && (reinterpret_cast<uintptr_t>(m) & 3u) == 0;
 }
 
 int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo, int kh,
                        int kw, int sh, int sw, int pt, int pl) {
   const int64_t total = (int64_t)n * ho * wo * c;
   if (total <= 0) return SN_OK;
+  const bool small = total < (1ll << 31) && (int64_t)n * h * w * c < (1ll << 31);
+  const bool v4 = pool_vec4(x, y, arg, c);
+  const dim3 grid(grid_for(ctx, v4 ? total / 4 : total, 256));
   LaunchScope scope(ctx, "maxpool_forward");
-  hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(ctx, total, 512)), dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo,
-                     kh, kw, sh, sw, pt, pl);
+#define SN_POOL_FWD(V, I) \
+  hipLaunchKernelGGL((maxpool_fwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl)
+  if (v4 && small) SN_POOL_FWD(4, uint32_t);
+  else if (v4) SN_POOL_FWD(4, uint64_t);
+  else if (small) SN_POOL_FWD(1, uint32_t);
+  else SN_POOL_FWD(1, uint64_t);
+#undef SN_POOL_FWD
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
 
 // Backward as a gather: each input element adds the gradients of the windows whose recorded
 // first maximum is this element (TF MaxPoolGradV2, math/nn/AllKernels.scala:305-324). No atomics.
+template <int V, typename I>
 __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
                                                            float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo,
                                                            int kh, int kw, int sh, int sw, int pt, int pl) {
-  const int64_t total = (int64_t)n * h * w * c;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int ch = (int)(i % c);
-    int64_t t = i / c;
+  const I cv = (I)(c / V);
+  const I total = (I)n * h * w * cv;
+  const I stride = (I)gridDim.x * blockDim.x;
+  for (I i = (I)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const I ch = (i % cv) * V;
+    I t = i / cv;
     const int ix = (int)(t % w); t /= w;
     const int iy = (int)(t % h);
-    const int b = (int)(t / h);
-    float s = 0.f;
+    const I b = t / h;
+    float s[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) s[v] = 0.f;
     // windows (oh, ow) with oh*sh - pt <= iy < oh*sh - pt + kh
     int oh_lo = iy + pt - kh + 1;
     oh_lo = oh_lo <= 0 ? 0 : (oh_lo + sh - 1) / sh;
@@ -465,11 +497,22 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restric
       const int r = iy - (oh * sh - pt);
       for (int ow = ow_lo; ow <= ow_hi; ++ow) {
         const int q = ix - (ow * sw - pl);
-        const int64_t o = (((int64_t)b * ho + oh) * wo + ow) * c + ch;
-        if (arg[o] == (uint8_t)(r * kw + q)) s += dy[o];
+        const I o = ((b * ho + oh) * wo + ow) * c + ch;
+        const uint32_t want = (uint32_t)(r * kw + q);
+        if constexpr (V == 4) {
+          const uint32_t a4 = *(const uint32_t*)(arg + o);
+          const float4 g = *(const float4*)(dy + o);
+          if ((a4 & 255u) == want) s[0] += g.x;
+          if (((a4 >> 8) & 255u) == want) s[1] += g.y;
+          if (((a4 >> 16) & 255u) == want) s[2] += g.z;
+          if ((a4 >> 24) == want) s[3] += g.w;
+        } else {
+          if (arg[o] == want) s[0] += dy[o];
+        }
       }
     }
-    dx[i] = s;
+    if constexpr (V == 4) *(float4*)(dx + i * 4) = make_float4(s[0], s[1], s[2], s[3]);
+    else dx[i] = s[0];
   }
 }
 
@@ -477,9 +520,17 @@ int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* 
                        int kh, int kw, int sh, int sw, int pt, int pl) {
   const int64_t total = (int64_t)n * h * w * c;
   if (total <= 0) return SN_OK;
+  const bool small = total < (1ll << 31) && (int64_t)n * ho * wo * c < (1ll << 31);
+  const bool v4 = pool_vec4(dy, dx, arg, c);
+  const dim3 grid(grid_for(ctx, v4 ? total / 4 : total, 256));
   LaunchScope scope(ctx, "maxpool_backward");
-  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(ctx, total, 512)), dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho,
-                     wo, kh, kw, sh, sw, pt, pl);
+#define SN_POOL_BWD(V, I) \
+  hipLaunchKernelGGL((maxpool_bwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl)
+  if (v4 && small) SN_POOL_BWD(4, uint32_t);
+  else if (v4) SN_POOL_BWD(4, uint64_t);
+  else if (small) SN_POOL_BWD(1, uint32_t);
+  else SN_POOL_BWD(1, uint64_t);
+#undef SN_POOL_BWD
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

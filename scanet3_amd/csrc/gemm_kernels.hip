@@ -440,12 +440,18 @@ struct LdsElem<true> { typedef __bf16 type; };
 template <int BM, int BN, bool BF16, int VEC, class AL, class BL, class EP>
 __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int k_per_split, AL al, BL bl, EP ep, float* ws) {
   typedef typename LdsElem<BF16>::type lds_t;
-  constexpr int EA = BM * BK / (THREADS * VEC), EB = BN * BK / (THREADS * VEC);
-  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  // the 4 waves form a 2x2 grid over the tile, or 4x1 when the tile is a single MFMA block wide
+  constexpr int WAVES_N = BN >= 64 ? 2 : 1, WAVES_M = 4 / WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+  // a B tile of fewer than THREADS vectors is copied by the first B_ACTIVE threads only
+  constexpr int B_ACTIVE = BN * BK / VEC < THREADS ? BN * BK / VEC : THREADS;
+  constexpr int EA = BM * BK / (THREADS * VEC), EB = BN * BK / (B_ACTIVE * VEC);
+  static_assert(TM >= 1 && TN >= 1 && EA >= 1, "tile too small for four waves");
   __shared__ lds_t As[BM * (BK + 1)];
   __shared__ lds_t Bs[BN * (BK + 1)];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bool b_on = tid < B_ACTIVE;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int k_begin = blockIdx.z * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
@@ -464,8 +470,9 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 #pragma unroll
   for (int e = 0; e < EB; ++e) {
     int nn, kk;
-    if (BL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; nn = tid / KV + e * (THREADS / KV); }
-    else { constexpr int OV = BN / VEC; nn = (tid % OV) * VEC; kk = tid / OV + e * (THREADS / OV); }
+    if (BL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; nn = tid / KV + e * (B_ACTIVE / KV); }
+    else { constexpr int OV = BN / VEC; nn = (tid % OV) * VEC; kk = tid / OV + e * (B_ACTIVE / OV); }
+    if (!b_on) { nn = 0; kk = 0; }
     bl.init(cb[e], n0 + nn, k_begin + kk);
     ib[e] = lds_index<BL::K_CONTIG, BN>(nn, kk);
   }
@@ -486,15 +493,17 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
       if constexpr (VEC == 4) al.load4(ca[e], k_end, ra[e]);
       else ra[e][0] = al.load(ca[e], k_end);
     }
+    if (b_on) {
 #pragma unroll
-    for (int e = 0; e < EB; ++e) {
-      if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[e]);
-      else rb[e][0] = bl.load(cb[e], k_end);
+      for (int e = 0; e < EB; ++e) {
+        if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[e]);
+        else rb[e][0] = bl.load(cb[e], k_end);
+      }
     }
   };
   fetch();
 
-  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
@@ -502,10 +511,12 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
     for (int e = 0; e < EA; ++e)
 #pragma unroll
       for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[e][i];
+    if (b_on) {
 #pragma unroll
-    for (int e = 0; e < EB; ++e)
+      for (int e = 0; e < EB; ++e)
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
+        for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
+    }
     __syncthreads();
     if (k0 + BK < k_end) {  // next tile's global loads fly while this tile is multiplied
 #pragma unroll
@@ -575,9 +586,85 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
+// ============================================================================ small output, long reduction
+// C[M,N] with M*N <= 1024 and K in the thousands (first-layer filter gradients, Dense layers onto a few
+// classes): too little output for MFMA tiles to occupy the chip. Workgroups stride over 64-long slices of K,
+// stage them in LDS, keep up to four outputs per thread in registers and leave one partial sum per workgroup
+// and output; a second kernel adds the partials in a fixed order.
+constexpr int SMALL_SLICE = 64, SMALL_MAX_OUT = 1024, SMALL_MAX_DIM = 128, SMALL_MIN_K = 2048;
+
+template <class AL, class BL>
+__global__ __launch_bounds__(256) void gemm_small_kernel(int M, int N, int K, AL al, BL bl, float* __restrict__ partial) {
+  extern __shared__ float small_lds[];
+  float* As = small_lds;                    // [SMALL_SLICE][M]
+  float* Bs = small_lds + SMALL_SLICE * M;  // [SMALL_SLICE][N]
+  const int tid = threadIdx.x, outs = M * N;
+  int om[4], on[4];
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int o = tid + j * 256;
+    om[j] = o < outs ? o / N : 0;
+    on[j] = o < outs ? o % N : 0;
+  }
+  const int slices = (K + SMALL_SLICE - 1) / SMALL_SLICE;
+  for (int sl = blockIdx.x; sl < slices; sl += gridDim.x) {
+    const int k0 = sl * SMALL_SLICE;
+    for (int e = tid; e < SMALL_SLICE * M; e += 256) {
+      int m, p;
+      if (AL::K_CONTIG) { p = e % SMALL_SLICE; m = e / SMALL_SLICE; }
+      else { m = e % M; p = e / M; }
+      typename AL::Cursor c;
+      al.init(c, m, k0 + p);
+      As[p * M + m] = al.load(c, K);
+    }
+    for (int e = tid; e < SMALL_SLICE * N; e += 256) {
+      int n, p;
+      if (BL::K_CONTIG) { p = e % SMALL_SLICE; n = e / SMALL_SLICE; }
+      else { n = e % N; p = e / N; }
+      typename BL::Cursor c;
+      bl.init(c, n, k0 + p);
+      Bs[p * N + n] = bl.load(c, K);
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int p = 0; p < SMALL_SLICE; ++p) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] += As[p * M + om[j]] * Bs[p * N + on[j]];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int o = tid + j * 256;
+    if (o < outs) partial[(int64_t)o * gridDim.x + blockIdx.x] = acc[j];
+  }
+}
+
+template <class EP>
+__global__ __launch_bounds__(256) void gemm_small_reduce_kernel(const float* __restrict__ partial, int parts, int M, int N, EP ep) {
+  const int lane = threadIdx.x & 63;
+  const int o = blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per output
+  if (o >= M * N) return;
+  float s = 0.f;
+  for (int i = lane; i < parts; i += 64) s += partial[(int64_t)o * parts + i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
+  if (lane == 0) ep.store(o / N, o % N, s);
+}
+
+static int small_parts(int m, int n, int k, int cu, int64_t ws_elems) {
+  if ((int64_t)m * n > SMALL_MAX_OUT || m > SMALL_MAX_DIM || n > SMALL_MAX_DIM || k < SMALL_MIN_K) return 0;
+  int64_t parts = std::min<int64_t>(ceil_div(k, SMALL_SLICE), (int64_t)4 * cu);
+  if (ws_elems >= 0) parts = std::min<int64_t>(parts, ws_elems / ((int64_t)m * n));
+  return parts >= 32 ? (int)parts : 0;
+}
+
 // ============================================================================ dispatch
 int64_t gemm_workspace_elems(int m, int n, int k, int cu) {
-  // room for the largest split count the heuristic below may pick
+  // room for the partial sums of the small-output kernel, or for the largest split count launch_tiles may pick
+  const int parts = small_parts(m, n, k, cu, -1);
+  if (parts) return (int64_t)parts * m * n;
   const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
   if (tiles >= cu || k <= 256) return 0;
   int64_t splits = std::min<int64_t>(ceil_div((int64_t)2 * cu, tiles), std::max<int64_t>(1, k / 128));
@@ -623,9 +710,22 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
                       int64_t ws_elems) {
   if (M <= 0 || N <= 0) return SN_OK;
   SN_REQUIRE(K > 0, "%s: empty reduction dimension", name);
+  if (const int parts = ws ? small_parts(M, N, K, ctx->compute_units, ws_elems) : 0) {
+    {
+      LaunchScope scope(ctx, name, M, N, K);
+      hipLaunchKernelGGL((gemm_small_kernel<AL, BL>), dim3((unsigned)parts), dim3(256), (size_t)SMALL_SLICE * (M + N) * sizeof(float),
+                         ctx->stream, M, N, K, al, bl, ws);
+    }
+    LaunchScope scope(ctx, "small_output_reduce");
+    hipLaunchKernelGGL((gemm_small_reduce_kernel<EP>), dim3((unsigned)ceil_div(M * N, 4)), dim3(256), 0, ctx->stream, (const float*)ws,
+                       parts, M, N, ep);
+    SN_HIP(hipGetLastError());
+    return SN_OK;
+  }
   bool big_m = M > 64, big_n = N > 64;
   // 128-wide tiles only when they still cover every CU at least once; otherwise more, smaller workgroups
   if (ceil_div(M, big_m ? 128 : 64) * ceil_div(N, big_n ? 128 : 64) < ctx->compute_units) big_m = big_n = false;
+  if (N <= 32 && M > 64) return launch_tiles<128, 32, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_m && big_n) return launch_tiles<128, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_m) return launch_tiles<128, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_n) return launch_tiles<64, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
