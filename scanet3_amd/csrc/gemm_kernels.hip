@@ -610,27 +610,51 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int M, int N, int K, AL
   const int slices = (K + SMALL_SLICE - 1) / SMALL_SLICE;
   for (int sl = blockIdx.x; sl < slices; sl += gridDim.x) {
     const int k0 = sl * SMALL_SLICE;
-    for (int e = tid; e < SMALL_SLICE * M; e += 256) {
-      int m, p;
-      if (AL::K_CONTIG) { p = e % SMALL_SLICE; m = e / SMALL_SLICE; }
-      else { m = e % M; p = e / M; }
-      typename AL::Cursor c;
-      al.init(c, m, k0 + p);
-      As[p * M + m] = al.load(c, K);
+    // batches of 8 loads per thread are issued before any of them is stored, so their latencies overlap
+    for (int base = 0; base < SMALL_SLICE * M; base += 256 * 8) {
+      float v[8];
+      int at[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = base + u * 256 + tid;
+        int m, p;
+        if (AL::K_CONTIG) { p = e % SMALL_SLICE; m = e / SMALL_SLICE; }
+        else { m = e % M; p = e / M; }
+        at[u] = e < SMALL_SLICE * M ? p * M + m : -1;
+        typename AL::Cursor c;
+        al.init(c, at[u] >= 0 ? m : M, k0 + p);
+        v[u] = al.load(c, K);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (at[u] >= 0) As[at[u]] = v[u];
     }
-    for (int e = tid; e < SMALL_SLICE * N; e += 256) {
-      int n, p;
-      if (BL::K_CONTIG) { p = e % SMALL_SLICE; n = e / SMALL_SLICE; }
-      else { n = e % N; p = e / N; }
-      typename BL::Cursor c;
-      bl.init(c, n, k0 + p);
-      Bs[p * N + n] = bl.load(c, K);
+    for (int base = 0; base < SMALL_SLICE * N; base += 256 * 8) {
+      float v[8];
+      int at[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = base + u * 256 + tid;
+        int n, p;
+        if (BL::K_CONTIG) { p = e % SMALL_SLICE; n = e / SMALL_SLICE; }
+        else { n = e % N; p = e / N; }
+        at[u] = e < SMALL_SLICE * N ? p * N + n : -1;
+        typename BL::Cursor c;
+        bl.init(c, at[u] >= 0 ? n : N, k0 + p);
+        v[u] = bl.load(c, K);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (at[u] >= 0) Bs[at[u]] = v[u];
     }
     __syncthreads();
-#pragma unroll 8
-    for (int p = 0; p < SMALL_SLICE; ++p) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] += As[p * M + om[j]] * Bs[p * N + on[j]];
+    for (int j = 0; j < 4; ++j) {
+      if ((tid & ~63) + j * 256 >= outs) break;  // the same for every lane of a wave
+      float a = acc[j];
+#pragma unroll 8
+      for (int p = 0; p < SMALL_SLICE; ++p) a += As[p * M + om[j]] * Bs[p * N + on[j]];
+      acc[j] = a;
     }
     __syncthreads();
   }
