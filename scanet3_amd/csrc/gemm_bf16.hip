@@ -179,24 +179,18 @@ __device__ __forceinline__ void gemm_bf16_tn_body(const bf16* __restrict__ A, in
   const int qa = (M - m0 - r0 + 7) >> 3, qb = (N - n0 - r0 + 7) >> 3;  // issues q >= qa / qb fall past the matrix
   const uint32_t a0 = (uint32_t)(((int64_t)(m0 + r0) * lda) * 2), b0 = (uint32_t)(((int64_t)(n0 + r0) * ldb) * 2);
   const uint32_t astep = (uint32_t)(lda * 16), bstep = (uint32_t)(ldb * 16);  // 8 rows in bytes
-  auto issue_stage = [&](int k0, int buf) {
-    // K is a multiple of 8, so a 16-byte chunk lies inside or outside its row as a whole
-    const uint32_t k_even = (k0 + lchunk[0] * 8 < K) ? (uint32_t)(k0 + lchunk[0] * 8) * 2 : OOB;
-    const uint32_t k_odd = (k0 + lchunk[1] * 8 < K) ? (uint32_t)(k0 + lchunk[1] * 8) * 2 : OOB;
-    char* da = sA + buf * STAGE + wave * (BT / 4) * 128;
-    char* db = sB + buf * STAGE + wave * (BT / 4) * 128;
-#pragma unroll
-    for (int q = 0; q < ISSUES; ++q) {
-      const uint32_t ko = (q & 1) ? k_odd : k_even;
-      const uint32_t off = q < qa ? (a0 + q * astep + ko) | (ko & OOB) : OOB;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr)(da + q * 1024), 16, (int)off, 0, 0, 0);
-    }
-#pragma unroll
-    for (int q = 0; q < ISSUES; ++q) {
-      const uint32_t ko = (q & 1) ? k_odd : k_even;
-      const uint32_t off = q < qb ? (b0 + q * bstep + ko) | (ko & OOB) : OOB;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr)(db + q * 1024), 16, (int)off, 0, 0, 0);
-    }
+  // One 1 KiB LDS-bound load: issue q of this wavefront for stage k0 of operand A / B.  A k0 at or past K
+  // gives out-of-range offsets, which the buffer load answers with zeros and no memory traffic.
+  // K is a multiple of 8, so a 16-byte chunk lies inside or outside its row as a whole.
+  auto issue_a = [&](int q, int k0, int buf) {
+    const int kc = k0 + lchunk[q & 1] * 8;
+    const uint32_t off = (q < qa && kc < K) ? a0 + q * astep + (uint32_t)kc * 2 : OOB;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr)(sA + buf * STAGE + wave * (BT / 4) * 128 + q * 1024), 16, (int)off, 0, 0, 0);
+  };
+  auto issue_b = [&](int q, int k0, int buf) {
+    const int kc = k0 + lchunk[q & 1] * 8;
+    const uint32_t off = (q < qb && kc < K) ? b0 + q * bstep + (uint32_t)kc * 2 : OOB;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr)(sB + buf * STAGE + wave * (BT / 4) * 128 + q * 1024), 16, (int)off, 0, 0, 0);
   };
 
   f16v acc[TI][TI];
@@ -208,20 +202,34 @@ __device__ __forceinline__ void gemm_bf16_tn_body(const bf16* __restrict__ A, in
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   bf16x8 f0a[TI], f0b[TI], f1a[TI], f1b[TI];
-  // fragments of k sub-step s (16 k-values) of the stage in buffer `buf`
-#define SN_READ_FRAGS(FA, FB, buf, s)                                                                            \
-  {                                                                                                              \
-    _Pragma("unroll") for (int i = 0; i < TI; ++i) FA[i] =                                                        \
-        *(const bf16x8*)(sA + (buf) * STAGE + swz(wm + i * 32 + l32, (s) * 2 + lhi));                             \
-    _Pragma("unroll") for (int j = 0; j < TI; ++j) FB[j] =                                                        \
-        *(const bf16x8*)(sB + (buf) * STAGE + swz(wn + j * 32 + l32, (s) * 2 + lhi));                             \
-  }
-#define SN_MMA(FA, FB)                                                                                           \
-  {                                                                                                              \
-    _Pragma("unroll") for (int i = 0; i < TI; ++i) _Pragma("unroll") for (int j = 0; j < TI; ++j) acc[i][j] =     \
-        __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0);                                \
+  // Fragment r of k sub-step s (16 k-values) of the stage in buffer `buf`, in the order the MFMAs of the next
+  // sub-step want them: A0, B0 .. B(TI-1), A1 .. A(TI-1).
+#define SN_READ_ONE(FA, FB, buf, s, r)                                                                              \
+  {                                                                                                                 \
+    if ((r) == 0) FA[0] = *(const bf16x8*)(sA + (buf) * STAGE + swz(wm + l32, (s) * 2 + lhi));                       \
+    else if ((r) <= TI) FB[(r) - 1] = *(const bf16x8*)(sB + (buf) * STAGE + swz(wn + ((r) - 1) * 32 + l32, (s) * 2 + lhi)); \
+    else FA[(r) - TI] = *(const bf16x8*)(sA + (buf) * STAGE + swz(wm + ((r) - TI) * 32 + l32, (s) * 2 + lhi));       \
   }
 #define SN_FENCE() __builtin_amdgcn_sched_barrier(0)
+  // One k sub-step: TI*TI MFMAs in pairs; behind each pair go two fragment reads for the next sub-step
+  // (DO_READ) and this pair's share of the stage loads of operand LOAD (0 none, 1 A, 2 B), so that LDS reads
+  // and global loads are issued in the shadow of the matrix cores instead of between their bursts.
+  constexpr int NG = TI * TI / 2, PPR = TI / 2, LPG = ISSUES / NG;
+#define SN_SUBSTEP(CA, CB, NA, NB, DO_READ, rbuf, rs, LOAD, lk0, lbuf)                                               \
+  {                                                                                                                 \
+    _Pragma("unroll") for (int g = 0; g < NG; ++g) {                                                                 \
+      const int i_ = g / PPR, j_ = (g % PPR) * 2;                                                                   \
+      acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(CA[i_], CB[j_], acc[i_][j_], 0, 0, 0);                   \
+      acc[i_][j_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(CA[i_], CB[j_ + 1], acc[i_][j_ + 1], 0, 0, 0);       \
+      if (DO_READ) {                                                                                                \
+        _Pragma("unroll") for (int r_ = 2 * g; r_ < 2 * g + 2; ++r_)                                                 \
+          if (r_ < 2 * TI) SN_READ_ONE(NA, NB, rbuf, rs, r_);                                                       \
+      }                                                                                                             \
+      if ((LOAD) == 1) { _Pragma("unroll") for (int q_ = g * LPG; q_ < (g + 1) * LPG; ++q_) issue_a(q_, lk0, lbuf); } \
+      if ((LOAD) == 2) { _Pragma("unroll") for (int q_ = g * LPG; q_ < (g + 1) * LPG; ++q_) issue_b(q_, lk0, lbuf); } \
+      SN_FENCE();                                                                                                   \
+    }                                                                                                               \
+  }
   // all of this wavefront's LDS-bound loads have landed, then everybody's
 #define SN_PUBLISH()                      \
   {                                       \
@@ -229,48 +237,37 @@ __device__ __forceinline__ void gemm_bf16_tn_body(const bf16* __restrict__ A, in
     __syncthreads();                      \
   }
 
-  // Pipeline over k stages of 64 (4 sub-steps of 16).  While the matrix cores work on sub-step s the LDS
-  // reads of sub-step s+1 are in flight.  One barrier per stage, before sub-step 3: it publishes stage kt+1
-  // (whose loads were issued a whole stage earlier) and frees the current buffer, into which the loads of
-  // stage kt+2 are issued at once; sub-step 3's MFMAs then cover the first fragment reads of stage kt+1.
+  // Pipeline over k stages of 64 (4 sub-steps of 16) and two LDS buffers.  One barrier per stage, before
+  // sub-step 3: it publishes stage kt+1 and frees the current buffer.  The A half of stage kt+2 is loaded
+  // into the freed buffer during sub-step 3, the B half during sub-step 0 of the next stage, one load
+  // behind every MFMA pair; sub-step 3 also covers the first fragment reads of stage kt+1.
   const int nk = (K + GBK - 1) / GBK;
-  issue_stage(0, 0);
+#pragma unroll
+  for (int q = 0; q < ISSUES; ++q) { issue_a(q, 0, 0); issue_b(q, 0, 0); }
   SN_PUBLISH();
-  if (nk > 1) issue_stage(GBK, 1);
-  SN_READ_FRAGS(f0a, f0b, 0, 0);
+#pragma unroll
+  for (int q = 0; q < ISSUES; ++q) issue_a(q, GBK, 1);
+#pragma unroll
+  for (int r = 0; r < 2 * TI; ++r) SN_READ_ONE(f0a, f0b, 0, 0, r);
+  SN_FENCE();
   for (int kt = 0; kt + 1 < nk; ++kt) {
     const int buf = kt & 1;
-    SN_FENCE();
-    SN_READ_FRAGS(f1a, f1b, buf, 1);
-    SN_MMA(f0a, f0b);
-    SN_FENCE();
-    SN_READ_FRAGS(f0a, f0b, buf, 2);
-    SN_MMA(f1a, f1b);
-    SN_FENCE();
-    SN_READ_FRAGS(f1a, f1b, buf, 3);
-    SN_MMA(f0a, f0b);
-    SN_FENCE();
+    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 1, 2, (kt + 1) * GBK, buf ^ 1);
+    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf, 2, 0, 0, 0);
+    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 3, 0, 0, 0);
     SN_PUBLISH();
-    if (kt + 2 < nk) issue_stage((kt + 2) * GBK, buf);
-    SN_READ_FRAGS(f0a, f0b, buf ^ 1, 0);
-    SN_MMA(f1a, f1b);
+    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf ^ 1, 0, 1, (kt + 2) * GBK, buf);
   }
   {
     const int buf = (nk - 1) & 1;
-    SN_FENCE();
-    SN_READ_FRAGS(f1a, f1b, buf, 1);
-    SN_MMA(f0a, f0b);
-    SN_FENCE();
-    SN_READ_FRAGS(f0a, f0b, buf, 2);
-    SN_MMA(f1a, f1b);
-    SN_FENCE();
-    SN_READ_FRAGS(f1a, f1b, buf, 3);
-    SN_MMA(f0a, f0b);
-    SN_FENCE();
-    SN_MMA(f1a, f1b);
+    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 1, 0, 0, 0);
+    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf, 2, 0, 0, 0);
+    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 3, 0, 0, 0);
+    SN_SUBSTEP(f1a, f1b, f0a, f0b, false, 0, 0, 0, 0, 0);
   }
-#undef SN_READ_FRAGS
-#undef SN_MMA
+  __builtin_amdgcn_s_waitcnt(0);  // the zero-filling loads past the last stage have landed before LDS is reused
+#undef SN_READ_ONE
+#undef SN_SUBSTEP
 #undef SN_FENCE
 #undef SN_PUBLISH
 

@@ -20,6 +20,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int BK = 16;
 constexpr int THREADS = 256;
+constexpr int PF = 1;  // k-tiles of global loads in flight per workgroup
 
 // ============================================================================ loaders
 // A loader describes one operand as a function (outer index, k) -> value, where the outer
@@ -146,8 +147,12 @@ struct ConvDgradA {  // m=(b,iy,ix), k=(r,q,co)
     f4v r = {0.f, 0.f, 0.f, 0.f};
     const int ny = c.ty - c.r, nx = c.tx - c.q;
     if (c.img && c.k < k_end && ny >= 0 && nx >= 0) {
-      const int oy = ny / g.sh, ox = nx / g.sw;
-      if (oy * g.sh == ny && ox * g.sw == nx && oy < g.ho && ox < g.wo) r = *(const f4v*)(c.img + ((int64_t)oy * g.wo + ox) * g.cout + c.co);
+      if (g.sh == 1 && g.sw == 1) {  // unit strides (the same for every lane): no divisions
+        if (ny < g.ho && nx < g.wo) r = *(const f4v*)(c.img + (ny * g.wo + nx) * g.cout + c.co);
+      } else {
+        const int oy = ny / g.sh, ox = nx / g.sw;
+        if (oy * g.sh == ny && ox * g.sw == nx && oy < g.ho && ox < g.wo) r = *(const f4v*)(c.img + ((int64_t)oy * g.wo + ox) * g.cout + c.co);
+      }
     }
     v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
   }
@@ -485,77 +490,84 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // both staging layouts put consecutive values of the contiguous index one LDS slot apart
-  float ra[EA][VEC], rb[EB][VEC];
-  auto fetch = [&]() {
+  // Both staging layouts put consecutive values of the contiguous index one LDS slot apart.
+  // Global loads run PF k-tiles ahead of the multiplication through a ring of register stages: with few
+  // workgroups per CU it is the load latency, not the matrix cores, that a short-K product waits on.
+  float ra[PF][EA][VEC], rb[PF][EB][VEC];
+  int k_fetch = k_begin;  // first k of the next tile to load
+  auto fetch = [&](int s) {  // loads the tile the cursors point at, unless it lies past k_end, and moves them on
+    if (k_fetch < k_end) {
 #pragma unroll
-    for (int e = 0; e < EA; ++e) {
-      if constexpr (VEC == 4) al.load4(ca[e], k_end, ra[e]);
-      else ra[e][0] = al.load(ca[e], k_end);
-    }
-    if (b_on) {
+      for (int e = 0; e < EA; ++e) {
+        if constexpr (VEC == 4) al.load4(ca[e], k_end, ra[s][e]);
+        else ra[s][e][0] = al.load(ca[e], k_end);
+        al.advance(ca[e], BK);
+      }
+      if (b_on) {
 #pragma unroll
-      for (int e = 0; e < EB; ++e) {
-        if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[e]);
-        else rb[e][0] = bl.load(cb[e], k_end);
+        for (int e = 0; e < EB; ++e) {
+          if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[s][e]);
+          else rb[s][e][0] = bl.load(cb[e], k_end);
+          bl.advance(cb[e], BK);
+        }
       }
     }
+    k_fetch += BK;
   };
-  fetch();
+#pragma unroll
+  for (int s = 0; s < PF; ++s) fetch(s);
 
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
-  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+  for (int kb = k_begin; kb < k_end; kb += BK * PF) {
 #pragma unroll
-    for (int e = 0; e < EA; ++e)
+    for (int s = 0; s < PF; ++s) {
+      if (kb + s * BK >= k_end) break;
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[e][i];
-    if (b_on) {
+      for (int e = 0; e < EA; ++e)
 #pragma unroll
-      for (int e = 0; e < EB; ++e)
+        for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[s][e][i];
+      if (b_on) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
-    }
-    __syncthreads();
-    if (k0 + BK < k_end) {  // next tile's global loads fly while this tile is multiplied
+        for (int e = 0; e < EB; ++e)
 #pragma unroll
-      for (int e = 0; e < EA; ++e) al.advance(ca[e], BK);
+          for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[s][e][i];
+      }
+      __syncthreads();
+      fetch(s);  // the tile PF steps ahead takes over this stage's registers
+      if constexpr (!BF16) {
 #pragma unroll
-      for (int e = 0; e < EB; ++e) bl.advance(cb[e], BK);
-      fetch();
-    }
-    if constexpr (!BF16) {
+        for (int ks = 0; ks < BK; ks += 2) {
+          const int k = ks + lhi;
+          float av[TM], bv[TN];
 #pragma unroll
-      for (int ks = 0; ks < BK; ks += 2) {
-        const int k = ks + lhi;
-        float av[TM], bv[TN];
+          for (int i = 0; i < TM; ++i) av[i] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, k)];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) av[i] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, k)];
+          for (int j = 0; j < TN; ++j) bv[j] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, k)];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bv[j] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, k)];
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+      } else {
+        // 32x32x16 bf16: lane supplies k = 8*(lane/32) .. +7 of row/col lane%32
+        bf16x8 av[TM], bv[TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+          for (int v = 0; v < 8; ++v) av[i][v] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int v = 0; v < 8; ++v) bv[j][v] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
       }
-    } else {
-      // 32x32x16 bf16: lane supplies k = 8*(lane/32) .. +7 of row/col lane%32
-      bf16x8 av[TM], bv[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int v = 0; v < 8; ++v) av[i][v] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, lhi * 8 + v)];
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int v = 0; v < 8; ++v) bv[j][v] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, lhi * 8 + v)];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+      __syncthreads();
     }
-    __syncthreads();
   }
 
   // accumulator element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
