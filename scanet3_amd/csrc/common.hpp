@@ -137,6 +137,8 @@ struct LstmGateBwdArgs {
   float* dc;            // [rows,H] in: dc_t carried from t+1 (or zeros), out: dc_{t-1}
   float* dz;            // [rows,4H]
   int dc_is_zero;       // first backward step: treat dc as zeros on input
+  int dh_parts = 1;     // dh is the sum of this many arrays, dh_part_stride elements apart (added in order)
+  int64_t dh_part_stride = 0;
 };
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
 
@@ -203,5 +205,14 @@ int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, cons
                       const LstmGrads& g, float* ws, int64_t ws_elems);
 
 int64_t gemm_workspace_elems(int m, int n, int k, int cu);
+
+// ---- fused LSTM steps (lstm_kernels.hip) ------------------------------------------------
+// true when the fused step kernels handle this layer (F % 4 == 0, H % 16 == 0, F + H <= 400, 16-byte aligned tensors)
+bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w);
+// gates, c_t, h_t of step t from x[:, t, :], h_prev, c_prev (both null at t == 0) in one kernel
+int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
+                         const LstmWeights& w, float* gates, float* c, float* h);
+// dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev
+int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_parts, int64_t part_stride);
 
 }  // namespace sn

@@ -581,7 +581,8 @@ __global__ __launch_bounds__(256) void lstm_gates_bwd_kernel(LstmGateBwdArgs a, 
     const int64_t zb = r * 4 * hidden + u;
     const float f = a.gates[zb], in = a.gates[zb + hidden], g = a.gates[zb + 2 * hidden], o = a.gates[zb + 3 * hidden];
     const float tc = tanhf(a.c[i]);
-    const float dh = a.dh[i];
+    float dh = a.dh[i];
+    for (int p = 1; p < a.dh_parts; ++p) dh += a.dh[i + p * a.dh_part_stride];
     const float d_o = dh * tc;
     float dc = a.dc_is_zero ? 0.f : a.dc[i];
     dc = dc + (1.0f - tc * tc) * (dh * o);

@@ -1,0 +1,278 @@
+// Fused LSTM time-step kernels for gfx950.
+//
+// One recurrent step multiplies a [rows, F+H] operand by weights that stay the same for the whole sequence
+// and is far too small to fill the chip as a tiled GEMM followed by an element-wise pass.  Here one workgroup
+// owns 32 batch rows x 64 output columns, stages the WHOLE reduction dimension of both operands in LDS with
+// every global load in flight at once, multiplies with v_mfma_f32_16x16x4_f32 (one 16-column block per
+// wavefront, two row blocks each) and finishes the step in its epilogue:
+//   forward  (layer/RNN.scala:303-340): the 64 columns are the four gates of 16 hidden units, so the
+//            workgroup applies the gate activations and writes gates, c_t and h_t itself;
+//   backward (the dz * Wr^T product of the reverse step): the reduction over 4H is cut per gate, each cut
+//            writes its own partial dh, and the gate-gradient kernel of the next (earlier) step adds the four.
+#include "common.hpp"
+
+namespace sn {
+namespace {
+
+typedef float f4v __attribute__((ext_vector_type(4)));
+constexpr int RB = 32;        // batch rows per workgroup
+constexpr int CB = 64;        // output columns per workgroup (16 per wavefront)
+constexpr int ZP = 17;        // row pitch of the pre-activation exchange area
+constexpr int MAX_K = 400;    // (32*(K+4) + 64*K + 4*32*17) floats of LDS must fit in 160 KiB
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__host__ __device__ inline int round16(int k) { return (k + 15) & ~15; }
+
+// acc0 / acc1 += A[rows 0..15 / 16..31][:] * B[:, 16 columns of this wavefront].
+// As: [RB][K16+4].  Bs: [4 wavefronts][K16/4][16 columns][4 consecutive k].  Lane (row = l%16, g = l/16) feeds
+// k = 16 kb + 4 g + j into the j-th MFMA of block kb, so both operands come from one 16-byte LDS read each.
+__device__ __forceinline__ void multiply_32x16(const float* As, const float* Bs, int K16, int wave, int lane, f4v& acc0, f4v& acc1) {
+  const int row = lane & 15, g = lane >> 4;
+  const float* ap0 = As + row * (K16 + 4) + 4 * g;
+  const float* ap1 = ap0 + 16 * (K16 + 4);
+  const float* bp = Bs + (((int64_t)wave * (K16 / 4) + g) * 16 + row) * 4;
+#pragma unroll 2
+  for (int kb = 0; kb < K16 / 16; ++kb) {
+    const f4v a0 = *(const f4v*)(ap0 + 16 * kb);
+    const f4v a1 = *(const f4v*)(ap1 + 16 * kb);
+    const f4v b = *(const f4v*)(bp + kb * 256);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[j], b[j], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[j], b[j], acc1, 0, 0, 0);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------- forward step
+struct StepFwdArgs {
+  const float* x;       // [rows, T, F]
+  const float* h_prev;  // [rows, H] or null (first step: h_{-1} = 0 drops out of the product)
+  const float* c_prev;  // [rows, H] or null
+  LstmWeights w;
+  float* gates;         // [rows, 4H] activated forget, input, gate, output
+  float* c;             // [rows, H]
+  float* h;             // [rows, H]
+  int rows, T, F, H, t;
+};
+
+__global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int K = a.h_prev ? a.F + a.H : a.F;
+  const int K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
+  float* As = lds;                 // [RB][KP]
+  float* Bs = lds + RB * KP;       // [4 gates][kq][16 units][4]
+  float* Zx = Bs + CB * K16;       // [4 gates][RB][ZP]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r0 = blockIdx.y * RB, u0 = blockIdx.x * 16;
+
+  // ---- stage both operands.  Every global load of a pass is issued before the first LDS write, and one
+  // pass covers F + H up to 384 (NA = 12 row vectors, NB = 24 weight cells per thread), so the whole tile
+  // costs one memory latency.
+  // Index maps without divisions: 8 threads per operand row take 16-byte vectors q = tid%8 + 8i; for the
+  // weights a thread owns unit tid%16 and the k quads q = tid/16 + 16i of every gate, gathering the 4 values
+  // of one LDS cell, so consecutive lanes write consecutive cells and read 64-byte runs of each weight row.
+  constexpr int NA = 12, NQ = 6;  // enough for MAX_K: 8 * NA and 16 * NQ quads
+  for (int pass = 0; pass * 8 * NA < kq; ++pass) {
+    f4v va[NA], vb[4][NQ];
+    const int arow = tid >> 3, bu = tid & 15;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int q = (pass * NA + i) * 8 + (tid & 7), k = q * 4;
+      va[i] = f4v{0.f, 0.f, 0.f, 0.f};
+      if (q < kq && r0 + arow < a.rows && k < K)
+        va[i] = k < a.F ? *(const f4v*)(a.x + ((int64_t)(r0 + arow) * a.T + a.t) * a.F + k)
+                        : *(const f4v*)(a.h_prev + (int64_t)(r0 + arow) * a.H + (k - a.F));
+    }
+    if (pass * 16 * NQ < kq) {
+#pragma unroll
+      for (int gate = 0; gate < 4; ++gate)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          const int q = (pass * NQ + i) * 16 + (tid >> 4), k = q * 4;
+          vb[gate][i] = f4v{0.f, 0.f, 0.f, 0.f};
+          if (q < kq && k < K) {
+            const float* src = (k < a.F ? a.w.wk[gate] + (int64_t)k * a.H : a.w.wr[gate] + (int64_t)(k - a.F) * a.H) + u0 + bu;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) vb[gate][i][j] = src[(int64_t)j * a.H];
+          }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int q = (pass * NA + i) * 8 + (tid & 7);
+      if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
+    }
+    if (pass * 16 * NQ < kq) {
+#pragma unroll
+      for (int gate = 0; gate < 4; ++gate)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          const int q = (pass * NQ + i) * 16 + (tid >> 4);
+          if (q < kq) *(f4v*)(Bs + ((gate * kq + q) * 16 + bu) * 4) = vb[gate][i];
+        }
+    }
+  }
+  __syncthreads();
+
+  f4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  multiply_32x16(As, Bs, K16, wave, lane, acc0, acc1);
+
+  // ---- pre-activations of gate `wave` to the exchange area: element v of a lane is row 4*(l/16) + v, column l%16
+  {
+    const int col = lane & 15, g = lane >> 4;
+    const float bias = a.w.b[wave] ? a.w.b[wave][u0 + col] : 0.f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      Zx[(wave * RB + 4 * g + v) * ZP + col] = acc0[v] + bias;
+      Zx[(wave * RB + 16 + 4 * g + v) * ZP + col] = acc1[v] + bias;
+    }
+  }
+  __syncthreads();
+  // ---- c = c_prev * f + i * g ; h = o * tanh(c)   (layer/RNN.scala:336-337)
+#pragma unroll
+  for (int e = tid; e < RB * 16; e += 256) {
+    const int row = e >> 4, u = e & 15;
+    if (r0 + row >= a.rows) continue;
+    const float f = sigmoidf_(Zx[(0 * RB + row) * ZP + u]);
+    const float in = sigmoidf_(Zx[(1 * RB + row) * ZP + u]);
+    const float g = tanhf(Zx[(2 * RB + row) * ZP + u]);
+    const float o = sigmoidf_(Zx[(3 * RB + row) * ZP + u]);
+    const int64_t i = (int64_t)(r0 + row) * a.H + u0 + u;
+    const int64_t zb = (int64_t)(r0 + row) * 4 * a.H + u0 + u;
+    const float cp = a.c_prev ? a.c_prev[i] : 0.f;
+    const float c = cp * f + in * g;
+    a.gates[zb] = f;
+    a.gates[zb + a.H] = in;
+    a.gates[zb + 2 * a.H] = g;
+    a.gates[zb + 3 * a.H] = o;
+    a.c[i] = c;
+    a.h[i] = o * tanhf(c);
+  }
+}
+
+// ---------------------------------------------------------------------------- backward: partial dh per gate
+struct StepDhArgs {
+  const float* dz;      // [rows, 4H]
+  const float* wr[4];   // [H, H] recurrent weights per gate
+  float* dh_parts;      // [4][part_stride] partial dh_prev, one per gate
+  int64_t part_stride;
+  int rows, H;
+};
+
+// dh_parts[gate][m, u] = sum_n dz[m, gate*H + n] * Wr_gate[u, n]
+__global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int K = a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
+  float* As = lds;            // [RB][KP]
+  float* Bs = lds + RB * KP;  // [4 wavefronts][kq][16 units][4]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r0 = blockIdx.y * RB, u0 = blockIdx.x * CB, gate = blockIdx.z;
+  const float* dzg = a.dz + (int64_t)gate * a.H;
+
+  // Staging as in the forward kernel: one pass (H up to 384) with every load in flight before the LDS writes.
+  // B(k = n, column = u) = Wr_gate[u][n]: n is contiguous in memory, so a 16-byte load is already one LDS cell.
+  constexpr int NA = 12, NQ = 6;
+  for (int pass = 0; pass * 8 * NA < kq; ++pass) {
+    f4v va[NA], vb[4][NQ];
+    const int arow = tid >> 3, bu = tid & 15;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int q = (pass * NA + i) * 8 + (tid & 7);
+      va[i] = f4v{0.f, 0.f, 0.f, 0.f};
+      if (q < kq && r0 + arow < a.rows && q * 4 < K) va[i] = *(const f4v*)(dzg + (int64_t)(r0 + arow) * 4 * a.H + q * 4);
+    }
+    if (pass * 16 * NQ < kq) {
+#pragma unroll
+      for (int wv = 0; wv < 4; ++wv)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          const int q = (pass * NQ + i) * 16 + (tid >> 4), u = u0 + wv * 16 + bu;
+          vb[wv][i] = f4v{0.f, 0.f, 0.f, 0.f};
+          if (q < kq && u < a.H && q * 4 < K) vb[wv][i] = *(const f4v*)(a.wr[gate] + (int64_t)u * a.H + q * 4);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int q = (pass * NA + i) * 8 + (tid & 7);
+      if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
+    }
+    if (pass * 16 * NQ < kq) {
+#pragma unroll
+      for (int wv = 0; wv < 4; ++wv)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+          const int q = (pass * NQ + i) * 16 + (tid >> 4);
+          if (q < kq) *(f4v*)(Bs + ((wv * kq + q) * 16 + bu) * 4) = vb[wv][i];
+        }
+    }
+  }
+  __syncthreads();
+
+  f4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  multiply_32x16(As, Bs, K16, wave, lane, acc0, acc1);
+
+  const int col = u0 + wave * 16 + (lane & 15), g = lane >> 4;
+  if (col < a.H) {
+    float* out = a.dh_parts + (int64_t)gate * a.part_stride;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int ra = r0 + 4 * g + v, rb = ra + 16;
+      if (ra < a.rows) out[(int64_t)ra * a.H + col] = acc0[v];
+      if (rb < a.rows) out[(int64_t)rb * a.H + col] = acc1[v];
+    }
+  }
+}
+
+size_t lds_bytes(int K) {
+  const int K16 = round16(K);
+  return ((size_t)RB * (K16 + 4) + (size_t)CB * K16 + 4 * RB * ZP) * sizeof(float);
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w) {
+  if (F % 4 != 0 || H % 16 != 0 || F + H > MAX_K || !aligned16(x)) return false;
+  for (int g = 0; g < 4; ++g)
+    if (!aligned16(w.wk[g]) || !aligned16(w.wr[g])) return false;
+  return true;
+}
+
+int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
+                         const LstmWeights& w, float* gates, float* c, float* h) {
+  if (rows <= 0) return SN_OK;
+  SN_REQUIRE(lstm_step_fused_ok(F, H, x, w), "lstm_step_forward: F=%d H=%d outside what the fused kernel handles", F, H);
+  static bool attr_set = false;
+  if (!attr_set) {
+    SN_HIP(hipFuncSetAttribute((const void*)lstm_step_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(MAX_K)));
+    attr_set = true;
+  }
+  StepFwdArgs a{x, h_prev, c_prev, w, gates, c, h, rows, T, F, H, t};
+  const dim3 grid((unsigned)(H / 16), (unsigned)ceil_div(rows, RB));
+  LaunchScope scope(ctx, "lstm_step_forward", rows, 4 * H, h_prev ? F + H : F);
+  hipLaunchKernelGGL(lstm_step_fwd_kernel, grid, dim3(256), lds_bytes(h_prev ? F + H : F), ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_parts, int64_t part_stride) {
+  if (rows <= 0) return SN_OK;
+  SN_REQUIRE(H % 4 == 0 && H <= MAX_K && aligned16(dz) && aligned16(w.wr[0]) && aligned16(w.wr[1]) && aligned16(w.wr[2]) && aligned16(w.wr[3]),
+             "lstm_step_hidden_gradient: H=%d outside what the fused kernel handles", H);
+  static bool attr_set = false;
+  if (!attr_set) {
+    SN_HIP(hipFuncSetAttribute((const void*)lstm_step_dh_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(MAX_K)));
+    attr_set = true;
+  }
+  StepDhArgs a{dz, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, dh_parts, part_stride, rows, H};
+  const dim3 grid((unsigned)ceil_div(H, CB), (unsigned)ceil_div(rows, RB), 4);
+  LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, 4 * H);
+  hipLaunchKernelGGL(lstm_step_dh_kernel, grid, dim3(256), lds_bytes(H), ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+}  // namespace sn

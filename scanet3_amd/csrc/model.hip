@@ -356,8 +356,8 @@ static int alloc_replica(sn_replica* r) {
     }
   }
   SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
-  SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h));
-  SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h));
+  SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h * 4));  // four per-gate partial sums each
+  SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h * 4));
   SN_TRY(dev_alloc(r, &r->lstm_dc, lstm_h));
   SN_TRY(dev_alloc(r, &r->grad_buf[0], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->grad_buf[1], B * m->max_act_elems));
@@ -452,8 +452,15 @@ static int forward(sn_replica* r, const float* x, int rows) {
         // time-major slices are laid out with the model's batch capacity so addresses do not depend on `rows`
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
+        const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
         for (int t = 0; t < op.T; ++t) {
           const float* h_prev = r->lstm_h[i] + (int64_t)t * bh;
+          if (fused) {
+            SN_TRY(launch_lstm_step_fwd(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh,
+                                        rows, op.H, w, r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
+                                        r->lstm_h[i] + (int64_t)(t + 1) * bh));
+            continue;
+          }
           SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, rows, op.H, w, r->lstm_z, r->ws, m->workspace_elems));
           LstmGateArgs a{r->lstm_z, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, r->lstm_gates[i] + (int64_t)t * bh * 4,
                          r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
@@ -567,15 +574,21 @@ static int backward(sn_replica* r, const float* x, int rows) {
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
         const float* dh = dy;  // gradient of the last hidden state
-        int hb = 0;
+        int hb = 0, dh_parts = 1;
+        const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
         for (int t = op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                             t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
-                            r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0};
+                            r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0, dh_parts, bh};
           SN_TRY(launch_lstm_gates_bwd(ctx, a, rows, op.H));
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
           if (t > 0) {
-            SN_TRY(launch_lstm_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], r->ws, m->workspace_elems));
+            if (fused) {  // four per-gate partial products; the next gate-gradient kernel adds them
+              SN_TRY(launch_lstm_step_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], bh));
+              dh_parts = 4;
+            } else {
+              SN_TRY(launch_lstm_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], r->ws, m->workspace_elems));
+            }
             dh = r->lstm_dh[hb];
             hb ^= 1;
           }
