@@ -20,7 +20,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int BK = 16;
 constexpr int THREADS = 256;
-constexpr int PF = 1;  // k-tiles of global loads in flight per workgroup
 
 // ============================================================================ loaders
 // A loader describes one operand as a function (outer index, k) -> value, where the outer
@@ -30,6 +29,37 @@ constexpr int PF = 1;  // k-tiles of global loads in flight per workgroup
 //   init     position a cursor at (outer, k)
 //   load     value at the cursor (0 outside the matrix or past k_end)
 //   advance  move the cursor dk along k
+// The kernel drives a loader through a second, finer interface that separates what is the same for the
+// whole workgroup in one k tile (struct Tile: the tile's first k and whatever follows from it, kept in
+// scalar registers) from what belongs to the thread (Cursor):
+//   init4(c, outer, k_begin, kk)   kk = the thread's fixed k offset inside every tile
+//   tile_init / tile_advance        uniform state for the tile starting at k0, then k0 += BK
+//   thread_advance                  per-thread part of moving on one tile (nothing for the FAST loaders)
+//   load_t / load4_t                value(s) at (cursor, tile)
+// Loaders written against the cursor interface only get the second one from SN_CURSOR_ONLY_API; the FAST
+// loaders implement it directly with 32-bit offsets, a per-thread validity mask and no branches.
+#define SN_CURSOR_ONLY_API                                                                                         \
+  static constexpr bool FAST = false;                                                                              \
+  struct Tile {};                                                                                                  \
+  __device__ __forceinline__ void tile_init(Tile&, int) const {}                                                   \
+  __device__ __forceinline__ void tile_advance(Tile&) const {}                                                     \
+  __device__ __forceinline__ void thread_advance(Cursor& c) const { advance(c, BK); }                              \
+  __device__ __forceinline__ void init4(Cursor& c, int outer, int kb, int kk) const { init(c, outer, kb + kk); }   \
+  __device__ __forceinline__ float load_t(const Cursor& c, const Tile&, int k_end) const { return load(c, k_end); } \
+  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile&, int k_end, float (&v)[4]) const { load4(c, k_end, v); }
+
+// 16-byte load without a branch: a lane whose element lies outside the matrix reads the first 16 bytes of
+// the tensor instead (always mapped, 16-byte aligned) and discards them.  Offsets are 32-bit: the host only
+// picks the FAST loaders for tensors below 2 GiB.
+constexpr int64_t FAST_SPAN = (int64_t)1 << 31;
+__device__ __forceinline__ void sel_load4(const float* base, uint32_t byte_off, bool valid, float (&v)[4]) {
+  const f4v r = *(const f4v*)((const char*)base + (valid ? byte_off : 0u));
+  v[0] = valid ? r[0] : 0.f;
+  v[1] = valid ? r[1] : 0.f;
+  v[2] = valid ? r[2] : 0.f;
+  v[3] = valid ? r[3] : 0.f;
+}
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <bool KC>
 struct StridedLoader {
@@ -60,6 +90,7 @@ struct StridedLoader {
     return KC ? (s_k == 1 && s_outer % 4 == 0 && K % 4 == 0 && aligned) : (s_outer == 1 && s_k % 4 == 0 && outer_n % 4 == 0 && aligned);
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+  SN_CURSOR_ONLY_API
 };
 
 // ---- Conv2D forward: A(m,k) = x[b, oh*sh-pt+r, ow*sw-pl+q, ci], m=(b,oh,ow), k=(r,q,ci)
@@ -108,6 +139,7 @@ struct ConvFwdA {
       if (++c.q == g.kw) { c.q = 0; ++c.r; }
     }
   }
+  SN_CURSOR_ONLY_API
 };
 
 // ---- Conv2D input gradient: dx[b,iy,ix,ci] = sum_{r,q,co} dy[b,(iy+pt-r)/sh,(ix+pl-q)/sw,co] * w[r,q,ci,co]
@@ -165,6 +197,7 @@ struct ConvDgradA {  // m=(b,iy,ix), k=(r,q,co)
       if (++c.q == g.kw) { c.q = 0; ++c.r; }
     }
   }
+  SN_CURSOR_ONLY_API
 };
 
 struct ConvDgradB {  // outer n = ci, k=(r,q,co): w[((r*kw+q)*cin + ci)*cout + co]
@@ -195,6 +228,7 @@ struct ConvDgradB {  // outer n = ci, k=(r,q,co): w[((r*kw+q)*cin + ci)*cout + c
     c.co += dk;
     while (c.co >= g.cout) { c.co -= g.cout; ++c.rq; }
   }
+  SN_CURSOR_ONLY_API
 };
 
 // ---- Conv2D filter gradient: dw[r,q,ci,co] = sum_{b,oh,ow} x[b,oh*sh-pt+r,ow*sw-pl+q,ci] * dy[b,oh,ow,co]
@@ -243,6 +277,7 @@ struct ConvWgradA {  // m=(r,q,ci) (ci fastest -> contiguous), k=(b,oh,ow)
       if (++c.oh == g.ho) { c.oh = 0; ++c.b; }
     }
   }
+  SN_CURSOR_ONLY_API
 };
 
 // ---- LSTM step: A(m,k) = k < F ? x[m, t, k] : h_prev[m, k-F]
@@ -272,6 +307,7 @@ struct LstmZA {
     return F % 4 == 0 && H % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(h_prev) & 15u) == 0;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+  SN_CURSOR_ONLY_API
 };
 
 // B(k,n) with n = gate*H + u: k < F ? Wk_gate[k, u] : Wr_gate[k-F, u]
@@ -306,6 +342,7 @@ struct LstmZB {
     return ok;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+  SN_CURSOR_ONLY_API
 };
 
 // B(k,n) = W_gate[n, u], k = gate*H + u (transposed gate weights: dh = dz Wr^T, dx = dz Wk^T)
@@ -336,6 +373,7 @@ struct LstmWT {
     return ok;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
+  SN_CURSOR_ONLY_API
 };
 
 // Weight gradients of all steps at once: A(m,k), k = t*rows + b:
@@ -377,6 +415,143 @@ struct LstmWgradA {
     c.b += dk;
     while (c.b >= rows) { c.b -= rows; ++c.t; }
   }
+  SN_CURSOR_ONLY_API
+};
+
+// ============================================================================ FAST loaders
+// Strided operand with unit stride along its contiguous index: value(outer, k) = p[outer*s_outer + k*s_k].
+template <bool KC>
+struct FlatLoader {
+  static constexpr bool K_CONTIG = KC, FAST = true;
+  const float* p;
+  int s_outer, s_k;  // elements; one of them is 1
+  int outer_n;
+  struct Cursor {
+    uint32_t base;  // byte offset of (outer, kk)
+    int kk;         // < 0: outside the matrix
+  };
+  struct Tile {
+    int k0;
+    uint32_t koff;  // byte offset of k0
+  };
+  __device__ __forceinline__ void init4(Cursor& c, int outer, int, int kk) const {
+    c.kk = outer < outer_n ? kk : -0x40000000;
+    c.base = ((uint32_t)outer * (uint32_t)s_outer + (uint32_t)kk * (uint32_t)s_k) * 4u;
+  }
+  __device__ __forceinline__ void tile_init(Tile& t, int k0) const { t.k0 = k0; t.koff = (uint32_t)k0 * (uint32_t)s_k * 4u; }
+  __device__ __forceinline__ void tile_advance(Tile& t) const { t.k0 += BK; t.koff += (uint32_t)BK * (uint32_t)s_k * 4u; }
+  __device__ __forceinline__ void thread_advance(Cursor&) const {}
+  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    sel_load4(p, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
+  }
+  __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }  // FAST loaders run VEC = 4 only
+  static bool ok(const float* p, int64_t s_outer, int64_t s_k, int outer_n, int K) {
+    if (!aligned16(p) || s_outer < 0 || s_k < 0 || ((int64_t)outer_n * s_outer + (int64_t)K * s_k) * 4 >= FAST_SPAN) return false;
+    return KC ? (s_k == 1 && s_outer % 4 == 0 && K % 4 == 0) : (s_outer == 1 && s_k % 4 == 0 && outer_n % 4 == 0);
+  }
+};
+
+// A operand of a convolution seen as a product: row m is a position (b, iy, ix) of the iteration space
+// (the output for the forward pass, the input for the input gradient), k = (tap r, tap q, channel) with the
+// channel fastest and the channel count a multiple of BK, so that a k tile lies inside one tap:
+//   value = src[b, iy*sy + oy + r*ty, ix*sx + ox + q*tx, channel]   (0 outside the source image)
+// forward: src = x, (sy, sx) = strides, (oy, ox) = -padding, (ty, tx) = (+1, +1);
+// input gradient with unit strides: src = dy, (sy, sx) = (1, 1), (oy, ox) = +padding, (ty, tx) = (-1, -1).
+// Which taps fall inside the image is fixed per row: a 32-bit mask computed once per thread.
+struct TapLoader {
+  static constexpr bool K_CONTIG = true, FAST = true;
+  const float* src;
+  int M, ih, iw;       // iteration space
+  int sy, sx, oy, ox, ty, tx;
+  int H, W, C;         // source image
+  int kh, kw;
+  struct Cursor {
+    uint32_t base;  // byte offset of (b, y0, x0, kk), possibly outside the tensor (then no tap is valid there)
+    uint32_t mask;  // bit r*kw+q: tap inside the image
+    int kk;
+  };
+  struct Tile {
+    int k0, r, q, c0, rq;
+    uint32_t tapoff;  // byte offset of (r*ty, q*tx, c0) relative to (y0, x0, 0)
+  };
+  __device__ __forceinline__ void init4(Cursor& c, int m, int, int kk) const {
+    c.kk = kk;
+    c.mask = 0;
+    c.base = 0;
+    if (m >= M) return;
+    const int ix = m % iw;
+    const int t = m / iw;
+    const int iy = t % ih;
+    const int b = t / ih;
+    const int y0 = iy * sy + oy, x0 = ix * sx + ox;
+    c.base = (uint32_t)(((b * H + y0) * W + x0) * C + kk) * 4u;
+    for (int r = 0; r < kh; ++r)
+      for (int q = 0; q < kw; ++q)
+        if ((unsigned)(y0 + r * ty) < (unsigned)H && (unsigned)(x0 + q * tx) < (unsigned)W) c.mask |= 1u << (r * kw + q);
+  }
+  __device__ __forceinline__ void set_tap(Tile& t) const { t.tapoff = (uint32_t)((t.r * ty * W + t.q * tx) * C + t.c0) * 4u; }
+  __device__ __forceinline__ void tile_init(Tile& t, int k0) const {
+    t.k0 = k0;
+    t.rq = k0 / C;
+    t.c0 = k0 - t.rq * C;
+    t.r = t.rq / kw;
+    t.q = t.rq - t.r * kw;
+    set_tap(t);
+  }
+  __device__ __forceinline__ void tile_advance(Tile& t) const {
+    t.k0 += BK;
+    t.c0 += BK;
+    if (t.c0 >= C) {
+      t.c0 = 0;
+      ++t.rq;
+      if (++t.q == kw) { t.q = 0; ++t.r; }
+    }
+    set_tap(t);
+  }
+  __device__ __forceinline__ void thread_advance(Cursor&) const {}
+  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    sel_load4(src, c.base + t.tapoff, ((c.mask >> (t.rq & 31)) & 1u) != 0 && t.k0 + c.kk < k_end, v);
+  }
+  __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
+  static bool ok(const float* src, int n, int H, int W, int C, int kh, int kw) {
+    return C % BK == 0 && kh * kw <= 32 && aligned16(src) && (int64_t)n * H * W * C * 4 < FAST_SPAN;
+  }
+};
+
+// B operand of the input gradient: column n = ci, k = (r, q, co): w[((r*kw+q)*cin + ci)*cout + co], cout % BK == 0
+struct DgradWLoader {
+  static constexpr bool K_CONTIG = true, FAST = true;
+  const float* w;
+  int cin, cout;
+  struct Cursor {
+    uint32_t base;  // byte offset of (tap 0, ci, kk)
+    int kk;         // < 0: outside the matrix
+  };
+  struct Tile {
+    int k0, c0, rq;
+    uint32_t koff;
+  };
+  __device__ __forceinline__ void init4(Cursor& c, int n, int, int kk) const {
+    c.kk = n < cin ? kk : -0x40000000;
+    c.base = (uint32_t)(n * cout + kk) * 4u;
+  }
+  __device__ __forceinline__ void tile_init(Tile& t, int k0) const {
+    t.k0 = k0;
+    t.rq = k0 / cout;
+    t.c0 = k0 - t.rq * cout;
+    t.koff = (uint32_t)(t.rq * cin * cout + t.c0) * 4u;
+  }
+  __device__ __forceinline__ void tile_advance(Tile& t) const {
+    t.k0 += BK;
+    t.c0 += BK;
+    if (t.c0 >= cout) { t.c0 = 0; ++t.rq; }
+    t.koff = (uint32_t)(t.rq * cin * cout + t.c0) * 4u;
+  }
+  __device__ __forceinline__ void thread_advance(Cursor&) const {}
+  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    sel_load4(w, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
+  }
+  __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
 };
 
 // ============================================================================ epilogues
@@ -463,13 +638,15 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 
   typename AL::Cursor ca[EA];
   typename BL::Cursor cb[EB];
+  typename AL::Tile ta;
+  typename BL::Tile tb;
   int ia[EA], ib[EB];  // LDS slot of the first value of each vector; the others follow one slot apart
 #pragma unroll
   for (int e = 0; e < EA; ++e) {
     int mm, kk;
     if (AL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; mm = tid / KV + e * (THREADS / KV); }
     else { constexpr int OV = BM / VEC; mm = (tid % OV) * VEC; kk = tid / OV + e * (THREADS / OV); }
-    al.init(ca[e], m0 + mm, k_begin + kk);
+    al.init4(ca[e], m0 + mm, k_begin, kk);
     ia[e] = lds_index<AL::K_CONTIG, BM>(mm, kk);
   }
 #pragma unroll
@@ -478,9 +655,11 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
     if (BL::K_CONTIG) { constexpr int KV = BK / VEC; kk = (tid % KV) * VEC; nn = tid / KV + e * (B_ACTIVE / KV); }
     else { constexpr int OV = BN / VEC; nn = (tid % OV) * VEC; kk = tid / OV + e * (B_ACTIVE / OV); }
     if (!b_on) { nn = 0; kk = 0; }
-    bl.init(cb[e], n0 + nn, k_begin + kk);
+    bl.init4(cb[e], n0 + nn, k_begin, kk);
     ib[e] = lds_index<BL::K_CONTIG, BN>(nn, kk);
   }
+  al.tile_init(ta, k_begin);
+  bl.tile_init(tb, k_begin);
 
   f16v acc[TM][TN];
 #pragma unroll
@@ -490,84 +669,75 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  // Both staging layouts put consecutive values of the contiguous index one LDS slot apart.
-  // Global loads run PF k-tiles ahead of the multiplication through a ring of register stages: with few
-  // workgroups per CU it is the load latency, not the matrix cores, that a short-K product waits on.
-  float ra[PF][EA][VEC], rb[PF][EB][VEC];
-  int k_fetch = k_begin;  // first k of the next tile to load
-  auto fetch = [&](int s) {  // loads the tile the cursors point at, unless it lies past k_end, and moves them on
-    if (k_fetch < k_end) {
+  // both staging layouts put consecutive values of the contiguous index one LDS slot apart
+  float ra[EA][VEC], rb[EB][VEC];
+  auto fetch = [&]() {  // loads the tile the loaders point at (zeros past k_end), then moves them on
 #pragma unroll
-      for (int e = 0; e < EA; ++e) {
-        if constexpr (VEC == 4) al.load4(ca[e], k_end, ra[s][e]);
-        else ra[s][e][0] = al.load(ca[e], k_end);
-        al.advance(ca[e], BK);
-      }
-      if (b_on) {
+    for (int e = 0; e < EA; ++e) {
+      if constexpr (VEC == 4) al.load4_t(ca[e], ta, k_end, ra[e]);
+      else ra[e][0] = al.load_t(ca[e], ta, k_end);
+      al.thread_advance(ca[e]);
+    }
+    if (b_on) {
 #pragma unroll
-        for (int e = 0; e < EB; ++e) {
-          if constexpr (VEC == 4) bl.load4(cb[e], k_end, rb[s][e]);
-          else rb[s][e][0] = bl.load(cb[e], k_end);
-          bl.advance(cb[e], BK);
-        }
+      for (int e = 0; e < EB; ++e) {
+        if constexpr (VEC == 4) bl.load4_t(cb[e], tb, k_end, rb[e]);
+        else rb[e][0] = bl.load_t(cb[e], tb, k_end);
+        bl.thread_advance(cb[e]);
       }
     }
-    k_fetch += BK;
+    al.tile_advance(ta);
+    bl.tile_advance(tb);
   };
-#pragma unroll
-  for (int s = 0; s < PF; ++s) fetch(s);
+  fetch();
 
   const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
-  for (int kb = k_begin; kb < k_end; kb += BK * PF) {
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
 #pragma unroll
-    for (int s = 0; s < PF; ++s) {
-      if (kb + s * BK >= k_end) break;
+    for (int e = 0; e < EA; ++e)
 #pragma unroll
-      for (int e = 0; e < EA; ++e)
+      for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[e][i];
+    if (b_on) {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[s][e][i];
-      if (b_on) {
+      for (int e = 0; e < EB; ++e)
 #pragma unroll
-        for (int e = 0; e < EB; ++e)
-#pragma unroll
-          for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[s][e][i];
-      }
-      __syncthreads();
-      fetch(s);  // the tile PF steps ahead takes over this stage's registers
-      if constexpr (!BF16) {
-#pragma unroll
-        for (int ks = 0; ks < BK; ks += 2) {
-          const int k = ks + lhi;
-          float av[TM], bv[TN];
-#pragma unroll
-          for (int i = 0; i < TM; ++i) av[i] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, k)];
-#pragma unroll
-          for (int j = 0; j < TN; ++j) bv[j] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, k)];
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
-        }
-      } else {
-        // 32x32x16 bf16: lane supplies k = 8*(lane/32) .. +7 of row/col lane%32
-        bf16x8 av[TM], bv[TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int v = 0; v < 8; ++v) av[i][v] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, lhi * 8 + v)];
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int v = 0; v < 8; ++v) bv[j][v] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, lhi * 8 + v)];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
-      }
-      __syncthreads();
+        for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
     }
+    __syncthreads();
+    if (k0 + BK < k_end) fetch();  // the next tile's global loads fly while this one is multiplied
+    if constexpr (!BF16) {
+#pragma unroll
+      for (int ks = 0; ks < BK; ks += 2) {
+        const int k = ks + lhi;
+        float av[TM], bv[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) av[i] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, k)];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bv[j] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, k)];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+      }
+    } else {
+      // 32x32x16 bf16: lane supplies k = 8*(lane/32) .. +7 of row/col lane%32
+      bf16x8 av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int v = 0; v < 8; ++v) av[i][v] = As[lds_index<AL::K_CONTIG, BM>(wm + i * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 8; ++v) bv[j][v] = Bs[lds_index<BL::K_CONTIG, BN>(wn + j * 32 + l32, lhi * 8 + v)];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
   }
 
   // accumulator element v of lane l sits at row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
@@ -724,12 +894,17 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   const dim3 grid((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), (unsigned)splits);
   {
     LaunchScope scope(ctx, name, M, N, K);
-    if (al.vec4_ok(K) && bl.vec4_ok(K))
+    if constexpr (AL::FAST && BL::FAST) {  // the caller has checked what 16-byte loads need
       hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 4, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
                          splits > 1 ? ws : nullptr);
-    else
-      hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 1, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
-                         splits > 1 ? ws : nullptr);
+    } else {
+      if (al.vec4_ok(K) && bl.vec4_ok(K))
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 4, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
+                           splits > 1 ? ws : nullptr);
+      else
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 1, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
+                           splits > 1 ? ws : nullptr);
+    }
   }
   if (splits > 1) {
     const int64_t total = (int64_t)M * N;
@@ -746,7 +921,8 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
                       int64_t ws_elems) {
   if (M <= 0 || N <= 0) return SN_OK;
   SN_REQUIRE(K > 0, "%s: empty reduction dimension", name);
-  if (const int parts = ws ? small_parts(M, N, K, ctx->compute_units, ws_elems) : 0) {
+  if constexpr (!(AL::FAST && BL::FAST)) {
+   if (const int parts = ws ? small_parts(M, N, K, ctx->compute_units, ws_elems) : 0) {
     {
       LaunchScope scope(ctx, name, M, N, K);
       hipLaunchKernelGGL((gemm_small_kernel<AL, BL>), dim3((unsigned)parts), dim3(256), (size_t)SMALL_SLICE * (M + N) * sizeof(float),
@@ -757,6 +933,7 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
                        parts, M, N, ep);
     SN_HIP(hipGetLastError());
     return SN_OK;
+   }
   }
   bool big_m = M > 64, big_n = N > 64;
   // 128-wide tiles only when they still cover every CU at least once; otherwise more, smaller workgroups
@@ -773,6 +950,27 @@ static int launch_gemm_t(sn_ctx* ctx, const GemmDesc& g, const Epilogue& e, floa
   StdEpilogue ep{e};
   const char* name = BF16 ? "gemm_bf16" : "gemm_f32";
   const bool akc = g.a_sk == 1, bkc = g.b_sk == 1 && g.b_sn != 1;
+  // FAST loaders whenever both operands allow 16-byte loads, unless the small-output kernel (cursor loaders) takes the problem
+  if (!(ws && small_parts(g.m, g.n, g.k, ctx->compute_units, ws_elems))) {
+    if (akc && bkc && FlatLoader<true>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) && FlatLoader<true>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k)) {
+      FlatLoader<true> al{g.a, (int)g.a_sm, (int)g.a_sk, g.m}, bl{g.b, (int)g.b_sn, (int)g.b_sk, g.n};
+      return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+    }
+    if (akc && !bkc && FlatLoader<true>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) && FlatLoader<false>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k)) {
+      FlatLoader<true> al{g.a, (int)g.a_sm, (int)g.a_sk, g.m};
+      FlatLoader<false> bl{g.b, (int)g.b_sn, (int)g.b_sk, g.n};
+      return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+    }
+    if (!akc && bkc && FlatLoader<false>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) && FlatLoader<true>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k)) {
+      FlatLoader<false> al{g.a, (int)g.a_sm, (int)g.a_sk, g.m};
+      FlatLoader<true> bl{g.b, (int)g.b_sn, (int)g.b_sk, g.n};
+      return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+    }
+    if (!akc && !bkc && FlatLoader<false>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) && FlatLoader<false>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k)) {
+      FlatLoader<false> al{g.a, (int)g.a_sm, (int)g.a_sk, g.m}, bl{g.b, (int)g.b_sn, (int)g.b_sk, g.n};
+      return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+    }
+  }
   if (akc && bkc) {
     StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
@@ -797,20 +995,31 @@ int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* works
 // ---------------------------------------------------------------------------- Conv2D
 int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e, float* ws, int64_t ws_elems) {
   const int M = g.n * g.ho * g.wo, N = g.cout, K = g.kh * g.kw * g.cin;
+  StdEpilogue ep{e};
+  if (TapLoader::ok(x, g.n, g.h, g.w, g.cin, g.kh, g.kw) && FlatLoader<false>::ok(w, 1, g.cout, N, K)) {
+    TapLoader al{x, M, g.ho, g.wo, g.sh, g.sw, -g.pt, -g.pl, 1, 1, g.h, g.w, g.cin, g.kh, g.kw};
+    FlatLoader<false> bl{w, 1, g.cout, N};
+    return launch_any<false>(ctx, "conv2d_forward", M, N, K, al, bl, ep, ws, ws_elems);
+  }
   ConvFwdA al{x, g, M};
   StridedLoader<false> bl{w, 1, (int64_t)g.cout, N};  // filter [kh,kw,cin,cout] is a row-major [K, cout] matrix
-  StdEpilogue ep{e};
   return launch_any<false>(ctx, "conv2d_forward", M, N, K, al, bl, ep, ws, ws_elems);
 }
 
 int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems) {
   const int M = g.n * g.h * g.w, N = g.cin, K = g.kh * g.kw * g.cout;
-  ConvDgradA al{dy, g, M};
-  ConvDgradB bl{w, g};
   Epilogue e;
   e.out = dx;
   e.ldo = g.cin;
   StdEpilogue ep{e};
+  if (g.sh == 1 && g.sw == 1 && TapLoader::ok(dy, g.n, g.ho, g.wo, g.cout, g.kh, g.kw) && aligned16(w) &&
+      (int64_t)K * g.cin * 4 < FAST_SPAN) {
+    TapLoader al{dy, M, g.h, g.w, 1, 1, g.pt, g.pl, -1, -1, g.ho, g.wo, g.cout, g.kh, g.kw};
+    DgradWLoader bl{w, g.cin, g.cout};
+    return launch_any<false>(ctx, "conv2d_input_gradient", M, N, K, al, bl, ep, ws, ws_elems);
+  }
+  ConvDgradA al{dy, g, M};
+  ConvDgradB bl{w, g};
   return launch_any<false>(ctx, "conv2d_input_gradient", M, N, K, al, bl, ep, ws, ws_elems);
 }
 
