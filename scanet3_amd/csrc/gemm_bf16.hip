@@ -349,12 +349,14 @@ int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt,
 __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __restrict__ src, int64_t ld, int rows, int cols,
                                                               bf16* __restrict__ out, bf16* __restrict__ out_t,
                                                               const float* __restrict__ y, int act, float act_param,
-                                                              float* __restrict__ dz) {
+                                                              float* __restrict__ dz, float* __restrict__ col_partials) {
   // 64x64 tile; a thread handles 4 consecutive columns of 4 rows (float4 in, 8-byte bf16x4 out), and on the
   // transposed side 4 consecutive rows of one column.  cols and rows are multiples of 4 (checked by the caller).
   __shared__ bf16 tile[64][68];
+  __shared__ float colp[16][64];
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const int tc = (threadIdx.x & 15) * 4, tr = threadIdx.x >> 4;
+  f4 csum = {0.f, 0.f, 0.f, 0.f};  // this thread's 4 rows of its 4 columns (fp32 values, before rounding)
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r0 + tr + 16 * i, c = c0 + tc;
@@ -372,11 +374,23 @@ __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __rest
       for (int e = 0; e < 4; ++e) b[e] = (bf16)v[e];
       if (out) *(bf16x4*)(out + (int64_t)r * cols + c) = b;
     }
+    csum += v;
 #pragma unroll
     for (int e = 0; e < 4; ++e) tile[tr + 16 * i][tc + e] = (bf16)v[e];
   }
   if (!out_t) return;
+  if (col_partials) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) colp[tr][tc + e] = csum[e];
+  }
   __syncthreads();
+  if (col_partials && threadIdx.x < 64 && c0 + threadIdx.x < cols) {  // column sums of this 64-row block, rows in a fixed order
+    float t = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) t += colp[j][threadIdx.x];
+    col_partials[(int64_t)blockIdx.y * cols + c0 + threadIdx.x] = t;
+  }
+  if (!out_t) return;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = c0 + tr + 16 * i, r = r0 + tc;  // column c of the source, rows r..r+3
@@ -390,12 +404,12 @@ __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __rest
 }
 
 int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
-                          int act, float act_param, float* dz) {
+                          int act, float act_param, float* dz, float* col_partials) {
   if (rows <= 0 || cols <= 0) return SN_OK;
   SN_REQUIRE(rows % 4 == 0 && cols % 4 == 0 && ld % 4 == 0, "cast_bf16: rows, cols and pitch must be multiples of 4");
   LaunchScope scope(ctx, y ? "activation_backward_cast_bf16" : "cast_bf16");
   hipLaunchKernelGGL(cast_transpose_kernel, dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256), 0, ctx->stream,
-                     src, ld, rows, cols, (bf16*)out, (bf16*)out_t, y, act, act_param, dz);
+                     src, ld, rows, cols, (bf16*)out, (bf16*)out_t, y, act, act_param, dz, col_partials);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

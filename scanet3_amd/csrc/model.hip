@@ -82,6 +82,7 @@ struct sn_replica {
   float* lstm_dc = nullptr;
   // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
   std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
+  float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
   bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
   std::vector<void*> owned;
 };
@@ -329,7 +330,7 @@ static int alloc_replica(sn_replica* r) {
   r->lstm_dz.assign(n_ops, nullptr);
   r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
   r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
-  int64_t lstm_z = 0, lstm_h = 0;
+  int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0;
   for (size_t i = 0; i < n_ops; ++i) {
     const Op& op = m->ops[i];
     if (op.kind == OP_FLATTEN) continue;  // a view of its input
@@ -353,8 +354,10 @@ static int alloc_replica(sn_replica* r) {
       SN_TRY(dev_alloc(r, &r->bf_dzt[i], B * op.out_elems));
       SN_TRY(dev_alloc(r, &r->bf_w[i], op.in_elems * op.out_elems));
       SN_TRY(dev_alloc(r, &r->bf_wt[i], op.in_elems * op.out_elems));
+      bf_colp = std::max(bf_colp, ceil_div(B, 64) * op.out_elems);
     }
   }
+  SN_TRY(dev_alloc(r, &r->bf_colp, bf_colp));
   SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
   SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h * 4));  // four per-gate partial sums each
   SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h * 4));
@@ -502,10 +505,12 @@ static int backward(sn_replica* r, const float* x, int rows) {
         const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
         if (dense_bf16_fast(m, op) && rows % 8 == 0) {
           // one pass: dZ = act'(Y) * dY in fp32 (bias gradient) and as bf16 in both orientations
+          // (the fp32 dZ itself is not kept: its only other reader would be the bias gradient, summed here per 64-row block)
           SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
-                                       op.act != SN_ACT_IDENTITY ? r->act[i] : nullptr, op.act, op.act_param,
-                                       op.act != SN_ACT_IDENTITY ? dy : nullptr));
-          if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
+                                       op.act != SN_ACT_IDENTITY ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
+                                       op.b >= 0 ? r->bf_colp : nullptr));
+          if (op.b >= 0)
+            SN_TRY(launch_col_sum(ctx, r->bf_colp, out_f, param_ptr(r, r->g, op.b), ceil_div(rows, 64), out_f, r->ws, m->workspace_elems));
           EpilogueBf16 ew;
           ew.e.out = param_ptr(r, r->g, op.w); ew.e.ldo = out_f;
           SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_xt[i], rows, r->bf_dzt[i], rows, in_f, out_f, rows, ew));  // dW = X^T . dZ
