@@ -112,6 +112,10 @@ int launch_softmax_bwd(sn_ctx* ctx, const float* p, const float* dp, float* dz, 
 // loss value (sum of per-element terms / divisor) into *loss_dev and d loss / d p into dp (dp may be null)
 int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp, float* loss_dev, float* partials,
                 int rows, int cols);
+// training step of a Softmax output under CategoricalCrossentropy: p, loss value and dz in one kernel per row
+// (row_loss: `rows` floats of scratch)
+int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
+                       int cols, bool stable);
 // out[c] = sum over rows of dy[r*ld + c]; `ws` (optional) lets many rows be summed in parallel slices
 int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems);
 int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev);

@@ -242,6 +242,63 @@ int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp
   return SN_OK;
 }
 
+// Softmax output + CategoricalCrossentropy in one pass per row (training step only): p, the row's loss term
+// and dz = p*dp - p*sum(p*dp) with dp = (y * -(1/rows)) / (p + e), i.e. exactly what softmax_fwd_kernel,
+// loss_stage1_kernel and softmax_bwd_kernel compute one after the other, without the dp round trip.
+__global__ __launch_bounds__(256) void softmax_cce_kernel(const float* __restrict__ z, const float* __restrict__ y, float* __restrict__ p,
+                                                           float* __restrict__ dz, float* __restrict__ row_loss, int cols, int stable,
+                                                           float neg_inv_rows) {
+  __shared__ float smem[4];
+  const int64_t base = (int64_t)blockIdx.x * cols;
+  const float eps = 1e-8f;
+  float mx = 0.f;
+  if (stable) {
+    float m = -INFINITY;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) m = fmaxf(m, z[base + c]);
+    mx = block_max(m, smem);
+  }
+  float s = 0.f;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float e = expf(z[base + c] - mx);
+    p[base + c] = e;  // re-read below by the thread that wrote it
+    s += e;
+  }
+  const float total = block_sum(s, smem);
+  float term = 0.f, dot = 0.f;
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float pi = p[base + c] / total, yi = y[base + c];
+    p[base + c] = pi;
+    term += yi * logf(pi + eps);
+    dot += pi * ((yi * neg_inv_rows) / (pi + eps));
+  }
+  const float row_term = block_sum(term, smem);
+  const float row_dot = block_sum(dot, smem);
+  for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+    const float pi = p[base + c];
+    const float dpi = (y[base + c] * neg_inv_rows) / (pi + eps);
+    dz[base + c] = pi * dpi - pi * row_dot;
+  }
+  if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
+}
+
+int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
+                       int cols, bool stable) {
+  SN_REQUIRE(rows > 0 && cols > 0, "loss over an empty batch");
+  {
+    LaunchScope scope(ctx, "softmax_crossentropy_fused");
+    const int threads = cols <= 64 ? 64 : 256;
+    hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0,
+                       -(1.0f / (float)rows));
+  }
+  {
+    LaunchScope scope(ctx, "loss_stage2");
+    hipLaunchKernelGGL(loss_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, (int)SN_LOSS_CATEGORICAL_CROSSENTROPY, (const float*)row_loss,
+                       rows, loss_dev, 0.f, (float)rows);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
 // ---------------------------------------------------------------------------- column sums (bias gradient)
 // out[c] = sum_r dy[r, c] (Plus's gradient: Sum over the broadcast axes, AllKernels.scala:21-31).
 // A block owns 64 columns; its 4 waves stride over the rows; partial sums meet in LDS.

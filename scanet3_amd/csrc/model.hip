@@ -366,7 +366,7 @@ static int alloc_replica(sn_replica* r) {
   SN_TRY(dev_alloc(r, &r->grad_buf[1], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->ws, m->workspace_elems));
   SN_TRY(dev_alloc(r, &r->loss_dev, 1));
-  SN_TRY(dev_alloc(r, &r->loss_partials, 1024));
+  SN_TRY(dev_alloc(r, &r->loss_partials, std::max<int64_t>(1024, m->batch)));
   SN_TRY(dev_alloc(r, &r->count_dev, 1));
   return SN_OK;
 }
@@ -391,7 +391,8 @@ static LstmWeights lstm_weights(sn_replica* r, const Op& op, float* base) {
   return w;
 }
 
-static int forward(sn_replica* r, const float* x, int rows) {
+// skip_last: leave out the last op (the training pass fuses a Softmax output into the loss kernel)
+static int forward(sn_replica* r, const float* x, int rows, bool skip_last = false) {
   sn_model* m = r->model;
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
@@ -403,7 +404,7 @@ static int forward(sn_replica* r, const float* x, int rows) {
     r->bf_weights_stale = false;
   }
   std::vector<char> bf_ready(m->ops.size() + 1, 0);  // op i's bf16 input copies were written by op i-1's epilogue
-  for (size_t i = 0; i < m->ops.size(); ++i) {
+  for (size_t i = 0; i + (skip_last ? 1 : 0) < m->ops.size(); ++i) {
     const Op& op = m->ops[i];
     const float* in = op_output(r, (int)i - 1, x, rows);
     switch (op.kind) {
@@ -476,25 +477,30 @@ static int forward(sn_replica* r, const float* x, int rows) {
   return SN_OK;
 }
 
+static int add_penalties(sn_replica* r) {
+  for (auto& p : r->model->params)
+    if (p.reg_kind != SN_REG_NONE)
+      SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev));
+  return SN_OK;
+}
+
 // loss (+ penalty) into loss_dev; dp (may be null) receives d loss / d prediction
 static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp) {
   sn_model* m = r->model;
   if (m->loss == SN_LOSS_IDENTITY)
     SN_REQUIRE((int64_t)rows * m->out_elems == 1, "Identity loss needs a scalar model output");
   SN_TRY(launch_loss(r->ctx, m->loss, pred, y, dp, r->loss_dev, r->loss_partials, rows, (int)m->out_elems));
-  for (auto& p : m->params)
-    if (p.reg_kind != SN_REG_NONE)
-      SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev));
-  return SN_OK;
+  return add_penalties(r);
 }
 
 // ---------------------------------------------------------------------------- backward
-static int backward(sn_replica* r, const float* x, int rows) {
+// Starts at op `first` (the last op by default) whose output gradient lies in grad_buf[cur].
+static int backward(sn_replica* r, const float* x, int rows, int first = -1, int cur = 0) {
   sn_model* m = r->model;
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
-  int cur = 0;  // grad_buf[cur] holds d loss / d (output of op i)
-  for (int i = (int)m->ops.size() - 1; i >= 0; --i) {
+  if (first < 0) first = (int)m->ops.size() - 1;
+  for (int i = first; i >= 0; --i) {  // grad_buf[cur] holds d loss / d (output of op i)
     const Op& op = m->ops[i];
     const float* in = op_output(r, i - 1, x, rows);
     float* dy = r->grad_buf[cur];
@@ -629,6 +635,16 @@ static int read_loss(sn_replica* r, float* loss_host) {
 }
 
 static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
+  sn_model* m = r->model;
+  const int last = (int)m->ops.size() - 1;
+  if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
+    // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
+    SN_TRY(forward(r, x, rows, true));
+    SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], r->loss_dev, r->loss_partials, rows,
+                              (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+    SN_TRY(add_penalties(r));
+    return backward(r, x, rows, last - 1, 1);
+  }
   SN_TRY(forward(r, x, rows));
   const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);
   SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0]));
