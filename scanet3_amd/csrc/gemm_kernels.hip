@@ -554,6 +554,64 @@ struct DgradWLoader {
   __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
 };
 
+// A operand of the filter gradient: row m = (r, q, ci) with ci fastest (4 consecutive ci per load), k = output
+// pixel (b, oh, ow): x[b, oh*sh - pt + r, ow*sw - pl + q, ci].  Every thread keeps its own pixel and moves it
+// BK pixels per tile, carrying into the next output row / image by additions only.
+struct WgradXLoader {
+  static constexpr bool K_CONTIG = false, FAST = true;
+  const float* x;
+  ConvGeom g;
+  int M;
+  int interior;  // no padding: every tap of every output pixel lies inside the image, no bounds checks
+  struct Cursor {
+    uint32_t off;  // byte offset of the element
+    int ow, oh, iy, ix, kk;  // kk < 0: row outside the matrix
+  };
+  struct Tile {
+    int k0;
+  };
+  __device__ __forceinline__ void init4(Cursor& c, int m, int kb, int kk) const {
+    c.kk = m < M ? kk : -0x40000000;
+    const int ci = m % g.cin;
+    const int rq = m / g.cin;
+    const int q = rq % g.kw, r = rq / g.kw;
+    const int p = kb + kk;
+    c.ow = p % g.wo;
+    const int t = p / g.wo;
+    c.oh = t % g.ho;
+    const int b = t / g.ho;
+    c.iy = c.oh * g.sh - g.pt + r;
+    c.ix = c.ow * g.sw - g.pl + q;
+    c.off = (uint32_t)(((b * g.h + c.iy) * g.w + c.ix) * g.cin + ci) * 4u;
+  }
+  __device__ __forceinline__ void tile_init(Tile& t, int k0) const { t.k0 = k0; }
+  __device__ __forceinline__ void tile_advance(Tile& t) const { t.k0 += BK; }
+  __device__ __forceinline__ void thread_advance(Cursor& c) const {
+    c.ow += BK;
+    c.ix += BK * g.sw;
+    c.off += (uint32_t)(BK * g.sw * g.cin) * 4u;
+    while (c.ow >= g.wo) {  // next output row: back wo pixels, down sh input rows
+      c.ow -= g.wo;
+      c.ix -= g.wo * g.sw;
+      c.off += (uint32_t)((g.sh * g.w - g.wo * g.sw) * g.cin) * 4u;
+      c.iy += g.sh;
+      if (++c.oh == g.ho) {  // next image
+        c.oh = 0;
+        c.iy -= g.ho * g.sh;
+        c.off += (uint32_t)((g.h - g.ho * g.sh) * g.w * g.cin) * 4u;
+      }
+    }
+  }
+  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    const bool inside = interior || ((unsigned)c.iy < (unsigned)g.h && (unsigned)c.ix < (unsigned)g.w);
+    sel_load4(x, c.off, c.kk >= 0 && t.k0 + c.kk < k_end && inside, v);
+  }
+  __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
+  static bool ok(const float* x, const ConvGeom& g) {
+    return g.cin % 4 == 0 && aligned16(x) && ((int64_t)g.n + 1) * g.h * g.w * g.cin * 4 < FAST_SPAN;
+  }
+};
+
 // ============================================================================ epilogues
 __device__ __forceinline__ float ep_act(int act, float v, float param) {
   switch (act) {
@@ -757,14 +815,25 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
     }
 }
 
+// Adds the split-K partial tiles.  Eight lanes share one output: lane g adds splits g, g+8, ... in order, then the
+// eight partial sums are combined pairwise (a fixed tree), so the result does not depend on the launch shape.
 template <class EP>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int M, int N, EP ep) {
   const int64_t total = (int64_t)M * N;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    float s = ws[i];
-    for (int z = 1; z < splits; ++z) s += ws[(int64_t)z * total + i];
-    ep.store((int)(i / N), (int)(i % N), s);
+  const int g = threadIdx.x >> 5, j = threadIdx.x & 31;  // 8 groups of 32 consecutive outputs
+  for (int64_t base = (int64_t)blockIdx.x * 32; base < total; base += (int64_t)gridDim.x * 32) {
+    const int64_t i = base + j;
+    float s = 0.f;
+    if (i < total)
+      for (int z = g; z < splits; z += 8) s += ws[(int64_t)z * total + i];
+    __shared__ float part[8][32];
+    part[g][j] = s;
+    __syncthreads();
+    if (g == 0 && i < total) {
+      const float t = ((part[0][j] + part[1][j]) + (part[2][j] + part[3][j])) + ((part[4][j] + part[5][j]) + (part[6][j] + part[7][j]));
+      ep.store((int)(i / N), (int)(i % N), t);
+    }
+    __syncthreads();
   }
 }
 
@@ -847,10 +916,11 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int M, int N, int K, AL
   }
 }
 
+// One wavefront per output adds its partial sums (contiguous in memory) in a fixed order.
 template <class EP>
 __global__ __launch_bounds__(256) void gemm_small_reduce_kernel(const float* __restrict__ partial, int parts, int M, int N, EP ep) {
   const int lane = threadIdx.x & 63;
-  const int o = blockIdx.x * 4 + (threadIdx.x >> 6);  // one wave per output
+  const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (o >= M * N) return;
   float s = 0.f;
   for (int i = lane; i < parts; i += 64) s += partial[(int64_t)o * parts + i];
@@ -908,7 +978,7 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   }
   if (splits > 1) {
     const int64_t total = (int64_t)M * N;
-    int64_t blocks = std::min<int64_t>(ceil_div(total, 256), (int64_t)ctx->compute_units * 8);
+    int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
     LaunchScope scope(ctx, "splitk_reduce");
     hipLaunchKernelGGL((splitk_reduce_kernel<EP>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, splits, M, N, ep);
   }
@@ -1025,6 +1095,16 @@ int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const flo
 
 int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems) {
   const int M = g.kh * g.kw * g.cin, N = g.cout, K = g.n * g.ho * g.wo;
+  if (!(ws && small_parts(M, N, K, ctx->compute_units, ws_elems)) && WgradXLoader::ok(x, g) && FlatLoader<false>::ok(dy, 1, g.cout, N, K)) {
+    const int interior = g.pt == 0 && g.pl == 0 && (g.ho - 1) * g.sh + g.kh <= g.h && (g.wo - 1) * g.sw + g.kw <= g.w;
+    WgradXLoader al{x, g, M, interior};
+    FlatLoader<false> bl{dy, 1, g.cout, N};
+    Epilogue e;
+    e.out = dw;
+    e.ldo = g.cout;
+    StdEpilogue ep{e};
+    return launch_any<false>(ctx, "conv2d_filter_gradient", M, N, K, al, bl, ep, ws, ws_elems);
+  }
   ConvWgradA al{x, g, M};
   StridedLoader<false> bl{dy, 1, (int64_t)g.cout, N};
   Epilogue e;
