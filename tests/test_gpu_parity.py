@@ -44,6 +44,10 @@ def round_at(x, p):
     return np.rint(x * s) / s
 
 
+TOL_BF16 = 2e-3   # bf16 Dense mode: operands are rounded to bf16 on both sides; what is left is accumulation order
+                  # and the few activations whose float32 last bit flips their bf16 rounding
+
+
 class Harness:
     """Compiles a model on the GPU and holds its oracle twin."""
 
@@ -392,6 +396,90 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
         yb.free()
 
 
+@pytest.fixture(scope="module")
+def sweep_vectors():
+    """100 M parameters ~N(0, 0.02) and gradients ~N(0, 1e-3): the memory-bound sweep at its full size."""
+    rng = np.random.default_rng(20251125 + 5)
+    n = 100_000_000
+    return rng.standard_normal(n, dtype=f32) * f32(0.02), rng.standard_normal(n, dtype=f32) * f32(1e-3)
+
+
+@pytest.mark.parametrize("name", [n for n, _, _ in optimizer_pairs()])
+def test_full_config_optimizer_update_100m(S, ctx, sweep_vectors, name):
+    """One fused update over 100 M elements against the oracle on the same data."""
+    w0, g = sweep_vectors
+    oalg, desc = {n: (o, d) for n, o, d in optimizer_pairs()}[name]
+    states = oalg.init_state(w0.shape)
+    wb, gb = ctx.to_device(w0), ctx.to_device(g)
+    sb = [ctx.to_device(s) for s in states]
+    ctx.optimizer_update(desc, wb, gb, sb, 1)
+    delta, states = oalg.build(g, states, 1)
+    assert rel_err(wb.numpy(), w0 - delta) <= TOL_ELEMENTWISE
+    for s_gpu, s_ref in zip(sb, states):
+        assert rel_err(s_gpu.numpy(), s_ref) <= TOL_ELEMENTWISE
+    for b in [wb, gb] + sb:
+        b.free()
+
+
+def test_full_config_average_8x25m(S, ctx):
+    """Mean of 8 replicas of 25 M parameters: identical to the oracle's left-to-right sum, plus two facts that hold
+    at any size."""
+    rng = np.random.default_rng(20251125 + 7)
+    m = 25_000_000
+    reps = [rng.standard_normal(m, dtype=f32) * f32(0.02) for _ in range(8)]
+    bufs = [ctx.to_device(r) for r in reps]
+    out = ctx.alloc(m)
+    ctx.average(bufs, out)
+    got = out.numpy()
+    np.testing.assert_array_equal(got, O.average_uniform(reps))
+    ctx.average([bufs[0]] * 2, out)                      # the mean of two copies of a vector is that vector (x + x and /2 are exact)
+    np.testing.assert_array_equal(out.numpy(), reps[0])
+    ctx.average([bufs[0]] * 8, out)                      # with 8 copies the running sums 3x, 5x, ... round: equal to 1 ulp
+    assert rel_err(out.numpy(), reps[0]) <= TOL_ELEMENTWISE
+    ctx.average(bufs[::-1], out)                         # summation order only moves the last bits
+    assert rel_err(out.numpy(), got) <= TOL_ELEMENTWISE
+    for b in bufs + [out]:
+        b.free()
+
+
+def test_full_config_wide_mlp_bf16_one_step(S, ctx):
+    """4096 -> 4096 (ReLU) -> 4096 (ReLU) -> 1000 (Softmax), batch 8192, bf16 matrix cores: forward, loss and every
+    gradient of one step against the oracle that rounds the GEMM operands to bf16."""
+    from scanet3_amd import _lib as L
+    dims, batch = (4096, 4096, 4096, 1000), 8192
+    spec = [("dense", 4096, "relu"), ("dense", 4096, "relu"), ("dense", 1000, "softmax")]
+    rng = np.random.default_rng(20251125 + 6)
+    h = Harness(S, ctx, spec, "cce", (dims[0],), batch, flags=L.FLAG_GEMM_BF16)
+    om = O.Model(h.omodel.layers, O.LOSS_CCE, bf16_dense=True)
+    params = glorot_params(om, (batch, dims[0]), rng)
+    x = rng.standard_normal((batch, dims[0]), dtype=f32)
+    y = one_hot(rng, batch, dims[-1])
+    h.rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    oloss, ograds = om.grad(x, y, params)
+    gloss = h.rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_BF16 * max(1.0, abs(float(oloss)))
+    ggrads = h.rep.get_grads()
+    # A different summation order inside a GEMM moves some activations across a bf16 rounding boundary or across
+    # zero (the ReLU mask), and at this size those few flips dominate the difference.  The yardstick is therefore the
+    # oracle against itself with the first layer's reduction index permuted (the same sums in another order): the
+    # GPU may differ from the oracle by at most 3 times what the oracle differs from itself.
+    perm = rng.permutation(dims[0])
+    p2 = dict(params)
+    p2["0/weights"] = params["0/weights"][perm]
+    _, g2 = om.grad(x[:, perm], y, p2)
+    g2["0/weights"] = g2["0/weights"][np.argsort(perm)]
+    for p in ograds:
+        noise = rel_err(g2[p], ograds[p])
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_BF16, 3 * noise), (p, noise)
+    pred = h.rep.forward(xb)
+    np.testing.assert_allclose(pred.sum(axis=1), 1.0, rtol=0, atol=1e-4)     # rows of a softmax
+    assert rel_err(pred, om.forward(x, params)) <= TOL_BF16
+    h.close()
+    xb.free()
+    yb.free()
+
+
 # ----------------------------------------------------------------------------- epoch loop, averaging, accuracy
 def test_train_epoch_semantics_and_replica_average(S, ctx, linear_function):
     X, Y = linear_function
@@ -518,8 +606,6 @@ def test_error_paths(S, ctx):
 
 
 # ----------------------------------------------------------------------------- bf16 Dense mode (no counterpart in the reference)
-TOL_BF16 = 2e-3   # operands are rounded to bf16 on both sides; what is left is accumulation order and the few
-                  # activations whose float32 last bit flips their bf16 rounding
 
 
 @pytest.mark.parametrize("dims,batch", [((64, 4096, 64, 8), 4096), ((256, 512, 104), 512), ((1000, 264, 40), 136)])
