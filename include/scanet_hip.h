@@ -31,6 +31,13 @@
 #include <stddef.h>
 #include <stdint.h>
 
+/* Every function below is exported; nothing else in the library is. */
+#if defined(__GNUC__) || defined(__clang__)
+#define SN_API __attribute__((visibility("default")))
+#else
+#define SN_API
+#endif
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -120,32 +127,32 @@ typedef struct sn_param_info {
 /* Replaces `new Session()` = Graph + TF Session (core/Session.scala:57-63).
  * `stream` is a hipStream_t to issue all work on, or NULL to let the context
  * create (and own) one. */
-int sn_ctx_create(int device, void* stream, sn_ctx** out);
+SN_API int sn_ctx_create(int device, void* stream, sn_ctx** out);
 /* Replaces Session.close (core/Session.scala:106). Waits for outstanding work. */
-int sn_ctx_destroy(sn_ctx* ctx);
+SN_API int sn_ctx_destroy(sn_ctx* ctx);
 /* Message of the calling thread's most recent failing call (never NULL). */
-const char* sn_last_error(void);
+SN_API const char* sn_last_error(void);
 /* Blocks until everything issued on the context's stream has finished. */
-int sn_sync(sn_ctx* ctx);
+SN_API int sn_sync(sn_ctx* ctx);
 /* Name, HBM bytes and compute-unit count of the context's device
  * (reference: core/Devices.scala:23-37 lists TF devices). */
-int sn_device_info(sn_ctx* ctx, char* name, int name_cap, int64_t* hbm_bytes, int32_t* compute_units);
+SN_API int sn_device_info(sn_ctx* ctx, char* name, int name_cap, int64_t* hbm_bytes, int32_t* compute_units);
 
 /* ---------------------------------------------------------------- tensors / memory */
 
 /* Replaces TF_AllocateTensor / TF_DeleteTensor (native/RawTensors.scala:81-88,106-115)
  * for device-resident tensors. */
-int sn_buffer_alloc(sn_ctx* ctx, size_t bytes, void** out_dev);
-int sn_buffer_free(sn_ctx* ctx, void* dev);
+SN_API int sn_buffer_alloc(sn_ctx* ctx, size_t bytes, void** out_dev);
+SN_API int sn_buffer_free(sn_ctx* ctx, void* dev);
 /* Pinned host memory a JVM can wrap as a read-only DirectBuffer
  * (native/RawTensors.scala:24-30, core/TensorCodec.scala:12-22). */
-int sn_host_alloc(sn_ctx* ctx, size_t bytes, void** out_host);
-int sn_host_free(sn_ctx* ctx, void* host);
+SN_API int sn_host_alloc(sn_ctx* ctx, size_t bytes, void** out_host);
+SN_API int sn_host_free(sn_ctx* ctx, void* host);
 /* Replaces the feed / fetch halves of Session.Runner (core/Session.scala:83-95).
  * h2d is asynchronous when src is pinned; d2h returns after the data has arrived. */
-int sn_copy_h2d(sn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
-int sn_copy_d2h(sn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
-int sn_fill(sn_ctx* ctx, float* dst_dev, float value, int64_t n);
+SN_API int sn_copy_h2d(sn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+SN_API int sn_copy_d2h(sn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+SN_API int sn_fill(sn_ctx* ctx, float* dst_dev, float value, int64_t n);
 
 /* ---------------------------------------------------------------- model = compiled step */
 
@@ -153,16 +160,16 @@ int sn_fill(sn_ctx* ctx, float* dst_dev, float value, int64_t n);
  * (models/Model.scala:84-119, optimizers/Optimizer.scala:163-194, core/TF.scala:391-438).
  * `input_dims` is the shape of ONE sample (e.g. {784}, {28,28,1}, {64,32}); `batch`
  * is the largest number of rows any call will pass. */
-int sn_model_create(sn_ctx* ctx, const sn_layer_desc* layers, int32_t n_layers, int32_t loss,
+SN_API int sn_model_create(sn_ctx* ctx, const sn_layer_desc* layers, int32_t n_layers, int32_t loss,
                     const int64_t* input_dims, int32_t input_rank, int32_t batch, uint32_t flags,
                     sn_model** out);
-int sn_model_destroy(sn_model* model);
+SN_API int sn_model_destroy(sn_model* model);
 /* `model.params(input)` restricted to trainable weights (models/Model.scala:18;
  * optimizers/Optimizer.scala:117-122), in flat-buffer order. */
-int sn_model_param_count(sn_model* model, int32_t* n_tensors, int64_t* flat_elems);
-int sn_model_param_info(sn_model* model, int32_t index, sn_param_info* out);
+SN_API int sn_model_param_count(sn_model* model, int32_t* n_tensors, int64_t* flat_elems);
+SN_API int sn_model_param_info(sn_model* model, int32_t index, sn_param_info* out);
 /* `model.outputShape(input)` for one sample (models/Model.scala:41). */
-int sn_model_output_shape(sn_model* model, int32_t* rank, int64_t* dims);
+SN_API int sn_model_output_shape(sn_model* model, int32_t* rank, int64_t* dims);
 
 /* ---------------------------------------------------------------- replica = params + optimizer state */
 
@@ -170,65 +177,65 @@ int sn_model_output_shape(sn_model* model, int32_t* rank, int64_t* dims);
  * buffers that optimizeOnPartition threads through its loop
  * (optimizers/Optimizer.scala:117-131). Weights start at zero, optimizer state at
  * `opt->init_acc` (ParamDef.initialize). `opt` may be NULL for inference only. */
-int sn_replica_create(sn_model* model, const sn_optimizer_desc* opt, sn_replica** out);
-int sn_replica_destroy(sn_replica* rep);
+SN_API int sn_replica_create(sn_model* model, const sn_optimizer_desc* opt, sn_replica** out);
+SN_API int sn_replica_destroy(sn_replica* rep);
 /* `.initParams(Params)` / reading `TrainedModel.params` (optimizers/Optimizer.scala:276-277,103). */
-int sn_params_set(sn_replica* rep, int32_t index, const float* src_host, int64_t n);
-int sn_params_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
+SN_API int sn_params_set(sn_replica* rep, int32_t index, const float* src_host, int64_t n);
+SN_API int sn_params_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
 /* Optimizer state tensor `<path>/<state name>` (optimizers/Optimizer.scala:118-121); slot order is
  * the order of the algorithm's `params` (e.g. Adam: 0 momentum, 1 velocity). */
-int sn_optstate_set(sn_replica* rep, int32_t index, int32_t slot, const float* src_host, int64_t n);
-int sn_optstate_get(sn_replica* rep, int32_t index, int32_t slot, float* dst_host, int64_t n);
+SN_API int sn_optstate_set(sn_replica* rep, int32_t index, int32_t slot, const float* src_host, int64_t n);
+SN_API int sn_optstate_get(sn_replica* rep, int32_t index, int32_t slot, float* dst_host, int64_t n);
 /* Gradient of the last sn_step / sn_grad for one tensor (`LossModel.grad`, models/Model.scala:107-111). */
-int sn_grads_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
+SN_API int sn_grads_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n);
 /* Device views of the flat buffers: slot -2 weights, -1 gradients, 0.. optimizer state tensors. */
-int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n);
+SN_API int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n);
 
 /* One call of the compiled backprop function (optimizers/Optimizer.scala:142-143, 169-194):
  * forward, loss, gradients of every weight, optimizer update w' = w - delta with iteration
  * number `iter` (1-based). `rows` <= batch. If `loss_host` is not NULL the loss of this batch
  * (before the update) is written there and the call waits for the device. */
-int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host);
+SN_API int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host);
 /* `LossModel.grad` (models/Model.scala:107-111): gradients only, no update. */
-int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
+SN_API int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
 /* `model.result` (models/Model.scala:35-36): out_dev receives rows x output elements. */
-int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
+SN_API int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
 /* `LossModel.loss` (models/Model.scala:101-102). */
-int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
+SN_API int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
 /* Per-batch body of `estimators.accuracy` (estimators/package.scala:28-32): rows whose every
  * rounded (half to even) output equals the label. */
-int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int64_t* count_host);
+SN_API int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int64_t* count_host);
 /* `optimizeOnPartition` (optimizers/Optimizer.scala:106-161) over a device-resident partition of
  * `total_rows` samples: every full batch in order with iter = global_iter + i + 1, partial batch
  * skipped (optimizers/Iterators.scala:90), then the loss of the last batch under the updated
  * weights. Fails with SN_E_INVALID when the partition holds no full batch. */
-int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch,
+SN_API int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch,
                    int32_t global_iter, int32_t* iterations_host, float* loss_host);
 
 /* `aggregateParams` (optimizers/Optimizer.scala:196-230) for K replicas of one model: weights and
  * every optimizer-state tensor become the uniform mean AddN(..)/K (models/Aggregation.scala:16-19)
  * and are written back to all K replicas (the next epoch's broadcast, Optimizer.scala:72-73). */
-int sn_replicas_average(sn_replica* const* reps, int32_t k);
+SN_API int sn_replicas_average(sn_replica* const* reps, int32_t k);
 
 /* ---------------------------------------------------------------- flat kernels (the memory-bound pair) */
 
 /* One fused `Algorithm.build` + `w - delta` over a flat vector (optimizers/Optimizer.scala:181-188):
  * w[i], state*[i] updated in place from g[i]. Unused state pointers may be NULL. */
-int sn_optimizer_update(sn_ctx* ctx, const sn_optimizer_desc* opt, float* w_dev, const float* g_dev,
+SN_API int sn_optimizer_update(sn_ctx* ctx, const sn_optimizer_desc* opt, float* w_dev, const float* g_dev,
                         float* s0_dev, float* s1_dev, float* s2_dev, int64_t n, int32_t iter);
 /* `Aggregation.Avg` over k inputs (models/Aggregation.scala:16-19): out = (in[0] + .. + in[k-1]) / k,
  * accumulated left to right. `inputs_host` is a host array of k device pointers; out may alias in[0]. */
-int sn_average(sn_ctx* ctx, const float* const* inputs_host, int32_t k, int64_t n, float* out_dev);
+SN_API int sn_average(sn_ctx* ctx, const float* const* inputs_host, int32_t k, int64_t n, float* out_dev);
 
 /* ---------------------------------------------------------------- per-kernel timing */
 
 /* When enabled every kernel launch of the context is bracketed by HIP events on the context's
  * stream (the reference only has wall-clock per epoch, optimizers/Optimizer.scala:74,87-89). */
-int sn_profile_enable(sn_ctx* ctx, int32_t on);
-int sn_profile_reset(sn_ctx* ctx);
+SN_API int sn_profile_enable(sn_ctx* ctx, int32_t on);
+SN_API int sn_profile_reset(sn_ctx* ctx);
 /* Number of distinct kernel names seen since the last reset (waits for the stream). */
-int sn_profile_count(sn_ctx* ctx, int32_t* n);
-int sn_profile_get(sn_ctx* ctx, int32_t index, char* name, int32_t name_cap, double* total_ms, int64_t* launches);
+SN_API int sn_profile_count(sn_ctx* ctx, int32_t* n);
+SN_API int sn_profile_get(sn_ctx* ctx, int32_t index, char* name, int32_t name_cap, double* total_ms, int64_t* launches);
 
 #ifdef __cplusplus
 }

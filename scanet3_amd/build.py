@@ -21,7 +21,7 @@ SOURCES = ["runtime.hip", "optim_kernels.hip", "elementwise_kernels.hip", "gemm_
 # -ffp-contract=off: one rounding per reference op (TensorFlow evaluates Mul and Add separately).
 # -packed-fp32-ops is switched off: some packed fp32 forms have produced wrong values on this hardware.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
