@@ -174,9 +174,10 @@ struct EpilogueBf16 {
 int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep);
 // bf16 copies out[rows,cols] and out_t[cols,rows] of an fp32 matrix; with y != null the activation gradient
 // act'(y) * src is what gets cast (and is written to dz in fp32 when dz != null).  col_partials (optional,
-// [ceil(rows/64), cols]) receives the column sums of every 64-row block of the fp32 values.
+// [ceil(rows/64), cols]) receives the column sums of every 64-row block of the fp32 values.  y_bf: the layer output
+// as bf16 [rows, cols], used in place of y when y is null (enough for ReLU, whose gradient only needs the sign).
 int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
-                          int act, float act_param, float* dz, float* col_partials = nullptr);
+                          int act, float act_param, float* dz, float* col_partials = nullptr, const void* y_bf = nullptr);
 
 struct ConvGeom {
   int n, h, w, cin;      // input

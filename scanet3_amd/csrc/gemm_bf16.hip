@@ -348,8 +348,8 @@ int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt,
 // the activation gradient act'(y) * src, which is also written back to dz (fp32) when dz != null.
 __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __restrict__ src, int64_t ld, int rows, int cols,
                                                               bf16* __restrict__ out, bf16* __restrict__ out_t,
-                                                              const float* __restrict__ y, int act, float act_param,
-                                                              float* __restrict__ dz, float* __restrict__ col_partials) {
+                                                              const float* __restrict__ y, const bf16* __restrict__ y_bf, int act,
+                                                              float act_param, float* __restrict__ dz, float* __restrict__ col_partials) {
   // 64x64 tile; a thread handles 4 consecutive columns of 4 rows (float4 in, 8-byte bf16x4 out), and on the
   // transposed side 4 consecutive rows of one column.  cols and rows are multiples of 4 (checked by the caller).
   __shared__ bf16 tile[64][68];
@@ -363,8 +363,14 @@ __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __rest
     f4 v = {0.f, 0.f, 0.f, 0.f};
     if (r < rows && c < cols) {
       v = *(const f4*)(src + (int64_t)r * ld + c);
-      if (y) {
-        const f4 yy = *(const f4*)(y + (int64_t)r * ld + c);
+      if (y || y_bf) {
+        f4 yy;
+        if (y) yy = *(const f4*)(y + (int64_t)r * ld + c);
+        else {  // the layer's output only exists as the bf16 copy its successor reads (pitch = cols)
+          const bf16x4 yb = *(const bf16x4*)(y_bf + (int64_t)r * cols + c);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) yy[e] = (float)yb[e];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = bf_act_grad(act, yy[e], v[e], act_param);
         if (dz) *(f4*)(dz + (int64_t)r * ld + c) = v;
@@ -404,12 +410,12 @@ __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __rest
 }
 
 int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
-                          int act, float act_param, float* dz, float* col_partials) {
+                          int act, float act_param, float* dz, float* col_partials, const void* y_bf) {
   if (rows <= 0 || cols <= 0) return SN_OK;
   SN_REQUIRE(rows % 4 == 0 && cols % 4 == 0 && ld % 4 == 0, "cast_bf16: rows, cols and pitch must be multiples of 4");
-  LaunchScope scope(ctx, y ? "activation_backward_cast_bf16" : "cast_bf16");
+  LaunchScope scope(ctx, (y || y_bf) ? "activation_backward_cast_bf16" : "cast_bf16");
   hipLaunchKernelGGL(cast_transpose_kernel, dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256), 0, ctx->stream,
-                     src, ld, rows, cols, (bf16*)out, (bf16*)out_t, y, act, act_param, dz, col_partials);
+                     src, ld, rows, cols, (bf16*)out, (bf16*)out_t, y, (const bf16*)y_bf, act, act_param, dz, col_partials);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

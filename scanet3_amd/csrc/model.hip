@@ -302,6 +302,16 @@ static int dev_alloc(sn_replica* r, T** out, int64_t elems) {
   return SN_OK;
 }
 
+static bool dense_bf16_fast(const sn_model* m, const struct Op& op);
+// A hidden Dense layer of the bf16 path whose successor is another one hands its output over as bf16 copies; its
+// fp32 output has no other reader when the activation's gradient needs only the sign of the output (ReLU) or nothing.
+static bool hidden_f32_not_needed(const sn_model* m, size_t i) {
+  if (i + 1 >= m->ops.size()) return false;
+  const Op& op = m->ops[i];
+  return dense_bf16_fast(m, op) && dense_bf16_fast(m, m->ops[i + 1]) && (op.act == SN_ACT_RELU || op.act == SN_ACT_IDENTITY) &&
+         m->batch % 8 == 0;
+}
+
 // The 256x256 bf16 kernel needs 16-byte chunks of 8 k-values in every operand row.
 static bool dense_bf16_fast(const sn_model* m, const Op& op) {
   return (m->flags & SN_FLAG_GEMM_BF16) && op.kind == OP_DENSE && op.in_elems % 8 == 0 && op.out_elems % 8 == 0 && m->batch % 8 == 0;
@@ -423,6 +433,7 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
             eb.out_bf_t = r->bf_xt[i + 1];
             eb.ld_t = rows;
             bf_ready[i + 1] = true;
+            if (hidden_f32_not_needed(m, i)) eb.e.out = nullptr;  // the next layer and the backward pass read the bf16 copies
           }
           SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_x[i], in_f, r->bf_wt[i], in_f, rows, out_f, in_f, eb));
         } else {
@@ -512,9 +523,11 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         if (dense_bf16_fast(m, op) && rows % 8 == 0) {
           // one pass: dZ = act'(Y) * dY in fp32 (bias gradient) and as bf16 in both orientations
           // (the fp32 dZ itself is not kept: its only other reader would be the bias gradient, summed here per 64-row block)
+          const bool y_from_bf = hidden_f32_not_needed(m, (size_t)i);
           SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
-                                       op.act != SN_ACT_IDENTITY ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
-                                       op.b >= 0 ? r->bf_colp : nullptr));
+                                       op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
+                                       op.b >= 0 ? r->bf_colp : nullptr,
+                                       op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
           if (op.b >= 0)
             SN_TRY(launch_col_sum(ctx, r->bf_colp, out_f, param_ptr(r, r->g, op.b), ceil_div(rows, 64), out_f, r->ws, m->workspace_elems));
           EpilogueBf16 ew;
