@@ -676,7 +676,7 @@ struct LdsElem<true> { typedef __bf16 type; };
 // VEC = 4: every tile copy moves 4 values per load along the operand's contiguous index (the host checks
 // vec4_ok() of both loaders); VEC = 1 is the general element-wise form.
 template <int BM, int BN, bool BF16, int VEC, class AL, class BL, class EP>
-__global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int k_per_split, AL al, BL bl, EP ep, float* ws) {
+__global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int k_per_split, AL al, BL bl, EP ep, float* ws, int splits) {
   typedef typename LdsElem<BF16>::type lds_t;
   // the 4 waves form a 2x2 grid over the tile, or 4x1 when the tile is a single MFMA block wide
   constexpr int WAVES_N = BN >= 64 ? 2 : 1, WAVES_M = 4 / WAVES_N;
@@ -690,8 +690,21 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const bool b_on = tid < B_ACTIVE;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const int k_begin = blockIdx.z * k_per_split;
+  // Split-K launches use a flat grid: consecutive workgroup ids land on different XCDs (8, each with its own L2),
+  // so XCD x takes the splits x, x+8, ... and walks all output tiles of one split before the next: the tiles
+  // that re-read the same K range of A and B then share one L2 instead of fetching it once per XCD.
+  int bm = blockIdx.y, bn = blockIdx.x, bz = blockIdx.z;
+  if (splits > 1) {
+    const int tiles_n = (N + BN - 1) / BN, tiles_mn = tiles_n * ((M + BM - 1) / BM);
+    const int slot = blockIdx.x >> 3;
+    bz = (blockIdx.x & 7) + 8 * (slot / tiles_mn);
+    if (bz >= splits) return;
+    const int tile = slot % tiles_mn;
+    bm = tile / tiles_n;
+    bn = tile - bm * tiles_n;
+  }
+  const int m0 = bm * BM, n0 = bn * BN;
+  const int k_begin = bz * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
 
   typename AL::Cursor ca[EA];
@@ -809,7 +822,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm + i * 32 + (v >> 2) * 8 + lhi * 4 + (v & 3);
         if (row >= M) continue;
-        if (ws) ws[((int64_t)blockIdx.z * M + row) * N + col] = acc[i][j][v];
+        if (ws) ws[((int64_t)bz * M + row) * N + col] = acc[i][j][v];
         else ep.store(row, col, acc[i][j][v]);
       }
     }
@@ -937,14 +950,15 @@ static int small_parts(int m, int n, int k, int cu, int64_t ws_elems) {
 }
 
 // ============================================================================ dispatch
+constexpr int SPLIT_WG_PER_CU = 8, SPLIT_MAX = 256;
 int64_t gemm_workspace_elems(int m, int n, int k, int cu) {
   // room for the partial sums of the small-output kernel, or for the largest split count launch_tiles may pick
   const int parts = small_parts(m, n, k, cu, -1);
   if (parts) return (int64_t)parts * m * n;
   const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
   if (tiles >= cu || k <= 256) return 0;
-  int64_t splits = std::min<int64_t>(ceil_div((int64_t)2 * cu, tiles), std::max<int64_t>(1, k / 128));
-  splits = std::min<int64_t>(splits, 64);
+  int64_t splits = std::min<int64_t>(ceil_div((int64_t)SPLIT_WG_PER_CU * cu, tiles), std::max<int64_t>(1, k / 128));
+  splits = std::min<int64_t>(splits, SPLIT_MAX);
   return splits * (int64_t)m * n;
 }
 
@@ -954,26 +968,29 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   const int64_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
   int splits = 1;
   if (tiles * 2 <= ctx->compute_units && K >= 512 && ws) {  // a split costs a second pass over M*N*splits floats
-    int64_t s = std::min<int64_t>(ceil_div((int64_t)2 * ctx->compute_units, tiles), std::max<int64_t>(1, K / 128));
-    s = std::min<int64_t>(s, 64);
+    // These kernels are a chain of load, stage, multiply per K tile: what hides its latency is other workgroups on
+    // the same CU, so aim for 8 per CU (measured: 2 per CU runs the LeNet filter gradient in 52 us, 8 per CU in 31).
+    int64_t s = std::min<int64_t>(ceil_div((int64_t)SPLIT_WG_PER_CU * ctx->compute_units, tiles), std::max<int64_t>(1, K / 128));
+    s = std::min<int64_t>(s, SPLIT_MAX);
     s = std::min<int64_t>(s, ws_elems / ((int64_t)M * N));
     splits = (int)std::max<int64_t>(1, s);
   }
   int k_per_split = (int)align_up(ceil_div(K, splits), BK);
   splits = (int)ceil_div(K, k_per_split);
-  const dim3 grid((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), (unsigned)splits);
+  const dim3 grid = splits > 1 ? dim3((unsigned)(8 * ceil_div(N, BN) * ceil_div(M, BM) * ceil_div(splits, 8)))
+                               : dim3((unsigned)ceil_div(N, BN), (unsigned)ceil_div(M, BM), 1);
   {
     LaunchScope scope(ctx, name, M, N, K);
     if constexpr (AL::FAST && BL::FAST) {  // the caller has checked what 16-byte loads need
       hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 4, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
-                         splits > 1 ? ws : nullptr);
+                         splits > 1 ? ws : nullptr, splits);
     } else {
       if (al.vec4_ok(K) && bl.vec4_ok(K))
         hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 4, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
-                           splits > 1 ? ws : nullptr);
+                           splits > 1 ? ws : nullptr, splits);
       else
         hipLaunchKernelGGL((gemm_kernel<BM, BN, BF16, 1, AL, BL, EP>), grid, dim3(THREADS), 0, ctx->stream, M, N, K, k_per_split, al, bl, ep,
-                           splits > 1 ? ws : nullptr);
+                           splits > 1 ? ws : nullptr, splits);
     }
   }
   if (splits > 1) {
@@ -1006,8 +1023,8 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
    }
   }
   bool big_m = M > 64, big_n = N > 64;
-  // 128-wide tiles only when they still cover every CU at least once; otherwise more, smaller workgroups
-  if (ceil_div(M, big_m ? 128 : 64) * ceil_div(N, big_n ? 128 : 64) < ctx->compute_units) big_m = big_n = false;
+  // 128-wide tiles only when they still cover every CU at least twice; otherwise more, smaller workgroups
+  if (ceil_div(M, big_m ? 128 : 64) * ceil_div(N, big_n ? 128 : 64) < (int64_t)2 * ctx->compute_units) big_m = big_n = false;
   if (N <= 32 && M > 64) return launch_tiles<128, 32, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_m && big_n) return launch_tiles<128, 128, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
   if (big_m) return launch_tiles<128, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
