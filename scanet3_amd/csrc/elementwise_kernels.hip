@@ -302,14 +302,27 @@ int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, fl
 // ---------------------------------------------------------------------------- column sums (bias gradient)
 // out[c] = sum_r dy[r, c] (Plus's gradient: Sum over the broadcast axes, AllKernels.scala:21-31).
 // A block owns 64 columns; its 4 waves stride over the rows; partial sums meet in LDS.
+// Rows r, r+4, ... below r1 of column c, added in that order; 8 loads are in flight at a time (one load per
+// loop trip would make the loop as slow as 8 memory latencies per 8 rows).
+__device__ __forceinline__ float sum_every_4th_row(const float* __restrict__ dy, int64_t ld, int c, int64_t r, int64_t r1) {
+  float s = 0.f;
+  for (; r + 28 < r1; r += 32) {
+    float a[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = dy[(r + 4 * u) * ld + c];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += a[u];
+  }
+  for (; r < r1; r += 4) s += dy[r * ld + c];
+  return s;
+}
+
 __global__ __launch_bounds__(256) void col_sum_kernel(const float* __restrict__ dy, int64_t ld, float* __restrict__ out, int64_t rows,
                                                        int cols) {
   __shared__ float smem[4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = blockIdx.x * 64 + lane;
-  float s = 0.f;
-  if (c < cols)
-    for (int64_t r = wave; r < rows; r += 4) s += dy[r * ld + c];
+  const float s = c < cols ? sum_every_4th_row(dy, ld, c, wave, rows) : 0.f;
   smem[wave][lane] = s;
   __syncthreads();
   if (wave == 0 && c < cols) out[c] = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];
@@ -324,9 +337,7 @@ __global__ __launch_bounds__(256) void col_sum_split_kernel(const float* __restr
   const int c = blockIdx.x * 64 + lane;
   const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
   const int64_t r1 = r0 + rows_per_slice < rows ? r0 + rows_per_slice : rows;
-  float s = 0.f;
-  if (c < cols)
-    for (int64_t r = r0 + wave; r < r1; r += 4) s += dy[r * ld + c];
+  const float s = c < cols ? sum_every_4th_row(dy, ld, c, r0 + wave, r1) : 0.f;
   smem[wave][lane] = s;
   __syncthreads();
   if (wave == 0 && c < cols) part[(int64_t)blockIdx.y * cols + c] = ((smem[0][lane] + smem[1][lane]) + smem[2][lane]) + smem[3][lane];

@@ -837,8 +837,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   for (int64_t base = (int64_t)blockIdx.x * 32; base < total; base += (int64_t)gridDim.x * 32) {
     const int64_t i = base + j;
     float s = 0.f;
-    if (i < total)
-      for (int z = g; z < splits; z += 8) s += ws[(int64_t)z * total + i];
+    if (i < total) {
+      int z = g;
+      for (; z + 24 < splits; z += 32) {  // 4 loads in flight, added in split order
+        float a[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a[u] = ws[(int64_t)(z + 8 * u) * total + i];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s += a[u];
+      }
+      for (; z < splits; z += 8) s += ws[(int64_t)z * total + i];
+    }
     __shared__ float part[8][32];
     part[g][j] = s;
     __syncthreads();
