@@ -864,7 +864,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // classes): too little output for MFMA tiles to occupy the chip. Workgroups stride over 64-long slices of K,
 // stage them in LDS, keep up to four outputs per thread in registers and leave one partial sum per workgroup
 // and output; a second kernel adds the partials in a fixed order.
-constexpr int SMALL_SLICE = 64, SMALL_MAX_OUT = 1024, SMALL_MAX_DIM = 128, SMALL_MIN_K = 2048;
+constexpr int SMALL_SLICE = 64, SMALL_MAX_OUT = 512, SMALL_MAX_DIM = 128, SMALL_MIN_K = 2048;
 
 template <class AL, class BL>
 __global__ __launch_bounds__(256) void gemm_small_kernel(int M, int N, int K, AL al, BL bl, float* __restrict__ partial) {
@@ -1089,8 +1089,65 @@ int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* works
 }
 
 // ---------------------------------------------------------------------------- Conv2D
+// First-layer convolutions (1 to 4 input channels): K = kh*kw*cin is a few dozen, far too short for MFMA tiles
+// to pay for their set-up, and the layer is bound by writing its output.  Direct form: the filter sits in LDS,
+// 8 neighbouring lanes share one output pixel and own 4 output channels each (so a pixel's channels leave as
+// one contiguous run), every lane gathers the pixel's K inputs itself (they stay in L1).
+constexpr int DIRECT_MAX_K = 64;
+__global__ __launch_bounds__(256) void conv_direct_fwd_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ w,
+                                                               Epilogue e, int pixels) {
+  extern __shared__ __attribute__((aligned(16))) float wl[];  // [K][cout]
+  const int K = g.kh * g.kw * g.cin;
+  for (int i = threadIdx.x; i < K * g.cout; i += 256) wl[i] = w[i];
+  __syncthreads();
+  const int quads = g.cout / 4;  // channel quads per pixel
+  const int64_t total = (int64_t)pixels * quads;
+  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
+    const int cq = (int)(t % quads);
+    const int p = (int)(t / quads);
+    const int ow = p % g.wo;
+    const int t2 = p / g.wo;
+    const int oh = t2 % g.ho;
+    const int b = t2 / g.ho;
+    const int iy0 = oh * g.sh - g.pt, ix0 = ow * g.sw - g.pl;
+    const float* img = x + (int64_t)b * g.h * g.w * g.cin;
+    f4v acc = {0.f, 0.f, 0.f, 0.f};
+    int k = 0;
+    for (int r = 0; r < g.kh; ++r) {
+      const int iy = iy0 + r;
+      for (int q = 0; q < g.kw; ++q) {
+        const int ix = ix0 + q;
+        const bool in = (unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w;
+        for (int ci = 0; ci < g.cin; ++ci, ++k) {
+          const float xv = in ? img[(iy * g.w + ix) * g.cin + ci] : 0.f;
+          const f4v wv = *(const f4v*)(wl + k * g.cout + cq * 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(xv, wv[i], acc[i]);  // fused like the matrix cores; k in (r, q, ci) order
+        }
+      }
+    }
+    const int col = cq * 4;
+    f4v out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = acc[i];
+      if (e.bias) v = v + e.bias[col + i];
+      out[i] = ep_act(e.act, v, e.act_param);
+    }
+    *(f4v*)(e.out + (int64_t)p * e.ldo + col) = out;
+  }
+}
+
 int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e, float* ws, int64_t ws_elems) {
   const int M = g.n * g.ho * g.wo, N = g.cout, K = g.kh * g.kw * g.cin;
+  if (g.cin <= 4 && K <= DIRECT_MAX_K && N % 4 == 0 && (size_t)K * N * sizeof(float) <= 48 * 1024 && e.ldo % 4 == 0 && aligned16(e.out) && M > 0) {
+    const int64_t total = (int64_t)M * (N / 4);
+    const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(total, 256), (int64_t)ctx->compute_units * 32);
+    LaunchScope scope(ctx, "conv2d_forward_direct", M, N, K);
+    hipLaunchKernelGGL(conv_direct_fwd_kernel, dim3(blocks), dim3(256), (size_t)K * N * sizeof(float), ctx->stream, g, x, w, e, M);
+    SN_HIP(hipGetLastError());
+    return SN_OK;
+  }
   StdEpilogue ep{e};
   if (TapLoader::ok(x, g.n, g.h, g.w, g.cin, g.kh, g.kw) && FlatLoader<false>::ok(w, 1, g.cout, N, K)) {
     TapLoader al{x, M, g.ho, g.wo, g.sh, g.sw, -g.pt, -g.pl, 1, 1, g.h, g.w, g.cin, g.kh, g.kw};
