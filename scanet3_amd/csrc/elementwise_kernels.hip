@@ -539,7 +539,8 @@ int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int 
 template <int V, typename I>
 __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
                                                            float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo,
-                                                           int kh, int kw, int sh, int sw, int pt, int pl) {
+                                                           int kh, int kw, int sh, int sw, int pt, int pl,
+                                                           const float* __restrict__ y_in, int act, float act_param) {
   const I cv = (I)(c / V);
   const I total = (I)n * h * w * cv;
   const I stride = (I)gridDim.x * blockDim.x;
@@ -579,21 +580,32 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restric
         }
       }
     }
+    if (y_in) {  // the pooled tensor is the output y of a layer with an activation: hand back act'(y) * gradient
+      if constexpr (V == 4) {
+        const float4 yv = *(const float4*)(y_in + i * 4);
+        s[0] = act_bwd(act, yv.x, s[0], act_param);
+        s[1] = act_bwd(act, yv.y, s[1], act_param);
+        s[2] = act_bwd(act, yv.z, s[2], act_param);
+        s[3] = act_bwd(act, yv.w, s[3], act_param);
+      } else {
+        s[0] = act_bwd(act, y_in[i], s[0], act_param);
+      }
+    }
     if constexpr (V == 4) *(float4*)(dx + i * 4) = make_float4(s[0], s[1], s[2], s[3]);
     else dx[i] = s[0];
   }
 }
 
 int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho, int wo,
-                       int kh, int kw, int sh, int sw, int pt, int pl) {
+                       int kh, int kw, int sh, int sw, int pt, int pl, const float* y_in, int act, float act_param) {
   const int64_t total = (int64_t)n * h * w * c;
   if (total <= 0) return SN_OK;
   const bool small = total < (1ll << 31) && (int64_t)n * ho * wo * c < (1ll << 31);
-  const bool v4 = pool_vec4(dy, dx, arg, c);
+  const bool v4 = pool_vec4(dy, dx, arg, c) && (reinterpret_cast<uintptr_t>(y_in) & 15u) == 0;
   const dim3 grid(grid_for(ctx, v4 ? total / 4 : total, 256));
-  LaunchScope scope(ctx, "maxpool_backward");
+  LaunchScope scope(ctx, y_in ? "maxpool_activation_backward" : "maxpool_backward");
 #define SN_POOL_BWD(V, I) \
-  hipLaunchKernelGGL((maxpool_bwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl)
+  hipLaunchKernelGGL((maxpool_bwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl, y_in, act, act_param)
   if (v4 && small) SN_POOL_BWD(4, uint32_t);
   else if (v4) SN_POOL_BWD(4, uint64_t);
   else if (small) SN_POOL_BWD(1, uint32_t);

@@ -511,6 +511,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
   if (first < 0) first = (int)m->ops.size() - 1;
+  bool act_grad_done = false;  // the op above already applied this op's activation gradient
   for (int i = first; i >= 0; --i) {  // grad_buf[cur] holds d loss / d (output of op i)
     const Op& op = m->ops[i];
     const float* in = op_output(r, i - 1, x, rows);
@@ -562,7 +563,8 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         ConvGeom g{rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2], (int)op.out_dims[0], (int)op.out_dims[1],
                    (int)op.out_dims[2], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl};
         const int64_t n_out = (int64_t)rows * op.out_elems;
-        if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
+        if (op.act != SN_ACT_IDENTITY && !act_grad_done) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
+        act_grad_done = false;
         if (op.b >= 0)
           SN_TRY(launch_col_sum(ctx, dy, g.cout, param_ptr(r, r->g, op.b), (int64_t)rows * g.ho * g.wo, g.cout, r->ws, m->workspace_elems));
         SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems));
@@ -574,8 +576,13 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
       }
       case OP_POOL:
         if (need_dx) {
+          // a convolution with an activation right below: its activation gradient rides along (one pass less over the tensor)
+          const Op& below = m->ops[i - 1];
+          const bool fuse = below.kind == OP_CONV && below.act != SN_ACT_IDENTITY;
           SN_TRY(launch_maxpool_bwd(ctx, dy, r->arg[i], dx, rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
-                                    (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl));
+                                    (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl,
+                                    fuse ? r->act[i - 1] : nullptr, below.act, below.act_param));
+          act_grad_done = fuse;
           cur ^= 1;
         }
         break;
