@@ -98,7 +98,19 @@ def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy
         step()
     ctx.sync()
     dt = time.perf_counter() - t0
-    first_loss = None
+    # the same steps fed from pinned HOST memory (batch i+1 copied while batch i trains): the PCIe-inclusive rate
+    Xp, Yp = ctx.pinned_array(X.shape), ctx.pinned_array(Y.shape)
+    Xp[...] = X
+    Yp[...] = Y
+    epochs = max(1, steps // n_batches)
+    rep.train_epoch_host(Xp, Yp, batch, it, want_loss=False)
+    t1 = time.perf_counter()
+    for e in range(epochs):
+        rep.train_epoch_host(Xp, Yp, batch, it + (e + 1) * n_batches, want_loss=False)
+    dt_host = time.perf_counter() - t1
+    it += (epochs + 1) * n_batches
+    host_fed = {"samples_per_s": batch * n_batches * epochs / dt_host, "ms_per_step": 1e3 * dt_host / (epochs * n_batches),
+                "bytes_per_step": 4 * batch * (cm.in_elems + cm.out_elems)}
     # second, instrumented pass: per-kernel durations from HIP events on the library's stream
     ctx.profile_reset()
     ctx.profile(True)
@@ -116,7 +128,7 @@ def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy
     Xb.free()
     Yb.free()
     return {"workload": name, "samples_per_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps, "steps": steps,
-            "batch": batch, "params": n_params, "loss_after": last_loss, "kernels": kernels}
+            "batch": batch, "params": n_params, "loss_after": last_loss, "kernels": kernels, "host_fed": host_fed}
 
 
 def dominant_gemm_roofline(kernels, peak_tflops):
@@ -329,6 +341,7 @@ def main():
                      "dtype": "bf16" if args.workload == "wide_mlp" else "f32",
                      "config": {"workload": main_res["workload"], "batch": main_res["batch"], "params": main_res["params"]},
                      "roofline": dominant_gemm_roofline(main_res["kernels"], peak),
+                     "host_fed": main_res["host_fed"],
                      "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                              sorted(main_res["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:12]}})
     if not args.no_extras:
@@ -346,7 +359,7 @@ def main():
             else:
                 peak = PEAK_BF16_MFMA if which == "wide_mlp" else PEAK_FP32_MFMA
                 extras[which] = {"workload": r["workload"], "samples_per_s": r["samples_per_s"], "ms_per_step": r["ms_per_step"],
-                                 "steps": r["steps"], "loss_after": r["loss_after"],
+                                 "steps": r["steps"], "loss_after": r["loss_after"], "host_fed": r["host_fed"],
                                  "roofline": dominant_gemm_roofline(r["kernels"], peak),
                                  "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                                          sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}

@@ -212,6 +212,13 @@ SN_API int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_
 SN_API int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch,
                    int32_t global_iter, int32_t* iterations_host, float* loss_host);
 
+/* The same epoch over a partition in HOST memory (best allocated with sn_host_alloc: pinned memory makes the copies
+ * asynchronous): batch i+1 is copied to the device on a second stream while batch i trains.  Replaces the
+ * TensorIterator -> feed path of optimizeOnPartition (optimizers/Iterators.scala:39-83, Optimizer.scala:136-157).
+ * Results are those of sn_train_epoch on a device-resident copy of the same partition. */
+SN_API int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_host, int64_t total_rows, int32_t batch,
+                               int32_t global_iter, int32_t* iterations_host, float* loss_host);
+
 /* `aggregateParams` (optimizers/Optimizer.scala:196-230) for K replicas of one model: weights and
  * every optimizer-state tensor become the uniform mean AddN(..)/K (models/Aggregation.scala:16-19)
  * and are written back to all K replicas (the next epoch's broadcast, Optimizer.scala:72-73). */

@@ -89,6 +89,7 @@ SIGNATURES = {
     "sn_loss": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_count_correct": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64)]),
     "sn_train_epoch": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), _F]),
+    "sn_train_epoch_host": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), _F]),
     "sn_replicas_average": (C.c_int, [C.POINTER(_P), C.c_int32]),
     "sn_optimizer_update": (C.c_int, [_P, C.POINTER(OptimizerDesc), _P, _P, _P, _P, _P, C.c_int64, C.c_int32]),
     "sn_average": (C.c_int, [_P, C.POINTER(_P), C.c_int32, C.c_int64, _P]),
@@ -102,7 +103,7 @@ SIGNATURES = {
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            f"{LIB_PATH} is missing: build the HIP library first with `python -m scanet3_amd.build` "
+            f"{LIB_PATH} is missing: build the HIP library first with `python scanet3_amd/build.py` "
             "(there is no CPU fallback)")
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():

@@ -1,6 +1,6 @@
 """Builds libscanet_hip.so (gfx950 only) from csrc/*.hip with hipcc.
 
-    python -m scanet3_amd.build
+    python scanet3_amd/build.py
 
 The objects and the library stay in-tree next to this file; nothing is installed.
 """

@@ -27,9 +27,13 @@ class Context:
         check(lib.sn_ctx_create(device, C.c_void_p(stream) if stream else None, C.byref(h)))
         self.handle = h
         self.device = device
+        self._pinned = []
 
     def close(self):
         if self.handle:
+            for p in self._pinned:
+                check(lib.sn_host_free(self.handle, p))
+            self._pinned = []
             check(lib.sn_ctx_destroy(self.handle))
             self.handle = None
 
@@ -49,6 +53,15 @@ class Context:
         return name.value.decode(), hbm.value, cu.value
 
     # ---- memory -------------------------------------------------------------
+    def pinned_array(self, shape) -> np.ndarray:
+        """float32 numpy array over page-locked host memory (`sn_host_alloc`); freed when the context closes."""
+        n = int(np.prod(shape))
+        p = C.c_void_p()
+        check(lib.sn_host_alloc(self.handle, max(n, 1) * 4, C.byref(p)))
+        self._pinned.append(p)
+        buf = (C.c_float * max(n, 1)).from_address(p.value)
+        return np.frombuffer(buf, dtype=np.float32, count=n).reshape(shape)
+
     def alloc(self, n_floats: int) -> "DeviceBuffer":
         return DeviceBuffer(self, int(n_floats))
 
@@ -259,6 +272,19 @@ class Replica:
         it, loss = C.c_int32(), C.c_float()
         check(lib.sn_train_epoch(self.handle, self._ptr(x), self._ptr(y), total_rows, batch, global_iter, C.byref(it),
                                  C.byref(loss) if want_loss else None))
+        return it.value, (loss.value if want_loss else None)
+
+
+    def train_epoch_host(self, x, y, batch: int, global_iter: int, want_loss: bool = True) -> Tuple[int, Optional[float]]:
+        """One epoch over a partition held in host memory (numpy float32 arrays, rows first; pinned ones from
+        `Context.pinned_array` make the batch copies overlap with training)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.ascontiguousarray(y, dtype=np.float32)
+        if x.shape[0] != y.shape[0]:
+            raise ValueError("x and y hold different numbers of rows")
+        it, loss = C.c_int32(), C.c_float()
+        check(lib.sn_train_epoch_host(self.handle, x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p), x.shape[0], batch,
+                                      global_iter, C.byref(it), C.byref(loss) if want_loss else None))
         return it.value, (loss.value if want_loss else None)
 
 

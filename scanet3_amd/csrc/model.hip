@@ -84,6 +84,11 @@ struct sn_replica {
   std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
   float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
   bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
+  // host-fed epochs: two device slots per tensor, a copy stream, "slot filled" / "slot consumed" events
+  float* stage_x[2] = {nullptr, nullptr};
+  float* stage_y[2] = {nullptr, nullptr};
+  hipStream_t copy_stream = nullptr;
+  hipEvent_t ev_filled[2] = {nullptr, nullptr}, ev_consumed[2] = {nullptr, nullptr};
   std::vector<void*> owned;
 };
 
@@ -799,6 +804,14 @@ int sn_replica_create(sn_model* model, const sn_optimizer_desc* opt, sn_replica*
 int sn_replica_destroy(sn_replica* rep) {
   SN_TRY(check_replica(rep));
   (void)hipStreamSynchronize(rep->ctx->stream);
+  if (rep->copy_stream) {
+    (void)hipStreamSynchronize(rep->copy_stream);
+    for (int i = 0; i < 2; ++i) {
+      (void)hipEventDestroy(rep->ev_filled[i]);
+      (void)hipEventDestroy(rep->ev_consumed[i]);
+    }
+    (void)hipStreamDestroy(rep->copy_stream);
+  }
   for (void* p : rep->owned) (void)hipFree(p);
   rep->model->live_replicas--;
   rep->magic = 0;
@@ -923,6 +936,64 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
     SN_TRY(loss_of(rep, pred, yl, batch, nullptr));
     SN_TRY(read_loss(rep, loss_host));
   }
+  return SN_OK;
+}
+
+// One epoch over a partition that lives in HOST memory (the reference's TensorIterator copies every batch into a
+// fresh tensor that the session then feeds, optimizers/Iterators.scala:57-78): batch i+1 travels to the device on a
+// second stream while batch i trains.  Two device slots; a slot is refilled only after the step that read it.
+int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_host, int64_t total_rows, int32_t batch,
+                        int32_t global_iter, int32_t* iterations_host, float* loss_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_host && y_host, "sn_train_epoch_host: null partition pointer");
+  SN_REQUIRE(batch >= 1 && batch <= rep->model->batch, "batch must be in 1..%d, got %d", rep->model->batch, batch);
+  SN_REQUIRE(global_iter >= 0, "global_iter must not be negative");
+  const int64_t n_batches = total_rows / batch;  // the partial batch is skipped (optimizers/Iterators.scala:90)
+  SN_REQUIRE(n_batches >= 1, "partition of %lld rows holds no full batch of %d (the reference's iterator throws here)",
+             (long long)total_rows, batch);
+  hipStream_t compute = rep->ctx->stream;
+  if (!rep->copy_stream) {
+    for (int i = 0; i < 2; ++i) {
+      SN_TRY(dev_alloc(rep, &rep->stage_x[i], rep->model->in_elems * rep->model->batch));
+      SN_TRY(dev_alloc(rep, &rep->stage_y[i], rep->model->out_elems * rep->model->batch));
+      SN_HIP(hipEventCreateWithFlags(&rep->ev_filled[i], hipEventDisableTiming));
+      SN_HIP(hipEventCreateWithFlags(&rep->ev_consumed[i], hipEventDisableTiming));
+    }
+    SN_HIP(hipStreamCreateWithFlags(&rep->copy_stream, hipStreamNonBlocking));
+  }
+  const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
+  auto fill = [&](int64_t i, int slot) -> int {
+    SN_HIP(hipMemcpyAsync(rep->stage_x[slot], x_host + i * xs, (size_t)xs * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
+    SN_HIP(hipMemcpyAsync(rep->stage_y[slot], y_host + i * ys, (size_t)ys * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
+    SN_HIP(hipEventRecord(rep->ev_filled[slot], rep->copy_stream));
+    return SN_OK;
+  };
+  // earlier work on the compute stream may still read the slots (a previous epoch's last loss)
+  SN_HIP(hipEventRecord(rep->ev_consumed[0], compute));
+  SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[0], 0));
+  SN_TRY(fill(0, 0));
+  for (int64_t i = 0; i < n_batches; ++i) {
+    const int slot = (int)(i & 1);
+    if (i + 1 < n_batches) {  // the other slot was last read by step i-1, already queued on the compute stream
+      if (i >= 1) SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[slot ^ 1], 0));
+      SN_TRY(fill(i + 1, slot ^ 1));
+    }
+    SN_HIP(hipStreamWaitEvent(compute, rep->ev_filled[slot], 0));
+    SN_TRY(grad_pass(rep, rep->stage_x[slot], rep->stage_y[slot], batch));
+    SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
+    SN_HIP(hipEventRecord(rep->ev_consumed[slot], compute));
+  }
+  if (iterations_host) *iterations_host = (int32_t)n_batches;
+  const int last = (int)((n_batches - 1) & 1);
+  if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
+    SN_TRY(forward(rep, rep->stage_x[last], batch));
+    const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, rep->stage_x[last], batch);
+    SN_TRY(loss_of(rep, pred, rep->stage_y[last], batch, nullptr));
+    SN_TRY(read_loss(rep, loss_host));
+  } else {
+    SN_HIP(hipStreamSynchronize(compute));  // the host buffers may be reused once this returns
+  }
+  SN_HIP(hipStreamSynchronize(rep->copy_stream));
   return SN_OK;
 }
 

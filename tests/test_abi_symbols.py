@@ -22,7 +22,7 @@ def test_header_declares_the_expected_surface():
 
 def test_library_exports_every_declared_symbol():
     path = os.path.join(ROOT, "scanet3_amd", "libscanet_hip.so")
-    assert os.path.exists(path), "build the library first: python -m scanet3_amd.build"
+    assert os.path.exists(path), "build the library first: python scanet3_amd/build.py"
     lib = ctypes.CDLL(path)
     for name in declared_functions():
         assert hasattr(lib, name), f"{name} is declared in include/scanet_hip.h but not exported"

@@ -523,6 +523,47 @@ def test_train_epoch_semantics_and_replica_average(S, ctx, linear_function):
     cm.close()
 
 
+@pytest.mark.parametrize("n_batches", [1, 2, 7])
+def test_train_epoch_from_host_memory_equals_resident_epoch(S, ctx, n_batches):
+    """`sn_train_epoch_host` (batches copied on a second stream while the previous one trains) must leave exactly the
+    weights, optimizer state and loss of `sn_train_epoch` on a device-resident copy: same kernels, same order."""
+    spec = [("dense", 24, "tanh"), ("dense", 3, "softmax")]
+    om, layers, sloss = build_pair(spec, "cce")
+    batch, rows = 32, 32 * n_batches + 5               # 5 rows of a partial batch that both paths skip
+    rng = np.random.default_rng(20251125 + 8)
+    params = glorot_params(om, (batch, 10), rng)
+    X = rng.standard_normal((rows, 10)).astype(f32)
+    Y = one_hot(rng, rows, 3)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (10,), batch)
+    res, host, pinned = cm.replica(S.Adam(0.01)), cm.replica(S.Adam(0.01)), cm.replica(S.Adam(0.01))
+    Xp, Yp = ctx.pinned_array(X.shape), ctx.pinned_array(Y.shape)
+    Xp[...] = X
+    Yp[...] = Y
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    for r in (res, host, pinned):
+        r.set_params(params)
+    git = 0
+    for epoch in range(3):                              # the staging slots are reused across epochs
+        a = res.train_epoch(Xb, Yb, rows, batch, git)
+        b = host.train_epoch_host(X, Y, batch, git)
+        c = pinned.train_epoch_host(Xp, Yp, batch, git)
+        assert a == b == c and a[0] == n_batches, (epoch, a, b, c)
+        git += a[0]
+    want, st = res.get_params(), res.get_opt_state(1)
+    for r in (host, pinned):
+        got, gst = r.get_params(), r.get_opt_state(1)
+        for p in want:
+            np.testing.assert_array_equal(got[p], want[p])
+            np.testing.assert_array_equal(gst[p], st[p])
+    with pytest.raises(S.ScanetError):
+        host.train_epoch_host(X[:10], Y[:10], batch, 0)   # no full batch
+    for r in (res, host, pinned):
+        r.close()
+    cm.close()
+    Xb.free()
+    Yb.free()
+
+
 def test_dsl_training_run_matches_oracle_and_thresholds(S, golden, linear_function, logistic_data):
     """The reference's own convergence tests, run through the DSL mirror on the GPU."""
     X, Y = linear_function
