@@ -145,7 +145,7 @@ def dominant_gemm_roofline(kernels, peak_tflops):
     name, k, fl = best
     ach = fl / (k["avg_us"] * 1e-6) / 1e12
     return {"kernel": name, "bound": "mfma", "achieved": ach, "peak": peak_tflops, "unit": "TFLOP/s", "frac": ach / peak_tflops,
-            "avg_launch_us": k["avg_us"], "flops_per_launch": fl, "traffic": None}
+            "avg_launch_us": k["avg_us"], "flops_per_launch": fl, "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(name)}
 
 
 def bench_lenet(S, ctx, steps, warmup, pool_stride=1):
@@ -184,6 +184,13 @@ def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
 # of known size: WRITE_SIZE x 1.0, FETCH_SIZE x 2.0); summary in profiles/optimizer_100M_and_average_8x25M_hbm_traffic_pmc.md
 MEASURED_TRAFFIC_BYTES = {"sgd": 2.000e9, "adagrad": 2.000e9, "rmsprop": 2.000e9, "adadelta": 2.800e9, "adam": 2.800e9,
                           "nadam": 2.800e9, "adamax": 2.800e9, "amsgrad": 3.600e9, "average": 0.900e9}
+# the same for the matrix kernels (profiles/lenet_and_wide_mlp_gemm_kernels_hbm_traffic_pmc.md); keyed by kernel label
+MEASURED_GEMM_TRAFFIC_BYTES = {
+    "conv2d_forward[52900x64x288]": 14.1e6 + 13.5e6,
+    "conv2d_input_gradient[62500x32x576]": 19.9e6 + 8.0e6,
+    "conv2d_filter_gradient[288x64x52900]": 23.4e6 + 18.8e6,
+    "gemm_bf16_256[8192x4096x4096]": 404e6 + 135e6,
+}
 OPT_BYTES = {"sgd": 20, "adagrad": 20, "rmsprop": 20, "adadelta": 28, "adam": 28, "nadam": 28, "adamax": 28, "amsgrad": 36}
 
 
