@@ -50,21 +50,62 @@ struct StepFwdArgs {
   const float* h_prev;  // [rows, H] or null (first step: h_{-1} = 0 drops out of the product)
   const float* c_prev;  // [rows, H] or null
   LstmWeights w;
+  const float* wpack;   // the weights in LDS order (pack_fwd_kernel)
   float* gates;         // [rows, 4H] activated forget, input, gate, output
   float* c;             // [rows, H]
   float* h;             // [rows, H]
   int rows, T, F, H, t;
 };
 
-// UB hidden units (x 4 gates) per workgroup: 16 (one gate per wavefront, two row blocks each) or 8 (two gates per
-// wavefront column block, one row block each; half the LDS, so two workgroups share a CU).
-template <int UB>
+// Weights in the order the step kernel's LDS wants them, rebuilt once per pass over the sequence (they change once
+// per training step, the step kernel runs T times): [unit group of 16][gate][k/4][16 units][4 consecutive k],
+// k over [Wk; Wr] padded with zeros to a multiple of 16.  The step kernel then copies its slab with contiguous
+// 16-byte loads instead of gathering 4-byte values from 4 rows per cell.
+__global__ __launch_bounds__(256) void pack_fwd_kernel(LstmWeights w, int F, int H, float* __restrict__ out) {
+  const int K = F + H, kq = round16(K) / 4;
+  const int64_t cells = (int64_t)(H / 16) * 4 * kq * 16;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < cells; e += (int64_t)gridDim.x * 256) {
+    const int bu = (int)(e & 15);
+    int64_t t = e >> 4;
+    const int q = (int)(t % kq); t /= kq;
+    const int gate = (int)(t & 3);
+    const int cg = (int)(t >> 2);
+    f4v v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * q + j;
+      if (k < F) v[j] = w.wk[gate][(int64_t)k * H + cg * 16 + bu];
+      else if (k < K) v[j] = w.wr[gate][(int64_t)(k - F) * H + cg * 16 + bu];
+    }
+    *(f4v*)(out + e * 4) = v;
+  }
+}
+
+// [gate][unit block of 16][n/4][16 units][4 consecutive n] of the recurrent weights Wr_gate[u][n], n padded to 16
+__global__ __launch_bounds__(256) void pack_dh_kernel(LstmWeights w, int H, float* __restrict__ out) {
+  const int kq = round16(H) / 4;
+  const int64_t cells = (int64_t)4 * (H / 16) * kq * 16;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < cells; e += (int64_t)gridDim.x * 256) {
+    const int bu = (int)(e & 15);
+    int64_t t = e >> 4;
+    const int q = (int)(t % kq); t /= kq;
+    const int ublk = (int)(t % (H / 16));
+    const int gate = (int)(t / (H / 16));
+    f4v v = {0.f, 0.f, 0.f, 0.f};
+    if (4 * q < H) v = *(const f4v*)(w.wr[gate] + (int64_t)(ublk * 16 + bu) * H + 4 * q);  // H % 16 == 0: whole quads
+    *(f4v*)(out + e * 4) = v;
+  }
+}
+
+// 16 hidden units (x 4 gates) per workgroup: one gate per wavefront, two row blocks each.
 __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
+  constexpr int UB = 16;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int K = a.h_prev ? a.F + a.H : a.F;
   const int K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
   float* As = lds;                 // [RB][KP]
   constexpr int NCB = UB / 4, NRB = NCB / 2;  // column blocks of 16 (column = gate * UB + unit); row blocks per wavefront
+  const int kq_full = round16(a.F + a.H) / 4;  // quads per gate in the packed weights (the first step uses only F/4 of them)
   float* Bs = lds + RB * KP;       // [NCB][kq][16 columns][4]
   float* Zx = lds;                 // [4 gates][RB][ZP], over the operand slabs once every wavefront has finished multiplying
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -90,17 +131,13 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
     }
     if (pass * 16 * NQ < kq) {
 #pragma unroll
-      for (int cbi = 0; cbi < NCB; ++cbi) {
-        const int col = cbi * 16 + bu, gate = col / UB, u = col % UB;
+      for (int cbi = 0; cbi < NCB; ++cbi) {  // column block = gate; the packed slab has the LDS cell order
+        const float* slab = a.wpack + ((int64_t)blockIdx.x * 4 + cbi) * kq_full * 64;
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-          const int q = (pass * NQ + i) * 16 + (tid >> 4), k = q * 4;
+          const int q = (pass * NQ + i) * 16 + (tid >> 4);
           vb[cbi][i] = f4v{0.f, 0.f, 0.f, 0.f};
-          if (q < kq && k < K) {
-            const float* src = (k < a.F ? a.w.wk[gate] + (int64_t)k * a.H : a.w.wr[gate] + (int64_t)(k - a.F) * a.H) + u0 + u;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) vb[cbi][i][j] = src[(int64_t)j * a.H];
-          }
+          if (q < kq) vb[cbi][i] = *(const f4v*)(slab + (q * 16 + bu) * 4);
         }
       }
     }
@@ -163,7 +200,7 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
 // ---------------------------------------------------------------------------- backward: partial dh per gate
 struct StepDhArgs {
   const float* dz;      // [rows, 4H]
-  const float* wr[4];   // [H, H] recurrent weights per gate
+  const float* wpack;   // recurrent weights in LDS order (pack_dh_kernel)
   float* dh_parts;      // [4][part_stride] partial dh_prev, one per gate
   int64_t part_stride;
   int rows, H;
@@ -183,7 +220,6 @@ __global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
   const float* dzg = a.dz + (int64_t)gate * a.H;
 
   // Staging as in the forward kernel: one pass (H up to 384) with every load in flight before the LDS writes.
-  // B(k = n, column = u) = Wr_gate[u][n]: n is contiguous in memory, so a 16-byte load is already one LDS cell.
   constexpr int NA = 12, NQ = 6;
   for (int pass = 0; pass * 8 * NA < kq; ++pass) {
     f4v va[NA], vb[NCB][NQ];
@@ -199,9 +235,9 @@ __global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
       for (int wv = 0; wv < NCB; ++wv)
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-          const int q = (pass * NQ + i) * 16 + (tid >> 4), u = u0 + wv * 16 + bu;
+          const int q = (pass * NQ + i) * 16 + (tid >> 4), ublk = (u0 >> 4) + wv;
           vb[wv][i] = f4v{0.f, 0.f, 0.f, 0.f};
-          if (q < kq && u < a.H && q * 4 < K) vb[wv][i] = *(const f4v*)(a.wr[gate] + (int64_t)u * a.H + q * 4);
+          if (q < kq && ublk * 16 < a.H) vb[wv][i] = *(const f4v*)(a.wpack + ((((int64_t)gate * (a.H / 16) + ublk) * kq + q) * 16 + bu) * 4);
         }
     }
 #pragma unroll
@@ -266,28 +302,44 @@ bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w) {
   return true;
 }
 
-int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
-                         const LstmWeights& w, float* gates, float* c, float* h) {
-  if (rows <= 0) return SN_OK;
-  SN_REQUIRE(lstm_step_fused_ok(F, H, x, w), "lstm_step_forward: F=%d H=%d outside what the fused kernel handles", F, H);
-  static bool attr_set = false;
-  StepFwdArgs a{x, h_prev, c_prev, w, gates, c, h, rows, T, F, H, t};
-  const int K = h_prev ? F + H : F;
-  // 16 units per workgroup.  The 8-unit form (two workgroups per CU) was measured slower here (13.0 vs 12.0 us per
-  // step at 512 x 1024 x 288): it re-reads the [x_t, h] slab twice as often, and the step is bound by that traffic.
-  LaunchScope scope(ctx, "lstm_step_forward", rows, 4 * H, K);
-  SN_TRY(allow_lds(lstm_step_fwd_kernel<16>, 64, &attr_set));
-  hipLaunchKernelGGL(lstm_step_fwd_kernel<16>, dim3((unsigned)(H / 16), (unsigned)ceil_div(rows, RB)), dim3(256), lds_bytes(K, 64), ctx->stream, a);
+int64_t lstm_pack_elems(int F, int H) { return (int64_t)4 * H * round16(F + H); }
+
+int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh) {
+  if (pack_fwd) {
+    const int64_t cells = (int64_t)H * round16(F + H);
+    LaunchScope scope(ctx, "lstm_pack_weights");
+    hipLaunchKernelGGL(pack_fwd_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, F, H, pack_fwd);
+  }
+  if (pack_dh) {
+    const int64_t cells = (int64_t)H * round16(H);
+    LaunchScope scope(ctx, "lstm_pack_weights");
+    hipLaunchKernelGGL(pack_dh_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, H, pack_dh);
+  }
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
 
-int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_parts, int64_t part_stride) {
+int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
+                         const LstmWeights& w, const float* wpack, float* gates, float* c, float* h) {
   if (rows <= 0) return SN_OK;
-  SN_REQUIRE(H % 4 == 0 && H <= MAX_K && aligned16(dz) && aligned16(w.wr[0]) && aligned16(w.wr[1]) && aligned16(w.wr[2]) && aligned16(w.wr[3]),
-             "lstm_step_hidden_gradient: H=%d outside what the fused kernel handles", H);
+  SN_REQUIRE(lstm_step_fused_ok(F, H, x, w), "lstm_step_forward: F=%d H=%d outside what the fused kernel handles", F, H);
+  static bool attr_set = false;
+  StepFwdArgs a{x, h_prev, c_prev, w, wpack, gates, c, h, rows, T, F, H, t};
+  const int K = h_prev ? F + H : F;
+  // 16 units per workgroup.  The 8-unit form (two workgroups per CU) was measured slower here (13.0 vs 12.0 us per
+  // step at 512 x 1024 x 288): it re-reads the [x_t, h] slab twice as often, and the step is bound by that traffic.
+  LaunchScope scope(ctx, "lstm_step_forward", rows, 4 * H, K);
+  SN_TRY(allow_lds(lstm_step_fwd_kernel, 64, &attr_set));
+  hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3((unsigned)(H / 16), (unsigned)ceil_div(rows, RB)), dim3(256), lds_bytes(K, 64), ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride) {
+  if (rows <= 0) return SN_OK;
+  SN_REQUIRE(H % 16 == 0 && H <= MAX_K && aligned16(dz) && aligned16(wpack), "lstm_step_hidden_gradient: H=%d outside what the fused kernel handles", H);
   static bool attr_set[2] = {false, false};
-  StepDhArgs a{dz, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, dh_parts, part_stride, rows, H};
+  StepDhArgs a{dz, wpack, dh_parts, part_stride, rows, H};
   // 32 units per workgroup (two workgroups per CU) when 64 would leave fewer than two per CU: 10.8 vs 11.4 us per step
   const bool narrow = ceil_div(H, 64) * ceil_div(rows, RB) * 4 < (int64_t)2 * ctx->compute_units;
   LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, 4 * H);

@@ -78,6 +78,7 @@ struct sn_replica {
   // lstm scratch (one set, shared by every LSTM op; sized for the largest)
   float* lstm_z = nullptr;
   std::vector<float*> lstm_gates, lstm_c, lstm_h, lstm_dz;  // per op
+  std::vector<float*> lstm_pk_fwd, lstm_pk_dh;              // per op: weights in the step kernels' LDS order
   float* lstm_dh[2] = {nullptr, nullptr};
   float* lstm_dc = nullptr;
   // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
@@ -343,6 +344,8 @@ static int alloc_replica(sn_replica* r) {
   r->lstm_c.assign(n_ops, nullptr);
   r->lstm_h.assign(n_ops, nullptr);
   r->lstm_dz.assign(n_ops, nullptr);
+  r->lstm_pk_fwd.assign(n_ops, nullptr);
+  r->lstm_pk_dh.assign(n_ops, nullptr);
   r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
   r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
   int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0;
@@ -355,6 +358,8 @@ static int alloc_replica(sn_replica* r) {
       SN_TRY(dev_alloc(r, &r->lstm_c[i], (int64_t)op.T * bh));
       SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = h_{-1}
       SN_TRY(dev_alloc(r, &r->lstm_dz[i], (int64_t)op.T * bh * 4));
+      SN_TRY(dev_alloc(r, &r->lstm_pk_fwd[i], lstm_pack_elems(op.F, op.H)));
+      SN_TRY(dev_alloc(r, &r->lstm_pk_dh[i], lstm_pack_elems(op.F, op.H)));
       SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
       lstm_z = std::max(lstm_z, bh * 4);
       lstm_h = std::max(lstm_h, bh);
@@ -473,11 +478,12 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
+        if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr));
         for (int t = 0; t < op.T; ++t) {
           const float* h_prev = r->lstm_h[i] + (int64_t)t * bh;
           if (fused) {
             SN_TRY(launch_lstm_step_fwd(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh,
-                                        rows, op.H, w, r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
+                                        rows, op.H, w, r->lstm_pk_fwd[i], r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                                         r->lstm_h[i] + (int64_t)(t + 1) * bh));
             continue;
           }
@@ -612,6 +618,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         const float* dh = dy;  // gradient of the last hidden state
         int hb = 0, dh_parts = 1;
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
+        if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
         for (int t = op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                             t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
@@ -620,7 +627,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
           if (t > 0) {
             if (fused) {  // four per-gate partial products; the next gate-gradient kernel adds them
-              SN_TRY(launch_lstm_step_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], bh));
+              SN_TRY(launch_lstm_step_dh(ctx, a.dz, rows, op.H, r->lstm_pk_dh[i], r->lstm_dh[hb], bh));
               dh_parts = 4;
             } else {
               SN_TRY(launch_lstm_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], r->ws, m->workspace_elems));
