@@ -63,6 +63,8 @@ struct sn_ctx {
   std::vector<hipEvent_t> event_pool;
   std::map<std::string, sn::ProfileEntry> profile;
   std::vector<std::string> profile_names;  // stable order for sn_profile_get
+  // kernels whose dynamic-LDS limit has been raised on this context's device, with the size granted
+  std::map<const void*, size_t> lds_limit;
 };
 
 namespace sn {
@@ -84,6 +86,15 @@ struct LaunchScope {
 int profile_drain(sn_ctx* ctx);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Kernels that use more than 64 KiB of dynamic LDS must have their limit raised once per device; remembered per context.
+inline int allow_dynamic_lds(sn_ctx* ctx, const void* kernel, size_t bytes) {
+  auto it = ctx->lds_limit.find(kernel);
+  if (it != ctx->lds_limit.end() && it->second >= bytes) return SN_OK;
+  SN_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  ctx->lds_limit[kernel] = bytes;
+  return SN_OK;
+}
 inline int64_t align_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
 
 // ---- optimizer / averaging kernels (optim_kernels.hip) ---------------------------------

@@ -301,22 +301,15 @@ void gemm_bf16_tn_128(const bf16* __restrict__ A, int64_t lda, const bf16* __res
 template <int MODE>
 static int launch_mode(sn_ctx* ctx, const bf16* a, int64_t lda, const bf16* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep) {
   const int64_t big_tiles = ceil_div(M, 256) * ceil_div(N, 256);
-  static bool attr_set[2] = {false, false};  // per instantiation
   if (big_tiles >= ctx->compute_units && M % 256 == 0 && N % 256 == 0) {
     const size_t smem = 4 * 128 * tr_pitch<128>() > 4 * 256 * 128 ? 4 * 128 * tr_pitch<128>() : 4 * 256 * 128;
-    if (!attr_set[0]) {
-      SN_HIP(hipFuncSetAttribute((const void*)gemm_bf16_tn_256<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-      attr_set[0] = true;
-    }
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_256<MODE>, smem));
     const int tm = (int)ceil_div(M, 256), tn = (int)ceil_div(N, 256);
     LaunchScope scope(ctx, "gemm_bf16_256", M, N, K);
     hipLaunchKernelGGL(gemm_bf16_tn_256<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);
   } else {
     const size_t smem = 4 * 64 * tr_pitch<64>() > 4 * 128 * 128 ? 4 * 64 * tr_pitch<64>() : 4 * 128 * 128;
-    if (!attr_set[1]) {
-      SN_HIP(hipFuncSetAttribute((const void*)gemm_bf16_tn_128<MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-      attr_set[1] = true;
-    }
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_128<MODE>, smem));
     const int tm = (int)ceil_div(M, 128), tn = (int)ceil_div(N, 128);
     LaunchScope scope(ctx, "gemm_bf16_128", M, N, K);
     hipLaunchKernelGGL(gemm_bf16_tn_128<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);

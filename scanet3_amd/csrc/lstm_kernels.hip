@@ -282,15 +282,6 @@ size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 o
   return (slabs > exchange ? slabs : exchange) * sizeof(float);
 }
 
-template <class KernelT>
-int allow_lds(KernelT kernel, int cols, bool* done) {
-  if (!*done) {
-    SN_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(MAX_K, cols)));
-    *done = true;
-  }
-  return SN_OK;
-}
-
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace
@@ -323,13 +314,12 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h) {
   if (rows <= 0) return SN_OK;
   SN_REQUIRE(lstm_step_fused_ok(F, H, x, w), "lstm_step_forward: F=%d H=%d outside what the fused kernel handles", F, H);
-  static bool attr_set = false;
   StepFwdArgs a{x, h_prev, c_prev, w, wpack, gates, c, h, rows, T, F, H, t};
   const int K = h_prev ? F + H : F;
   // 16 units per workgroup.  The 8-unit form (two workgroups per CU) was measured slower here (13.0 vs 12.0 us per
   // step at 512 x 1024 x 288): it re-reads the [x_t, h] slab twice as often, and the step is bound by that traffic.
   LaunchScope scope(ctx, "lstm_step_forward", rows, 4 * H, K);
-  SN_TRY(allow_lds(lstm_step_fwd_kernel, 64, &attr_set));
+  SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_fwd_kernel, lds_bytes(MAX_K, 64)));
   hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3((unsigned)(H / 16), (unsigned)ceil_div(rows, RB)), dim3(256), lds_bytes(K, 64), ctx->stream, a);
   SN_HIP(hipGetLastError());
   return SN_OK;
@@ -338,17 +328,16 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
 int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride) {
   if (rows <= 0) return SN_OK;
   SN_REQUIRE(H % 16 == 0 && H <= MAX_K && aligned16(dz) && aligned16(wpack), "lstm_step_hidden_gradient: H=%d outside what the fused kernel handles", H);
-  static bool attr_set[2] = {false, false};
   StepDhArgs a{dz, wpack, dh_parts, part_stride, rows, H};
   // 32 units per workgroup (two workgroups per CU) when 64 would leave fewer than two per CU: 10.8 vs 11.4 us per step
   const bool narrow = ceil_div(H, 64) * ceil_div(rows, RB) * 4 < (int64_t)2 * ctx->compute_units;
   LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, 4 * H);
   if (narrow) {
-    SN_TRY(allow_lds(lstm_step_dh_kernel<32>, 32, &attr_set[0]));
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_dh_kernel<32>, lds_bytes(MAX_K, 32)));
     hipLaunchKernelGGL(lstm_step_dh_kernel<32>, dim3((unsigned)ceil_div(H, 32), (unsigned)ceil_div(rows, RB), 4), dim3(256), lds_bytes(H, 32),
                        ctx->stream, a);
   } else {
-    SN_TRY(allow_lds(lstm_step_dh_kernel<64>, 64, &attr_set[1]));
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_dh_kernel<64>, lds_bytes(MAX_K, 64)));
     hipLaunchKernelGGL(lstm_step_dh_kernel<64>, dim3((unsigned)ceil_div(H, 64), (unsigned)ceil_div(rows, RB), 4), dim3(256), lds_bytes(H, 64),
                        ctx->stream, a);
   }
