@@ -464,6 +464,16 @@ int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, 
   return SN_OK;
 }
 
+// Consecutive workgroup ids land on different XCDs (8, each with its own L2).  Stencil kernels whose neighbouring
+// workgroups read overlapping rows use this block number instead: XCD x gets the x-th contiguous eighth of the
+// blocks, so the shared rows are fetched into one L2 only.  The grid must be a multiple of 8.
+__device__ __forceinline__ unsigned xcd_contiguous_block() {
+  return (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+}
+static inline unsigned grid_for_xcd(sn_ctx* ctx, int64_t n, int per_block) {
+  return (grid_for(ctx, n, per_block) + 7u) & ~7u;
+}
+
 // ---------------------------------------------------------------------------- max pooling (NHWC)
 // Forward keeps, per output element, the window offset (r*kw + q) of the first maximum in
 // row-major window order; padding cells never win (TF MaxPoolV2, math/nn/AllKernels.scala:270-303).
@@ -475,7 +485,7 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restric
   const I cv = (I)(c / V);
   const I total = (I)n * ho * wo * cv;
   const I stride = (I)gridDim.x * blockDim.x;
-  for (I i = (I)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+  for (I i = (I)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
     const I ch = (i % cv) * V;
     I t = i / cv;
     const int ow = (int)(t % wo); t /= wo;
@@ -521,7 +531,7 @@ int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int 
   if (total <= 0) return SN_OK;
   const bool small = total < (1ll << 31) && (int64_t)n * h * w * c < (1ll << 31);
   const bool v4 = pool_vec4(x, y, arg, c);
-  const dim3 grid(grid_for(ctx, v4 ? total / 4 : total, 256));
+  const dim3 grid(grid_for_xcd(ctx, v4 ? total / 4 : total, 256));
   LaunchScope scope(ctx, "maxpool_forward");
 #define SN_POOL_FWD(V, I) \
   hipLaunchKernelGGL((maxpool_fwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl)
@@ -544,7 +554,7 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restric
   const I cv = (I)(c / V);
   const I total = (I)n * h * w * cv;
   const I stride = (I)gridDim.x * blockDim.x;
-  for (I i = (I)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+  for (I i = (I)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
     const I ch = (i % cv) * V;
     I t = i / cv;
     const int ix = (int)(t % w); t /= w;
@@ -602,7 +612,7 @@ int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* 
   if (total <= 0) return SN_OK;
   const bool small = total < (1ll << 31) && (int64_t)n * ho * wo * c < (1ll << 31);
   const bool v4 = pool_vec4(dy, dx, arg, c) && (reinterpret_cast<uintptr_t>(y_in) & 15u) == 0;
-  const dim3 grid(grid_for(ctx, v4 ? total / 4 : total, 256));
+  const dim3 grid(grid_for_xcd(ctx, v4 ? total / 4 : total, 256));
   LaunchScope scope(ctx, y_in ? "maxpool_activation_backward" : "maxpool_backward");
 #define SN_POOL_BWD(V, I) \
   hipLaunchKernelGGL((maxpool_bwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl, y_in, act, act_param)
