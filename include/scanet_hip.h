@@ -56,7 +56,7 @@ enum {
 
 /* ---- layer list (models/layer/*.scala, flattened as layer/Composed.scala:89-99 does) ---- */
 enum { SN_LAYER_DENSE = 0, SN_LAYER_BIAS = 1, SN_LAYER_ACTIVATE = 2, SN_LAYER_FLATTEN = 3,
-       SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6 };
+       SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6, SN_LAYER_SIMPLE_RNN = 7 };
 /* models/Activation.scala:32-83 */
 enum { SN_ACT_IDENTITY = 0, SN_ACT_SIGMOID = 1, SN_ACT_TANH = 2, SN_ACT_RELU = 3, SN_ACT_SOFTMAX = 4 };
 /* models/Loss.scala:18-57 */
@@ -80,15 +80,16 @@ enum {
  * "<index in this list>/weights" exactly as Composed.params builds them. */
 typedef struct sn_layer_desc {
   int32_t kind;          /* SN_LAYER_* */
-  int32_t units;         /* Dense outputs / Bias features / Conv2D filters / LSTM units */
-  int32_t activation;    /* ACTIVATE: SN_ACT_*  (LSTM: cell activation, must be SN_ACT_TANH) */
+  int32_t units;         /* Dense outputs / Bias features / Conv2D filters / LSTM or SimpleRNN units */
+  int32_t activation;    /* ACTIVATE: SN_ACT_*  (LSTM: cell activation, must be SN_ACT_TANH; SIMPLE_RNN: the cell's
+                            activation, layer/RNN.scala:115,162) */
   float act_param;       /* ReLU threshold (Activation.scala:79-82) */
   int32_t kernel_h, kernel_w;   /* Conv2D kernel / Pool2D window */
   int32_t stride_h, stride_w;
   int32_t padding;       /* SN_PAD_* */
   int32_t reg_kind;      /* Dense/Bias: SN_REG_* */
   float reg_lambda;
-  int32_t use_bias;      /* LSTM only: per-gate bias vectors (layer/RNN.scala:215) */
+  int32_t use_bias;      /* LSTM: per-gate bias vectors (layer/RNN.scala:215); SIMPLE_RNN: the cell's Bias (RNN.scala:116) */
 } sn_layer_desc;
 
 /* An `Algorithm` case class (optimizers/Algorithm.scala:6-11).  Field use per kind:

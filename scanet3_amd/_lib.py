@@ -17,7 +17,7 @@ SN_MAX_OPT_STATES = 3
 SN_MAX_AVG_INPUTS = 32
 
 # enums of include/scanet_hip.h
-LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM = range(7)
+LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM, LAYER_SIMPLE_RNN = range(8)
 ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = range(5)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
 PAD_VALID, PAD_SAME = 0, 1

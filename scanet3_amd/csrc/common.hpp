@@ -214,15 +214,17 @@ struct LstmGrads {
 };
 // z[rows,4H] = [x_t, h_prev] * [Wk; Wr] + b   (x_t = x[:, t, :] of a [rows,T,F] tensor)
 int launch_lstm_z(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, int rows, int H, const LstmWeights& w,
-                  float* z, float* ws, int64_t ws_elems);
+                  float* z, float* ws, int64_t ws_elems, int gates = 4);
 // dh_prev[rows,H] = dz[rows,4H] * Wr^T
-int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems);
+int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems,
+                   int gates = 4);
 // dx[:, t, :] = dz * Wk^T
 int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, int T, const LstmWeights& w, float* dx, float* ws,
-                   int64_t ws_elems);
+                   int64_t ws_elems, int gates = 4);
 // dWk = X^T dZ, dWr = Hprev^T dZ over all steps (dz_all, h_all time-major [T,rows,*]; h_all[t] = h_{t-1})
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
-                      const LstmGrads& g, float* ws, int64_t ws_elems);
+                      const LstmGrads& g, float* ws, int64_t ws_elems, int gates = 4);
+// The simple recurrent cell is the same four products with one gate (gates = 1): its weights sit in slot 0.
 
 int64_t gemm_workspace_elems(int m, int n, int k, int cu);
 

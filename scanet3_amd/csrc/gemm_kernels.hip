@@ -314,7 +314,7 @@ struct LstmZA {
 struct LstmZB {
   static constexpr bool K_CONTIG = false;
   LstmWeights w;
-  int F, H;
+  int F, H, G;  // G gates side by side (4 for the LSTM, 1 for the simple cell)
   struct Cursor {
     const float* wk;  // column base inside the gate's kernel matrix, null outside
     const float* wr;
@@ -322,7 +322,7 @@ struct LstmZB {
   };
   __device__ __forceinline__ void init(Cursor& c, int n, int k) const {
     c.k = k;
-    if (n >= 4 * H) { c.wk = c.wr = nullptr; return; }
+    if (n >= G * H) { c.wk = c.wr = nullptr; return; }
     const int gate = n / H, u = n % H;
     c.wk = w.wk[gate] + u;
     c.wr = w.wr[gate] + u;
@@ -338,7 +338,7 @@ struct LstmZB {
   }
   bool vec4_ok(int) const {
     bool ok = H % 4 == 0;
-    for (int g = 0; g < 4; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w.wk[g]) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w.wr[g]) & 15u) == 0;
+    for (int g = 0; g < G; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w.wk[g]) & 15u) == 0 && (reinterpret_cast<uintptr_t>(w.wr[g]) & 15u) == 0;
     return ok;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
@@ -349,7 +349,7 @@ struct LstmZB {
 struct LstmWT {
   static constexpr bool K_CONTIG = true;
   const float* w[4];
-  int n_rows, H;  // W_gate is [n_rows, H]
+  int n_rows, H, G;  // W_gate is [n_rows, H]; G gates
   struct Cursor {
     int n, k;
   };
@@ -369,7 +369,7 @@ struct LstmWT {
   }
   bool vec4_ok(int) const {
     bool ok = H % 4 == 0;
-    for (int g = 0; g < 4; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w[g]) & 15u) == 0;
+    for (int g = 0; g < G; ++g) ok = ok && (reinterpret_cast<uintptr_t>(w[g]) & 15u) == 0;
     return ok;
   }
   __device__ __forceinline__ void advance(Cursor& c, int dk) const { c.k += dk; }
@@ -634,12 +634,12 @@ struct StdEpilogue {
 struct LstmZEpilogue {  // z[m, n] = acc + b_gate[u]
   float* z;
   const float* b[4];
-  int H;
+  int H, G;
   __device__ __forceinline__ void store(int m, int n, float acc) const {
     const int gate = n / H, u = n - gate * H;
     float v = acc;
     if (b[gate]) v = v + b[gate][u];
-    z[(int64_t)m * 4 * H + n] = v;
+    z[(int64_t)m * G * H + n] = v;
   }
 };
 
@@ -1199,39 +1199,40 @@ int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const floa
 
 // ---------------------------------------------------------------------------- LSTM
 int launch_lstm_z(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, int rows, int H, const LstmWeights& w,
-                  float* z, float* ws, int64_t ws_elems) {
+                  float* z, float* ws, int64_t ws_elems, int gates) {
   LstmZA al{x, h_prev, rows, T, F, H, t};
-  LstmZB bl{w, F, H};
-  LstmZEpilogue ep{z, {w.b[0], w.b[1], w.b[2], w.b[3]}, H};
-  return launch_any<false>(ctx, "lstm_gate_gemm", rows, 4 * H, F + H, al, bl, ep, ws, ws_elems);
+  LstmZB bl{w, F, H, gates};
+  LstmZEpilogue ep{z, {w.b[0], w.b[1], w.b[2], w.b[3]}, H, gates};
+  return launch_any<false>(ctx, "lstm_gate_gemm", rows, gates * H, F + H, al, bl, ep, ws, ws_elems);
 }
 
-int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems) {
-  StridedLoader<true> al{dz, (int64_t)4 * H, 1, rows};
-  LstmWT bl{{w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, H, H};
+int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeights& w, float* dh_prev, float* ws, int64_t ws_elems,
+                   int gates) {
+  StridedLoader<true> al{dz, (int64_t)gates * H, 1, rows};
+  LstmWT bl{{w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, H, H, gates};
   Epilogue e;
   e.out = dh_prev;
   e.ldo = H;
   StdEpilogue ep{e};
-  return launch_any<false>(ctx, "lstm_hidden_gradient", rows, H, 4 * H, al, bl, ep, ws, ws_elems);
+  return launch_any<false>(ctx, "lstm_hidden_gradient", rows, H, gates * H, al, bl, ep, ws, ws_elems);
 }
 
 int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, int T, const LstmWeights& w, float* dx, float* ws,
-                   int64_t ws_elems) {
-  StridedLoader<true> al{dz, (int64_t)4 * H, 1, rows};
-  LstmWT bl{{w.wk[0], w.wk[1], w.wk[2], w.wk[3]}, F, H};
+                   int64_t ws_elems, int gates) {
+  StridedLoader<true> al{dz, (int64_t)gates * H, 1, rows};
+  LstmWT bl{{w.wk[0], w.wk[1], w.wk[2], w.wk[3]}, F, H, gates};
   DxScatterEpilogue ep{dx, T, F, t};
-  return launch_any<false>(ctx, "lstm_input_gradient", rows, F, 4 * H, al, bl, ep, ws, ws_elems);
+  return launch_any<false>(ctx, "lstm_input_gradient", rows, F, gates * H, al, bl, ep, ws, ws_elems);
 }
 
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
-                      const LstmGrads& g, float* ws, int64_t ws_elems) {
+                      const LstmGrads& g, float* ws, int64_t ws_elems, int gates) {
   const bool has_bias = g.b[0] != nullptr;
   const int M = F + H + (has_bias ? 1 : 0);
   LstmWgradA al{x, h_prev_all, rows, T, F, H, M};
-  StridedLoader<false> bl{dz_all, 1, (int64_t)4 * H, 4 * H};
+  StridedLoader<false> bl{dz_all, 1, (int64_t)gates * H, gates * H};
   LstmWgradEpilogue ep{g, F, H};
-  return launch_any<false>(ctx, "lstm_weight_gradient", M, 4 * H, T * rows, al, bl, ep, ws, ws_elems);
+  return launch_any<false>(ctx, "lstm_weight_gradient", M, gates * H, T * rows, al, bl, ep, ws, ws_elems);
 }
 
 }  // namespace sn

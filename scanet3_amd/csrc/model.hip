@@ -14,7 +14,7 @@
 
 namespace sn {
 
-enum OpKind { OP_DENSE, OP_CONV, OP_POOL, OP_FLATTEN, OP_BIASACT, OP_SOFTMAX, OP_LSTM };
+enum OpKind { OP_DENSE, OP_CONV, OP_POOL, OP_FLATTEN, OP_BIASACT, OP_SOFTMAX, OP_LSTM, OP_SRNN };
 
 struct ParamDef {
   sn_param_info info;
@@ -279,6 +279,26 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ++i;
         break;
       }
+      case SN_LAYER_SIMPLE_RNN: {
+        // RNN(SimpleRNNCell ?>> Bias ?>> activation), layer/RNN.scala:113-163; one "gate" whose weights use slot 0
+        SN_REQUIRE(cur.size() == 2, "layer %d: RNN requires input to have Shape(batch, time, features)", i);
+        SN_REQUIRE(L.units > 0, "layer %d: RNN Cell should contain at least one unit", i);
+        SN_REQUIRE(L.activation >= SN_ACT_IDENTITY && L.activation <= SN_ACT_RELU, "layer %d: unknown cell activation %d", i, L.activation);
+        op.kind = OP_SRNN;
+        op.T = (int)cur[0]; op.F = (int)cur[1]; op.H = L.units;
+        op.act = L.activation;
+        op.act_param = L.act_param;
+        op.lstm_p[0][0] = add_param(m, prefix(i) + "0/kernel_weights", {op.F, op.H}, SN_REG_NONE, 0.f);  // RNN.scala:165-166,198-203
+        op.lstm_p[0][1] = add_param(m, prefix(i) + "0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
+        if (L.use_bias) op.b = add_param(m, prefix(i) + "1/weights", {op.H}, SN_REG_NONE, 0.f);
+        op.out_dims = {L.units};
+        ws = std::max(ws, gemm_workspace_elems(B, op.H, op.F + op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(B, op.H, op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(B, op.F, op.H, cu));
+        ws = std::max(ws, gemm_workspace_elems(op.F + op.H, op.H, op.T * B, cu));
+        ++i;
+        break;
+      }
       default:
         return fail(SN_E_INVALID, "layer %d: unknown layer kind %d", i, L.kind);
     }
@@ -366,6 +386,12 @@ static int alloc_replica(sn_replica* r) {
       continue;  // output = last slice of lstm_h
     }
     SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
+    if (op.kind == OP_SRNN) {  // the carried state of every step and its gradient, time-major like the LSTM's
+      const int64_t bh = B * op.H;
+      SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = the initial state
+      SN_TRY(dev_alloc(r, &r->lstm_dz[i], (int64_t)op.T * bh));
+      SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
+    }
     if (op.kind == OP_POOL) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
     if (dense_bf16_fast(m, op)) {
       SN_TRY(dev_alloc(r, &r->bf_x[i], B * op.in_elems));
@@ -402,7 +428,7 @@ static const float* op_output(sn_replica* r, int i, const float* x, int rows) {
 }
 
 static LstmWeights lstm_weights(sn_replica* r, const Op& op, float* base) {
-  LstmWeights w;
+  LstmWeights w{};
   for (int gi = 0; gi < 4; ++gi) {
     w.wk[gi] = param_ptr(r, base, op.lstm_p[gi][0]);
     w.wr[gi] = param_ptr(r, base, op.lstm_p[gi][1]);
@@ -492,6 +518,18 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
                          r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
           SN_TRY(launch_lstm_gates_fwd(ctx, a, rows, op.H));
         }
+        break;
+      }
+      case OP_SRNN: {
+        // The state carried from step to step is the cell's product before bias and activation
+        // (layer/RNN.scala:189-196), so the recurrence is r_t = x_t Wk + r_{t-1} Wr and only the last step's
+        // output act(r + b) leaves the layer (RNN.scala:60-77 without returnSequence).
+        const int64_t bh = (int64_t)m->batch * op.H;
+        const LstmWeights w = lstm_weights(r, op, r->w);  // slot 0 only, no bias inside the recurrence
+        for (int t = 0; t < op.T; ++t)
+          SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, t == 0 ? nullptr : r->lstm_h[i] + (int64_t)t * bh, rows, op.H, w,
+                               r->lstm_h[i] + (int64_t)(t + 1) * bh, r->ws, m->workspace_elems, 1));
+        SN_TRY(launch_bias_act(ctx, r->lstm_h[i] + (int64_t)op.T * bh, param_ptr(r, r->w, op.b), r->act[i], rows, op.H, op.act, op.act_param));
         break;
       }
     }
@@ -643,6 +681,26 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           gr.b[gi] = param_ptr(r, r->g, op.lstm_p[gi][2]);
         }
         SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems));
+        if (need_dx) cur ^= 1;
+        break;
+      }
+      case OP_SRNN: {
+        SN_REQUIRE(rows == m->batch, "RNN training needs rows == batch (%d), got %d", m->batch, rows);
+        const int64_t bh = (int64_t)m->batch * op.H;
+        const LstmWeights w = lstm_weights(r, op, r->w);
+        // bias and activation touch the last step only; every earlier step acts through the carried state
+        float* dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
+        SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dr, (int64_t)rows * op.H, op.act, op.act_param));
+        if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dr, op.H, param_ptr(r, r->g, op.b), rows, op.H, r->ws, m->workspace_elems));
+        for (int t = op.T - 1; t >= 0; --t) {
+          dr = r->lstm_dz[i] + (int64_t)t * bh;
+          if (need_dx) SN_TRY(launch_lstm_dx(ctx, dr, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
+          if (t > 0) SN_TRY(launch_lstm_dh(ctx, dr, rows, op.H, w, dr - bh, r->ws, m->workspace_elems, 1));
+        }
+        LstmGrads gr{};
+        gr.wk[0] = param_ptr(r, r->g, op.lstm_p[0][0]);
+        gr.wr[0] = param_ptr(r, r->g, op.lstm_p[0][1]);
+        SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems, 1));
         if (need_dx) cur ^= 1;
         break;
       }

@@ -247,6 +247,15 @@ def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotU
                  inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
 
 
+def SimpleRNN(units: int, activation: Activation = Tanh, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
+              recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros) -> Layer:
+    """layer/RNN.scala:96-137: `RNN(SimpleRNNCell(..))`; the last step's output leaves the layer."""
+    if activation.kind == L.ACT_SOFTMAX:
+        raise ValueError("requirement failed: Softmax is not a cell activation")
+    return Layer(L.LAYER_SIMPLE_RNN, f"RNN(SimpleRNNCell({units},{activation!r},{'true' if bias else 'false'}))", units=units,
+                 activation=activation, use_bias=bias, inits=(kernelInitializer, recurrentInitializer, biasInitializer))
+
+
 def LinearRegression(reg: Regularization = Zero, bias: bool = True):
     """models/LinearRegression.scala: Dense(1), zero-initialised."""
     return Dense(1, Identity, reg, bias, Zeros, Zeros)
@@ -345,6 +354,12 @@ def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndar
         pre = "" if single else f"{i}/"
         if l.kind in (L.LAYER_DENSE, L.LAYER_BIAS, L.LAYER_CONV2D):
             out[pre + "weights"] = l.inits[0].build(shapes[pre + "weights"], rng)
+        elif l.kind == L.LAYER_SIMPLE_RNN:
+            k_init, r_init, b_init = l.inits
+            out[pre + "0/kernel_weights"] = k_init.build(shapes[pre + "0/kernel_weights"], rng)
+            out[pre + "0/recurrent_weights"] = r_init.build(shapes[pre + "0/recurrent_weights"], rng)
+            if l.use_bias:
+                out[pre + "1/weights"] = b_init.build(shapes[pre + "1/weights"], rng)
         elif l.kind == L.LAYER_LSTM:
             k_init, r_init, b_init, bf_init = l.inits
             for gate in ("forget", "input", "gate", "output"):

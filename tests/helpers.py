@@ -13,7 +13,7 @@ f32 = np.float32
 
 def build_pair(spec: List[tuple], loss: str):
     """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
-    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("activate", act) | ("bias", features)
+    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("activate", act) | ("bias", features)
     Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
     import scanet3_amd as S
     acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
@@ -51,6 +51,11 @@ def build_pair(spec: List[tuple], loss: str):
             bias = e[2] if len(e) > 2 else True
             ol.append(O.LSTM(e[1], bias=bias))
             add(S.LSTM(e[1], bias=bias))
+        elif k == "simple_rnn":  # ("simple_rnn", units[, act[, bias]])
+            act = e[2] if len(e) > 2 else "tanh"
+            bias = e[3] if len(e) > 3 else True
+            ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias))
+            add(S.SimpleRNN(e[1], acts_s[act], bias=bias))
         elif k == "activate":
             ol.append([O.Layer("activate", activation=acts_o[e[1]])])
             add(S.Activate(acts_s[e[1]]))

@@ -270,6 +270,17 @@ def test_golden_lstm_forward(S, ctx, golden):
     h.close()
 
 
+def test_golden_simple_rnn_forward(S, ctx, golden):
+    g = golden["simple_rnn"]
+    h = Harness(S, ctx, [("simple_rnn", 2, "identity")], "mse", (3, 1), 1)
+    params = {"0/kernel_weights": A(g["wx"]), "0/recurrent_weights": A(g["wh"]), "1/weights": A(g["b"])}
+    assert sorted(p for p, _, _ in h.cm.params) == sorted(params)
+    h.rep.set_params(params)
+    out = h.rep.forward(ctx.to_device(A(g["x"]).reshape(1, 3, 1)))
+    np.testing.assert_array_equal(round_at(out, 6), A(g["y_6dp"]))
+    h.close()
+
+
 def test_cnn_shape_table(S, ctx, golden):
     g = golden["cnn_shapes"]
     spec = [("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
@@ -294,6 +305,11 @@ MODELS = {
     "cnn_same_stride2_bias": ([("conv", 5, (3, 2), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "same"),
                                ("activate", "relu"), ("flatten",), ("dense", 4, "softmax")], "cce", (9, 10, 3), 7, "uniform_onehot"),
     "lstm_small": ([("lstm", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
+    "lstm_after_activation": ([("activate", "tanh"), ("lstm", 8), ("dense", 1, "tanh")], "mse", (5, 6), 12, "normal_regression"),
+    "simple_rnn_small": ([("simple_rnn", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
+    "simple_rnn_relu_nobias_after_activation": ([("activate", "tanh"), ("simple_rnn", 17, "relu", False), ("dense", 3, "identity")],
+                                                "mse", (6, 7), 21, "normal_regression"),
+    "simple_rnn_wide": ([("simple_rnn", 128, "sigmoid"), ("dense", 1, "tanh")], "mse", (16, 32), 256, "normal_regression"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
 }
 
@@ -339,7 +355,8 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     h.close()
 
 
-@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("mlp_bce_l2", 25)])
+@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("simple_rnn_small", 30),
+                                        ("mlp_bce_l2", 25)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
 def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
     spec, loss, in_shape, batch, kind = MODELS[name]
@@ -375,6 +392,7 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
           ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
           ("flatten",), ("dense", 10, "softmax")], "cce", (28, 28, 1), 100, "uniform_onehot"),
         ([("lstm", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),
+        ([("simple_rnn", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),   # the same shape, simple cell
     ]
     for spec, loss, in_shape, batch, kind in cases:
         rng = np.random.default_rng(20251125 + 2)
