@@ -56,7 +56,7 @@ enum {
 
 /* ---- layer list (models/layer/*.scala, flattened as layer/Composed.scala:89-99 does) ---- */
 enum { SN_LAYER_DENSE = 0, SN_LAYER_BIAS = 1, SN_LAYER_ACTIVATE = 2, SN_LAYER_FLATTEN = 3,
-       SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6, SN_LAYER_SIMPLE_RNN = 7 };
+       SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6, SN_LAYER_SIMPLE_RNN = 7, SN_LAYER_BATCHNORM = 8 };
 /* models/Activation.scala:32-83 */
 enum { SN_ACT_IDENTITY = 0, SN_ACT_SIGMOID = 1, SN_ACT_TANH = 2, SN_ACT_RELU = 3, SN_ACT_SOFTMAX = 4 };
 /* models/Loss.scala:18-57 */
@@ -90,6 +90,11 @@ typedef struct sn_layer_desc {
   int32_t reg_kind;      /* Dense/Bias: SN_REG_* */
   float reg_lambda;
   int32_t use_bias;      /* LSTM: per-gate bias vectors (layer/RNN.scala:215); SIMPLE_RNN: the cell's Bias (RNN.scala:116) */
+  float bn_momentum;     /* BATCHNORM (layer/BatchNorm.scala:64-76, axes = Seq(-1)): decay of the moving statistics */
+  float bn_epsilon;      /* BATCHNORM: added to the variance */
+  int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  Only the generic
+                            form (math/nn/AllKernels.scala:663-684) is built: whenever the reference would take
+                            FusedBatchNormV3 (rank-4 input unless fused = Some(false)) model creation fails. */
 } sn_layer_desc;
 
 /* An `Algorithm` case class (optimizers/Algorithm.scala:6-11).  Field use per kind:
@@ -121,6 +126,9 @@ typedef struct sn_param_info {
   int64_t size;                  /* number of elements */
   int32_t rank;
   int64_t dims[SN_MAX_RANK];
+  int32_t trainable;             /* 0: layer state (BatchNorm moving statistics, `ParamDef.trainable = false`): no gradient,
+                                    no optimizer state; the step replaces it with the layer's own update
+                                    (optimizers/Optimizer.scala:118-122,142-144) */
 } sn_param_info;
 
 /* ---------------------------------------------------------------- context / errors */
@@ -199,9 +207,15 @@ SN_API int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64
 SN_API int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host);
 /* `LossModel.grad` (models/Model.scala:107-111): gradients only, no update. */
 SN_API int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
-/* `model.result` (models/Model.scala:35-36): out_dev receives rows x output elements. */
+/* `model.result` (models/Model.scala:35-36) of the frozen model, the one `LossModel.trained` hands to
+ * `TrainedModel` (Model.scala:126-127): out_dev receives rows x output elements.  BatchNorm reads its
+ * moving statistics. */
 SN_API int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
-/* `LossModel.loss` (models/Model.scala:101-102). */
+/* Output of `model.resultStateful` (models/Model.scala:38-41) for the model as the optimizer compiles it:
+ * BatchNorm normalises with the statistics of these `rows`.  The next state it would return is not applied;
+ * only sn_step and the epoch calls move layer state. */
+SN_API int sn_forward_training(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
+/* `LossModel.loss` (models/Model.scala:101-102) of the frozen model. */
 SN_API int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
 /* Per-batch body of `estimators.accuracy` (estimators/package.scala:28-32): rows whose every
  * rounded (half to even) output equals the label. */

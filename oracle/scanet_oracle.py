@@ -18,12 +18,18 @@ What pins each part (see tests/test_oracle_golden.py):
   * max pool (same/valid, stride 1/2), max-pool grad with ties .... reference goldens + brute force
   * SimpleRNN and LSTM forward ................................... reference goldens
   * LSTM / conv / pool / softmax+CCE backward .................... float64 numerical gradients + torch autograd
+  * BatchNorm (generic form): training output, next moving
+    statistics, frozen output ................................... reference goldens
+  * BatchNorm backward through the batch statistics .............. float64 numerical gradients (rank 2 and rank 4)
   * decayingAvg / boost / sqrtZeroSafe ........................... reference goldens
   * optimizer trajectories ....................................... reference convergence thresholds + closed forms
 Parity unpinned (only running TensorFlow-CPU could pin them): last-ulp
 behaviour of TF's Exp/Tanh/Sigmoid/Log/Pow, summation order inside TF's
 MatMul/Conv2D/Sum, averaging of more than one replica and the multi-partition
-iteration counter (no reference test runs with more than one partition).
+iteration counter (no reference test runs with more than one partition), and
+the FusedBatchNormV3 form BatchNorm takes for rank-4 input unless `fused =
+Some(false)` (not restated: its saved-statistics outputs are wired by index in
+math/nn/AllKernels.scala:443-452 and no reference test holds values for it).
 """
 from __future__ import annotations
 
@@ -348,7 +354,7 @@ REG_NONE, REG_L1, REG_L2 = 0, 1, 2
 @dataclass
 class Layer:
     """One entry of the flattened layer list of `Composed` (layer/Composed.scala:89-99)."""
-    kind: str                       # dense | bias | activate | flatten | conv2d | pool2d | lstm | simple_rnn
+    kind: str                       # dense | bias | activate | flatten | conv2d | pool2d | lstm | simple_rnn | batchnorm
     units: int = 0
     activation: int = ACT_IDENTITY
     act_param: float = 0.0
@@ -359,6 +365,8 @@ class Layer:
     reg_lambda: float = 0.0
     bias: bool = True               # lstm / simple_rnn only
     rnn_activation: int = ACT_TANH  # simple_rnn cell activation / lstm `activation`
+    momentum: float = 0.99          # batchnorm (BatchNorm.scala:66-67)
+    epsilon: float = 1e-3
 
     # ---- parameter definitions, in flat-buffer order ---------------------- #
     def params(self, in_shape) -> List[Tuple[str, Tuple[int, ...]]]:
@@ -383,12 +391,15 @@ class Layer:
             if self.bias:
                 out.append(("1/weights", (h,)))
             return out
+        if self.kind == "batchnorm":    # BatchNorm.scala:80-98: normalised axis keeps its size, every other becomes 1
+            shape = (1,) * (len(in_shape) - 1) + (in_shape[-1],)
+            return [(name, shape) for name in BN_PARAMS]
         return []
 
     def out_shape(self, s):
         if self.kind == "dense":
             return (s[0], self.units)
-        if self.kind in ("bias", "activate"):
+        if self.kind in ("bias", "activate", "batchnorm"):
             return tuple(s)
         if self.kind == "flatten":      # Flatten.scala:12-18
             return (s[0], int(np.prod(s[1:])))
@@ -441,6 +452,66 @@ def SimpleRNN(units, activation=ACT_TANH, bias=True):
     return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation)]
 
 
+BN_PARAMS = ("beta", "gamma", "moving_mean", "moving_variance")   # BatchNorm.scala:92-97,170-173
+BN_STATE = ("moving_mean", "moving_variance")                      # not trainable: replaced by the layer, not by the optimizer
+
+
+def BatchNorm(momentum=0.99, epsilon=1e-3):
+    """`BatchNorm(axes = Seq(-1), fused = Some(false))` (BatchNorm.scala:64-76): the generic `batchNorm` form
+    (math/nn/AllKernels.scala:663-684).  The FusedBatchNormV3 form the layer picks for rank-4 input by default is
+    not restated here."""
+    return [Layer("batchnorm", momentum=momentum, epsilon=epsilon)]
+
+
+def is_state_path(path: str) -> bool:
+    """Parameters with `trainable = false` (ParamDef of MovingMean / MovingVariance, BatchNorm.scala:96-97)."""
+    return path.rsplit("/", 1)[-1] in BN_STATE
+
+
+def batchnorm_forward(x, params, pre, l: Layer, training: bool):
+    """math/nn/AllKernels.scala:663-684 in its op order; returns (y, cache, next_state).
+
+    training: moments over every axis but the last (alg/AllKernels.scala:505-513, biased variance);
+    frozen: the moving statistics.  next_state = decayingAvg(moving, batch, momentum) (BatchNorm.scala:146-149,
+    alg/AllKernels.scala:541-544), present only when training."""
+    dt = x.dtype
+    gamma, beta = params[pre + "gamma"], params[pre + "beta"]
+    axes = tuple(range(x.ndim - 1))
+    if training:
+        n = dt.type(np.prod([x.shape[a] for a in axes]))
+        mean = x.sum(axis=axes, keepdims=True, dtype=dt) / n
+        var = sqr(x - mean).sum(axis=axes, keepdims=True, dtype=dt) / n
+    else:
+        mean, var = params[pre + "moving_mean"], params[pre + "moving_variance"]
+    r = dt.type(1.0) / np.sqrt(var + dt.type(l.epsilon))
+    inv = r * gamma
+    y = ((x * inv) - (mean * inv)) + beta
+    nxt = {}
+    if training:
+        mom = dt.type(l.momentum)
+        nxt[pre + "moving_mean"] = mom * params[pre + "moving_mean"] + (dt.type(1.0) - mom) * mean
+        nxt[pre + "moving_variance"] = mom * params[pre + "moving_variance"] + (dt.type(1.0) - mom) * var
+    return y, (x, mean, r, gamma, training), nxt
+
+
+def batchnorm_backward(dy, cache, pre, grads):
+    """Reverse mode through `((x*inv) - (mean*inv)) + beta`, inv = rsqrt(var+eps)*gamma, with mean and var
+    functions of x when training."""
+    x, mean, r, gamma, training = cache
+    dt = dy.dtype
+    axes = tuple(range(x.ndim - 1))
+    xc = x - mean
+    s1 = dy.sum(axis=axes, keepdims=True, dtype=dt)
+    s2 = (dy * xc).sum(axis=axes, keepdims=True, dtype=dt)
+    grads[pre + "beta"] = s1
+    grads[pre + "gamma"] = s2 * r
+    inv = r * gamma
+    if not training:
+        return dy * inv
+    n = dt.type(np.prod([x.shape[a] for a in axes]))
+    return inv * (dy - s1 / n - xc * (r * r * s2 / n))
+
+
 class Model:
     """A `Composed` model: flattened layers, index-prefixed parameter paths (Composed.scala:22-31)."""
 
@@ -470,7 +541,10 @@ class Model:
         return s
 
     # ---- forward ---------------------------------------------------------- #
-    def forward(self, x, params: Dict[str, np.ndarray], cache: Optional[list] = None):
+    def forward(self, x, params: Dict[str, np.ndarray], cache: Optional[list] = None, training: bool = False,
+                next_state: Optional[dict] = None):
+        """training = the model as `Optimizer` compiles it; False = frozen, as `LossModel.trained` hands it to
+        `TrainedModel` (Model.scala:126-127).  Only stateful layers (BatchNorm) tell the two apart."""
         for i, l in enumerate(self.layers):
             pre = self._prefix(i)
             k = l.kind
@@ -500,6 +574,10 @@ class Model:
                 y, c = lstm_forward(x, params, pre, l)
             elif k == "simple_rnn":
                 y, c = simple_rnn_forward(x, params, pre, l)
+            elif k == "batchnorm":
+                y, c, nxt = batchnorm_forward(x, params, pre, l, training)
+                if next_state is not None:
+                    next_state.update(nxt)
             else:
                 raise ValueError(k)
             if cache is not None:
@@ -520,16 +598,22 @@ class Model:
                     total = total + dt.type(l.reg_lambda) * np.abs(w).sum(dtype=dt) / dt.type(2.0)
         return total
 
-    def loss_of(self, x, y, params):
+    def loss_of(self, x, y, params, training: bool = False):
         """LossModel.buildStateful (Model.scala:92-99): loss(model(x), y) + penalty."""
-        p = self.forward(x, params)
+        p = self.forward(x, params, training=training)
         return loss_value(self.loss, p, y) + self.penalty(params)
 
     # ---- backward: gradients w.r.t. every weight -------------------------- #
     def grad(self, x, y, params):
         """LossModel.grad (Model.scala:107-119): returns (loss, {path: gradient})."""
+        loss, grads, _ = self.grad_stateful(x, y, params)
+        return loss, grads
+
+    def grad_stateful(self, x, y, params):
+        """LossModel.gradStateful (Model.scala:113-119): (loss, {weight path: gradient}, {state path: next value})."""
         cache: list = []
-        p = self.forward(x, params, cache)
+        next_state: dict = {}
+        p = self.forward(x, params, cache, training=True, next_state=next_state)
         loss = loss_value(self.loss, p, y) + self.penalty(params)
         dy = np.ones_like(p) if self.loss == LOSS_IDENTITY else loss_grad(self.loss, p, y)
         grads: Dict[str, np.ndarray] = {}
@@ -559,6 +643,8 @@ class Model:
                 dy = lstm_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
             elif k == "simple_rnn":
                 dy = simple_rnn_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
+            elif k == "batchnorm":
+                dy = batchnorm_backward(dy, c, pre, grads)
             if l.kind in ("dense", "bias") and l.reg != REG_NONE:
                 w = params[pre + "weights"]
                 lam = w.dtype.type(l.reg_lambda)
@@ -566,7 +652,7 @@ class Model:
                     grads[pre + "weights"] = grads[pre + "weights"] + (w * w.dtype.type(2.0)) * (lam / w.dtype.type(2.0))
                 else:                     # Abs grad in the reference is |parent| (AllKernels.scala:330-335)
                     grads[pre + "weights"] = grads[pre + "weights"] + np.abs(np.ones_like(w) * (lam / w.dtype.type(2.0)))
-        return loss, grads
+        return loss, grads, next_state
 
 
 # --------------------------------------------------------------------------- #
@@ -807,9 +893,14 @@ def train_step(model: Model, alg: Algorithm, x, y, params, opt_state, it: int, m
     """`compileBackprop`'s function (Optimizer.scala:169-194): one update of every weight.
 
     Returns (new_params, new_opt_state, loss_before_update, grads)."""
-    loss, grads = model.grad(x, y, params)
+    loss, grads, next_state = model.grad_stateful(x, y, params)
     new_params, new_state = {}, {}
     for path, w in params.items():
+        if path in next_state:      # `nextWeights ++ nextState` (Optimizer.scala:142-144): state bypasses the algorithm
+            new_params[path] = next_state[path]
+            if path in opt_state:
+                new_state[path] = opt_state[path]
+            continue
         delta, st = alg.build(grads[path], opt_state[path], it)
         new_params[path] = w - delta if minimizing else w + delta    # Optimizer.scala:186
         new_state[path] = st
@@ -833,7 +924,7 @@ def optimize_on_partition(model, alg, X, Y, batch, global_iter, params, opt_stat
     for i in range(n_batches):
         xb, yb = X[i * batch:(i + 1) * batch], Y[i * batch:(i + 1) * batch]
         params, opt_state, _, _ = train_step(model, alg, xb, yb, params, opt_state, global_iter + i + 1)
-    loss = model.loss_of(xb, yb, params)
+    loss = model.loss_of(xb, yb, params, training=True)     # `lossModel.lossStateful`, not frozen (Optimizer.scala:148,163-167)
     return n_batches, params, opt_state, loss
 
 

@@ -17,7 +17,7 @@ SN_MAX_OPT_STATES = 3
 SN_MAX_AVG_INPUTS = 32
 
 # enums of include/scanet_hip.h
-LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM, LAYER_SIMPLE_RNN = range(8)
+LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM, LAYER_SIMPLE_RNN, LAYER_BATCHNORM = range(9)
 ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = range(5)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
 PAD_VALID, PAD_SAME = 0, 1
@@ -39,7 +39,8 @@ class ScanetError(RuntimeError):
 class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("units", C.c_int32), ("activation", C.c_int32), ("act_param", C.c_float),
                 ("kernel_h", C.c_int32), ("kernel_w", C.c_int32), ("stride_h", C.c_int32), ("stride_w", C.c_int32),
-                ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32)]
+                ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32),
+                ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float), ("bn_fused", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):
@@ -49,7 +50,7 @@ class OptimizerDesc(C.Structure):
 
 class ParamInfo(C.Structure):
     _fields_ = [("path", C.c_char * 96), ("offset", C.c_int64), ("size", C.c_int64), ("rank", C.c_int32),
-                ("dims", C.c_int64 * SN_MAX_RANK)]
+                ("dims", C.c_int64 * SN_MAX_RANK), ("trainable", C.c_int32)]
 
 
 _P = C.c_void_p
@@ -86,6 +87,7 @@ SIGNATURES = {
     "sn_step": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, _F]),
     "sn_grad": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_forward": (C.c_int, [_P, _P, C.c_int32, _P]),
+    "sn_forward_training": (C.c_int, [_P, _P, C.c_int32, _P]),
     "sn_loss": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_count_correct": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64)]),
     "sn_train_epoch": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), _F]),

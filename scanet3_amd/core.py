@@ -155,10 +155,13 @@ class CompiledModel:
         check(lib.sn_model_param_count(h, C.byref(n), C.byref(flat)))
         self.flat_elems = flat.value
         self.params: List[Tuple[str, Tuple[int, ...], int]] = []     # (path, shape, offset)
+        self.state_paths = set()     # layer state (`trainable = false`): no gradient, no optimizer state
         for i in range(n.value):
             info = L.ParamInfo()
             check(lib.sn_model_param_info(h, i, C.byref(info)))
             self.params.append((info.path.decode(), tuple(info.dims[:info.rank]), info.offset))
+            if not info.trainable:
+                self.state_paths.add(info.path.decode())
         rank, odims = C.c_int32(), (C.c_int64 * L.SN_MAX_RANK)()
         check(lib.sn_model_output_shape(h, C.byref(rank), odims))
         self.output_shape = tuple(odims[:rank.value])
@@ -205,9 +208,11 @@ class Replica:
             a = _f32c(value)
             check(lib.sn_params_set(self.handle, self.model.index[path], a.ctypes.data_as(C.c_void_p), a.size))
 
-    def _get(self, fn, *lead) -> Dict[str, np.ndarray]:
+    def _get(self, fn, *lead, weights_only: bool = False) -> Dict[str, np.ndarray]:
         out = {}
         for i, (path, shape, _) in enumerate(self.model.params):
+            if weights_only and path in self.model.state_paths:
+                continue
             a = np.empty(int(np.prod(shape)) if shape else 1, np.float32)
             check(fn(self.handle, i, *lead, a.ctypes.data_as(C.c_void_p), a.size))
             out[path] = a.reshape(shape)
@@ -217,10 +222,10 @@ class Replica:
         return self._get(lib.sn_params_get)
 
     def get_grads(self) -> Dict[str, np.ndarray]:
-        return self._get(lib.sn_grads_get)
+        return self._get(lib.sn_grads_get, weights_only=True)
 
     def get_opt_state(self, slot: int) -> Dict[str, np.ndarray]:
-        return self._get(lib.sn_optstate_get, slot)
+        return self._get(lib.sn_optstate_get, slot, weights_only=True)
 
     def set_opt_state(self, slot: int, values: Dict[str, np.ndarray]):
         for path, value in values.items():
@@ -248,11 +253,12 @@ class Replica:
         check(lib.sn_grad(self.handle, self._ptr(x), self._ptr(y), self.model.batch if rows is None else rows, C.byref(loss)))
         return loss.value
 
-    def forward(self, x, rows: Optional[int] = None) -> np.ndarray:
+    def forward(self, x, rows: Optional[int] = None, training: bool = False) -> np.ndarray:
+        """training=False: the frozen model (`TrainedModel.result`); True: `model.resultStateful`'s output."""
         rows = self.model.batch if rows is None else rows
         out = DeviceBuffer(self.ctx, rows * self.model.out_elems, (rows,) + self.model.output_shape)
         try:
-            check(lib.sn_forward(self.handle, self._ptr(x), rows, out.ptr))
+            check((lib.sn_forward_training if training else lib.sn_forward)(self.handle, self._ptr(x), rows, out.ptr))
             return out.numpy()
         finally:
             out.free()

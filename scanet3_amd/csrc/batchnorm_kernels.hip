@@ -1,0 +1,286 @@
+// Batch normalisation over the last axis of a channels-last tensor viewed as [rows, C]
+// (generic `batchNorm`, math/nn/AllKernels.scala:663-684, as the BatchNorm layer calls it for
+// `axes = Seq(-1)`, models/layer/BatchNorm.scala:123-143).
+//
+//   training:  mean = sum(x)/rows, var = sum((x-mean)^2)/rows   (alg/AllKernels.scala:505-513)
+//   frozen:    mean, var = the moving statistics
+//   inv = rsqrt(var + eps) * gamma;  y = (x*inv - mean*inv) + beta
+//
+// All of it is memory bound: every pass reads the activation once with 8 row-loads in flight per
+// lane; the per-channel reductions are cut into row slices so the grid covers the chip, and the
+// slices are added in slice order by one thread per channel (deterministic, no atomics).
+#include "common.hpp"
+
+namespace sn {
+namespace {
+
+typedef float bn_f4 __attribute__((ext_vector_type(4)));
+
+enum { BN_SUM = 0, BN_SQDIFF = 1, BN_GRAD = 2 };
+
+// Block = 64 columns x 4 waves; wave w takes rows r0+w, r0+w+4, ... of its slice.
+// BN_SUM:    part0 = sum x
+// BN_SQDIFF: part0 = sum (x - mean)^2
+// BN_GRAD:   part0 = sum dy, part1 = sum dy * (x - mean)
+template <int MODE>
+__global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                         const float* __restrict__ mean, float* __restrict__ part0,
+                                                         float* __restrict__ part1, int64_t rows, int cols, int64_t rows_per_slice) {
+  __shared__ float smem[2][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_slice;
+  const int64_t r1 = r0 + rows_per_slice < rows ? r0 + rows_per_slice : rows;
+  float s0 = 0.f, s1 = 0.f;
+  if (c < cols) {
+    const float m = MODE == BN_SUM ? 0.f : mean[c];
+    int64_t r = r0 + wave;
+    for (; r + 28 < r1; r += 32) {
+      float a[8], b[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) a[u] = x[(r + 4 * u) * cols + c];
+      if (MODE == BN_GRAD) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) b[u] = dy[(r + 4 * u) * cols + c];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (MODE == BN_SUM) s0 += a[u];
+        if (MODE == BN_SQDIFF) { const float d = a[u] - m; s0 += d * d; }
+        if (MODE == BN_GRAD) { s0 += b[u]; s1 += b[u] * (a[u] - m); }
+      }
+    }
+    for (; r < r1; r += 4) {
+      const float a = x[r * cols + c];
+      if (MODE == BN_SUM) s0 += a;
+      if (MODE == BN_SQDIFF) { const float d = a - m; s0 += d * d; }
+      if (MODE == BN_GRAD) { const float b = dy[r * cols + c]; s0 += b; s1 += b * (a - m); }
+    }
+  }
+  smem[0][wave][lane] = s0;
+  if (MODE == BN_GRAD) smem[1][wave][lane] = s1;
+  __syncthreads();
+  if (wave == 0 && c < cols) {
+    part0[(int64_t)blockIdx.y * cols + c] = ((smem[0][0][lane] + smem[0][1][lane]) + smem[0][2][lane]) + smem[0][3][lane];
+    if (MODE == BN_GRAD)
+      part1[(int64_t)blockIdx.y * cols + c] = ((smem[1][0][lane] + smem[1][1][lane]) + smem[1][2][lane]) + smem[1][3][lane];
+  }
+}
+
+__device__ __forceinline__ float add_slices(const float* __restrict__ part, int slices, int cols, int c) {
+  float s = 0.f;
+  int i = 0;
+  for (; i + 4 <= slices; i += 4) {  // four loads in flight, added in slice order
+    const float a = part[(int64_t)i * cols + c], b = part[(int64_t)(i + 1) * cols + c], d = part[(int64_t)(i + 2) * cols + c],
+                e = part[(int64_t)(i + 3) * cols + c];
+    s = (((s + a) + b) + d) + e;
+  }
+  for (; i < slices; ++i) s += part[(int64_t)i * cols + c];
+  return s;
+}
+
+// One thread per channel.
+__global__ __launch_bounds__(256) void bn_mean_kernel(const float* __restrict__ part, int slices, int cols, float n, float* __restrict__ mean) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c < cols) mean[c] = add_slices(part, slices, cols, c) / n;
+}
+
+// var from the slices (training) or from the moving variance (part == null), then r = 1/sqrt(var+eps), inv = r*gamma
+__global__ __launch_bounds__(256) void bn_scale_kernel(const float* __restrict__ part, int slices, int cols, float n, float eps,
+                                                        const float* __restrict__ gamma, const float* __restrict__ moving_mean,
+                                                        const float* __restrict__ moving_var, float* __restrict__ mean,
+                                                        float* __restrict__ var, float* __restrict__ r, float* __restrict__ inv) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  float v;
+  if (part) {
+    v = add_slices(part, slices, cols, c) / n;
+  } else {
+    v = moving_var[c];
+    mean[c] = moving_mean[c];
+  }
+  var[c] = v;
+  const float rr = 1.0f / sqrtf(v + eps);
+  r[c] = rr;
+  inv[c] = rr * gamma[c];
+}
+
+template <bool V4>
+__global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__ x, const float* __restrict__ mean,
+                                                        const float* __restrict__ inv, const float* __restrict__ beta,
+                                                        float* __restrict__ y, int64_t n, int cols) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  if (V4) {
+    const int64_t n4 = n / 4;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+      const int c = (int)((i * 4) % cols);
+      const bn_f4 xv = *(const bn_f4*)(x + i * 4), iv = *(const bn_f4*)(inv + c), mv = *(const bn_f4*)(mean + c), bv = *(const bn_f4*)(beta + c);
+      bn_f4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (xv[e] * iv[e] - mv[e] * iv[e]) + bv[e];
+      *(bn_f4*)(y + i * 4) = o;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+      const int c = (int)(i % cols);
+      y[i] = (x[i] * inv[c] - mean[c] * inv[c]) + beta[c];
+    }
+  }
+}
+
+// d beta = S1, d gamma = S2 * r; k1 = S1/n, k2 = r*r*S2/n for the input gradient
+__global__ __launch_bounds__(256) void bn_grad_finish_kernel(const float* __restrict__ part0, const float* __restrict__ part1, int slices,
+                                                              int cols, float n, const float* __restrict__ r, float* __restrict__ dbeta,
+                                                              float* __restrict__ dgamma, float* __restrict__ k1, float* __restrict__ k2) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  const float s1 = add_slices(part0, slices, cols, c), s2 = add_slices(part1, slices, cols, c);
+  const float rr = r[c];
+  dbeta[c] = s1;
+  dgamma[c] = s2 * rr;
+  k1[c] = s1 / n;
+  k2[c] = rr * rr * s2 / n;
+}
+
+// dx = inv * (dy - k1 - (x - mean) * k2)
+template <bool V4>
+__global__ __launch_bounds__(256) void bn_dx_kernel(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ mean,
+                                                     const float* __restrict__ inv, const float* __restrict__ k1,
+                                                     const float* __restrict__ k2, float* __restrict__ dx, int64_t n, int cols) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  if (V4) {
+    const int64_t n4 = n / 4;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
+      const int c = (int)((i * 4) % cols);
+      const bn_f4 xv = *(const bn_f4*)(x + i * 4), gv = *(const bn_f4*)(dy + i * 4), iv = *(const bn_f4*)(inv + c),
+                  mv = *(const bn_f4*)(mean + c), a = *(const bn_f4*)(k1 + c), b = *(const bn_f4*)(k2 + c);
+      bn_f4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = iv[e] * ((gv[e] - a[e]) - (xv[e] - mv[e]) * b[e]);
+      *(bn_f4*)(dx + i * 4) = o;
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+      const int c = (int)(i % cols);
+      dx[i] = inv[c] * ((dy[i] - k1[c]) - (x[i] - mean[c]) * k2[c]);
+    }
+  }
+}
+
+// decayingAvg (alg/AllKernels.scala:541-544): moving = momentum*moving + (1-momentum)*batch
+__global__ __launch_bounds__(256) void bn_moving_kernel(float* __restrict__ moving_mean, float* __restrict__ moving_var,
+                                                         const float* __restrict__ mean, const float* __restrict__ var, int cols, float momentum) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  const float keep = 1.0f - momentum;
+  moving_mean[c] = momentum * moving_mean[c] + keep * mean[c];
+  moving_var[c] = momentum * moving_var[c] + keep * var[c];
+}
+
+unsigned grid_for(const sn_ctx* ctx, int64_t n, int per_block) {
+  int64_t blocks = ceil_div(n, per_block);
+  const int64_t cap = (int64_t)ctx->compute_units * 16;
+  if (blocks > cap) blocks = cap;
+  return blocks < 1 ? 1u : (unsigned)blocks;
+}
+
+int slices_for(const sn_ctx* ctx, int64_t rows, int cols) {
+  const int64_t col_blocks = ceil_div((int64_t)cols, (int64_t)64);
+  int64_t s = ceil_div((int64_t)ctx->compute_units * 4, col_blocks);
+  const int64_t by_rows = ceil_div(rows, (int64_t)64);  // at least 64 rows (16 per wave) in a slice
+  if (s > by_rows) s = by_rows;
+  if (s > 1024) s = 1024;
+  return s < 1 ? 1 : (int)s;
+}
+
+bool vec4_ok(int cols, std::initializer_list<const void*> ptrs) {
+  if (cols % 4 != 0) return false;
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15u) return false;
+  return true;
+}
+
+}  // namespace
+
+int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols) { return (int64_t)2 * slices_for(ctx, rows, cols) * cols; }
+
+int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, int cols, const BatchNormArgs& a, bool training, float* ws,
+                         int64_t ws_elems) {
+  if (rows <= 0 || cols <= 0) return SN_OK;
+  SN_REQUIRE(rows * cols <= (int64_t)INT32_MAX * 4, "batch norm over %lld elements exceeds one launch", (long long)(rows * cols));
+  const int cb = (int)ceil_div((int64_t)cols, (int64_t)256);
+  if (training) {
+    const int s = slices_for(ctx, rows, cols);
+    SN_REQUIRE((int64_t)s * cols <= ws_elems, "batch norm needs %lld workspace elements, %lld given", (long long)s * cols, (long long)ws_elems);
+    const int64_t per = ceil_div(rows, (int64_t)s);
+    const dim3 grid((unsigned)ceil_div((int64_t)cols, (int64_t)64), (unsigned)s);
+    {
+      LaunchScope scope(ctx, "batchnorm_mean");
+      hipLaunchKernelGGL((bn_reduce_kernel<BN_SUM>), grid, dim3(256), 0, ctx->stream, x, (const float*)nullptr, (const float*)nullptr, ws,
+                         (float*)nullptr, rows, cols, per);
+      hipLaunchKernelGGL(bn_mean_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, s, cols, (float)rows, a.mean);
+    }
+    {
+      LaunchScope scope(ctx, "batchnorm_variance");
+      hipLaunchKernelGGL((bn_reduce_kernel<BN_SQDIFF>), grid, dim3(256), 0, ctx->stream, x, (const float*)nullptr, (const float*)a.mean, ws,
+                         (float*)nullptr, rows, cols, per);
+      hipLaunchKernelGGL(bn_scale_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, s, cols, (float)rows, a.epsilon, a.gamma,
+                         (const float*)nullptr, (const float*)nullptr, a.mean, a.var, a.r, a.inv);
+    }
+  } else {
+    LaunchScope scope(ctx, "batchnorm_frozen_scale");
+    hipLaunchKernelGGL(bn_scale_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)nullptr, 0, cols, 1.0f, a.epsilon, a.gamma,
+                       a.moving_mean, a.moving_var, a.mean, a.var, a.r, a.inv);
+  }
+  const int64_t n = rows * cols;
+  LaunchScope scope(ctx, "batchnorm_apply");
+  if (vec4_ok(cols, {x, y, a.mean, a.inv, a.beta}))
+    hipLaunchKernelGGL((bn_apply_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, (const float*)a.mean,
+                       (const float*)a.inv, a.beta, y, n, cols);
+  else
+    hipLaunchKernelGGL((bn_apply_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, (const float*)a.mean,
+                       (const float*)a.inv, a.beta, y, n, cols);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx, int64_t rows, int cols, const BatchNormArgs& a,
+                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems) {
+  if (rows <= 0 || cols <= 0) return SN_OK;
+  const int s = slices_for(ctx, rows, cols);
+  SN_REQUIRE((int64_t)2 * s * cols <= ws_elems, "batch norm gradient needs %lld workspace elements, %lld given", (long long)2 * s * cols,
+             (long long)ws_elems);
+  const int64_t per = ceil_div(rows, (int64_t)s);
+  const int cb = (int)ceil_div((int64_t)cols, (int64_t)256);
+  float* part1 = ws + (int64_t)s * cols;
+  {
+    LaunchScope scope(ctx, "batchnorm_gradient_sums");
+    hipLaunchKernelGGL((bn_reduce_kernel<BN_GRAD>), dim3((unsigned)ceil_div((int64_t)cols, (int64_t)64), (unsigned)s), dim3(256), 0,
+                       ctx->stream, x, dy, (const float*)a.mean, ws, part1, rows, cols, per);
+    hipLaunchKernelGGL(bn_grad_finish_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, (const float*)part1, s, cols,
+                       (float)rows, (const float*)a.r, dbeta, dgamma, a.k1, a.k2);
+  }
+  if (dx) {
+    const int64_t n = rows * cols;
+    LaunchScope scope(ctx, "batchnorm_input_gradient");
+    if (vec4_ok(cols, {x, dy, dx, a.mean, a.inv, a.k1, a.k2}))
+      hipLaunchKernelGGL((bn_dx_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
+                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols);
+    else
+      hipLaunchKernelGGL((bn_dx_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
+                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_batchnorm_moving(sn_ctx* ctx, const BatchNormArgs& a, float* moving_mean, float* moving_var, int cols) {
+  if (cols <= 0) return SN_OK;
+  LaunchScope scope(ctx, "batchnorm_moving_statistics");
+  hipLaunchKernelGGL(bn_moving_kernel, dim3((unsigned)ceil_div((int64_t)cols, (int64_t)256)), dim3(256), 0, ctx->stream, moving_mean,
+                     moving_var, (const float*)a.mean, (const float*)a.var, cols, a.momentum);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+}  // namespace sn

@@ -160,6 +160,31 @@ struct LstmGateBwdArgs {
 };
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
 
+// ---- batch normalisation over the last axis (batchnorm_kernels.hip) ---------------------
+struct BatchNormArgs {
+  const float* gamma;        // [C]
+  const float* beta;         // [C]
+  const float* moving_mean;  // [C], read by the frozen form
+  const float* moving_var;
+  float* mean;               // [C] statistics the output was built from (batch or moving), kept for the gradient
+  float* var;
+  float* r;                  // 1/sqrt(var + epsilon)
+  float* inv;                // r * gamma
+  float* k1;                 // [C] scratch of the gradient
+  float* k2;
+  float epsilon, momentum;
+};
+// workspace (elements) the reductions need for a [rows, cols] activation
+int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols);
+// y = (x*inv - mean*inv) + beta; training: batch statistics, else the moving ones
+int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, int cols, const BatchNormArgs& a, bool training, float* ws,
+                         int64_t ws_elems);
+// gradients of beta, gamma and (dx != null) the input, through the batch statistics
+int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx, int64_t rows, int cols, const BatchNormArgs& a,
+                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems);
+// moving = momentum*moving + (1-momentum)*batch
+int launch_batchnorm_moving(sn_ctx* ctx, const BatchNormArgs& a, float* moving_mean, float* moving_var, int cols);
+
 // ---- GEMM family (gemm_kernels.hip) ----------------------------------------------------
 struct Epilogue {
   float* out = nullptr;

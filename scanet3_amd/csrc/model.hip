@@ -14,7 +14,7 @@
 
 namespace sn {
 
-enum OpKind { OP_DENSE, OP_CONV, OP_POOL, OP_FLATTEN, OP_BIASACT, OP_SOFTMAX, OP_LSTM, OP_SRNN };
+enum OpKind { OP_DENSE, OP_CONV, OP_POOL, OP_FLATTEN, OP_BIASACT, OP_SOFTMAX, OP_LSTM, OP_SRNN, OP_BATCHNORM };
 
 struct ParamDef {
   sn_param_info info;
@@ -34,6 +34,9 @@ struct Op {
   // lstm
   int T = 0, F = 0, H = 0;
   int lstm_p[4][3] = {{-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}};  // gate x {kernel, recurrent, bias}
+  // batch norm: beta, gamma, moving mean, moving variance
+  int bn_p[4] = {-1, -1, -1, -1};
+  float bn_momentum = 0.99f, bn_epsilon = 1e-3f;
   // buffers (indices into replica buffer table), assigned at replica creation
   int out_buf = -1;
 };
@@ -51,6 +54,7 @@ struct sn_model {
   std::vector<sn::Op> ops;
   std::vector<sn::ParamDef> params;
   int64_t flat_elems;  // padded length of the flat parameter buffer
+  std::vector<std::pair<int64_t, int64_t>> trainable_runs;  // [begin, end) element ranges the optimizer updates
   std::vector<int64_t> out_dims;
   int64_t out_elems;
   int64_t max_act_elems;   // per sample, over every op input/output
@@ -83,6 +87,7 @@ struct sn_replica {
   float* lstm_dc = nullptr;
   // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
   std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
+  std::vector<float*> bn_buf;  // per batch-norm op: mean, var, 1/sqrt(var+eps), scale, two gradient vectors
   float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
   bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
   // host-fed epochs: two device slots per tensor, a copy stream, "slot filled" / "slot consumed" events
@@ -122,9 +127,11 @@ static void conv_out(int padding, int in, int k, int s, int* out, int* pad_befor
   }
 }
 
-static int add_param(sn_model* m, const std::string& path, const std::vector<int64_t>& dims, int reg_kind, float reg_lambda) {
+static int add_param(sn_model* m, const std::string& path, const std::vector<int64_t>& dims, int reg_kind, float reg_lambda,
+                     bool trainable = true) {
   ParamDef p;
   memset(&p.info, 0, sizeof(p.info));
+  p.info.trainable = trainable ? 1 : 0;
   snprintf(p.info.path, sizeof(p.info.path), "%s", path.c_str());
   p.info.rank = (int32_t)dims.size();
   p.info.size = 1;
@@ -279,6 +286,26 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ++i;
         break;
       }
+      case SN_LAYER_BATCHNORM: {
+        // BatchNorm(axes = Seq(-1)) in its generic form (layer/BatchNorm.scala:123-143, math/nn/AllKernels.scala:663-684)
+        SN_REQUIRE(cur.size() >= 1, "layer %d: rank should be >= 2", i);
+        SN_REQUIRE(L.bn_fused >= -1 && L.bn_fused <= 1, "layer %d: fused must be -1 (None), 0 or 1", i);
+        const bool wants_fused = cur.size() == 3 && L.bn_fused != 0;  // BatchNorm.scala:100-107,118-121
+        SN_REQUIRE(!wants_fused, "layer %d: the FusedBatchNormV3 form of BatchNorm is not built; pass fused = Some(false)", i);
+        SN_REQUIRE(L.bn_fused != 1, "layer %d: Cannot use fused implementation with this input rank", i);  // BatchNorm.scala:134-136
+        SN_REQUIRE(L.bn_epsilon > 0.f, "layer %d: epsilon must be positive", i);
+        op.kind = OP_BATCHNORM;
+        op.bn_momentum = L.bn_momentum;
+        op.bn_epsilon = L.bn_epsilon;
+        op.out_dims = cur;
+        std::vector<int64_t> shape(cur.size() + 1, 1);  // every axis but the normalised one becomes 1 (BatchNorm.scala:80-88)
+        shape.back() = cur.back();
+        static const char* names[4] = {"beta", "gamma", "moving_mean", "moving_variance"};  // BatchNorm.scala:92-97,170-173
+        for (int k = 0; k < 4; ++k) op.bn_p[k] = add_param(m, prefix(i) + names[k], shape, SN_REG_NONE, 0.f, k < 2);
+        ws = std::max(ws, batchnorm_workspace_elems(m->ctx, (int64_t)B * (prod(cur) / cur.back()), (int)cur.back()));
+        ++i;
+        break;
+      }
       case SN_LAYER_SIMPLE_RNN: {
         // RNN(SimpleRNNCell ?>> Bias ?>> activation), layer/RNN.scala:113-163; one "gate" whose weights use slot 0
         SN_REQUIRE(cur.size() == 2, "layer %d: RNN requires input to have Shape(batch, time, features)", i);
@@ -310,6 +337,13 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
   m->out_dims = cur;
   m->out_elems = prod(cur);
   m->max_act_elems = max_act;
+  // runs of trainable tensors in the flat buffer (padding included): what one optimizer launch covers
+  for (const ParamDef& p : m->params) {
+    if (!p.info.trainable) continue;
+    const int64_t end = p.info.offset + align_up(p.info.size, 64);
+    if (!m->trainable_runs.empty() && m->trainable_runs.back().second == p.info.offset) m->trainable_runs.back().second = end;
+    else m->trainable_runs.push_back({p.info.offset, end});
+  }
   // column sums over many rows use the workspace too
   ws = std::max<int64_t>(ws, (int64_t)cu * 4 * 64 * 4);
   m->workspace_elems = ws;
@@ -366,6 +400,7 @@ static int alloc_replica(sn_replica* r) {
   r->lstm_dz.assign(n_ops, nullptr);
   r->lstm_pk_fwd.assign(n_ops, nullptr);
   r->lstm_pk_dh.assign(n_ops, nullptr);
+  r->bn_buf.assign(n_ops, nullptr);
   r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
   r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
   int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0;
@@ -386,6 +421,7 @@ static int alloc_replica(sn_replica* r) {
       continue;  // output = last slice of lstm_h
     }
     SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
+    if (op.kind == OP_BATCHNORM) SN_TRY(dev_alloc(r, &r->bn_buf[i], 6 * align_up(op.out_dims.back(), 64)));
     if (op.kind == OP_SRNN) {  // the carried state of every step and its gradient, time-major like the LSTM's
       const int64_t bh = B * op.H;
       SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = the initial state
@@ -437,8 +473,17 @@ static LstmWeights lstm_weights(sn_replica* r, const Op& op, float* base) {
   return w;
 }
 
+static BatchNormArgs batchnorm_args(sn_replica* r, const Op& op, int i) {
+  const int64_t c = align_up(op.out_dims.back(), 64);
+  float* b = r->bn_buf[i];
+  return BatchNormArgs{param_ptr(r, r->w, op.bn_p[1]), param_ptr(r, r->w, op.bn_p[0]), param_ptr(r, r->w, op.bn_p[2]),
+                       param_ptr(r, r->w, op.bn_p[3]), b, b + c, b + 2 * c, b + 3 * c, b + 4 * c, b + 5 * c, op.bn_epsilon, op.bn_momentum};
+}
+
 // skip_last: leave out the last op (the training pass fuses a Softmax output into the loss kernel)
-static int forward(sn_replica* r, const float* x, int rows, bool skip_last = false) {
+// training: the model as the optimizer compiles it; false = frozen, as a trained model predicts (models/Model.scala:126-127).
+//           Only batch normalisation tells the two apart.
+static int forward(sn_replica* r, const float* x, int rows, bool skip_last = false, bool training = false) {
   sn_model* m = r->model;
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
@@ -518,6 +563,12 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
                          r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
           SN_TRY(launch_lstm_gates_fwd(ctx, a, rows, op.H));
         }
+        break;
+      }
+      case OP_BATCHNORM: {
+        const int c = (int)op.out_dims.back();
+        SN_TRY(launch_batchnorm_fwd(ctx, in, r->act[i], (int64_t)rows * (op.out_elems / c), c, batchnorm_args(r, op, (int)i), training, r->ws,
+                                    m->workspace_elems));
         break;
       }
       case OP_SRNN: {
@@ -684,6 +735,13 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         if (need_dx) cur ^= 1;
         break;
       }
+      case OP_BATCHNORM: {
+        const int c = (int)op.out_dims.back();
+        SN_TRY(launch_batchnorm_bwd(ctx, in, dy, need_dx ? dx : nullptr, (int64_t)rows * (op.out_elems / c), c, batchnorm_args(r, op, i),
+                                    param_ptr(r, r->g, op.bn_p[0]), param_ptr(r, r->g, op.bn_p[1]), r->ws, m->workspace_elems));
+        if (need_dx) cur ^= 1;
+        break;
+      }
       case OP_SRNN: {
         SN_REQUIRE(rows == m->batch, "RNN training needs rows == batch (%d), got %d", m->batch, rows);
         const int64_t bh = (int64_t)m->batch * op.H;
@@ -729,13 +787,13 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
   const int last = (int)m->ops.size() - 1;
   if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
     // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
-    SN_TRY(forward(r, x, rows, true));
+    SN_TRY(forward(r, x, rows, true, true));
     SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], r->loss_dev, r->loss_partials, rows,
                               (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
     SN_TRY(add_penalties(r));
     return backward(r, x, rows, last - 1, 1);
   }
-  SN_TRY(forward(r, x, rows));
+  SN_TRY(forward(r, x, rows, false, true));
   const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);
   SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0]));
   SN_TRY(backward(r, x, rows));
@@ -745,13 +803,24 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
 static int update(sn_replica* r, int iter) {
   SN_REQUIRE(r->has_opt, "replica was created without an optimizer");
   r->bf_weights_stale = true;
-  return launch_optimizer(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], r->model->flat_elems, iter);
+  sn_model* m = r->model;
+  // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
+  // the statistics are those of the gradient pass that has just run
+  for (const auto& run : m->trainable_runs)
+    SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,
+                            r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter));
+  for (size_t i = 0; i < m->ops.size(); ++i)
+    if (m->ops[i].kind == OP_BATCHNORM)
+      SN_TRY(launch_batchnorm_moving(r->ctx, batchnorm_args(r, m->ops[i], (int)i), param_ptr(r, r->w, m->ops[i].bn_p[2]),
+                                     param_ptr(r, r->w, m->ops[i].bn_p[3]), (int)m->ops[i].out_dims.back()));
+  return SN_OK;
 }
 
-static int tensor_io(sn_replica* r, float* base, int index, float* host, const float* src, int64_t n) {
+static int tensor_io(sn_replica* r, float* base, int index, float* host, const float* src, int64_t n, bool weights_only = false) {
   sn_model* m = r->model;
   SN_REQUIRE(index >= 0 && index < (int)m->params.size(), "parameter index %d out of range (model has %zu)", index, m->params.size());
   const sn_param_info& p = m->params[index].info;
+  SN_REQUIRE(!weights_only || p.trainable, "%s is layer state: it has no gradient and no optimizer state", p.path);
   SN_REQUIRE(n == p.size, "parameter %s holds %lld elements, caller passed %lld", p.path, (long long)p.size, (long long)n);
   SN_REQUIRE(base != nullptr, "replica has no such buffer");
   if (src) {
@@ -899,18 +968,18 @@ int sn_optstate_set(sn_replica* rep, int32_t index, int32_t slot, const float* s
   SN_TRY(check_replica(rep));
   SN_REQUIRE(src_host != nullptr, "sn_optstate_set: source is NULL");
   SN_REQUIRE(slot >= 0 && slot < rep->n_states, "optimizer has %d state tensors per weight, slot %d asked", rep->n_states, slot);
-  return tensor_io(rep, rep->s[slot], index, nullptr, src_host, n);
+  return tensor_io(rep, rep->s[slot], index, nullptr, src_host, n, true);
 }
 int sn_optstate_get(sn_replica* rep, int32_t index, int32_t slot, float* dst_host, int64_t n) {
   SN_TRY(check_replica(rep));
   SN_REQUIRE(dst_host != nullptr, "sn_optstate_get: destination is NULL");
   SN_REQUIRE(slot >= 0 && slot < rep->n_states, "optimizer has %d state tensors per weight, slot %d asked", rep->n_states, slot);
-  return tensor_io(rep, rep->s[slot], index, dst_host, nullptr, n);
+  return tensor_io(rep, rep->s[slot], index, dst_host, nullptr, n, true);
 }
 int sn_grads_get(sn_replica* rep, int32_t index, float* dst_host, int64_t n) {
   SN_TRY(check_replica(rep));
   SN_REQUIRE(dst_host != nullptr, "sn_grads_get: destination is NULL");
-  return tensor_io(rep, rep->g, index, dst_host, nullptr, n);
+  return tensor_io(rep, rep->g, index, dst_host, nullptr, n, true);
 }
 
 int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64_t* n) {
@@ -942,14 +1011,18 @@ int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   return read_loss(rep, loss_host);
 }
 
-int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) {
+static int forward_to(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev, bool training) {
   SN_TRY(check_replica(rep));
   SN_REQUIRE(x_dev && out_dev, "sn_forward: null pointer");
   SN_TRY(check_rows(rep, rows));
-  SN_TRY(forward(rep, x_dev, rows));
+  SN_TRY(forward(rep, x_dev, rows, false, training));
   const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
   SN_HIP(hipMemcpyAsync(out_dev, pred, (size_t)rows * rep->model->out_elems * sizeof(float), hipMemcpyDeviceToDevice, rep->ctx->stream));
   return SN_OK;
+}
+int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) { return forward_to(rep, x_dev, rows, out_dev, false); }
+int sn_forward_training(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) {
+  return forward_to(rep, x_dev, rows, out_dev, true);
 }
 
 int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host) {
@@ -996,7 +1069,7 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
   if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
     const float* xl = x_dev + (n_batches - 1) * xs;
     const float* yl = y_dev + (n_batches - 1) * ys;
-    SN_TRY(forward(rep, xl, batch));
+    SN_TRY(forward(rep, xl, batch, false, true));  // `lossModel.lossStateful`: not frozen (Optimizer.scala:163-167)
     const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, xl, batch);
     SN_TRY(loss_of(rep, pred, yl, batch, nullptr));
     SN_TRY(read_loss(rep, loss_host));
@@ -1051,7 +1124,7 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
   if (iterations_host) *iterations_host = (int32_t)n_batches;
   const int last = (int)((n_batches - 1) & 1);
   if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
-    SN_TRY(forward(rep, rep->stage_x[last], batch));
+    SN_TRY(forward(rep, rep->stage_x[last], batch, false, true));
     const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, rep->stage_x[last], batch);
     SN_TRY(loss_of(rep, pred, rep->stage_y[last], batch, nullptr));
     SN_TRY(read_loss(rep, loss_host));

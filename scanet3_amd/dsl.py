@@ -163,6 +163,9 @@ class Layer:
     reg: Regularization = Zero
     use_bias: bool = True
     inits: Tuple[Initializer, ...] = ()
+    momentum: float = 0.99        # BatchNorm only
+    epsilon: float = 1e-3
+    fused: int = -1               # BatchNorm `fused`: -1 None, 0 Some(false), 1 Some(true)
 
     def __rshift__(self, other):
         return Composed.of(self, other)
@@ -173,7 +176,8 @@ class Layer:
 
     def desc(self) -> L.LayerDesc:
         return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
-                           self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0)
+                           self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
+                           self.momentum, self.epsilon, self.fused)
 
     def __repr__(self):
         return self.text
@@ -245,6 +249,18 @@ def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotU
     return Layer(L.LAYER_LSTM, f"RNN(LSTMCell({units},Tanh,Sigmoid,{'true' if bias else 'false'}))", units=units,
                  activation=Tanh, use_bias=bias,
                  inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
+
+
+def BatchNorm(axes: Sequence[int] = (-1,), momentum: float = 0.99, epsilon: float = 1e-3, betaInitializer: Initializer = Zeros,
+              gammaInitializer: Initializer = Ones, movingMeanInitializer: Initializer = Zeros,
+              movingVarianceInitializer: Initializer = Ones, fused: Optional[bool] = None) -> Layer:
+    """layer/BatchNorm.scala:64-76 over the last axis.  Only the generic form is built: for rank-4 input the
+    reference picks FusedBatchNormV3 unless `fused=False`, and the library refuses that case."""
+    if tuple(axes) != (-1,):
+        raise ValueError("only axes = Seq(-1) is built")
+    return Layer(L.LAYER_BATCHNORM, f"BatchNorm({list(axes)})", momentum=momentum, epsilon=epsilon,
+                 fused=-1 if fused is None else int(bool(fused)),
+                 inits=(betaInitializer, gammaInitializer, movingMeanInitializer, movingVarianceInitializer))
 
 
 def SimpleRNN(units: int, activation: Activation = Tanh, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
@@ -354,6 +370,9 @@ def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndar
         pre = "" if single else f"{i}/"
         if l.kind in (L.LAYER_DENSE, L.LAYER_BIAS, L.LAYER_CONV2D):
             out[pre + "weights"] = l.inits[0].build(shapes[pre + "weights"], rng)
+        elif l.kind == L.LAYER_BATCHNORM:
+            for name, init in zip(("beta", "gamma", "moving_mean", "moving_variance"), l.inits):
+                out[pre + name] = init.build(shapes[pre + name], rng)
         elif l.kind == L.LAYER_SIMPLE_RNN:
             k_init, r_init, b_init = l.inits
             out[pre + "0/kernel_weights"] = k_init.build(shapes[pre + "0/kernel_weights"], rng)

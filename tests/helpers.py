@@ -13,7 +13,7 @@ f32 = np.float32
 
 def build_pair(spec: List[tuple], loss: str):
     """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
-    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("activate", act) | ("bias", features)
+    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon) | ("activate", act) | ("bias", features)
     Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
     import scanet3_amd as S
     acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
@@ -56,6 +56,9 @@ def build_pair(spec: List[tuple], loss: str):
             bias = e[3] if len(e) > 3 else True
             ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias))
             add(S.SimpleRNN(e[1], acts_s[act], bias=bias))
+        elif k == "batchnorm":   # ("batchnorm", momentum, epsilon): the generic form (fused = Some(false))
+            ol.append(O.BatchNorm(e[1], e[2]))
+            add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=False))
         elif k == "activate":
             ol.append([O.Layer("activate", activation=acts_o[e[1]])])
             add(S.Activate(acts_s[e[1]]))
@@ -73,7 +76,10 @@ def glorot_params(model: O.Model, in_shape, rng: np.random.Generator, scale: flo
     """Xavier-uniform weights, zero biases (forget-gate bias one), from the harness' own generator."""
     out = {}
     for path, shape in model.param_defs(in_shape):
-        if len(shape) == 1:
+        leaf = path.rsplit("/", 1)[-1]
+        if leaf in O.BN_PARAMS:      # gamma and the moving variance start at one (BatchNorm.scala:68-71)
+            out[path] = np.ones(shape, f32) if leaf in ("gamma", "moving_variance") else np.zeros(shape, f32)
+        elif len(shape) == 1:
             out[path] = np.ones(shape, f32) if "forget/1/" in path else np.zeros(shape, f32)
         else:
             fan_in = int(np.prod(shape[:-1]))

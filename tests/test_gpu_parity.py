@@ -281,6 +281,29 @@ def test_golden_simple_rnn_forward(S, ctx, golden):
     h.close()
 
 
+def test_golden_batch_norm(S, ctx, golden):
+    """BatchNormSpec.scala:30-65 through the library: training-mode output, the state one step leaves behind
+    (SGD with rate 0 moves no weight), and the frozen model on its moving statistics."""
+    g = golden["batch_norm"]
+    h = Harness(S, ctx, [("dense", 4, "identity"), ("batchnorm", 0.5, 1e-3)], "mse", (3,), 4, S.SGD(0.0))
+    assert [(p, s) for p, s, _ in h.cm.params][2:] == [(f"2/{k}", (1, 4)) for k in O.BN_PARAMS]
+    x = ctx.to_device(A(g["x"]))
+    t = g["training"]
+    h.rep.set_params({"0/weights": A(g["dense_w"]), "1/weights": A(g["dense_b"]), **{f"2/{k}": A(t[k]) for k in O.BN_PARAMS}})
+    np.testing.assert_array_equal(round_at(h.rep.forward(x, training=True), 3), A(t["y_3dp"]))
+    np.testing.assert_array_equal(h.rep.get_params()["2/moving_mean"], A(t["moving_mean"]))      # a forward pass applies no state
+    h.rep.step(x, ctx.to_device(np.zeros((4, 4), f32)), 1)
+    after = h.rep.get_params()
+    np.testing.assert_array_equal(round_at(after["2/moving_mean"], 3), A(t["next_moving_mean_3dp"]))
+    np.testing.assert_array_equal(round_at(after["2/moving_variance"], 3), A(t["next_moving_variance_3dp"]))
+    np.testing.assert_array_equal(after["0/weights"], A(g["dense_w"]))
+    t = g["frozen"]
+    h.rep.set_params({f"2/{k}": A(t[k]) for k in O.BN_PARAMS})
+    np.testing.assert_array_equal(round_at(h.rep.forward(x), 3), A(t["y_3dp"]))
+    assert set(h.rep.get_grads()) == {"0/weights", "1/weights", "2/beta", "2/gamma"}
+    h.close()
+
+
 def test_cnn_shape_table(S, ctx, golden):
     g = golden["cnn_shapes"]
     spec = [("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
@@ -310,6 +333,11 @@ MODELS = {
     "simple_rnn_relu_nobias_after_activation": ([("activate", "tanh"), ("simple_rnn", 17, "relu", False), ("dense", 3, "identity")],
                                                 "mse", (6, 7), 21, "normal_regression"),
     "simple_rnn_wide": ([("simple_rnn", 128, "sigmoid"), ("dense", 1, "tanh")], "mse", (16, 32), 256, "normal_regression"),
+    "mlp_batchnorm": ([("dense", 33, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 7, "softmax")], "cce", (19,), 130, "normal_onehot"),
+    "batchnorm_first_unaligned": ([("batchnorm", 0.5, 1e-2), ("dense", 3, "identity")], "mse", (13,), 77, "normal_regression"),
+    "cnn_batchnorm": ([("conv", 8, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3), ("pool", (2, 2), (2, 2), "valid"),
+                       ("conv", 6, (3, 3), (1, 1), "same", "relu", True), ("batchnorm", 0.9, 1e-3), ("flatten",), ("dense", 5, "softmax")],
+                      "cce", (12, 12, 2), 24, "uniform_onehot"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
 }
 
@@ -333,7 +361,10 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     om = h.omodel
     params = glorot_params(om, (batch,) + in_shape, rng)
     for p in params:                      # non-zero biases so their gradients and use are exercised
-        if params[p].ndim == 1:
+        leaf = p.rsplit("/", 1)[-1]
+        if leaf == "moving_variance":
+            params[p] = params[p] + rng.uniform(0.0, 0.5, params[p].shape).astype(f32)
+        elif params[p].ndim == 1 or leaf in O.BN_PARAMS:
             params[p] = params[p] + rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
     out_dim = om.out_shape((batch,) + in_shape)[-1]
     x, y = make_data(kind, rng, batch, in_shape, out_dim)
@@ -344,7 +375,9 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     oloss, ograds = om.grad(x, y, params)
     gloss = h.rep.grad(xb, yb)
     assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
-    assert abs(h.rep.loss(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    floss = float(om.loss_of(x, y, params))              # the frozen model: differs from `oloss` only with BatchNorm
+    assert abs(h.rep.loss(xb, yb) - floss) <= TOL_GEMM * max(1.0, abs(floss))
+    assert rel_err(h.rep.forward(xb, training=True), om.forward(x, params, training=True)) <= TOL_GEMM
     ggrads = h.rep.get_grads()
     assert set(ggrads) == set(ograds)
     for p in ograds:
@@ -356,7 +389,7 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
 
 
 @pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("simple_rnn_small", 30),
-                                        ("mlp_bce_l2", 25)])
+                                        ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("mlp_bce_l2", 25)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
 def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
     spec, loss, in_shape, batch, kind = MODELS[name]
@@ -541,6 +574,45 @@ def test_train_epoch_semantics_and_replica_average(S, ctx, linear_function):
     cm.close()
 
 
+def test_train_epoch_with_layer_state_and_its_average(S, ctx):
+    """A BatchNorm model through the partition loop: the moving statistics follow every batch, the loss after the
+    last batch is that of the model as trained (batch statistics, Optimizer.scala:148,163-167), a prediction
+    afterwards is the frozen model's, and the replica average covers the statistics (Aggregation Avg,
+    BatchNorm.scala:96-97)."""
+    spec = [("dense", 12, "tanh"), ("batchnorm", 0.8, 1e-3), ("dense", 2, "identity")]
+    om, layers, sloss = build_pair(spec, "mse")
+    rng = np.random.default_rng(20251125 + 9)
+    batch, n_batches = 32, 5
+    X = rng.standard_normal((batch * n_batches + 7, 6)).astype(f32) * f32(2.0) + f32(0.5)
+    Y = rng.uniform(-1, 1, (X.shape[0], 2)).astype(f32)
+    init = glorot_params(om, (batch, 6), rng)
+    oalg, desc = O.Adam(0.01), S.Adam(0.01)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (6,), batch)
+    rep = cm.replica(desc)
+    rep.set_params(init)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    iters, loss = rep.train_epoch(Xb, Yb, X.shape[0], batch, 0)
+    oi, op_, _, oloss = O.optimize_on_partition(om, oalg, X, Y, batch, 0, init, O.init_opt_state(oalg, init))
+    assert iters == oi == n_batches
+    assert abs(loss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    got = rep.get_params()
+    assert np.any(got["3/moving_mean"] != init["3/moving_mean"])
+    for p in op_:
+        assert rel_err(got[p], op_[p]) <= 1e-4, p
+    xs = ctx.to_device(X[:batch])
+    assert rel_err(rep.forward(xs), om.forward(X[:batch], op_)) <= TOL_GEMM
+    assert abs(rep.loss(xs, ctx.to_device(Y[:batch])) - float(om.loss_of(X[:batch], Y[:batch], op_))) <= TOL_GEMM
+    rep2 = cm.replica(desc)
+    rep2.set_params(init)
+    S.average_replicas([rep, rep2])
+    avg = rep2.get_params()
+    for p in got:
+        np.testing.assert_array_equal(avg[p], O.average_uniform([got[p], init[p]]))
+    rep.close()
+    rep2.close()
+    cm.close()
+
+
 @pytest.mark.parametrize("n_batches", [1, 2, 7])
 def test_train_epoch_from_host_memory_equals_resident_epoch(S, ctx, n_batches):
     """`sn_train_epoch_host` (batches copied on a second stream while the previous one trains) must leave exactly the
@@ -660,6 +732,17 @@ def test_error_paths(S, ctx):
         S.CompiledModel(ctx, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3, 3, 1), 8)
     with pytest.raises(S.ScanetError):                      # kernel larger than the input
         S.CompiledModel(ctx, [S.Conv2D(2, (5, 5)).desc()], S.MeanSquaredError.kind, (3, 3, 1), 8)
+    for fused in (None, True):                              # rank 4: the reference would take FusedBatchNormV3, which is not built
+        with pytest.raises(S.ScanetError, match="FusedBatchNormV3"):
+            S.CompiledModel(ctx, [S.BatchNorm(fused=fused).desc()], S.MeanSquaredError.kind, (3, 3, 2), 8)
+    with pytest.raises(S.ScanetError, match="fused"):       # rank 2 has no fused form (BatchNorm.scala:134-136)
+        S.CompiledModel(ctx, [S.BatchNorm(fused=True).desc()], S.MeanSquaredError.kind, (5,), 8)
+    bn = S.CompiledModel(ctx, [S.BatchNorm().desc()], S.MeanSquaredError.kind, (5,), 8)
+    bn_rep = bn.replica(S.Adam())
+    with pytest.raises(S.ScanetError, match="layer state"):
+        bn_rep.set_opt_state(0, {"moving_mean": np.zeros((1, 5), f32)})
+    bn_rep.close()
+    bn.close()
     x.free()
     y.free()
 

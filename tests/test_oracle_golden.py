@@ -240,6 +240,46 @@ def test_simple_rnn_golden(golden):
     np.testing.assert_array_equal(round_at(y, 6), A(g["y_6dp"]))
 
 
+def _batch_norm_case(g, mode):
+    t = g[mode]
+    p = {"0/weights": A(g["dense_w"]), "1/weights": A(g["dense_b"])}
+    p.update({f"2/{k}": A(t[k]) for k in O.BN_PARAMS})
+    return t, p
+
+
+def test_batch_norm_golden(golden):
+    """BatchNormSpec.scala:30-65: training mode (output and the next moving statistics) and the frozen model."""
+    g = golden["batch_norm"]
+    m = O.Model([O.Dense(4), O.BatchNorm(momentum=0.5)])
+    assert [p for p, _ in m.param_defs((4, 3))][2:] == ["2/beta", "2/gamma", "2/moving_mean", "2/moving_variance"]
+    assert all(s == (1, 4) for _, s in m.param_defs((4, 3))[2:])
+    t, p = _batch_norm_case(g, "training")
+    nxt = {}
+    y = m.forward(A(g["x"]), p, training=True, next_state=nxt)
+    np.testing.assert_array_equal(round_at(y, 3), A(t["y_3dp"]))
+    np.testing.assert_array_equal(round_at(nxt["2/moving_mean"], 3), A(t["next_moving_mean_3dp"]))
+    np.testing.assert_array_equal(round_at(nxt["2/moving_variance"], 3), A(t["next_moving_variance_3dp"]))
+    t, p = _batch_norm_case(g, "frozen")
+    np.testing.assert_array_equal(round_at(m.forward(A(g["x"]), p), 3), A(t["y_3dp"]))
+
+
+def test_batch_norm_state_bypasses_the_algorithm(golden):
+    """`nextWeights ++ nextState` (Optimizer.scala:142-144): moving statistics are replaced by the layer's own
+    update, every other tensor by the algorithm; a training-mode output has zero mean and unit variance."""
+    g = golden["batch_norm"]
+    m = O.Model([O.Dense(4), O.BatchNorm(momentum=0.5)], O.LOSS_MSE)
+    _, p = _batch_norm_case(g, "training")
+    x, y = A(g["x"]), np.zeros((4, 4), np.float32)
+    alg = O.SGD(0.1)
+    new_p, _, _, grads = O.train_step(m, alg, x, y, p, O.init_opt_state(alg, p), 1)
+    assert set(grads) == {"0/weights", "1/weights", "2/beta", "2/gamma"}
+    np.testing.assert_array_equal(round_at(new_p["2/moving_mean"], 3), A(g["training"]["next_moving_mean_3dp"]))
+    np.testing.assert_array_equal(new_p["2/beta"], p["2/beta"] - np.float32(0.1) * grads["2/beta"])
+    out = m.forward(x, p, training=True)
+    np.testing.assert_allclose(out.mean(axis=0), 0.0, atol=1e-6)
+    np.testing.assert_allclose(out.var(axis=0), 1.0, atol=1e-3)      # var / (var + epsilon)
+
+
 def _lstm_params(g, pre=""):
     p = {}
     for gate in O.GATES:
@@ -271,7 +311,7 @@ def test_cnn_shape_table_golden(golden):
 
 
 # ----------------------------------------------------------------- gradients: float64 numerics + torch
-def _numeric_grad(m, x, y, params, path, eps=1e-6):
+def _numeric_grad(m, x, y, params, path, eps=1e-6, training=False):
     w = params[path]
     g = np.zeros_like(w)
     it = np.nditer(w, flags=["multi_index"])
@@ -279,9 +319,9 @@ def _numeric_grad(m, x, y, params, path, eps=1e-6):
         idx = it.multi_index
         old = w[idx]
         w[idx] = old + eps
-        lp = float(m.loss_of(x, y, params))
+        lp = float(m.loss_of(x, y, params, training=training))
         w[idx] = old - eps
-        lm = float(m.loss_of(x, y, params))
+        lm = float(m.loss_of(x, y, params, training=training))
         w[idx] = old
         g[idx] = (lp - lm) / (2 * eps)
     return g
@@ -291,7 +331,7 @@ def _rand_params(m, in_shape, rng, dt=np.float64, scale=0.4):
     return {p: (rng.standard_normal(s) * scale).astype(dt) for p, s in m.param_defs(in_shape)}
 
 
-@pytest.mark.parametrize("name", ["mlp_cce", "cnn_cce", "lstm_mse", "rnn_mse", "mlp_bce_l2"])
+@pytest.mark.parametrize("name", ["mlp_cce", "cnn_cce", "lstm_mse", "rnn_mse", "mlp_batchnorm", "cnn_batchnorm", "mlp_bce_l2"])
 def test_model_gradients_match_numeric_float64(name):
     rng = np.random.default_rng(11)
     if name == "mlp_cce":
@@ -311,14 +351,26 @@ def test_model_gradients_match_numeric_float64(name):
         m = O.Model([O.SimpleRNN(3), O.Dense(2)], O.LOSS_MSE)
         x = rng.standard_normal((2, 4, 3))
         y = rng.uniform(-1, 1, (2, 2))
+    elif name == "mlp_batchnorm":     # batch statistics depend on the input: the gradient runs through mean and variance
+        m = O.Model([O.Dense(5, O.ACT_TANH), O.BatchNorm(0.9, 1e-3), O.Dense(3, O.ACT_SOFTMAX)], O.LOSS_CCE)
+        x = rng.standard_normal((6, 4))
+        y = np.eye(3)[rng.integers(0, 3, 6)]
+    elif name == "cnn_batchnorm":     # rank 4: statistics over batch, height and width
+        m = O.Model([O.Conv2D(3, activation=O.ACT_RELU), O.BatchNorm(0.9, 1e-2), O.Pool2D(), O.Flatten(), O.Dense(2)], O.LOSS_MSE)
+        x = rng.random((3, 6, 5, 2))
+        y = rng.uniform(-1, 1, (3, 2))
     else:
         m = O.Model([O.Dense(3, O.ACT_SIGMOID, reg=O.REG_L2, reg_lambda=0.3), O.Dense(2, O.ACT_SIGMOID)], O.LOSS_BCE)
         x = rng.random((4, 3))
         y = rng.integers(0, 2, (4, 2)).astype(np.float64)
     params = _rand_params(m, x.shape, rng)
-    _, grads = m.grad(x, y, params)
     for path in params:
-        num = _numeric_grad(m, x, y, params, path)
+        if O.is_state_path(path):
+            params[path] = np.abs(params[path]) + 0.5
+    _, grads = m.grad(x, y, params)
+    assert set(grads) == {p for p in params if not O.is_state_path(p)}
+    for path in grads:
+        num = _numeric_grad(m, x, y, params, path, training=True)
         np.testing.assert_allclose(grads[path], num, rtol=2e-5, atol=2e-8, err_msg=path)
 
 
