@@ -49,7 +49,10 @@ def glorot(rng, shape):
 def init_params(cm, rng):
     out = {}
     for path, shape, _ in cm.params:
-        if len(shape) == 1:
+        leaf = path.rsplit("/", 1)[-1]
+        if leaf in ("beta", "gamma", "moving_mean", "moving_variance"):      # BatchNorm.scala:68-71
+            out[path] = np.ones(shape, np.float32) if leaf in ("gamma", "moving_variance") else np.zeros(shape, np.float32)
+        elif len(shape) == 1:
             out[path] = np.ones(shape, np.float32) if "forget/1/" in path else np.zeros(shape, np.float32)
         else:
             out[path] = glorot(rng, shape)
@@ -165,6 +168,34 @@ def bench_mlp(S, ctx, steps, warmup):
 def bench_lstm(S, ctx, steps, warmup):
     return run_model_workload(
         S, ctx, "LSTM(256)->Dense(1,tanh), batch 512, T 64, F 32, Adam, MSE, fp32", S.LSTM(256) >> S.Dense(1, S.Tanh),
+        S.MeanSquaredError, (64, 32), 512, S.Adam(),
+        lambda rng, n: (rng.standard_normal((n, 64, 32)).astype(np.float32), rng.uniform(-1, 1, (n, 1)).astype(np.float32)),
+        4, steps, warmup)
+
+
+def bench_cnn_bn(S, ctx, steps, warmup):
+    """The CNN the reference trains on MNIST (test models/CNNSpec.scala:22-35), BatchNorm in its generic form."""
+    layers = (S.Conv2D(32, activation=S.ReLU()) >> S.BatchNorm(fused=False) >> S.Pool2D(strides=(2, 2))
+              >> S.Conv2D(64, activation=S.ReLU()) >> S.Pool2D(strides=(2, 2)) >> S.Activate(S.ReLU()) >> S.Flatten
+              >> S.Dense(64, S.ReLU()) >> S.Dense(10, S.Softmax))
+    r = run_model_workload(
+        S, ctx, "CNN with BatchNorm 28x28x1 (Conv32-BN-Pool/2-Conv64-Pool/2-Dense64-Dense10), batch 1000, Adam, fp32", layers,
+        S.CategoricalCrossentropy, (28, 28, 1), 1000, S.Adam(),
+        lambda rng, n: (rng.random((n, 28, 28, 1), np.float32), one_hot(rng, n, 10)), 4, steps, warmup)
+    # the batch-norm kernels stream a [1000*26*26, 32] activation: bytes each pass has to move / its measured time
+    elems = 1000 * 26 * 26 * 32
+    passes = {"batchnorm_mean": 1, "batchnorm_variance": 1, "batchnorm_apply": 2, "batchnorm_gradient_sums": 2,
+              "batchnorm_input_gradient": 3}
+    r["batchnorm_hbm"] = {k: {"bytes": 4 * elems * p, "avg_us": r["kernels"][k]["avg_us"],
+                              "GBps": 4 * elems * p / (r["kernels"][k]["avg_us"] * 1e-6) / 1e9,
+                              "frac_of_peak": 4 * elems * p / (r["kernels"][k]["avg_us"] * 1e-6) / 1e9 / PEAK_HBM_GBS}
+                          for k, p in passes.items() if k in r["kernels"]}
+    return r
+
+
+def bench_simple_rnn(S, ctx, steps, warmup):
+    return run_model_workload(
+        S, ctx, "SimpleRNN(256)->Dense(1,tanh), batch 512, T 64, F 32, Adam, MSE, fp32", S.SimpleRNN(256) >> S.Dense(1, S.Tanh),
         S.MeanSquaredError, (64, 32), 512, S.Adam(),
         lambda rng, n: (rng.standard_normal((n, 64, 32)).astype(np.float32), rng.uniform(-1, 1, (n, 1)).astype(np.float32)),
         4, steps, warmup)
@@ -305,7 +336,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="lenet", choices=["lenet", "mlp", "lstm", "wide_mlp", "optim"])
+    ap.add_argument("--workload", default="lenet", choices=["lenet", "mlp", "lstm", "wide_mlp", "optim", "cnn_bn", "simple_rnn"])
     ap.add_argument("--pool-stride", type=int, default=1, help="LeNet pool stride (reference default 1)")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -328,6 +359,10 @@ def main():
             return bench_lstm(S, ctx, st, wu)
         if which == "wide_mlp":
             return bench_wide_mlp(S, ctx, st, wu)
+        if which == "cnn_bn":
+            return bench_cnn_bn(S, ctx, st, wu)
+        if which == "simple_rnn":
+            return bench_simple_rnn(S, ctx, st, wu)
         return bench_optim(S, ctx, st, wu)
 
     main_res = run(args.workload, steps, warmup)
@@ -351,9 +386,12 @@ def main():
                      "host_fed": main_res["host_fed"],
                      "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                              sorted(main_res["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:12]}})
+        if "batchnorm_hbm" in main_res:
+            line["batchnorm_hbm"] = main_res["batchnorm_hbm"]
     if not args.no_extras:
         extras = {}
-        for which, st, wu in (("mlp", 100, 10), ("lstm", 10, 2), ("wide_mlp", 5, 2), ("optim", 10, 3), ("lenet", 50, 5)):
+        for which, st, wu in (("mlp", 100, 10), ("lstm", 10, 2), ("wide_mlp", 5, 2), ("optim", 10, 3), ("lenet", 50, 5),
+                               ("cnn_bn", 10, 2), ("simple_rnn", 10, 2)):
             if which == args.workload:
                 continue
             try:
@@ -370,6 +408,8 @@ def main():
                                  "roofline": dominant_gemm_roofline(r["kernels"], peak),
                                  "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                                          sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}
+                if "batchnorm_hbm" in r:
+                    extras[which]["batchnorm_hbm"] = r["batchnorm_hbm"]
         line["other_configs"] = extras
         # the two rooflines the memory-bound and the GEMM-bound configurations are judged on
         rl = {}

@@ -67,22 +67,88 @@ __global__ __launch_bounds__(256) void bn_reduce_kernel(const float* __restrict_
   }
 }
 
-__device__ __forceinline__ float add_slices(const float* __restrict__ part, int slices, int cols, int c) {
-  float s = 0.f;
-  int i = 0;
-  for (; i + 4 <= slices; i += 4) {  // four loads in flight, added in slice order
-    const float a = part[(int64_t)i * cols + c], b = part[(int64_t)(i + 1) * cols + c], d = part[(int64_t)(i + 2) * cols + c],
-                e = part[(int64_t)(i + 3) * cols + c];
-    s = (((s + a) + b) + d) + e;
+// Few channels (C/4 divides 256): the tensor is read as one stream of float4; a thread's float4 index moves in steps
+// of 256, so it stays on the same four channels and every wavefront load covers 1 KiB of consecutive memory.
+// A block owns `per4` consecutive float4 (a multiple of 256); threads with equal t % (C/4) meet in LDS.
+template <int MODE>
+__global__ __launch_bounds__(256) void bn_reduce_v4_kernel(const bn_f4* __restrict__ x, const bn_f4* __restrict__ dy,
+                                                            const float* __restrict__ mean, float* __restrict__ part0,
+                                                            float* __restrict__ part1, int64_t n4, int cols, int64_t per4) {
+  __shared__ bn_f4 smem[2][256];
+  const int t = threadIdx.x, cg = cols / 4, g = t % cg;
+  const int64_t begin = (int64_t)blockIdx.x * per4;
+  const int64_t end = begin + per4 < n4 ? begin + per4 : n4;
+  bn_f4 m = {0.f, 0.f, 0.f, 0.f};
+  if (MODE != BN_SUM) m = *(const bn_f4*)(mean + 4 * g);
+  bn_f4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+  int64_t i = begin + t;
+  for (; i + 7 * 256 < end; i += 8 * 256) {
+    bn_f4 a[8], b[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a[u] = __builtin_nontemporal_load(x + i + u * 256);
+    if (MODE == BN_GRAD) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) b[u] = __builtin_nontemporal_load(dy + i + u * 256);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (MODE == BN_SUM) s0 = s0 + a[u];
+      if (MODE == BN_SQDIFF) { const bn_f4 d = a[u] - m; s0 = s0 + d * d; }
+      if (MODE == BN_GRAD) { s0 = s0 + b[u]; s1 = s1 + b[u] * (a[u] - m); }
+    }
   }
-  for (; i < slices; ++i) s += part[(int64_t)i * cols + c];
-  return s;
+  for (; i < end; i += 256) {
+    const bn_f4 a = x[i];
+    if (MODE == BN_SUM) s0 = s0 + a;
+    if (MODE == BN_SQDIFF) { const bn_f4 d = a - m; s0 = s0 + d * d; }
+    if (MODE == BN_GRAD) { const bn_f4 b = dy[i]; s0 = s0 + b; s1 = s1 + b * (a - m); }
+  }
+  smem[0][t] = s0;
+  if (MODE == BN_GRAD) smem[1][t] = s1;
+  __syncthreads();
+  if (t < cg) {
+    bn_f4 r0 = smem[0][t], r1 = smem[1][t];
+    for (int j = t + cg; j < 256; j += cg) {
+      r0 = r0 + smem[0][j];
+      if (MODE == BN_GRAD) r1 = r1 + smem[1][j];
+    }
+    *(bn_f4*)(part0 + (int64_t)blockIdx.x * cols + 4 * t) = r0;
+    if (MODE == BN_GRAD) *(bn_f4*)(part1 + (int64_t)blockIdx.x * cols + 4 * t) = r1;
+  }
 }
 
-// One thread per channel.
+// Sum of one channel's slices by 16 threads: a block is 16 channels x 16 slice lanes; lane j adds slices j, j+16, ...
+// (8 loads in flight), the 16 lane sums are added in lane order.  Every thread of the block must call it; the total is
+// returned to all of them.  (One thread per channel would walk up to 1024 slices one memory latency after another.)
+__device__ __forceinline__ float slices_total(const float* __restrict__ part, int slices, int cols, int c, float (*smem)[16]) {
+  const int cl = threadIdx.x & 15, sl = threadIdx.x >> 4;
+  float s = 0.f;
+  if (c < cols) {
+    int i = sl;
+    for (; i + 7 * 16 < slices; i += 8 * 16) {
+      float a[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) a[u] = part[(int64_t)(i + 16 * u) * cols + c];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += a[u];
+    }
+    for (; i < slices; i += 16) s += part[(int64_t)i * cols + c];
+  }
+  __syncthreads();  // a previous call's readers are done with smem
+  smem[sl][cl] = s;
+  __syncthreads();
+  float total = smem[0][cl];
+#pragma unroll
+  for (int j = 1; j < 16; ++j) total += smem[j][cl];
+  return total;
+}
+
+// Finishing kernels: block = 16 channels x 16 slice lanes, grid = ceil(C/16).
 __global__ __launch_bounds__(256) void bn_mean_kernel(const float* __restrict__ part, int slices, int cols, float n, float* __restrict__ mean) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c < cols) mean[c] = add_slices(part, slices, cols, c) / n;
+  __shared__ float smem[16][16];
+  const int c = blockIdx.x * 16 + (threadIdx.x & 15);
+  const float total = slices_total(part, slices, cols, c, smem);
+  if (threadIdx.x < 16 && c < cols) mean[c] = total / n;
 }
 
 // var from the slices (training) or from the moving variance (part == null), then r = 1/sqrt(var+eps), inv = r*gamma
@@ -90,11 +156,14 @@ __global__ __launch_bounds__(256) void bn_scale_kernel(const float* __restrict__
                                                         const float* __restrict__ gamma, const float* __restrict__ moving_mean,
                                                         const float* __restrict__ moving_var, float* __restrict__ mean,
                                                         float* __restrict__ var, float* __restrict__ r, float* __restrict__ inv) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cols) return;
+  __shared__ float smem[16][16];
+  const int c = blockIdx.x * 16 + (threadIdx.x & 15);
+  float total = 0.f;
+  if (part) total = slices_total(part, slices, cols, c, smem);  // uniform over the block
+  if (threadIdx.x >= 16 || c >= cols) return;
   float v;
   if (part) {
-    v = add_slices(part, slices, cols, c) / n;
+    v = total / n;
   } else {
     v = moving_var[c];
     mean[c] = moving_mean[c];
@@ -132,9 +201,11 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__
 __global__ __launch_bounds__(256) void bn_grad_finish_kernel(const float* __restrict__ part0, const float* __restrict__ part1, int slices,
                                                               int cols, float n, const float* __restrict__ r, float* __restrict__ dbeta,
                                                               float* __restrict__ dgamma, float* __restrict__ k1, float* __restrict__ k2) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cols) return;
-  const float s1 = add_slices(part0, slices, cols, c), s2 = add_slices(part1, slices, cols, c);
+  __shared__ float smem[16][16];
+  const int c = blockIdx.x * 16 + (threadIdx.x & 15);
+  const float s1 = slices_total(part0, slices, cols, c, smem);
+  const float s2 = slices_total(part1, slices, cols, c, smem);
+  if (threadIdx.x >= 16 || c >= cols) return;
   const float rr = r[c];
   dbeta[c] = s1;
   dgamma[c] = s2 * rr;
@@ -193,6 +264,43 @@ int slices_for(const sn_ctx* ctx, int64_t rows, int cols) {
   return s < 1 ? 1 : (int)s;
 }
 
+// the float4-stream reduction: C/4 divides 256 and enough data for more than one block
+bool stream_form(int64_t rows, int cols) { return cols % 4 == 0 && cols <= 1024 && 256 % (cols / 4) == 0 && rows * cols >= 4 * 8 * 256; }
+int stream_slices(const sn_ctx* ctx, int64_t n4) {
+  int64_t s = ceil_div(n4, (int64_t)8 * 256);  // at least one full trip of 8 loads per thread
+  const int64_t cap = (int64_t)ctx->compute_units * 4;
+  if (s > cap) s = cap;
+  return s < 1 ? 1 : (int)s;
+}
+
+// One reduction pass in whichever form fits; returns the number of slices written to part0 (and part1).
+template <int MODE>
+int reduce_pass(sn_ctx* ctx, const float* x, const float* dy, const float* mean, float* part0, int64_t part1_offset, int64_t rows,
+                int cols, int* slices_out) {
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(part0)) & 15u) == 0;
+  if (stream_form(rows, cols) && aligned && part1_offset % 4 == 0) {
+    const int64_t n4 = rows * cols / 4;
+    const int s = stream_slices(ctx, n4);
+    const int64_t per4 = align_up(ceil_div(n4, (int64_t)s), 256);
+    hipLaunchKernelGGL((bn_reduce_v4_kernel<MODE>), dim3((unsigned)s), dim3(256), 0, ctx->stream, (const bn_f4*)x, (const bn_f4*)dy, mean,
+                       part0, part0 + part1_offset, n4, cols, per4);
+    *slices_out = s;
+  } else {
+    const int s = slices_for(ctx, rows, cols);
+    hipLaunchKernelGGL((bn_reduce_kernel<MODE>), dim3((unsigned)ceil_div((int64_t)cols, (int64_t)64), (unsigned)s), dim3(256), 0,
+                       ctx->stream, x, dy, mean, part0, part0 + part1_offset, rows, cols, ceil_div(rows, (int64_t)s));
+    *slices_out = s;
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int max_slices(const sn_ctx* ctx, int64_t rows, int cols) {
+  int s = slices_for(ctx, rows, cols);
+  if (stream_form(rows, cols)) s = std::max(s, stream_slices(ctx, rows * cols / 4));
+  return s;
+}
+
 bool vec4_ok(int cols, std::initializer_list<const void*> ptrs) {
   if (cols % 4 != 0) return false;
   for (const void* p : ptrs)
@@ -202,28 +310,25 @@ bool vec4_ok(int cols, std::initializer_list<const void*> ptrs) {
 
 }  // namespace
 
-int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols) { return (int64_t)2 * slices_for(ctx, rows, cols) * cols; }
+int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols) { return (int64_t)2 * max_slices(ctx, rows, cols) * cols; }
 
 int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, int cols, const BatchNormArgs& a, bool training, float* ws,
                          int64_t ws_elems) {
   if (rows <= 0 || cols <= 0) return SN_OK;
   SN_REQUIRE(rows * cols <= (int64_t)INT32_MAX * 4, "batch norm over %lld elements exceeds one launch", (long long)(rows * cols));
-  const int cb = (int)ceil_div((int64_t)cols, (int64_t)256);
+  const int cb = (int)ceil_div((int64_t)cols, (int64_t)16);  // finishing kernels: 16 channels per block
   if (training) {
-    const int s = slices_for(ctx, rows, cols);
-    SN_REQUIRE((int64_t)s * cols <= ws_elems, "batch norm needs %lld workspace elements, %lld given", (long long)s * cols, (long long)ws_elems);
-    const int64_t per = ceil_div(rows, (int64_t)s);
-    const dim3 grid((unsigned)ceil_div((int64_t)cols, (int64_t)64), (unsigned)s);
+    const int64_t need = (int64_t)max_slices(ctx, rows, cols) * cols;
+    SN_REQUIRE(need <= ws_elems, "batch norm needs %lld workspace elements, %lld given", (long long)need, (long long)ws_elems);
+    int s = 0;
     {
       LaunchScope scope(ctx, "batchnorm_mean");
-      hipLaunchKernelGGL((bn_reduce_kernel<BN_SUM>), grid, dim3(256), 0, ctx->stream, x, (const float*)nullptr, (const float*)nullptr, ws,
-                         (float*)nullptr, rows, cols, per);
+      SN_TRY(reduce_pass<BN_SUM>(ctx, x, nullptr, nullptr, ws, 0, rows, cols, &s));
       hipLaunchKernelGGL(bn_mean_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, s, cols, (float)rows, a.mean);
     }
     {
       LaunchScope scope(ctx, "batchnorm_variance");
-      hipLaunchKernelGGL((bn_reduce_kernel<BN_SQDIFF>), grid, dim3(256), 0, ctx->stream, x, (const float*)nullptr, (const float*)a.mean, ws,
-                         (float*)nullptr, rows, cols, per);
+      SN_TRY(reduce_pass<BN_SQDIFF>(ctx, x, nullptr, a.mean, ws, 0, rows, cols, &s));
       hipLaunchKernelGGL(bn_scale_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, s, cols, (float)rows, a.epsilon, a.gamma,
                          (const float*)nullptr, (const float*)nullptr, a.mean, a.var, a.r, a.inv);
     }
@@ -247,16 +352,14 @@ int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, in
 int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx, int64_t rows, int cols, const BatchNormArgs& a,
                          float* dbeta, float* dgamma, float* ws, int64_t ws_elems) {
   if (rows <= 0 || cols <= 0) return SN_OK;
-  const int s = slices_for(ctx, rows, cols);
-  SN_REQUIRE((int64_t)2 * s * cols <= ws_elems, "batch norm gradient needs %lld workspace elements, %lld given", (long long)2 * s * cols,
-             (long long)ws_elems);
-  const int64_t per = ceil_div(rows, (int64_t)s);
-  const int cb = (int)ceil_div((int64_t)cols, (int64_t)256);
-  float* part1 = ws + (int64_t)s * cols;
+  const int64_t half = (int64_t)max_slices(ctx, rows, cols) * cols;
+  SN_REQUIRE(2 * half <= ws_elems, "batch norm gradient needs %lld workspace elements, %lld given", (long long)(2 * half), (long long)ws_elems);
+  const int cb = (int)ceil_div((int64_t)cols, (int64_t)16);  // finishing kernels: 16 channels per block
+  float* part1 = ws + half;
   {
     LaunchScope scope(ctx, "batchnorm_gradient_sums");
-    hipLaunchKernelGGL((bn_reduce_kernel<BN_GRAD>), dim3((unsigned)ceil_div((int64_t)cols, (int64_t)64), (unsigned)s), dim3(256), 0,
-                       ctx->stream, x, dy, (const float*)a.mean, ws, part1, rows, cols, per);
+    int s = 0;
+    SN_TRY(reduce_pass<BN_GRAD>(ctx, x, dy, a.mean, ws, half, rows, cols, &s));
     hipLaunchKernelGGL(bn_grad_finish_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, (const float*)part1, s, cols,
                        (float)rows, (const float*)a.r, dbeta, dgamma, a.k1, a.k2);
   }

@@ -338,6 +338,9 @@ MODELS = {
     "cnn_batchnorm": ([("conv", 8, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3), ("pool", (2, 2), (2, 2), "valid"),
                        ("conv", 6, (3, 3), (1, 1), "same", "relu", True), ("batchnorm", 0.9, 1e-3), ("flatten",), ("dense", 5, "softmax")],
                       "cce", (12, 12, 2), 24, "uniform_onehot"),
+    "cnn_batchnorm_32_channels": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3),
+                                   ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 10, "softmax")],
+                                  "cce", (14, 14, 1), 50, "uniform_onehot"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
 }
 
