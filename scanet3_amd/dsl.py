@@ -552,7 +552,7 @@ class Builder:
             final = reps[0].get_params()
             n_states = len(STATE_NAMES[self.alg.kind])
             slots = [reps[0].get_opt_state(s) for s in range(n_states)]
-            opt_state = {p: [slots[s][p] for s in range(n_states)] for p in final}
+            opt_state = {p: [slots[s][p] for s in range(n_states)] for p in final if p not in cm.state_paths}   # weights only
             return TrainedModel(self.model, self.loss_fn, final, opt_state, history, global_iter, tuple(in_shape), self.flags)
         finally:
             for r in reps:

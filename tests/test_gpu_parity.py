@@ -711,6 +711,29 @@ def test_k_replica_training_matches_oracle(S, linear_function):
         assert rel_err(trained.params[p], oparams[p]) <= 1e-4
 
 
+def test_dsl_batch_norm_training_over_two_partitions(S):
+    """Dense >> BatchNorm >> Dense through the DSL mirror on two partitions: weights, optimizer state and the moving
+    statistics are averaged after every epoch; the trained model predicts with the moving statistics."""
+    rng = np.random.default_rng(20251125 + 11)
+    X = (rng.standard_normal((200, 5)) * 3.0 + 1.0).astype(f32)
+    Y = (X[:, :1] * f32(0.3) - X[:, 1:2] * f32(0.2) + f32(0.1)).astype(f32)
+    model = S.Dense(8, S.Tanh) >> S.BatchNorm(momentum=0.9) >> S.Dense(1)
+    om = O.Model([O.Dense(8, O.ACT_TANH), O.BatchNorm(0.9), O.Dense(1)], O.LOSS_MSE)
+    init = glorot_params(om, (20, 5), rng)
+    trained = S.Dataset(X, Y, partitions=2).train(model).loss(S.MeanSquaredError).using(S.Adam(0.01)).initParams(init) \
+        .batch(20).epochs(6).run()
+    parts = [(X[:100], Y[:100]), (X[100:], Y[100:])]
+    oparams, _, ohist = O.train(om, O.Adam(0.01), parts, 20, 6, init)
+    assert trained.iterations == 6 * 10
+    np.testing.assert_allclose(trained.history, ohist, rtol=TOL_TRAJECTORY)
+    assert set(trained.params) == set(oparams)
+    assert set(trained.opt_state) == {p for p in oparams if not O.is_state_path(p)}
+    for p in oparams:
+        assert rel_err(trained.params[p], oparams[p]) <= 1e-4, p
+    assert np.all(trained.params["3/moving_variance"] != 1.0)
+    assert rel_err(trained.result(X[:7]), om.forward(X[:7], oparams)) <= TOL_GEMM
+
+
 def test_error_paths(S, ctx):
     with pytest.raises(S.ScanetError):
         S.Context(99)
