@@ -959,13 +959,13 @@ static int small_parts(int m, int n, int k, int cu, int64_t ws_elems) {
 }
 
 // ============================================================================ dispatch
-constexpr int SPLIT_WG_PER_CU = 8, SPLIT_MAX = 256;
+constexpr int SPLIT_WG_PER_CU = 8, SPLIT_MAX = 256, SPLIT_MIN_K = 256;
 int64_t gemm_workspace_elems(int m, int n, int k, int cu) {
   // room for the partial sums of the small-output kernel, or for the largest split count launch_tiles may pick
   const int parts = small_parts(m, n, k, cu, -1);
   if (parts) return (int64_t)parts * m * n;
   const int64_t tiles = ceil_div(m, 64) * ceil_div(n, 64);
-  if (tiles >= cu || k < 256) return 0;
+  if (tiles >= cu || k < SPLIT_MIN_K) return 0;
   int64_t splits = std::min<int64_t>(ceil_div((int64_t)SPLIT_WG_PER_CU * cu, tiles), std::max<int64_t>(1, k / 32));
   splits = std::min<int64_t>(splits, SPLIT_MAX);
   return splits * (int64_t)m * n;
@@ -976,7 +976,7 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
                         int64_t ws_elems) {
   const int64_t tiles = ceil_div(M, BM) * ceil_div(N, BN);
   int splits = 1;
-  if (tiles * 2 <= ctx->compute_units && K >= 256 && ws) {  // a split costs a second pass over M*N*splits floats
+  if (tiles * 2 <= ctx->compute_units && K >= SPLIT_MIN_K && ws) {  // a split costs a second pass over M*N*splits floats
     // These kernels are a chain of load, stage, multiply per K tile: what hides its latency is other workgroups on
     // the same CU, so aim for 8 per CU (measured: 2 per CU runs the LeNet filter gradient in 52 us, 8 per CU in 31).
     int64_t s = std::min<int64_t>(ceil_div((int64_t)SPLIT_WG_PER_CU * ctx->compute_units, tiles), std::max<int64_t>(1, K / 32));
