@@ -255,15 +255,18 @@ int64_t gemm_workspace_elems(int m, int n, int k, int cu);
 
 // ---- fused LSTM steps (lstm_kernels.hip) ------------------------------------------------
 // true when the fused step kernels handle this layer (F % 4 == 0, H % 16 == 0, F + H <= 400, 16-byte aligned tensors)
-bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w);
+bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w, int gates = 4);
 // gates, c_t, h_t of step t from x[:, t, :], h_prev, c_prev (both null at t == 0) in one kernel
 // The step kernels read the weights from copies in their LDS order: pack_fwd ([Wk; Wr] of the 4 gates) and pack_dh
 // (Wr of the 4 gates), lstm_pack_elems(F, H) floats each at most; rebuilt once per pass over the sequence.
 int64_t lstm_pack_elems(int F, int H);
-int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh);
+int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh, int gates = 4);
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h);
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev
-int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride);
+int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride,
+                        int gates = 4);
+// simple cell: r_t[rows, H] = [x[:, t, :], r_prev] * [Wk; Wr] from the one-gate pack (r_prev null at t == 0)
+int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* r_prev, int rows, int H, const float* wpack, float* out);
 
 }  // namespace sn

@@ -61,15 +61,15 @@ struct StepFwdArgs {
 // per training step, the step kernel runs T times): [unit group of 16][gate][k/4][16 units][4 consecutive k],
 // k over [Wk; Wr] padded with zeros to a multiple of 16.  The step kernel then copies its slab with contiguous
 // 16-byte loads instead of gathering 4-byte values from 4 rows per cell.
-__global__ __launch_bounds__(256) void pack_fwd_kernel(LstmWeights w, int F, int H, float* __restrict__ out) {
+__global__ __launch_bounds__(256) void pack_fwd_kernel(LstmWeights w, int F, int H, int G, float* __restrict__ out) {
   const int K = F + H, kq = round16(K) / 4;
-  const int64_t cells = (int64_t)(H / 16) * 4 * kq * 16;
+  const int64_t cells = (int64_t)(H / 16) * G * kq * 16;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < cells; e += (int64_t)gridDim.x * 256) {
     const int bu = (int)(e & 15);
     int64_t t = e >> 4;
     const int q = (int)(t % kq); t /= kq;
-    const int gate = (int)(t & 3);
-    const int cg = (int)(t >> 2);
+    const int gate = (int)(t % G);
+    const int cg = (int)(t / G);
     f4v v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -82,9 +82,9 @@ __global__ __launch_bounds__(256) void pack_fwd_kernel(LstmWeights w, int F, int
 }
 
 // [gate][unit block of 16][n/4][16 units][4 consecutive n] of the recurrent weights Wr_gate[u][n], n padded to 16
-__global__ __launch_bounds__(256) void pack_dh_kernel(LstmWeights w, int H, float* __restrict__ out) {
+__global__ __launch_bounds__(256) void pack_dh_kernel(LstmWeights w, int H, int G, float* __restrict__ out) {
   const int kq = round16(H) / 4;
-  const int64_t cells = (int64_t)4 * (H / 16) * kq * 16;
+  const int64_t cells = (int64_t)G * (H / 16) * kq * 16;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < cells; e += (int64_t)gridDim.x * 256) {
     const int bu = (int)(e & 15);
     int64_t t = e >> 4;
@@ -197,38 +197,52 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
   }
 }
 
-// ---------------------------------------------------------------------------- backward: partial dh per gate
-struct StepDhArgs {
-  const float* dz;      // [rows, 4H]
-  const float* wpack;   // recurrent weights in LDS order (pack_dh_kernel)
-  float* dh_parts;      // [4][part_stride] partial dh_prev, one per gate
-  int64_t part_stride;
-  int rows, H;
+// ---------------------------------------------------------------------------- one product per step, whole K in LDS
+// out_z[m, u] = sum_k A[m, k] * W_z[u, k] for z = blockIdx.z, where a row of A is [a0 row (k0 values), a1 row (k1 values)]
+// and W_z comes packed as [unit block of 16][k/4][16 units][4 consecutive k] with `kq_pack` quads per unit block.
+//   LSTM backward:      A = dz of gate z (a0 = dz + z*H, a1 = null), W = recurrent weights, out = partial dh of gate z
+//   simple cell forward: A = [x_t, r_{t-1}], W = [Wk; Wr] columns, out = r_t            (layer/RNN.scala:189-196)
+//   simple cell backward: A = dr_t, W = recurrent weights, out = dr_{t-1}
+struct StepMulArgs {
+  const float* a0;
+  int64_t ld0;          // row stride of a0
+  int k0;
+  const float* a1;      // or null
+  int64_t ld1;
+  int k1;
+  int64_t a0_z_stride;  // added to a0 per blockIdx.z
+  const float* wpack;
+  int kq_pack;          // quads per unit block in the pack (>= the quads this launch reads)
+  int64_t pack_z_stride;
+  float* out;           // [rows, out_ld]
+  int64_t out_ld, out_z_stride;
+  int rows, cols;
 };
 
-// dh_parts[gate][m, u] = sum_n dz[m, gate*H + n] * Wr_gate[u, n]
 // CBT output units per workgroup: 64 (one column block per wavefront, two row blocks each) or 32 (half the LDS).
 template <int CBT>
-__global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
+__global__ __launch_bounds__(256) void step_product_kernel(StepMulArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int K = a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
+  const int K = a.k0 + (a.a1 ? a.k1 : 0), K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
   float* As = lds;            // [RB][KP]
   constexpr int NCB = CBT / 16, NRB = NCB / 2;
   float* Bs = lds + RB * KP;  // [NCB][kq][16 units][4]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r0 = blockIdx.y * RB, u0 = blockIdx.x * CBT, gate = blockIdx.z;
-  const float* dzg = a.dz + (int64_t)gate * a.H;
+  const int r0 = blockIdx.y * RB, u0 = blockIdx.x * CBT, z = blockIdx.z;
+  const float* a0 = a.a0 + (int64_t)z * a.a0_z_stride;
+  const float* wp = a.wpack + (int64_t)z * a.pack_z_stride;
 
-  // Staging as in the forward kernel: one pass (H up to 384) with every load in flight before the LDS writes.
+  // Staging as in the forward kernel: one pass (K up to 384) with every load in flight before the LDS writes.
   constexpr int NA = 12, NQ = 6;
   for (int pass = 0; pass * 8 * NA < kq; ++pass) {
     f4v va[NA], vb[NCB][NQ];
     const int arow = tid >> 3, bu = tid & 15;
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-      const int q = (pass * NA + i) * 8 + (tid & 7);
+      const int q = (pass * NA + i) * 8 + (tid & 7), k = q * 4;
       va[i] = f4v{0.f, 0.f, 0.f, 0.f};
-      if (q < kq && r0 + arow < a.rows && q * 4 < K) va[i] = *(const f4v*)(dzg + (int64_t)(r0 + arow) * 4 * a.H + q * 4);
+      if (q < kq && r0 + arow < a.rows && k < K)
+        va[i] = k < a.k0 ? *(const f4v*)(a0 + (int64_t)(r0 + arow) * a.ld0 + k) : *(const f4v*)(a.a1 + (int64_t)(r0 + arow) * a.ld1 + (k - a.k0));
     }
     if (pass * 16 * NQ < kq) {
 #pragma unroll
@@ -237,7 +251,7 @@ __global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
         for (int i = 0; i < NQ; ++i) {
           const int q = (pass * NQ + i) * 16 + (tid >> 4), ublk = (u0 >> 4) + wv;
           vb[wv][i] = f4v{0.f, 0.f, 0.f, 0.f};
-          if (q < kq && ublk * 16 < a.H) vb[wv][i] = *(const f4v*)(a.wpack + ((((int64_t)gate * (a.H / 16) + ublk) * kq + q) * 16 + bu) * 4);
+          if (q < kq && ublk * 16 < a.cols) vb[wv][i] = *(const f4v*)(wp + (((int64_t)ublk * a.kq_pack + q) * 16 + bu) * 4);
         }
     }
 #pragma unroll
@@ -264,14 +278,14 @@ __global__ __launch_bounds__(256) void lstm_step_dh_kernel(StepDhArgs a) {
   multiply_blocks<NRB>(As, Bs, K16, cb, rb0, lane, acc);
 
   const int col = u0 + cb * 16 + (lane & 15), g = lane >> 4;
-  if (col < a.H) {
-    float* out = a.dh_parts + (int64_t)gate * a.part_stride;
+  if (col < a.cols) {
+    float* out = a.out + (int64_t)z * a.out_z_stride;
 #pragma unroll
     for (int r = 0; r < NRB; ++r)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int row = r0 + (rb0 + r) * 16 + 4 * g + v;
-        if (row < a.rows) out[(int64_t)row * a.H + col] = acc[r][v];
+        if (row < a.rows) out[(int64_t)row * a.out_ld + col] = acc[r][v];
       }
   }
 }
@@ -286,29 +300,50 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 }  // namespace
 
-bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w) {
+bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w, int gates) {
   if (F % 4 != 0 || H % 16 != 0 || F + H > MAX_K || !aligned16(x)) return false;
-  for (int g = 0; g < 4; ++g)
+  for (int g = 0; g < gates; ++g)
     if (!aligned16(w.wk[g]) || !aligned16(w.wr[g])) return false;
   return true;
 }
 
 int64_t lstm_pack_elems(int F, int H) { return (int64_t)4 * H * round16(F + H); }
 
-int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh) {
+int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh, int gates) {
   if (pack_fwd) {
-    const int64_t cells = (int64_t)H * round16(F + H);
+    const int64_t cells = (int64_t)gates * (H / 4) * round16(F + H);
     LaunchScope scope(ctx, "lstm_pack_weights");
-    hipLaunchKernelGGL(pack_fwd_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, F, H, pack_fwd);
+    hipLaunchKernelGGL(pack_fwd_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, F, H, gates,
+                       pack_fwd);
   }
   if (pack_dh) {
-    const int64_t cells = (int64_t)H * round16(H);
+    const int64_t cells = (int64_t)gates * (H / 4) * round16(H);
     LaunchScope scope(ctx, "lstm_pack_weights");
-    hipLaunchKernelGGL(pack_dh_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, H, pack_dh);
+    hipLaunchKernelGGL(pack_dh_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, H, gates,
+                       pack_dh);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
+
+namespace {
+// 32 units per workgroup (two workgroups per CU) when 64 would leave fewer than two per CU: 10.8 vs 11.4 us per LSTM step
+int launch_step_product(sn_ctx* ctx, const StepMulArgs& a, int zs) {
+  const int K = a.k0 + (a.a1 ? a.k1 : 0);
+  const bool narrow = ceil_div(a.cols, 64) * ceil_div(a.rows, RB) * zs < (int64_t)2 * ctx->compute_units;
+  if (narrow) {
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)step_product_kernel<32>, lds_bytes(MAX_K, 32)));
+    hipLaunchKernelGGL(step_product_kernel<32>, dim3((unsigned)ceil_div(a.cols, 32), (unsigned)ceil_div(a.rows, RB), (unsigned)zs), dim3(256),
+                       lds_bytes(K, 32), ctx->stream, a);
+  } else {
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)step_product_kernel<64>, lds_bytes(MAX_K, 64)));
+    hipLaunchKernelGGL(step_product_kernel<64>, dim3((unsigned)ceil_div(a.cols, 64), (unsigned)ceil_div(a.rows, RB), (unsigned)zs), dim3(256),
+                       lds_bytes(K, 64), ctx->stream, a);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+}  // namespace
 
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h) {
@@ -325,24 +360,23 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
   return SN_OK;
 }
 
-int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride) {
+int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride, int gates) {
   if (rows <= 0) return SN_OK;
   SN_REQUIRE(H % 16 == 0 && H <= MAX_K && aligned16(dz) && aligned16(wpack), "lstm_step_hidden_gradient: H=%d outside what the fused kernel handles", H);
-  StepDhArgs a{dz, wpack, dh_parts, part_stride, rows, H};
-  // 32 units per workgroup (two workgroups per CU) when 64 would leave fewer than two per CU: 10.8 vs 11.4 us per step
-  const bool narrow = ceil_div(H, 64) * ceil_div(rows, RB) * 4 < (int64_t)2 * ctx->compute_units;
-  LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, 4 * H);
-  if (narrow) {
-    SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_dh_kernel<32>, lds_bytes(MAX_K, 32)));
-    hipLaunchKernelGGL(lstm_step_dh_kernel<32>, dim3((unsigned)ceil_div(H, 32), (unsigned)ceil_div(rows, RB), 4), dim3(256), lds_bytes(H, 32),
-                       ctx->stream, a);
-  } else {
-    SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_dh_kernel<64>, lds_bytes(MAX_K, 64)));
-    hipLaunchKernelGGL(lstm_step_dh_kernel<64>, dim3((unsigned)ceil_div(H, 64), (unsigned)ceil_div(rows, RB), 4), dim3(256), lds_bytes(H, 64),
-                       ctx->stream, a);
-  }
-  SN_HIP(hipGetLastError());
-  return SN_OK;
+  const int kq = round16(H) / 4;
+  StepMulArgs a{dz, (int64_t)gates * H, H, nullptr, 0, 0, H, wpack, kq, (int64_t)(H / 16) * kq * 64, dh_parts, H, part_stride, rows, H};
+  LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, gates * H);
+  return launch_step_product(ctx, a, gates);
+}
+
+// r_t[rows, H] = [x_t, r_prev] * [Wk; Wr]: the simple cell's step (pack from launch_lstm_pack(.., gates = 1))
+int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* r_prev, int rows, int H, const float* wpack, float* out) {
+  if (rows <= 0) return SN_OK;
+  SN_REQUIRE(F % 4 == 0 && H % 16 == 0 && F + H <= MAX_K && aligned16(x) && aligned16(wpack) && (!r_prev || aligned16(r_prev)),
+             "rnn_step_forward: F=%d H=%d outside what the fused kernel handles", F, H);
+  StepMulArgs a{x + (int64_t)t * F, (int64_t)T * F, F, r_prev, H, H, 0, wpack, round16(F + H) / 4, 0, out, H, 0, rows, H};
+  LaunchScope scope(ctx, "rnn_step_forward", rows, H, r_prev ? F + H : F);
+  return launch_step_product(ctx, a, 1);
 }
 
 }  // namespace sn

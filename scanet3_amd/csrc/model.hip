@@ -426,6 +426,8 @@ static int alloc_replica(sn_replica* r) {
       const int64_t bh = B * op.H;
       SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = the initial state
       SN_TRY(dev_alloc(r, &r->lstm_dz[i], (int64_t)op.T * bh));
+      SN_TRY(dev_alloc(r, &r->lstm_pk_fwd[i], lstm_pack_elems(op.F, op.H) / 4));  // one gate
+      SN_TRY(dev_alloc(r, &r->lstm_pk_dh[i], lstm_pack_elems(op.F, op.H) / 4));
       SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
     }
     if (op.kind == OP_POOL) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
@@ -577,9 +579,14 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         // output act(r + b) leaves the layer (RNN.scala:60-77 without returnSequence).
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);  // slot 0 only, no bias inside the recurrence
-        for (int t = 0; t < op.T; ++t)
-          SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, t == 0 ? nullptr : r->lstm_h[i] + (int64_t)t * bh, rows, op.H, w,
-                               r->lstm_h[i] + (int64_t)(t + 1) * bh, r->ws, m->workspace_elems, 1));
+        const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
+        if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr, 1));
+        for (int t = 0; t < op.T; ++t) {
+          const float* r_prev = t == 0 ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
+          float* r_t = r->lstm_h[i] + (int64_t)(t + 1) * bh;
+          if (fused) SN_TRY(launch_rnn_step_fwd(ctx, in, t, op.T, op.F, r_prev, rows, op.H, r->lstm_pk_fwd[i], r_t));
+          else SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, r_prev, rows, op.H, w, r_t, r->ws, m->workspace_elems, 1));
+        }
         SN_TRY(launch_bias_act(ctx, r->lstm_h[i] + (int64_t)op.T * bh, param_ptr(r, r->w, op.b), r->act[i], rows, op.H, op.act, op.act_param));
         break;
       }
@@ -750,10 +757,15 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         float* dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
         SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dr, (int64_t)rows * op.H, op.act, op.act_param));
         if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dr, op.H, param_ptr(r, r->g, op.b), rows, op.H, r->ws, m->workspace_elems));
+        const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
+        if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));
         for (int t = op.T - 1; t >= 0; --t) {
           dr = r->lstm_dz[i] + (int64_t)t * bh;
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, dr, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
-          if (t > 0) SN_TRY(launch_lstm_dh(ctx, dr, rows, op.H, w, dr - bh, r->ws, m->workspace_elems, 1));
+          if (t > 0) {
+            if (fused) SN_TRY(launch_lstm_step_dh(ctx, dr, rows, op.H, r->lstm_pk_dh[i], dr - bh, 0, 1));
+            else SN_TRY(launch_lstm_dh(ctx, dr, rows, op.H, w, dr - bh, r->ws, m->workspace_elems, 1));
+          }
         }
         LstmGrads gr{};
         gr.wk[0] = param_ptr(r, r->g, op.lstm_p[0][0]);
