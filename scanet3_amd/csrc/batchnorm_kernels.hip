@@ -213,11 +213,22 @@ __global__ __launch_bounds__(256) void bn_grad_finish_kernel(const float* __rest
   k2[c] = rr * rr * s2 / n;
 }
 
-// dx = inv * (dy - k1 - (x - mean) * k2)
+// Gradient of the activation that produced x (the layer below), from its output: models/Activation.scala:32-83.
+__device__ __forceinline__ float below_act_grad(int act, float y, float dy, float param) {
+  switch (act) {
+    case SN_ACT_SIGMOID: return (y * (1.0f - y)) * dy;
+    case SN_ACT_TANH: return (1.0f - y * y) * dy;
+    case SN_ACT_RELU: return (param < y ? 1.0f : 0.0f) * dy;
+    default: return dy;
+  }
+}
+
+// dx = inv * (dy - k1 - (x - mean) * k2), then (act != identity) through the activation of the layer that wrote x
 template <bool V4>
 __global__ __launch_bounds__(256) void bn_dx_kernel(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ mean,
                                                      const float* __restrict__ inv, const float* __restrict__ k1,
-                                                     const float* __restrict__ k2, float* __restrict__ dx, int64_t n, int cols) {
+                                                     const float* __restrict__ k2, float* __restrict__ dx, int64_t n, int cols, int act,
+                                                     float act_param) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   if (V4) {
     const int64_t n4 = n / 4;
@@ -227,13 +238,13 @@ __global__ __launch_bounds__(256) void bn_dx_kernel(const float* __restrict__ x,
                   mv = *(const bn_f4*)(mean + c), a = *(const bn_f4*)(k1 + c), b = *(const bn_f4*)(k2 + c);
       bn_f4 o;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = iv[e] * ((gv[e] - a[e]) - (xv[e] - mv[e]) * b[e]);
+      for (int e = 0; e < 4; ++e) o[e] = below_act_grad(act, xv[e], iv[e] * ((gv[e] - a[e]) - (xv[e] - mv[e]) * b[e]), act_param);
       *(bn_f4*)(dx + i * 4) = o;
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
       const int c = (int)(i % cols);
-      dx[i] = inv[c] * ((dy[i] - k1[c]) - (x[i] - mean[c]) * k2[c]);
+      dx[i] = below_act_grad(act, x[i], inv[c] * ((dy[i] - k1[c]) - (x[i] - mean[c]) * k2[c]), act_param);
     }
   }
 }
@@ -350,7 +361,7 @@ int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, in
 }
 
 int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx, int64_t rows, int cols, const BatchNormArgs& a,
-                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems) {
+                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems, int below_act, float below_act_param) {
   if (rows <= 0 || cols <= 0) return SN_OK;
   const int64_t half = (int64_t)max_slices(ctx, rows, cols) * cols;
   SN_REQUIRE(2 * half <= ws_elems, "batch norm gradient needs %lld workspace elements, %lld given", (long long)(2 * half), (long long)ws_elems);
@@ -368,10 +379,10 @@ int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx
     LaunchScope scope(ctx, "batchnorm_input_gradient");
     if (vec4_ok(cols, {x, dy, dx, a.mean, a.inv, a.k1, a.k2}))
       hipLaunchKernelGGL((bn_dx_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
-                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols);
+                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
     else
       hipLaunchKernelGGL((bn_dx_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
-                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols);
+                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;

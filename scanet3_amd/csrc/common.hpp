@@ -179,9 +179,11 @@ int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols);
 // y = (x*inv - mean*inv) + beta; training: batch statistics, else the moving ones
 int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, int cols, const BatchNormArgs& a, bool training, float* ws,
                          int64_t ws_elems);
-// gradients of beta, gamma and (dx != null) the input, through the batch statistics
+// gradients of beta, gamma and (dx != null) the input, through the batch statistics; with below_act the input
+// gradient also passes through the activation that produced x (x is that activation's output)
 int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx, int64_t rows, int cols, const BatchNormArgs& a,
-                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems);
+                         float* dbeta, float* dgamma, float* ws, int64_t ws_elems, int below_act = SN_ACT_IDENTITY,
+                         float below_act_param = 0.f);
 // moving = momentum*moving + (1-momentum)*batch
 int launch_batchnorm_moving(sn_ctx* ctx, const BatchNormArgs& a, float* moving_mean, float* moving_var, int cols);
 

@@ -744,8 +744,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
       }
       case OP_BATCHNORM: {
         const int c = (int)op.out_dims.back();
+        // a convolution right below: its activation gradient rides along in the input-gradient pass (x is its output)
+        const bool fuse = need_dx && m->ops[i - 1].kind == OP_CONV && m->ops[i - 1].act != SN_ACT_IDENTITY;
         SN_TRY(launch_batchnorm_bwd(ctx, in, dy, need_dx ? dx : nullptr, (int64_t)rows * (op.out_elems / c), c, batchnorm_args(r, op, i),
-                                    param_ptr(r, r->g, op.bn_p[0]), param_ptr(r, r->g, op.bn_p[1]), r->ws, m->workspace_elems));
+                                    param_ptr(r, r->g, op.bn_p[0]), param_ptr(r, r->g, op.bn_p[1]), r->ws, m->workspace_elems,
+                                    fuse ? m->ops[i - 1].act : SN_ACT_IDENTITY, fuse ? m->ops[i - 1].act_param : 0.f));
+        act_grad_done = fuse;
         if (need_dx) cur ^= 1;
         break;
       }
