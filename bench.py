@@ -298,6 +298,23 @@ def bench_optim(S, ctx, steps, warmup, n=100_000_000, k=8, n_avg=25_000_000):
                       "frac_of_peak": 8 * n_avg / avg_s / 1e9 / PEAK_HBM_GBS}
     for b in reps_bufs + [dst]:
         b.free()
+    # seeded initializer draws (TensorFlow-compatible Philox streams): 4 bytes written per element
+    from scanet3_amd import _lib as L
+    rbuf = ctx.alloc(n)
+    for label, dist in (("random_uniform", L.RANDOM_UNIFORM), ("random_normal", L.RANDOM_NORMAL),
+                        ("random_truncated_normal", L.RANDOM_TRUNCATED_NORMAL)):
+        ctx.random_fill(rbuf, dist, 7)
+        ctx.sync()
+        ctx.profile_reset()
+        ctx.profile(True)
+        for _ in range(steps):
+            ctx.random_fill(rbuf, dist, 7, 0.1, -0.05)
+        ctx.profile(False)
+        kern = ctx.profile_report()[label]
+        avg_s = kern[0] / kern[1] * 1e-3
+        out[label] = {"n": n, "bytes_per_elem": 4, "kernel_avg_us": avg_s * 1e6, "GBps": 4 * n / avg_s / 1e9,
+                      "frac_of_peak": 4 * n / avg_s / 1e9 / PEAK_HBM_GBS, "elems_per_s": n / avg_s}
+    rbuf.free()
     return {"workload": f"fused optimizer updates over {n} fp32 params + average of {k} x {n_avg}", "n": n, "results": out}
 
 

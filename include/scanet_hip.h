@@ -68,6 +68,8 @@ enum { SN_REG_NONE = 0, SN_REG_L1 = 1, SN_REG_L2 = 2 };
 /* optimizers/{SGD,AdaGrad,AdaDelta,RMSProp,Adam,Nadam,Adamax,AMSGrad}.scala */
 enum { SN_OPT_SGD = 0, SN_OPT_ADAGRAD = 1, SN_OPT_ADADELTA = 2, SN_OPT_RMSPROP = 3,
        SN_OPT_ADAM = 4, SN_OPT_NADAM = 5, SN_OPT_ADAMAX = 6, SN_OPT_AMSGRAD = 7 };
+/* math/rand/AllKernels.scala:45-50 (Dist) */
+enum { SN_RANDOM_UNIFORM = 0, SN_RANDOM_NORMAL = 1, SN_RANDOM_TRUNCATED_NORMAL = 2 };
 /* model flags */
 enum {
   SN_FLAG_GEMM_BF16 = 1,       /* Dense GEMMs take bf16 inputs (fp32 accumulate, fp32 master weights) */
@@ -248,6 +250,14 @@ SN_API int sn_optimizer_update(sn_ctx* ctx, const sn_optimizer_desc* opt, float*
 /* `Aggregation.Avg` over k inputs (models/Aggregation.scala:16-19): out = (in[0] + .. + in[k-1]) / k,
  * accumulated left to right. `inputs_host` is a host array of k device pointers; out may alias in[0]. */
 SN_API int sn_average(sn_ctx* ctx, const float* const* inputs_host, int32_t k, int64_t n, float* out_dev);
+
+/* `rand(shape, dist, seed, scale, shift)` (math/rand/AllKernels.scala:68-81), the draw under every seeded
+ * initializer of models/Initializer.scala:48-219: n values of the TensorFlow op the reference lowers to
+ * (RandomUniform in [0,1), RandomStandardNormal, TruncatedNormal at two standard deviations) for op seed
+ * `seed` (non-zero), then `* scale` and `+ shift` where the pointers are not NULL. The stream is the one
+ * TensorFlow's CPU kernels produce, so the same seed gives the reference's initial weights. */
+SN_API int sn_random_fill(sn_ctx* ctx, float* dst_dev, int64_t n, int32_t dist, uint64_t seed, const float* scale_host,
+                          const float* shift_host);
 
 /* ---------------------------------------------------------------- per-kernel timing */
 

@@ -975,3 +975,143 @@ def count_correct(model, x, y, params):
     p = rint(model.forward(x, params))
     matched = (y == p).astype(np.int32).sum(axis=1)
     return int((matched == model.out_shape(x.shape)[-1]).astype(np.int32).sum())
+
+
+# --------------------------------------------------------------------------- #
+# seeded initializers (models/Initializer.scala over math/rand/AllKernels.scala)
+# --------------------------------------------------------------------------- #
+# The reference draws with TensorFlow's RandomUniform / RandomStandardNormal / TruncatedNormal ops and their `seed`
+# attribute (math/rand/AllKernels.scala:12-43).  TensorFlow is a dependency that does not ship with the reference
+# (build.sbt:13, "org.tensorflow" % "tensorflow-core-platform" % "0.5.0", i.e. TensorFlow 2.10): what follows restates
+# the published algorithm of those CPU kernels (tensorflow/core/lib/random/philox_random.h, random_distributions.h,
+# kernels/random_op_cpu.h): Philox4x32-10 keyed by the op seed (seed2 = 0), counter = output group, four outputs per
+# counter, uint32 -> [0,1) through the float mantissa, Box-Muller for normals, and for the truncated normal a
+# rejection loop per group of four outputs that starts 256 counters after the previous group's start.
+# Pinned by the values models/InitializerSpec.scala:23-66 records for seeds 1 and 2.
+
+_M32 = np.uint64(0xFFFFFFFF)
+
+
+def philox4x32_10(counter: np.ndarray, key: Tuple[int, int]) -> np.ndarray:
+    """counter: uint32 [n, 4]; returns uint32 [n, 4] (philox_random.h: ten rounds, key raised between rounds)."""
+    c = counter.astype(np.uint64)
+    k0, k1 = np.uint64(key[0]), np.uint64(key[1])
+    for rnd in range(10):
+        if rnd:
+            k0 = (k0 + np.uint64(0x9E3779B9)) & _M32
+            k1 = (k1 + np.uint64(0xBB67AE85)) & _M32
+        p0 = np.uint64(0xD2511F53) * c[:, 0]
+        p1 = np.uint64(0xCD9E8D57) * c[:, 2]
+        c = np.stack([(p1 >> np.uint64(32)) ^ c[:, 1] ^ k0, p1 & _M32, (p0 >> np.uint64(32)) ^ c[:, 3] ^ k1, p0 & _M32], axis=1)
+    return c.astype(np.uint32)
+
+
+def _philox_blocks(seed: int, first: np.ndarray) -> np.ndarray:
+    """Outputs of the counters `first` (uint64 [n]) under PhiloxRandom(seed, 0): key = the seed's two halves."""
+    ctr = np.zeros((first.shape[0], 4), np.uint32)
+    ctr[:, 0] = (first & _M32).astype(np.uint32)
+    ctr[:, 1] = (first >> np.uint64(32)).astype(np.uint32)
+    return philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))
+
+
+def uint32_to_float(x: np.ndarray) -> np.ndarray:
+    """random_distributions.h Uint32ToFloat: 23 mantissa bits under exponent 127, minus one."""
+    return ((x & np.uint32(0x7FFFFF)) | np.uint32(127 << 23)).view(np.float32) - F32(1.0)
+
+
+def box_muller(x0: np.ndarray, x1: np.ndarray):
+    """random_distributions.h BoxMullerFloat."""
+    u1 = np.maximum(uint32_to_float(x0), F32(1.0e-7))
+    v1 = (2.0 * math.pi * uint32_to_float(x1).astype(np.float64)).astype(np.float32)     # `2.0f * M_PI * u` is a double product
+    u2 = np.sqrt(F32(-2.0) * np.log(u1))
+    return np.sin(v1) * u2, np.cos(v1) * u2
+
+
+def tf_random_uniform(n: int, seed: int) -> np.ndarray:
+    groups = np.arange((n + 3) // 4, dtype=np.uint64)
+    return uint32_to_float(_philox_blocks(seed, groups).reshape(-1))[:n]
+
+
+def tf_random_normal(n: int, seed: int) -> np.ndarray:
+    r = _philox_blocks(seed, np.arange((n + 3) // 4, dtype=np.uint64))
+    f0, f1 = box_muller(r[:, 0], r[:, 1])
+    f2, f3 = box_muller(r[:, 2], r[:, 3])
+    return np.stack([f0, f1, f2, f3], axis=1).reshape(-1)[:n]
+
+
+def tf_truncated_normal(n: int, seed: int) -> np.ndarray:
+    """Group g of four outputs reads single samples from counter 256 g on and keeps normals with |f| < 2."""
+    out = np.empty(((n + 3) // 4) * 4, np.float32)
+    for g in range((n + 3) // 4):
+        got, block = 0, 0
+        while got < 4:
+            r = _philox_blocks(seed, np.array([256 * g + block], np.uint64))[0]
+            block += 1
+            for a, b in ((0, 1), (2, 3)):
+                for f in box_muller(r[a:a + 1], r[b:b + 1]):
+                    if got < 4 and abs(float(f[0])) < 2.0:
+                        out[4 * g + got] = f[0]
+                        got += 1
+                if got >= 4:
+                    break
+    return out[:n]
+
+
+def initializer_fans(shape) -> Tuple[int, int]:
+    """Initializer.fans (Initializer.scala:16-25), including its `out :: in :: receptive` reading of rank > 2."""
+    s = list(shape)
+    if not s:
+        return 1, 1
+    if len(s) == 1:
+        return s[0], s[0]
+    if len(s) == 2:
+        return s[0], s[1]
+    size = int(np.prod(s[2:]))
+    return size * s[1], size * s[0]
+
+
+_TRUNC_COEF = F32(0.87962566103423978)     # Initializer.scala:30
+
+
+def tf_rand(shape, dist: str, seed: int, scale=None, shift=None) -> np.ndarray:
+    """`rand` (math/rand/AllKernels.scala:68-81): draw, then `* scale`, then `+ shift`, each only when given."""
+    n = int(np.prod(shape)) if len(shape) else 1
+    x = {"uniform": tf_random_uniform, "normal": tf_random_normal, "truncated": tf_truncated_normal}[dist](n, seed)
+    if scale is not None:
+        x = x * F32(scale)
+    if shift is not None:
+        x = x + F32(shift)
+    return x.reshape(shape)
+
+
+def initialize(name: str, shape, seed: int, **kw) -> np.ndarray:
+    """The seeded initializers of models/Initializer.scala:48-219 by name."""
+    shape = tuple(shape)
+    fan_in, fan_out = initializer_fans(shape)
+    sq = lambda v: F32(math.sqrt(float(F32(v))))            # `math.sqrt(6f / n).toFloat`
+    if name == "RandomUniform":
+        lo, hi = F32(kw.get("min", -0.05)), F32(kw.get("max", 0.05))
+        return tf_rand(shape, "uniform", seed, hi - lo, lo)
+    if name == "RandomNormal":
+        return tf_rand(shape, "normal", seed, kw.get("std", 0.05), kw.get("mean", 0.0))
+    if name == "RandomNormalTruncated":
+        return tf_rand(shape, "truncated", seed, kw.get("std", 0.05), kw.get("mean", 0.0))
+    if name in ("GlorotUniform", "HeUniform", "LecunUniform"):
+        limit = {"GlorotUniform": sq(F32(6.0) / F32(fan_in + fan_out)), "HeUniform": sq(F32(6.0) / F32(fan_in)),
+                 "LecunUniform": sq(F32(3.0) / F32(fan_in))}[name]
+        return tf_rand(shape, "uniform", seed, F32(2.0) * limit, -limit)
+    if name in ("GlorotNormal", "HeNormal", "LecunNormal"):
+        std = {"GlorotNormal": sq(F32(2.0) / F32(fan_in + fan_out)), "HeNormal": sq(F32(2.0) / F32(fan_in)),
+               "LecunNormal": sq(F32(1.0) / F32(fan_in))}[name] / _TRUNC_COEF
+        return tf_rand(shape, "truncated", seed, std)
+    if name == "Orthogonal":                                # Initializer.scala:202-219
+        rows, cols = int(np.prod(shape[:-1])), shape[-1]
+        a = tf_rand((max(rows, cols), min(rows, cols)), "normal", seed)
+        q, r = np.linalg.qr(a)
+        q = q * np.sign(np.diag(r))
+        if rows < cols:
+            q = q.T
+        if kw.get("gain") is not None:
+            q = q * F32(kw["gain"])
+        return q.reshape(shape).astype(np.float32)
+    raise ValueError(name)

@@ -19,6 +19,7 @@ SN_MAX_AVG_INPUTS = 32
 # enums of include/scanet_hip.h
 LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM, LAYER_SIMPLE_RNN, LAYER_BATCHNORM = range(9)
 ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = range(5)
+RANDOM_UNIFORM, RANDOM_NORMAL, RANDOM_TRUNCATED_NORMAL = range(3)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
 PAD_VALID, PAD_SAME = 0, 1
 REG_NONE, REG_L1, REG_L2 = 0, 1, 2
@@ -95,6 +96,7 @@ SIGNATURES = {
     "sn_replicas_average": (C.c_int, [C.POINTER(_P), C.c_int32]),
     "sn_optimizer_update": (C.c_int, [_P, C.POINTER(OptimizerDesc), _P, _P, _P, _P, _P, C.c_int64, C.c_int32]),
     "sn_average": (C.c_int, [_P, C.POINTER(_P), C.c_int32, C.c_int64, _P]),
+    "sn_random_fill": (C.c_int, [_P, _P, C.c_int64, C.c_int32, C.c_uint64, _F, _F]),
     "sn_profile_enable": (C.c_int, [_P, C.c_int32]),
     "sn_profile_reset": (C.c_int, [_P]),
     "sn_profile_count": (C.c_int, [_P, C.POINTER(C.c_int32)]),

@@ -82,6 +82,24 @@ class Context:
         arr = (C.c_void_p * len(inputs))(*[b.ptr for b in inputs])
         check(lib.sn_average(self.handle, arr, len(inputs), out.size if n is None else n, out.ptr))
 
+    def random_fill(self, out: "DeviceBuffer", dist: int, seed: int, scale: Optional[float] = None,
+                    shift: Optional[float] = None, n: Optional[int] = None):
+        """`rand(shape, dist, seed, scale, shift)` (math/rand/AllKernels.scala:68-81) with TensorFlow's seeded stream."""
+        sc = None if scale is None else C.byref(C.c_float(scale))
+        sh = None if shift is None else C.byref(C.c_float(shift))
+        ptr = out.ptr if isinstance(out, DeviceBuffer) else out          # a raw device pointer needs `n`
+        count = out.size if n is None else n
+        check(lib.sn_random_fill(self.handle, ptr, count, dist, C.c_uint64(seed), sc, sh))
+
+    def random(self, shape, dist: int, seed: int, scale: Optional[float] = None, shift: Optional[float] = None) -> np.ndarray:
+        shape = tuple(int(d) for d in shape)
+        buf = DeviceBuffer(self, int(np.prod(shape)) if shape else 1, shape)
+        try:
+            self.random_fill(buf, dist, seed, scale, shift)
+            return buf.numpy()
+        finally:
+            buf.free()
+
     # ---- per-kernel timing ------------------------------------------------------
     def profile(self, on: bool):
         check(lib.sn_profile_enable(self.handle, 1 if on else 0))

@@ -160,6 +160,9 @@ struct LstmGateBwdArgs {
 };
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
 
+// ---- seeded random tensors (random_kernels.hip): scale / shift may be null
+int launch_random_fill(sn_ctx* ctx, float* out, int64_t n, int dist, uint64_t seed, const float* scale, const float* shift);
+
 // ---- batch normalisation over the last axis (batchnorm_kernels.hip) ---------------------
 struct BatchNormArgs {
   const float* gamma;        // [C]

@@ -233,6 +233,13 @@ int sn_average(sn_ctx* ctx, const float* const* inputs_host, int32_t k, int64_t 
   return launch_average(ctx, in, k, n, out_dev, nullptr, 0);
 }
 
+int sn_random_fill(sn_ctx* ctx, float* dst_dev, int64_t n, int32_t dist, uint64_t seed, const float* scale_host, const float* shift_host) {
+  SN_TRY(check_ctx(ctx));
+  SN_REQUIRE(dst_dev || n == 0, "sn_random_fill: null pointer");
+  SN_REQUIRE(n >= 0, "sn_random_fill: negative length");
+  return launch_random_fill(ctx, dst_dev, n, dist, seed, scale_host, shift_host);
+}
+
 int sn_profile_enable(sn_ctx* ctx, int32_t on) {
   SN_TRY(check_ctx(ctx));
   if (!on) SN_TRY(profile_drain(ctx));

@@ -100,35 +100,61 @@ def fans(shape: Sequence[int]) -> Tuple[int, int]:
     return size * s[1], size * s[0]
 
 
+_TRUNC_COEF = np.float32(0.87962566103423978)     # Initializer.scala:30
+
+
+def _sqrt32(v) -> np.float32:
+    return np.float32(math.sqrt(float(np.float32(v))))     # `math.sqrt(6f / n).toFloat`
+
+
 @dataclass(frozen=True)
 class Initializer:
-    """Draws come from numpy, not from TensorFlow's Philox stream: seeded values differ from the
-    reference's; the distributions are the same. Use `.initParams(..)` for bit-identical starts."""
+    """models/Initializer.scala:28-219.  Random draws are made on the device by `sn_random_fill`, which produces the
+    stream of the TensorFlow op the reference uses: a seeded initializer gives the reference's values.  Without a
+    seed the reference lets TensorFlow pick one at random; here it is taken from the builder's generator."""
     name: str
     value: float = 0.0
     seed: Optional[int] = None
+    args: Tuple[float, ...] = ()
 
-    def build(self, shape, rng: np.random.Generator) -> np.ndarray:
-        shape = tuple(shape)
+    def build(self, shape, ctx: Context, rng: np.random.Generator) -> np.ndarray:
+        shape = tuple(int(d) for d in shape)
         if self.name == "Zeros":
             return np.zeros(shape, np.float32)
         if self.name == "Ones":
             return np.ones(shape, np.float32)
         if self.name == "Const":
             return np.full(shape, self.value, np.float32)
-        r = np.random.default_rng(self.seed) if self.seed is not None else rng
-        if self.name == "GlorotUniform":                      # Initializer.scala:83-90
-            fan_in, fan_out = fans(shape)
-            limit = np.float32(math.sqrt(np.float32(6.0) / (fan_in + fan_out)))
-            return (r.random(shape, np.float32) * (2 * limit) - limit).astype(np.float32)
-        if self.name == "Orthogonal":                         # Initializer.scala:202-219
+        seed = int(self.seed) if self.seed is not None else int(rng.integers(1, 2 ** 31))
+        fan_in, fan_out = fans(shape)
+        f32 = np.float32
+        if self.name == "RandomUniform":                      # Initializer.scala:48-53
+            lo, hi = f32(self.args[0]), f32(self.args[1])
+            return ctx.random(shape, L.RANDOM_UNIFORM, seed, float(hi - lo), float(lo))
+        if self.name == "RandomNormal":                       # :55-60
+            return ctx.random(shape, L.RANDOM_NORMAL, seed, self.args[1], self.args[0])
+        if self.name == "RandomNormalTruncated":              # :62-70
+            return ctx.random(shape, L.RANDOM_TRUNCATED_NORMAL, seed, self.args[1], self.args[0])
+        if self.name in ("GlorotUniform", "HeUniform", "LecunUniform"):     # :83-90, 121-128, 159-166
+            limit = {"GlorotUniform": _sqrt32(f32(6.0) / f32(fan_in + fan_out)), "HeUniform": _sqrt32(f32(6.0) / f32(fan_in)),
+                     "LecunUniform": _sqrt32(f32(3.0) / f32(fan_in))}[self.name]
+            return ctx.random(shape, L.RANDOM_UNIFORM, seed, float(f32(2.0) * limit), float(-limit))
+        if self.name in ("GlorotNormal", "HeNormal", "LecunNormal"):        # :103-110, 140-147, 178-185
+            std = {"GlorotNormal": _sqrt32(f32(2.0) / f32(fan_in + fan_out)), "HeNormal": _sqrt32(f32(2.0) / f32(fan_in)),
+                   "LecunNormal": _sqrt32(f32(1.0) / f32(fan_in))}[self.name] / _TRUNC_COEF
+            return ctx.random(shape, L.RANDOM_TRUNCATED_NORMAL, seed, float(std))
+        if self.name == "Orthogonal":                         # :202-219; the QR of the small matrix stays on the host
+            if len(shape) < 2:
+                raise ValueError(f"requirement failed: at least rank 2 is required but was {len(shape)}")
             rows, cols = int(np.prod(shape[:-1])), shape[-1]
-            a = r.standard_normal((max(rows, cols), min(rows, cols)))
+            a = ctx.random((max(rows, cols), min(rows, cols)), L.RANDOM_NORMAL, seed)
             q, rr = np.linalg.qr(a)
             q = q * np.sign(np.diag(rr))
             if rows < cols:
                 q = q.T
-            return q.reshape(shape).astype(np.float32)
+            if self.args:
+                q = q * np.float32(self.args[0])
+            return np.ascontiguousarray(q.reshape(shape), np.float32)
         raise ValueError(self.name)
 
 
@@ -139,12 +165,44 @@ def Const(v: float) -> Initializer:
     return Initializer("Const", float(v))
 
 
+def RandomUniform(min: float = -0.05, max: float = 0.05, seed: Optional[int] = None) -> Initializer:
+    return Initializer("RandomUniform", seed=seed, args=(float(min), float(max)))
+
+
+def RandomNormal(mean: float = 0.0, std: float = 0.05, seed: Optional[int] = None) -> Initializer:
+    return Initializer("RandomNormal", seed=seed, args=(float(mean), float(std)))
+
+
+def RandomNormalTruncated(mean: float = 0.0, std: float = 0.05, seed: Optional[int] = None) -> Initializer:
+    return Initializer("RandomNormalTruncated", seed=seed, args=(float(mean), float(std)))
+
+
 def GlorotUniform(seed: Optional[int] = None) -> Initializer:
     return Initializer("GlorotUniform", seed=seed)
 
 
-def Orthogonal(seed: Optional[int] = None) -> Initializer:
-    return Initializer("Orthogonal", seed=seed)
+def GlorotNormal(seed: Optional[int] = None) -> Initializer:
+    return Initializer("GlorotNormal", seed=seed)
+
+
+def HeUniform(seed: Optional[int] = None) -> Initializer:
+    return Initializer("HeUniform", seed=seed)
+
+
+def HeNormal(seed: Optional[int] = None) -> Initializer:
+    return Initializer("HeNormal", seed=seed)
+
+
+def LecunUniform(seed: Optional[int] = None) -> Initializer:
+    return Initializer("LecunUniform", seed=seed)
+
+
+def LecunNormal(seed: Optional[int] = None) -> Initializer:
+    return Initializer("LecunNormal", seed=seed)
+
+
+def Orthogonal(gain: Optional[float] = None, seed: Optional[int] = None) -> Initializer:
+    return Initializer("Orthogonal", seed=seed, args=() if gain is None else (float(gain),))
 
 
 # --------------------------------------------------------------------------- layers
@@ -369,24 +427,24 @@ def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndar
     for i, l in enumerate(layers):
         pre = "" if single else f"{i}/"
         if l.kind in (L.LAYER_DENSE, L.LAYER_BIAS, L.LAYER_CONV2D):
-            out[pre + "weights"] = l.inits[0].build(shapes[pre + "weights"], rng)
+            out[pre + "weights"] = l.inits[0].build(shapes[pre + "weights"], compiled.ctx, rng)
         elif l.kind == L.LAYER_BATCHNORM:
             for name, init in zip(("beta", "gamma", "moving_mean", "moving_variance"), l.inits):
-                out[pre + name] = init.build(shapes[pre + name], rng)
+                out[pre + name] = init.build(shapes[pre + name], compiled.ctx, rng)
         elif l.kind == L.LAYER_SIMPLE_RNN:
             k_init, r_init, b_init = l.inits
-            out[pre + "0/kernel_weights"] = k_init.build(shapes[pre + "0/kernel_weights"], rng)
-            out[pre + "0/recurrent_weights"] = r_init.build(shapes[pre + "0/recurrent_weights"], rng)
+            out[pre + "0/kernel_weights"] = k_init.build(shapes[pre + "0/kernel_weights"], compiled.ctx, rng)
+            out[pre + "0/recurrent_weights"] = r_init.build(shapes[pre + "0/recurrent_weights"], compiled.ctx, rng)
             if l.use_bias:
-                out[pre + "1/weights"] = b_init.build(shapes[pre + "1/weights"], rng)
+                out[pre + "1/weights"] = b_init.build(shapes[pre + "1/weights"], compiled.ctx, rng)
         elif l.kind == L.LAYER_LSTM:
             k_init, r_init, b_init, bf_init = l.inits
             for gate in ("forget", "input", "gate", "output"):
-                out[f"{pre}{gate}/0/kernel_weights"] = k_init.build(shapes[f"{pre}{gate}/0/kernel_weights"], rng)
-                out[f"{pre}{gate}/0/recurrent_weights"] = r_init.build(shapes[f"{pre}{gate}/0/recurrent_weights"], rng)
+                out[f"{pre}{gate}/0/kernel_weights"] = k_init.build(shapes[f"{pre}{gate}/0/kernel_weights"], compiled.ctx, rng)
+                out[f"{pre}{gate}/0/recurrent_weights"] = r_init.build(shapes[f"{pre}{gate}/0/recurrent_weights"], compiled.ctx, rng)
                 if l.use_bias:
                     b = bf_init if gate == "forget" else b_init
-                    out[f"{pre}{gate}/1/weights"] = b.build(shapes[f"{pre}{gate}/1/weights"], rng)
+                    out[f"{pre}{gate}/1/weights"] = b.build(shapes[f"{pre}{gate}/1/weights"], compiled.ctx, rng)
     return out
 
 

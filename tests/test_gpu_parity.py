@@ -805,3 +805,82 @@ def test_bf16_dense_path_matches_bf16_rounded_oracle(S, ctx, dims, batch):
     h.close()
     xb.free()
     yb.free()
+
+
+# ----------------------------------------------------------------------------- seeded initializers (TensorFlow's Philox streams)
+def test_golden_seeded_initializers(S, ctx, golden):
+    """InitializerSpec.scala:23-66 through the DSL's initializers, which draw on the device."""
+    made = {"RandomUniform": S.RandomUniform, "RandomNormal": S.RandomNormal, "RandomNormalTruncated": S.RandomNormalTruncated,
+            "GlorotUniform": S.GlorotUniform, "GlorotNormal": S.GlorotNormal, "Orthogonal": S.Orthogonal}
+    rng = np.random.default_rng(0)
+    for case in golden["initializers"]["cases"]:
+        init = made[case["name"]](seed=case["seed"], **case["args"])
+        out = init.build(tuple(case["shape"]), ctx, rng)
+        assert out.dtype == np.float32 and out.shape == tuple(case["shape"])
+        np.testing.assert_array_equal(round_at(out, case["digits"]), A(case["out"]), err_msg=case["name"])
+    # a model's parameters, as `ParamDef.initialize` would draw them (Optimizer.scala:124-128)
+    from scanet3_amd.dsl import _init_params
+    model = S.Conv2D(4, kernelInitializer=S.HeNormal(seed=5)) >> S.Flatten >> S.Dense(3, kernelInitializer=S.GlorotUniform(seed=6)) \
+        >> S.Activate(S.Tanh)
+    cm = S.CompiledModel(ctx, [l.desc() for l in model.layers], S.MeanSquaredError.kind, (5, 5, 2), 4)
+    params = _init_params(model, cm, 0)
+    np.testing.assert_allclose(params["0/weights"], O.initialize("HeNormal", (3, 3, 2, 4), 5), rtol=0, atol=4e-6)
+    np.testing.assert_array_equal(params["2/weights"], O.initialize("GlorotUniform", (36, 3), 6))
+    np.testing.assert_array_equal(params["3/weights"], np.zeros(3, f32))
+    cm.close()
+    lstm = S.LSTM(4, recurrentInitializer=S.Orthogonal(seed=8))
+    cm = S.CompiledModel(ctx, [lstm.desc()], S.MeanSquaredError.kind, (3, 2), 4)
+    params = _init_params(lstm, cm, 0)
+    np.testing.assert_allclose(params["forget/0/recurrent_weights"], O.initialize("Orthogonal", (4, 4), 8), rtol=0, atol=2e-6)
+    np.testing.assert_array_equal(params["forget/1/weights"], np.ones(4, f32))       # forget bias one (RNN.scala:262-265)
+    cm.close()
+    assert np.array_equal(S.Zeros.build((2, 2), ctx, rng), np.zeros((2, 2), f32))
+    assert np.array_equal(S.Const(0.5).build((3,), ctx, rng), np.full(3, 0.5, f32))
+
+
+@pytest.mark.parametrize("n", [1, 3, 5, 1000, (1 << 20) + 3])
+def test_random_streams_match_oracle(S, ctx, n):
+    from scanet3_amd import _lib as L
+    seed = 1234567 + n
+    np.testing.assert_array_equal(ctx.random((n,), L.RANDOM_UNIFORM, seed), O.tf_random_uniform(n, seed))      # integer work + exact float ops
+    np.testing.assert_array_equal(ctx.random((n,), L.RANDOM_UNIFORM, seed, 0.25, -3.0), O.tf_rand((n,), "uniform", seed, 0.25, -3.0))
+    # log / sin / cos come from different maths libraries: a few ulp on values up to ~5
+    np.testing.assert_allclose(ctx.random((n,), L.RANDOM_NORMAL, seed), O.tf_random_normal(n, seed), rtol=0, atol=4e-6)
+    m = min(n, 4000)                                                     # the oracle's rejection loop is plain Python
+    got, ref = ctx.random((m,), L.RANDOM_TRUNCATED_NORMAL, seed, 0.5, 1.0), O.tf_rand((m,), "truncated", seed, 0.5, 1.0)
+    np.testing.assert_allclose(got, ref, rtol=0, atol=4e-6)
+
+
+def test_random_streams_large_seed_unaligned_and_errors(S, ctx):
+    from scanet3_amd import _lib as L
+    seed = (7 << 32) | 9                                                  # both halves of the key
+    n = 1001
+    big = ctx.alloc(n + 1)
+    big.fill(-1.0)
+    ctx.random_fill(big.offset(1), L.RANDOM_UNIFORM, seed, n=n)           # 4 bytes off a 16-byte boundary
+    got = big.numpy()
+    assert got[0] == -1.0
+    np.testing.assert_array_equal(got[1:], O.tf_random_uniform(n, seed))
+    big.free()
+    with pytest.raises(S.ScanetError, match="seed 0"):
+        ctx.random((4,), L.RANDOM_UNIFORM, 0)
+    with pytest.raises(S.ScanetError, match="distribution"):
+        ctx.random((4,), 7, 1)
+
+
+def test_random_stream_full_size(S, ctx):
+    """100 M draws (the size of the optimizer sweep): the last group is the generator block at its own counter,
+    and the moments are those of the distribution."""
+    from scanet3_amd import _lib as L
+    n, seed = 100_000_000, 42
+    buf = ctx.alloc(n)
+    ctx.random_fill(buf, L.RANDOM_UNIFORM, seed)
+    u = buf.numpy()
+    g = n // 4 - 1
+    np.testing.assert_array_equal(u[4 * g:4 * g + 4], O.uint32_to_float(O._philox_blocks(seed, np.array([g], np.uint64))[0]))
+    assert abs(float(u.mean(dtype=np.float64)) - 0.5) < 1e-4 and abs(float(u.var(dtype=np.float64)) - 1 / 12) < 1e-4
+    ctx.random_fill(buf, L.RANDOM_TRUNCATED_NORMAL, seed)
+    t = buf.numpy()
+    assert float(np.abs(t).max()) < 2.0 and abs(float(t.std(dtype=np.float64)) - 0.87962566) < 2e-4
+    np.testing.assert_allclose(t[:64], O.tf_truncated_normal(64, seed), rtol=0, atol=4e-6)
+    buf.free()

@@ -280,6 +280,41 @@ def test_batch_norm_state_bypasses_the_algorithm(golden):
     np.testing.assert_allclose(out.var(axis=0), 1.0, atol=1e-3)      # var / (var + epsilon)
 
 
+def test_seeded_initializers_golden(golden):
+    """InitializerSpec.scala:23-66: TensorFlow's seeded streams, restated."""
+    for case in golden["initializers"]["cases"]:
+        out = O.initialize(case["name"], tuple(case["shape"]), case["seed"], **case["args"])
+        assert out.dtype == np.float32 and out.shape == tuple(case["shape"])
+        np.testing.assert_array_equal(round_at(out, case["digits"]), A(case["out"]), err_msg=case["name"])
+
+
+def test_seeded_streams_structure():
+    """What the goldens (3 values each) leave open, fixed by the construction: four outputs per counter whatever the
+    length asked for, Philox's published known-answer vector, the truncation, the moments."""
+    # Random123 known-answer test for philox4x32-10: zero counter and key; and the all-ones one
+    kat = O.philox4x32_10(np.zeros((1, 4), np.uint32), (0, 0))[0]
+    assert [hex(int(v)) for v in kat] == ["0x6627e8d5", "0xe169c58d", "0xbc57ac4c", "0x9b00dbd8"]
+    kat = O.philox4x32_10(np.full((1, 4), 0xFFFFFFFF, np.uint32), (0xFFFFFFFF, 0xFFFFFFFF))[0]
+    assert [hex(int(v)) for v in kat] == ["0x408f276d", "0x41c83b0e", "0xa20bc7c6", "0x6d5451fd"]
+    for fn in (O.tf_random_uniform, O.tf_random_normal, O.tf_truncated_normal):
+        np.testing.assert_array_equal(fn(1001, 5)[:37], fn(37, 5))          # a prefix does not depend on the length
+        assert not np.array_equal(fn(16, 5), fn(16, 6))
+    u = O.tf_random_uniform(200000, 3)
+    assert 0.0 <= u.min() and u.max() < 1.0 and abs(u.mean() - 0.5) < 2e-3 and abs(u.var() - 1 / 12) < 1e-3
+    z = O.tf_random_normal(200000, 3)
+    assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3
+    t = O.tf_truncated_normal(8000, 3)
+    assert np.abs(t).max() < 2.0 and abs(t.std() - 0.8796) < 2e-2
+    # the first group of the truncated stream is the normal stream with rejections removed
+    zn = O.tf_random_normal(64, 11)
+    np.testing.assert_array_equal(O.tf_truncated_normal(4, 11), zn[np.abs(zn) < 2.0][:4])
+    q = O.initialize("Orthogonal", (5, 3), 4)
+    np.testing.assert_allclose(q.T @ q, np.eye(3), atol=1e-6)
+    q = O.initialize("Orthogonal", (3, 5), 4, gain=2.0)
+    np.testing.assert_allclose(q @ q.T, 4.0 * np.eye(3), atol=1e-5)
+    assert O.initializer_fans((3, 3, 2, 8)) == (16 * 3, 16 * 3)              # `out :: in :: receptive` (Initializer.scala:20-23)
+
+
 def _lstm_params(g, pre=""):
     p = {}
     for gate in O.GATES:
