@@ -70,6 +70,8 @@ enum { SN_OPT_SGD = 0, SN_OPT_ADAGRAD = 1, SN_OPT_ADADELTA = 2, SN_OPT_RMSPROP =
        SN_OPT_ADAM = 4, SN_OPT_NADAM = 5, SN_OPT_ADAMAX = 6, SN_OPT_AMSGRAD = 7 };
 /* math/rand/AllKernels.scala:45-50 (Dist) */
 enum { SN_RANDOM_UNIFORM = 0, SN_RANDOM_NORMAL = 1, SN_RANDOM_TRUNCATED_NORMAL = 2 };
+/* error terms of the regression estimators (estimators/package.scala:56-70) */
+enum { SN_ERROR_SQUARED = 0, SN_ERROR_ABSOLUTE = 1 };
 /* model flags */
 enum {
   SN_FLAG_GEMM_BF16 = 1,       /* Dense GEMMs take bf16 inputs (fp32 accumulate, fp32 master weights) */
@@ -222,6 +224,10 @@ SN_API int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int3
 /* Per-batch body of `estimators.accuracy` (estimators/package.scala:28-32): rows whose every
  * rounded (half to even) output equals the label. */
 SN_API int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int64_t* count_host);
+/* Per-batch body of `estimators.MSE` / `RMSE` / `MAE` (estimators/package.scala:50-101, `errorSum`): the sum over
+ * every output element of (predicted - expected)^2 or |predicted - expected| for the frozen model; the caller
+ * adds the sums of its batches and divides by the row count as the reference does. */
+SN_API int sn_error_sum(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t kind, float* sum_host);
 /* `optimizeOnPartition` (optimizers/Optimizer.scala:106-161) over a device-resident partition of
  * `total_rows` samples: every full batch in order with iter = global_iter + i + 1, partial batch
  * skipped (optimizers/Iterators.scala:90), then the loss of the last batch under the updated

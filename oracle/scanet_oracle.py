@@ -969,6 +969,28 @@ def train(model, alg, partitions, batch, epochs, init_params, avg="uniform"):
     return params, opt_state, history
 
 
+def error_sum(model, x, y, params, absolute=False):
+    """`errorSum` of the regression estimators (estimators/package.scala:80-84): sum over every output element of
+    (predicted - expected)^2 (MSE, :56-62) or |predicted - expected| (MAE, :64-70) for the frozen model."""
+    d = model.forward(x, params) - y
+    return (np.abs(d) if absolute else sqr(d)).sum(dtype=d.dtype)
+
+
+def mean_error(model, X, Y, params, batch=1000, absolute=False):
+    """`meanError` (estimators/package.scala:72-101): batch sums added in float, divided by the row count."""
+    total = F32(0.0)
+    for s in range(0, X.shape[0], batch):
+        total = F32(total + error_sum(model, X[s:s + batch], Y[s:s + batch], params, absolute))
+    return float(total / F32(X.shape[0]))
+
+
+def r2_score(model, X, Y, params, batch=1000):
+    """`R2Score` (estimators/package.scala:103-138), with its total sum of squares around the mean prediction."""
+    pred = np.concatenate([model.forward(X[s:s + batch], params).reshape(-1) for s in range(0, X.shape[0], batch)]).astype(np.float64)
+    exp = Y.reshape(-1).astype(np.float64)
+    return float(F32(1.0 - ((pred - exp) ** 2).sum() / ((pred - pred.mean()) ** 2).sum()))
+
+
 def count_correct(model, x, y, params):
     """`estimators.accuracy`'s per-batch count (estimators/package.scala:28-32):
     rows whose every rounded output equals the label."""

@@ -20,6 +20,7 @@ SN_MAX_AVG_INPUTS = 32
 LAYER_DENSE, LAYER_BIAS, LAYER_ACTIVATE, LAYER_FLATTEN, LAYER_CONV2D, LAYER_POOL2D, LAYER_LSTM, LAYER_SIMPLE_RNN, LAYER_BATCHNORM = range(9)
 ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = range(5)
 RANDOM_UNIFORM, RANDOM_NORMAL, RANDOM_TRUNCATED_NORMAL = range(3)
+ERROR_SQUARED, ERROR_ABSOLUTE = range(2)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
 PAD_VALID, PAD_SAME = 0, 1
 REG_NONE, REG_L1, REG_L2 = 0, 1, 2
@@ -89,6 +90,7 @@ SIGNATURES = {
     "sn_grad": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_forward": (C.c_int, [_P, _P, C.c_int32, _P]),
     "sn_forward_training": (C.c_int, [_P, _P, C.c_int32, _P]),
+    "sn_error_sum": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, _F]),
     "sn_loss": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_count_correct": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64)]),
     "sn_train_epoch": (C.c_int, [_P, _P, _P, C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_int32), _F]),

@@ -286,6 +286,12 @@ class Replica:
         check(lib.sn_loss(self.handle, self._ptr(x), self._ptr(y), self.model.batch if rows is None else rows, C.byref(loss)))
         return loss.value
 
+    def error_sum(self, x, y, kind: int, rows: Optional[int] = None) -> float:
+        """Sum of squared (kind 0) or absolute (kind 1) errors of the frozen model over one batch."""
+        out = C.c_float()
+        check(lib.sn_error_sum(self.handle, self._ptr(x), self._ptr(y), self.model.batch if rows is None else rows, kind, C.byref(out)))
+        return out.value
+
     def count_correct(self, x, y, rows: Optional[int] = None) -> int:
         n = C.c_int64()
         check(lib.sn_count_correct(self.handle, self._ptr(x), self._ptr(y), self.model.batch if rows is None else rows,

@@ -121,6 +121,8 @@ int launch_act_bwd(sn_ctx* ctx, const float* y, const float* dy, float* dx, int6
 int launch_softmax_fwd(sn_ctx* ctx, const float* z, float* p, int rows, int cols, bool stable);
 int launch_softmax_bwd(sn_ctx* ctx, const float* p, const float* dp, float* dz, int rows, int cols);
 // loss value (sum of per-element terms / divisor) into *loss_dev and d loss / d p into dp (dp may be null)
+// loss kinds beyond the public SN_LOSS_*: plain sums of the error terms the regression estimators use
+constexpr int LOSS_SUM_SQUARED_ERROR = 100, LOSS_SUM_ABSOLUTE_ERROR = 101;
 int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp, float* loss_dev, float* partials,
                 int rows, int cols);
 // training step of a Softmax output under CategoricalCrossentropy: p, loss value and dz in one kernel per row

@@ -199,6 +199,11 @@ __global__ __launch_bounds__(256) void loss_stage1_kernel(int kind, const float*
     } else if (kind == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
       s += yi * logf(pi + eps);
       if (dp) dp[i] = (yi * neg_inv_rows) / (pi + eps);
+    } else if (kind == LOSS_SUM_SQUARED_ERROR) {  // estimators/package.scala:56-62
+      const float d = pi - yi;
+      s += d * d;
+    } else if (kind == LOSS_SUM_ABSOLUTE_ERROR) {  // estimators/package.scala:64-70
+      s += fabsf(pi - yi);
     } else {  // identity: the prediction is the loss (Loss.scala:10-14); callers guarantee n == 1
       s += pi;
       if (dp) dp[i] = 1.0f;
@@ -216,7 +221,7 @@ __global__ __launch_bounds__(256) void loss_stage2_kernel(int kind, const float*
   const float t = block_sum(s, smem);
   if (threadIdx.x == 0) {
     if (kind == SN_LOSS_CATEGORICAL_CROSSENTROPY) *loss = (-t) / rows;
-    else if (kind == SN_LOSS_IDENTITY) *loss = t;
+    else if (kind == SN_LOSS_IDENTITY || kind == LOSS_SUM_SQUARED_ERROR || kind == LOSS_SUM_ABSOLUTE_ERROR) *loss = t;
     else *loss = t * inv_size;
   }
 }

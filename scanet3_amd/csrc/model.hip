@@ -1067,6 +1067,18 @@ int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, in
   return SN_OK;
 }
 
+int sn_error_sum(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t kind, float* sum_host) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && y_dev && sum_host, "sn_error_sum: null pointer");
+  SN_REQUIRE(kind == SN_ERROR_SQUARED || kind == SN_ERROR_ABSOLUTE, "unknown error kind %d", kind);
+  SN_TRY(check_rows(rep, rows));
+  SN_TRY(forward(rep, x_dev, rows));
+  const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
+  SN_TRY(launch_loss(rep->ctx, kind == SN_ERROR_SQUARED ? LOSS_SUM_SQUARED_ERROR : LOSS_SUM_ABSOLUTE_ERROR, pred, y_dev, nullptr,
+                     rep->loss_dev, rep->loss_partials, rows, (int)rep->model->out_elems));
+  return read_loss(rep, sum_host);
+}
+
 int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int64_t total_rows, int32_t batch, int32_t global_iter,
                    int32_t* iterations_host, float* loss_host) {
   SN_TRY(check_replica(rep));

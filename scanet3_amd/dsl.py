@@ -520,6 +520,68 @@ def accuracy(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
     return trained._run(ds.x, batch, go)
 
 
+def _mean_error(trained: TrainedModel, ds: Dataset, batch: int, kind: int) -> float:
+    """estimators.meanError (estimators/package.scala:72-101): per-batch error sums (on the device), added in float
+    on the host, divided by the number of rows."""
+    n = len(ds)
+    batch = min(batch, n)
+
+    def go(ctx, cm, rep):
+        total = np.float32(0.0)
+        for s in range(0, n, batch):
+            xs, ys = ds.x[s:s + batch], ds.y[s:s + batch]
+            xb, yb = ctx.to_device(xs), ctx.to_device(ys)
+            try:
+                total = np.float32(total + np.float32(rep.error_sum(xb, yb, kind, xs.shape[0])))
+            finally:
+                xb.free()
+                yb.free()
+        return float(total / np.float32(n))
+    return trained._run(ds.x, batch, go)
+
+
+def MSE(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
+    """estimators.MSE (estimators/package.scala:56-62)."""
+    return _mean_error(trained, ds, batch, L.ERROR_SQUARED)
+
+
+def RMSE(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
+    """estimators.RMSE (estimators/package.scala:50-54)."""
+    return float(np.float32(math.sqrt(MSE(trained, ds, batch))))
+
+
+def MAE(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
+    """estimators.MAE (estimators/package.scala:64-70)."""
+    return _mean_error(trained, ds, batch, L.ERROR_ABSOLUTE)
+
+
+def R2Score(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
+    """estimators.R2Score (estimators/package.scala:103-138): predictions per batch from the device, the two sums in
+    double on the host.  As in the reference the total sum of squares is taken around the mean PREDICTION
+    (`mean = expectedVsPredicted.map(_._2)`, :126-131), not around the mean label."""
+    if tuple(ds.y.shape[1:]) != (1,):
+        raise ValueError("requirement failed: labels should have shape (1)")
+    n = len(ds)
+    batch = min(batch, n)
+
+    def go(ctx, cm, rep):
+        preds = []
+        for s in range(0, n, batch):
+            xs = ds.x[s:s + batch]
+            xb = ctx.to_device(xs)
+            try:
+                preds.append(rep.forward(xb, xs.shape[0]).reshape(-1))
+            finally:
+                xb.free()
+        predicted = np.concatenate(preds).astype(np.float64)
+        expected = ds.y.reshape(-1).astype(np.float64)
+        mean = predicted.mean()
+        ssr = float(((predicted - expected) ** 2).sum())
+        sst = float(((predicted - mean) ** 2).sum())
+        return float(np.float32(1.0 - ssr / sst))
+    return trained._run(ds.x, batch, go)
+
+
 @dataclass
 class Builder:
     """The type-state builder of the reference without the types (optimizers/Optimizer.scala:267-310)."""

@@ -38,3 +38,38 @@ def logistic_data():
     d = load_scv("logistic_regression_1.scv")
     # test/Datasets.scala:42-56 scales both features by 1/100
     return (d[:, :2] / np.float32(100)).astype(np.float32), d[:, 2:3].copy()
+
+
+def load_sunspots():
+    """`monthlySunspots(12)` of the reference's tests (test/Datasets.scala:72-97) from its own resource file: counts scaled
+    to [0, 1] by the series' minimum and maximum, grouped by floor((year*12 + month) / 12) (so a group runs from
+    December to November), a group of 12 is one sample and the first value of the next group its label.
+    Returns (X [n, 12, 1], Y [n, 1]) in time order."""
+    months, values = [], []
+    with open(os.path.join(GOLDEN_DIR, "monthly-sunspots.csv")) as f:
+        next(f)
+        for line in f:
+            line = line.strip()
+            if not line:
+                continue
+            date, v = line.split(",")
+            y, m = date.strip('"').split("-")
+            months.append(int(y) * 12 + int(m))
+            values.append(float(v))
+    v = np.asarray(values, np.float32)
+    lo, hi = v.min(), v.max()
+    scaled = ((v - lo) / (hi - lo)).astype(np.float32)
+    groups = {}
+    for mth, s in zip(months, scaled):
+        groups.setdefault(mth // 12, []).append(s)
+    xs, ys = [], []
+    for step in sorted(groups):
+        if len(groups[step]) == 12 and step + 1 in groups:
+            xs.append(groups[step])
+            ys.append([groups[step + 1][0]])
+    return np.asarray(xs, np.float32).reshape(-1, 12, 1), np.asarray(ys, np.float32)
+
+
+@pytest.fixture(scope="session")
+def sunspots():
+    return load_sunspots()

@@ -734,6 +734,34 @@ def test_dsl_batch_norm_training_over_two_partitions(S):
     assert rel_err(trained.result(X[:7]), om.forward(X[:7], oparams)) <= TOL_GEMM
 
 
+def test_rnn_forecast_and_regression_estimators(S, ctx, sunspots):
+    """RNNSpec.scala:22-47 through the DSL mirror: the same seeded start as the oracle, the reference's thresholds,
+    and MSE / RMSE / MAE / R2Score (estimators/package.scala:50-138) against the oracle's."""
+    from tests.test_oracle_golden import forecast_case
+    om, init, (xtr, ytr), (xte, yte) = forecast_case(sunspots)
+    model = S.SimpleRNN(3, kernelInitializer=S.GlorotUniform(seed=11), recurrentInitializer=S.Orthogonal(seed=12)) \
+        >> S.Dense(1, S.Tanh, kernelInitializer=S.GlorotUniform(seed=13))
+    trained = S.Dataset(xtr, ytr).train(model).loss(S.MeanSquaredError).using(S.Adam(0.01)).batch(10).epochs(100).run()
+    oparams, _, ohist = O.train(om, O.Adam(0.01), [(xtr, ytr)], 10, 100, init)
+    np.testing.assert_allclose(trained.history[:10], ohist[:10], rtol=TOL_TRAJECTORY)     # same start, same first epochs
+    test = S.Dataset(xte, yte)
+    rmse, r2 = S.RMSE(trained, test), S.R2Score(trained, test)
+    assert rmse < 0.2 and r2 > 0.78
+    assert abs(rmse - np.sqrt(O.mean_error(om, xte, yte, oparams))) < 5e-3
+    # the estimators themselves, on the oracle's parameters
+    fixed = S.TrainedModel(model, S.MeanSquaredError, oparams, {}, [], 0, (12, 1))
+    assert S.MSE(fixed, test, batch=20) == pytest.approx(O.mean_error(om, xte, yte, oparams, batch=20), rel=1e-5)
+    assert S.MAE(fixed, test, batch=20) == pytest.approx(O.mean_error(om, xte, yte, oparams, batch=20, absolute=True), rel=1e-5)
+    assert S.RMSE(fixed, test) == pytest.approx(float(np.sqrt(O.mean_error(om, xte, yte, oparams))), rel=1e-5)
+    assert S.R2Score(fixed, test, batch=20) == pytest.approx(O.r2_score(om, xte, yte, oparams, batch=20), rel=1e-4)
+    with pytest.raises(S.ScanetError, match="error kind"):
+        h = Harness(S, ctx, [("dense", 1, "identity")], "mse", (2,), 4)
+        try:
+            h.rep.error_sum(ctx.alloc(8), ctx.alloc(4), 5)
+        finally:
+            h.close()
+
+
 def test_error_paths(S, ctx):
     with pytest.raises(S.ScanetError):
         S.Context(99)

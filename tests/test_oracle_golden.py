@@ -315,6 +315,34 @@ def test_seeded_streams_structure():
     assert O.initializer_fans((3, 3, 2, 8)) == (16 * 3, 16 * 3)              # `out :: in :: receptive` (Initializer.scala:20-23)
 
 
+def forecast_case(sunspots):
+    """RNNSpec.scala:22-33: SimpleRNN(3) >> Dense(1, Tanh), Adam(0.01), batch 10, 100 epochs on the sunspot series.
+    The reference splits 80/20 at random through Spark; here every fifth sample is held out.  Initial weights come
+    from seeded initializers so that both sides of a parity test start from the same point."""
+    X, Y = sunspots
+    held = np.arange(X.shape[0]) % 5 == 4
+    m = O.Model([O.SimpleRNN(3), O.Dense(1, O.ACT_TANH)], O.LOSS_MSE)
+    init = {"0/0/kernel_weights": O.initialize("GlorotUniform", (1, 3), 11),
+            "0/0/recurrent_weights": O.initialize("Orthogonal", (3, 3), 12), "0/1/weights": np.zeros(3, f32),
+            "1/weights": O.initialize("GlorotUniform", (3, 1), 13), "2/weights": np.zeros(1, f32)}
+    return m, init, (X[~held], Y[~held]), (X[held], Y[held])
+
+
+def test_rnn_forecast_reaches_the_reference_thresholds(sunspots):
+    """RNNSpec.scala:46-47: RMSE < 0.2 and R2Score > 0.78 on the held-out part."""
+    assert sunspots[0].shape == (234, 12, 1)
+    m, init, (xtr, ytr), (xte, yte) = forecast_case(sunspots)
+    params, _, hist = O.train(m, O.Adam(0.01), [(xtr, ytr)], 10, 100, init)
+    assert hist[-1] < hist[0]
+    mse = O.mean_error(m, xte, yte, params)
+    assert np.sqrt(mse) < 0.2 and O.r2_score(m, xte, yte, params) > 0.78
+    # the estimators against their definitions on one batch
+    pred = m.forward(xte, params).astype(np.float64)
+    assert mse == pytest.approx(float(((pred - yte) ** 2).sum() / len(xte)), rel=1e-5)
+    assert O.mean_error(m, xte, yte, params, absolute=True) == pytest.approx(float(np.abs(pred - yte).sum() / len(xte)), rel=1e-5)
+    assert O.mean_error(m, xte, yte, params, batch=7) == pytest.approx(mse, rel=1e-5)          # batch sums add up
+
+
 def _lstm_params(g, pre=""):
     p = {}
     for gate in O.GATES:
