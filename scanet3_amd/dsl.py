@@ -21,6 +21,7 @@ import numpy as np
 
 from . import _lib as L
 from .core import CompiledModel, Context, DeviceBuffer, Replica, average_replicas
+from .formats import TensorBoard
 
 # --------------------------------------------------------------------------- activations / losses / misc
 
@@ -582,6 +583,36 @@ def R2Score(trained: TrainedModel, ds: Dataset, batch: int = 1000) -> float:
     return trained._run(ds.x, batch, go)
 
 
+class RecordLoss:
+    """Effect.RecordLoss (optimizers/Effect.scala:41-52): the epoch's loss to the console and, if asked, as the
+    scalar "loss" at the current iteration to the builder's TensorBoard directory."""
+    wants_context = True
+
+    def __init__(self, console: bool = True, tensorboard: bool = False):
+        self.console, self.tensorboard = console, tensorboard
+
+    def __call__(self, epoch, iterations, loss, board=None, trained=None, batch=None):
+        if self.tensorboard and board is not None:
+            board.add_scalar("loss", loss, iterations)
+        if self.console:
+            print(f"{epoch}/{iterations} loss: {loss}")
+
+
+class RecordAccuracy:
+    """Effect.RecordAccuracy (optimizers/Effect.scala:54-66): accuracy of the model as trained so far on `ds`."""
+    wants_context = True
+
+    def __init__(self, ds: "Dataset", console: bool = True, tensorboard: bool = False):
+        self.ds, self.console, self.tensorboard = ds, console, tensorboard
+
+    def __call__(self, epoch, iterations, loss, board=None, trained=None, batch=None):
+        a = accuracy(trained(), self.ds, batch or 1000)
+        if self.tensorboard and board is not None:
+            board.add_scalar("accuracy", a, iterations)
+        if self.console:
+            print(f"{epoch}/{iterations} accuracy: {a}")
+
+
 @dataclass
 class Builder:
     """The type-state builder of the reference without the types (optimizers/Optimizer.scala:267-310)."""
@@ -597,6 +628,11 @@ class Builder:
     flags: int = 0
     seed: int = 0
     device: int = 0
+    board_dir: str = "board"                     # Optimizer.scala:54
+
+    def board(self, directory: str):
+        """Directory of the TensorBoard event files effects write (Optimizer.scala:297-298)."""
+        return replace(self, board_dir=directory)
 
     def loss(self, loss: Loss):
         return replace(self, loss_fn=loss)
@@ -653,6 +689,7 @@ class Builder:
                 rep.set_params(params)
                 reps.append(rep)
             global_iter, epoch, history = 0, 0, []
+            board = None
             while True:
                 iters, losses = 0, []
                 for rep, (xb, yb, rows) in zip(reps, data):       # one partition after the other on the one GPU
@@ -665,7 +702,14 @@ class Builder:
                 epoch += 1
                 history.append(loss)
                 for e in self.effects:
-                    e(epoch, global_iter, loss)
+                    if getattr(e, "wants_context", False):
+                        if board is None and getattr(e, "tensorboard", False):
+                            board = TensorBoard(self.board_dir)
+                        e(epoch, global_iter, loss, board=board, batch=self.batch_size,
+                          trained=lambda: TrainedModel(self.model, self.loss_fn, reps[0].get_params(), {}, list(history), global_iter,
+                                                       tuple(in_shape), self.flags))
+                    else:
+                        e(epoch, global_iter, loss)
                 if (self.n_epochs is not None and epoch >= self.n_epochs) or \
                         (self.n_iterations is not None and global_iter >= self.n_iterations):
                     break

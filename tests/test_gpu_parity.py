@@ -912,3 +912,26 @@ def test_random_stream_full_size(S, ctx):
     assert float(np.abs(t).max()) < 2.0 and abs(float(t.std(dtype=np.float64)) - 0.87962566) < 2e-4
     np.testing.assert_allclose(t[:64], O.tf_truncated_normal(64, seed), rtol=0, atol=4e-6)
     buf.free()
+
+
+def test_dsl_effects_write_tensorboard_scalars(S, logistic_data, tmp_path, capsys):
+    """`.each(RecordLoss(tensorboard = true))` and RecordAccuracy (optimizers/Effect.scala:41-66): one events file per
+    call under the builder's board directory, holding the epoch's loss / accuracy at the iteration count."""
+    from scanet3_amd import formats as F
+    X, Y = logistic_data
+    ds = S.Dataset(X, Y)
+    trained = ds.train(S.LogisticRegression()).loss(S.BinaryCrossentropy).using(S.Adam(0.1)).batch(50).epochs(3) \
+        .board(str(tmp_path / "board")).each(S.RecordLoss(console=True, tensorboard=True)) \
+        .each(S.RecordAccuracy(ds, console=False, tensorboard=True)).run()
+    files = sorted((tmp_path / "board").iterdir(), key=lambda p: int(p.name.rsplit(".", 1)[-1]))
+    assert len(files) == 6
+    seen = []
+    for f in files:
+        records = F.read_tf_records(f.read_bytes())
+        assert records[0] == F.event_file_version() and len(records) == 2
+        seen.append(records[1])
+    per_epoch = X.shape[0] // 50
+    for i, loss in enumerate(trained.history):
+        assert F.event_scalar("loss", loss, (i + 1) * per_epoch, 0.0)[-10:] == seen[2 * i][-10:]      # tag + value bytes
+        assert b"accuracy" in seen[2 * i + 1]
+    assert "loss:" in capsys.readouterr().out
