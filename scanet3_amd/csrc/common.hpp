@@ -199,13 +199,20 @@ struct Epilogue {
   const float* bias = nullptr;  // per output column, may be null
   int act = SN_ACT_IDENTITY;    // identity / sigmoid / tanh / relu (softmax is a row kernel)
   float act_param = 0.f;
+  // one row of the product goes elsewhere, untouched by bias and activation (the bias gradient that rides along
+  // in a weight-gradient GEMM as an all-ones row of A)
+  int row_index = -1;
+  float* row_out = nullptr;
 };
 // C[M,N] = A[M,K] * B[K,N] with arbitrary element strides (covers NN, NT, TN).
 struct GemmDesc {
   const float* a; int64_t a_sm, a_sk;   // A(m,k) = a[m*a_sm + k*a_sk]
   const float* b; int64_t b_sk, b_sn;   // B(k,n) = b[k*b_sk + n*b_sn]
   int m, n, k;
+  bool a_ones_row = false;              // A's last row (index m-1) is all ones and is not read from `a`
 };
+// true when launch_gemm would take its 16-byte loaders for this problem (they have no all-ones row)
+bool gemm_takes_fast_loaders(const sn_ctx* ctx, const GemmDesc& g, const float* workspace, int64_t workspace_elems);
 int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* workspace, int64_t workspace_elems, bool bf16);
 
 // bf16 fast path (gemm_bf16.hip): C[M,N] = A[M,K] * Bt[N,K]^T, operands bf16 with k contiguous.

@@ -67,15 +67,19 @@ struct StridedLoader {
   const float* p;
   int64_t s_outer, s_k;
   int outer_n;
+  int ones_outer = -1;  // this outer index (just past the matrix) reads as all ones; -1: none
   struct Cursor {
     const float* ptr;
     int k;
+    bool ones;
   };
   __device__ __forceinline__ void init(Cursor& c, int outer, int k) const {
     c.ptr = outer < outer_n ? p + (int64_t)outer * s_outer : nullptr;
     c.k = k;
+    c.ones = outer == ones_outer;
   }
   __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
+    if (c.ones) return c.k < k_end ? 1.0f : 0.f;
     return (c.ptr && c.k < k_end) ? c.ptr[(int64_t)c.k * s_k] : 0.f;
   }
   // 4 values along the contiguous index (k when KC, the outer index otherwise); vec4_ok() guarantees that the
@@ -83,6 +87,9 @@ struct StridedLoader {
   __device__ __forceinline__ void load4(const Cursor& c, int k_end, float (&v)[4]) const {
     f4v r = {0.f, 0.f, 0.f, 0.f};
     if (c.ptr && c.k < k_end) r = *(const f4v*)(c.ptr + (int64_t)c.k * s_k);
+    // the ones row starts a group of 4 outer indices (outer_n % 4 == 0) whose other three lie outside the matrix;
+    // along k (KC) it is four ones
+    if (c.ones && c.k < k_end) r = KC ? f4v{1.f, 1.f, 1.f, 1.f} : f4v{1.f, 0.f, 0.f, 0.f};
     v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
   }
   bool vec4_ok(int K) const {
@@ -625,6 +632,10 @@ __device__ __forceinline__ float ep_act(int act, float v, float param) {
 struct StdEpilogue {
   Epilogue e;
   __device__ __forceinline__ void store(int m, int n, float acc) const {
+    if (m == e.row_index) {
+      e.row_out[n] = acc;
+      return;
+    }
     float v = acc;
     if (e.bias) v = v + e.bias[n];
     e.out[(int64_t)m * e.ldo + n] = ep_act(e.act, v, e.act_param);
@@ -1041,13 +1052,25 @@ static int launch_any(sn_ctx* ctx, const char* name, int M, int N, int K, const 
   return launch_tiles<64, 64, BF16>(ctx, name, M, N, K, al, bl, ep, ws, ws_elems);
 }
 
+static bool fast_pair_ok(const sn_ctx* ctx, const GemmDesc& g, const float* ws, int64_t ws_elems) {
+  if (g.a_ones_row || (ws && small_parts(g.m, g.n, g.k, ctx->compute_units, ws_elems))) return false;
+  const bool akc = g.a_sk == 1, bkc = g.b_sk == 1 && g.b_sn != 1;
+  const bool a_ok = akc ? FlatLoader<true>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) : FlatLoader<false>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k);
+  const bool b_ok = bkc ? FlatLoader<true>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k) : FlatLoader<false>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k);
+  return a_ok && b_ok;
+}
+
+bool gemm_takes_fast_loaders(const sn_ctx* ctx, const GemmDesc& g, const float* workspace, int64_t workspace_elems) {
+  return fast_pair_ok(ctx, g, workspace, workspace_elems);
+}
+
 template <bool BF16>
 static int launch_gemm_t(sn_ctx* ctx, const GemmDesc& g, const Epilogue& e, float* ws, int64_t ws_elems) {
   StdEpilogue ep{e};
   const char* name = BF16 ? "gemm_bf16" : "gemm_f32";
   const bool akc = g.a_sk == 1, bkc = g.b_sk == 1 && g.b_sn != 1;
   // FAST loaders whenever both operands allow 16-byte loads, unless the small-output kernel (cursor loaders) takes the problem
-  if (!(ws && small_parts(g.m, g.n, g.k, ctx->compute_units, ws_elems))) {
+  if (fast_pair_ok(ctx, g, ws, ws_elems)) {
     if (akc && bkc && FlatLoader<true>::ok(g.a, g.a_sm, g.a_sk, g.m, g.k) && FlatLoader<true>::ok(g.b, g.b_sn, g.b_sk, g.n, g.k)) {
       FlatLoader<true> al{g.a, (int)g.a_sm, (int)g.a_sk, g.m}, bl{g.b, (int)g.b_sn, (int)g.b_sk, g.n};
       return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
@@ -1067,19 +1090,20 @@ static int launch_gemm_t(sn_ctx* ctx, const GemmDesc& g, const Epilogue& e, floa
       return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
     }
   }
+  const int a_rows = g.a_ones_row ? g.m - 1 : g.m, a_ones = g.a_ones_row ? g.m - 1 : -1;
   if (akc && bkc) {
-    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones}, bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   } else if (akc) {
-    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m};
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones};
     StridedLoader<false> bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   } else if (bkc) {
-    StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m};
+    StridedLoader<false> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones};
     StridedLoader<true> bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   }
-  StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
+  StridedLoader<false> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones}, bl{g.b, g.b_sn, g.b_sk, g.n};
   return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
 }
 

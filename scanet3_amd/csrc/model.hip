@@ -181,7 +181,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         }
         const int in_f = (int)cur[0], out_f = L.units;
         ws = std::max(ws, gemm_workspace_elems(B, out_f, in_f, cu));
-        ws = std::max(ws, gemm_workspace_elems(in_f, out_f, B, cu));
+        ws = std::max(ws, gemm_workspace_elems(in_f + 1, out_f, B, cu));  // + the bias-gradient row
         ws = std::max(ws, gemm_workspace_elems(B, in_f, out_f, cu));
         break;
       }
@@ -650,11 +650,21 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           break;
         }
         if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
-        if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
         {  // dW = X^T . dY (math/alg/AllKernels.scala:382-388)
           GemmDesc g{in, 1, in_f, dy, out_f, 1, in_f, out_f, rows};
           Epilogue ep;
           ep.out = param_ptr(r, r->g, op.w); ep.ldo = out_f;
+          // the bias gradient (column sums of dY) is the product's row for an all-ones row of X^T: it rides along
+          // unless the GEMM takes its 16-byte loaders, which have no such row
+          const bool ride = op.b >= 0 && !gemm_takes_fast_loaders(ctx, g, r->ws, m->workspace_elems);
+          if (ride) {
+            g.m = in_f + 1;
+            g.a_ones_row = true;
+            ep.row_index = in_f;
+            ep.row_out = param_ptr(r, r->g, op.b);
+          } else if (op.b >= 0) {
+            SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
+          }
           SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
         }
         if (need_dx) {  // dX = dY . W^T
