@@ -61,7 +61,9 @@ __device__ __forceinline__ void sel_load4(const float* base, uint32_t byte_off, 
 }
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <bool KC>
+// ONES: the loader knows one extra outer index that reads as all ones (a separate type, so the plain loader's
+// cursor and loads stay as lean as they were)
+template <bool KC, bool ONES = false>
 struct StridedLoader {
   static constexpr bool K_CONTIG = KC;
   const float* p;
@@ -76,10 +78,10 @@ struct StridedLoader {
   __device__ __forceinline__ void init(Cursor& c, int outer, int k) const {
     c.ptr = outer < outer_n ? p + (int64_t)outer * s_outer : nullptr;
     c.k = k;
-    c.ones = outer == ones_outer;
+    c.ones = ONES && outer == ones_outer;
   }
   __device__ __forceinline__ float load(const Cursor& c, int k_end) const {
-    if (c.ones) return c.k < k_end ? 1.0f : 0.f;
+    if (ONES && c.ones) return c.k < k_end ? 1.0f : 0.f;
     return (c.ptr && c.k < k_end) ? c.ptr[(int64_t)c.k * s_k] : 0.f;
   }
   // 4 values along the contiguous index (k when KC, the outer index otherwise); vec4_ok() guarantees that the
@@ -89,7 +91,7 @@ struct StridedLoader {
     if (c.ptr && c.k < k_end) r = *(const f4v*)(c.ptr + (int64_t)c.k * s_k);
     // the ones row starts a group of 4 outer indices (outer_n % 4 == 0) whose other three lie outside the matrix;
     // along k (KC) it is four ones
-    if (c.ones && c.k < k_end) r = KC ? f4v{1.f, 1.f, 1.f, 1.f} : f4v{1.f, 0.f, 0.f, 0.f};
+    if (ONES && c.ones && c.k < k_end) r = KC ? f4v{1.f, 1.f, 1.f, 1.f} : f4v{1.f, 0.f, 0.f, 0.f};
     v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
   }
   bool vec4_ok(int K) const {
@@ -1090,20 +1092,25 @@ static int launch_gemm_t(sn_ctx* ctx, const GemmDesc& g, const Epilogue& e, floa
       return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
     }
   }
-  const int a_rows = g.a_ones_row ? g.m - 1 : g.m, a_ones = g.a_ones_row ? g.m - 1 : -1;
+  if (g.a_ones_row) {  // the weight-gradient form: A = X^T (outer index contiguous) plus the ones row, B = dY (row major)
+    SN_REQUIRE(!akc && !bkc, "gemm: the all-ones row is built for A^T-major A and row-major B only");
+    StridedLoader<false, true> al{g.a, g.a_sm, g.a_sk, g.m - 1, g.m - 1};
+    StridedLoader<false> bl{g.b, g.b_sn, g.b_sk, g.n};
+    return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
+  }
   if (akc && bkc) {
-    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones}, bl{g.b, g.b_sn, g.b_sk, g.n};
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   } else if (akc) {
-    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones};
+    StridedLoader<true> al{g.a, g.a_sm, g.a_sk, g.m};
     StridedLoader<false> bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   } else if (bkc) {
-    StridedLoader<false> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones};
+    StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m};
     StridedLoader<true> bl{g.b, g.b_sn, g.b_sk, g.n};
     return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
   }
-  StridedLoader<false> al{g.a, g.a_sm, g.a_sk, a_rows, a_ones}, bl{g.b, g.b_sn, g.b_sk, g.n};
+  StridedLoader<false> al{g.a, g.a_sm, g.a_sk, g.m}, bl{g.b, g.b_sn, g.b_sk, g.n};
   return launch_any<BF16>(ctx, name, g.m, g.n, g.k, al, bl, ep, ws, ws_elems);
 }
 

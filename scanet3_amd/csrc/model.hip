@@ -656,7 +656,8 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           ep.out = param_ptr(r, r->g, op.w); ep.ldo = out_f;
           // the bias gradient (column sums of dY) is the product's row for an all-ones row of X^T: it rides along
           // unless the GEMM takes its 16-byte loaders, which have no such row
-          const bool ride = op.b >= 0 && !gemm_takes_fast_loaders(ctx, g, r->ws, m->workspace_elems);
+          // (with a single input feature X^T is also K-contiguous and takes another loader: plain column sums then)
+          const bool ride = op.b >= 0 && in_f > 1 && !gemm_takes_fast_loaders(ctx, g, r->ws, m->workspace_elems);
           if (ride) {
             g.m = in_f + 1;
             g.a_ones_row = true;
