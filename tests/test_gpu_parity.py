@@ -936,3 +936,57 @@ def test_dsl_effects_write_tensorboard_scalars(S, logistic_data, tmp_path, capsy
         assert F.event_scalar("loss", loss, (i + 1) * per_epoch, 0.0)[-10:] == seen[2 * i][-10:]      # tag + value bytes
         assert b"accuracy" in seen[2 * i + 1]
     assert "loss:" in capsys.readouterr().out
+
+
+# ----------------------------------------------------------------------------- small and degenerate shapes
+@pytest.mark.parametrize("spec,in_shape,batch", [
+    ([("lstm", 16), ("dense", 1, "identity")], (1, 4), 5),                      # a single time step, fused-kernel shape
+    ([("simple_rnn", 16, "tanh"), ("dense", 1, "identity")], (1, 4), 5),
+    ([("simple_rnn", 3, "relu")], (4, 2), 1),                                   # batch of one, the layer alone
+    ([("dense", 4, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 2, "identity")], (3,), 1),   # variance of one row is zero
+    ([("conv", 4, (1, 1), (1, 1), "valid", "identity", False), ("batchnorm", 0.5, 1e-3), ("flatten",), ("dense", 1, "identity")],
+     (1, 1, 4), 3),                     # 1x1 image, 1x1 kernel (no conv bias: in front of a BatchNorm its gradient is pure rounding noise)
+])
+def test_degenerate_shapes_match_oracle(S, ctx, spec, in_shape, batch):
+    rng = np.random.default_rng(20251125 + 17)
+    h = Harness(S, ctx, spec, "mse", in_shape, batch, S.Adam(0.01))
+    om = h.omodel
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    out_dim = int(np.prod(om.out_shape((batch,) + in_shape)[1:]))
+    x = rng.standard_normal((batch,) + in_shape).astype(f32)
+    y = rng.uniform(-1, 1, (batch, out_dim)).astype(f32)
+    h.rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    assert rel_err(h.rep.forward(xb), om.forward(x, params)) <= TOL_GEMM
+    oloss, ograds = om.grad(x, y.reshape(om.out_shape((batch,) + in_shape)), params)
+    gloss = h.rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ggrads = h.rep.get_grads()
+    # a gradient that is zero in exact arithmetic (a bias in front of a BatchNorm) is rounding noise on both sides:
+    # the yardstick is the tensor's own maximum or, if larger, a hundredth of the model's largest gradient
+    overall = max(float(np.abs(g).max()) for g in ograds.values())
+    for p in ograds:
+        scale = max(float(np.abs(ograds[p]).max()), 1e-2 * overall)
+        assert float(np.abs(ggrads[p] - ograds[p]).max()) <= TOL_GEMM * scale, p
+    ostate = O.init_opt_state(O.Adam(0.01), params)
+    new_params, _, _, _ = O.train_step(om, O.Adam(0.01), x, y.reshape(om.out_shape((batch,) + in_shape)), params, ostate, 1)
+    h.rep.step(xb, yb, 1)
+    got = h.rep.get_params()
+    for p in new_params:
+        assert rel_err(got[p], new_params[p]) <= 1e-4, p
+    h.close()
+
+
+def test_zero_length_calls_are_no_ops(S, ctx):
+    from scanet3_amd import _lib as L
+    from scanet3_amd._lib import check, lib
+    import ctypes as C
+    buf = ctx.alloc(4)
+    buf.fill(7.0)
+    check(lib.sn_random_fill(ctx.handle, buf.ptr, 0, L.RANDOM_NORMAL, C.c_uint64(3), None, None))
+    check(lib.sn_fill(ctx.handle, buf.ptr, C.c_float(1.0), 0))
+    desc = S.Adam()
+    check(lib.sn_optimizer_update(ctx.handle, C.byref(desc), buf.ptr, buf.ptr, buf.ptr, buf.ptr, None, 0, 1))
+    ctx.sync()
+    np.testing.assert_array_equal(buf.numpy(), np.full(4, 7.0, f32))
+    buf.free()
