@@ -342,6 +342,12 @@ MODELS = {
     "cnn_batchnorm_32_channels": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3),
                                    ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 10, "softmax")],
                                   "cce", (14, 14, 1), 50, "uniform_onehot"),
+    # tens of thousands of output positions over 4 input channels: padding, bias, strides, channel counts that are
+    # multiples of 4 but not of 16
+    "conv_many_positions_same_bias": ([("conv", 8, (3, 3), (1, 1), "same", "tanh", True), ("flatten",), ("dense", 3, "softmax")],
+                                  "cce", (20, 20, 4), 104, "uniform_onehot"),
+    "conv_many_positions_stride2": ([("conv", 12, (3, 3), (2, 2), "valid", "relu", False), ("flatten",), ("dense", 3, "softmax")],
+                                "cce", (40, 40, 4), 100, "uniform_onehot"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
 }
 
