@@ -348,6 +348,9 @@ MODELS = {
                                   "cce", (20, 20, 4), 104, "uniform_onehot"),
     "conv_many_positions_stride2": ([("conv", 12, (3, 3), (2, 2), "valid", "relu", False), ("flatten",), ("dense", 3, "softmax")],
                                 "cce", (40, 40, 4), 100, "uniform_onehot"),
+    # BatchNorm reductions: 200 channels take the row-walking form with four column blocks, 256 the float4 stream form
+    "batchnorm_200_channels": ([("dense", 200, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
+    "batchnorm_256_channels": ([("dense", 256, "relu"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
 }
 
@@ -436,8 +439,12 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
           ("flatten",), ("dense", 10, "softmax")], "cce", (28, 28, 1), 100, "uniform_onehot"),
         ([("lstm", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),
         ([("simple_rnn", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),   # the same shape, simple cell
+        # the CNN of the reference's MNIST test (CNNSpec.scala:22-35) with BatchNorm in its generic form, batch 1000
+        ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3), ("pool", (2, 2), (2, 2), "valid"),
+          ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "valid"), ("activate", "relu"), ("flatten",),
+          ("dense", 64, "relu"), ("dense", 10, "softmax")], "cce", (28, 28, 1), 1000, "uniform_onehot"),
     ]
-    for spec, loss, in_shape, batch, kind in cases:
+    for case_no, (spec, loss, in_shape, batch, kind) in enumerate(cases):
         rng = np.random.default_rng(20251125 + 2)
         h = Harness(S, ctx, spec, loss, in_shape, batch)
         om = h.omodel
@@ -448,10 +455,21 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
         xb, yb = ctx.to_device(x), ctx.to_device(y)
         oloss, ograds = om.grad(x, y, params)
         gloss = h.rep.grad(xb, yb)
-        assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
         ggrads = h.rep.get_grads()
-        for p in ograds:
-            assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        if case_no < 3:
+            assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+            for p in ograds:
+                assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        else:
+            # Nine layers at batch 1000 with a saturated softmax: float32 itself is the yardstick.  The oracle is run
+            # again in float64; the library may be as far from that as three times what the float32 oracle is
+            # (pooling ties and ReLU zeros fall differently under any other summation order), never less than 1e-4.
+            loss64, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
+            own = abs(float(oloss) - float(loss64)) / max(1.0, abs(float(loss64)))
+            assert abs(gloss - float(loss64)) / max(1.0, abs(float(loss64))) <= max(TOL_GEMM, 3.0 * own), (gloss, float(loss64), own)
+            for p in grads64:
+                own = rel_err(ograds[p], grads64[p])
+                assert rel_err(ggrads[p], grads64[p]) <= max(TOL_GEMM, 3.0 * own), (p, own)
         h.close()
         xb.free()
         yb.free()
