@@ -94,6 +94,8 @@ typedef struct sn_layer_desc {
   int32_t reg_kind;      /* Dense/Bias: SN_REG_* */
   float reg_lambda;
   int32_t use_bias;      /* LSTM: per-gate bias vectors (layer/RNN.scala:215); SIMPLE_RNN: the cell's Bias (RNN.scala:116) */
+  int32_t return_sequence; /* LSTM / SIMPLE_RNN: `returnSequence` (layer/RNN.scala:27,74-77): the output is every step's
+                              output, (batch, time, units), instead of the last one */
   float bn_momentum;     /* BATCHNORM (layer/BatchNorm.scala:64-76, axes = Seq(-1)): decay of the moving statistics */
   float bn_epsilon;      /* BATCHNORM: added to the variance */
   int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  Only the generic

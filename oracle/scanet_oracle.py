@@ -365,6 +365,7 @@ class Layer:
     reg_lambda: float = 0.0
     bias: bool = True               # lstm / simple_rnn only
     rnn_activation: int = ACT_TANH  # simple_rnn cell activation / lstm `activation`
+    return_sequence: bool = False   # lstm / simple_rnn: every step's output, (batch, time, units) (RNN.scala:27,75-77)
     momentum: float = 0.99          # batchnorm (BatchNorm.scala:66-67)
     epsilon: float = 1e-3
 
@@ -409,8 +410,8 @@ class Layer:
         if self.kind == "pool2d":
             return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0]),
                     out_size(self.padding, s[2], self.kernel[1], self.strides[1]), s[3])
-        if self.kind in ("lstm", "simple_rnn"):
-            return (s[0], self.units)
+        if self.kind in ("lstm", "simple_rnn"):    # RNN.scala:84-90
+            return (s[0], s[1], self.units) if self.return_sequence else (s[0], self.units)
         raise ValueError(self.kind)
 
 
@@ -444,12 +445,12 @@ def Flatten():
     return [Layer("flatten")]
 
 
-def LSTM(units, bias=True):
-    return [Layer("lstm", units=units, bias=bias)]
+def LSTM(units, bias=True, return_sequence=False):
+    return [Layer("lstm", units=units, bias=bias, return_sequence=return_sequence)]
 
 
-def SimpleRNN(units, activation=ACT_TANH, bias=True):
-    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation)]
+def SimpleRNN(units, activation=ACT_TANH, bias=True, return_sequence=False):
+    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation, return_sequence=return_sequence)]
 
 
 BN_PARAMS = ("beta", "gamma", "moving_mean", "moving_variance")   # BatchNorm.scala:92-97,170-173
@@ -670,6 +671,7 @@ def lstm_forward(x, params, pre, l: Layer):
     c = np.zeros((b, h_units), dt)
     h = np.zeros((b, h_units), dt)
     steps = []
+    outs = []
     for t in range(t_steps):
         xt = x[:, t, :]
         z = {}
@@ -686,19 +688,26 @@ def lstm_forward(x, params, pre, l: Layer):
         h_new = o * activate(l.rnn_activation, c_new)   # RNN.scala:337
         steps.append((xt, h, c, z, f, i, g, o, c_new))
         c, h = c_new, h_new
-    return h, (x.shape, steps)
+        outs.append(h_new)
+    out = np.stack(outs, axis=1) if l.return_sequence else h     # `joinAlong(outputs, 1)` or `outputs.last` (RNN.scala:74-77)
+    return out, (x.shape, steps)
 
 
-def lstm_backward(dh_last, cache, params, pre, l: Layer, grads, need_dx=False):
+def lstm_backward(dout, cache, params, pre, l: Layer, grads, need_dx=False):
+    """dout: gradient of the layer's output, (batch, units) or with `return_sequence` (batch, time, units): every
+    step's output then adds its own gradient to the one carried back from the step after it."""
     xshape, steps = cache
-    dt = dh_last.dtype
+    dt = dout.dtype
     b = xshape[0]
-    dh = dh_last
-    dc = np.zeros_like(dh_last)
+    seq = l.return_sequence
+    dh = np.zeros((b, l.units), dt) if seq else dout
+    dc = np.zeros((b, l.units), dt)
     acc = {}
     dx = np.zeros(xshape, dt) if need_dx else None
     for t in range(len(steps) - 1, -1, -1):
         xt, h_prev, c_prev, z, f, i, g, o, c_new = steps[t]
+        if seq:
+            dh = dh + dout[:, t, :]
         a = activate(l.rnn_activation, c_new)
         do = dh * a
         dc = dc + activate_grad(l.rnn_activation, c_new, dh * o)
@@ -738,13 +747,17 @@ def simple_rnn_forward(x, params, pre, l: Layer):
     s = np.zeros((b, l.units), dt)
     steps = []
     out = None
+    outs = []
     for t in range(t_steps):
         xt = x[:, t, :]
         r = (xt @ wk) + (s @ wr)
         zz = r + params[pre + "1/weights"] if l.bias else r
         out = activate(l.rnn_activation, zz)
+        outs.append(out)
         steps.append((xt, s, zz))
         s = r
+    if l.return_sequence:
+        out = np.stack(outs, axis=1)
     return out, (x.shape, steps)
 
 
@@ -756,14 +769,16 @@ def simple_rnn_backward(dout, cache, params, pre, l: Layer, grads, need_dx=False
     gk = np.zeros_like(wk)
     gr = np.zeros_like(wr)
     gb = np.zeros((l.units,), dt)
-    # only the last step's output feeds the loss; earlier steps act through the state
+    # without `return_sequence` only the last step's output feeds the loss; earlier steps act through the state
     t_last = len(steps) - 1
-    xt, s_prev, zz = steps[t_last]
-    dz = activate_grad(l.rnn_activation, zz, dout)
-    gb += dz.sum(axis=0, dtype=dt)
-    dr = dz
+    seq = l.return_sequence
+    dr = np.zeros((xshape[0], l.units), dt)
     for t in range(t_last, -1, -1):
-        xt, s_prev, _ = steps[t]
+        xt, s_prev, zz = steps[t]
+        if seq or t == t_last:
+            dz = activate_grad(l.rnn_activation, zz, dout[:, t, :] if seq else dout)
+            gb += dz.sum(axis=0, dtype=dt)
+            dr = dr + dz
         gk += xt.T @ dr
         gr += s_prev.T @ dr
         if need_dx:

@@ -42,7 +42,7 @@ class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("units", C.c_int32), ("activation", C.c_int32), ("act_param", C.c_float),
                 ("kernel_h", C.c_int32), ("kernel_w", C.c_int32), ("stride_h", C.c_int32), ("stride_w", C.c_int32),
                 ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32),
-                ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float), ("bn_fused", C.c_int32)]
+                ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float), ("bn_fused", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):

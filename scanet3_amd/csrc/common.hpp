@@ -157,9 +157,16 @@ struct LstmGateBwdArgs {
   float* dc;            // [rows,H] in: dc_t carried from t+1 (or zeros), out: dc_{t-1}
   float* dz;            // [rows,4H]
   int dc_is_zero;       // first backward step: treat dc as zeros on input
-  int dh_parts = 1;     // dh is the sum of this many arrays, dh_part_stride elements apart (added in order)
+  int dh_parts = 1;     // dh is the sum of this many arrays, dh_part_stride elements apart (added in order); 0: none
   int64_t dh_part_stride = 0;
+  const float* dy_seq = nullptr;  // this step's slice of the gradient of a returned sequence: row r at dy_seq + r * dy_seq_ld
+  int64_t dy_seq_ld = 0;
 };
+// out[r, t, :] = slices[(first + t) * slice_stride + r * H ...]: time-major step outputs as the (batch, time, units)
+// tensor `returnSequence` hands to the next layer (layer/RNN.scala:74-77)
+int launch_sequence_gather(sn_ctx* ctx, const float* slices, int64_t slice_stride, int first, float* out, int rows, int T, int H);
+// dst[r, :] (= or +=) src[r * src_ld ...] for rows x H values: one time step cut out of a (batch, time, units) gradient
+int launch_step_slice_add(sn_ctx* ctx, float* dst, const float* src, int64_t src_ld, int rows, int H, bool accumulate);
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
 
 // ---- seeded random tensors (random_kernels.hip): scale / shift may be null

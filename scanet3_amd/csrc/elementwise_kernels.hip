@@ -676,8 +676,9 @@ __global__ __launch_bounds__(256) void lstm_gates_bwd_kernel(LstmGateBwdArgs a, 
     const int64_t zb = r * 4 * hidden + u;
     const float f = a.gates[zb], in = a.gates[zb + hidden], g = a.gates[zb + 2 * hidden], o = a.gates[zb + 3 * hidden];
     const float tc = tanhf(a.c[i]);
-    float dh = a.dh[i];
+    float dh = a.dh_parts > 0 ? a.dh[i] : 0.f;
     for (int p = 1; p < a.dh_parts; ++p) dh += a.dh[i + p * a.dh_part_stride];
+    if (a.dy_seq) dh = dh + a.dy_seq[r * a.dy_seq_ld + u];
     const float d_o = dh * tc;
     float dc = a.dc_is_zero ? 0.f : a.dc[i];
     dc = dc + (1.0f - tc * tc) * (dh * o);
@@ -689,6 +690,51 @@ __global__ __launch_bounds__(256) void lstm_gates_bwd_kernel(LstmGateBwdArgs a, 
     a.dz[zb + 2 * hidden] = (1.0f - g * g) * dg;
     a.dz[zb + 3 * hidden] = (o * (1.0f - o)) * d_o;
   }
+}
+
+__global__ __launch_bounds__(256) void sequence_gather_kernel(const float* __restrict__ slices, int64_t slice_stride, int first,
+                                                               float* __restrict__ out, int rows, int T, int H) {
+  const int64_t total = (int64_t)rows * T * H;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int u = (int)(i % H);
+    const int64_t rt = i / H;
+    const int t = (int)(rt % T);
+    const int64_t r = rt / T;
+    out[i] = slices[(int64_t)(first + t) * slice_stride + r * H + u];
+  }
+}
+
+int launch_sequence_gather(sn_ctx* ctx, const float* slices, int64_t slice_stride, int first, float* out, int rows, int T, int H) {
+  const int64_t total = (int64_t)rows * T * H;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "sequence_gather");
+  hipLaunchKernelGGL(sequence_gather_kernel, dim3(grid_for(ctx, total, 1024)), dim3(256), 0, ctx->stream, slices, slice_stride, first, out, rows,
+                     T, H);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+__global__ __launch_bounds__(256) void step_slice_add_kernel(float* __restrict__ dst, const float* __restrict__ src, int64_t src_ld,
+                                                              int rows, int H, int accumulate) {
+  const int64_t total = (int64_t)rows * H;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / H;
+    const int u = (int)(i % H);
+    const float v = src[r * src_ld + u];
+    dst[i] = accumulate ? dst[i] + v : v;
+  }
+}
+
+int launch_step_slice_add(sn_ctx* ctx, float* dst, const float* src, int64_t src_ld, int rows, int H, bool accumulate) {
+  const int64_t total = (int64_t)rows * H;
+  if (total <= 0) return SN_OK;
+  LaunchScope scope(ctx, "sequence_step_gradient");
+  hipLaunchKernelGGL(step_slice_add_kernel, dim3(grid_for(ctx, total, 1024)), dim3(256), 0, ctx->stream, dst, src, src_ld, rows, H,
+                     accumulate ? 1 : 0);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
 }
 
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden) {

@@ -33,6 +33,7 @@ struct Op {
   int kh = 0, kw = 0, sh = 1, sw = 1, pt = 0, pl = 0;
   // lstm
   int T = 0, F = 0, H = 0;
+  bool ret_seq = false;  // the layer's output is every step's output, [T, H] per sample (layer/RNN.scala:74-77)
   int lstm_p[4][3] = {{-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}};  // gate x {kernel, recurrent, bias}
   // batch norm: beta, gamma, moving mean, moving variance
   int bn_p[4] = {-1, -1, -1, -1};
@@ -278,7 +279,8 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
           op.lstm_p[gi][1] = add_param(m, gp + "/0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
           if (L.use_bias) op.lstm_p[gi][2] = add_param(m, gp + "/1/weights", {op.H}, SN_REG_NONE, 0.f);
         }
-        op.out_dims = {L.units};
+        op.ret_seq = L.return_sequence != 0;
+        op.out_dims = op.ret_seq ? std::vector<int64_t>{op.T, L.units} : std::vector<int64_t>{L.units};  // RNN.scala:84-90
         ws = std::max(ws, gemm_workspace_elems(B, 4 * op.H, op.F + op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.H, 4 * op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.F, 4 * op.H, cu));
@@ -318,7 +320,8 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         op.lstm_p[0][0] = add_param(m, prefix(i) + "0/kernel_weights", {op.F, op.H}, SN_REG_NONE, 0.f);  // RNN.scala:165-166,198-203
         op.lstm_p[0][1] = add_param(m, prefix(i) + "0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
         if (L.use_bias) op.b = add_param(m, prefix(i) + "1/weights", {op.H}, SN_REG_NONE, 0.f);
-        op.out_dims = {L.units};
+        op.ret_seq = L.return_sequence != 0;
+        op.out_dims = op.ret_seq ? std::vector<int64_t>{op.T, L.units} : std::vector<int64_t>{L.units};
         ws = std::max(ws, gemm_workspace_elems(B, op.H, op.F + op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.H, op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.F, op.H, cu));
@@ -418,7 +421,8 @@ static int alloc_replica(sn_replica* r) {
       SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
       lstm_z = std::max(lstm_z, bh * 4);
       lstm_h = std::max(lstm_h, bh);
-      continue;  // output = last slice of lstm_h
+      if (op.ret_seq) SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
+      continue;  // output = last slice of lstm_h unless the whole sequence is returned
     }
     SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
     if (op.kind == OP_BATCHNORM) SN_TRY(dev_alloc(r, &r->bn_buf[i], 6 * align_up(op.out_dims.back(), 64)));
@@ -461,7 +465,7 @@ static const float* op_output(sn_replica* r, int i, const float* x, int rows) {
   if (i < 0) return x;
   const Op& op = r->model->ops[i];
   if (op.kind == OP_FLATTEN) return op_output(r, i - 1, x, rows);
-  if (op.kind == OP_LSTM) return r->lstm_h[i] + (int64_t)op.T * r->model->batch * op.H;
+  if (op.kind == OP_LSTM && !op.ret_seq) return r->lstm_h[i] + (int64_t)op.T * r->model->batch * op.H;
   return r->act[i];
 }
 
@@ -565,6 +569,7 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
                          r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
           SN_TRY(launch_lstm_gates_fwd(ctx, a, rows, op.H));
         }
+        if (op.ret_seq) SN_TRY(launch_sequence_gather(ctx, r->lstm_h[i], bh, 1, r->act[i], rows, op.T, op.H));
         break;
       }
       case OP_BATCHNORM: {
@@ -587,7 +592,13 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
           if (fused) SN_TRY(launch_rnn_step_fwd(ctx, in, t, op.T, op.F, r_prev, rows, op.H, r->lstm_pk_fwd[i], r_t));
           else SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, r_prev, rows, op.H, w, r_t, r->ws, m->workspace_elems, 1));
         }
-        SN_TRY(launch_bias_act(ctx, r->lstm_h[i] + (int64_t)op.T * bh, param_ptr(r, r->w, op.b), r->act[i], rows, op.H, op.act, op.act_param));
+        if (op.ret_seq) {  // every step's act(r_t + b), as (batch, time, units)
+          SN_TRY(launch_sequence_gather(ctx, r->lstm_h[i], bh, 1, r->act[i], rows, op.T, op.H));
+          SN_TRY(launch_bias_act(ctx, r->act[i], param_ptr(r, r->w, op.b), r->act[i], (int64_t)rows * op.T, op.H, op.act, op.act_param));
+        } else {
+          SN_TRY(launch_bias_act(ctx, r->lstm_h[i] + (int64_t)op.T * bh, param_ptr(r, r->w, op.b), r->act[i], rows, op.H, op.act,
+                                 op.act_param));
+        }
         break;
       }
     }
@@ -722,14 +733,18 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         SN_REQUIRE(rows == m->batch, "LSTM training needs rows == batch (%d), got %d", m->batch, rows);
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
-        const float* dh = dy;  // gradient of the last hidden state
-        int hb = 0, dh_parts = 1;
+        const float* dh = op.ret_seq ? nullptr : dy;  // gradient of the last hidden state (a returned sequence adds its own per step)
+        int hb = 0, dh_parts = op.ret_seq ? 0 : 1;
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
         if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
         for (int t = op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                             t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
                             r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0, dh_parts, bh};
+          if (op.ret_seq) {  // this step's own output gradient joins what the later steps carried back
+            a.dy_seq = dy + (int64_t)t * op.H;
+            a.dy_seq_ld = (int64_t)op.T * op.H;
+          }
           SN_TRY(launch_lstm_gates_bwd(ctx, a, rows, op.H));
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
           if (t > 0) {
@@ -738,6 +753,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
               dh_parts = 4;
             } else {
               SN_TRY(launch_lstm_dh(ctx, a.dz, rows, op.H, w, r->lstm_dh[hb], r->ws, m->workspace_elems));
+              dh_parts = 1;
             }
             dh = r->lstm_dh[hb];
             hb ^= 1;
@@ -768,14 +784,23 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         SN_REQUIRE(rows == m->batch, "RNN training needs rows == batch (%d), got %d", m->batch, rows);
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
-        // bias and activation touch the last step only; every earlier step acts through the carried state
         float* dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
-        SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dr, (int64_t)rows * op.H, op.act, op.act_param));
-        if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dr, op.H, param_ptr(r, r->g, op.b), rows, op.H, r->ws, m->workspace_elems));
+        if (op.ret_seq) {
+          // every step has an output: dz = act'(out) * dout over the whole (batch, time, units) tensor, in place; each
+          // step below adds its slice to the gradient carried back from the step after it
+          SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * op.T * op.H, op.act, op.act_param));
+          if (op.b >= 0)
+            SN_TRY(launch_col_sum(ctx, dy, op.H, param_ptr(r, r->g, op.b), (int64_t)rows * op.T, op.H, r->ws, m->workspace_elems));
+        } else {
+          // bias and activation touch the last step only; every earlier step acts through the carried state
+          SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dr, (int64_t)rows * op.H, op.act, op.act_param));
+          if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dr, op.H, param_ptr(r, r->g, op.b), rows, op.H, r->ws, m->workspace_elems));
+        }
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
         if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));
         for (int t = op.T - 1; t >= 0; --t) {
           dr = r->lstm_dz[i] + (int64_t)t * bh;
+          if (op.ret_seq) SN_TRY(launch_step_slice_add(ctx, dr, dy + (int64_t)t * op.H, (int64_t)op.T * op.H, rows, op.H, t < op.T - 1));
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, dr, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
           if (t > 0) {
             if (fused) SN_TRY(launch_lstm_step_dh(ctx, dr, rows, op.H, r->lstm_pk_dh[i], dr - bh, 0, 1));

@@ -222,6 +222,7 @@ class Layer:
     reg: Regularization = Zero
     use_bias: bool = True
     inits: Tuple[Initializer, ...] = ()
+    return_sequence: bool = False  # RNN layers only
     momentum: float = 0.99        # BatchNorm only
     epsilon: float = 1e-3
     fused: int = -1               # BatchNorm `fused`: -1 None, 0 Some(false), 1 Some(true)
@@ -236,7 +237,7 @@ class Layer:
     def desc(self) -> L.LayerDesc:
         return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
                            self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
-                           self.momentum, self.epsilon, self.fused)
+                           1 if self.return_sequence else 0, self.momentum, self.epsilon, self.fused)
 
     def __repr__(self):
         return self.text
@@ -303,10 +304,10 @@ Flatten = Layer(L.LAYER_FLATTEN, "Flatten")
 
 def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
          recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
-         biasForgetInitializer: Initializer = Ones) -> Layer:
+         biasForgetInitializer: Initializer = Ones, returnSequence: bool = False) -> Layer:
     """layer/RNN.scala:208-258: tanh cell, sigmoid gates, forget bias one."""
     return Layer(L.LAYER_LSTM, f"RNN(LSTMCell({units},Tanh,Sigmoid,{'true' if bias else 'false'}))", units=units,
-                 activation=Tanh, use_bias=bias,
+                 activation=Tanh, use_bias=bias, return_sequence=returnSequence,
                  inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
 
 
@@ -323,12 +324,14 @@ def BatchNorm(axes: Sequence[int] = (-1,), momentum: float = 0.99, epsilon: floa
 
 
 def SimpleRNN(units: int, activation: Activation = Tanh, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
-              recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros) -> Layer:
+              recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
+              returnSequence: bool = False) -> Layer:
     """layer/RNN.scala:96-137: `RNN(SimpleRNNCell(..))`; the last step's output leaves the layer."""
     if activation.kind == L.ACT_SOFTMAX:
         raise ValueError("requirement failed: Softmax is not a cell activation")
     return Layer(L.LAYER_SIMPLE_RNN, f"RNN(SimpleRNNCell({units},{activation!r},{'true' if bias else 'false'}))", units=units,
-                 activation=activation, use_bias=bias, inits=(kernelInitializer, recurrentInitializer, biasInitializer))
+                 activation=activation, use_bias=bias, return_sequence=returnSequence,
+                 inits=(kernelInitializer, recurrentInitializer, biasInitializer))
 
 
 def LinearRegression(reg: Regularization = Zero, bias: bool = True):

@@ -47,15 +47,17 @@ def build_pair(spec: List[tuple], loss: str):
         elif k == "flatten":
             ol.append(O.Flatten())
             add(S.Flatten)
-        elif k == "lstm":
+        elif k == "lstm":     # ("lstm", units[, bias[, return_sequence]])
             bias = e[2] if len(e) > 2 else True
-            ol.append(O.LSTM(e[1], bias=bias))
-            add(S.LSTM(e[1], bias=bias))
-        elif k == "simple_rnn":  # ("simple_rnn", units[, act[, bias]])
+            seq = e[3] if len(e) > 3 else False
+            ol.append(O.LSTM(e[1], bias=bias, return_sequence=seq))
+            add(S.LSTM(e[1], bias=bias, returnSequence=seq))
+        elif k == "simple_rnn":  # ("simple_rnn", units[, act[, bias[, return_sequence]]])
             act = e[2] if len(e) > 2 else "tanh"
             bias = e[3] if len(e) > 3 else True
-            ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias))
-            add(S.SimpleRNN(e[1], acts_s[act], bias=bias))
+            seq = e[4] if len(e) > 4 else False
+            ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias, return_sequence=seq))
+            add(S.SimpleRNN(e[1], acts_s[act], bias=bias, returnSequence=seq))
         elif k == "batchnorm":   # ("batchnorm", momentum, epsilon): the generic form (fused = Some(false))
             ol.append(O.BatchNorm(e[1], e[2]))
             add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=False))

@@ -329,6 +329,14 @@ MODELS = {
                                ("activate", "relu"), ("flatten",), ("dense", 4, "softmax")], "cce", (9, 10, 3), 7, "uniform_onehot"),
     "lstm_small": ([("lstm", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
     "lstm_fused_shape": ([("lstm", 32), ("dense", 2, "identity")], "mse", (7, 8), 50, "normal_regression"),
+    # `returnSequence = true` stacks recurrent layers (layer/RNN.scala:27,74-77): fused-kernel shapes and general ones
+    "lstm_stacked": ([("lstm", 16, True, True), ("lstm", 8), ("dense", 1, "tanh")], "mse", (6, 8), 20, "normal_regression"),
+    "lstm_stacked_general": ([("activate", "tanh"), ("lstm", 5, False, True), ("lstm", 3), ("dense", 2, "identity")], "mse", (4, 3), 9,
+                             "normal_regression"),
+    "simple_rnn_stacked": ([("simple_rnn", 16, "relu", True, True), ("simple_rnn", 4, "tanh"), ("dense", 2, "identity")], "mse", (6, 8), 20,
+                           "normal_regression"),
+    "simple_rnn_stacked_general": ([("activate", "tanh"), ("simple_rnn", 5, "sigmoid", False, True), ("simple_rnn", 3), ("dense", 1, "tanh")],
+                                   "mse", (4, 3), 9, "normal_regression"),
     "lstm_after_activation": ([("activate", "tanh"), ("lstm", 8), ("dense", 1, "tanh")], "mse", (5, 6), 12, "normal_regression"),
     "simple_rnn_small": ([("simple_rnn", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
     "simple_rnn_relu_nobias_after_activation": ([("activate", "tanh"), ("simple_rnn", 17, "relu", False), ("dense", 3, "identity")],
@@ -401,7 +409,7 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     h.close()
 
 
-@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("simple_rnn_small", 30),
+@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
                                         ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("mlp_bce_l2", 25)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
 def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):

@@ -394,7 +394,8 @@ def _rand_params(m, in_shape, rng, dt=np.float64, scale=0.4):
     return {p: (rng.standard_normal(s) * scale).astype(dt) for p, s in m.param_defs(in_shape)}
 
 
-@pytest.mark.parametrize("name", ["mlp_cce", "cnn_cce", "lstm_mse", "rnn_mse", "mlp_batchnorm", "cnn_batchnorm", "mlp_bce_l2"])
+@pytest.mark.parametrize("name", ["mlp_cce", "cnn_cce", "lstm_mse", "rnn_mse", "lstm_stacked", "rnn_stacked", "mlp_batchnorm",
+                                  "cnn_batchnorm", "mlp_bce_l2"])
 def test_model_gradients_match_numeric_float64(name):
     rng = np.random.default_rng(11)
     if name == "mlp_cce":
@@ -414,6 +415,14 @@ def test_model_gradients_match_numeric_float64(name):
         m = O.Model([O.SimpleRNN(3), O.Dense(2)], O.LOSS_MSE)
         x = rng.standard_normal((2, 4, 3))
         y = rng.uniform(-1, 1, (2, 2))
+    elif name == "lstm_stacked":      # `returnSequence = true` feeds every step's output to the next layer (RNN.scala:74-77)
+        m = O.Model([O.LSTM(3, return_sequence=True), O.LSTM(2), O.Dense(1)], O.LOSS_MSE)
+        x = rng.standard_normal((3, 4, 2))
+        y = rng.uniform(-1, 1, (3, 1))
+    elif name == "rnn_stacked":
+        m = O.Model([O.SimpleRNN(3, O.ACT_SIGMOID, return_sequence=True), O.SimpleRNN(2), O.Dense(1)], O.LOSS_MSE)
+        x = rng.standard_normal((3, 4, 2))
+        y = rng.uniform(-1, 1, (3, 1))
     elif name == "mlp_batchnorm":     # batch statistics depend on the input: the gradient runs through mean and variance
         m = O.Model([O.Dense(5, O.ACT_TANH), O.BatchNorm(0.9, 1e-3), O.Dense(3, O.ACT_SOFTMAX)], O.LOSS_CCE)
         x = rng.standard_normal((6, 4))
