@@ -62,7 +62,7 @@ enum { SN_ACT_IDENTITY = 0, SN_ACT_SIGMOID = 1, SN_ACT_TANH = 2, SN_ACT_RELU = 3
 /* models/Loss.scala:18-57 */
 enum { SN_LOSS_IDENTITY = 0, SN_LOSS_MSE = 1, SN_LOSS_BINARY_CROSSENTROPY = 2, SN_LOSS_CATEGORICAL_CROSSENTROPY = 3 };
 /* math/nn/AllKernels.scala:25-103 */
-enum { SN_PAD_VALID = 0, SN_PAD_SAME = 1 };
+enum { SN_PAD_VALID = 0, SN_PAD_SAME = 1, SN_PAD_EXPLICIT = 2 /* Conv2D only: pad_top .. pad_right below */ };
 /* models/Regularization.scala:16-44 */
 enum { SN_REG_NONE = 0, SN_REG_L1 = 1, SN_REG_L2 = 2 };
 /* optimizers/{SGD,AdaGrad,AdaDelta,RMSProp,Adam,Nadam,Adamax,AMSGrad}.scala */
@@ -98,6 +98,8 @@ typedef struct sn_layer_desc {
                               output, (batch, time, units), instead of the last one */
   float bn_momentum;     /* BATCHNORM (layer/BatchNorm.scala:64-76, axes = Seq(-1)): decay of the moving statistics */
   float bn_epsilon;      /* BATCHNORM: added to the variance */
+  int32_t pad_top, pad_bottom, pad_left, pad_right; /* CONV2D with SN_PAD_EXPLICIT: `Explicit((top, bottom), (left, right))`,
+                            output size ceil((in + pads - window) / stride) + 1 (math/nn/AllKernels.scala:67-91) */
   int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  Only the generic
                             form (math/nn/AllKernels.scala:663-684) is built: whenever the reference would take
                             FusedBatchNormV3 (rank-4 input unless fused = Some(false)) model creation fails. */

@@ -361,6 +361,7 @@ class Layer:
     kernel: Tuple[int, int] = (3, 3)
     strides: Tuple[int, int] = (1, 1)
     padding: int = PAD_VALID
+    explicit: Tuple[int, int, int, int] = (0, 0, 0, 0)   # conv2d with PAD_EXPLICIT: top, bottom, left, right (AllKernels.scala:67-100)
     reg: int = REG_NONE
     reg_lambda: float = 0.0
     bias: bool = True               # lstm / simple_rnn only
@@ -405,8 +406,8 @@ class Layer:
         if self.kind == "flatten":      # Flatten.scala:12-18
             return (s[0], int(np.prod(s[1:])))
         if self.kind == "conv2d":
-            return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0]),
-                    out_size(self.padding, s[2], self.kernel[1], self.strides[1]), self.units)
+            return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0], self.explicit[0:2]),
+                    out_size(self.padding, s[2], self.kernel[1], self.strides[1], self.explicit[2:4]), self.units)
         if self.kind == "pool2d":
             return (s[0], out_size(self.padding, s[1], self.kernel[0], self.strides[0]),
                     out_size(self.padding, s[2], self.kernel[1], self.strides[1]), s[3])
@@ -426,9 +427,9 @@ def Dense(units, activation=ACT_IDENTITY, act_param=0.0, reg=REG_NONE, reg_lambd
 
 
 def Conv2D(filters, kernel=(3, 3), strides=(1, 1), padding=PAD_VALID, activation=ACT_IDENTITY,
-           act_param=0.0, bias=False):
-    """Conv2D.scala:54-68: defaults Valid, stride 1, no bias."""
-    out = [Layer("conv2d", units=filters, kernel=kernel, strides=strides, padding=padding)]
+           act_param=0.0, bias=False, explicit=(0, 0, 0, 0)):
+    """Conv2D.scala:54-68: defaults Valid, stride 1, no bias; `explicit` = (top, bottom, left, right) with PAD_EXPLICIT."""
+    out = [Layer("conv2d", units=filters, kernel=kernel, strides=strides, padding=padding, explicit=tuple(explicit))]
     if bias:
         out.append(Layer("bias", units=filters))
     if activation != ACT_IDENTITY:
@@ -566,7 +567,7 @@ class Model:
                 c = x.shape
             elif k == "conv2d":
                 w = params[pre + "weights"]
-                y = conv2d(x, w, l.strides, l.padding)
+                y = conv2d(x, w, l.strides, l.padding, l.explicit)
                 c = (x, w)
             elif k == "pool2d":
                 y = max_pool(x, l.kernel, l.strides, l.padding)
@@ -636,8 +637,8 @@ class Model:
                 dy = dy.reshape(c)
             elif k == "conv2d":
                 xi, w = c
-                grads[pre + "weights"] = conv2d_grad_filter(xi, w.shape, dy, l.strides, l.padding)
-                dy = conv2d_grad_input(xi.shape, w, dy, l.strides, l.padding) if i > 0 else None
+                grads[pre + "weights"] = conv2d_grad_filter(xi, w.shape, dy, l.strides, l.padding, l.explicit)
+                dy = conv2d_grad_input(xi.shape, w, dy, l.strides, l.padding, l.explicit) if i > 0 else None
             elif k == "pool2d":
                 dy = max_pool_grad(c, dy, l.kernel, l.strides, l.padding)
             elif k == "lstm":

@@ -22,7 +22,7 @@ ACT_IDENTITY, ACT_SIGMOID, ACT_TANH, ACT_RELU, ACT_SOFTMAX = range(5)
 RANDOM_UNIFORM, RANDOM_NORMAL, RANDOM_TRUNCATED_NORMAL = range(3)
 ERROR_SQUARED, ERROR_ABSOLUTE = range(2)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
-PAD_VALID, PAD_SAME = 0, 1
+PAD_VALID, PAD_SAME, PAD_EXPLICIT = 0, 1, 2
 REG_NONE, REG_L1, REG_L2 = 0, 1, 2
 OPT_SGD, OPT_ADAGRAD, OPT_ADADELTA, OPT_RMSPROP, OPT_ADAM, OPT_NADAM, OPT_ADAMAX, OPT_AMSGRAD = range(8)
 FLAG_GEMM_BF16 = 1
@@ -42,7 +42,9 @@ class LayerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("units", C.c_int32), ("activation", C.c_int32), ("act_param", C.c_float),
                 ("kernel_h", C.c_int32), ("kernel_w", C.c_int32), ("stride_h", C.c_int32), ("stride_w", C.c_int32),
                 ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32),
-                ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float), ("bn_fused", C.c_int32)]
+                ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float),
+                ("pad_top", C.c_int32), ("pad_bottom", C.c_int32), ("pad_left", C.c_int32), ("pad_right", C.c_int32),
+                ("bn_fused", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):

@@ -117,8 +117,12 @@ static int64_t prod(const std::vector<int64_t>& d) {
 }
 
 // Padding.size / TensorFlow's SAME rule (math/nn/AllKernels.scala:39-65): extra padding goes after.
-static void conv_out(int padding, int in, int k, int s, int* out, int* pad_before) {
-  if (padding == SN_PAD_SAME) {
+static void conv_out(int padding, int in, int k, int s, int* out, int* pad_before, int lo = 0, int hi = 0) {
+  if (padding == SN_PAD_EXPLICIT) {  // math/nn/AllKernels.scala:74-91
+    const int span = in + lo + hi - k;
+    *out = span < 0 ? 0 : (span + s - 1) / s + 1;
+    *pad_before = lo;
+  } else if (padding == SN_PAD_SAME) {
     *out = (in + s - 1) / s;
     const int total = std::max((*out - 1) * s + k - in, 0);
     *pad_before = total / 2;
@@ -190,12 +194,14 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         SN_REQUIRE(cur.size() == 3, "layer %d: Conv2D input should have a shape (NHWC) but was rank %zu", i, cur.size() + 1);
         SN_REQUIRE(L.units > 0 && L.kernel_h > 0 && L.kernel_w > 0 && L.stride_h > 0 && L.stride_w > 0,
                    "layer %d: Conv2D needs positive filters, kernel and strides", i);
-        SN_REQUIRE(L.padding == SN_PAD_VALID || L.padding == SN_PAD_SAME, "layer %d: unknown padding %d", i, L.padding);
+        SN_REQUIRE(L.padding >= SN_PAD_VALID && L.padding <= SN_PAD_EXPLICIT, "layer %d: unknown padding %d", i, L.padding);
+        SN_REQUIRE(L.padding != SN_PAD_EXPLICIT || (L.pad_top >= 0 && L.pad_bottom >= 0 && L.pad_left >= 0 && L.pad_right >= 0),
+                   "layer %d: explicit paddings must not be negative", i);
         op.kind = OP_CONV;
         op.kh = L.kernel_h; op.kw = L.kernel_w; op.sh = L.stride_h; op.sw = L.stride_w;
         int ho, wo;
-        conv_out(L.padding, (int)cur[0], op.kh, op.sh, &ho, &op.pt);
-        conv_out(L.padding, (int)cur[1], op.kw, op.sw, &wo, &op.pl);
+        conv_out(L.padding, (int)cur[0], op.kh, op.sh, &ho, &op.pt, L.pad_top, L.pad_bottom);
+        conv_out(L.padding, (int)cur[1], op.kw, op.sw, &wo, &op.pl, L.pad_left, L.pad_right);
         SN_REQUIRE(ho > 0 && wo > 0, "layer %d: Conv2D kernel larger than its input", i);
         op.w = add_param(m, prefix(i) + "weights", {op.kh, op.kw, cur[2], L.units}, SN_REG_NONE, 0.f);
         op.out_dims = {ho, wo, L.units};

@@ -85,6 +85,17 @@ def L2(lam: float = 0.01) -> Regularization:
 Valid, Same = L.PAD_VALID, L.PAD_SAME
 _PAD_NAME = {Valid: "Valid", Same: "Same"}
 
+
+@dataclass(frozen=True)
+class Explicit:
+    """`Padding.Explicit((pad_top, pad_bottom), (pad_left, pad_right))` (math/nn/AllKernels.scala:67-100); Conv2D only."""
+    height: Tuple[int, int]
+    width: Tuple[int, int]
+
+    def __repr__(self):
+        return f"Explicit({tuple(self.height)},{tuple(self.width)})"
+
+
 # --------------------------------------------------------------------------- initializers (models/Initializer.scala)
 
 
@@ -222,6 +233,7 @@ class Layer:
     reg: Regularization = Zero
     use_bias: bool = True
     inits: Tuple[Initializer, ...] = ()
+    explicit: Tuple[int, int, int, int] = (0, 0, 0, 0)   # Conv2D with explicit padding: top, bottom, left, right
     return_sequence: bool = False  # RNN layers only
     momentum: float = 0.99        # BatchNorm only
     epsilon: float = 1e-3
@@ -237,7 +249,8 @@ class Layer:
     def desc(self) -> L.LayerDesc:
         return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
                            self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
-                           1 if self.return_sequence else 0, self.momentum, self.epsilon, self.fused)
+                           1 if self.return_sequence else 0, self.momentum, self.epsilon,
+                           self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused)
 
     def __repr__(self):
         return self.text
@@ -286,9 +299,15 @@ def Dense(outputs: int, activation: Activation = Identity, reg: Regularization =
 def Conv2D(filters: int, kernel: Tuple[int, int] = (3, 3), strides: Tuple[int, int] = (1, 1), padding: int = Valid,
            activation: Activation = Identity, bias: bool = False, kernelInitializer: Initializer = GlorotUniform(),
            biasInitializer: Initializer = Zeros):
-    """layer/Conv2D.scala:54-68."""
-    conv = Layer(L.LAYER_CONV2D, f"Conv2D({filters},{tuple(kernel)},{tuple(strides)},{_PAD_NAME[padding]},NHWC)".replace(" ", ""),
-                 units=filters, kernel=tuple(kernel), strides=tuple(strides), padding=padding, inits=(kernelInitializer,))
+    """layer/Conv2D.scala:54-68; `padding` is Valid, Same or an `Explicit(..)`."""
+    explicit = (0, 0, 0, 0)
+    pad_name = repr(padding) if isinstance(padding, Explicit) else _PAD_NAME[padding]
+    if isinstance(padding, Explicit):
+        explicit = (int(padding.height[0]), int(padding.height[1]), int(padding.width[0]), int(padding.width[1]))
+        padding = L.PAD_EXPLICIT
+    conv = Layer(L.LAYER_CONV2D, f"Conv2D({filters},{tuple(kernel)},{tuple(strides)},{pad_name},NHWC)".replace(" ", ""),
+                 units=filters, kernel=tuple(kernel), strides=tuple(strides), padding=padding, explicit=explicit,
+                 inits=(kernelInitializer,))
     return _chain(conv, Bias(filters, Zero, biasInitializer) if bias else None,
                   Activate(activation) if not activation.identity else None)
 

@@ -38,8 +38,12 @@ def build_pair(spec: List[tuple], loss: str):
             add(S.Dense(units, acts_s[act], reg=sreg))
         elif k == "conv":
             _, filters, kernel, strides, pad, act, bias = e
-            ol.append(O.Conv2D(filters, kernel, strides, pads_o[pad], acts_o[act], bias=bias))
-            add(S.Conv2D(filters, kernel, strides, pads_s[pad], acts_s[act], bias=bias))
+            if isinstance(pad, tuple):      # explicit paddings (top, bottom, left, right)
+                ol.append(O.Conv2D(filters, kernel, strides, O.PAD_EXPLICIT, acts_o[act], bias=bias, explicit=pad))
+                add(S.Conv2D(filters, kernel, strides, S.Explicit(pad[0:2], pad[2:4]), acts_s[act], bias=bias))
+            else:
+                ol.append(O.Conv2D(filters, kernel, strides, pads_o[pad], acts_o[act], bias=bias))
+                add(S.Conv2D(filters, kernel, strides, pads_s[pad], acts_s[act], bias=bias))
         elif k == "pool":
             _, window, strides, pad = e
             ol.append(O.Pool2D(window, strides, pads_o[pad]))

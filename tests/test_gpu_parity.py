@@ -228,6 +228,17 @@ def test_golden_conv_and_pool(S, ctx, golden, key, strides, pad):
     h.close()
 
 
+def test_golden_conv_explicit_padding(S, ctx, golden):
+    """math/nn/KernelsSpec.scala (explicit paddings (1, 0), (1, 0), stride 2) through the layer."""
+    g = golden["conv2d"]
+    h = Harness(S, ctx, [("conv", 1, (2, 2), (2, 2), (1, 0, 1, 0), "identity", False)], "mse", (5, 5, 1), 1)
+    assert h.cm.output_shape == (3, 3, 1)
+    h.rep.set_params({"weights": A(golden["filter_2x2"]).reshape(2, 2, 1, 1)})
+    out = h.rep.forward(ctx.to_device(A(golden["image_5x5"]).reshape(1, 5, 5, 1)))
+    np.testing.assert_array_equal(out.reshape(3, 3), A(g["explicit_1010_s2"]))
+    h.close()
+
+
 def test_golden_conv_pool_gradients(S, ctx, golden):
     """d sum(conv)/d filter and d sum(pool(conv))/.. via a model whose loss gradient is all ones:
     MSE against y = out - size/2 gives d loss / d out = 1 exactly."""
@@ -327,6 +338,8 @@ MODELS = {
                      ("flatten",), ("dense", 10, "softmax")], "cce", (12, 12, 1), 20, "uniform_onehot"),
     "cnn_same_stride2_bias": ([("conv", 5, (3, 2), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "same"),
                                ("activate", "relu"), ("flatten",), ("dense", 4, "softmax")], "cce", (9, 10, 3), 7, "uniform_onehot"),
+    "cnn_explicit_padding": ([("conv", 6, (3, 2), (2, 1), (1, 0, 2, 1), "tanh", True), ("conv", 4, (2, 2), (1, 1), (0, 1, 0, 0), "relu", False),
+                              ("flatten",), ("dense", 3, "softmax")], "cce", (7, 6, 2), 11, "uniform_onehot"),
     "lstm_small": ([("lstm", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),
     "lstm_fused_shape": ([("lstm", 32), ("dense", 2, "identity")], "mse", (7, 8), 50, "normal_regression"),
     # `returnSequence = true` stacks recurrent layers (layer/RNN.scala:27,74-77): fused-kernel shapes and general ones
