@@ -62,6 +62,10 @@ enum { SN_ACT_IDENTITY = 0, SN_ACT_SIGMOID = 1, SN_ACT_TANH = 2, SN_ACT_RELU = 3
 /* models/Loss.scala:18-57 */
 enum { SN_LOSS_IDENTITY = 0, SN_LOSS_MSE = 1, SN_LOSS_BINARY_CROSSENTROPY = 2, SN_LOSS_CATEGORICAL_CROSSENTROPY = 3 };
 /* math/nn/AllKernels.scala:25-103 */
+/* `Reduce` of `pool2D` (math/nn/AllKernels.scala:383-397).  The reference's Pool2D LAYER never hands its `reduce` to
+ * the kernel (layer/Pool2D.scala:36-42), so every model it builds max-pools; a binding that mirrors the layer as it is
+ * passes SN_POOL_MAX whatever the layer says, one that mirrors the kernel function passes the argument through. */
+enum { SN_POOL_MAX = 0, SN_POOL_AVG = 1 };
 enum { SN_PAD_VALID = 0, SN_PAD_SAME = 1, SN_PAD_EXPLICIT = 2 /* Conv2D only: pad_top .. pad_right below */ };
 /* models/Regularization.scala:16-44 */
 enum { SN_REG_NONE = 0, SN_REG_L1 = 1, SN_REG_L2 = 2 };
@@ -103,6 +107,7 @@ typedef struct sn_layer_desc {
   int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  Only the generic
                             form (math/nn/AllKernels.scala:663-684) is built: whenever the reference would take
                             FusedBatchNormV3 (rank-4 input unless fused = Some(false)) model creation fails. */
+  int32_t pool_reduce;   /* POOL2D: SN_POOL_*.  AVG divides by the number of window cells inside the input (TF AvgPool) */
 } sn_layer_desc;
 
 /* An `Algorithm` case class (optimizers/Algorithm.scala:6-11).  Field use per kind:

@@ -16,6 +16,7 @@ What pins each part (see tests/test_oracle_golden.py):
   * softmax rows, tanh, relu, exp, log, sigmoid points ........... reference goldens
   * conv2d (same/valid/explicit, stride 1/2), both conv grads ..... reference goldens + brute force + torch
   * max pool (same/valid, stride 1/2), max-pool grad with ties .... reference goldens + brute force
+  * average pool and its gradient (padding cells not counted) ..... reference goldens + brute force + numeric gradient
   * SimpleRNN and LSTM forward ................................... reference goldens
   * LSTM / conv / pool / softmax+CCE backward .................... float64 numerical gradients + torch autograd
   * BatchNorm (generic form): training output, next moving
@@ -344,6 +345,49 @@ def max_pool_grad(x, dy, window=(2, 2), strides=(1, 1), padding=PAD_VALID):
     return dxp[:, pt:pt + h, pl:pl + wd, :]
 
 
+def _window_cells(shape, window, strides, padding):
+    """Number of cells of each pooling window that lie inside the input: [Ho, Wo]."""
+    kh, kw = window
+    n, h, wd, _ = shape
+    ho, wo, pt, pb, pl, pr = _geometry(shape, kh, kw, strides, padding, (0, 0, 0, 0))
+    y0 = np.arange(ho) * strides[0] - pt
+    x0 = np.arange(wo) * strides[1] - pl
+    rows = np.minimum(y0 + kh, h) - np.maximum(y0, 0)
+    cols = np.minimum(x0 + kw, wd) - np.maximum(x0, 0)
+    return rows[:, None] * cols[None, :]
+
+
+def avg_pool(x, window=(2, 2), strides=(1, 1), padding=PAD_VALID):
+    """TF `AvgPool`, NHWC (nn/AllKernels.scala:326-353): the mean over the window's cells inside the input (padding
+    cells are not counted)."""
+    kh, kw = window
+    ho, wo, pt, pb, pl, pr = _geometry(x.shape, kh, kw, strides, padding, (0, 0, 0, 0))
+    xp = np.pad(x, ((0, 0), (pt, pb), (pl, pr), (0, 0)))
+    p = _patches(xp, kh, kw, strides[0], strides[1], ho, wo)       # [N,Ho,Wo,kh,kw,C]
+    total = np.zeros(p.shape[:3] + p.shape[5:], dtype=x.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            total = total + p[:, :, :, r, q, :]
+    cells = _window_cells(x.shape, window, strides, padding).astype(x.dtype)
+    return total / cells[None, :, :, None]
+
+
+def avg_pool_grad(xshape, dy, window=(2, 2), strides=(1, 1), padding=PAD_VALID):
+    """TF `AvgPoolGrad` (nn/AllKernels.scala:355-381): every cell of a window gets the window's gradient times
+    1 / (its cells inside the input)."""
+    kh, kw = window
+    sh, sw = strides
+    n, h, wd, c = xshape
+    ho, wo, pt, pb, pl, pr = _geometry(xshape, kh, kw, strides, padding, (0, 0, 0, 0))
+    share = (dy.dtype.type(1) / _window_cells(xshape, window, strides, padding).astype(dy.dtype))[None, :, :, None]
+    part = dy * share
+    dxp = np.zeros((n, h + pt + pb, wd + pl + pr, c), dtype=dy.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            dxp[:, r:r + sh * ho:sh, q:q + sw * wo:sw, :] += part
+    return dxp[:, pt:pt + h, pl:pl + wd, :]
+
+
 # --------------------------------------------------------------------------- #
 # layers (models/layer/*.scala) -- the flattened `Composed` list
 # --------------------------------------------------------------------------- #
@@ -369,6 +413,7 @@ class Layer:
     return_sequence: bool = False   # lstm / simple_rnn: every step's output, (batch, time, units) (RNN.scala:27,75-77)
     momentum: float = 0.99          # batchnorm (BatchNorm.scala:66-67)
     epsilon: float = 1e-3
+    pool_avg: bool = False          # pool2d: mean of the window (kernel-level `Reduce.Avg`) instead of its maximum
 
     # ---- parameter definitions, in flat-buffer order ---------------------- #
     def params(self, in_shape) -> List[Tuple[str, Tuple[int, ...]]]:
@@ -437,9 +482,11 @@ def Conv2D(filters, kernel=(3, 3), strides=(1, 1), padding=PAD_VALID, activation
     return out
 
 
-def Pool2D(window=(2, 2), strides=(1, 1), padding=PAD_VALID):
-    """Pool2D.scala:28-42: the layer always max-pools."""
-    return [Layer("pool2d", kernel=window, strides=strides, padding=padding)]
+def Pool2D(window=(2, 2), strides=(1, 1), padding=PAD_VALID, reduce="Max", as_reference_layer=True):
+    """Pool2D.scala:28-42.  `build` (:36-42) calls `pool2D` without `reduce`, so the reference's layer max-pools
+    whatever it was given; `as_reference_layer=False` gives the layer the kernel function's `Reduce.Avg` instead."""
+    avg = reduce == "Avg" and not as_reference_layer
+    return [Layer("pool2d", kernel=window, strides=strides, padding=padding, pool_avg=avg)]
 
 
 def Flatten():
@@ -570,7 +617,7 @@ class Model:
                 y = conv2d(x, w, l.strides, l.padding, l.explicit)
                 c = (x, w)
             elif k == "pool2d":
-                y = max_pool(x, l.kernel, l.strides, l.padding)
+                y = (avg_pool if l.pool_avg else max_pool)(x, l.kernel, l.strides, l.padding)
                 c = x
             elif k == "lstm":
                 y, c = lstm_forward(x, params, pre, l)
@@ -640,7 +687,8 @@ class Model:
                 grads[pre + "weights"] = conv2d_grad_filter(xi, w.shape, dy, l.strides, l.padding, l.explicit)
                 dy = conv2d_grad_input(xi.shape, w, dy, l.strides, l.padding, l.explicit) if i > 0 else None
             elif k == "pool2d":
-                dy = max_pool_grad(c, dy, l.kernel, l.strides, l.padding)
+                dy = (avg_pool_grad(c.shape, dy, l.kernel, l.strides, l.padding) if l.pool_avg
+                      else max_pool_grad(c, dy, l.kernel, l.strides, l.padding))
             elif k == "lstm":
                 dy = lstm_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
             elif k == "simple_rnn":

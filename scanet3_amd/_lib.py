@@ -23,6 +23,7 @@ RANDOM_UNIFORM, RANDOM_NORMAL, RANDOM_TRUNCATED_NORMAL = range(3)
 ERROR_SQUARED, ERROR_ABSOLUTE = range(2)
 LOSS_IDENTITY, LOSS_MSE, LOSS_BINARY_CROSSENTROPY, LOSS_CATEGORICAL_CROSSENTROPY = range(4)
 PAD_VALID, PAD_SAME, PAD_EXPLICIT = 0, 1, 2
+POOL_MAX, POOL_AVG = 0, 1
 REG_NONE, REG_L1, REG_L2 = 0, 1, 2
 OPT_SGD, OPT_ADAGRAD, OPT_ADADELTA, OPT_RMSPROP, OPT_ADAM, OPT_NADAM, OPT_ADAMAX, OPT_AMSGRAD = range(8)
 FLAG_GEMM_BF16 = 1
@@ -44,7 +45,7 @@ class LayerDesc(C.Structure):
                 ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32),
                 ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float),
                 ("pad_top", C.c_int32), ("pad_bottom", C.c_int32), ("pad_left", C.c_int32), ("pad_right", C.c_int32),
-                ("bn_fused", C.c_int32)]
+                ("bn_fused", C.c_int32), ("pool_reduce", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):

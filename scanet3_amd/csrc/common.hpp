@@ -134,11 +134,11 @@ int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t
 int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev);
 int launch_penalty_grad(sn_ctx* ctx, const float* w, float* g, int64_t n, int reg_kind, float lambda);
 int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, int cols, unsigned long long* count_dev);
-int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo,
+int launch_pool_fwd(sn_ctx* ctx, bool avg, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo,
                        int kh, int kw, int sh, int sw, int pt, int pl);
 // y_in (optional): the pooled tensor when it is the output of a layer with activation `act`; the kernel then
 // returns act'(y_in) * gradient, i.e. that layer's pre-activation gradient, saving a pass over the tensor
-int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho,
+int launch_pool_bwd(sn_ctx* ctx, bool avg, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho,
                        int wo, int kh, int kw, int sh, int sw, int pt, int pl, const float* y_in = nullptr, int act = SN_ACT_IDENTITY,
                        float act_param = 0.f);
 struct LstmGateArgs {

@@ -1,5 +1,5 @@
 // Memory-bound layer kernels: bias + activation, activation backward, softmax rows,
-// losses, column sums (bias gradients), regularisation, max pooling, LSTM gate maths
+// losses, column sums (bias gradients), regularisation, max and average pooling, LSTM gate maths
 // and the accuracy count.  All arithmetic is float32 in the reference's operation
 // order (no fused multiply-add; the file is compiled with -ffp-contract=off).
 #include "common.hpp"
@@ -479,12 +479,14 @@ static inline unsigned grid_for_xcd(sn_ctx* ctx, int64_t n, int per_block) {
   return (grid_for(ctx, n, per_block) + 7u) & ~7u;
 }
 
-// ---------------------------------------------------------------------------- max pooling (NHWC)
+// ---------------------------------------------------------------------------- pooling (NHWC)
 // Forward keeps, per output element, the window offset (r*kw + q) of the first maximum in
 // row-major window order; padding cells never win (TF MaxPoolV2, math/nn/AllKernels.scala:270-303).
 // V channels per thread (V = 4 needs c % 4 == 0 and 16-byte aligned tensors); I is the index type.
-template <int V, typename I>
-__global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
+// AVG: the mean over the window's cells that lie inside the input instead (TF AvgPool, math/nn/AllKernels.scala:326-353);
+// nothing is recorded for the backward pass.
+template <int V, typename I, bool AVG>
+__global__ __launch_bounds__(256) void pool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
                                                            int n, int h, int w, int c, int ho, int wo, int kh, int kw, int sh,
                                                            int sw, int pt, int pl) {
   const I cv = (I)(c / V);
@@ -499,7 +501,8 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restric
     float best[V];
     int at[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) { best[v] = -INFINITY; at[v] = 0; }
+    for (int v = 0; v < V; ++v) { best[v] = AVG ? 0.f : -INFINITY; at[v] = 0; }
+    int cells = 0;
     for (int r = 0; r < kh; ++r) {
       const int iy = oh * sh - pt + r;
       if (iy < 0 || iy >= h) continue;
@@ -510,18 +513,26 @@ __global__ __launch_bounds__(256) void maxpool_fwd_kernel(const float* __restric
         float val[V];
         if constexpr (V == 4) { const float4 f = *(const float4*)src; val[0] = f.x; val[1] = f.y; val[2] = f.z; val[3] = f.w; }
         else val[0] = *src;
+        ++cells;
 #pragma unroll
-        for (int v = 0; v < V; ++v)
-          if (val[v] > best[v]) { best[v] = val[v]; at[v] = r * kw + q; }
+        for (int v = 0; v < V; ++v) {
+          if constexpr (AVG) best[v] += val[v];
+          else if (val[v] > best[v]) { best[v] = val[v]; at[v] = r * kw + q; }
+        }
       }
+    }
+    if constexpr (AVG) {
+      const float count = (float)(cells > 0 ? cells : 1);
+#pragma unroll
+      for (int v = 0; v < V; ++v) best[v] = best[v] / count;
     }
     const I o = i * V;
     if constexpr (V == 4) {
       *(float4*)(y + o) = make_float4(best[0], best[1], best[2], best[3]);
-      *(uint32_t*)(arg + o) = (uint32_t)at[0] | ((uint32_t)at[1] << 8) | ((uint32_t)at[2] << 16) | ((uint32_t)at[3] << 24);
+      if constexpr (!AVG) *(uint32_t*)(arg + o) = (uint32_t)at[0] | ((uint32_t)at[1] << 8) | ((uint32_t)at[2] << 16) | ((uint32_t)at[3] << 24);
     } else {
       y[o] = best[0];
-      arg[o] = (uint8_t)at[0];
+      if constexpr (!AVG) arg[o] = (uint8_t)at[0];
     }
   }
 }
@@ -530,16 +541,19 @@ static bool pool_vec4(const void* a, const void* b, const void* m, int c) {
   return c % 4 == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0 && (reinterpret_cast<uintptr_t>(m) & 3u) == 0;
 }
 
-int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo, int kh,
-                       int kw, int sh, int sw, int pt, int pl) {
+int launch_pool_fwd(sn_ctx* ctx, bool avg, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo, int kh,
+                    int kw, int sh, int sw, int pt, int pl) {
   const int64_t total = (int64_t)n * ho * wo * c;
   if (total <= 0) return SN_OK;
   const bool small = total < (1ll << 31) && (int64_t)n * h * w * c < (1ll << 31);
   const bool v4 = pool_vec4(x, y, arg, c);
   const dim3 grid(grid_for_xcd(ctx, v4 ? total / 4 : total, 256));
-  LaunchScope scope(ctx, "maxpool_forward");
-#define SN_POOL_FWD(V, I) \
-  hipLaunchKernelGGL((maxpool_fwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl)
+  LaunchScope scope(ctx, avg ? "avgpool_forward" : "maxpool_forward");
+#define SN_POOL_FWD(V, I)                                                                                                              \
+  do {                                                                                                                                 \
+    if (avg) hipLaunchKernelGGL((pool_fwd_kernel<V, I, true>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl); \
+    else hipLaunchKernelGGL((pool_fwd_kernel<V, I, false>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl);    \
+  } while (0)
   if (v4 && small) SN_POOL_FWD(4, uint32_t);
   else if (v4) SN_POOL_FWD(4, uint64_t);
   else if (small) SN_POOL_FWD(1, uint32_t);
@@ -551,8 +565,10 @@ int launch_maxpool_fwd(sn_ctx* ctx, const float* x, float* y, uint8_t* arg, int 
 
 // Backward as a gather: each input element adds the gradients of the windows whose recorded
 // first maximum is this element (TF MaxPoolGradV2, math/nn/AllKernels.scala:305-324). No atomics.
-template <int V, typename I>
-__global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
+// AVG: every window that covers the element hands it its gradient times 1 / (the window's cells inside the input)
+// (TF AvgPoolGrad, math/nn/AllKernels.scala:355-381).
+template <int V, typename I, bool AVG>
+__global__ __launch_bounds__(256) void pool_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
                                                            float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo,
                                                            int kh, int kw, int sh, int sw, int pt, int pl,
                                                            const float* __restrict__ y_in, int act, float act_param) {
@@ -579,9 +595,23 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restric
     if (ow_hi > wo - 1) ow_hi = wo - 1;
     for (int oh = oh_lo; oh <= oh_hi; ++oh) {
       const int r = iy - (oh * sh - pt);
+      const int y0 = oh * sh - pt;
+      const int rows_in = (y0 + kh < h ? y0 + kh : h) - (y0 > 0 ? y0 : 0);
       for (int ow = ow_lo; ow <= ow_hi; ++ow) {
         const int q = ix - (ow * sw - pl);
         const I o = ((b * ho + oh) * wo + ow) * c + ch;
+        if constexpr (AVG) {
+          const int x0 = ow * sw - pl;
+          const int cols_in = (x0 + kw < w ? x0 + kw : w) - (x0 > 0 ? x0 : 0);
+          const float share = 1.0f / (float)(rows_in * cols_in);
+          if constexpr (V == 4) {
+            const float4 g = *(const float4*)(dy + o);
+            s[0] += g.x * share; s[1] += g.y * share; s[2] += g.z * share; s[3] += g.w * share;
+          } else {
+            s[0] += dy[o] * share;
+          }
+          continue;
+        }
         const uint32_t want = (uint32_t)(r * kw + q);
         if constexpr (V == 4) {
           const uint32_t a4 = *(const uint32_t*)(arg + o);
@@ -611,16 +641,23 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const float* __restric
   }
 }
 
-int launch_maxpool_bwd(sn_ctx* ctx, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho, int wo,
-                       int kh, int kw, int sh, int sw, int pt, int pl, const float* y_in, int act, float act_param) {
+int launch_pool_bwd(sn_ctx* ctx, bool avg, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho, int wo,
+                    int kh, int kw, int sh, int sw, int pt, int pl, const float* y_in, int act, float act_param) {
   const int64_t total = (int64_t)n * h * w * c;
   if (total <= 0) return SN_OK;
   const bool small = total < (1ll << 31) && (int64_t)n * ho * wo * c < (1ll << 31);
   const bool v4 = pool_vec4(dy, dx, arg, c) && (reinterpret_cast<uintptr_t>(y_in) & 15u) == 0;
   const dim3 grid(grid_for_xcd(ctx, v4 ? total / 4 : total, 256));
-  LaunchScope scope(ctx, y_in ? "maxpool_activation_backward" : "maxpool_backward");
-#define SN_POOL_BWD(V, I) \
-  hipLaunchKernelGGL((maxpool_bwd_kernel<V, I>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl, y_in, act, act_param)
+  LaunchScope scope(ctx, avg ? (y_in ? "avgpool_activation_backward" : "avgpool_backward") : (y_in ? "maxpool_activation_backward" : "maxpool_backward"));
+#define SN_POOL_BWD(V, I)                                                                                                     \
+  do {                                                                                                                        \
+    if (avg)                                                                                                                  \
+      hipLaunchKernelGGL((pool_bwd_kernel<V, I, true>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, \
+                         pt, pl, y_in, act, act_param);                                                                       \
+    else                                                                                                                      \
+      hipLaunchKernelGGL((pool_bwd_kernel<V, I, false>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, \
+                         pt, pl, y_in, act, act_param);                                                                       \
+  } while (0)
   if (v4 && small) SN_POOL_BWD(4, uint32_t);
   else if (v4) SN_POOL_BWD(4, uint64_t);
   else if (small) SN_POOL_BWD(1, uint32_t);

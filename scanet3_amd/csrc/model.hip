@@ -31,6 +31,7 @@ struct Op {
   float act_param = 0.f;
   // conv / pool geometry (per sample: h, w, c)
   int kh = 0, kw = 0, sh = 1, sw = 1, pt = 0, pl = 0;
+  bool pool_avg = false;  // Pool2D: mean of the window instead of its maximum
   // lstm
   int T = 0, F = 0, H = 0;
   bool ret_seq = false;  // the layer's output is every step's output, [T, H] per sample (layer/RNN.scala:74-77)
@@ -227,7 +228,9 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         SN_REQUIRE(L.kernel_h > 0 && L.kernel_w > 0 && L.stride_h > 0 && L.stride_w > 0 && L.kernel_h * L.kernel_w <= 255,
                    "layer %d: Pool2D needs a positive window (at most 255 cells) and strides", i);
         SN_REQUIRE(L.padding == SN_PAD_VALID || L.padding == SN_PAD_SAME, "layer %d: only [Same, Valid] paddings are supported", i);
+        SN_REQUIRE(L.pool_reduce == SN_POOL_MAX || L.pool_reduce == SN_POOL_AVG, "layer %d: unknown pooling reduction %d", i, L.pool_reduce);
         op.kind = OP_POOL;
+        op.pool_avg = L.pool_reduce == SN_POOL_AVG;
         op.kh = L.kernel_h; op.kw = L.kernel_w; op.sh = L.stride_h; op.sw = L.stride_w;
         int ho, wo;
         conv_out(L.padding, (int)cur[0], op.kh, op.sh, &ho, &op.pt);
@@ -440,7 +443,7 @@ static int alloc_replica(sn_replica* r) {
       SN_TRY(dev_alloc(r, &r->lstm_pk_dh[i], lstm_pack_elems(op.F, op.H) / 4));
       SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
     }
-    if (op.kind == OP_POOL) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
+    if (op.kind == OP_POOL && !op.pool_avg) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
     if (dense_bf16_fast(m, op)) {
       SN_TRY(dev_alloc(r, &r->bf_x[i], B * op.in_elems));
       SN_TRY(dev_alloc(r, &r->bf_xt[i], B * op.in_elems));
@@ -544,7 +547,7 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         break;
       }
       case OP_POOL:
-        SN_TRY(launch_maxpool_fwd(ctx, in, r->act[i], r->arg[i], rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
+        SN_TRY(launch_pool_fwd(ctx, op.pool_avg, in, r->act[i], r->arg[i], rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
                                   (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl));
         break;
       case OP_FLATTEN:
@@ -714,7 +717,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           // a convolution with an activation right below: its activation gradient rides along (one pass less over the tensor)
           const Op& below = m->ops[i - 1];
           const bool fuse = below.kind == OP_CONV && below.act != SN_ACT_IDENTITY;
-          SN_TRY(launch_maxpool_bwd(ctx, dy, r->arg[i], dx, rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
+          SN_TRY(launch_pool_bwd(ctx, op.pool_avg, dy, r->arg[i], dx, rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
                                     (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl,
                                     fuse ? r->act[i - 1] : nullptr, below.act, below.act_param));
           act_grad_done = fuse;

@@ -238,6 +238,7 @@ class Layer:
     momentum: float = 0.99        # BatchNorm only
     epsilon: float = 1e-3
     fused: int = -1               # BatchNorm `fused`: -1 None, 0 Some(false), 1 Some(true)
+    pool_reduce: int = 0          # Pool2D: L.POOL_MAX or L.POOL_AVG
 
     def __rshift__(self, other):
         return Composed.of(self, other)
@@ -250,7 +251,7 @@ class Layer:
         return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
                            self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
                            1 if self.return_sequence else 0, self.momentum, self.epsilon,
-                           self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused)
+                           self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused, self.pool_reduce)
 
     def __repr__(self):
         return self.text
@@ -312,10 +313,20 @@ def Conv2D(filters: int, kernel: Tuple[int, int] = (3, 3), strides: Tuple[int, i
                   Activate(activation) if not activation.identity else None)
 
 
-def Pool2D(window: Tuple[int, int] = (2, 2), strides: Tuple[int, int] = (1, 1), padding: int = Valid) -> Layer:
-    """layer/Pool2D.scala:28-42 (always max pooling)."""
-    return Layer(L.LAYER_POOL2D, f"Pool2D({tuple(window)},{tuple(strides)},{_PAD_NAME[padding]},NHWC,Max)".replace(" ", ""),
-                 kernel=tuple(window), strides=tuple(strides), padding=padding)
+ReduceMax, ReduceAvg = "Max", "Avg"
+
+
+def Pool2D(window: Tuple[int, int] = (2, 2), strides: Tuple[int, int] = (1, 1), padding: int = Valid, reduce: str = ReduceMax,
+           as_reference_layer: bool = True) -> Layer:
+    """layer/Pool2D.scala:28-42.  The reference's layer does not hand `reduce` to `pool2D` when it builds its graph
+    (:36-42), so a model with `reduce = Avg` max-pools there; `as_reference_layer=True` (the default) does the same.
+    With `as_reference_layer=False` the layer computes what the kernel function `pool2D(reduce = Avg)` computes
+    (math/nn/AllKernels.scala:326-397)."""
+    if reduce not in (ReduceMax, ReduceAvg):
+        raise ValueError(f"reduce should be Max or Avg, got {reduce!r}")
+    avg = reduce == ReduceAvg and not as_reference_layer
+    return Layer(L.LAYER_POOL2D, f"Pool2D({tuple(window)},{tuple(strides)},{_PAD_NAME[padding]},NHWC,{reduce})".replace(" ", ""),
+                 kernel=tuple(window), strides=tuple(strides), padding=padding, pool_reduce=L.POOL_AVG if avg else L.POOL_MAX)
 
 
 Flatten = Layer(L.LAYER_FLATTEN, "Flatten")

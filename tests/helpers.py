@@ -13,7 +13,7 @@ f32 = np.float32
 
 def build_pair(spec: List[tuple], loss: str):
     """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
-    | ("pool", window, strides, pad) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon) | ("activate", act) | ("bias", features)
+    | ("pool", window, strides, pad[, "avg"]) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon) | ("activate", act) | ("bias", features)
     Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
     import scanet3_amd as S
     acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
@@ -45,9 +45,13 @@ def build_pair(spec: List[tuple], loss: str):
                 ol.append(O.Conv2D(filters, kernel, strides, pads_o[pad], acts_o[act], bias=bias))
                 add(S.Conv2D(filters, kernel, strides, pads_s[pad], acts_s[act], bias=bias))
         elif k == "pool":
-            _, window, strides, pad = e
-            ol.append(O.Pool2D(window, strides, pads_o[pad]))
-            add(S.Pool2D(window, strides, pads_s[pad]))
+            _, window, strides, pad = e[:4]
+            if len(e) > 4 and e[4] == "avg":    # the kernel function's Reduce.Avg, not the reference layer's behaviour
+                ol.append(O.Pool2D(window, strides, pads_o[pad], reduce="Avg", as_reference_layer=False))
+                add(S.Pool2D(window, strides, pads_s[pad], reduce=S.ReduceAvg, as_reference_layer=False))
+            else:
+                ol.append(O.Pool2D(window, strides, pads_o[pad]))
+                add(S.Pool2D(window, strides, pads_s[pad]))
         elif k == "flatten":
             ol.append(O.Flatten())
             add(S.Flatten)

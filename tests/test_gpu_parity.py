@@ -266,6 +266,37 @@ def test_golden_conv_pool_gradients(S, ctx, golden):
     h.close()
 
 
+def test_golden_avg_pool(S, ctx, golden):
+    """math/nn/KernelsSpec.scala:212-223,290-305 (`pool2D(reduce = Avg)`, Same padding) through the library: the forward
+    values, and the input gradient of sum(pool) read through a 1x1 convolution in front (its weight gradient is
+    sum(x * d pool input))."""
+    img = A(golden["image_5x5"]).reshape(1, 5, 5, 1)
+    x = ctx.to_device(img)
+    h = Harness(S, ctx, [("conv", 1, (1, 1), (1, 1), "valid", "identity", False), ("pool", (2, 2), (1, 1), "same", "avg")],
+                "mse", (5, 5, 1), 1)
+    h.rep.set_params({"0/weights": np.ones((1, 1, 1, 1), f32)})
+    out = h.rep.forward(x)
+    np.testing.assert_array_equal(out.reshape(5, 5), A(golden["avg_pool_2x2"]["same_s1"]))
+    y = ctx.to_device(out - f32(out.size / 2.0))
+    h.rep.grad(x, y)
+    share = A(golden["avg_pool_2x2"]["same_s1_grad_input_of_sum"])
+    np.testing.assert_allclose(h.rep.get_grads()["0/weights"].ravel()[0], float((img.reshape(5, 5) * share).sum()), rtol=1e-6)
+    h.close()
+
+
+def test_pool2d_layer_ignores_reduce_like_the_reference(S, ctx, golden):
+    """layer/Pool2D.scala:36-42 builds `pool2D` without `reduce`: a layer declared with Avg max-pools.  The mirror does
+    the same unless told to follow the kernel function instead."""
+    x = ctx.to_device(A(golden["image_5x5"]).reshape(1, 5, 5, 1))
+    for layer, key in ((S.Pool2D(padding=S.Same, reduce=S.ReduceAvg), "max_pool_2x2"),
+                       (S.Pool2D(padding=S.Same, reduce=S.ReduceAvg, as_reference_layer=False), "avg_pool_2x2")):
+        cm = S.CompiledModel(ctx, [layer.desc()], S.MeanSquaredError.kind, (5, 5, 1), 1, 0)
+        rep = cm.replica(None)
+        np.testing.assert_array_equal(rep.forward(x).reshape(5, 5), A(golden[key]["same_s1"]))
+        rep.close()
+        cm.close()
+
+
 def test_golden_lstm_forward(S, ctx, golden):
     g = golden["lstm"]
     h = Harness(S, ctx, [("lstm", 2)], "mse", (3, 1), 1)
@@ -338,6 +369,13 @@ MODELS = {
                      ("flatten",), ("dense", 10, "softmax")], "cce", (12, 12, 1), 20, "uniform_onehot"),
     "cnn_same_stride2_bias": ([("conv", 5, (3, 2), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "same"),
                                ("activate", "relu"), ("flatten",), ("dense", 4, "softmax")], "cce", (9, 10, 3), 7, "uniform_onehot"),
+    # kernel-level average pooling (math/nn/AllKernels.scala:326-381): one channel count that takes the 4-wide kernels, one that
+    # does not; Same padding makes edge windows smaller
+    "cnn_avg_pool": ([("conv", 8, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "same", "avg"),
+                      ("conv", 3, (2, 2), (1, 1), "same", "tanh", True), ("pool", (3, 2), (1, 2), "same", "avg"), ("flatten",),
+                      ("dense", 4, "softmax")], "cce", (9, 8, 2), 13, "uniform_onehot"),
+    "cnn_avg_pool_valid": ([("conv", 4, (2, 2), (1, 1), "valid", "sigmoid", True), ("pool", (2, 2), (1, 1), "valid", "avg"), ("flatten",),
+                            ("dense", 2, "identity")], "mse", (6, 6, 1), 10, "normal_regression"),
     "cnn_explicit_padding": ([("conv", 6, (3, 2), (2, 1), (1, 0, 2, 1), "tanh", True), ("conv", 4, (2, 2), (1, 1), (0, 1, 0, 0), "relu", False),
                               ("flatten",), ("dense", 3, "softmax")], "cce", (7, 6, 2), 11, "uniform_onehot"),
     "lstm_small": ([("lstm", 24), ("dense", 1, "tanh")], "mse", (9, 5), 33, "normal_regression"),

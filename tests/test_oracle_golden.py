@@ -66,6 +66,15 @@ def test_max_pool_grad_ties_golden(golden):
     np.testing.assert_array_equal(g.reshape(5, 5), A(golden["max_pool_2x2"]["same_s1_grad_input_of_sum"], np.float64))
 
 
+def test_avg_pool_golden(golden):
+    """Kernel-level `pool2D(reduce = Avg)` with Same padding: windows at the bottom / right edge average fewer cells."""
+    x = A(golden["image_5x5"], np.float64).reshape(1, 5, 5, 1)
+    out = O.avg_pool(x, (2, 2), (1, 1), O.PAD_SAME)
+    np.testing.assert_array_equal(out.reshape(5, 5), A(golden["avg_pool_2x2"]["same_s1"], np.float64))
+    g = O.avg_pool_grad(x.shape, np.ones((1, 5, 5, 1)), (2, 2), (1, 1), O.PAD_SAME)
+    np.testing.assert_array_equal(g.reshape(5, 5), A(golden["avg_pool_2x2"]["same_s1_grad_input_of_sum"], np.float64))
+
+
 # ----------------------------------------------------------------- brute force + torch
 def _brute_conv(x, w, strides, padding):
     n, h, wd, c = x.shape
@@ -131,6 +140,37 @@ def test_max_pool_brute_first_max(strides, padding):
         dx[b, at[0], at[1], ch] += dy[b, i, j, ch]
     np.testing.assert_array_equal(O.max_pool(x, (2, 2), strides, padding), out)
     np.testing.assert_allclose(O.max_pool_grad(x, dy, (2, 2), strides, padding), dx, rtol=0, atol=1e-15)
+
+
+@pytest.mark.parametrize("window,strides", [((2, 2), (1, 1)), ((2, 2), (2, 2)), ((3, 2), (2, 1))])
+@pytest.mark.parametrize("padding", [O.PAD_VALID, O.PAD_SAME])
+def test_avg_pool_brute_and_torch(window, strides, padding):
+    """Cell-by-cell mean over the in-bounds part of each window, its transpose as the gradient, and (where torch's
+    padding can express TF's) torch's avg_pool2d with count_include_pad=False."""
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((2, 6, 5, 3))
+    kh, kw = window
+    n, h, wd, c = x.shape
+    ho, wo = O.out_size(padding, h, kh, strides[0]), O.out_size(padding, wd, kw, strides[1])
+    pt, _ = O.pads_for(padding, h, kh, strides[0])
+    pl, _ = O.pads_for(padding, wd, kw, strides[1])
+    dy = rng.standard_normal((n, ho, wo, c))
+    out = np.zeros((n, ho, wo, c))
+    dx = np.zeros_like(x)
+    for b, i, j, ch in itertools.product(range(n), range(ho), range(wo), range(c)):
+        cells = [(i * strides[0] + r - pt, j * strides[1] + q - pl) for r, q in itertools.product(range(kh), range(kw))]
+        cells = [(y, xx) for y, xx in cells if 0 <= y < h and 0 <= xx < wd]
+        out[b, i, j, ch] = sum(x[b, y, xx, ch] for y, xx in cells) / len(cells)
+        for y, xx in cells:
+            dx[b, y, xx, ch] += dy[b, i, j, ch] / len(cells)
+    np.testing.assert_allclose(O.avg_pool(x, window, strides, padding), out, rtol=1e-13, atol=1e-13)
+    np.testing.assert_allclose(O.avg_pool_grad(x.shape, dy, window, strides, padding), dx, rtol=1e-13, atol=1e-13)
+    if padding == O.PAD_VALID:
+        xt = torch.tensor(x.transpose(0, 3, 1, 2), requires_grad=True)
+        yt = torch.nn.functional.avg_pool2d(xt, window, strides, count_include_pad=False)
+        np.testing.assert_allclose(yt.detach().numpy().transpose(0, 2, 3, 1), out, rtol=1e-12, atol=1e-12)
+        yt.backward(torch.tensor(dy.transpose(0, 3, 1, 2)))
+        np.testing.assert_allclose(xt.grad.numpy().transpose(0, 2, 3, 1), dx, rtol=1e-12, atol=1e-12)
 
 
 # ----------------------------------------------------------------- layer goldens
