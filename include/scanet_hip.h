@@ -104,9 +104,13 @@ typedef struct sn_layer_desc {
   float bn_epsilon;      /* BATCHNORM: added to the variance */
   int32_t pad_top, pad_bottom, pad_left, pad_right; /* CONV2D with SN_PAD_EXPLICIT: `Explicit((top, bottom), (left, right))`,
                             output size ceil((in + pads - window) / stride) + 1 (math/nn/AllKernels.scala:67-91) */
-  int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  Only the generic
-                            form (math/nn/AllKernels.scala:663-684) is built: whenever the reference would take
-                            FusedBatchNormV3 (rank-4 input unless fused = Some(false)) model creation fails. */
+  int32_t bn_fused;      /* BATCHNORM: `fused` of the reference: -1 None, 0 Some(false), 1 Some(true).  As in the reference
+                            (layer/BatchNorm.scala:98-133) rank-4 input takes the FusedBatchNormV3 branch unless fused =
+                            Some(false), every other rank the generic form (math/nn/AllKernels.scala:663-684), and
+                            Some(true) with another rank fails.  The fused branch is built AS THE REFERENCE WIRES THE
+                            OP'S OUTPUTS (math/nn/AllKernels.scala:437-448): same output as the generic form, but the
+                            moving variance follows the batch mean and the gradient op receives the unbiased batch
+                            variance as its mean and the batch mean as its variance. */
   int32_t pool_reduce;   /* POOL2D: SN_POOL_*.  AVG divides by the number of window cells inside the input (TF AvgPool) */
 } sn_layer_desc;
 

@@ -22,15 +22,20 @@ What pins each part (see tests/test_oracle_golden.py):
   * BatchNorm (generic form): training output, next moving
     statistics, frozen output ................................... reference goldens
   * BatchNorm backward through the batch statistics .............. float64 numerical gradients (rank 2 and rank 4)
+  * FusedBatchNormV3 / GradV3 as TensorFlow defines them .......... the generic form's goldens (same y), numpy's unbiased
+    variance, float64 numerical gradients when handed the true statistics
   * decayingAvg / boost / sqrtZeroSafe ........................... reference goldens
   * optimizer trajectories ....................................... reference convergence thresholds + closed forms
 Parity unpinned (only running TensorFlow-CPU could pin them): last-ulp
 behaviour of TF's Exp/Tanh/Sigmoid/Log/Pow, summation order inside TF's
 MatMul/Conv2D/Sum, averaging of more than one replica and the multi-partition
 iteration counter (no reference test runs with more than one partition), and
-the FusedBatchNormV3 form BatchNorm takes for rank-4 input unless `fused =
-Some(false)` (not restated: its saved-statistics outputs are wired by index in
-math/nn/AllKernels.scala:443-452 and no reference test holds values for it).
+the WIRING of the FusedBatchNormV3 branch BatchNorm takes for rank-4 input
+unless `fused = Some(false)` (`batchnorm_fused_forward/backward`): which of
+the op's outputs reach the moving statistics and the gradient op is read off
+math/nn/AllKernels.scala:437-448, and what TensorFlow's CPU kernel puts into
+those outputs is restated from its published source (TF 2.10,
+core/kernels/fused_batch_norm_op.cc); no reference test holds values for it.
 """
 from __future__ import annotations
 
@@ -413,6 +418,7 @@ class Layer:
     return_sequence: bool = False   # lstm / simple_rnn: every step's output, (batch, time, units) (RNN.scala:27,75-77)
     momentum: float = 0.99          # batchnorm (BatchNorm.scala:66-67)
     epsilon: float = 1e-3
+    fused: bool = False             # batchnorm: the FusedBatchNormV3 branch as the reference wires it (rank-4 input)
     pool_avg: bool = False          # pool2d: mean of the window (kernel-level `Reduce.Avg`) instead of its maximum
 
     # ---- parameter definitions, in flat-buffer order ---------------------- #
@@ -505,11 +511,12 @@ BN_PARAMS = ("beta", "gamma", "moving_mean", "moving_variance")   # BatchNorm.sc
 BN_STATE = ("moving_mean", "moving_variance")                      # not trainable: replaced by the layer, not by the optimizer
 
 
-def BatchNorm(momentum=0.99, epsilon=1e-3):
-    """`BatchNorm(axes = Seq(-1), fused = Some(false))` (BatchNorm.scala:64-76): the generic `batchNorm` form
-    (math/nn/AllKernels.scala:663-684).  The FusedBatchNormV3 form the layer picks for rank-4 input by default is
-    not restated here."""
-    return [Layer("batchnorm", momentum=momentum, epsilon=epsilon)]
+def BatchNorm(momentum=0.99, epsilon=1e-3, fused=False):
+    """`BatchNorm(axes = Seq(-1))` (BatchNorm.scala:64-76).  fused=False: the generic `batchNorm` form
+    (math/nn/AllKernels.scala:663-684), which the layer takes for `fused = Some(false)` and for any input that is not
+    rank 4.  fused=True: the FusedBatchNormV3 branch it takes for rank-4 input otherwise, wired as the reference
+    wires it (`batchnorm_fused_forward`)."""
+    return [Layer("batchnorm", momentum=momentum, epsilon=epsilon, fused=fused)]
 
 
 def is_state_path(path: str) -> bool:
@@ -559,6 +566,83 @@ def batchnorm_backward(dy, cache, pre, grads):
         return dy * inv
     n = dt.type(np.prod([x.shape[a] for a in axes]))
     return inv * (dy - s1 / n - xc * (r * r * s2 / n))
+
+
+# ---- the FusedBatchNormV3 form (rank-4 input unless `fused = Some(false)`, BatchNorm.scala:98-130) ------------------ #
+def fused_batch_norm(x, scale, offset, mean_in, var_in, eps, training):
+    """The six outputs of TensorFlow's `FusedBatchNormV3` on the CPU, NHWC, exponential_avg_factor = 1 (the op the
+    reference builds at nn/AllKernels.scala:399-421): (y, batch_mean, batch_variance, reserve_space_1,
+    reserve_space_2, reserve_space_3).
+
+    training: batch_mean = mean over all axes but the last; y = (x - mean) * (rsqrt(var + eps) * scale) + offset with
+    the biased variance; `batch_variance` (the value meant for the running average) is the UNBIASED variance
+    var * n / max(n - 1, 1); reserve_space_1 / 2 keep the mean and the biased variance for the gradient.
+    inference: the given population statistics everywhere."""
+    dt = x.dtype
+    c = x.shape[-1]
+    x2 = x.reshape(-1, c)
+    n = x2.shape[0]
+    scale, offset = scale.reshape(c), offset.reshape(c)
+    if training:
+        mean = x2.sum(axis=0, dtype=dt) / dt.type(n)
+        xc = x2 - mean
+        var = (xc * xc).sum(axis=0, dtype=dt) / dt.type(n)
+        y = xc * ((dt.type(1.0) / np.sqrt(var + dt.type(eps))) * scale) + offset
+        unbiased = var * (dt.type(n) / dt.type(max(n - 1, 1)))
+        return y.reshape(x.shape), mean, unbiased, mean, var, np.zeros(0, dt)
+    mean, var = mean_in.reshape(c), var_in.reshape(c)
+    y = (x2 - mean) * ((dt.type(1.0) / np.sqrt(var + dt.type(eps))) * scale) + offset
+    return y.reshape(x.shape), mean, var, mean, var, np.zeros(0, dt)
+
+
+def fused_batch_norm_grad(dy, x, scale, reserve_1, reserve_2, eps):
+    """`FusedBatchNormGradV3` on the CPU with is_training = true (nn/AllKernels.scala:503-531): it takes reserve_1 as
+    the batch mean m and reserve_2 as the batch variance v and returns
+        dx      = scale * rsqrt(v + eps) * (dy - mean(dy) - (x - m) * mean(dy * (x - m)) / (v + eps))
+        dscale  = sum(dy * (x - m) * rsqrt(v + eps))
+        doffset = sum(dy)."""
+    dt = dy.dtype
+    c = x.shape[-1]
+    x2, dy2 = x.reshape(-1, c), dy.reshape(-1, c)
+    n = dt.type(x2.shape[0])
+    m, v, scale = reserve_1.reshape(c), reserve_2.reshape(c), scale.reshape(c)
+    r = dt.type(1.0) / np.sqrt(v + dt.type(eps))
+    xc = x2 - m
+    s1 = dy2.sum(axis=0, dtype=dt)
+    s2 = (dy2 * xc).sum(axis=0, dtype=dt)
+    dx = (scale * r) * (dy2 - s1 / n - xc * (r * r * s2 / n))
+    return dx.reshape(x.shape), s2 * r, s1
+
+
+def batchnorm_fused_forward(x, params, pre, l: Layer, training: bool):
+    """The layer's fused branch AS THE REFERENCE WIRES IT (BatchNorm.scala:117-130, nn/AllKernels.scala:437-448):
+    `outputs` takes TF output 1 for batchMean AND for batchVariance, output 2 for reserveSpace1, 3 for reserveSpace2
+    and 4 for reserveSpace3.  So the moving variance follows the batch MEAN, and the gradient op receives the
+    unbiased batch variance where it expects the mean and the batch mean where it expects the variance.
+    Returns (y, cache, next_state)."""
+    dt = x.dtype
+    outs = fused_batch_norm(x, params[pre + "gamma"], params[pre + "beta"], params[pre + "moving_mean"],
+                            params[pre + "moving_variance"], l.epsilon, training)
+    y = outs[0]
+    batch_mean, batch_variance = outs[1], outs[1]
+    reserve_1, reserve_2 = outs[2], outs[3]
+    nxt = {}
+    if training:
+        mom = dt.type(l.momentum)
+        shape = params[pre + "moving_mean"].shape
+        nxt[pre + "moving_mean"] = mom * params[pre + "moving_mean"] + (dt.type(1.0) - mom) * batch_mean.reshape(shape)
+        nxt[pre + "moving_variance"] = mom * params[pre + "moving_variance"] + (dt.type(1.0) - mom) * batch_variance.reshape(shape)
+    return y, (x, reserve_1, reserve_2, params[pre + "gamma"], l.epsilon, training), nxt
+
+
+def batchnorm_fused_backward(dy, cache, pre, grads):
+    x, reserve_1, reserve_2, gamma, eps, training = cache
+    if not training:
+        raise NotImplementedError("the gradient of the frozen fused form is not on the training path")
+    dx, dscale, doffset = fused_batch_norm_grad(dy, x, gamma, reserve_1, reserve_2, eps)
+    grads[pre + "gamma"] = dscale.reshape(gamma.shape)
+    grads[pre + "beta"] = doffset.reshape(gamma.shape)
+    return dx
 
 
 class Model:
@@ -624,7 +708,7 @@ class Model:
             elif k == "simple_rnn":
                 y, c = simple_rnn_forward(x, params, pre, l)
             elif k == "batchnorm":
-                y, c, nxt = batchnorm_forward(x, params, pre, l, training)
+                y, c, nxt = (batchnorm_fused_forward if l.fused else batchnorm_forward)(x, params, pre, l, training)
                 if next_state is not None:
                     next_state.update(nxt)
             else:
@@ -694,7 +778,7 @@ class Model:
             elif k == "simple_rnn":
                 dy = simple_rnn_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
             elif k == "batchnorm":
-                dy = batchnorm_backward(dy, c, pre, grads)
+                dy = (batchnorm_fused_backward if l.fused else batchnorm_backward)(dy, c, pre, grads)
             if l.kind in ("dense", "bias") and l.reg != REG_NONE:
                 w = params[pre + "weights"]
                 lam = w.dtype.type(l.reg_lambda)

@@ -177,7 +177,8 @@ __global__ __launch_bounds__(256) void bn_scale_kernel(const float* __restrict__
 template <bool V4>
 __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__ x, const float* __restrict__ mean,
                                                         const float* __restrict__ inv, const float* __restrict__ beta,
-                                                        float* __restrict__ y, int64_t n, int cols) {
+                                                        float* __restrict__ y, int64_t n, int cols, int centred) {
+  // generic form: (x*inv - mean*inv) + beta (math/nn/AllKernels.scala:676-683); the fused op: (x - mean)*inv + beta
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   if (V4) {
     const int64_t n4 = n / 4;
@@ -186,15 +187,28 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__
       const bn_f4 xv = *(const bn_f4*)(x + i * 4), iv = *(const bn_f4*)(inv + c), mv = *(const bn_f4*)(mean + c), bv = *(const bn_f4*)(beta + c);
       bn_f4 o;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = (xv[e] * iv[e] - mv[e] * iv[e]) + bv[e];
+      for (int e = 0; e < 4; ++e) o[e] = centred ? (xv[e] - mv[e]) * iv[e] + bv[e] : (xv[e] * iv[e] - mv[e] * iv[e]) + bv[e];
       *(bn_f4*)(y + i * 4) = o;
     }
   } else {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
       const int c = (int)(i % cols);
-      y[i] = (x[i] * inv[c] - mean[c] * inv[c]) + beta[c];
+      y[i] = centred ? (x[i] - mean[c]) * inv[c] + beta[c] : (x[i] * inv[c] - mean[c] * inv[c]) + beta[c];
     }
   }
+}
+
+// The statistics the reference's wiring hands to the fused gradient op: "mean" = the unbiased variance, "variance" = the mean.
+__global__ __launch_bounds__(256) void bn_fused_wiring_kernel(const float* __restrict__ mean, const float* __restrict__ var,
+                                                               const float* __restrict__ gamma, float unbias, float eps,
+                                                               float* __restrict__ g_mean, float* __restrict__ g_r,
+                                                               float* __restrict__ g_inv, int cols) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  g_mean[c] = var[c] * unbias;
+  const float rr = 1.0f / sqrtf(mean[c] + eps);   // NaN for a channel whose mean is below -epsilon, as in the reference
+  g_r[c] = rr;
+  g_inv[c] = rr * gamma[c];
 }
 
 // d beta = S1, d gamma = S2 * r; k1 = S1/n, k2 = r*r*S2/n for the input gradient
@@ -343,6 +357,12 @@ int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, in
       hipLaunchKernelGGL(bn_scale_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, s, cols, (float)rows, a.epsilon, a.gamma,
                          (const float*)nullptr, (const float*)nullptr, a.mean, a.var, a.r, a.inv);
     }
+    if (a.fused_wiring) {
+      LaunchScope scope(ctx, "batchnorm_fused_wiring");
+      const float unbias = (float)rows / (float)(rows > 1 ? rows - 1 : 1);
+      hipLaunchKernelGGL(bn_fused_wiring_kernel, dim3((unsigned)ceil_div((int64_t)cols, (int64_t)256)), dim3(256), 0, ctx->stream,
+                         (const float*)a.mean, (const float*)a.var, a.gamma, unbias, a.epsilon, a.g_mean, a.g_r, a.g_inv, cols);
+    }
   } else {
     LaunchScope scope(ctx, "batchnorm_frozen_scale");
     hipLaunchKernelGGL(bn_scale_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)nullptr, 0, cols, 1.0f, a.epsilon, a.gamma,
@@ -352,10 +372,10 @@ int launch_batchnorm_fwd(sn_ctx* ctx, const float* x, float* y, int64_t rows, in
   LaunchScope scope(ctx, "batchnorm_apply");
   if (vec4_ok(cols, {x, y, a.mean, a.inv, a.beta}))
     hipLaunchKernelGGL((bn_apply_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, (const float*)a.mean,
-                       (const float*)a.inv, a.beta, y, n, cols);
+                       (const float*)a.inv, a.beta, y, n, cols, a.fused_wiring ? 1 : 0);
   else
     hipLaunchKernelGGL((bn_apply_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, (const float*)a.mean,
-                       (const float*)a.inv, a.beta, y, n, cols);
+                       (const float*)a.inv, a.beta, y, n, cols, a.fused_wiring ? 1 : 0);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
@@ -367,22 +387,25 @@ int launch_batchnorm_bwd(sn_ctx* ctx, const float* x, const float* dy, float* dx
   SN_REQUIRE(2 * half <= ws_elems, "batch norm gradient needs %lld workspace elements, %lld given", (long long)(2 * half), (long long)ws_elems);
   const int cb = (int)ceil_div((int64_t)cols, (int64_t)16);  // finishing kernels: 16 channels per block
   float* part1 = ws + half;
+  const float* mean = a.fused_wiring ? a.g_mean : a.mean;
+  const float* r = a.fused_wiring ? a.g_r : a.r;
+  const float* inv = a.fused_wiring ? a.g_inv : a.inv;
   {
     LaunchScope scope(ctx, "batchnorm_gradient_sums");
     int s = 0;
-    SN_TRY(reduce_pass<BN_GRAD>(ctx, x, dy, a.mean, ws, half, rows, cols, &s));
+    SN_TRY(reduce_pass<BN_GRAD>(ctx, x, dy, mean, ws, half, rows, cols, &s));
     hipLaunchKernelGGL(bn_grad_finish_kernel, dim3(cb), dim3(256), 0, ctx->stream, (const float*)ws, (const float*)part1, s, cols,
-                       (float)rows, (const float*)a.r, dbeta, dgamma, a.k1, a.k2);
+                       (float)rows, r, dbeta, dgamma, a.k1, a.k2);
   }
   if (dx) {
     const int64_t n = rows * cols;
     LaunchScope scope(ctx, "batchnorm_input_gradient");
-    if (vec4_ok(cols, {x, dy, dx, a.mean, a.inv, a.k1, a.k2}))
-      hipLaunchKernelGGL((bn_dx_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
-                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
+    if (vec4_ok(cols, {x, dy, dx, mean, inv, a.k1, a.k2}))
+      hipLaunchKernelGGL((bn_dx_kernel<true>), dim3(grid_for(ctx, n / 4, 1024)), dim3(256), 0, ctx->stream, x, dy, mean, inv,
+                         (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
     else
-      hipLaunchKernelGGL((bn_dx_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, dy, (const float*)a.mean,
-                         (const float*)a.inv, (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
+      hipLaunchKernelGGL((bn_dx_kernel<false>), dim3(grid_for(ctx, n, 1024)), dim3(256), 0, ctx->stream, x, dy, mean, inv,
+                         (const float*)a.k1, (const float*)a.k2, dx, n, cols, below_act, below_act_param);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
@@ -392,7 +415,7 @@ int launch_batchnorm_moving(sn_ctx* ctx, const BatchNormArgs& a, float* moving_m
   if (cols <= 0) return SN_OK;
   LaunchScope scope(ctx, "batchnorm_moving_statistics");
   hipLaunchKernelGGL(bn_moving_kernel, dim3((unsigned)ceil_div((int64_t)cols, (int64_t)256)), dim3(256), 0, ctx->stream, moving_mean,
-                     moving_var, (const float*)a.mean, (const float*)a.var, cols, a.momentum);
+                     moving_var, (const float*)a.mean, (const float*)(a.fused_wiring ? a.mean : a.var), cols, a.momentum);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

@@ -185,6 +185,13 @@ struct BatchNormArgs {
   float* k1;                 // [C] scratch of the gradient
   float* k2;
   float epsilon, momentum;
+  // The FusedBatchNormV3 branch as the reference wires the op's outputs (math/nn/AllKernels.scala:437-448): the
+  // gradient op is handed the unbiased batch variance where it expects the mean and the batch mean where it expects
+  // the variance, and the moving variance follows the batch mean.  g_* hold those substituted statistics.
+  bool fused_wiring = false;
+  float* g_mean = nullptr;   // [C] var * n / max(n - 1, 1)
+  float* g_r = nullptr;      // 1/sqrt(mean + epsilon)
+  float* g_inv = nullptr;    // g_r * gamma
 };
 // workspace (elements) the reductions need for a [rows, cols] activation
 int64_t batchnorm_workspace_elems(const sn_ctx* ctx, int64_t rows, int cols);

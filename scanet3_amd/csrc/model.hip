@@ -39,6 +39,7 @@ struct Op {
   // batch norm: beta, gamma, moving mean, moving variance
   int bn_p[4] = {-1, -1, -1, -1};
   float bn_momentum = 0.99f, bn_epsilon = 1e-3f;
+  bool bn_fused = false;  // the FusedBatchNormV3 branch (rank-4 input unless fused = Some(false)), wired as the reference wires it
   // buffers (indices into replica buffer table), assigned at replica creation
   int out_buf = -1;
 };
@@ -298,12 +299,12 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         break;
       }
       case SN_LAYER_BATCHNORM: {
-        // BatchNorm(axes = Seq(-1)) in its generic form (layer/BatchNorm.scala:123-143, math/nn/AllKernels.scala:663-684)
+        // BatchNorm(axes = Seq(-1)): the generic form (layer/BatchNorm.scala:123-143, math/nn/AllKernels.scala:663-684), or for
+        // NHWC input unless fused = Some(false) the FusedBatchNormV3 branch (BatchNorm.scala:100-107,116-130)
         SN_REQUIRE(cur.size() >= 1, "layer %d: rank should be >= 2", i);
         SN_REQUIRE(L.bn_fused >= -1 && L.bn_fused <= 1, "layer %d: fused must be -1 (None), 0 or 1", i);
-        const bool wants_fused = cur.size() == 3 && L.bn_fused != 0;  // BatchNorm.scala:100-107,118-121
-        SN_REQUIRE(!wants_fused, "layer %d: the FusedBatchNormV3 form of BatchNorm is not built; pass fused = Some(false)", i);
-        SN_REQUIRE(L.bn_fused != 1, "layer %d: Cannot use fused implementation with this input rank", i);  // BatchNorm.scala:134-136
+        op.bn_fused = cur.size() == 3 && L.bn_fused != 0;
+        SN_REQUIRE(op.bn_fused || L.bn_fused != 1, "layer %d: Cannot use fused implementation with this input rank", i);  // BatchNorm.scala:131-133
         SN_REQUIRE(L.bn_epsilon > 0.f, "layer %d: epsilon must be positive", i);
         op.kind = OP_BATCHNORM;
         op.bn_momentum = L.bn_momentum;
@@ -434,7 +435,7 @@ static int alloc_replica(sn_replica* r) {
       continue;  // output = last slice of lstm_h unless the whole sequence is returned
     }
     SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
-    if (op.kind == OP_BATCHNORM) SN_TRY(dev_alloc(r, &r->bn_buf[i], 6 * align_up(op.out_dims.back(), 64)));
+    if (op.kind == OP_BATCHNORM) SN_TRY(dev_alloc(r, &r->bn_buf[i], 9 * align_up(op.out_dims.back(), 64)));
     if (op.kind == OP_SRNN) {  // the carried state of every step and its gradient, time-major like the LSTM's
       const int64_t bh = B * op.H;
       SN_TRY(dev_alloc(r, &r->lstm_h[i], (int64_t)(op.T + 1) * bh));  // slice 0 = zeros = the initial state
@@ -492,7 +493,8 @@ static BatchNormArgs batchnorm_args(sn_replica* r, const Op& op, int i) {
   const int64_t c = align_up(op.out_dims.back(), 64);
   float* b = r->bn_buf[i];
   return BatchNormArgs{param_ptr(r, r->w, op.bn_p[1]), param_ptr(r, r->w, op.bn_p[0]), param_ptr(r, r->w, op.bn_p[2]),
-                       param_ptr(r, r->w, op.bn_p[3]), b, b + c, b + 2 * c, b + 3 * c, b + 4 * c, b + 5 * c, op.bn_epsilon, op.bn_momentum};
+                       param_ptr(r, r->w, op.bn_p[3]), b, b + c, b + 2 * c, b + 3 * c, b + 4 * c, b + 5 * c, op.bn_epsilon, op.bn_momentum,
+                       op.bn_fused, b + 6 * c, b + 7 * c, b + 8 * c};
 }
 
 // skip_last: leave out the last op (the training pass fuses a Softmax output into the loss kernel)

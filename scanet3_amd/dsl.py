@@ -344,8 +344,9 @@ def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotU
 def BatchNorm(axes: Sequence[int] = (-1,), momentum: float = 0.99, epsilon: float = 1e-3, betaInitializer: Initializer = Zeros,
               gammaInitializer: Initializer = Ones, movingMeanInitializer: Initializer = Zeros,
               movingVarianceInitializer: Initializer = Ones, fused: Optional[bool] = None) -> Layer:
-    """layer/BatchNorm.scala:64-76 over the last axis.  Only the generic form is built: for rank-4 input the
-    reference picks FusedBatchNormV3 unless `fused=False`, and the library refuses that case."""
+    """layer/BatchNorm.scala:64-76 over the last axis.  As in the reference, rank-4 input takes the FusedBatchNormV3
+    branch unless `fused=False` (wired as the reference wires that op's outputs, which is not the generic form's
+    gradient nor its moving variance); every other rank takes the generic form."""
     if tuple(axes) != (-1,):
         raise ValueError("only axes = Seq(-1) is built")
     return Layer(L.LAYER_BATCHNORM, f"BatchNorm({list(axes)})", momentum=momentum, epsilon=epsilon,

@@ -13,7 +13,7 @@ f32 = np.float32
 
 def build_pair(spec: List[tuple], loss: str):
     """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
-    | ("pool", window, strides, pad[, "avg"]) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon) | ("activate", act) | ("bias", features)
+    | ("pool", window, strides, pad[, "avg"]) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon[, "fused"]) | ("activate", act) | ("bias", features)
     Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
     import scanet3_amd as S
     acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
@@ -66,9 +66,10 @@ def build_pair(spec: List[tuple], loss: str):
             seq = e[4] if len(e) > 4 else False
             ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias, return_sequence=seq))
             add(S.SimpleRNN(e[1], acts_s[act], bias=bias, returnSequence=seq))
-        elif k == "batchnorm":   # ("batchnorm", momentum, epsilon): the generic form (fused = Some(false))
-            ol.append(O.BatchNorm(e[1], e[2]))
-            add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=False))
+        elif k == "batchnorm":   # ("batchnorm", momentum, epsilon[, "fused"]): the generic form (fused = Some(false)) unless asked
+            fused = len(e) > 3 and e[3] == "fused"   # rank-4 input only: the layer's default there (fused = None)
+            ol.append(O.BatchNorm(e[1], e[2], fused=fused))
+            add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=None if fused else False))
         elif k == "activate":
             ol.append([O.Layer("activate", activation=acts_o[e[1]])])
             add(S.Activate(acts_s[e[1]]))

@@ -401,6 +401,13 @@ MODELS = {
     "cnn_batchnorm_32_channels": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3),
                                    ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 10, "softmax")],
                                   "cce", (14, 14, 1), 50, "uniform_onehot"),
+    # the layer's default for images: the FusedBatchNormV3 branch as the reference wires it (moving variance <- batch mean,
+    # gradient op fed the unbiased variance and the mean).  Channel means stay >= 0 behind a ReLU, so mean + epsilon has a root.
+    "cnn_batchnorm_fused": ([("conv", 8, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3, "fused"), ("pool", (2, 2), (2, 2), "valid"),
+                             ("conv", 6, (3, 3), (1, 1), "same", "relu", True), ("batchnorm", 0.9, 1e-3, "fused"), ("flatten",), ("dense", 5, "softmax")],
+                            "cce", (12, 12, 2), 24, "uniform_onehot"),
+    "batchnorm_fused_first": ([("batchnorm", 0.5, 1e-2, "fused"), ("conv", 3, (2, 2), (1, 1), "valid", "tanh", True), ("flatten",), ("dense", 2, "identity")],
+                              "mse", (5, 4, 3), 9, "uniform_binary"),     # inputs in [0, 1): positive channel means
     # tens of thousands of output positions over 4 input channels: padding, bias, strides, channel counts that are
     # multiples of 4 but not of 16
     "conv_many_positions_same_bias": ([("conv", 8, (3, 3), (1, 1), "same", "tanh", True), ("flatten",), ("dense", 3, "softmax")],
@@ -461,7 +468,7 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
 
 
 @pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
-                                        ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("mlp_bce_l2", 25)])
+                                        ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("cnn_batchnorm_fused", 12), ("mlp_bce_l2", 25)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
 def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
     spec, loss, in_shape, batch, kind = MODELS[name]
@@ -870,9 +877,6 @@ def test_error_paths(S, ctx):
         S.CompiledModel(ctx, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3, 3, 1), 8)
     with pytest.raises(S.ScanetError):                      # kernel larger than the input
         S.CompiledModel(ctx, [S.Conv2D(2, (5, 5)).desc()], S.MeanSquaredError.kind, (3, 3, 1), 8)
-    for fused in (None, True):                              # rank 4: the reference would take FusedBatchNormV3, which is not built
-        with pytest.raises(S.ScanetError, match="FusedBatchNormV3"):
-            S.CompiledModel(ctx, [S.BatchNorm(fused=fused).desc()], S.MeanSquaredError.kind, (3, 3, 2), 8)
     with pytest.raises(S.ScanetError, match="fused"):       # rank 2 has no fused form (BatchNorm.scala:134-136)
         S.CompiledModel(ctx, [S.BatchNorm(fused=True).desc()], S.MeanSquaredError.kind, (5,), 8)
     bn = S.CompiledModel(ctx, [S.BatchNorm().desc()], S.MeanSquaredError.kind, (5,), 8)

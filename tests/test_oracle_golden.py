@@ -320,6 +320,72 @@ def test_batch_norm_state_bypasses_the_algorithm(golden):
     np.testing.assert_allclose(out.var(axis=0), 1.0, atol=1e-3)      # var / (var + epsilon)
 
 
+def test_fused_batch_norm_op_definitions(golden):
+    """`FusedBatchNormV3` / `GradV3` as TensorFlow defines them, before the reference's wiring: y is the generic form's y
+    (so the reference's BatchNormSpec values hold for it, in training and in inference mode), output 2 is the unbiased
+    variance, and the gradient op handed the true batch statistics returns the true gradient."""
+    g = golden["batch_norm"]
+    x = (A(g["x"]) @ A(g["dense_w"]) + A(g["dense_b"])).reshape(4, 1, 1, 4)     # the Dense output, as an NHWC image
+    ones, zeros = np.ones(4, np.float32), np.zeros(4, np.float32)
+    outs = O.fused_batch_norm(x, ones, zeros, zeros, ones, 1e-3, True)
+    np.testing.assert_array_equal(round_at(outs[0].reshape(4, 4), 3), A(g["training"]["y_3dp"]))
+    np.testing.assert_allclose(outs[1], x.reshape(4, 4).mean(axis=0), rtol=1e-6)
+    np.testing.assert_allclose(outs[2], x.reshape(4, 4).astype(np.float64).var(axis=0, ddof=1), rtol=1e-5)
+    np.testing.assert_allclose(outs[4], x.reshape(4, 4).astype(np.float64).var(axis=0), rtol=1e-5)
+    np.testing.assert_array_equal(outs[3], outs[1])
+    t = g["frozen"]
+    frozen = O.fused_batch_norm(x, A(t["gamma"]), A(t["beta"]), A(t["moving_mean"]), A(t["moving_variance"]), 1e-3, False)
+    np.testing.assert_array_equal(round_at(frozen[0].reshape(4, 4), 3), A(t["y_3dp"]))
+    # a single row: n - 1 is taken as 1
+    one = O.fused_batch_norm(x[:1], ones, zeros, zeros, ones, 1e-3, True)
+    np.testing.assert_array_equal(one[2], np.zeros(4, np.float32))
+    # the gradient op with the true statistics against central differences of sum(y * dy), float64
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((3, 2, 2, 5))
+    scale, offset, dy = rng.uniform(0.5, 1.5, 5), rng.standard_normal(5), rng.standard_normal((3, 2, 2, 5))
+    f = lambda xx, sc, of: float((O.fused_batch_norm(xx, sc, of, None, None, 1e-3, True)[0] * dy).sum())
+    outs = O.fused_batch_norm(x, scale, offset, None, None, 1e-3, True)
+    dx, dscale, doffset = O.fused_batch_norm_grad(dy, x, scale, outs[3], outs[4], 1e-3)
+    h = 1e-6
+    for idx in [(0, 0, 0, 0), (2, 1, 0, 3), (1, 1, 1, 4)]:
+        e = np.zeros_like(x); e[idx] = h
+        assert abs((f(x + e, scale, offset) - f(x - e, scale, offset)) / (2 * h) - dx[idx]) < 1e-7
+    for ch in range(5):
+        e = np.zeros(5); e[ch] = h
+        assert abs((f(x, scale + e, offset) - f(x, scale - e, offset)) / (2 * h) - dscale[ch]) < 1e-7
+        assert abs((f(x, scale, offset + e) - f(x, scale, offset - e)) / (2 * h) - doffset[ch]) < 1e-7
+
+
+def test_fused_batch_norm_layer_wiring():
+    """The layer's fused branch as the reference wires the op's outputs (math/nn/AllKernels.scala:437-448): the output
+    is the op's; the moving variance moves towards the batch MEAN; the gradient op is handed the unbiased variance as
+    its mean and the batch mean as its variance.  (Read off the reference's source: no reference test holds values.)"""
+    rng = np.random.default_rng(13)
+    x = rng.uniform(0.5, 2.0, (6, 3, 2, 4)).astype(np.float32)          # positive, so that `mean + epsilon` has a root
+    m = O.Model([O.BatchNorm(momentum=0.9, epsilon=1e-3, fused=True)], O.LOSS_MSE)
+    p = {"beta": rng.standard_normal((1, 1, 1, 4)).astype(np.float32), "gamma": rng.uniform(0.5, 1.5, (1, 1, 1, 4)).astype(np.float32),
+         "moving_mean": np.zeros((1, 1, 1, 4), np.float32), "moving_variance": np.ones((1, 1, 1, 4), np.float32)}
+    assert [s for _, s in m.param_defs((6, 3, 2, 4))] == [(1, 1, 1, 4)] * 4
+    generic = O.Model([O.BatchNorm(momentum=0.9, epsilon=1e-3)], O.LOSS_MSE)
+    nxt, nxt_g = {}, {}
+    y = m.forward(x, p, training=True, next_state=nxt)
+    np.testing.assert_allclose(y, generic.forward(x, p, training=True, next_state=nxt_g), rtol=1e-5, atol=1e-6)
+    mean = x.reshape(-1, 4).mean(axis=0)
+    var = x.reshape(-1, 4).var(axis=0)
+    np.testing.assert_allclose(nxt["moving_mean"].ravel(), 0.1 * mean, rtol=1e-5)
+    np.testing.assert_allclose(nxt["moving_variance"].ravel(), 0.9 + 0.1 * mean, rtol=1e-5)
+    np.testing.assert_allclose(nxt_g["moving_variance"].ravel(), 0.9 + 0.1 * var, rtol=1e-5)
+    target = rng.standard_normal(y.shape).astype(np.float32)
+    grads = m.grad_stateful(x, target, p)[1]
+    dy = (y - target) * np.float32(2.0 / y.size)
+    n = 36
+    _, dscale, doffset = O.fused_batch_norm_grad(dy, x, p["gamma"], var * n / (n - 1), mean, 1e-3)
+    np.testing.assert_allclose(grads["gamma"].ravel(), dscale, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(grads["beta"].ravel(), doffset, rtol=1e-5, atol=1e-7)
+    true_grads = generic.grad_stateful(x, target, p)[1]
+    assert not np.allclose(grads["gamma"], true_grads["gamma"], rtol=1e-2)     # the wiring is not the true gradient
+
+
 def test_seeded_initializers_golden(golden):
     """InitializerSpec.scala:23-66: TensorFlow's seeded streams, restated."""
     for case in golden["initializers"]["cases"]:
