@@ -174,8 +174,8 @@ def bench_lstm(S, ctx, steps, warmup):
 
 
 def bench_cnn_bn(S, ctx, steps, warmup):
-    """The CNN the reference trains on MNIST (test models/CNNSpec.scala:22-35), BatchNorm in its generic form."""
-    layers = (S.Conv2D(32, activation=S.ReLU()) >> S.BatchNorm(fused=False) >> S.Pool2D(strides=(2, 2))
+    """The CNN the reference trains on MNIST (test models/CNNSpec.scala:22-35), BatchNorm(fused = Some(true)) as there."""
+    layers = (S.Conv2D(32, activation=S.ReLU()) >> S.BatchNorm(fused=True) >> S.Pool2D(strides=(2, 2))
               >> S.Conv2D(64, activation=S.ReLU()) >> S.Pool2D(strides=(2, 2)) >> S.Activate(S.ReLU()) >> S.Flatten
               >> S.Dense(64, S.ReLU()) >> S.Dense(10, S.Softmax))
     r = run_model_workload(

@@ -505,8 +505,8 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
           ("flatten",), ("dense", 10, "softmax")], "cce", (28, 28, 1), 100, "uniform_onehot"),
         ([("lstm", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),
         ([("simple_rnn", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression"),   # the same shape, simple cell
-        # the CNN of the reference's MNIST test (CNNSpec.scala:22-35) with BatchNorm in its generic form, batch 1000
-        ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3), ("pool", (2, 2), (2, 2), "valid"),
+        # the CNN of the reference's MNIST test (CNNSpec.scala:22-35), BatchNorm(fused = Some(true)) as there, batch 1000
+        ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("batchnorm", 0.99, 1e-3, "fused"), ("pool", (2, 2), (2, 2), "valid"),
           ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "valid"), ("activate", "relu"), ("flatten",),
           ("dense", 64, "relu"), ("dense", 10, "softmax")], "cce", (28, 28, 1), 1000, "uniform_onehot"),
     ]
