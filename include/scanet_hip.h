@@ -95,7 +95,10 @@ typedef struct sn_layer_desc {
   int32_t kernel_h, kernel_w;   /* Conv2D kernel / Pool2D window */
   int32_t stride_h, stride_w;
   int32_t padding;       /* SN_PAD_* */
-  int32_t reg_kind;      /* Dense/Bias: SN_REG_* */
+  int32_t reg_kind;      /* Dense/Bias: SN_REG_*; LSTM / SIMPLE_RNN: `kernelReg`; BATCHNORM: `betaRegularizer` (the reference adds
+                            betaRegularizer(gamma) twice and never uses gammaRegularizer, layer/BatchNorm.scala:158-160; the library
+                            does the same).  Bias and BatchNorm penalties count only while the model is trainable: sn_loss, the
+                            frozen model's loss, leaves them out (layer/Bias.scala:35-36) */
   float reg_lambda;
   int32_t use_bias;      /* LSTM: per-gate bias vectors (layer/RNN.scala:215); SIMPLE_RNN: the cell's Bias (RNN.scala:116) */
   int32_t return_sequence; /* LSTM / SIMPLE_RNN: `returnSequence` (layer/RNN.scala:27,74-77): the output is every step's
@@ -111,6 +114,10 @@ typedef struct sn_layer_desc {
                             OP'S OUTPUTS (math/nn/AllKernels.scala:437-448): same output as the generic form, but the
                             moving variance follows the batch mean and the gradient op receives the unbiased batch
                             variance as its mean and the batch mean as its variance. */
+  int32_t recurrent_reg_kind;   /* LSTM / SIMPLE_RNN: `recurrentReg` and `biasReg` (layer/RNN.scala:120-122,233-235) */
+  float recurrent_reg_lambda;
+  int32_t bias_reg_kind;
+  float bias_reg_lambda;
   int32_t pool_reduce;   /* POOL2D: SN_POOL_*.  AVG divides by the number of window cells inside the input (TF AvgPool) */
 } sn_layer_desc;
 

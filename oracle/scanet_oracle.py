@@ -411,8 +411,12 @@ class Layer:
     strides: Tuple[int, int] = (1, 1)
     padding: int = PAD_VALID
     explicit: Tuple[int, int, int, int] = (0, 0, 0, 0)   # conv2d with PAD_EXPLICIT: top, bottom, left, right (AllKernels.scala:67-100)
-    reg: int = REG_NONE
+    reg: int = REG_NONE             # dense / bias; lstm / simple_rnn: kernelReg; batchnorm: betaRegularizer
     reg_lambda: float = 0.0
+    recurrent_reg: int = REG_NONE   # lstm / simple_rnn: recurrentReg and biasReg (RNN.scala:120-122,233-235)
+    recurrent_lambda: float = 0.0
+    bias_reg: int = REG_NONE
+    bias_lambda: float = 0.0
     bias: bool = True               # lstm / simple_rnn only
     rnn_activation: int = ACT_TANH  # simple_rnn cell activation / lstm `activation`
     return_sequence: bool = False   # lstm / simple_rnn: every step's output, (batch, time, units) (RNN.scala:27,75-77)
@@ -499,24 +503,28 @@ def Flatten():
     return [Layer("flatten")]
 
 
-def LSTM(units, bias=True, return_sequence=False):
-    return [Layer("lstm", units=units, bias=bias, return_sequence=return_sequence)]
+def LSTM(units, bias=True, return_sequence=False, kernel_reg=(REG_NONE, 0.0), recurrent_reg=(REG_NONE, 0.0), bias_reg=(REG_NONE, 0.0)):
+    return [Layer("lstm", units=units, bias=bias, return_sequence=return_sequence, reg=kernel_reg[0], reg_lambda=kernel_reg[1],
+                  recurrent_reg=recurrent_reg[0], recurrent_lambda=recurrent_reg[1], bias_reg=bias_reg[0], bias_lambda=bias_reg[1])]
 
 
-def SimpleRNN(units, activation=ACT_TANH, bias=True, return_sequence=False):
-    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation, return_sequence=return_sequence)]
+def SimpleRNN(units, activation=ACT_TANH, bias=True, return_sequence=False, kernel_reg=(REG_NONE, 0.0), recurrent_reg=(REG_NONE, 0.0),
+              bias_reg=(REG_NONE, 0.0)):
+    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation, return_sequence=return_sequence,
+                  reg=kernel_reg[0], reg_lambda=kernel_reg[1], recurrent_reg=recurrent_reg[0], recurrent_lambda=recurrent_reg[1],
+                  bias_reg=bias_reg[0], bias_lambda=bias_reg[1])]
 
 
 BN_PARAMS = ("beta", "gamma", "moving_mean", "moving_variance")   # BatchNorm.scala:92-97,170-173
 BN_STATE = ("moving_mean", "moving_variance")                      # not trainable: replaced by the layer, not by the optimizer
 
 
-def BatchNorm(momentum=0.99, epsilon=1e-3, fused=False):
+def BatchNorm(momentum=0.99, epsilon=1e-3, fused=False, beta_reg=(REG_NONE, 0.0)):
     """`BatchNorm(axes = Seq(-1))` (BatchNorm.scala:64-76).  fused=False: the generic `batchNorm` form
     (math/nn/AllKernels.scala:663-684), which the layer takes for `fused = Some(false)` and for any input that is not
     rank 4.  fused=True: the FusedBatchNormV3 branch it takes for rank-4 input otherwise, wired as the reference
     wires it (`batchnorm_fused_forward`)."""
-    return [Layer("batchnorm", momentum=momentum, epsilon=epsilon, fused=fused)]
+    return [Layer("batchnorm", momentum=momentum, epsilon=epsilon, fused=fused, reg=beta_reg[0], reg_lambda=beta_reg[1])]
 
 
 def is_state_path(path: str) -> bool:
@@ -719,22 +727,48 @@ class Model:
         return x
 
     # ---- penalty (Regularization.scala:30-44; Composed.scala:66-75) -------- #
-    def penalty(self, params):
+    def regularized(self, training: bool = True):
+        """(path, kind, lambda, times) of every penalty term of the model.
+
+        Dense: reg(weights), always (Dense.scala:63-64).  Bias (also the ones inside Dense, Conv2D and the RNN cells):
+        reg(weights) only while trainable (Bias.scala:35-36), so not in the frozen model a TrainedModel holds.
+        SimpleRNNCell: kernelReg(kernel) + recurrentReg(recurrent), always (RNN.scala:198-199); an LSTM sums its four
+        gate cells (:341-346).  BatchNorm: betaRegularizer(gamma) + betaRegularizer(gamma) while trainable
+        (BatchNorm.scala:158-160; gammaRegularizer is never used)."""
+        out = []
+        for i, l in enumerate(self.layers):
+            pre = self._prefix(i)
+            if l.kind == "dense":
+                out.append((pre + "weights", l.reg, l.reg_lambda, 1))
+            elif l.kind == "bias" and training:
+                out.append((pre + "weights", l.reg, l.reg_lambda, 1))
+            elif l.kind in ("lstm", "simple_rnn"):
+                for g in ([f"{gate}/" for gate in GATES] if l.kind == "lstm" else [""]):
+                    out.append((pre + g + "0/kernel_weights", l.reg, l.reg_lambda, 1))
+                    out.append((pre + g + "0/recurrent_weights", l.recurrent_reg, l.recurrent_lambda, 1))
+                    if l.bias and training:
+                        out.append((pre + g + "1/weights", l.bias_reg, l.bias_lambda, 1))
+            elif l.kind == "batchnorm" and training:
+                out.append((pre + "gamma", l.reg, l.reg_lambda, 2))
+        return [t for t in out if t[1] != REG_NONE]
+
+    def penalty(self, params, training: bool = True):
         dt = next(iter(params.values())).dtype if params else np.dtype(F32)
         total = dt.type(0.0)
-        for i, l in enumerate(self.layers):
-            if l.kind in ("dense", "bias") and l.reg != REG_NONE:
-                w = params[self._prefix(i) + "weights"]
-                if l.reg == REG_L2:
-                    total = total + dt.type(l.reg_lambda) * sqr(w).sum(dtype=dt) / dt.type(2.0)
-                else:
-                    total = total + dt.type(l.reg_lambda) * np.abs(w).sum(dtype=dt) / dt.type(2.0)
+        for path, kind, lam, times in self.regularized(training):
+            w = params[path]
+            if kind == REG_L2:
+                term = dt.type(lam) * sqr(w).sum(dtype=dt) / dt.type(2.0)
+            else:
+                term = dt.type(lam) * np.abs(w).sum(dtype=dt) / dt.type(2.0)
+            for _ in range(times):
+                total = total + term
         return total
 
     def loss_of(self, x, y, params, training: bool = False):
         """LossModel.buildStateful (Model.scala:92-99): loss(model(x), y) + penalty."""
         p = self.forward(x, params, training=training)
-        return loss_value(self.loss, p, y) + self.penalty(params)
+        return loss_value(self.loss, p, y) + self.penalty(params, training)
 
     # ---- backward: gradients w.r.t. every weight -------------------------- #
     def grad(self, x, y, params):
@@ -779,13 +813,14 @@ class Model:
                 dy = simple_rnn_backward(dy, c, params, pre, l, grads, need_dx=i > 0)
             elif k == "batchnorm":
                 dy = (batchnorm_fused_backward if l.fused else batchnorm_backward)(dy, c, pre, grads)
-            if l.kind in ("dense", "bias") and l.reg != REG_NONE:
-                w = params[pre + "weights"]
-                lam = w.dtype.type(l.reg_lambda)
-                if l.reg == REG_L2:       # d/dw lambda * sum(w^2) / 2 through Pow's grad: (w^1 * 2) * (lambda/2)
-                    grads[pre + "weights"] = grads[pre + "weights"] + (w * w.dtype.type(2.0)) * (lam / w.dtype.type(2.0))
+        for path, kind, lam_f, times in self.regularized(True):
+            w = params[path]
+            lam = w.dtype.type(lam_f)
+            for _ in range(times):
+                if kind == REG_L2:        # d/dw lambda * sum(w^2) / 2 through Pow's grad: (w^1 * 2) * (lambda/2)
+                    grads[path] = grads[path] + (w * w.dtype.type(2.0)) * (lam / w.dtype.type(2.0))
                 else:                     # Abs grad in the reference is |parent| (AllKernels.scala:330-335)
-                    grads[pre + "weights"] = grads[pre + "weights"] + np.abs(np.ones_like(w) * (lam / w.dtype.type(2.0)))
+                    grads[path] = grads[path] + np.abs(np.ones_like(w) * (lam / w.dtype.type(2.0)))
         return loss, grads, next_state
 
 

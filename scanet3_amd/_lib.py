@@ -45,7 +45,8 @@ class LayerDesc(C.Structure):
                 ("padding", C.c_int32), ("reg_kind", C.c_int32), ("reg_lambda", C.c_float), ("use_bias", C.c_int32),
                 ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float),
                 ("pad_top", C.c_int32), ("pad_bottom", C.c_int32), ("pad_left", C.c_int32), ("pad_right", C.c_int32),
-                ("bn_fused", C.c_int32), ("pool_reduce", C.c_int32)]
+                ("bn_fused", C.c_int32), ("recurrent_reg_kind", C.c_int32), ("recurrent_reg_lambda", C.c_float),
+                ("bias_reg_kind", C.c_int32), ("bias_reg_lambda", C.c_float), ("pool_reduce", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):

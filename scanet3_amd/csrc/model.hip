@@ -20,6 +20,9 @@ struct ParamDef {
   sn_param_info info;
   int reg_kind = SN_REG_NONE;
   float reg_lambda = 0.f;
+  // Bias and BatchNorm add their penalty only while trainable (layer/Bias.scala:35-36, layer/BatchNorm.scala:158-160):
+  // the frozen model a TrainedModel holds leaves it out; Dense and the RNN cells add theirs always.
+  bool penalty_when_frozen = true;
 };
 
 struct Op {
@@ -135,7 +138,7 @@ static void conv_out(int padding, int in, int k, int s, int* out, int* pad_befor
 }
 
 static int add_param(sn_model* m, const std::string& path, const std::vector<int64_t>& dims, int reg_kind, float reg_lambda,
-                     bool trainable = true) {
+                     bool trainable = true, bool penalty_when_frozen = true) {
   ParamDef p;
   memset(&p.info, 0, sizeof(p.info));
   p.info.trainable = trainable ? 1 : 0;
@@ -149,6 +152,7 @@ static int add_param(sn_model* m, const std::string& path, const std::vector<int
   p.info.offset = m->flat_elems;
   p.reg_kind = reg_kind;
   p.reg_lambda = reg_lambda;
+  p.penalty_when_frozen = penalty_when_frozen;
   m->flat_elems += align_up(p.info.size, 64);  // every tensor starts on a 256-byte boundary
   m->params.push_back(p);
   return (int)m->params.size() - 1;
@@ -178,7 +182,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ++i;
         if (i < n_layers && layers[i].kind == SN_LAYER_BIAS) {
           SN_REQUIRE(layers[i].units == L.units, "layer %d: Bias has %d features, input has %d", i, layers[i].units, L.units);
-          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda);
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda, true, false);
           ++i;
         }
         if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
@@ -210,7 +214,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ++i;
         if (i < n_layers && layers[i].kind == SN_LAYER_BIAS) {
           SN_REQUIRE(layers[i].units == L.units, "layer %d: Bias has %d features, input has %d", i, layers[i].units, L.units);
-          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda);
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, layers[i].reg_kind, layers[i].reg_lambda, true, false);
           ++i;
         }
         if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
@@ -260,7 +264,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         op.kind = OP_BIASACT;
         if (L.kind == SN_LAYER_BIAS) {
           SN_REQUIRE(L.units == cur.back(), "layer %d: Bias has %d features, input has %lld", i, L.units, (long long)cur.back());
-          op.b = add_param(m, prefix(i) + "weights", {L.units}, L.reg_kind, L.reg_lambda);
+          op.b = add_param(m, prefix(i) + "weights", {L.units}, L.reg_kind, L.reg_lambda, true, false);
           ++i;
           if (i < n_layers && layers[i].kind == SN_LAYER_ACTIVATE && layers[i].activation != SN_ACT_SOFTMAX) {
             op.act = layers[i].activation;
@@ -285,9 +289,10 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         static const char* gates[4] = {"forget", "input", "gate", "output"};  // layer/RNN.scala:285-289
         for (int gi = 0; gi < 4; ++gi) {
           const std::string gp = prefix(i) + gates[gi];
-          op.lstm_p[gi][0] = add_param(m, gp + "/0/kernel_weights", {op.F, op.H}, SN_REG_NONE, 0.f);
-          op.lstm_p[gi][1] = add_param(m, gp + "/0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
-          if (L.use_bias) op.lstm_p[gi][2] = add_param(m, gp + "/1/weights", {op.H}, SN_REG_NONE, 0.f);
+          // every gate is a SimpleRNNCell ?>> Bias with the layer's three regularizers (RNN.scala:270-283,198-199)
+          op.lstm_p[gi][0] = add_param(m, gp + "/0/kernel_weights", {op.F, op.H}, L.reg_kind, L.reg_lambda);
+          op.lstm_p[gi][1] = add_param(m, gp + "/0/recurrent_weights", {op.H, op.H}, L.recurrent_reg_kind, L.recurrent_reg_lambda);
+          if (L.use_bias) op.lstm_p[gi][2] = add_param(m, gp + "/1/weights", {op.H}, L.bias_reg_kind, L.bias_reg_lambda, true, false);
         }
         op.ret_seq = L.return_sequence != 0;
         op.out_dims = op.ret_seq ? std::vector<int64_t>{op.T, L.units} : std::vector<int64_t>{L.units};  // RNN.scala:84-90
@@ -313,7 +318,10 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         std::vector<int64_t> shape(cur.size() + 1, 1);  // every axis but the normalised one becomes 1 (BatchNorm.scala:80-88)
         shape.back() = cur.back();
         static const char* names[4] = {"beta", "gamma", "moving_mean", "moving_variance"};  // BatchNorm.scala:92-97,170-173
-        for (int k = 0; k < 4; ++k) op.bn_p[k] = add_param(m, prefix(i) + names[k], shape, SN_REG_NONE, 0.f, k < 2);
+        // penalty = betaRegularizer(gamma) + betaRegularizer(gamma) while trainable (BatchNorm.scala:158-160): the beta
+        // regularizer, on gamma, twice; doubling lambda is the same number bit for bit
+        for (int k = 0; k < 4; ++k)
+          op.bn_p[k] = add_param(m, prefix(i) + names[k], shape, k == 1 ? L.reg_kind : SN_REG_NONE, k == 1 ? 2.0f * L.reg_lambda : 0.f, k < 2, false);
         ws = std::max(ws, batchnorm_workspace_elems(m->ctx, (int64_t)B * (prod(cur) / cur.back()), (int)cur.back()));
         ++i;
         break;
@@ -327,9 +335,9 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         op.T = (int)cur[0]; op.F = (int)cur[1]; op.H = L.units;
         op.act = L.activation;
         op.act_param = L.act_param;
-        op.lstm_p[0][0] = add_param(m, prefix(i) + "0/kernel_weights", {op.F, op.H}, SN_REG_NONE, 0.f);  // RNN.scala:165-166,198-203
-        op.lstm_p[0][1] = add_param(m, prefix(i) + "0/recurrent_weights", {op.H, op.H}, SN_REG_NONE, 0.f);
-        if (L.use_bias) op.b = add_param(m, prefix(i) + "1/weights", {op.H}, SN_REG_NONE, 0.f);
+        op.lstm_p[0][0] = add_param(m, prefix(i) + "0/kernel_weights", {op.F, op.H}, L.reg_kind, L.reg_lambda);  // RNN.scala:165-166,198-203
+        op.lstm_p[0][1] = add_param(m, prefix(i) + "0/recurrent_weights", {op.H, op.H}, L.recurrent_reg_kind, L.recurrent_reg_lambda);
+        if (L.use_bias) op.b = add_param(m, prefix(i) + "1/weights", {op.H}, L.bias_reg_kind, L.bias_reg_lambda, true, false);
         op.ret_seq = L.return_sequence != 0;
         op.out_dims = op.ret_seq ? std::vector<int64_t>{op.T, L.units} : std::vector<int64_t>{L.units};
         ws = std::max(ws, gemm_workspace_elems(B, op.H, op.F + op.H, cu));
@@ -617,20 +625,20 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
   return SN_OK;
 }
 
-static int add_penalties(sn_replica* r) {
+static int add_penalties(sn_replica* r, bool training) {
   for (auto& p : r->model->params)
-    if (p.reg_kind != SN_REG_NONE)
+    if (p.reg_kind != SN_REG_NONE && (training || p.penalty_when_frozen))
       SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev));
   return SN_OK;
 }
 
 // loss (+ penalty) into loss_dev; dp (may be null) receives d loss / d prediction
-static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp) {
+static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp, bool training) {
   sn_model* m = r->model;
   if (m->loss == SN_LOSS_IDENTITY)
     SN_REQUIRE((int64_t)rows * m->out_elems == 1, "Identity loss needs a scalar model output");
   SN_TRY(launch_loss(r->ctx, m->loss, pred, y, dp, r->loss_dev, r->loss_partials, rows, (int)m->out_elems));
-  return add_penalties(r);
+  return add_penalties(r, training);
 }
 
 // ---------------------------------------------------------------------------- backward
@@ -853,12 +861,12 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
     SN_TRY(forward(r, x, rows, true, true));
     SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], r->loss_dev, r->loss_partials, rows,
                               (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
-    SN_TRY(add_penalties(r));
+    SN_TRY(add_penalties(r, true));
     return backward(r, x, rows, last - 1, 1);
   }
   SN_TRY(forward(r, x, rows, false, true));
   const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);
-  SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0]));
+  SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0], true));
   SN_TRY(backward(r, x, rows));
   return SN_OK;
 }
@@ -1094,7 +1102,7 @@ int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   SN_TRY(check_rows(rep, rows));
   SN_TRY(forward(rep, x_dev, rows));
   const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
-  SN_TRY(loss_of(rep, pred, y_dev, rows, nullptr));
+  SN_TRY(loss_of(rep, pred, y_dev, rows, nullptr, false));  // the frozen model of a TrainedModel (models/Model.scala:126-127)
   return read_loss(rep, loss_host);
 }
 
@@ -1146,7 +1154,7 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
     const float* yl = y_dev + (n_batches - 1) * ys;
     SN_TRY(forward(rep, xl, batch, false, true));  // `lossModel.lossStateful`: not frozen (Optimizer.scala:163-167)
     const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, xl, batch);
-    SN_TRY(loss_of(rep, pred, yl, batch, nullptr));
+    SN_TRY(loss_of(rep, pred, yl, batch, nullptr, true));
     SN_TRY(read_loss(rep, loss_host));
   }
   return SN_OK;
@@ -1201,7 +1209,7 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
   if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
     SN_TRY(forward(rep, rep->stage_x[last], batch, false, true));
     const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, rep->stage_x[last], batch);
-    SN_TRY(loss_of(rep, pred, rep->stage_y[last], batch, nullptr));
+    SN_TRY(loss_of(rep, pred, rep->stage_y[last], batch, nullptr, true));
     SN_TRY(read_loss(rep, loss_host));
   } else {
     SN_HIP(hipStreamSynchronize(compute));  // the host buffers may be reused once this returns

@@ -239,6 +239,8 @@ class Layer:
     epsilon: float = 1e-3
     fused: int = -1               # BatchNorm `fused`: -1 None, 0 Some(false), 1 Some(true)
     pool_reduce: int = 0          # Pool2D: L.POOL_MAX or L.POOL_AVG
+    recurrent_reg: Regularization = Zero   # RNN layers: `recurrentReg`, `biasReg` (`reg` is their `kernelReg`)
+    bias_reg: Regularization = Zero
 
     def __rshift__(self, other):
         return Composed.of(self, other)
@@ -251,7 +253,8 @@ class Layer:
         return L.LayerDesc(self.kind, self.units, self.activation.kind, self.activation.param, self.kernel[0], self.kernel[1],
                            self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
                            1 if self.return_sequence else 0, self.momentum, self.epsilon,
-                           self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused, self.pool_reduce)
+                           self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused,
+                           self.recurrent_reg.kind, self.recurrent_reg.lam, self.bias_reg.kind, self.bias_reg.lam, self.pool_reduce)
 
     def __repr__(self):
         return self.text
@@ -334,35 +337,40 @@ Flatten = Layer(L.LAYER_FLATTEN, "Flatten")
 
 def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
          recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
-         biasForgetInitializer: Initializer = Ones, returnSequence: bool = False) -> Layer:
-    """layer/RNN.scala:208-258: tanh cell, sigmoid gates, forget bias one."""
+         biasForgetInitializer: Initializer = Ones, returnSequence: bool = False, kernelReg: Regularization = Zero,
+         recurrentReg: Regularization = Zero, biasReg: Regularization = Zero) -> Layer:
+    """layer/RNN.scala:208-258: tanh cell, sigmoid gates, forget bias one; the three regularizers apply to every gate."""
     return Layer(L.LAYER_LSTM, f"RNN(LSTMCell({units},Tanh,Sigmoid,{'true' if bias else 'false'}))", units=units,
-                 activation=Tanh, use_bias=bias, return_sequence=returnSequence,
+                 activation=Tanh, use_bias=bias, return_sequence=returnSequence, reg=kernelReg, recurrent_reg=recurrentReg,
+                 bias_reg=biasReg,
                  inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
 
 
 def BatchNorm(axes: Sequence[int] = (-1,), momentum: float = 0.99, epsilon: float = 1e-3, betaInitializer: Initializer = Zeros,
               gammaInitializer: Initializer = Ones, movingMeanInitializer: Initializer = Zeros,
-              movingVarianceInitializer: Initializer = Ones, fused: Optional[bool] = None) -> Layer:
+              movingVarianceInitializer: Initializer = Ones, fused: Optional[bool] = None,
+              betaRegularizer: Regularization = Zero, gammaRegularizer: Regularization = Zero) -> Layer:
     """layer/BatchNorm.scala:64-76 over the last axis.  As in the reference, rank-4 input takes the FusedBatchNormV3
     branch unless `fused=False` (wired as the reference wires that op's outputs, which is not the generic form's
-    gradient nor its moving variance); every other rank takes the generic form."""
+    gradient nor its moving variance); every other rank takes the generic form.  The reference's penalty is
+    betaRegularizer(gamma) + betaRegularizer(gamma) (:158-160); `gammaRegularizer` is accepted and, as there, unused."""
     if tuple(axes) != (-1,):
         raise ValueError("only axes = Seq(-1) is built")
     return Layer(L.LAYER_BATCHNORM, f"BatchNorm({list(axes)})", momentum=momentum, epsilon=epsilon,
-                 fused=-1 if fused is None else int(bool(fused)),
+                 fused=-1 if fused is None else int(bool(fused)), reg=betaRegularizer,
                  inits=(betaInitializer, gammaInitializer, movingMeanInitializer, movingVarianceInitializer))
 
 
 def SimpleRNN(units: int, activation: Activation = Tanh, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
               recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
-              returnSequence: bool = False) -> Layer:
+              returnSequence: bool = False, kernelReg: Regularization = Zero, recurrentReg: Regularization = Zero,
+              biasReg: Regularization = Zero) -> Layer:
     """layer/RNN.scala:96-137: `RNN(SimpleRNNCell(..))`; the last step's output leaves the layer."""
     if activation.kind == L.ACT_SOFTMAX:
         raise ValueError("requirement failed: Softmax is not a cell activation")
     return Layer(L.LAYER_SIMPLE_RNN, f"RNN(SimpleRNNCell({units},{activation!r},{'true' if bias else 'false'}))", units=units,
-                 activation=activation, use_bias=bias, return_sequence=returnSequence,
-                 inits=(kernelInitializer, recurrentInitializer, biasInitializer))
+                 activation=activation, use_bias=bias, return_sequence=returnSequence, reg=kernelReg, recurrent_reg=recurrentReg,
+                 bias_reg=biasReg, inits=(kernelInitializer, recurrentInitializer, biasInitializer))
 
 
 def LinearRegression(reg: Regularization = Zero, bias: bool = True):

@@ -13,7 +13,7 @@ f32 = np.float32
 
 def build_pair(spec: List[tuple], loss: str):
     """spec entries: ("dense", units, act[, reg, lam]) | ("conv", filters, kernel, strides, pad, act, bias)
-    | ("pool", window, strides, pad[, "avg"]) | ("flatten",) | ("lstm", units[, bias]) | ("simple_rnn", units[, act[, bias]]) | ("batchnorm", momentum, epsilon[, "fused"]) | ("activate", act) | ("bias", features)
+    | ("pool", window, strides, pad[, "avg"]) | ("flatten",) | ("lstm", units[, bias[, seq[, regs]]]) | ("simple_rnn", units[, act[, bias[, seq[, regs]]]]) | ("batchnorm", momentum, epsilon[, "fused" or None[, regs]]) | ("activate", act) | ("bias", features)
     Returns (oracle Model, scanet3_amd layer composition, scanet3_amd loss)."""
     import scanet3_amd as S
     acts_o = {"identity": O.ACT_IDENTITY, "sigmoid": O.ACT_SIGMOID, "tanh": O.ACT_TANH, "relu": O.ACT_RELU,
@@ -23,6 +23,13 @@ def build_pair(spec: List[tuple], loss: str):
     pads_s = {"valid": S.Valid, "same": S.Same}
     regs_o = {"none": O.REG_NONE, "l1": O.REG_L1, "l2": O.REG_L2}
     ol, sl = [], None
+
+    def regs(entry, at):
+        """Optional trailing tuple of (kind, lambda) pairs -> (oracle pairs, library Regularizations)."""
+        given = entry[at] if len(entry) > at else ()
+        o = [(regs_o[k], lam) for k, lam in given]
+        s_ = [S.Zero if k == "none" else (S.L1(lam) if k == "l1" else S.L2(lam)) for k, lam in given]
+        return o, s_
 
     def add(layer):
         nonlocal sl
@@ -58,18 +65,23 @@ def build_pair(spec: List[tuple], loss: str):
         elif k == "lstm":     # ("lstm", units[, bias[, return_sequence]])
             bias = e[2] if len(e) > 2 else True
             seq = e[3] if len(e) > 3 else False
-            ol.append(O.LSTM(e[1], bias=bias, return_sequence=seq))
-            add(S.LSTM(e[1], bias=bias, returnSequence=seq))
+            ro, rs = regs(e, 4)           # ((kernel), (recurrent), (bias)) regularizers
+            names_o, names_s = ("kernel_reg", "recurrent_reg", "bias_reg"), ("kernelReg", "recurrentReg", "biasReg")
+            ol.append(O.LSTM(e[1], bias=bias, return_sequence=seq, **dict(zip(names_o, ro))))
+            add(S.LSTM(e[1], bias=bias, returnSequence=seq, **dict(zip(names_s, rs))))
         elif k == "simple_rnn":  # ("simple_rnn", units[, act[, bias[, return_sequence]]])
             act = e[2] if len(e) > 2 else "tanh"
             bias = e[3] if len(e) > 3 else True
             seq = e[4] if len(e) > 4 else False
-            ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias, return_sequence=seq))
-            add(S.SimpleRNN(e[1], acts_s[act], bias=bias, returnSequence=seq))
+            ro, rs = regs(e, 5)
+            names_o, names_s = ("kernel_reg", "recurrent_reg", "bias_reg"), ("kernelReg", "recurrentReg", "biasReg")
+            ol.append(O.SimpleRNN(e[1], acts_o[act], bias=bias, return_sequence=seq, **dict(zip(names_o, ro))))
+            add(S.SimpleRNN(e[1], acts_s[act], bias=bias, returnSequence=seq, **dict(zip(names_s, rs))))
         elif k == "batchnorm":   # ("batchnorm", momentum, epsilon[, "fused"]): the generic form (fused = Some(false)) unless asked
             fused = len(e) > 3 and e[3] == "fused"   # rank-4 input only: the layer's default there (fused = None)
-            ol.append(O.BatchNorm(e[1], e[2], fused=fused))
-            add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=None if fused else False))
+            ro, rs = regs(e, 4)           # ((beta regularizer),)
+            ol.append(O.BatchNorm(e[1], e[2], fused=fused, **({"beta_reg": ro[0]} if ro else {})))
+            add(S.BatchNorm(momentum=e[1], epsilon=e[2], fused=None if fused else False, **({"betaRegularizer": rs[0]} if rs else {})))
         elif k == "activate":
             ol.append([O.Layer("activate", activation=acts_o[e[1]])])
             add(S.Activate(acts_s[e[1]]))

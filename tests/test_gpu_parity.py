@@ -408,6 +408,14 @@ MODELS = {
                             "cce", (12, 12, 2), 24, "uniform_onehot"),
     "batchnorm_fused_first": ([("batchnorm", 0.5, 1e-2, "fused"), ("conv", 3, (2, 2), (1, 1), "valid", "tanh", True), ("flatten",), ("dense", 2, "identity")],
                               "mse", (5, 4, 3), 9, "uniform_binary"),     # inputs in [0, 1): positive channel means
+    # regularizers on recurrent and batch-norm weights (layer/RNN.scala:120-122,198-199,233-235; BatchNorm.scala:158-160:
+    # the beta regularizer lands on gamma, twice); bias and batch-norm penalties drop out of the frozen model's loss
+    "lstm_regularized": ([("lstm", 6, True, False, (("l2", 0.05), ("l1", 0.02), ("l2", 0.3))), ("dense", 2, "identity", "l1", 0.01)],
+                         "mse", (5, 3), 12, "normal_regression"),
+    "simple_rnn_regularized": ([("simple_rnn", 16, "tanh", True, False, (("l1", 0.03), ("l2", 0.04), ("l1", 0.2))), ("dense", 1, "tanh")],
+                               "mse", (6, 8), 20, "normal_regression"),
+    "batchnorm_regularized": ([("dense", 9, "tanh", "l2", 0.02), ("batchnorm", 0.9, 1e-3, None, (("l2", 0.1),)), ("dense", 3, "softmax")],
+                              "cce", (7,), 40, "normal_onehot"),
     # tens of thousands of output positions over 4 input channels: padding, bias, strides, channel counts that are
     # multiples of 4 but not of 16
     "conv_many_positions_same_bias": ([("conv", 8, (3, 3), (1, 1), "same", "tanh", True), ("flatten",), ("dense", 3, "softmax")],
@@ -468,7 +476,8 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
 
 
 @pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
-                                        ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("cnn_batchnorm_fused", 12), ("mlp_bce_l2", 25)])
+                                        ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("cnn_batchnorm_fused", 12), ("mlp_bce_l2", 25),
+                                        ("lstm_regularized", 15), ("batchnorm_regularized", 15)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
 def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
     spec, loss, in_shape, batch, kind = MODELS[name]

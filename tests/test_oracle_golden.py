@@ -386,6 +386,38 @@ def test_fused_batch_norm_layer_wiring():
     assert not np.allclose(grads["gamma"], true_grads["gamma"], rtol=1e-2)     # the wiring is not the true gradient
 
 
+def test_penalties_of_recurrent_and_batch_norm_layers():
+    """Which weights a penalty lands on (RNN.scala:198-199,341-346; BatchNorm.scala:158-160; Bias.scala:35-36), checked
+    against the closed forms, and the L2 part of the gradient against central differences in float64."""
+    rng = np.random.default_rng(0)
+    m = O.Model([O.LSTM(4, kernel_reg=(O.REG_L2, 0.05), recurrent_reg=(O.REG_L1, 0.02), bias_reg=(O.REG_L2, 0.3)),
+                 O.BatchNorm(beta_reg=(O.REG_L2, 0.1)), O.Dense(2, reg=O.REG_L2, reg_lambda=0.01)], O.LOSS_MSE)
+    x, y = rng.standard_normal((5, 3, 2)), rng.standard_normal((5, 2))
+    params = {p: rng.standard_normal(s) * 0.5 for p, s in m.param_defs(x.shape)}
+    params["1/moving_variance"] = np.abs(params["1/moving_variance"]) + 0.5
+    sq = lambda p: float((params[p] ** 2).sum())
+    ab = lambda p: float(np.abs(params[p]).sum())
+    always = sum(0.05 * sq(f"0/{g}/0/kernel_weights") / 2 + 0.02 * ab(f"0/{g}/0/recurrent_weights") / 2 for g in O.GATES) \
+        + 0.01 * sq("2/weights") / 2
+    trainable_only = sum(0.3 * sq(f"0/{g}/1/weights") / 2 for g in O.GATES) + 2 * (0.1 * sq("1/gamma") / 2) + 0.01 * sq("3/weights") / 2
+    np.testing.assert_allclose(m.penalty(params, training=True), always + trainable_only, rtol=1e-12)
+    np.testing.assert_allclose(m.penalty(params, training=False), always, rtol=1e-12)        # the frozen model
+    # gradient of loss + penalty for the L2-regularised tensors (the reference's L1 gradient is |parent| by construction)
+    _, grads, _ = m.grad_stateful(x, y, params)
+    for p in ("0/forget/0/kernel_weights", "0/gate/1/weights", "1/gamma", "2/weights", "3/weights"):
+        w = params[p]
+        idx = tuple(int(rng.integers(0, d)) for d in w.shape)
+        e = np.zeros_like(w)
+        e[idx] = 1e-6
+        up, down = dict(params), dict(params)
+        up[p], down[p] = w + e, w - e
+        num = (m.loss_of(x, y, up, training=True) - m.loss_of(x, y, down, training=True)) / 2e-6
+        assert abs(num - grads[p][idx]) < 1e-6 * max(1.0, abs(num)), p
+    # beta itself carries no penalty, whatever regularizer the layer was given
+    plain = O.Model([O.LSTM(4), O.BatchNorm(), O.Dense(2)], O.LOSS_MSE)
+    np.testing.assert_allclose(grads["1/beta"], plain.grad_stateful(x, y, params)[1]["1/beta"], rtol=1e-12)
+
+
 def test_seeded_initializers_golden(golden):
     """InitializerSpec.scala:23-66: TensorFlow's seeded streams, restated."""
     for case in golden["initializers"]["cases"]:
