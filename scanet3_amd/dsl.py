@@ -460,6 +460,53 @@ class Dataset:
         return Builder(model=model, dataset=self)
 
 
+Skip, Partial, PadZeros = "Skip", "Partial", "PadZeros"
+
+
+class TensorIterator:
+    """optimizers/Iterators.scala:39-83: groups (features, labels) records into batches of `batch` rows.  What is left
+    over at the end is dropped (`Skip`, what the optimizer uses, Optimizer.scala:115), handed out short (`Partial`, what
+    the estimators use, estimators/package.scala:25) or filled up with zero rows (`PadZeros`)."""
+
+    def __init__(self, rows, shapes, batch: int, remaining: str = Skip):
+        if remaining not in (Skip, Partial, PadZeros):
+            raise ValueError(f"remaining should be Skip, Partial or PadZeros, got {remaining!r}")
+        self._rows = iter(rows)
+        self.shape_x, self.shape_y = tuple(shapes[0]), tuple(shapes[1])
+        self.batch = int(batch)
+        self.remaining = remaining
+        self._group = None
+
+    def _fill(self):
+        if self._group is None:
+            group = []
+            for record in self._rows:
+                group.append(record)
+                if len(group) == self.batch:
+                    break
+            if group and (len(group) == self.batch or self.remaining != Skip):
+                self._group = group
+        return self._group is not None
+
+    def __iter__(self):
+        return self
+
+    def has_next(self) -> bool:
+        return self._fill()
+
+    def __next__(self):
+        if not self._fill():
+            raise StopIteration
+        group, self._group = self._group, None
+        rows = self.batch if self.remaining == PadZeros else len(group)
+        x = np.zeros((rows,) + self.shape_x, np.float32)
+        y = np.zeros((rows,) + self.shape_y, np.float32)
+        for i, (fx, fy) in enumerate(group):
+            x[i] = np.asarray(fx, np.float32).reshape(self.shape_x)
+            y[i] = np.asarray(fy, np.float32).reshape(self.shape_y)
+        return x, y
+
+
 def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndarray]:
     """ParamDef.initialize for every weight (optimizers/Optimizer.scala:124-128)."""
     rng = np.random.default_rng(seed)

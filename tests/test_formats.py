@@ -123,3 +123,35 @@ def test_kryo_tensor_layout():
         F.kryo_tensor_read(blob[:19] + bytes([13]) + blob[20:])
     with pytest.raises(ValueError):
         F.kryo_tensor_bytes(np.array(["a"]))
+
+
+# --------------------------------------------------------------------------- batching of records (optimizers/IteratorsSpec.scala)
+def _records(n):
+    return [([3 * i + 1, 3 * i + 2], [3 * i + 3]) for i in range(n)]
+
+
+def test_tensor_iterator_known_answers():
+    """The four cases of IteratorsSpec.scala:11-78, plus the default (`Skip`) the optimizer relies on."""
+    from scanet3_amd import dsl as S
+    it = S.TensorIterator(_records(2), ((2,), (1,)), 2)
+    assert it.has_next()
+    x, y = next(it)
+    np.testing.assert_array_equal(x, [[1, 2], [4, 5]])
+    np.testing.assert_array_equal(y, [[3], [6]])
+    assert not it.has_next()
+    batches = list(S.TensorIterator(_records(4), ((2,), (1,)), 2))
+    assert len(batches) == 2
+    np.testing.assert_array_equal(batches[1][0], [[7, 8], [10, 11]])
+    np.testing.assert_array_equal(batches[1][1], [[9], [12]])
+    (x, y), = list(S.TensorIterator(_records(2), ((2,), (1,)), 3, remaining=S.PadZeros))
+    np.testing.assert_array_equal(x, [[1, 2], [4, 5], [0, 0]])
+    np.testing.assert_array_equal(y, [[3], [6], [0]])
+    (x, y), = list(S.TensorIterator(_records(2), ((2,), (1,)), 3, remaining=S.Partial))
+    np.testing.assert_array_equal(x, [[1, 2], [4, 5]])
+    np.testing.assert_array_equal(y, [[3], [6]])
+    assert list(S.TensorIterator(_records(2), ((2,), (1,)), 3)) == []          # Skip: a short batch is dropped
+    assert len(list(S.TensorIterator(_records(7), ((2,), (1,)), 3))) == 2
+    assert [b[0].shape[0] for b in S.TensorIterator(_records(7), ((2,), (1,)), 3, remaining=S.Partial)] == [3, 3, 1]
+    assert x.dtype == np.float32
+    with pytest.raises(ValueError):
+        S.TensorIterator(_records(1), ((2,), (1,)), 1, remaining="Wrap")
