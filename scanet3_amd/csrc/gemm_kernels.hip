@@ -947,21 +947,28 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int M, int N, int K, AL
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int o = tid + j * 256;
-    if (o < outs) partial[(int64_t)o * gridDim.x + blockIdx.x] = acc[j];
+    if (o < outs) partial[(int64_t)blockIdx.x * outs + o] = acc[j];  // [part][output]: a workgroup's outputs leave as one run
   }
 }
 
-// One wavefront per output adds its partial sums (contiguous in memory) in a fixed order.
+// Adds the partial sums [parts][M*N] in a fixed order: a workgroup owns 4 outputs, 64 lanes each walk every 64th part.
 template <class EP>
 __global__ __launch_bounds__(256) void gemm_small_reduce_kernel(const float* __restrict__ partial, int parts, int M, int N, EP ep) {
-  const int lane = threadIdx.x & 63;
-  const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (o >= M * N) return;
+  __shared__ float sm[64][4];
+  const int outs = M * N;
+  const int ol = threadIdx.x & 3, pl = threadIdx.x >> 2;
+  const int o = blockIdx.x * 4 + ol;
   float s = 0.f;
-  for (int i = lane; i < parts; i += 64) s += partial[(int64_t)o * parts + i];
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
-  if (lane == 0) ep.store(o / N, o % N, s);
+  if (o < outs)
+    for (int i = pl; i < parts; i += 64) s += partial[(int64_t)i * outs + o];
+  sm[pl][ol] = s;
+  __syncthreads();
+  if (threadIdx.x < 4 && o < outs) {
+    float t = 0.f;
+#pragma unroll 8
+    for (int j = 0; j < 64; ++j) t += sm[j][ol];
+    ep.store(o / N, o % N, t);
+  }
 }
 
 static int small_parts(int m, int n, int k, int cu, int64_t ws_elems) {
@@ -1207,8 +1214,131 @@ int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const flo
   return launch_any<false>(ctx, "conv2d_input_gradient", M, N, K, al, bl, ep, ws, ws_elems);
 }
 
+// Filter gradient of a first-layer convolution (a few input channels, at most 64 filters): M = kh*kw*cin is a few
+// dozen rows, N = cout a few dozen columns and K = every output position of the batch, so the work is reading dy
+// once.  Direct form: a workgroup takes a band of output rows of one image, keeps the input rows under it in LDS
+// (zero-padded, so taps need no bounds checks), a group of `1 << cshift` >= cout lanes owns one output position at a
+// time, each lane one filter, and keeps all M sums of that filter in registers.  The lanes' sums meet in LDS and
+// leave as one partial [M][cout] per workgroup; gemm_small_reduce_kernel adds the partials in a fixed order.
+constexpr int WGRAD_DIRECT_MAX_TAPS = 36;
+
+template <int MT>  // upper bound of kh*kw*cin
+__global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ dy,
+                                                                 float* __restrict__ partial, int rows_per_band, int bands_per_image,
+                                                                 int items, int lw, int cshift, int staged_full) {
+  extern __shared__ float wg_lds[];
+  const int tid = threadIdx.x;
+  const int M = g.kh * g.kw * g.cin;
+  const int row_elems = lw * g.cin;
+  int off[MT];  // LDS offset of tap m = (r, q, ci) from a position's top-left input element
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int mm = m < M ? m : 0;
+    const int ci = mm % g.cin, rq = mm / g.cin;
+    off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
+  }
+  float acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+  const int lanes = 1 << cshift;
+  const int c = tid & (lanes - 1);
+  const int slot = tid >> cshift, slots = 256 >> cshift;
+  const bool live = c < g.cout;
+  const int cc = live ? c : 0;
+  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+    const int b = item / bands_per_image, band = item % bands_per_image;
+    const int oh0 = band * rows_per_band;
+    const int oh1 = oh0 + rows_per_band < g.ho ? oh0 + rows_per_band : g.ho;
+    const int iy0 = oh0 * g.sh - g.pt;
+    const int staged = ((oh1 - oh0 - 1) * g.sh + g.kh) * row_elems;
+    const int P = (oh1 - oh0) * g.wo;
+    const float* dyb = dy + ((int64_t)b * g.ho + oh0) * g.wo * g.cout;
+    constexpr int U = 16;  // positions per lane whose dy loads are in flight together
+    int* origin = reinterpret_cast<int*>(wg_lds + staged_full);  // per position of the band: LDS offset of its top-left input element
+    __syncthreads();  // the previous item's readers are done with the staged rows
+    for (int e = tid; e < staged; e += 256) {
+      const int row = e / row_elems, rem = e % row_elems;
+      const int iy = iy0 + row, ix = rem / g.cin - g.pl, ci = rem % g.cin;
+      wg_lds[e] = ((unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w) ? x[(((int64_t)b * g.h + iy) * g.w + ix) * g.cin + ci] : 0.f;
+    }
+    for (int p = tid; p < P; p += 256) origin[p] = (p / g.wo) * g.sh * row_elems + (p % g.wo) * g.sw * g.cin;  // one division per position, not per lane
+    __syncthreads();
+    for (int p0 = slot; p0 < P; p0 += slots * U) {
+      float d[U];
+      int base[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int p = p0 + u * slots;
+        const bool in = p < P;
+        const int pp = in ? p : 0;
+        const float v = dyb[(int64_t)pp * g.cout + cc];  // always a valid address: no branch around the load
+        d[u] = (in && live) ? v : 0.f;
+        base[u] = origin[pp];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)  // rows m >= M repeat tap 0 and are dropped at the end: no branch between the LDS reads
+          acc[m] = __builtin_fmaf(wg_lds[base[u] + off[m]], d[u], acc[m]);
+      }
+    }
+  }
+  __syncthreads();
+  // [slot][m][lane] -> one sum per (m, filter), slots added in order
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+    if (m < M) wg_lds[(slot * M + m) * lanes + c] = acc[m];
+  __syncthreads();
+  const int outs = M * g.cout;
+  for (int o = tid; o < outs; o += 256) {
+    const int m = o / g.cout, co = o % g.cout;
+    float t = 0.f;
+    for (int sl = 0; sl < slots; ++sl) t += wg_lds[(sl * M + m) * lanes + co];
+    partial[(int64_t)blockIdx.x * outs + o] = t;
+  }
+}
+
+static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems, int* rc) {
+  const int M = g.kh * g.kw * g.cin, N = g.cout;
+  const int64_t K = (int64_t)g.n * g.ho * g.wo;
+  if (!ws || g.cin > 4 || M > WGRAD_DIRECT_MAX_TAPS || N > 64 || K < SMALL_MIN_K) return false;
+  const int64_t room = std::min<int64_t>((int64_t)4 * ctx->compute_units, ws_elems / ((int64_t)M * N));
+  if (room < 32) return false;
+  int cshift = 0;
+  while ((1 << cshift) < N) ++cshift;
+  const int lw = (g.wo - 1) * g.sw + g.kw;
+  int rows_per_band = (int)std::min<int64_t>(g.ho, std::max<int64_t>(1, ceil_div((int64_t)g.n * g.ho, room)));
+  const int bands = (int)ceil_div((int64_t)g.ho, (int64_t)rows_per_band);
+  const int64_t items = (int64_t)g.n * bands;
+  const int64_t staged = (int64_t)((rows_per_band - 1) * g.sh + g.kh) * lw * g.cin;
+  const int64_t lds_floats = std::max<int64_t>(staged + (int64_t)rows_per_band * g.wo, (int64_t)256 * M);
+  if (lds_floats * 4 > 48 * 1024 || items >= (int64_t)1 << 30) return false;
+  const int parts = (int)std::min<int64_t>(items, room);
+  {
+    LaunchScope scope(ctx, "conv2d_filter_gradient_direct", M, N, (int)K);
+#define SN_WGRAD_DIRECT(MT)                                                                                                        \
+  hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float), ctx->stream, g, \
+                     x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged)
+    if (M <= 9) SN_WGRAD_DIRECT(9);
+    else if (M <= 18) SN_WGRAD_DIRECT(18);
+    else SN_WGRAD_DIRECT(36);
+#undef SN_WGRAD_DIRECT
+  }
+  Epilogue e;
+  e.out = dw;
+  e.ldo = g.cout;
+  StdEpilogue ep{e};
+  LaunchScope scope(ctx, "small_output_reduce");
+  hipLaunchKernelGGL((gemm_small_reduce_kernel<StdEpilogue>), dim3((unsigned)ceil_div(M * N, 4)), dim3(256), 0, ctx->stream, (const float*)ws,
+                     parts, M, N, ep);
+  *rc = hipGetLastError() == hipSuccess ? SN_OK : fail(SN_E_HIP, "conv2d_filter_gradient_direct: launch failed");
+  return true;
+}
+
 int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems) {
   const int M = g.kh * g.kw * g.cin, N = g.cout, K = g.n * g.ho * g.wo;
+  int rc = SN_OK;
+  if (conv_wgrad_direct(ctx, g, x, dy, dw, ws, ws_elems, &rc)) return rc;
   if (!(ws && small_parts(M, N, K, ctx->compute_units, ws_elems)) && WgradXLoader::ok(x, g) && FlatLoader<false>::ok(dy, 1, g.cout, N, K)) {
     const int interior = g.pt == 0 && g.pl == 0 && (g.ho - 1) * g.sh + g.kh <= g.h && (g.wo - 1) * g.sw + g.kw <= g.w;
     WgradXLoader al{x, g, M, interior};

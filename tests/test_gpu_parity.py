@@ -422,6 +422,11 @@ MODELS = {
                                   "cce", (20, 20, 4), 104, "uniform_onehot"),
     "conv_many_positions_stride2": ([("conv", 12, (3, 3), (2, 2), "valid", "relu", False), ("flatten",), ("dense", 3, "softmax")],
                                 "cce", (40, 40, 4), 100, "uniform_onehot"),
+    # first-layer filter gradient in its direct form with an uneven kernel, strides, Same padding and a filter count that is no power of two
+    "conv_first_layer_uneven": ([("conv", 5, (3, 2), (2, 1), "same", "tanh", True), ("flatten",), ("dense", 3, "softmax")],
+                                "cce", (18, 17, 3), 30, "uniform_onehot"),
+    "conv_first_layer_5x5": ([("conv", 6, (5, 5), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 4, "softmax")],
+                             "cce", (16, 16, 1), 40, "uniform_onehot"),
     # BatchNorm reductions: 200 channels take the row-walking form with four column blocks, 256 the float4 stream form
     "batchnorm_200_channels": ([("dense", 200, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
     "batchnorm_256_channels": ([("dense", 256, "relu"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
