@@ -228,6 +228,17 @@ struct GemmDesc {
 // true when launch_gemm would take its 16-byte loaders for this problem (they have no all-ones row)
 bool gemm_takes_fast_loaders(const sn_ctx* ctx, const GemmDesc& g, const float* workspace, int64_t workspace_elems);
 int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* workspace, int64_t workspace_elems, bool bf16);
+// Gradients of a Dense layer from many features onto at most 16 units, as row streams over X (fp32, contiguous
+// [rows, in_f] / [in_f, out_f] / [rows, out_f] tensors); dense_skinny_shape says whether a shape is in their range.
+bool dense_skinny_shape(int rows, int in_f, int out_f);
+int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f);
+int launch_dense_skinny_dx(sn_ctx* ctx, const float* dy, const float* w, float* dx, int rows, int in_f, int out_f);
+// The same layer forward for small batches (partial sums per feature chunk in the workspace, then a fixed-order reduction
+// that applies e's bias and activation); dense_skinny_fwd_shape says whether shape and workspace are in its range.
+bool dense_skinny_fwd_shape(int rows, int in_f, int out_f, int64_t ws_elems);
+int64_t dense_skinny_fwd_workspace(int rows, int in_f, int out_f);  // floats of workspace the forward form needs
+int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,
+                            int64_t ws_elems);
 
 // bf16 fast path (gemm_bf16.hip): C[M,N] = A[M,K] * Bt[N,K]^T, operands bf16 with k contiguous.
 // Besides the fp32 result (e.out, may be null) the epilogue can emit bf16 copies in both orientations,

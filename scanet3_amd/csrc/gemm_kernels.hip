@@ -852,7 +852,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     float s = 0.f;
     if (i < total) {
       int z = g;
-      for (; z + 24 < splits; z += 32) {  // 4 loads in flight, added in split order
+      for (; z + 120 < splits; z += 128) {  // 16 loads in flight, added in split order
+        float a[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) a[u] = ws[(int64_t)(z + 8 * u) * total + i];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) s += a[u];
+      }
+      for (; z + 24 < splits; z += 32) {  // 4 loads in flight
         float a[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) a[u] = ws[(int64_t)(z + 8 * u) * total + i];
@@ -959,8 +966,15 @@ __global__ __launch_bounds__(256) void gemm_small_reduce_kernel(const float* __r
   const int ol = threadIdx.x & 3, pl = threadIdx.x >> 2;
   const int o = blockIdx.x * 4 + ol;
   float s = 0.f;
-  if (o < outs)
-    for (int i = pl; i < parts; i += 64) s += partial[(int64_t)i * outs + o];
+  if (o < outs) {
+    for (int i = pl; i < parts; i += 64 * 8) {  // 8 loads in flight, added in part order
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = i + 64 * u < parts ? partial[(int64_t)(i + 64 * u) * outs + o] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+  }
   sm[pl][ol] = s;
   __syncthreads();
   if (threadIdx.x < 4 && o < outs) {
@@ -1176,8 +1190,121 @@ __global__ __launch_bounds__(256) void conv_direct_fwd_kernel(ConvGeom g, const 
   }
 }
 
+// U pixels of one lane (p0, p0 + slots, ...; all inside the band): taps outermost, so a tap's weights are used U times.
+template <int MT, int U>
+__device__ __forceinline__ void fwd_rows_pixels(const float* lds, const int* origin, const int (&off)[MT], const f4v (&wr)[MT], const f4v& bias,
+                                                const Epilogue& e, float* outb, int p0, int slots) {
+  f4v acc[U];
+  int base[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    base[u] = origin[p0 + u * slots];
+    acc[u] = f4v{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float xv = lds[base[u] + off[m]];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[u][i] = __builtin_fmaf(xv, wr[m][i], acc[u][i]);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    f4v out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = ep_act(e.act, acc[u][i] + bias[i], e.act_param);
+    *(f4v*)(outb + (int64_t)(p0 + u * slots) * e.ldo) = out;
+  }
+}
+
+// The same layer when the filter count is 4 << j (j = 0..6) and there are at most 18 taps: a workgroup takes a band of
+// output rows of one image and keeps the input rows under it in LDS, zero-padded; a lane owns 4 filters, holds their
+// weights for every tap in registers and walks pixels, so a pixel costs its taps' LDS reads (shared by the lanes of the
+// pixel) and 4 FMAs per tap; the pixel's channels leave as one contiguous run.  Same (r, q, ci) accumulation order.
+// Rows m >= taps of the register arrays carry zero weights (they re-read tap 0), so the tap loop has no branch.
+template <int MT>
+__global__ __launch_bounds__(256) void conv_direct_fwd_rows_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ w,
+                                                                    Epilogue e, int rows_per_band, int bands_per_image, int items, int lw,
+                                                                    int qshift, int staged_full) {
+  extern __shared__ float fw_lds[];
+  const int tid = threadIdx.x;
+  const int M = g.kh * g.kw * g.cin;
+  const int row_elems = lw * g.cin;
+  const int quads = 1 << qshift;
+  const int col = (tid & (quads - 1)) * 4;
+  const int slot = tid >> qshift, slots = 256 >> qshift;
+  f4v wr[MT];
+  int off[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int mm = m < M ? m : 0;
+    const int ci = mm % g.cin, rq = mm / g.cin;
+    off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
+    const f4v zero = {0.f, 0.f, 0.f, 0.f};
+    wr[m] = m < M ? *(const f4v*)(w + (int64_t)m * g.cout + col) : zero;
+  }
+  f4v bias = {0.f, 0.f, 0.f, 0.f};
+  if (e.bias) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bias[i] = e.bias[col + i];
+  }
+  int* origin = reinterpret_cast<int*>(fw_lds + staged_full);
+  constexpr int U = 4;  // pixels per lane in flight
+  for (int item = blockIdx.x; item < items; item += gridDim.x) {
+    const int b = item / bands_per_image, band = item % bands_per_image;
+    const int oh0 = band * rows_per_band;
+    const int oh1 = oh0 + rows_per_band < g.ho ? oh0 + rows_per_band : g.ho;
+    const int iy0 = oh0 * g.sh - g.pt;
+    const int staged = ((oh1 - oh0 - 1) * g.sh + g.kh) * row_elems;
+    const int P = (oh1 - oh0) * g.wo;
+    __syncthreads();  // the previous item's readers are done with the staged rows
+    for (int el = tid; el < staged; el += 256) {
+      const int row = el / row_elems, rem = el % row_elems;
+      const int iy = iy0 + row, ix = rem / g.cin - g.pl, ci = rem % g.cin;
+      fw_lds[el] = ((unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w) ? x[(((int64_t)b * g.h + iy) * g.w + ix) * g.cin + ci] : 0.f;
+    }
+    for (int p = tid; p < P; p += 256) origin[p] = (p / g.wo) * g.sh * row_elems + (p % g.wo) * g.sw * g.cin;
+    __syncthreads();
+    float* outb = e.out + (((int64_t)b * g.ho + oh0) * g.wo) * e.ldo + col;
+    int p0 = slot;
+    for (; p0 + (U - 1) * slots < P; p0 += slots * U) fwd_rows_pixels<MT, U>(fw_lds, origin, off, wr, bias, e, outb, p0, slots);
+    for (; p0 < P; p0 += slots) fwd_rows_pixels<MT, 1>(fw_lds, origin, off, wr, bias, e, outb, p0, slots);
+  }
+}
+
+static bool conv_fwd_rows(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e, int* rc) {
+  const int N = g.cout, K = g.kh * g.kw * g.cin;
+  const int64_t pixels = (int64_t)g.n * g.ho * g.wo;
+  if (g.cin > 4 || K > 18 || N % 4 != 0 || N > 256 || ((N / 4) & (N / 4 - 1)) != 0 || pixels < 2048) return false;
+  if (e.ldo % 4 != 0 || !aligned16(e.out) || !aligned16(w)) return false;
+  int qshift = 0;
+  while ((4 << qshift) < N) ++qshift;
+  const int lw = (g.wo - 1) * g.sw + g.kw;
+  // a band holds at least ~4 pixels per lane, so staging its input rows is a small part of the work
+  const int rows_per_band = (int)std::min<int64_t>(g.ho, std::max<int64_t>(1, ceil_div((int64_t)1024, (int64_t)(N / 4) * g.wo)));
+  const int bands = (int)ceil_div((int64_t)g.ho, (int64_t)rows_per_band);
+  const int64_t items = (int64_t)g.n * bands;
+  const int64_t staged = (int64_t)((rows_per_band - 1) * g.sh + g.kh) * lw * g.cin;
+  const int64_t lds_floats = staged + (int64_t)rows_per_band * g.wo;
+  if (lds_floats * 4 > 48 * 1024 || items >= (int64_t)1 << 30) return false;
+  const unsigned blocks = (unsigned)std::min<int64_t>(items, (int64_t)ctx->compute_units * 8);
+  LaunchScope scope(ctx, "conv2d_forward_direct", (int)pixels, N, K);
+#define SN_FWD_ROWS(MT)                                                                                                                  \
+  hipLaunchKernelGGL((conv_direct_fwd_rows_kernel<MT>), dim3(blocks), dim3(256), (size_t)lds_floats * sizeof(float), ctx->stream, g, x, w, e, \
+                     rows_per_band, bands, (int)items, lw, qshift, (int)staged)
+  if (K <= 9) SN_FWD_ROWS(9);
+  else SN_FWD_ROWS(18);
+#undef SN_FWD_ROWS
+  *rc = hipGetLastError() == hipSuccess ? SN_OK : fail(SN_E_HIP, "conv2d_forward_direct: launch failed");
+  return true;
+}
+
 int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e, float* ws, int64_t ws_elems) {
   const int M = g.n * g.ho * g.wo, N = g.cout, K = g.kh * g.kw * g.cin;
+  int rows_rc = SN_OK;
+  if (conv_fwd_rows(ctx, g, x, w, e, &rows_rc)) return rows_rc;
   if (g.cin <= 4 && K <= DIRECT_MAX_K && N % 4 == 0 && (size_t)K * N * sizeof(float) <= 48 * 1024 && e.ldo % 4 == 0 && aligned16(e.out) && M > 0) {
     const int64_t total = (int64_t)M * (N / 4);
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div(total, 256), (int64_t)ctx->compute_units * 32);
@@ -1394,6 +1521,314 @@ int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, cons
   StridedLoader<false> bl{dz_all, 1, (int64_t)gates * H, gates * H};
   LstmWgradEpilogue ep{g, F, H};
   return launch_any<false>(ctx, "lstm_weight_gradient", M, gates * H, T * rows, al, bl, ep, ws, ws_elems);
+}
+
+// ============================================================================ Dense onto a few units: backward
+// A Dense layer from tens of thousands of features onto at most 16 units (a classifier head behind Flatten) with a
+// batch of a few hundred rows: its gradients are memory-bound streams over X, not matrix-core work.  A workgroup of
+// 4 wavefronts owns 64 consecutive features; wavefront w takes every row b with b / rows_per_wave == w, a lane one
+// feature, so every load or store of a wavefront is one contiguous 256-byte run of a row of X (or dX).  dY sits in LDS
+// as [rows + 1][4 NQ] floats (units padded with zeros, one all-zero row for out-of-range rows) and is read as broadcasts.
+constexpr int SKINNY_MAX_UNITS = 16, SKINNY_MIN_FEATURES = 2048, SKINNY_MAX_LDS_FLOATS = 8192, SKINNY_ROWS_IN_FLIGHT = 32;
+
+template <int NQ>
+__device__ __forceinline__ void skinny_stage_dy(f4v* dyl, const float* __restrict__ dy, int rows, int out_f) {
+  float* flat = reinterpret_cast<float*>(dyl);
+  constexpr int padded = NQ * 4;
+  const int total = (rows + 1) * padded;
+  for (int base = 0; base < total; base += 256 * 8) {  // 8 loads per thread are issued before any of them is stored
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = base + u * 256 + (int)threadIdx.x;
+      const int b = e / padded, n = e % padded;
+      v[u] = (b < rows && n < out_f) ? dy[(int64_t)b * out_f + n] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = base + u * 256 + (int)threadIdx.x;
+      if (e < total) flat[e] = v[u];
+    }
+  }
+}
+
+// dW[i, n] = sum_b X[b, i] dY[b, n] (math/alg/AllKernels.scala:382-388, the left operand's gradient of a matrix product
+// seen from the weights), db[n] = sum_b dY[b, n].  The four wavefronts' partial sums meet in LDS and are added in wavefront order.
+template <int NQ>
+__global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dw,
+                                                               float* __restrict__ db, int rows, int in_f, int out_f, int rows_per_wave) {
+  extern __shared__ f4v skinny_lds[];
+  f4v* dyl = skinny_lds;                         // [rows + 1][NQ]
+  f4v* part = skinny_lds + (rows + 1) * NQ;      // [3][NQ][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  const bool live = i < in_f;
+  const float* xp = x + (live ? i : 0);
+  const int b0 = wave * rows_per_wave;
+  const int b1 = b0 + rows_per_wave < rows ? b0 + rows_per_wave : rows;
+  constexpr int U = SKINNY_ROWS_IN_FLIGHT;
+  float xv[U];
+  // the first batch of X is on its way while dY is staged
+#pragma unroll
+  for (int u = 0; u < U; ++u) xv[u] = b0 + u < b1 ? xp[(int64_t)(b0 + u) * in_f] : 0.f;
+  skinny_stage_dy<NQ>(dyl, dy, rows, out_f);
+  __syncthreads();
+  f4v acc[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) acc[q] = f4v{0.f, 0.f, 0.f, 0.f};
+  for (int b = b0; b < b1; b += U) {
+    if (b != b0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) xv[u] = b + u < b1 ? xp[(int64_t)(b + u) * in_f] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = b + u < b1 ? b + u : rows;  // the all-zero row
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const f4v d = dyl[row * NQ + q];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[q][k] = __builtin_fmaf(xv[u], d[k], acc[q][k]);
+      }
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) part[((wave - 1) * NQ + q) * 64 + lane] = acc[q];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        const f4v p = part[(w * NQ + q) * 64 + lane];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[q][k] = acc[q][k] + p[k];
+      }
+    }
+    if (live) {
+      float* o = dw + (int64_t)i * out_f;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (q * 4 + k < out_f) o[q * 4 + k] = acc[q][k];
+      }
+    }
+  } else if (wave == 1 && blockIdx.x == 0 && db && lane < out_f) {
+    const float* flat = reinterpret_cast<const float*>(dyl);
+    float s = 0.f;
+    for (int b = 0; b < rows; ++b) s += flat[b * NQ * 4 + lane];
+    db[lane] = s;
+  }
+}
+
+// dX[b, i] = sum_n dY[b, n] W[i, n] (AllKernels.scala:382-388, the right operand's side): a lane keeps its feature's
+// weight row in registers and walks its wavefront's rows.
+template <int NQ>
+__global__ __launch_bounds__(256) void dense_skinny_dx_kernel(const float* __restrict__ dy, const float* __restrict__ w, float* __restrict__ dx,
+                                                               int rows, int in_f, int out_f, int rows_per_wave) {
+  extern __shared__ f4v skinny_lds[];
+  f4v* dyl = skinny_lds;
+  skinny_stage_dy<NQ>(dyl, dy, rows, out_f);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  const bool live = i < in_f;
+  f4v wr[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) wr[q][k] = (live && q * 4 + k < out_f) ? w[(int64_t)i * out_f + q * 4 + k] : 0.f;
+  }
+  __syncthreads();
+  const int b0 = wave * rows_per_wave;
+  const int b1 = b0 + rows_per_wave < rows ? b0 + rows_per_wave : rows;
+  if (!live) return;
+  float* o = dx + i;
+#pragma unroll 4
+  for (int b = b0; b < b1; ++b) {
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const f4v d = dyl[b * NQ + q];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) s = __builtin_fmaf(d[k], wr[q][k], s);
+    }
+    o[(int64_t)b * in_f] = s;
+  }
+}
+
+bool dense_skinny_shape(int rows, int in_f, int out_f) {
+  const int nq = (out_f + 3) / 4;
+  return rows >= 4 && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES && (int64_t)(rows + 1) * nq * 4 <= SKINNY_MAX_LDS_FLOATS;
+}
+
+int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f) {
+  SN_REQUIRE(dense_skinny_shape(rows, in_f, out_f), "dense_weight_gradient_rows: shape outside the kernel's range");
+  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, 4);
+  const unsigned blocks = (unsigned)ceil_div(in_f, 64);
+  const size_t lds = ((size_t)(rows + 1) * nq + (size_t)3 * nq * 64) * sizeof(f4v);
+  LaunchScope scope(ctx, "dense_weight_gradient_rows", in_f, out_f, rows);
+#define SN_SKINNY_DW(NQ) \
+  hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ>), dim3(blocks), dim3(256), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f, rows_per_wave)
+  switch (nq) {
+    case 1: SN_SKINNY_DW(1); break;
+    case 2: SN_SKINNY_DW(2); break;
+    case 3: SN_SKINNY_DW(3); break;
+    default: SN_SKINNY_DW(4); break;
+  }
+#undef SN_SKINNY_DW
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_dense_skinny_dx(sn_ctx* ctx, const float* dy, const float* w, float* dx, int rows, int in_f, int out_f) {
+  SN_REQUIRE(dense_skinny_shape(rows, in_f, out_f), "dense_input_gradient_rows: shape outside the kernel's range");
+  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, 4);
+  const unsigned blocks = (unsigned)ceil_div(in_f, 64);
+  const size_t lds = (size_t)(rows + 1) * nq * sizeof(f4v);
+  LaunchScope scope(ctx, "dense_input_gradient_rows", rows, in_f, out_f);
+#define SN_SKINNY_DX(NQ) \
+  hipLaunchKernelGGL((dense_skinny_dx_kernel<NQ>), dim3(blocks), dim3(256), lds, ctx->stream, dy, w, dx, rows, in_f, out_f, rows_per_wave)
+  switch (nq) {
+    case 1: SN_SKINNY_DX(1); break;
+    case 2: SN_SKINNY_DX(2); break;
+    case 3: SN_SKINNY_DX(3); break;
+    default: SN_SKINNY_DX(4); break;
+  }
+#undef SN_SKINNY_DX
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+// The same layer forward for a batch of at most SKINNY_FWD_MAX_ROWS rows: Y = X W is 4 B of X per 2 out_f flops.  A workgroup
+// owns SKINNY_FWD_CHUNK consecutive features: its wavefronts fetch their rows of that chunk in one go (a lane takes two
+// neighbouring features, so a wavefront reads 512 contiguous bytes per row, all rows in flight), the chunk turns in
+// LDS ([row][129]: rows on different banks), then thread (row pair, unit quad) adds its 128 products per output in feature order and the
+// workgroup leaves one partial [rows][out_f]; gemm_small_reduce_kernel adds the partials in a fixed order and applies the
+// bias and the activation.
+constexpr int SKINNY_FWD_CHUNK = 128, SKINNY_FWD_MAX_ROWS = 112, SKINNY_FWD_ROWS_PER_WAVE = SKINNY_FWD_MAX_ROWS / 4;
+
+template <int NQ>
+__global__ __launch_bounds__(256) void dense_skinny_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ partial,
+                                                                int rows, int in_f, int out_f) {
+  constexpr int KC = SKINNY_FWD_CHUNK, PITCH = KC + 1, R = SKINNY_FWD_ROWS_PER_WAVE;
+  extern __shared__ __attribute__((aligned(16))) float skinny_fwd_lds[];
+  float* xs = skinny_fwd_lds;                                  // [rows][PITCH]
+  f4v* wsm = reinterpret_cast<f4v*>(skinny_fwd_lds + ((rows * PITCH + 3) & ~3));  // [KC][NQ]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i0 = blockIdx.x * KC;
+  const int fa = i0 + 2 * lane;  // this lane's two features
+  // whole chunks of rows that start on 8-byte boundaries take 8-byte loads without a branch (rows past the batch re-read the last row)
+  const bool whole = i0 + KC <= in_f && (in_f & 1) == 0 && (reinterpret_cast<uintptr_t>(x) & 7) == 0;
+  float2 xv[R];
+  if (whole) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int b = wave + 4 * u < rows ? wave + 4 * u : rows - 1;
+      xv[u] = *reinterpret_cast<const float2*>(x + (int64_t)b * in_f + fa);
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int b = wave + 4 * u < rows ? wave + 4 * u : rows - 1;
+      const float* rp = x + (int64_t)b * in_f;
+      xv[u].x = fa < in_f ? rp[fa] : 0.f;
+      xv[u].y = fa + 1 < in_f ? rp[fa + 1] : 0.f;
+    }
+  }
+  {  // the chunk's weight rows, units padded to quads with zeros; features past in_f are zero rows
+    float* wflat = reinterpret_cast<float*>(wsm);
+    constexpr int total = KC * NQ * 4;
+    for (int base = 0; base < total; base += 256 * 8) {  // 8 loads per thread are issued before any of them is stored
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = base + u * 256 + (int)threadIdx.x;
+        const int k = e / (NQ * 4), n = e % (NQ * 4);
+        v[u] = (e < total && i0 + k < in_f && n < out_f) ? w[(int64_t)(i0 + k) * out_f + n] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int e = base + u * 256 + (int)threadIdx.x;
+        if (e < total) wflat[e] = v[u];
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < R; ++u) {
+    const int b = wave + 4 * u;
+    if (b < rows) {
+      xs[b * PITCH + 2 * lane] = xv[u].x;
+      xs[b * PITCH + 2 * lane + 1] = xv[u].y;
+    }
+  }
+  __syncthreads();
+  // thread (row pair, unit quad): a weight quad read from LDS serves both rows; at most 56 pairs x 4 quads = 224 threads
+  float* out = partial + (int64_t)blockIdx.x * rows * out_f;
+  const int item = threadIdx.x;
+  if (item < ((rows + 1) / 2) * NQ) {
+    const int b = (item / NQ) * 2, q = item % NQ;
+    const bool second = b + 1 < rows;
+    const float* xr0 = xs + b * PITCH;
+    const float* xr1 = xs + (second ? b + 1 : b) * PITCH;
+    f4v acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 16
+    for (int k = 0; k < KC; ++k) {
+      const float x0 = xr0[k], x1 = xr1[k];
+      const f4v wk = wsm[k * NQ + q];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        acc0[c] = __builtin_fmaf(x0, wk[c], acc0[c]);
+        acc1[c] = __builtin_fmaf(x1, wk[c], acc1[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (q * 4 + c < out_f) {
+        out[b * out_f + q * 4 + c] = acc0[c];
+        if (second) out[(b + 1) * out_f + q * 4 + c] = acc1[c];
+      }
+    }
+  }
+}
+
+int64_t dense_skinny_fwd_workspace(int rows, int in_f, int out_f) { return ceil_div(in_f, SKINNY_FWD_CHUNK) * rows * out_f; }
+
+static size_t skinny_fwd_lds_bytes(int rows, int out_f) {
+  return ((size_t)((rows * (SKINNY_FWD_CHUNK + 1) + 3) & ~3) + (size_t)SKINNY_FWD_CHUNK * ((out_f + 3) / 4) * 4) * sizeof(float);
+}
+
+bool dense_skinny_fwd_shape(int rows, int in_f, int out_f, int64_t ws_elems) {
+  return rows >= 1 && rows <= SKINNY_FWD_MAX_ROWS && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES &&
+         skinny_fwd_lds_bytes(rows, out_f) <= 64 * 1024 && dense_skinny_fwd_workspace(rows, in_f, out_f) <= ws_elems;
+}
+
+int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,
+                            int64_t ws_elems) {
+  SN_REQUIRE(ws && dense_skinny_fwd_shape(rows, in_f, out_f, ws_elems), "dense_forward_rows: shape outside the kernel's range");
+  const int nq = (out_f + 3) / 4;
+  const int parts = (int)ceil_div(in_f, SKINNY_FWD_CHUNK);
+  const size_t lds = skinny_fwd_lds_bytes(rows, out_f);
+  {
+    LaunchScope scope(ctx, "dense_forward_rows", rows, out_f, in_f);
+#define SN_SKINNY_FWD(NQ) \
+  hipLaunchKernelGGL((dense_skinny_fwd_kernel<NQ>), dim3((unsigned)parts), dim3(256), lds, ctx->stream, x, w, ws, rows, in_f, out_f)
+    switch (nq) {
+      case 1: SN_SKINNY_FWD(1); break;
+      case 2: SN_SKINNY_FWD(2); break;
+      case 3: SN_SKINNY_FWD(3); break;
+      default: SN_SKINNY_FWD(4); break;
+    }
+#undef SN_SKINNY_FWD
+  }
+  StdEpilogue ep{e};
+  LaunchScope scope(ctx, "small_output_reduce");
+  hipLaunchKernelGGL((gemm_small_reduce_kernel<StdEpilogue>), dim3((unsigned)ceil_div(rows * out_f, 4)), dim3(256), 0, ctx->stream,
+                     (const float*)ws, parts, rows, out_f, ep);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
 }
 
 }  // namespace sn

@@ -192,6 +192,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         }
         const int in_f = (int)cur[0], out_f = L.units;
         ws = std::max(ws, gemm_workspace_elems(B, out_f, in_f, cu));
+        if (dense_skinny_fwd_shape(B, in_f, out_f, INT64_MAX)) ws = std::max(ws, dense_skinny_fwd_workspace(B, in_f, out_f));
         ws = std::max(ws, gemm_workspace_elems(in_f + 1, out_f, B, cu));  // + the bias-gradient row
         ws = std::max(ws, gemm_workspace_elems(B, in_f, out_f, cu));
         break;
@@ -542,6 +543,8 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
             if (hidden_f32_not_needed(m, i)) eb.e.out = nullptr;  // the next layer and the backward pass read the bf16 copies
           }
           SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_x[i], in_f, r->bf_wt[i], in_f, rows, out_f, in_f, eb));
+        } else if (!bf16 && r->ws && dense_skinny_fwd_shape(rows, in_f, out_f, m->workspace_elems)) {
+          SN_TRY(launch_dense_skinny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f, r->ws, m->workspace_elems));
         } else {
           GemmDesc g{in, in_f, 1, param_ptr(r, r->w, op.w), out_f, 1, rows, out_f, in_f};
           SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
@@ -680,6 +683,14 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           break;
         }
         if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
+        if (!bf16 && dense_skinny_shape(rows, in_f, out_f)) {  // a few units behind many features: row streams, no matrix tiles
+          SN_TRY(launch_dense_skinny_dw(ctx, in, dy, param_ptr(r, r->g, op.w), param_ptr(r, r->g, op.b), rows, in_f, out_f));
+          if (need_dx) {
+            SN_TRY(launch_dense_skinny_dx(ctx, dy, param_ptr(r, r->w, op.w), dx, rows, in_f, out_f));
+            cur ^= 1;
+          }
+          break;
+        }
         {  // dW = X^T . dY (math/alg/AllKernels.scala:382-388)
           GemmDesc g{in, 1, in_f, dy, out_f, 1, in_f, out_f, rows};
           Epilogue ep;

@@ -427,6 +427,19 @@ MODELS = {
                                 "cce", (18, 17, 3), 30, "uniform_onehot"),
     "conv_first_layer_5x5": ([("conv", 6, (5, 5), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 4, "softmax")],
                              "cce", (16, 16, 1), 40, "uniform_onehot"),
+    # first-layer forward in its row-band form (at most 18 taps, 4 << j filters, >= 2048 output pixels): several bands per image with
+    # Same padding above and below, strides and a bias; and 4 filters (one lane per pixel) over 3 channels
+    "conv_first_layer_bands_same_stride": ([("conv", 64, (3, 3), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "valid"), ("flatten",),
+                                            ("dense", 3, "softmax")], "cce", (21, 19, 2), 40, "uniform_onehot"),
+    "conv_first_layer_four_filters": ([("conv", 4, (2, 2), (1, 1), "valid", "relu", False), ("flatten",), ("dense", 3, "softmax")],
+                                      "cce", (30, 30, 3), 8, "uniform_onehot"),
+    # Dense from thousands of features onto a few units: gradients as row streams (2048+ features, at most 16 units); a feature count
+    # that leaves a partial block of 64, 7 rows over 4 wavefronts, 16 and 5 units, an L2 penalty on the streamed weights
+    "dense_many_features_few_units": ([("dense", 2050, "tanh"), ("dense", 5, "softmax", "l2", 0.01)], "cce", (33,), 7, "normal_onehot"),
+    "dense_many_features_16_units": ([("dense", 4100, "relu"), ("dense", 16, "tanh"), ("dense", 2, "identity")], "mse", (21,), 130,
+                                     "normal_regression"),
+    # an odd feature count (no 8-byte loads in the forward form) and 9 units (three quads, one of them partial)
+    "dense_odd_feature_count_9_units": ([("dense", 2049, "sigmoid"), ("dense", 9, "softmax")], "cce", (12,), 33, "normal_onehot"),
     # BatchNorm reductions: 200 channels take the row-walking form with four column blocks, 256 the float4 stream form
     "batchnorm_200_channels": ([("dense", 200, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
     "batchnorm_256_channels": ([("dense", 256, "relu"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
