@@ -248,6 +248,13 @@ struct EpilogueBf16 {
   void* out_bf = nullptr;    // bf16 [M, e.ldo]
   void* out_bf_t = nullptr;  // bf16 [N, ld_t]
   int64_t ld_t = 0;
+  // Gradient hand-over to the Dense layer below (dX products only; full 128-row / 128-column tiles, out_bf_t set, e.act
+  // identity): the result is multiplied by that layer's ReLU gradient, read off the sign of its output's transposed bf16
+  // copy grad_mask_t [N, ld_t] (null: identity activation, nothing to multiply), before it is cast and stored, and
+  // col_partials [M / 64, N] (optional) receives the column sums of every 64-row block of the fp32 values.
+  bool grad_handover = false;
+  const void* grad_mask_t = nullptr;
+  float* col_partials = nullptr;
 };
 int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep);
 // bf16 copies out[rows,cols] and out_t[cols,rows] of an fp32 matrix; with y != null the activation gradient

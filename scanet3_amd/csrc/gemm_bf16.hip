@@ -73,6 +73,8 @@ __device__ __forceinline__ float bf_act_grad(int act, float y, float dy, float p
 template <int WT>
 constexpr int tr_pitch() { return WT * 2 + 8; }  // bytes per staged column
 
+constexpr int MODE_HANDOVER = 8;  // EpilogueBf16::grad_handover (full tiles only)
+
 template <int MODE, bool FULL, int TI>
 __device__ __forceinline__ void store_tile(const f16v (&acc)[TI][TI], const EpilogueBf16& ep, int mbase, int nbase, int lane, int M,
                                            int N, char* stage) {
@@ -87,10 +89,34 @@ __device__ __forceinline__ void store_tile(const f16v (&acc)[TI][TI], const Epil
   float* out = ep.e.out ? ep.e.out + origin : nullptr;
   bf16* obf = ep.out_bf ? (bf16*)ep.out_bf + origin : nullptr;
   const bool transposed = ep.out_bf_t != nullptr;
+  // Hand-over mode: the 4 rows a lane holds per (i, vq) are 8 contiguous bytes of the transposed output copy of the layer
+  // below; a column's 4 TI masks are requested one column ahead of their use (requesting the whole tile's masks up front
+  // was measured and is slower).
+  constexpr bool HAND = MODE == MODE_HANDOVER;
+  constexpr int MT = HAND ? TI : 1;
+  const bf16* ym = (HAND && ep.grad_mask_t) ? (const bf16*)ep.grad_mask_t + (int64_t)col0 * ep.ld_t + row0 : nullptr;
+  bf16x4 mk[2][MT][4];
+  if (HAND && ym) {
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) mk[0][i][vq] = *(const bf16x4*)(ym + i * 32 + vq * 8);
+    }
+  }
 #pragma unroll
   for (int j = 0; j < TI; ++j) {
     if (!FULL && col0 + j * 32 >= N) continue;
     const float bias = ep.e.bias ? ep.e.bias[col0 + j * 32] : 0.f;
+    if (HAND && ym && j + 1 < TI) {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) mk[(j + 1) & 1][i][vq] = *(const bf16x4*)(ym + (int64_t)(j + 1) * 32 * ep.ld_t + i * 32 + vq * 8);
+      }
+    }
+    float csum[(TI + 1) / 2];
+#pragma unroll
+    for (int b = 0; b < (TI + 1) / 2; ++b) csum[b] = 0.f;
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
       // keep the scheduler from hoisting every tile's loads to the top: the accumulators fill the register file
@@ -102,6 +128,10 @@ __device__ __forceinline__ void store_tile(const f16v (&acc)[TI][TI], const Epil
         for (int e = 0; e < 4; ++e) {
           const int r = i * 32 + vq * 8 + e;
           float x = acc[i][j][vq * 4 + e];
+          if (HAND) {
+            if (ym) x = (ep.e.act_param < (float)mk[j & 1][HAND ? i : 0][vq][e] ? 1.0f : 0.0f) * x;
+            csum[i / 2] += x;
+          }
           if (FULL || row0 + r < M) {
             if (ep.e.bias) x = x + bias;
             if (MODE == SN_ACT_SIGMOID) x = fast_sigmoid(x);
@@ -115,6 +145,13 @@ __device__ __forceinline__ void store_tile(const f16v (&acc)[TI][TI], const Epil
         }
         // 4 consecutive rows of one column are 8 contiguous bytes of the transposed tile
         if (transposed) *(bf16x4*)(stage + (j * 32 + l32) * PITCH + (i * 32 + vq * 8 + lhi * 4) * 2) = packed;
+      }
+    }
+    if (HAND && ep.col_partials) {  // this column's sums over the wavefront's 64-row blocks: the two half-waves hold 4 rows of every 8 each
+#pragma unroll
+      for (int b = 0; b < (TI + 1) / 2; ++b) {
+        const float t = csum[b] + __shfl_xor(csum[b], 32, 64);
+        if (lhi == 0) ep.col_partials[(int64_t)(mbase / 64 + b) * N + col0 + j * 32] = t;
       }
     }
   }
@@ -305,13 +342,13 @@ static int launch_mode(sn_ctx* ctx, const bf16* a, int64_t lda, const bf16* bt, 
     const size_t smem = 4 * 128 * tr_pitch<128>() > 4 * 256 * 128 ? 4 * 128 * tr_pitch<128>() : 4 * 256 * 128;
     SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_256<MODE>, smem));
     const int tm = (int)ceil_div(M, 256), tn = (int)ceil_div(N, 256);
-    LaunchScope scope(ctx, "gemm_bf16_256", M, N, K);
+    LaunchScope scope(ctx, MODE == MODE_HANDOVER ? "gemm_bf16_256_handover" : "gemm_bf16_256", M, N, K);
     hipLaunchKernelGGL(gemm_bf16_tn_256<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);
   } else {
     const size_t smem = 4 * 64 * tr_pitch<64>() > 4 * 128 * 128 ? 4 * 64 * tr_pitch<64>() : 4 * 128 * 128;
     SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_128<MODE>, smem));
     const int tm = (int)ceil_div(M, 128), tn = (int)ceil_div(N, 128);
-    LaunchScope scope(ctx, "gemm_bf16_128", M, N, K);
+    LaunchScope scope(ctx, MODE == MODE_HANDOVER ? "gemm_bf16_128_handover" : "gemm_bf16_128", M, N, K);
     hipLaunchKernelGGL(gemm_bf16_tn_128<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);
   }
   SN_HIP(hipGetLastError());
@@ -328,6 +365,11 @@ int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt,
   if (M <= 0 || N <= 0) return SN_OK;
   const bf16* A = (const bf16*)a;
   const bf16* B = (const bf16*)bt;
+  if (ep.grad_handover) {
+    SN_REQUIRE(M % 128 == 0 && N % 128 == 0 && ep.out_bf_t && ep.e.act == SN_ACT_IDENTITY && !ep.e.bias && ep.ld_t % 4 == 0,
+               "gemm_bf16: the gradient hand-over needs full 128 x 128 tiles, a transposed output and a plain product (got %d x %d)", M, N);
+    return launch_mode<MODE_HANDOVER>(ctx, A, lda, B, ldb, M, N, K, ep);
+  }
   switch (ep.e.act) {
     case SN_ACT_SIGMOID: return launch_mode<SN_ACT_SIGMOID>(ctx, A, lda, B, ldb, M, N, K, ep);
     case SN_ACT_TANH: return launch_mode<SN_ACT_TANH>(ctx, A, lda, B, ldb, M, N, K, ep);

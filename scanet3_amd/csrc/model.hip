@@ -652,6 +652,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
   if (first < 0) first = (int)m->ops.size() - 1;
   bool act_grad_done = false;  // the op above already applied this op's activation gradient
+  bool dz_handed_over = false;  // the bf16 Dense op above already wrote this op's dZ copies and bias-gradient block sums
   for (int i = first; i >= 0; --i) {  // grad_buf[cur] holds d loss / d (output of op i)
     const Op& op = m->ops[i];
     const float* in = op_output(r, i - 1, x, rows);
@@ -665,10 +666,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           // one pass: dZ = act'(Y) * dY in fp32 (bias gradient) and as bf16 in both orientations
           // (the fp32 dZ itself is not kept: its only other reader would be the bias gradient, summed here per 64-row block)
           const bool y_from_bf = hidden_f32_not_needed(m, (size_t)i);
-          SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
-                                       op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
-                                       op.b >= 0 ? r->bf_colp : nullptr,
-                                       op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
+          if (!dz_handed_over)
+            SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
+                                         op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
+                                         op.b >= 0 ? r->bf_colp : nullptr,
+                                         op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
+          dz_handed_over = false;
           if (op.b >= 0)
             SN_TRY(launch_col_sum(ctx, r->bf_colp, out_f, param_ptr(r, r->g, op.b), ceil_div(rows, 64), out_f, r->ws, m->workspace_elems));
           EpilogueBf16 ew;
@@ -677,6 +680,21 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           if (need_dx) {
             EpilogueBf16 ex;
             ex.e.out = dx; ex.e.ldo = in_f;
+            // A bf16 Dense layer below whose output only lives as bf16 copies (ReLU or no activation) takes its dZ straight
+            // from this product's epilogue: activation gradient, both bf16 orientations and the bias gradient's block sums,
+            // instead of an fp32 dX that a second kernel would read back, mask and cast.
+            if (hidden_f32_not_needed(m, (size_t)i - 1) && rows % 128 == 0 && in_f % 128 == 0) {
+              const Op& below = m->ops[i - 1];
+              ex.e.out = nullptr;
+              ex.out_bf = r->bf_dz[i - 1];
+              ex.out_bf_t = r->bf_dzt[i - 1];
+              ex.ld_t = rows;
+              ex.grad_handover = true;
+              ex.grad_mask_t = below.act == SN_ACT_RELU ? r->bf_xt[i] : nullptr;
+              ex.e.act_param = below.act_param;
+              ex.col_partials = below.b >= 0 ? r->bf_colp : nullptr;
+              dz_handed_over = true;
+            }
             SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
             cur ^= 1;
           }
