@@ -537,6 +537,42 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(const float* __restrict__
   }
 }
 
+// The same forward pass for 2x2 max windows, 4 channels per thread, 32-bit indices: the four window cells are requested
+// together (cells outside the input re-read the tensor's first element and never win), then compared in window order.
+__global__ __launch_bounds__(256) void pool2x2_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
+                                                           int n, int h, int w, int c, int ho, int wo, int sh, int sw, int pt, int pl) {
+  const uint32_t cv = (uint32_t)(c / 4);
+  const uint32_t total = (uint32_t)n * ho * wo * cv;
+  const uint32_t stride = (uint32_t)gridDim.x * blockDim.x;
+  for (uint32_t i = (uint32_t)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t ch = (i % cv) * 4;
+    uint32_t t = i / cv;
+    const int ow = (int)(t % wo); t /= wo;
+    const int oh = (int)(t % ho);
+    const uint32_t b = t / ho;
+    float4 val[4];
+    bool in[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int iy = oh * sh - pt + (k >> 1), ix = ow * sw - pl + (k & 1);
+      in[k] = (unsigned)iy < (unsigned)h && (unsigned)ix < (unsigned)w;
+      val[k] = *(const float4*)(x + (in[k] ? ((b * h + iy) * w + ix) * c + ch : 0u));
+    }
+    float best[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    uint32_t at[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float v[4] = {val[k].x, val[k].y, val[k].z, val[k].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (in[k] && v[e] > best[e]) { best[e] = v[e]; at[e] = (uint32_t)k; }
+    }
+    const uint32_t o = i * 4;
+    *(float4*)(y + o) = make_float4(best[0], best[1], best[2], best[3]);
+    *(uint32_t*)(arg + o) = at[0] | (at[1] << 8) | (at[2] << 16) | (at[3] << 24);
+  }
+}
+
 static bool pool_vec4(const void* a, const void* b, const void* m, int c) {
   return c % 4 == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0 && (reinterpret_cast<uintptr_t>(m) & 3u) == 0;
 }
@@ -554,7 +590,9 @@ int launch_pool_fwd(sn_ctx* ctx, bool avg, const float* x, float* y, uint8_t* ar
     if (avg) hipLaunchKernelGGL((pool_fwd_kernel<V, I, true>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl); \
     else hipLaunchKernelGGL((pool_fwd_kernel<V, I, false>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl);    \
   } while (0)
-  if (v4 && small) SN_POOL_FWD(4, uint32_t);
+  if (v4 && small && !avg && kh == 2 && kw == 2)
+    hipLaunchKernelGGL(pool2x2_fwd_kernel, grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, sh, sw, pt, pl);
+  else if (v4 && small) SN_POOL_FWD(4, uint32_t);
   else if (v4) SN_POOL_FWD(4, uint64_t);
   else if (small) SN_POOL_FWD(1, uint32_t);
   else SN_POOL_FWD(1, uint64_t);
@@ -641,6 +679,62 @@ __global__ __launch_bounds__(256) void pool_bwd_kernel(const float* __restrict__
   }
 }
 
+// The same backward pass for 2x2 max windows, 4 channels per thread, 32-bit indices: an input element lies in at most 2 x 2
+// windows (oh_hi - a, ow_hi - d for a, d in {0, 1}); their argmax words and gradients are requested together (windows that do
+// not exist re-read the first element and are ignored) and added in the order of the general kernel (oh, then ow, ascending).
+__global__ __launch_bounds__(256) void pool2x2_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
+                                                           float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo, int sh,
+                                                           int sw, int pt, int pl, const float* __restrict__ y_in, int act, float act_param) {
+  const uint32_t cv = (uint32_t)(c / 4);
+  const uint32_t total = (uint32_t)n * h * w * cv;
+  const uint32_t stride = (uint32_t)gridDim.x * blockDim.x;
+  for (uint32_t i = (uint32_t)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const uint32_t ch = (i % cv) * 4;
+    uint32_t t = i / cv;
+    const int ix = (int)(t % w); t /= w;
+    const int iy = (int)(t % h);
+    const uint32_t b = t / h;
+    int oh_lo = iy + pt - 1;
+    oh_lo = oh_lo <= 0 ? 0 : (oh_lo + sh - 1) / sh;
+    int oh_hi = (iy + pt) / sh;
+    if (oh_hi > ho - 1) oh_hi = ho - 1;
+    int ow_lo = ix + pl - 1;
+    ow_lo = ow_lo <= 0 ? 0 : (ow_lo + sw - 1) / sw;
+    int ow_hi = (ix + pl) / sw;
+    if (ow_hi > wo - 1) ow_hi = wo - 1;
+    float4 yv = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (y_in) yv = *(const float4*)(y_in + i * 4);
+    uint32_t a4[4], want[4];
+    float4 g[4];
+    bool on[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int oh = oh_lo + (k >> 1), ow = ow_lo + (k & 1);
+      on[k] = oh <= oh_hi && ow <= ow_hi;
+      const uint32_t o = on[k] ? ((b * ho + oh) * wo + ow) * c + ch : 0u;
+      want[k] = (uint32_t)((iy - (oh * sh - pt)) * 2 + (ix - (ow * sw - pl)));
+      a4[k] = *(const uint32_t*)(arg + o);
+      g[k] = *(const float4*)(dy + o);
+    }
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (!on[k]) continue;
+      if ((a4[k] & 255u) == want[k]) s[0] += g[k].x;
+      if (((a4[k] >> 8) & 255u) == want[k]) s[1] += g[k].y;
+      if (((a4[k] >> 16) & 255u) == want[k]) s[2] += g[k].z;
+      if ((a4[k] >> 24) == want[k]) s[3] += g[k].w;
+    }
+    if (y_in) {
+      s[0] = act_bwd(act, yv.x, s[0], act_param);
+      s[1] = act_bwd(act, yv.y, s[1], act_param);
+      s[2] = act_bwd(act, yv.z, s[2], act_param);
+      s[3] = act_bwd(act, yv.w, s[3], act_param);
+    }
+    *(float4*)(dx + i * 4) = make_float4(s[0], s[1], s[2], s[3]);
+  }
+}
+
 int launch_pool_bwd(sn_ctx* ctx, bool avg, const float* dy, const uint8_t* arg, float* dx, int n, int h, int w, int c, int ho, int wo,
                     int kh, int kw, int sh, int sw, int pt, int pl, const float* y_in, int act, float act_param) {
   const int64_t total = (int64_t)n * h * w * c;
@@ -658,7 +752,9 @@ int launch_pool_bwd(sn_ctx* ctx, bool avg, const float* dy, const uint8_t* arg, 
       hipLaunchKernelGGL((pool_bwd_kernel<V, I, false>), grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, kh, kw, sh, sw, \
                          pt, pl, y_in, act, act_param);                                                                       \
   } while (0)
-  if (v4 && small) SN_POOL_BWD(4, uint32_t);
+  if (v4 && small && !avg && kh == 2 && kw == 2)
+    hipLaunchKernelGGL(pool2x2_bwd_kernel, grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, sh, sw, pt, pl, y_in, act, act_param);
+  else if (v4 && small) SN_POOL_BWD(4, uint32_t);
   else if (v4) SN_POOL_BWD(4, uint64_t);
   else if (small) SN_POOL_BWD(1, uint32_t);
   else SN_POOL_BWD(1, uint64_t);
