@@ -407,8 +407,8 @@ def main():
             line["batchnorm_hbm"] = main_res["batchnorm_hbm"]
     if not args.no_extras:
         extras = {}
-        for which, st, wu in (("mlp", 100, 10), ("lstm", 10, 2), ("wide_mlp", 5, 2), ("optim", 10, 3), ("lenet", 50, 5),
-                               ("cnn_bn", 10, 2), ("simple_rnn", 10, 2)):
+        for which, st, wu in (("mlp", 100, 10), ("lstm", 50, 5), ("wide_mlp", 20, 3), ("optim", 10, 3), ("lenet", 50, 5),
+                               ("cnn_bn", 30, 3), ("simple_rnn", 30, 3)):
             if which == args.workload:
                 continue
             try:
