@@ -46,18 +46,22 @@ constexpr int THREADS = 256;
   __device__ __forceinline__ void thread_advance(Cursor& c) const { advance(c, BK); }                              \
   __device__ __forceinline__ void init4(Cursor& c, int outer, int kb, int kk) const { init(c, outer, kb + kk); }   \
   __device__ __forceinline__ float load_t(const Cursor& c, const Tile&, int k_end) const { return load(c, k_end); } \
-  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile&, int k_end, float (&v)[4]) const { load4(c, k_end, v); }
+  __device__ __forceinline__ bool load4_t(const Cursor& c, const Tile&, int k_end, float (&v)[4]) const { load4(c, k_end, v); return true; }
 
 // 16-byte load without a branch: a lane whose element lies outside the matrix reads the first 16 bytes of
 // the tensor instead (always mapped, 16-byte aligned) and discards them.  Offsets are 32-bit: the host only
 // picks the FAST loaders for tensors below 2 GiB.
 constexpr int64_t FAST_SPAN = (int64_t)1 << 31;
-__device__ __forceinline__ void sel_load4(const float* base, uint32_t byte_off, bool valid, float (&v)[4]) {
+// Returns `valid` and leaves the select to the caller, who applies it when the values go to LDS one K tile later: a select
+// right here would make the loads' consumer sit directly behind them, and the wait for the data would land in front of
+// the current tile's MFMAs instead of behind them.
+__device__ __forceinline__ bool sel_load4(const float* base, uint32_t byte_off, bool valid, float (&v)[4]) {
   const f4v r = *(const f4v*)((const char*)base + (valid ? byte_off : 0u));
-  v[0] = valid ? r[0] : 0.f;
-  v[1] = valid ? r[1] : 0.f;
-  v[2] = valid ? r[2] : 0.f;
-  v[3] = valid ? r[3] : 0.f;
+  v[0] = r[0];
+  v[1] = r[1];
+  v[2] = r[2];
+  v[3] = r[3];
+  return valid;
 }
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -450,8 +454,8 @@ struct FlatLoader {
   __device__ __forceinline__ void tile_init(Tile& t, int k0) const { t.k0 = k0; t.koff = (uint32_t)k0 * (uint32_t)s_k * 4u; }
   __device__ __forceinline__ void tile_advance(Tile& t) const { t.k0 += BK; t.koff += (uint32_t)BK * (uint32_t)s_k * 4u; }
   __device__ __forceinline__ void thread_advance(Cursor&) const {}
-  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
-    sel_load4(p, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
+  __device__ __forceinline__ bool load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    return sel_load4(p, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
   }
   __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }  // FAST loaders run VEC = 4 only
   static bool ok(const float* p, int64_t s_outer, int64_t s_k, int outer_n, int K) {
@@ -518,8 +522,8 @@ struct TapLoader {
     set_tap(t);
   }
   __device__ __forceinline__ void thread_advance(Cursor&) const {}
-  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
-    sel_load4(src, c.base + t.tapoff, ((c.mask >> (t.rq & 31)) & 1u) != 0 && t.k0 + c.kk < k_end, v);
+  __device__ __forceinline__ bool load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    return sel_load4(src, c.base + t.tapoff, ((c.mask >> (t.rq & 31)) & 1u) != 0 && t.k0 + c.kk < k_end, v);
   }
   __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
   static bool ok(const float* src, int n, int H, int W, int C, int kh, int kw) {
@@ -557,8 +561,8 @@ struct DgradWLoader {
     t.koff = (uint32_t)(t.rq * cin * cout + t.c0) * 4u;
   }
   __device__ __forceinline__ void thread_advance(Cursor&) const {}
-  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
-    sel_load4(w, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
+  __device__ __forceinline__ bool load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+    return sel_load4(w, c.base + t.koff, c.kk >= 0 && t.k0 + c.kk < k_end, v);
   }
   __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
 };
@@ -611,9 +615,9 @@ struct WgradXLoader {
       }
     }
   }
-  __device__ __forceinline__ void load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
+  __device__ __forceinline__ bool load4_t(const Cursor& c, const Tile& t, int k_end, float (&v)[4]) const {
     const bool inside = interior || ((unsigned)c.iy < (unsigned)g.h && (unsigned)c.ix < (unsigned)g.w);
-    sel_load4(x, c.off, c.kk >= 0 && t.k0 + c.kk < k_end && inside, v);
+    return sel_load4(x, c.off, c.kk >= 0 && t.k0 + c.kk < k_end && inside, v);
   }
   __device__ __forceinline__ float load_t(const Cursor&, const Tile&, int) const { return 0.f; }
   static bool ok(const float* x, const ConvGeom& g) {
@@ -825,17 +829,20 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 
   // both staging layouts put consecutive values of the contiguous index one LDS slot apart
   float ra[EA][VEC], rb[EB][VEC];
+  bool va[EA], vb[EB];  // false: the vector lies outside the operand and goes to LDS as zeros
   auto fetch = [&]() {  // loads the tile the loaders point at (zeros past k_end), then moves them on
 #pragma unroll
     for (int e = 0; e < EA; ++e) {
-      if constexpr (VEC == 4) al.load4_t(ca[e], ta, k_end, ra[e]);
+      va[e] = true;
+      if constexpr (VEC == 4) va[e] = al.load4_t(ca[e], ta, k_end, ra[e]);
       else ra[e][0] = al.load_t(ca[e], ta, k_end);
       al.thread_advance(ca[e]);
     }
     if (b_on) {
 #pragma unroll
       for (int e = 0; e < EB; ++e) {
-        if constexpr (VEC == 4) bl.load4_t(cb[e], tb, k_end, rb[e]);
+        vb[e] = true;
+        if constexpr (VEC == 4) vb[e] = bl.load4_t(cb[e], tb, k_end, rb[e]);
         else rb[e][0] = bl.load_t(cb[e], tb, k_end);
         bl.thread_advance(cb[e]);
       }
@@ -852,12 +859,12 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(int M, int N, int K, int 
 #pragma unroll
     for (int e = 0; e < EA; ++e)
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)ra[e][i];
+      for (int i = 0; i < VEC; ++i) As[ia[e] + i] = (lds_t)(va[e] ? ra[e][i] : 0.f);
     if (b_on) {
 #pragma unroll
       for (int e = 0; e < EB; ++e)
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)rb[e][i];
+        for (int i = 0; i < VEC; ++i) Bs[ib[e] + i] = (lds_t)(vb[e] ? rb[e][i] : 0.f);
     }
     __syncthreads();
     if (k0 + BK < k_end) fetch();  // the next tile's global loads fly while this one is multiplied
