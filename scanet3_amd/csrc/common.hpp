@@ -123,10 +123,11 @@ int launch_softmax_bwd(sn_ctx* ctx, const float* p, const float* dp, float* dz, 
 // loss value (sum of per-element terms / divisor) into *loss_dev and d loss / d p into dp (dp may be null)
 // loss kinds beyond the public SN_LOSS_*: plain sums of the error terms the regression estimators use
 constexpr int LOSS_SUM_SQUARED_ERROR = 100, LOSS_SUM_ABSOLUTE_ERROR = 101;
+// loss_dev == nullptr: only dp is wanted (the per-block partial sums are still written, the final reduction is skipped)
 int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp, float* loss_dev, float* partials,
                 int rows, int cols);
 // training step of a Softmax output under CategoricalCrossentropy: p, loss value and dz in one kernel per row
-// (row_loss: `rows` floats of scratch)
+// (row_loss: `rows` floats of scratch; loss_dev == nullptr: the loss value is not wanted, its final reduction is skipped)
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
                        int cols, bool stable);
 // out[c] = sum over rows of dy[r*ld + c]; `ws` (optional) lets many rows be summed in parallel slices

@@ -238,7 +238,7 @@ int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp
     hipLaunchKernelGGL(loss_stage1_kernel, dim3(blocks), dim3(256), 0, ctx->stream, kind, p, y, dp, partials, n, inv_size,
                        neg_inv_rows);
   }
-  {
+  if (loss_dev) {
     LaunchScope scope(ctx, "loss_stage2");
     hipLaunchKernelGGL(loss_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, kind, partials, (int)blocks, loss_dev, inv_size,
                        (float)rows);
@@ -295,7 +295,7 @@ int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, fl
     hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0,
                        -(1.0f / (float)rows));
   }
-  {
+  if (loss_dev) {
     LaunchScope scope(ctx, "loss_stage2");
     hipLaunchKernelGGL(loss_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, (int)SN_LOSS_CATEGORICAL_CROSSENTROPY, (const float*)row_loss,
                        rows, loss_dev, 0.f, (float)rows);

@@ -636,12 +636,14 @@ static int add_penalties(sn_replica* r, bool training) {
 }
 
 // loss (+ penalty) into loss_dev; dp (may be null) receives d loss / d prediction
-static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp, bool training) {
+// want_value = false: only dp is wanted (a training step whose caller does not read the loss): the final reduction and
+// the penalty terms, which only the value needs, are skipped
+static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, float* dp, bool training, bool want_value = true) {
   sn_model* m = r->model;
   if (m->loss == SN_LOSS_IDENTITY)
     SN_REQUIRE((int64_t)rows * m->out_elems == 1, "Identity loss needs a scalar model output");
-  SN_TRY(launch_loss(r->ctx, m->loss, pred, y, dp, r->loss_dev, r->loss_partials, rows, (int)m->out_elems));
-  return add_penalties(r, training);
+  SN_TRY(launch_loss(r->ctx, m->loss, pred, y, dp, want_value ? r->loss_dev : nullptr, r->loss_partials, rows, (int)m->out_elems));
+  return want_value ? add_penalties(r, training) : SN_OK;
 }
 
 // ---------------------------------------------------------------------------- backward
@@ -882,20 +884,22 @@ static int read_loss(sn_replica* r, float* loss_host) {
   return SN_OK;
 }
 
-static int grad_pass(sn_replica* r, const float* x, const float* y, int rows) {
+// want_loss = false: the caller does not read this step's loss value (the steps inside an epoch, sn_step / sn_grad without a
+// loss pointer), so the kernels that only finish the scalar are not launched
+static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss) {
   sn_model* m = r->model;
   const int last = (int)m->ops.size() - 1;
   if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
     // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
     SN_TRY(forward(r, x, rows, true, true));
-    SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], r->loss_dev, r->loss_partials, rows,
-                              (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
-    SN_TRY(add_penalties(r, true));
+    SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], want_loss ? r->loss_dev : nullptr,
+                              r->loss_partials, rows, (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+    if (want_loss) SN_TRY(add_penalties(r, true));
     return backward(r, x, rows, last - 1, 1);
   }
   SN_TRY(forward(r, x, rows, false, true));
   const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);
-  SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0], true));
+  SN_TRY(loss_of(r, pred, y, rows, r->grad_buf[0], true, want_loss));
   SN_TRY(backward(r, x, rows));
   return SN_OK;
 }
@@ -1098,7 +1102,7 @@ int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   SN_TRY(check_rows(rep, rows));
   SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
   SN_REQUIRE(rep->has_opt, "replica was created without an optimizer");
-  SN_TRY(grad_pass(rep, x_dev, y_dev, rows));
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr));
   SN_TRY(update(rep, iter));
   return read_loss(rep, loss_host);
 }
@@ -1107,7 +1111,7 @@ int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   SN_TRY(check_replica(rep));
   SN_REQUIRE(x_dev && y_dev, "sn_grad: null batch pointer");
   SN_TRY(check_rows(rep, rows));
-  SN_TRY(grad_pass(rep, x_dev, y_dev, rows));
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr));
   return read_loss(rep, loss_host);
 }
 
@@ -1174,7 +1178,7 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
              (long long)total_rows, batch);
   const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
   for (int64_t i = 0; i < n_batches; ++i) {
-    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch));
+    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch, false));  // the epoch's loss is evaluated after its last update
     SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
   }
   if (iterations_host) *iterations_host = (int32_t)n_batches;
@@ -1229,7 +1233,7 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
       SN_TRY(fill(i + 1, slot ^ 1));
     }
     SN_HIP(hipStreamWaitEvent(compute, rep->ev_filled[slot], 0));
-    SN_TRY(grad_pass(rep, rep->stage_x[slot], rep->stage_y[slot], batch));
+    SN_TRY(grad_pass(rep, rep->stage_x[slot], rep->stage_y[slot], batch, false));
     SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
     SN_HIP(hipEventRecord(rep->ev_consumed[slot], compute));
   }
