@@ -959,6 +959,42 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
+// The same reduction when M*N is a multiple of 4 (every partial tile then starts on a 16-byte boundary): a lane owns 4
+// consecutive outputs and reads them as one 16-byte load per split; every output sees the same additions in the same order.
+template <class EP>
+__global__ __launch_bounds__(256) void splitk_reduce4_kernel(const float* __restrict__ ws, int splits, int M, int N, EP ep) {
+  const int64_t total4 = (int64_t)M * N / 4;
+  const int g = threadIdx.x >> 5, j = threadIdx.x & 31;  // 8 groups of 32 lanes x 4 consecutive outputs
+  for (int64_t base = (int64_t)blockIdx.x * 32; base < total4; base += (int64_t)gridDim.x * 32) {
+    const int64_t i = base + j;
+    f4v s = {0.f, 0.f, 0.f, 0.f};
+    if (i < total4) {
+      const f4v* w4 = reinterpret_cast<const f4v*>(ws) + i;
+      int z = g;
+      for (; z + 56 < splits; z += 64) {  // 8 loads of 16 bytes in flight, added in split order
+        f4v a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = w4[(int64_t)(z + 8 * u) * total4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += a[u];
+      }
+      for (; z < splits; z += 8) s += w4[(int64_t)z * total4];
+    }
+    __shared__ f4v part4[8][32];
+    part4[g][j] = s;
+    __syncthreads();
+    if (g == 0 && i < total4) {
+      const f4v t = ((part4[0][j] + part4[1][j]) + (part4[2][j] + part4[3][j])) + ((part4[4][j] + part4[5][j]) + (part4[6][j] + part4[7][j]));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int64_t o = i * 4 + e;
+        ep.store((int)(o / N), (int)(o % N), t[e]);
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // ============================================================================ small output, long reduction
 // C[M,N] with M*N <= 1024 and K in the thousands (first-layer filter gradients, Dense layers onto a few
 // classes): too little output for MFMA tiles to occupy the chip. Workgroups stride over 64-long slices of K,
@@ -1118,9 +1154,14 @@ static int launch_tiles(sn_ctx* ctx, const char* name, int M, int N, int K, cons
   }
   if (splits > 1) {
     const int64_t total = (int64_t)M * N;
-    int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
     LaunchScope scope(ctx, "splitk_reduce");
-    hipLaunchKernelGGL((splitk_reduce_kernel<EP>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, splits, M, N, ep);
+    if (total % 4 == 0 && total >= 4096 && aligned16(ws)) {
+      const int64_t blocks = std::min<int64_t>(ceil_div(total / 4, 32), (int64_t)ctx->compute_units * 16);
+      hipLaunchKernelGGL((splitk_reduce4_kernel<EP>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, splits, M, N, ep);
+    } else {
+      const int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
+      hipLaunchKernelGGL((splitk_reduce_kernel<EP>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, splits, M, N, ep);
+    }
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
