@@ -227,7 +227,8 @@ SN_API int sn_replica_flat(sn_replica* rep, int32_t slot, float** out_dev, int64
 /* One call of the compiled backprop function (optimizers/Optimizer.scala:142-143, 169-194):
  * forward, loss, gradients of every weight, optimizer update w' = w - delta with iteration
  * number `iter` (1-based). `rows` <= batch. If `loss_host` is not NULL the loss of this batch
- * (before the update) is written there and the call waits for the device. */
+ * (before the update) is written there and the call waits for the device; with NULL the kernels that
+ * only finish the loss value (its final reduction, the penalty terms) are not launched. */
 SN_API int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, int32_t iter, float* loss_host);
 /* `LossModel.grad` (models/Model.scala:107-111): gradients only, no update. */
 SN_API int sn_grad(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
