@@ -286,14 +286,79 @@ __global__ __launch_bounds__(256) void softmax_cce_kernel(const float* __restric
   if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
 }
 
+// The same row kernel when a thread's share of the row (E values: columns threadIdx.x + k * blockDim.x) fits in registers:
+// z and y are read once, p and dz written once; every sum sees the same values in the same order as above.
+template <int E>
+__global__ __launch_bounds__(256) void softmax_cce_reg_kernel(const float* __restrict__ z, const float* __restrict__ y, float* __restrict__ p,
+                                                               float* __restrict__ dz, float* __restrict__ row_loss, int cols, int stable,
+                                                               float neg_inv_rows) {
+  __shared__ float smem[4];
+  const int64_t base = (int64_t)blockIdx.x * cols;
+  const float eps = 1e-8f;
+  float zv[E], yv[E];
+#pragma unroll
+  for (int k = 0; k < E; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    zv[k] = c < cols ? z[base + c] : 0.f;
+    yv[k] = c < cols ? y[base + c] : 0.f;
+  }
+  float mx = 0.f;
+  if (stable) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < E; ++k)
+      if ((int)(threadIdx.x + k * blockDim.x) < cols) m = fmaxf(m, zv[k]);
+    mx = block_max(m, smem);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < E; ++k) {
+    if ((int)(threadIdx.x + k * blockDim.x) < cols) {
+      zv[k] = expf(zv[k] - mx);
+      s += zv[k];
+    }
+  }
+  const float total = block_sum(s, smem);
+  float term = 0.f, dot = 0.f;
+#pragma unroll
+  for (int k = 0; k < E; ++k) {
+    if ((int)(threadIdx.x + k * blockDim.x) < cols) {
+      const float pi = zv[k] / total;
+      zv[k] = pi;
+      term += yv[k] * logf(pi + eps);
+      dot += pi * ((yv[k] * neg_inv_rows) / (pi + eps));
+    }
+  }
+  const float row_term = block_sum(term, smem);
+  const float row_dot = block_sum(dot, smem);
+#pragma unroll
+  for (int k = 0; k < E; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < cols) {
+      const float pi = zv[k];
+      const float dpi = (yv[k] * neg_inv_rows) / (pi + eps);
+      p[base + c] = pi;
+      dz[base + c] = pi * dpi - pi * row_dot;
+    }
+  }
+  if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
+}
+
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
                        int cols, bool stable) {
   SN_REQUIRE(rows > 0 && cols > 0, "loss over an empty batch");
   {
     LaunchScope scope(ctx, "softmax_crossentropy_fused");
     const int threads = cols <= 64 ? 64 : 256;
-    hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0,
-                       -(1.0f / (float)rows));
+    const float neg_inv_rows = -(1.0f / (float)rows);
+#define SN_SOFTMAX_CCE_REG(E) \
+  hipLaunchKernelGGL((softmax_cce_reg_kernel<E>), dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows)
+    if (cols <= threads) SN_SOFTMAX_CCE_REG(1);
+    else if (cols <= 2 * threads) SN_SOFTMAX_CCE_REG(2);
+    else if (cols <= 4 * threads) SN_SOFTMAX_CCE_REG(4);
+    else
+      hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows);
+#undef SN_SOFTMAX_CCE_REG
   }
   if (loss_dev) {
     LaunchScope scope(ctx, "loss_stage2");
