@@ -240,6 +240,14 @@ SN_API int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* 
  * BatchNorm normalises with the statistics of these `rows`.  The next state it would return is not applied;
  * only sn_step and the epoch calls move layer state. */
 SN_API int sn_forward_training(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
+/* sn_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same result as sn_forward, but every
+ * intermediate of the pass (layer outputs, pooling offsets, BatchNorm vectors, the GEMM workspace) lives in one
+ * 64 MiB device array that is part of the library image (each GPU the library runs on holds its copy until the
+ * process ends), and the call makes no hipMalloc / hipFree.  Fails with SN_E_INVALID when `rows` of this model need
+ * more than 64 MiB, for models with recurrent layers and for SN_FLAG_GEMM_BF16.  Per-kernel timing is off inside the
+ * call.  All calls on one GPU share the array: calls that overlap on one GPU (two contexts, two streams) race. */
+SN_API int sn_forward_static(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
 /* `LossModel.loss` (models/Model.scala:101-102) of the frozen model. */
 SN_API int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host);
 /* Per-batch body of `estimators.accuracy` (estimators/package.scala:28-32): rows whose every

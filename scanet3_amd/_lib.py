@@ -94,6 +94,7 @@ SIGNATURES = {
     "sn_grad": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_forward": (C.c_int, [_P, _P, C.c_int32, _P]),
     "sn_forward_training": (C.c_int, [_P, _P, C.c_int32, _P]),
+    "sn_forward_static": (C.c_int, [_P, _P, C.c_int32, _P]),
     "sn_error_sum": (C.c_int, [_P, _P, _P, C.c_int32, C.c_int32, _F]),
     "sn_loss": (C.c_int, [_P, _P, _P, C.c_int32, _F]),
     "sn_count_correct": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64)]),

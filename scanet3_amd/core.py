@@ -281,6 +281,10 @@ class Replica:
         finally:
             out.free()
 
+    def forward_static(self, x, out: "DeviceBuffer", rows: Optional[int] = None) -> None:
+        """`sn_forward_static`: the frozen forward pass into the caller's buffer, with no device allocation in the call."""
+        check(lib.sn_forward_static(self.handle, self._ptr(x), self.model.batch if rows is None else rows, self._ptr(out)))
+
     def loss(self, x, y, rows: Optional[int] = None) -> float:
         loss = C.c_float()
         check(lib.sn_loss(self.handle, self._ptr(x), self._ptr(y), self.model.batch if rows is None else rows, C.byref(loss)))

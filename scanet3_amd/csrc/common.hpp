@@ -84,6 +84,8 @@ struct LaunchScope {
   ~LaunchScope();
 };
 int profile_drain(sn_ctx* ctx);
+// looks up this device's address of the library's static scratch array (model.hip); `device` must be current
+int static_scratch_init(int device);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -11,6 +11,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <mutex>
 
 namespace sn {
 
@@ -939,6 +940,31 @@ static int tensor_io(sn_replica* r, float* base, int index, float* host, const f
 
 }  // namespace sn
 
+// ---- the forward pass for callers that cannot allocate -----------------------------------------------------------
+// Every intermediate of the pass (layer outputs, pooling window offsets, BatchNorm vectors, the GEMM workspace)
+// lives in one file-scope device array instead of the replica's own allocations.  Each device the library runs on
+// holds its own copy of the array at its own address; the address is looked up once per device.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)64 << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+static unsigned char* g_scratch_ptr[STATIC_SCRATCH_MAX_DEVICES];  // device address of `scratch` per device, null until looked up
+static std::mutex g_scratch_mutex;
+
+namespace sn {
+// Called by sn_ctx_create with `device` current.
+int static_scratch_init(int device) {
+  SN_REQUIRE(device >= 0 && device < STATIC_SCRATCH_MAX_DEVICES, "device %d is beyond the %d the library keeps scratch addresses for", device,
+             STATIC_SCRATCH_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device]) return SN_OK;
+  unsigned char* ptr = nullptr;
+  SN_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+  SN_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the static scratch array");
+  g_scratch_ptr[device] = ptr;
+  return SN_OK;
+}
+}  // namespace sn
+
 using namespace sn;
 
 extern "C" {
@@ -1127,6 +1153,59 @@ static int forward_to(sn_replica* rep, const float* x_dev, int32_t rows, float* 
 int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) { return forward_to(rep, x_dev, rows, out_dev, false); }
 int sn_forward_training(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) {
   return forward_to(rep, x_dev, rows, out_dev, true);
+}
+
+int sn_forward_static(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev) {
+  SN_TRY(check_replica(rep));
+  SN_REQUIRE(x_dev && out_dev, "sn_forward_static: null pointer");
+  SN_TRY(check_rows(rep, rows));
+  sn_model* m = rep->model;
+  sn_ctx* ctx = rep->ctx;
+  SN_REQUIRE((m->flags & SN_FLAG_GEMM_BF16) == 0, "sn_forward_static: models with SN_FLAG_GEMM_BF16 keep bf16 operand copies it has no room for");
+  for (const Op& op : m->ops)
+    SN_REQUIRE(op.kind != OP_LSTM && op.kind != OP_SRNN, "sn_forward_static: recurrent layers keep per-step state it has no room for");
+  unsigned char* base = ctx->device >= 0 && ctx->device < STATIC_SCRATCH_MAX_DEVICES ? g_scratch_ptr[ctx->device] : nullptr;
+  SN_REQUIRE(base != nullptr, "sn_forward_static: the scratch array of device %d was never looked up", ctx->device);
+  // carve the array: every piece starts on a 256-byte boundary
+  const size_t n_ops = m->ops.size();
+  std::vector<float*> act(n_ops, nullptr), bn(n_ops, nullptr);
+  std::vector<uint8_t*> arg(n_ops, nullptr);
+  size_t used = 0;
+  auto carve = [&](size_t bytes) {
+    unsigned char* p = base + used;  // an address past the end is never used: the size check below comes first
+    used += (size_t)align_up((int64_t)bytes, 256);
+    return p;
+  };
+  for (size_t i = 0; i < n_ops; ++i) {
+    const Op& op = m->ops[i];
+    if (op.kind == OP_FLATTEN) continue;
+    act[i] = (float*)carve((size_t)rows * op.out_elems * sizeof(float));
+    if (op.kind == OP_BATCHNORM) bn[i] = (float*)carve((size_t)9 * align_up(op.out_dims.back(), 64) * sizeof(float));
+    if (op.kind == OP_POOL && !op.pool_avg) arg[i] = (uint8_t*)carve((size_t)rows * op.out_elems);
+  }
+  float* ws = (float*)carve((size_t)m->workspace_elems * sizeof(float));
+  SN_REQUIRE(used <= STATIC_SCRATCH_BYTES,
+             "sn_forward_static: %d rows of this model need %zu bytes of intermediates, the static scratch array holds %zu", rows, used,
+             STATIC_SCRATCH_BYTES);
+  // The pass itself is sn_forward's, pointed at the static pieces.  Per-kernel timing creates events: off for this call.
+  const bool profiling = ctx->profiling;
+  ctx->profiling = false;
+  std::swap(rep->act, act);
+  std::swap(rep->arg, arg);
+  std::swap(rep->bn_buf, bn);
+  std::swap(rep->ws, ws);
+  int rc = forward(rep, x_dev, rows, false, false);
+  if (rc == SN_OK) {
+    const float* pred = op_output(rep, (int)n_ops - 1, x_dev, rows);
+    hipError_t e = hipMemcpyAsync(out_dev, pred, (size_t)rows * m->out_elems * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream);
+    if (e != hipSuccess) rc = fail(SN_E_HIP, "hipMemcpyAsync failed: %s", hipGetErrorString(e));
+  }
+  std::swap(rep->act, act);
+  std::swap(rep->arg, arg);
+  std::swap(rep->bn_buf, bn);
+  std::swap(rep->ws, ws);
+  ctx->profiling = profiling;
+  return rc;
 }
 
 int sn_loss(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t rows, float* loss_host) {

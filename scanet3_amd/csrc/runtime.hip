@@ -102,6 +102,7 @@ int sn_ctx_create(int device, void* stream, sn_ctx** out) {
   SN_HIP(hipGetDeviceProperties(&prop, device));
   SN_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, "device %d is %s; this library holds gfx950 code only", device,
              prop.gcnArchName);
+  SN_TRY(static_scratch_init(device));
   sn_ctx* ctx = new sn_ctx();
   ctx->magic = CTX_MAGIC;
   ctx->device = device;
