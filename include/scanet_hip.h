@@ -119,6 +119,9 @@ typedef struct sn_layer_desc {
   int32_t bias_reg_kind;
   float bias_reg_lambda;
   int32_t pool_reduce;   /* POOL2D: SN_POOL_*.  AVG divides by the number of window cells inside the input (TF AvgPool) */
+  int32_t stateful;      /* LSTM / SIMPLE_RNN: `stateful` (layer/RNN.scala:27,34,66-67): the state the last time step leaves
+                            (LSTM "cell_state" and "hidden_state", simple cell "0/state"; (batch, units), zeros at first) is a
+                            non-trainable parameter that the next sn_step starts from; sn_replicas_average re-initialises it */
 } sn_layer_desc;
 
 /* An `Algorithm` case class (optimizers/Algorithm.scala:6-11).  Field use per kind:
@@ -137,6 +140,8 @@ typedef struct sn_optimizer_desc {
   float epsilon;
   float init_acc;        /* initial value of every state tensor (Nadam.scala:26-35, Adamax.scala:30-39) */
   int32_t nesterov;
+  int32_t maximize;      /* 0: w' = w - delta (`Optimizer.minimize`); 1: w' = w + delta (`Optimizer.maximize`,
+                            optimizers/Optimizer.scala:186,326-336) */
 } sn_optimizer_desc;
 
 #define SN_MAX_RANK 8
@@ -153,6 +158,8 @@ typedef struct sn_param_info {
   int32_t trainable;             /* 0: layer state (BatchNorm moving statistics, `ParamDef.trainable = false`): no gradient,
                                     no optimizer state; the step replaces it with the layer's own update
                                     (optimizers/Optimizer.scala:118-122,142-144) */
+  int32_t aggregated;            /* `ParamDef.aggregation`: 1 Some(Avg), averaged by sn_replicas_average; 0 None (the carried
+                                    state of a stateful RNN), re-initialised to zeros there (Optimizer.scala:205-210) */
 } sn_param_info;
 
 /* ---------------------------------------------------------------- context / errors */
@@ -273,7 +280,15 @@ SN_API int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float
 
 /* `aggregateParams` (optimizers/Optimizer.scala:196-230) for K replicas of one model: weights and
  * every optimizer-state tensor become the uniform mean AddN(..)/K (models/Aggregation.scala:16-19)
- * and are written back to all K replicas (the next epoch's broadcast, Optimizer.scala:72-73). */
+ * and are written back to all K replicas (the next epoch's broadcast, Optimizer.scala:72-73); tensors
+ * without an aggregation (the carried state of a stateful RNN, layer/RNN.scala:188,302-303) are
+ * re-initialised to zeros in every replica (Optimizer.scala:207-210).
+ * DEVIATION for K > 2: the reference only ever averages PAIRS -- Spark's treeReduce folds
+ * avg2(l, r) = AddN(l, r) / 2 and (l.loss + r.loss) / 2 in an order Spark chooses, so three partitions
+ * end up weighted 1/4, 1/4, 1/2 in arrival order.  K = 2 is the reference's avg2 bit for bit; for K > 2 this
+ * call takes the uniform mean the build target names, no reference test runs more than one partition, and
+ * parity is unpinned.  A caller that wants one particular pairwise fold calls sn_average with k = 2 on the
+ * flat views (sn_replica_flat) in its own order. */
 SN_API int sn_replicas_average(sn_replica* const* reps, int32_t k);
 
 /* ---------------------------------------------------------------- flat kernels (the memory-bound pair) */

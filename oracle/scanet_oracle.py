@@ -420,6 +420,7 @@ class Layer:
     bias: bool = True               # lstm / simple_rnn only
     rnn_activation: int = ACT_TANH  # simple_rnn cell activation / lstm `activation`
     return_sequence: bool = False   # lstm / simple_rnn: every step's output, (batch, time, units) (RNN.scala:27,75-77)
+    stateful: bool = False          # lstm / simple_rnn: the cell state after one batch is the start of the next (RNN.scala:27,34,66-67)
     momentum: float = 0.99          # batchnorm (BatchNorm.scala:66-67)
     epsilon: float = 1e-3
     fused: bool = False             # batchnorm: the FusedBatchNormV3 branch as the reference wires it (rank-4 input)
@@ -435,7 +436,8 @@ class Layer:
             return [("weights", (self.kernel[0], self.kernel[1], in_shape[3], self.units))]
         if self.kind == "lstm":         # RNN.scala:285-305 (gate order forget,input,gate,output)
             f, h = in_shape[2], self.units
-            out = []
+            # `if (stateful) state ++ weights else weights` (RNN.scala:32-35); states (batch, units), Zeros, no aggregation (:302-303)
+            out = [("cell_state", (in_shape[0], h)), ("hidden_state", (in_shape[0], h))] if self.stateful else []
             for gate in ("forget", "input", "gate", "output"):
                 out.append((f"{gate}/0/kernel_weights", (f, h)))
                 out.append((f"{gate}/0/recurrent_weights", (h, h)))
@@ -444,7 +446,8 @@ class Layer:
             return out
         if self.kind == "simple_rnn":   # RNN.scala:170-206
             f, h = in_shape[2], self.units
-            out = [("0/kernel_weights", (f, h)), ("0/recurrent_weights", (h, h))]
+            out = [("0/state", (in_shape[0], h))] if self.stateful else []     # RNN.scala:188: `State -> ParamDef(outputShape(input), Zeros)`
+            out += [("0/kernel_weights", (f, h)), ("0/recurrent_weights", (h, h))]
             if self.bias:
                 out.append(("1/weights", (h,)))
             return out
@@ -503,14 +506,15 @@ def Flatten():
     return [Layer("flatten")]
 
 
-def LSTM(units, bias=True, return_sequence=False, kernel_reg=(REG_NONE, 0.0), recurrent_reg=(REG_NONE, 0.0), bias_reg=(REG_NONE, 0.0)):
-    return [Layer("lstm", units=units, bias=bias, return_sequence=return_sequence, reg=kernel_reg[0], reg_lambda=kernel_reg[1],
+def LSTM(units, bias=True, return_sequence=False, kernel_reg=(REG_NONE, 0.0), recurrent_reg=(REG_NONE, 0.0), bias_reg=(REG_NONE, 0.0),
+         stateful=False):
+    return [Layer("lstm", units=units, bias=bias, return_sequence=return_sequence, stateful=stateful, reg=kernel_reg[0], reg_lambda=kernel_reg[1],
                   recurrent_reg=recurrent_reg[0], recurrent_lambda=recurrent_reg[1], bias_reg=bias_reg[0], bias_lambda=bias_reg[1])]
 
 
 def SimpleRNN(units, activation=ACT_TANH, bias=True, return_sequence=False, kernel_reg=(REG_NONE, 0.0), recurrent_reg=(REG_NONE, 0.0),
-              bias_reg=(REG_NONE, 0.0)):
-    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation, return_sequence=return_sequence,
+              bias_reg=(REG_NONE, 0.0), stateful=False):
+    return [Layer("simple_rnn", units=units, bias=bias, rnn_activation=activation, return_sequence=return_sequence, stateful=stateful,
                   reg=kernel_reg[0], reg_lambda=kernel_reg[1], recurrent_reg=recurrent_reg[0], recurrent_lambda=recurrent_reg[1],
                   bias_reg=bias_reg[0], bias_lambda=bias_reg[1])]
 
@@ -527,9 +531,19 @@ def BatchNorm(momentum=0.99, epsilon=1e-3, fused=False, beta_reg=(REG_NONE, 0.0)
     return [Layer("batchnorm", momentum=momentum, epsilon=epsilon, fused=fused, reg=beta_reg[0], reg_lambda=beta_reg[1])]
 
 
+RNN_STATE = ("state", "cell_state", "hidden_state")                # RNN.scala:167,253-254
+
+
 def is_state_path(path: str) -> bool:
-    """Parameters with `trainable = false` (ParamDef of MovingMean / MovingVariance, BatchNorm.scala:96-97)."""
-    return path.rsplit("/", 1)[-1] in BN_STATE
+    """Parameters with `trainable = false`: MovingMean / MovingVariance (BatchNorm.scala:96-97) and the carried state of
+    a stateful RNN (RNN.scala:188,302-303; `ParamDef.trainable` defaults to false)."""
+    return path.rsplit("/", 1)[-1] in BN_STATE + RNN_STATE
+
+
+def is_unaggregated_path(path: str) -> bool:
+    """Parameters whose ParamDef has `aggregation = None`: `aggregateParams` re-initialises them instead of averaging
+    (Optimizer.scala:205-210).  Only the RNN states (Zeros) are such."""
+    return path.rsplit("/", 1)[-1] in RNN_STATE
 
 
 def batchnorm_forward(x, params, pre, l: Layer, training: bool):
@@ -712,9 +726,13 @@ class Model:
                 y = (avg_pool if l.pool_avg else max_pool)(x, l.kernel, l.strides, l.padding)
                 c = x
             elif k == "lstm":
-                y, c = lstm_forward(x, params, pre, l)
+                y, c, nxt = lstm_forward(x, params, pre, l)
+                if next_state is not None:
+                    next_state.update(nxt)
             elif k == "simple_rnn":
-                y, c = simple_rnn_forward(x, params, pre, l)
+                y, c, nxt = simple_rnn_forward(x, params, pre, l)
+                if next_state is not None:
+                    next_state.update(nxt)
             elif k == "batchnorm":
                 y, c, nxt = (batchnorm_fused_forward if l.fused else batchnorm_forward)(x, params, pre, l, training)
                 if next_state is not None:
@@ -832,12 +850,15 @@ GATES = ("forget", "input", "gate", "output")
 
 
 def lstm_forward(x, params, pre, l: Layer):
-    """RNN.build + LSTMCell.build (RNN.scala:40-72, 320-338); returns the last hidden state."""
+    """RNN.build + LSTMCell.build (RNN.scala:40-72, 320-338); returns (output, cache, next state).
+
+    `stateful`: the first step starts from the `cell_state` / `hidden_state` parameters instead of zeros and the last
+    step's c and h are the layer's next state (RNN.scala:66-72, 338)."""
     b, t_steps, _ = x.shape
     h_units = l.units
     dt = x.dtype
-    c = np.zeros((b, h_units), dt)
-    h = np.zeros((b, h_units), dt)
+    c = params[pre + "cell_state"][:b] if l.stateful else np.zeros((b, h_units), dt)
+    h = params[pre + "hidden_state"][:b] if l.stateful else np.zeros((b, h_units), dt)
     steps = []
     outs = []
     for t in range(t_steps):
@@ -858,7 +879,8 @@ def lstm_forward(x, params, pre, l: Layer):
         c, h = c_new, h_new
         outs.append(h_new)
     out = np.stack(outs, axis=1) if l.return_sequence else h     # `joinAlong(outputs, 1)` or `outputs.last` (RNN.scala:74-77)
-    return out, (x.shape, steps)
+    nxt = {pre + "cell_state": c, pre + "hidden_state": h} if l.stateful else {}
+    return out, (x.shape, steps), nxt
 
 
 def lstm_backward(dout, cache, params, pre, l: Layer, grads, need_dx=False):
@@ -912,7 +934,7 @@ def simple_rnn_forward(x, params, pre, l: Layer):
     b, t_steps, _ = x.shape
     dt = x.dtype
     wk, wr = params[pre + "0/kernel_weights"], params[pre + "0/recurrent_weights"]
-    s = np.zeros((b, l.units), dt)
+    s = params[pre + "0/state"][:b] if l.stateful else np.zeros((b, l.units), dt)
     steps = []
     out = None
     outs = []
@@ -926,7 +948,7 @@ def simple_rnn_forward(x, params, pre, l: Layer):
         s = r
     if l.return_sequence:
         out = np.stack(outs, axis=1)
-    return out, (x.shape, steps)
+    return out, (x.shape, steps), ({pre + "0/state": s} if l.stateful else {})
 
 
 def simple_rnn_backward(dout, cache, params, pre, l: Layer, grads, need_dx=False):
@@ -1143,7 +1165,9 @@ def train(model, alg, partitions, batch, epochs, init_params, avg="uniform"):
             iters, params, opt_state, loss = results[0]
         else:
             iters = sum(r[0] for r in results)
-            params = {p: average_uniform([r[1][p] for r in results]) for p in params}
+            # tensors without an aggregation are re-initialised (Optimizer.scala:207-210): the RNN states, to zeros
+            params = {p: np.zeros_like(params[p]) if is_unaggregated_path(p) else average_uniform([r[1][p] for r in results])
+                      for p in params}
             opt_state = {p: [average_uniform([r[2][p][s] for r in results])
                              for s in range(len(alg.state_names))] for p in params}
             loss = float(np.mean([r[3] for r in results]))

@@ -46,17 +46,17 @@ class LayerDesc(C.Structure):
                 ("return_sequence", C.c_int32), ("bn_momentum", C.c_float), ("bn_epsilon", C.c_float),
                 ("pad_top", C.c_int32), ("pad_bottom", C.c_int32), ("pad_left", C.c_int32), ("pad_right", C.c_int32),
                 ("bn_fused", C.c_int32), ("recurrent_reg_kind", C.c_int32), ("recurrent_reg_lambda", C.c_float),
-                ("bias_reg_kind", C.c_int32), ("bias_reg_lambda", C.c_float), ("pool_reduce", C.c_int32)]
+                ("bias_reg_kind", C.c_int32), ("bias_reg_lambda", C.c_float), ("pool_reduce", C.c_int32), ("stateful", C.c_int32)]
 
 
 class OptimizerDesc(C.Structure):
     _fields_ = [("kind", C.c_int32), ("rate", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float),
-                ("epsilon", C.c_float), ("init_acc", C.c_float), ("nesterov", C.c_int32)]
+                ("epsilon", C.c_float), ("init_acc", C.c_float), ("nesterov", C.c_int32), ("maximize", C.c_int32)]
 
 
 class ParamInfo(C.Structure):
     _fields_ = [("path", C.c_char * 96), ("offset", C.c_int64), ("size", C.c_int64), ("rank", C.c_int32),
-                ("dims", C.c_int64 * SN_MAX_RANK), ("trainable", C.c_int32)]
+                ("dims", C.c_int64 * SN_MAX_RANK), ("trainable", C.c_int32), ("aggregated", C.c_int32)]
 
 
 _P = C.c_void_p

@@ -45,7 +45,10 @@ def _compile(src: str) -> str:
 
 def build_library(verbose: bool = True) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    sources = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    missing = [s for s in SOURCES if not os.path.exists(os.path.join(CSRC, s))]
+    if missing:
+        raise FileNotFoundError(f"sources listed in build.py are missing from {CSRC}: {missing}")
+    sources = list(SOURCES)
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         objs = list(pool.map(_compile, sources))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]

@@ -106,6 +106,7 @@ struct OptScalars {
   float one_minus_b1, one_minus_b2;  // `1f.const - beta` evaluated in float32
   float bc1, bc2;                    // 1 - beta^iter, the divisor of `boost`
   int nesterov;
+  int maximize;                      // w + delta instead of w - delta (`Optimizer.maximize`, optimizers/Optimizer.scala:186)
 };
 OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter);
 int opt_state_count(int kind);
@@ -134,7 +135,8 @@ int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, fl
                        int cols, bool stable);
 // out[c] = sum over rows of dy[r*ld + c]; `ws` (optional) lets many rows be summed in parallel slices
 int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems);
-int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev);
+// partials: at least 1024 floats of scratch
+int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev, float* partials);
 int launch_penalty_grad(sn_ctx* ctx, const float* w, float* g, int64_t n, int reg_kind, float lambda);
 int launch_count_correct(sn_ctx* ctx, const float* p, const float* y, int rows, int cols, unsigned long long* count_dev);
 int launch_pool_fwd(sn_ctx* ctx, bool avg, const float* x, float* y, uint8_t* arg, int n, int h, int w, int c, int ho, int wo,

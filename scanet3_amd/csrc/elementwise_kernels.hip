@@ -478,17 +478,29 @@ int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t
 
 // ---------------------------------------------------------------------------- regularisation
 // L2: lambda * sum(w^2) / 2 ; L1: lambda * sum(|w|) / 2 (Regularization.scala:30-44); added to *loss.
-__global__ __launch_bounds__(256) void penalty_kernel(const float* __restrict__ w, int64_t n, int reg, float lambda, float* loss) {
+// Two stages like the losses: per-block partial sums, then one block adds them in order and finishes the term.
+__global__ __launch_bounds__(256) void penalty_stage1_kernel(const float* __restrict__ w, int64_t n, int reg, float* __restrict__ partials) {
   __shared__ float smem[4];
   float s = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += reg == SN_REG_L2 ? w[i] * w[i] : fabsf(w[i]);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) s += reg == SN_REG_L2 ? w[i] * w[i] : fabsf(w[i]);
+  const float t = block_sum(s, smem);
+  if (threadIdx.x == 0) partials[blockIdx.x] = t;
+}
+
+__global__ __launch_bounds__(256) void penalty_stage2_kernel(const float* __restrict__ partials, int n_partials, float lambda, float* loss) {
+  __shared__ float smem[4];
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n_partials; i += blockDim.x) s += partials[i];
   const float t = block_sum(s, smem);
   if (threadIdx.x == 0) *loss = *loss + (lambda * t) / 2.0f;
 }
 
-int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev) {
+int launch_penalty(sn_ctx* ctx, const float* w, int64_t n, int reg_kind, float lambda, float* loss_dev, float* partials) {
+  const unsigned blocks = (unsigned)std::min<int64_t>(LOSS_BLOCKS_MAX, std::max<int64_t>(1, ceil_div(n, 2048)));
   LaunchScope scope(ctx, "penalty");
-  hipLaunchKernelGGL(penalty_kernel, dim3(1), dim3(256), 0, ctx->stream, w, n, reg_kind, lambda, loss_dev);
+  hipLaunchKernelGGL(penalty_stage1_kernel, dim3(blocks), dim3(256), 0, ctx->stream, w, n, reg_kind, partials);
+  hipLaunchKernelGGL(penalty_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, (const float*)partials, (int)blocks, lambda, loss_dev);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

@@ -25,6 +25,8 @@ struct ParamDef {
   // the frozen model a TrainedModel holds leaves it out; Dense and the RNN cells add theirs always.
   bool penalty_when_frozen = true;
 };
+// ParamDef.aggregation of the tensor is `Some(Avg)` (info.aggregated = 1) for everything but the carried state of a
+// stateful RNN (layer/RNN.scala:188,302-303), which aggregateParams re-initialises (optimizers/Optimizer.scala:207-210).
 
 struct Op {
   OpKind kind;
@@ -42,6 +44,9 @@ struct Op {
   int lstm_p[4][3] = {{-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}, {-1, -1, -1}};  // gate x {kernel, recurrent, bias}
   // batch norm: beta, gamma, moving mean, moving variance
   int bn_p[4] = {-1, -1, -1, -1};
+  // stateful RNN (layer/RNN.scala:27,34,66-67): parameter indices of the carried state, LSTM {cell_state, hidden_state},
+  // simple cell {state, -}; -1 = the layer starts every batch from zeros
+  int state_p[2] = {-1, -1};
   float bn_momentum = 0.99f, bn_epsilon = 1e-3f;
   bool bn_fused = false;  // the FusedBatchNormV3 branch (rank-4 input unless fused = Some(false)), wired as the reference wires it
   // buffers (indices into replica buffer table), assigned at replica creation
@@ -139,10 +144,11 @@ static void conv_out(int padding, int in, int k, int s, int* out, int* pad_befor
 }
 
 static int add_param(sn_model* m, const std::string& path, const std::vector<int64_t>& dims, int reg_kind, float reg_lambda,
-                     bool trainable = true, bool penalty_when_frozen = true) {
+                     bool trainable = true, bool penalty_when_frozen = true, bool aggregated = true) {
   ParamDef p;
   memset(&p.info, 0, sizeof(p.info));
   p.info.trainable = trainable ? 1 : 0;
+  p.info.aggregated = aggregated ? 1 : 0;
   snprintf(p.info.path, sizeof(p.info.path), "%s", path.c_str());
   p.info.rank = (int32_t)dims.size();
   p.info.size = 1;
@@ -289,6 +295,10 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         op.kind = OP_LSTM;
         op.T = (int)cur[0]; op.F = (int)cur[1]; op.H = L.units;
         static const char* gates[4] = {"forget", "input", "gate", "output"};  // layer/RNN.scala:285-289
+        if (L.stateful) {  // `state ++ weights` (RNN.scala:32-35): (batch, units), Zeros, not trainable, no aggregation (:302-303)
+          op.state_p[0] = add_param(m, prefix(i) + "cell_state", {B, op.H}, SN_REG_NONE, 0.f, false, false, false);
+          op.state_p[1] = add_param(m, prefix(i) + "hidden_state", {B, op.H}, SN_REG_NONE, 0.f, false, false, false);
+        }
         for (int gi = 0; gi < 4; ++gi) {
           const std::string gp = prefix(i) + gates[gi];
           // every gate is a SimpleRNNCell ?>> Bias with the layer's three regularizers (RNN.scala:270-283,198-199)
@@ -337,6 +347,8 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         op.T = (int)cur[0]; op.F = (int)cur[1]; op.H = L.units;
         op.act = L.activation;
         op.act_param = L.act_param;
+        if (L.stateful)  // the cell's previous product (RNN.scala:188,195-196)
+          op.state_p[0] = add_param(m, prefix(i) + "0/state", {B, op.H}, SN_REG_NONE, 0.f, false, false, false);
         op.lstm_p[0][0] = add_param(m, prefix(i) + "0/kernel_weights", {op.F, op.H}, L.reg_kind, L.reg_lambda);  // RNN.scala:165-166,198-203
         op.lstm_p[0][1] = add_param(m, prefix(i) + "0/recurrent_weights", {op.H, op.H}, L.recurrent_reg_kind, L.recurrent_reg_lambda);
         if (L.use_bias) op.b = add_param(m, prefix(i) + "1/weights", {op.H}, L.bias_reg_kind, L.bias_reg_lambda, true, false);
@@ -387,12 +399,14 @@ static int dev_alloc(sn_replica* r, T** out, int64_t elems) {
 
 static bool dense_bf16_fast(const sn_model* m, const struct Op& op);
 // A hidden Dense layer of the bf16 path whose successor is another one hands its output over as bf16 copies; its
-// fp32 output has no other reader when the activation's gradient needs only the sign of the output (ReLU) or nothing.
+// fp32 output has no other reader when the activation's gradient needs only the sign of the output (ReLU at zero) or nothing.
 static bool hidden_f32_not_needed(const sn_model* m, size_t i) {
   if (i + 1 >= m->ops.size()) return false;
   const Op& op = m->ops[i];
-  return dense_bf16_fast(m, op) && dense_bf16_fast(m, m->ops[i + 1]) && (op.act == SN_ACT_RELU || op.act == SN_ACT_IDENTITY) &&
-         m->batch % 8 == 0;
+  // ReLU with a threshold other than zero keeps its fp32 output: the gradient is (threshold < y) in fp32 (`Max.localGrad`),
+  // clamped outputs equal the threshold exactly, and bf16 may round the threshold to either side of itself.
+  const bool sign_is_enough = op.act == SN_ACT_IDENTITY || (op.act == SN_ACT_RELU && op.act_param == 0.f);
+  return dense_bf16_fast(m, op) && dense_bf16_fast(m, m->ops[i + 1]) && sign_is_enough && m->batch % 8 == 0;
 }
 
 // The 256x256 bf16 kernel needs 16-byte chunks of 8 k-values in every operand row.
@@ -579,16 +593,22 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         const LstmWeights w = lstm_weights(r, op, r->w);
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
         if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr));
+        // stateful: the first step starts from the carried state (slice 0 of the hidden slices otherwise stays zero)
+        const bool carried = op.state_p[0] >= 0;
+        if (carried)
+          SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[1]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
+                                ctx->stream));
         for (int t = 0; t < op.T; ++t) {
-          const float* h_prev = r->lstm_h[i] + (int64_t)t * bh;
+          const float* h_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
+          const float* c_prev = t == 0 ? (carried ? param_ptr(r, r->w, op.state_p[0]) : nullptr) : r->lstm_c[i] + (int64_t)(t - 1) * bh;
           if (fused) {
-            SN_TRY(launch_lstm_step_fwd(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh,
+            SN_TRY(launch_lstm_step_fwd(ctx, in, t, op.T, op.F, h_prev, c_prev,
                                         rows, op.H, w, r->lstm_pk_fwd[i], r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                                         r->lstm_h[i] + (int64_t)(t + 1) * bh));
             continue;
           }
-          SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, t == 0 ? nullptr : h_prev, rows, op.H, w, r->lstm_z, r->ws, m->workspace_elems));
-          LstmGateArgs a{r->lstm_z, t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, r->lstm_gates[i] + (int64_t)t * bh * 4,
+          SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, h_prev, rows, op.H, w, r->lstm_z, r->ws, m->workspace_elems));
+          LstmGateArgs a{r->lstm_z, c_prev, r->lstm_gates[i] + (int64_t)t * bh * 4,
                          r->lstm_c[i] + (int64_t)t * bh, r->lstm_h[i] + (int64_t)(t + 1) * bh};
           SN_TRY(launch_lstm_gates_fwd(ctx, a, rows, op.H));
         }
@@ -609,8 +629,12 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         const LstmWeights w = lstm_weights(r, op, r->w);  // slot 0 only, no bias inside the recurrence
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
         if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr, 1));
+        const bool carried = op.state_p[0] >= 0;  // stateful: slice 0 is the product the previous batch ended with
+        if (carried)
+          SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[0]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
+                                ctx->stream));
         for (int t = 0; t < op.T; ++t) {
-          const float* r_prev = t == 0 ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
+          const float* r_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
           float* r_t = r->lstm_h[i] + (int64_t)(t + 1) * bh;
           if (fused) SN_TRY(launch_rnn_step_fwd(ctx, in, t, op.T, op.F, r_prev, rows, op.H, r->lstm_pk_fwd[i], r_t));
           else SN_TRY(launch_lstm_z(ctx, in, t, op.T, op.F, r_prev, rows, op.H, w, r_t, r->ws, m->workspace_elems, 1));
@@ -632,7 +656,7 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
 static int add_penalties(sn_replica* r, bool training) {
   for (auto& p : r->model->params)
     if (p.reg_kind != SN_REG_NONE && (training || p.penalty_when_frozen))
-      SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev));
+      SN_TRY(launch_penalty(r->ctx, r->w + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda, r->loss_dev, r->loss_partials));
   return SN_OK;
 }
 
@@ -790,7 +814,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
         for (int t = op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
-                            t == 0 ? nullptr : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
+                            t == 0 ? param_ptr(r, r->w, op.state_p[0]) : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
                             r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0, dh_parts, bh};
           if (op.ret_seq) {  // this step's own output gradient joins what the later steps carried back
             a.dy_seq = dy + (int64_t)t * op.H;
@@ -914,10 +938,25 @@ static int update(sn_replica* r, int iter) {
   for (const auto& run : m->trainable_runs)
     SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,
                             r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter));
-  for (size_t i = 0; i < m->ops.size(); ++i)
-    if (m->ops[i].kind == OP_BATCHNORM)
-      SN_TRY(launch_batchnorm_moving(r->ctx, batchnorm_args(r, m->ops[i], (int)i), param_ptr(r, r->w, m->ops[i].bn_p[2]),
-                                     param_ptr(r, r->w, m->ops[i].bn_p[3]), (int)m->ops[i].out_dims.back()));
+  for (size_t i = 0; i < m->ops.size(); ++i) {
+    const Op& op = m->ops[i];
+    if (op.kind == OP_BATCHNORM)
+      SN_TRY(launch_batchnorm_moving(r->ctx, batchnorm_args(r, op, (int)i), param_ptr(r, r->w, op.bn_p[2]),
+                                     param_ptr(r, r->w, op.bn_p[3]), (int)op.out_dims.back()));
+    if ((op.kind == OP_LSTM || op.kind == OP_SRNN) && op.state_p[0] >= 0) {
+      // the state the last step left is where the next batch starts (layer/RNN.scala:66-72; LSTM: c and h, :338; simple
+      // cell: its product, :195-196).  Training passes always run full batches, so whole slices move.
+      const size_t bytes = (size_t)m->batch * op.H * sizeof(float);
+      const int64_t bh = (int64_t)m->batch * op.H;
+      const float* last_h = r->lstm_h[i] + (int64_t)op.T * bh;
+      if (op.kind == OP_LSTM) {
+        SN_HIP(hipMemcpyAsync(param_ptr(r, r->w, op.state_p[0]), r->lstm_c[i] + (int64_t)(op.T - 1) * bh, bytes, hipMemcpyDeviceToDevice, r->ctx->stream));
+        SN_HIP(hipMemcpyAsync(param_ptr(r, r->w, op.state_p[1]), last_h, bytes, hipMemcpyDeviceToDevice, r->ctx->stream));
+      } else {
+        SN_HIP(hipMemcpyAsync(param_ptr(r, r->w, op.state_p[0]), last_h, bytes, hipMemcpyDeviceToDevice, r->ctx->stream));
+      }
+    }
+  }
   return SN_OK;
 }
 
@@ -1336,6 +1375,8 @@ int sn_replicas_average(sn_replica* const* reps, int32_t k) {
   for (int i = 0; i < k; ++i) {
     SN_TRY(check_replica(reps[i]));
     SN_REQUIRE(reps[i]->model == reps[0]->model, "replica %d belongs to another model", i);
+    // replicas of one model share its context, hence its stream: the launches below are ordered behind every replica's steps
+    SN_REQUIRE(reps[i]->ctx == reps[0]->ctx, "replica %d lives in another context", i);
     SN_REQUIRE(reps[i]->n_states == reps[0]->n_states && (!reps[i]->has_opt || reps[i]->opt.kind == reps[0]->opt.kind),
                "replica %d uses another optimizer", i);
   }
@@ -1353,6 +1394,10 @@ int sn_replicas_average(sn_replica* const* reps, int32_t k) {
     }
     SN_TRY(launch_average(ctx, in, k, n, outs[0], outs + 1, k - 1));
   }
+  // tensors without an aggregation start over from their initializer, Zeros (optimizers/Optimizer.scala:207-210)
+  for (const ParamDef& p : reps[0]->model->params)
+    if (!p.info.aggregated)
+      for (int i = 0; i < k; ++i) SN_TRY(launch_fill(ctx, reps[i]->w + p.info.offset, 0.f, p.info.size));
   return SN_OK;
 }
 

@@ -26,6 +26,7 @@ OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter) {
   s.bc1 = 1.0f - (float)std::pow((double)d.beta1, (double)iter);
   s.bc2 = 1.0f - (float)std::pow((double)d.beta2, (double)iter);
   s.nesterov = d.nesterov;
+  s.maximize = d.maximize;
   return s;
 }
 
@@ -92,7 +93,7 @@ __device__ __forceinline__ void update_one(float& w, float g, float& s0, float& 
     s1 = v_cur;
     s2 = v;
   }
-  w = w - delta;  // Optimizer.scala:186 (minimizing)
+  w = p.maximize ? w + delta : w - delta;  // Optimizer.scala:186: `if (minimizing) w - del else w + del`
 }
 
 template <int KIND>

@@ -241,6 +241,7 @@ class Layer:
     pool_reduce: int = 0          # Pool2D: L.POOL_MAX or L.POOL_AVG
     recurrent_reg: Regularization = Zero   # RNN layers: `recurrentReg`, `biasReg` (`reg` is their `kernelReg`)
     bias_reg: Regularization = Zero
+    stateful: bool = False        # RNN layers: the state the last step leaves starts the next batch (layer/RNN.scala:27)
 
     def __rshift__(self, other):
         return Composed.of(self, other)
@@ -254,7 +255,8 @@ class Layer:
                            self.strides[0], self.strides[1], self.padding, self.reg.kind, self.reg.lam, 1 if self.use_bias else 0,
                            1 if self.return_sequence else 0, self.momentum, self.epsilon,
                            self.explicit[0], self.explicit[1], self.explicit[2], self.explicit[3], self.fused,
-                           self.recurrent_reg.kind, self.recurrent_reg.lam, self.bias_reg.kind, self.bias_reg.lam, self.pool_reduce)
+                           self.recurrent_reg.kind, self.recurrent_reg.lam, self.bias_reg.kind, self.bias_reg.lam, self.pool_reduce,
+                           1 if self.stateful else 0)
 
     def __repr__(self):
         return self.text
@@ -338,11 +340,11 @@ Flatten = Layer(L.LAYER_FLATTEN, "Flatten")
 def LSTM(units: int, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
          recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
          biasForgetInitializer: Initializer = Ones, returnSequence: bool = False, kernelReg: Regularization = Zero,
-         recurrentReg: Regularization = Zero, biasReg: Regularization = Zero) -> Layer:
+         recurrentReg: Regularization = Zero, biasReg: Regularization = Zero, stateful: bool = False) -> Layer:
     """layer/RNN.scala:208-258: tanh cell, sigmoid gates, forget bias one; the three regularizers apply to every gate."""
     return Layer(L.LAYER_LSTM, f"RNN(LSTMCell({units},Tanh,Sigmoid,{'true' if bias else 'false'}))", units=units,
                  activation=Tanh, use_bias=bias, return_sequence=returnSequence, reg=kernelReg, recurrent_reg=recurrentReg,
-                 bias_reg=biasReg,
+                 bias_reg=biasReg, stateful=stateful,
                  inits=(kernelInitializer, recurrentInitializer, biasInitializer, biasForgetInitializer))
 
 
@@ -364,13 +366,13 @@ def BatchNorm(axes: Sequence[int] = (-1,), momentum: float = 0.99, epsilon: floa
 def SimpleRNN(units: int, activation: Activation = Tanh, bias: bool = True, kernelInitializer: Initializer = GlorotUniform(),
               recurrentInitializer: Initializer = Orthogonal(), biasInitializer: Initializer = Zeros,
               returnSequence: bool = False, kernelReg: Regularization = Zero, recurrentReg: Regularization = Zero,
-              biasReg: Regularization = Zero) -> Layer:
+              biasReg: Regularization = Zero, stateful: bool = False) -> Layer:
     """layer/RNN.scala:96-137: `RNN(SimpleRNNCell(..))`; the last step's output leaves the layer."""
     if activation.kind == L.ACT_SOFTMAX:
         raise ValueError("requirement failed: Softmax is not a cell activation")
     return Layer(L.LAYER_SIMPLE_RNN, f"RNN(SimpleRNNCell({units},{activation!r},{'true' if bias else 'false'}))", units=units,
                  activation=activation, use_bias=bias, return_sequence=returnSequence, reg=kernelReg, recurrent_reg=recurrentReg,
-                 bias_reg=biasReg, inits=(kernelInitializer, recurrentInitializer, biasInitializer))
+                 bias_reg=biasReg, stateful=stateful, inits=(kernelInitializer, recurrentInitializer, biasInitializer))
 
 
 def LinearRegression(reg: Regularization = Zero, bias: bool = True):
@@ -387,7 +389,7 @@ def LogisticRegression(reg: Regularization = Zero, bias: bool = True):
 
 
 def _alg(kind, rate=0.0, beta1=0.0, beta2=0.0, epsilon=0.0, init_acc=0.0, nesterov=False) -> L.OptimizerDesc:
-    return L.OptimizerDesc(kind, rate, beta1, beta2, epsilon, init_acc, 1 if nesterov else 0)
+    return L.OptimizerDesc(kind, rate, beta1, beta2, epsilon, init_acc, 1 if nesterov else 0, 0)
 
 
 def SGD(rate=0.01, momentum=0.0, nesterov=False):
@@ -460,6 +462,16 @@ class Dataset:
         return Builder(model=model, dataset=self)
 
 
+def minimize(model) -> "Builder":
+    """`Optimizer.minimize(model)` (optimizers/Optimizer.scala:312-324)."""
+    return Builder(model=model)
+
+
+def maximize(model) -> "Builder":
+    """`Optimizer.maximize(model)` (optimizers/Optimizer.scala:326-336): every update adds its delta."""
+    return Builder(model=model, minimizing=False)
+
+
 Skip, Partial, PadZeros = "Skip", "Partial", "PadZeros"
 
 
@@ -522,12 +534,17 @@ def _init_params(model, compiled: CompiledModel, seed: int) -> Dict[str, np.ndar
             for name, init in zip(("beta", "gamma", "moving_mean", "moving_variance"), l.inits):
                 out[pre + name] = init.build(shapes[pre + name], compiled.ctx, rng)
         elif l.kind == L.LAYER_SIMPLE_RNN:
+            if l.stateful:
+                out[pre + "0/state"] = np.zeros(shapes[pre + "0/state"], np.float32)          # RNN.scala:188
             k_init, r_init, b_init = l.inits
             out[pre + "0/kernel_weights"] = k_init.build(shapes[pre + "0/kernel_weights"], compiled.ctx, rng)
             out[pre + "0/recurrent_weights"] = r_init.build(shapes[pre + "0/recurrent_weights"], compiled.ctx, rng)
             if l.use_bias:
                 out[pre + "1/weights"] = b_init.build(shapes[pre + "1/weights"], compiled.ctx, rng)
         elif l.kind == L.LAYER_LSTM:
+            if l.stateful:
+                for name in ("cell_state", "hidden_state"):                                      # RNN.scala:302-303
+                    out[pre + name] = np.zeros(shapes[pre + name], np.float32)
             k_init, r_init, b_init, bf_init = l.inits
             for gate in ("forget", "input", "gate", "output"):
                 out[f"{pre}{gate}/0/kernel_weights"] = k_init.build(shapes[f"{pre}{gate}/0/kernel_weights"], compiled.ctx, rng)
@@ -718,6 +735,7 @@ class Builder:
     seed: int = 0
     device: int = 0
     board_dir: str = "board"                     # Optimizer.scala:54
+    minimizing: bool = True                      # Optimizer.scala:186: w - delta, or w + delta for `Optimizer.maximize`
 
     def board(self, directory: str):
         """Directory of the TensorBoard event files effects write (Optimizer.scala:297-298)."""
@@ -774,7 +792,9 @@ class Builder:
                 xb, yb = ctx.to_device(px), ctx.to_device(py)
                 bufs += [xb, yb]
                 data.append((xb, yb, px.shape[0]))
-                rep = cm.replica(self.alg)
+                alg = L.OptimizerDesc.from_buffer_copy(self.alg)
+                alg.maximize = 0 if self.minimizing else 1
+                rep = cm.replica(alg)
                 rep.set_params(params)
                 reps.append(rep)
             global_iter, epoch, history = 0, 0, []

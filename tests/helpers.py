@@ -116,8 +116,27 @@ def one_hot(rng, rows, classes):
     return np.eye(classes, dtype=f32)[rng.integers(0, classes, rows)]
 
 
-def rel_err(a: np.ndarray, b: np.ndarray) -> float:
-    """max |a-b| relative to the largest magnitude of the reference tensor b."""
+ATOL_FRACTION = 0.25
+
+
+def rel_err(a: np.ndarray, b: np.ndarray, atol_fraction: float = ATOL_FRACTION) -> float:
+    """Mixed elementwise error of `a` against the reference tensor `b`: max_i |a_i - b_i| / (|b_i| + f * max|b|).
+
+    `rel_err(a, b) <= tol` therefore means |a_i - b_i| <= tol * |b_i| + f * tol * max|b| for every element: relative to
+    the element itself, plus an absolute floor of a quarter of the tolerance at the tensor's scale (an entry that is
+    small because its terms cancel carries the rounding error of those terms, not of its own size)."""
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    if a.size != b.size:
+        raise AssertionError(f"size mismatch: {a.shape} vs {b.shape}")
+    a = a.reshape(b.shape)
+    if b.size == 0:
+        return 0.0
+    floor = atol_fraction * max(float(np.max(np.abs(b))), 1e-30)
+    return float(np.max(np.abs(a - b) / (np.abs(b) + floor)))
+
+
+def norm_err(a: np.ndarray, b: np.ndarray) -> float:
+    """max |a-b| relative to the largest magnitude of the reference tensor b (a yardstick for noise estimates)."""
     a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
     denom = max(float(np.max(np.abs(b))), 1e-30)
     return float(np.max(np.abs(a - b))) / denom

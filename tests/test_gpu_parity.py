@@ -1,7 +1,9 @@
 """Parity of the HIP library (through its C ABI) with the CPU oracle on identical seeded inputs,
 and with the reference's own golden vectors.  Needs an MI355X: run with `-m gpu`.
 
-Tolerances (relative to the largest magnitude of the reference tensor):
+Tolerances (helpers.rel_err: |a - b| <= tol * |b| + tol/4 * max|b| for every element; the bf16 mode, where a flipped
+rounding of one activation moves a gradient entry by an amount unrelated to that entry's size, is measured relative to
+the largest magnitude of the reference tensor, helpers.norm_err):
   optimizer updates, activations, averaging ... 1e-6
   GEMM / convolution outputs and gradients ..... 1e-4
   loss trajectories ............................ 1e-3
@@ -13,13 +15,14 @@ import numpy as np
 import pytest
 
 from oracle import scanet_oracle as O
-from tests.helpers import build_pair, f32, glorot_params, one_hot, optimizer_pairs, rel_err
+from tests.helpers import build_pair, f32, glorot_params, norm_err, one_hot, optimizer_pairs, rel_err
 
 pytestmark = pytest.mark.gpu
 
 TOL_ELEMENTWISE = 1e-6
 TOL_GEMM = 1e-4
 TOL_TRAJECTORY = 1e-3
+TOL_FINAL_WEIGHTS = 2e-4   # weights after a short trajectory, unless float32 rounding itself moves them further (see the tests)
 
 
 @pytest.fixture(scope="module")
@@ -485,8 +488,11 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     assert rel_err(h.rep.forward(xb, training=True), om.forward(x, params, training=True)) <= TOL_GEMM
     ggrads = h.rep.get_grads()
     assert set(ggrads) == set(ograds)
+    # the same gradients in float64 say how far float32 rounding alone moves each tensor of THIS model: the library may be
+    # 3 times as far from the float32 oracle as that, and never has to be closer than the fixed tolerance
+    _, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
     for p in ograds:
-        assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_GEMM, 3.0 * rel_err(ograds[p], grads64[p])), p
     # partial batch (the accuracy estimator feeds one): rows < batch must give the same per-row predictions
     rows = max(1, batch // 3)
     np.testing.assert_allclose(h.rep.forward(xb, rows), pred[:rows], rtol=1e-6, atol=1e-7)
@@ -512,15 +518,23 @@ def test_loss_trajectory_matches_oracle(S, ctx, name, steps, alg):
     h.rep.set_params(params)
     Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
     ostate = O.init_opt_state(oalg, params)
+    # the same steps in float64: how far rounding alone moves this trajectory (see test_full_config_trajectory_matches_oracle)
+    params64 = {p: v.astype(np.float64) for p, v in params.items()}
+    ostate64 = O.init_opt_state(oalg, params64)
+    noise = 0.0
     for t in range(1, steps + 1):
         b = (t - 1) % n_batches
         xs, ys = X[b * batch:(b + 1) * batch], Y[b * batch:(b + 1) * batch]
         params, ostate, oloss, _ = O.train_step(om, oalg, xs, ys, params, ostate, t)
+        params64, ostate64, oloss64, _ = O.train_step(om, oalg, xs.astype(np.float64), ys.astype(np.float64), params64, ostate64, t)
+        scale = max(1.0, abs(float(oloss)))
+        noise = max(noise, abs(float(oloss64) - float(oloss)) / scale)
         gloss = h.rep.step(Xb.offset(b * batch * int(np.prod(in_shape))), Yb.offset(b * batch * out_dim), t, want_loss=True)
-        assert abs(gloss - float(oloss)) <= TOL_TRAJECTORY * max(1.0, abs(float(oloss))), (t, gloss, float(oloss))
+        assert abs(gloss - float(oloss)) / scale <= max(TOL_TRAJECTORY, 3.0 * noise), (t, gloss, float(oloss), noise)
     got = h.rep.get_params()
+    own = max(rel_err(params[p], params64[p]) for p in params)
     for p in params:
-        assert rel_err(got[p], params[p]) <= 2e-3, p
+        assert rel_err(got[p], params[p]) <= max(TOL_FINAL_WEIGHTS, 10.0 * own), (p, own)
     h.close()
 
 
@@ -566,6 +580,91 @@ def test_full_config_lenet_and_lstm_one_step(S, ctx):
         h.close()
         xb.free()
         yb.free()
+
+
+# The benchmark configurations at their own size AND length: every step's loss, then the final weights and both Adam
+# state tensors.  name -> (layer spec, loss, sample shape, batch, data kind, Adam rate, steps, bf16 Dense mode, twin)
+# `twin`: None where float32 rounding stays small over the whole run (the tolerances are then fixed numbers), else the
+# kind of second oracle run that measures how far rounding alone moves THIS trajectory: "float64" = the same steps
+# in double precision, "permuted" = the same bf16-rounded steps with the first layer's reduction index permuted.
+FULL_TRAJECTORIES = {
+    "mlp_784_50_10_batch1000_10_steps": ([("dense", 50, "sigmoid"), ("dense", 10, "softmax")], "cce", (784,), 1000, "uniform_onehot",
+                                         0.01, 10, False, None),
+    "lenet_batch100_100_steps": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+                                  ("conv", 64, (3, 3), (1, 1), "valid", "relu", False), ("pool", (2, 2), (1, 1), "valid"),
+                                  ("flatten",), ("dense", 10, "softmax")], "cce", (28, 28, 1), 100, "uniform_onehot", 1e-3, 100, False,
+                                 "float64"),
+    "lstm256_batch512_T64_50_steps": ([("lstm", 256), ("dense", 1, "tanh")], "mse", (64, 32), 512, "normal_regression", 1e-3, 50, False,
+                                      None),
+    "wide_mlp_bf16_batch8192_20_steps": ([("dense", 4096, "relu"), ("dense", 4096, "relu"), ("dense", 1000, "softmax")], "cce", (4096,),
+                                         8192, "normal_onehot", 1e-3, 20, True, "permuted"),
+}
+# without a twin: loss of every step, final weights, final Adam moments (observed: 1e-7, 7e-6, 5e-5)
+TOL_FULL_LOSS, TOL_FULL_WEIGHTS, TOL_FULL_MOMENTS = 1e-5, 5e-5, 2e-4
+
+
+@pytest.mark.parametrize("name", list(FULL_TRAJECTORIES))
+def test_full_config_trajectory_matches_oracle(S, ctx, name):
+    """`optimizeOnPartition`'s loop (Optimizer.scala:136-157) at a benchmark configuration's own size for its own
+    number of steps: the loss of every step against the oracle's, then weights and Adam moments at the end.
+
+    The LeNet run (uniform [0,1) pixels, random labels, Adam) drives its loss from 2.4 up to 9 and back down: rounding
+    differences grow along it, and the float32 oracle itself ends 2e-3 away from the same steps in float64.  For that
+    run and for the bf16 one the library may be at most 3 times as far from the oracle as the oracle is from its twin
+    (largest distance seen so far along the run) in every step's loss; at the end every tensor may be 10 times as far as
+    the twin's worst tensor of the same kind (two float32 runs differ from each other by more than either differs from
+    float64, and the per-tensor ratio of two noise samples scatters widely: measured 0.3 to 6).  Neither has to be
+    closer than the fixed tolerances."""
+    from scanet3_amd import _lib as L
+    spec, loss, in_shape, batch, kind, rate, steps, bf16, twin = FULL_TRAJECTORIES[name]
+    rng = np.random.default_rng(20251125 + 11)
+    h = Harness(S, ctx, spec, loss, in_shape, batch, S.Adam(rate), flags=L.FLAG_GEMM_BF16 if bf16 else 0)
+    om = O.Model(h.omodel.layers, h.omodel.loss, bf16_dense=True) if bf16 else h.omodel
+    oalg = O.Adam(rate)
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    out_dim = om.out_shape((batch,) + in_shape)[-1]
+    n_batches = 2 if bf16 else 4            # the steps cycle over a few resident batches, as an epoch loop would
+    X, Y = make_data(kind, rng, batch * n_batches, in_shape, out_dim)
+    h.rep.set_params(params)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    ostate = O.init_opt_state(oalg, params)
+    # the twin run and how to read its tensors back in the first run's layout
+    first = next(iter(params))
+    if twin == "float64":
+        X2, Y2 = X.astype(np.float64), Y.astype(np.float64)
+        params2 = {p: v.astype(np.float64) for p, v in params.items()}
+    elif twin == "permuted":
+        perm = rng.permutation(in_shape[0])
+        X2, Y2 = np.ascontiguousarray(X[:, perm]), Y
+        params2 = dict(params)
+        params2[first] = np.ascontiguousarray(params[first][perm])
+    if twin:
+        ostate2 = O.init_opt_state(oalg, params2)
+    back = (lambda p, v: v[np.argsort(perm)] if p == first else v) if twin == "permuted" else (lambda p, v: v)
+    xs_elems = batch * int(np.prod(in_shape))
+    tol_loss = (TOL_BF16 if bf16 else TOL_TRAJECTORY) if twin else TOL_FULL_LOSS
+    noise = 0.0
+    for t in range(1, steps + 1):
+        b = (t - 1) % n_batches
+        rows = slice(b * batch, (b + 1) * batch)
+        params, ostate, oloss, _ = O.train_step(om, oalg, X[rows], Y[rows], params, ostate, t)
+        scale = max(1.0, abs(float(oloss)))
+        if twin:
+            params2, ostate2, oloss2, _ = O.train_step(om, oalg, X2[rows], Y2[rows], params2, ostate2, t)
+            noise = max(noise, abs(float(oloss2) - float(oloss)) / scale)
+        gloss = h.rep.step(Xb.offset(b * xs_elems), Yb.offset(b * batch * out_dim), t, want_loss=True)
+        assert abs(gloss - float(oloss)) / scale <= max(tol_loss, 3.0 * noise), (t, gloss, float(oloss), noise)
+    got = [h.rep.get_params(), h.rep.get_opt_state(0), h.rep.get_opt_state(1)]
+    measure = norm_err if bf16 else rel_err
+    want = {p: (params[p], ostate[p][0], ostate[p][1]) for p in params}
+    for k, tol in enumerate((TOL_FULL_WEIGHTS, TOL_FULL_MOMENTS, TOL_FULL_MOMENTS)):
+        # the twin's largest distance among the tensors of this kind (weights, first moments, second moments)
+        own = max(measure(back(p, (params2[p], ostate2[p][0], ostate2[p][1])[k]), want[p][k]) for p in params) if twin else 0.0
+        for p in params:
+            assert measure(got[k][p], want[p][k]) <= max(tol, 10.0 * own), (p, k, own)
+    h.close()
+    Xb.free()
+    Yb.free()
 
 
 @pytest.fixture(scope="module")
@@ -642,11 +741,11 @@ def test_full_config_wide_mlp_bf16_one_step(S, ctx):
     _, g2 = om.grad(x[:, perm], y, p2)
     g2["0/weights"] = g2["0/weights"][np.argsort(perm)]
     for p in ograds:
-        noise = rel_err(g2[p], ograds[p])
-        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_BF16, 3 * noise), (p, noise)
+        noise = norm_err(g2[p], ograds[p])
+        assert norm_err(ggrads[p], ograds[p]) <= max(TOL_BF16, 3 * noise), (p, noise)
     pred = h.rep.forward(xb)
     np.testing.assert_allclose(pred.sum(axis=1), 1.0, rtol=0, atol=1e-4)     # rows of a softmax
-    assert rel_err(pred, om.forward(x, params)) <= TOL_BF16
+    assert norm_err(pred, om.forward(x, params)) <= TOL_BF16
     h.close()
     xb.free()
     yb.free()
@@ -814,7 +913,10 @@ def test_dsl_training_run_matches_oracle_and_thresholds(S, golden, linear_functi
 
 
 def test_k_replica_training_matches_oracle(S, linear_function):
-    """K = 3 partitions: per-epoch broadcast, independent epochs, uniform average, summed iterations."""
+    """K = 3 partitions: per-epoch broadcast, independent epochs, summed iterations, and the UNIFORM mean of the three
+    replicas, checked against the oracle's own uniform mean.  The reference folds pairs in Spark's order instead
+    (Optimizer.scala:86,205-210: weights like 1/4, 1/4, 1/2) and no reference test runs it, so this pins the library
+    against the build's stated K-way mean, not against the reference; K > 2 parity is unpinned."""
     X, Y = linear_function
     X, Y = X[:96], Y[:96]
     om = O.Model([O.Dense(1)], O.LOSS_MSE)
@@ -827,6 +929,138 @@ def test_k_replica_training_matches_oracle(S, linear_function):
     np.testing.assert_allclose(trained.history, ohist, rtol=TOL_TRAJECTORY)
     for p in oparams:
         assert rel_err(trained.params[p], oparams[p]) <= 1e-4
+
+
+@pytest.mark.parametrize("kind,units,features,batch", [("lstm", 32, 8, 64), ("lstm", 6, 3, 10), ("simple_rnn", 32, 8, 64), ("simple_rnn", 5, 3, 9)])
+def test_stateful_rnn_steps_match_oracle(S, ctx, kind, units, features, batch):
+    """`RNN(cell, stateful = true)` (RNN.scala:27,34,66-72) through the fused step kernels (32 units) and the tiled path:
+    every step starts from the state the one before left, which sits in the parameter table as a non-trainable,
+    non-aggregated tensor; `sn_grad` and the forward calls read it without moving it."""
+    T, steps = 5, 6
+    rng = np.random.default_rng(20251125 + 13)
+    olayer = O.LSTM(units, stateful=True) if kind == "lstm" else O.SimpleRNN(units, O.ACT_TANH, stateful=True)
+    slayer = S.LSTM(units, stateful=True) if kind == "lstm" else S.SimpleRNN(units, S.Tanh, stateful=True)
+    om = O.Model([olayer, O.Dense(1, O.ACT_TANH)], O.LOSS_MSE)
+    layers = slayer >> S.Dense(1, S.Tanh)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+    state_paths = sorted(p for p, _ in om.param_defs((batch, T, features)) if O.is_unaggregated_path(p))
+    assert sorted(cm.state_paths) == state_paths and len(state_paths) == (2 if kind == "lstm" else 1)
+    oalg, desc = O.Adam(0.01), S.Adam(0.01)
+    rep = cm.replica(desc)
+    params = glorot_params(om, (batch, T, features), rng)
+    for p in state_paths:                     # zeros at first (RNN.scala:188,302-303)
+        params[p] = np.zeros((batch, units), f32)
+    rep.set_params(params)
+    X = rng.standard_normal((steps * batch, T, features)).astype(f32)
+    Y = rng.uniform(-1, 1, (steps * batch, 1)).astype(f32)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    ostate = O.init_opt_state(oalg, params)
+    for t in range(1, steps + 1):
+        rows = slice((t - 1) * batch, t * batch)
+        if t == 3:      # a gradient and two forward passes in between must leave the carried state where it is
+            oloss, ograds = om.grad(X[rows], Y[rows], params)
+            assert abs(rep.grad(Xb.offset(rows.start * T * features), Yb.offset(rows.start)) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+            ggrads = rep.get_grads()
+            assert set(ggrads) == set(ograds)
+            for p in ograds:
+                assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+            assert rel_err(rep.forward(Xb.offset(rows.start * T * features)), om.forward(X[rows], params)) <= TOL_GEMM
+            assert rel_err(rep.forward(Xb, 3), om.forward(X[:3], params)) <= TOL_GEMM          # fewer rows than the state holds
+        params, ostate, oloss, _ = O.train_step(om, oalg, X[rows], Y[rows], params, ostate, t)
+        gloss = rep.step(Xb.offset(rows.start * T * features), Yb.offset(rows.start), t, want_loss=True)
+        assert abs(gloss - float(oloss)) <= TOL_TRAJECTORY * max(1.0, abs(float(oloss))), t
+    got = rep.get_params()
+    for p in params:
+        assert rel_err(got[p], params[p]) <= TOL_FINAL_WEIGHTS, p
+    assert all(np.any(got[p]) for p in state_paths)
+    # aggregateParams re-initialises tensors without an aggregation (Optimizer.scala:207-210)
+    rep2 = cm.replica(desc)
+    rep2.set_params(got)
+    S.average_replicas([rep, rep2])
+    for r in (rep, rep2):
+        after = r.get_params()
+        for p in params:
+            if p in state_paths:
+                assert not np.any(after[p]), p
+            else:
+                np.testing.assert_array_equal(after[p], got[p])
+    for o in (rep, rep2, cm):
+        o.close()
+    Xb.free()
+    Yb.free()
+
+
+def test_maximizing_step_adds_the_delta(S, ctx):
+    """`Optimizer.maximize` (Optimizer.scala:186,326-336): w + delta, through the flat kernel and through sn_step."""
+    from scanet3_amd import _lib as L
+    rng = np.random.default_rng(20251125 + 14)
+    for name, oalg, desc in optimizer_pairs():
+        up = L.OptimizerDesc.from_buffer_copy(desc)
+        up.maximize = 1
+        n = 1003
+        w, g = (rng.standard_normal(n) * 0.02).astype(f32), (rng.standard_normal(n) * 1e-3).astype(f32)
+        states = oalg.init_state((n,))
+        wb, gb, sb = ctx.to_device(w), ctx.to_device(g), [ctx.to_device(s_) for s_ in states]
+        ctx.optimizer_update(up, wb, gb, sb, 3)
+        delta, _ = oalg.build(g, states, 3)
+        assert rel_err(wb.numpy(), w + delta) <= TOL_ELEMENTWISE, name
+        for b in [wb, gb] + sb:
+            b.free()
+    om, layers, sloss = build_pair([("dense", 4, "tanh"), ("dense", 2, "identity")], "mse")
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (3,), 16)
+    desc = L.OptimizerDesc.from_buffer_copy(S.Adam(0.05))
+    desc.maximize = 1
+    rep = cm.replica(desc)
+    params = glorot_params(om, (16, 3), rng)
+    rep.set_params(params)
+    x, y = rng.standard_normal((16, 3)).astype(f32), rng.standard_normal((16, 2)).astype(f32)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    oalg = O.Adam(0.05)
+    ostate = O.init_opt_state(oalg, params)
+    losses = []
+    for t in range(1, 6):
+        params, ostate, oloss, _ = O.train_step(om, oalg, x, y, params, ostate, t, minimizing=False)
+        gloss = rep.step(xb, yb, t, want_loss=True)
+        assert abs(gloss - float(oloss)) <= TOL_TRAJECTORY * max(1.0, abs(float(oloss)))
+        losses.append(gloss)
+    assert losses[-1] > losses[0]                 # the loss climbs
+    got = rep.get_params()
+    for p in params:
+        assert rel_err(got[p], params[p]) <= TOL_FINAL_WEIGHTS, p
+    rep.close()
+    cm.close()
+    xb.free()
+    yb.free()
+
+
+def test_pairwise_fold_of_three_replicas_through_the_flat_average(S, ctx):
+    """What the reference's treeReduce computes for three partitions in one particular order: avg2(avg2(a, b), c), i.e.
+    weights 1/4, 1/4, 1/2 (Optimizer.scala:86,205-210).  `sn_replicas_average` takes the uniform mean instead; a caller that
+    wants a pairwise fold runs `sn_average` with k = 2 over the flat views in its own order."""
+    import ctypes as C
+    from scanet3_amd._lib import check, lib
+    om, layers, sloss = build_pair([("dense", 7, "tanh"), ("dense", 3, "identity")], "mse")
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (5,), 4)
+    rng = np.random.default_rng(20251125 + 15)
+    reps, values = [], []
+    for _ in range(3):
+        r = cm.replica(S.Adam())
+        v = {p: rng.standard_normal(shape).astype(f32) for p, shape, _ in cm.params}
+        r.set_params(v)
+        reps.append(r)
+        values.append(v)
+    flats = [r.flat(-2) for r in reps]
+    n = flats[0][1]
+    for a, b in ((0, 1), (0, 2)):                 # a <- avg2(a, b), twice: ((a, b), c)
+        arr = (C.c_void_p * 2)(flats[a][0], flats[b][0])
+        check(lib.sn_average(ctx.handle, arr, 2, n, flats[a][0]))
+    got = reps[0].get_params()
+    for p in got:
+        np.testing.assert_array_equal(got[p], O.avg2(O.avg2(values[0][p], values[1][p]), values[2][p]))
+        assert np.any(got[p] != O.average_uniform([v[p] for v in values]))
+    for r in reps:
+        r.close()
+    cm.close()
 
 
 def test_dsl_batch_norm_training_over_two_partitions(S):
@@ -935,17 +1169,48 @@ def test_bf16_dense_path_matches_bf16_rounded_oracle(S, ctx, dims, batch):
     y = one_hot(rng, batch, dims[-1])
     h.rep.set_params(params)
     xb, yb = ctx.to_device(x), ctx.to_device(y)
-    assert rel_err(h.rep.forward(xb), om.forward(x, params)) <= TOL_BF16
+    assert norm_err(h.rep.forward(xb), om.forward(x, params)) <= TOL_BF16
     oloss, ograds = om.grad(x, y, params)
     gloss = h.rep.grad(xb, yb)
     assert abs(gloss - float(oloss)) <= TOL_BF16 * max(1.0, abs(float(oloss)))
     ggrads = h.rep.get_grads()
     for p in ograds:
-        assert rel_err(ggrads[p], ograds[p]) <= TOL_BF16, p
+        assert norm_err(ggrads[p], ograds[p]) <= TOL_BF16, p
     # and the bf16 result stays close to the float32 one (sanity of the mode itself)
     o32 = O.Model(h.omodel.layers, O.LOSS_CCE)
     assert abs(gloss - float(o32.loss_of(x, y, params))) <= 2e-2 * max(1.0, abs(gloss))
     h.close()
+    xb.free()
+    yb.free()
+
+
+def test_bf16_hidden_relu_with_threshold_masks_in_float32(S, ctx):
+    """Hidden bf16 Dense layers under ReLU(0.1): clamped outputs equal the threshold exactly and bf16 rounds 0.1 upwards
+    (0.10009765625), so a mask read off a bf16 copy of the output would let every clamped unit pass its gradient.  The
+    reference's gradient is (threshold < x) in float32 (`Max.localGrad`, Activation.scala:79-82)."""
+    from scanet3_amd import _lib as L
+    dims, batch, t = (256, 512, 384, 104), 512, 0.1
+    olayers = [O.Dense(dims[1], O.ACT_RELU, act_param=t), O.Dense(dims[2], O.ACT_RELU, act_param=t), O.Dense(dims[3], O.ACT_SOFTMAX)]
+    om = O.Model(olayers, O.LOSS_CCE, bf16_dense=True)
+    layers = S.Dense(dims[1], S.ReLU(t)) >> S.Dense(dims[2], S.ReLU(t)) >> S.Dense(dims[3], S.Softmax)
+    rng = np.random.default_rng(20251125 + 12)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.CategoricalCrossentropy.kind, (dims[0],), batch, L.FLAG_GEMM_BF16)
+    rep = cm.replica(None)
+    params = glorot_params(om, (batch, dims[0]), rng)
+    x = rng.standard_normal((batch, dims[0])).astype(f32)
+    y = one_hot(rng, batch, dims[-1])
+    rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    hidden = O.Model(olayers[:1], O.LOSS_CCE, bf16_dense=True).forward(x, params)
+    assert 0.2 < float(np.mean(hidden == f32(t))) < 0.8          # a good share of the units sits on the threshold
+    oloss, ograds = om.grad(x, y, params)
+    gloss = rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_BF16 * max(1.0, abs(float(oloss)))
+    ggrads = rep.get_grads()
+    for p in ograds:
+        assert norm_err(ggrads[p], ograds[p]) <= TOL_BF16, p
+    rep.close()
+    cm.close()
     xb.free()
     yb.free()
 

@@ -584,6 +584,70 @@ def test_model_gradients_match_numeric_float64(name):
         np.testing.assert_allclose(grads[path], num, rtol=2e-5, atol=2e-8, err_msg=path)
 
 
+@pytest.mark.parametrize("kind", ["lstm", "simple_rnn"])
+def test_stateful_rnn_carries_its_state_between_batches(kind):
+    """`RNN(cell, stateful = true)` (RNN.scala:27,34,66-72).  No reference test runs it, so the restatement is pinned by
+    what the definition fixes: (1) with a zero state it is the stateless layer; (2) a sequence of 6 steps fed as two
+    batches of 3 steps, the second starting from the state the first one left, gives the output of the 6 steps in one
+    go; (3) the state takes no gradient and bypasses the algorithm; (4) float64 numerical gradients from a non-zero
+    state; (5) averaging re-initialises it (Optimizer.scala:207-210)."""
+    rng = np.random.default_rng(5)
+    make = (lambda **kw: O.LSTM(4, **kw)) if kind == "lstm" else (lambda **kw: O.SimpleRNN(4, O.ACT_TANH, **kw))
+    m_state = O.Model([make(stateful=True), O.Dense(1)], O.LOSS_MSE)
+    m_plain = O.Model([make(), O.Dense(1)], O.LOSS_MSE)
+    b = 3
+    x = rng.standard_normal((b, 6, 2))
+    y = rng.uniform(-1, 1, (b, 1))
+    plain = _rand_params(m_plain, x.shape, rng)
+    state_paths = [p for p, _ in m_state.param_defs(x.shape) if O.is_state_path(p)]
+    assert state_paths == (["0/cell_state", "0/hidden_state"] if kind == "lstm" else ["0/0/state"])
+    assert all(O.is_unaggregated_path(p) for p in state_paths)
+    with_state = dict(plain)
+    for p in state_paths:
+        with_state[p] = np.zeros((b, 4))
+    # (1)
+    np.testing.assert_array_equal(m_state.forward(x, with_state), m_plain.forward(x, plain))
+    # (2)
+    nxt = {}
+    m_state.forward(x[:, :3], with_state, training=True, next_state=nxt)
+    assert set(nxt) == set(state_paths)
+    second = dict(with_state)
+    second.update(nxt)
+    np.testing.assert_allclose(m_state.forward(x[:, 3:], second), m_plain.forward(x, plain), rtol=1e-12)
+    # (3)
+    alg = O.SGD(0.1)
+    new_params, _, _, grads = O.train_step(m_state, alg, x[:, :3], y, with_state, O.init_opt_state(alg, with_state), 1)
+    assert set(grads) == set(plain)
+    for p in state_paths:
+        np.testing.assert_array_equal(new_params[p], nxt[p])
+    # (4)
+    loss, grads = m_state.grad(x[:, 3:], y, second)
+    for path in grads:
+        num = _numeric_grad(m_state, x[:, 3:], y, second, path, training=True)
+        np.testing.assert_allclose(grads[path], num, rtol=2e-5, atol=2e-8, err_msg=path)
+    # (5)
+    parts = [(x[:, :3].astype(f32), y.astype(f32)), (x[:, 3:].astype(f32), y.astype(f32))]
+    init = {p: v.astype(f32) for p, v in with_state.items()}
+    trained, _, _ = O.train(m_state, O.Adam(0.01), parts, b, 2, init)
+    for p in state_paths:
+        assert not np.any(trained[p])
+
+
+def test_maximizing_adds_the_delta():
+    """`Optimizer.maximize` (Optimizer.scala:186,326-336): `if (minimizing) w - del else w + del`."""
+    rng = np.random.default_rng(3)
+    m = O.Model([O.Dense(2)], O.LOSS_MSE)
+    x, y = rng.standard_normal((5, 3)).astype(f32), rng.standard_normal((5, 2)).astype(f32)
+    params = {p: rng.standard_normal(s_).astype(f32) for p, s_ in m.param_defs(x.shape)}
+    alg = O.Adam(0.1)
+    down, st_down, _, grads = O.train_step(m, alg, x, y, params, O.init_opt_state(alg, params), 1)
+    up, st_up, _, _ = O.train_step(m, alg, x, y, params, O.init_opt_state(alg, params), 1, minimizing=False)
+    for p in params:
+        np.testing.assert_allclose(up[p] - params[p], -(down[p] - params[p]), rtol=0, atol=1e-6)     # the same delta, other sign
+        np.testing.assert_array_equal(st_up[p][0], st_down[p][0])
+    assert float(m.loss_of(x, y, up)) > float(m.loss_of(x, y, params)) > float(m.loss_of(x, y, down))
+
+
 def test_lstm_matches_torch_lstm_cell():
     """Independent library check: torch.nn.LSTM (gate order i,f,g,o) with the reference's weights mapped in."""
     rng = np.random.default_rng(2)
