@@ -69,11 +69,79 @@ def kernel_table(ctx):
 
 
 def gemm_flops(name):
+    """2 M N K of the bracketed shape in a kernel label (the implicit GEMM's own, possibly padded, shape)."""
     m = re.search(r"\[(\d+)x(\d+)x(\d+)\]", name)
     if not m:
         return None
     M, N, K = (int(v) for v in m.groups())
     return 2.0 * M * N * K
+
+
+def _out_size(pad, size, k, s):
+    from scanet3_amd import _lib as L
+    return -(-size // s) if pad == L.PAD_SAME else -(-(size - k + 1) // s)
+
+
+def model_work(layers, in_shape, batch):
+    """Algorithmic flops of one training step and of its matrix kernels, from the layer list alone.
+
+    Returns (flops per step, {kernel label: algorithmic flops per launch}).  Per layer (B = batch):
+      Dense in->out ........ 2 B in out for each of forward, weight gradient and (not for the first layer) input gradient
+      Conv2D ................ 2 B Ho Wo Cout kh kw Cin for each of the same three; the input-gradient kernel's label carries
+                              the padded implicit GEMM B H W x Cin x kh kw Cout, which counts border taps that do not exist
+      LSTM (T steps) ........ forward 2 B 4H (F + H) per step, hidden gradient 2 B H 4H per step but the first,
+                              weight gradient 2 (F + H) 4H (T B), input gradient 2 B F 4H per step unless first layer
+      SimpleRNN ............. the same with one gate
+    Element-wise work (activations, pooling, softmax, optimizer) is not counted: the roofline here is the matrix one."""
+    from scanet3_amd import _lib as L
+    shape = tuple(in_shape)
+    total, labels, first = 0.0, {}, True
+    for l in layers:
+        if l.kind == L.LAYER_DENSE:
+            f = 2.0 * batch * shape[0] * l.units
+            total += f * (2 if first else 3)
+            labels[f"[{batch}x{l.units}x{shape[0]}]"] = f
+            labels[f"[{shape[0]}x{l.units}x{batch}]"] = f
+            labels[f"[{shape[0] + 1}x{l.units}x{batch}]"] = f            # with the bias-gradient row riding along
+            labels[f"[{batch}x{shape[0]}x{l.units}]"] = f
+            shape, first = (l.units,), False
+        elif l.kind == L.LAYER_CONV2D:
+            h, w, cin = shape
+            ho, wo = _out_size(l.padding, h, l.kernel[0], l.strides[0]), _out_size(l.padding, w, l.kernel[1], l.strides[1])
+            k = l.kernel[0] * l.kernel[1] * cin
+            f = 2.0 * batch * ho * wo * l.units * k
+            total += f * (2 if first else 3)
+            labels[f"[{batch * ho * wo}x{l.units}x{k}]"] = f
+            labels[f"[{k}x{l.units}x{batch * ho * wo}]"] = f
+            labels[f"[{batch * h * w}x{cin}x{l.kernel[0] * l.kernel[1] * l.units}]"] = f
+            shape, first = (ho, wo, l.units), False
+        elif l.kind == L.LAYER_POOL2D:
+            h, w, c = shape
+            shape = (_out_size(l.padding, h, l.kernel[0], l.strides[0]), _out_size(l.padding, w, l.kernel[1], l.strides[1]), c)
+        elif l.kind == L.LAYER_FLATTEN:
+            shape = (int(np.prod(shape)),)
+        elif l.kind in (L.LAYER_LSTM, L.LAYER_SIMPLE_RNN):
+            T, F = shape
+            H, G = l.units, (4 if l.kind == L.LAYER_LSTM else 1)
+            fwd, dh, wg, dx = 2.0 * batch * G * H * (F + H), 2.0 * batch * H * G * H, 2.0 * (F + H) * G * H * T * batch, 2.0 * batch * F * G * H
+            total += T * fwd + (T - 1) * dh + wg + (0 if first else T * dx)
+            labels[f"[{batch}x{G * H}x{F + H}]"] = fwd
+            labels[f"[{batch}x{G * H}x{H}]"] = 2.0 * batch * G * H * H       # the recurrent half alone (input half hoisted)
+            labels[f"[{batch * T}x{G * H}x{F}]"] = 2.0 * batch * T * G * H * F
+            labels[f"[{batch}x{H}x{G * H}]"] = dh
+            labels[f"[{batch}x{H}x{H}]"] = dh
+            labels[f"[{F + H}x{G * H}x{T * batch}]"] = wg
+            labels[f"[{F + H + 1}x{G * H}x{T * batch}]"] = wg
+            shape, first = ((T, H) if l.return_sequence else (H,)), False
+    return total, labels
+
+
+def algorithmic_flops(name, labels):
+    """Algorithmic flops of one launch of the kernel labelled `name` (None when it is not a matrix kernel)."""
+    m = re.search(r"\[\d+x\d+x\d+\]", name)
+    if not m:
+        return None
+    return labels.get(m.group(0), gemm_flops(name))
 
 
 def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy, n_batches, steps, warmup, flags=0):
@@ -126,19 +194,24 @@ def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy
         k["per_step_us"] = 1e3 * k["total_ms"] / prof_steps
     last_loss = rep.loss(Xb.offset(0), Yb.offset(0))
     n_params = sum(int(np.prod(s)) for _, s, _ in cm.params)
+    step_flops, labels = model_work(layers.layers, in_shape, batch)
+    for kname, k in kernels.items():
+        k["flops_per_launch"] = algorithmic_flops(kname, labels)
     rep.close()
     cm.close()
     Xb.free()
     Yb.free()
     return {"workload": name, "samples_per_s": batch * steps / dt, "ms_per_step": 1e3 * dt / steps, "steps": steps,
-            "batch": batch, "params": n_params, "loss_after": last_loss, "kernels": kernels, "host_fed": host_fed}
+            "batch": batch, "params": n_params, "loss_after": last_loss, "kernels": kernels, "host_fed": host_fed,
+            "flops_per_step": step_flops}
 
 
 def dominant_gemm_roofline(kernels, peak_tflops):
-    """Roofline entry for the matrix-core kernel that takes the most time."""
+    """Roofline entry for the matrix-core kernel that takes the most time: ALGORITHMIC flops of one launch (model_work)
+    divided by the launch's average duration (HIP events on the library's stream)."""
     best = None
     for name, k in kernels.items():
-        fl = gemm_flops(name)
+        fl = k.get("flops_per_launch")
         if fl is None:
             continue
         if best is None or k["total_ms"] > best[1]["total_ms"]:
@@ -148,7 +221,15 @@ def dominant_gemm_roofline(kernels, peak_tflops):
     name, k, fl = best
     ach = fl / (k["avg_us"] * 1e-6) / 1e12
     return {"kernel": name, "bound": "mfma", "achieved": ach, "peak": peak_tflops, "unit": "TFLOP/s", "frac": ach / peak_tflops,
-            "avg_launch_us": k["avg_us"], "flops_per_launch": fl, "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(name)}
+            "avg_launch_us": k["avg_us"], "flops_per_launch": fl, "traffic": measured_traffic(name)}
+
+
+def whole_step_roofline(res, peak_tflops):
+    """Every matrix flop the step has to do divided by the step's wall time (launch gaps, element-wise kernels and the
+    optimizer all count against it)."""
+    ach = res["flops_per_step"] / (res["ms_per_step"] * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": ach, "peak": peak_tflops, "unit": "TFLOP/s", "frac": ach / peak_tflops,
+            "flops_per_step": res["flops_per_step"], "ms_per_step": res["ms_per_step"]}
 
 
 def bench_lenet(S, ctx, steps, warmup, pool_stride=1):
@@ -211,17 +292,33 @@ def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
         flags=L.FLAG_GEMM_BF16 if bf16 else 0)
 
 
-# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` (two runs, scaled by a copy kernel
-# of known size: WRITE_SIZE x 1.0, FETCH_SIZE x 2.0); summary in profiles/optimizer_100M_and_average_8x25M_hbm_traffic_pmc.md
-MEASURED_TRAFFIC_BYTES = {"sgd": 2.000e9, "adagrad": 2.000e9, "rmsprop": 2.000e9, "adadelta": 2.800e9, "adam": 2.800e9,
-                          "nadam": 2.800e9, "adamax": 2.800e9, "amsgrad": 3.600e9, "average": 0.900e9}
-# the same for the matrix kernels (profiles/lenet_and_wide_mlp_gemm_kernels_hbm_traffic_pmc.md); keyed by kernel label
-MEASURED_GEMM_TRAFFIC_BYTES = {
-    "conv2d_forward[52900x64x288]": 14.1e6 + 13.5e6,
-    "conv2d_input_gradient[62500x32x576]": 19.9e6 + 8.0e6,
-    "conv2d_filter_gradient[288x64x52900]": 23.4e6 + 18.8e6,
-    "gemm_bf16_256[8192x4096x4096]": 404e6 + 135e6,
+# HBM bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` (two runs, each scaled by what the same counter
+# reads for a one-input average = a plain copy of known size; summaries under profiles/).  A figure belongs to the kernel
+# source it was measured on: every entry carries the SHA-1 of that source file, and `measured_traffic` returns None
+# (JSON null) when the file has changed since.
+CSRC = os.path.join(ROOT, "scanet3_amd", "csrc")
+MEASURED_TRAFFIC = {
+    # kernel label (or optimizer name): (bytes per launch, source file, sha1 of the file when measured)
 }
+
+
+def _sha1(path):
+    import hashlib
+    try:
+        with open(path, "rb") as f:
+            return hashlib.sha1(f.read()).hexdigest()
+    except OSError:
+        return None
+
+
+def measured_traffic(key):
+    entry = MEASURED_TRAFFIC.get(key)
+    if entry is None:
+        return None
+    nbytes, source, sha = entry
+    return nbytes if _sha1(os.path.join(CSRC, source)) == sha else None
+
+
 OPT_BYTES = {"sgd": 20, "adagrad": 20, "rmsprop": 20, "adadelta": 28, "adam": 28, "nadam": 28, "adamax": 28, "amsgrad": 36}
 
 
@@ -392,7 +489,7 @@ def main():
                      "value": adam["elems_per_s"], "ms_per_step": adam["ms_per_step"],
                      "config": {"workload": main_res["workload"]},
                      "roofline": {"kernel": "optimizer_adam", "bound": "hbm", "achieved": adam["GBps"], "peak": PEAK_HBM_GBS,
-                                  "unit": "GB/s", "frac": adam["frac_of_peak"], "traffic": MEASURED_TRAFFIC_BYTES["adam"]},
+                                  "unit": "GB/s", "frac": adam["frac_of_peak"], "traffic": measured_traffic("adam")},
                      "optimizers": main_res["results"]})
     else:
         peak = PEAK_BF16_MFMA if args.workload == "wide_mlp" else PEAK_FP32_MFMA
@@ -400,6 +497,7 @@ def main():
                      "dtype": "bf16" if args.workload == "wide_mlp" else "f32",
                      "config": {"workload": main_res["workload"], "batch": main_res["batch"], "params": main_res["params"]},
                      "roofline": dominant_gemm_roofline(main_res["kernels"], peak),
+                     "roofline_whole_step": whole_step_roofline(main_res, peak),
                      "host_fed": main_res["host_fed"],
                      "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                              sorted(main_res["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:12]}})
@@ -423,6 +521,7 @@ def main():
                 extras[which] = {"workload": r["workload"], "samples_per_s": r["samples_per_s"], "ms_per_step": r["ms_per_step"],
                                  "steps": r["steps"], "loss_after": r["loss_after"], "host_fed": r["host_fed"],
                                  "roofline": dominant_gemm_roofline(r["kernels"], peak),
+                                 "roofline_whole_step": whole_step_roofline(r, peak),
                                  "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                                          sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}
                 if "batchnorm_hbm" in r:
@@ -436,7 +535,7 @@ def main():
                 v = opt["results"][k]
                 rl["optimizer_adam_100M" if k == "adam" else "average_8x25M"] = {
                     "bound": "hbm", "achieved": v["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": v["frac_of_peak"],
-                    "traffic": MEASURED_TRAFFIC_BYTES[k]}
+                    "traffic": measured_traffic(k)}
         wide = extras.get("wide_mlp")
         if wide and wide.get("roofline"):
             rl["wide_mlp_gemm_bf16"] = wide["roofline"]

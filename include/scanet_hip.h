@@ -54,7 +54,7 @@ enum {
   SN_E_STATE = -4        /* object used after destroy / wrong context */
 };
 
-/* ---- layer list (models/layer/*.scala, flattened as layer/Composed.scala:89-99 does) ---- */
+/* ---- layer list (the layers under models/layer/, flattened as layer/Composed.scala:89-99 does) ---- */
 enum { SN_LAYER_DENSE = 0, SN_LAYER_BIAS = 1, SN_LAYER_ACTIVATE = 2, SN_LAYER_FLATTEN = 3,
        SN_LAYER_CONV2D = 4, SN_LAYER_POOL2D = 5, SN_LAYER_LSTM = 6, SN_LAYER_SIMPLE_RNN = 7, SN_LAYER_BATCHNORM = 8 };
 /* models/Activation.scala:32-83 */

@@ -57,6 +57,7 @@ struct sn_ctx {
   hipStream_t stream;
   bool owns_stream;
   int compute_units;
+  int live_models = 0;  // models created from this context and not yet destroyed
   // timing
   bool profiling;
   std::vector<sn::PendingEvent> pending;

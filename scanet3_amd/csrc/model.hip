@@ -1040,13 +1040,15 @@ int sn_model_create(sn_ctx* ctx, const sn_layer_desc* layers, int32_t n_layers, 
     delete m;
     return rc;
   }
+  ctx->live_models++;
   *out = m;
   return SN_OK;
 }
 
 int sn_model_destroy(sn_model* model) {
   SN_TRY(check_model(model));
-  SN_REQUIRE(model->live_replicas == 0, "model still has %d live replicas", model->live_replicas);
+  if (model->live_replicas != 0) return fail(SN_E_STATE, "model still has %d live replicas", model->live_replicas);
+  model->ctx->live_models--;
   model->magic = 0;
   delete model;
   return SN_OK;
@@ -1263,7 +1265,8 @@ int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, in
   SN_TRY(check_rows(rep, rows));
   SN_TRY(forward(rep, x_dev, rows));
   const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, x_dev, rows);
-  SN_HIP(hipMemsetAsync(rep->count_dev, 0, sizeof(unsigned long long), rep->ctx->stream));
+  // cleared by a kernel, not a memset node: the call may be recorded into a HIP graph (all-zero bits are 0.0f twice)
+  SN_TRY(launch_fill(rep->ctx, (float*)rep->count_dev, 0.f, 2));
   const int cols = (int)rep->model->out_dims.back();
   SN_TRY(launch_count_correct(rep->ctx, pred, y_dev, (int)((int64_t)rows * rep->model->out_elems / cols), cols, rep->count_dev));
   unsigned long long c = 0;
@@ -1325,13 +1328,41 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
              (long long)total_rows, batch);
   hipStream_t compute = rep->ctx->stream;
   if (!rep->copy_stream) {
-    for (int i = 0; i < 2; ++i) {
-      SN_TRY(dev_alloc(rep, &rep->stage_x[i], rep->model->in_elems * rep->model->batch));
-      SN_TRY(dev_alloc(rep, &rep->stage_y[i], rep->model->out_elems * rep->model->batch));
-      SN_HIP(hipEventCreateWithFlags(&rep->ev_filled[i], hipEventDisableTiming));
-      SN_HIP(hipEventCreateWithFlags(&rep->ev_consumed[i], hipEventDisableTiming));
+    // Staging buffers, events and the copy stream are made in locals and handed to the replica only when all of them
+    // exist, so a failure half way leaves nothing behind and the next call starts over.
+    float* sx[2] = {nullptr, nullptr};
+    float* sy[2] = {nullptr, nullptr};
+    hipEvent_t filled[2] = {nullptr, nullptr}, consumed[2] = {nullptr, nullptr};
+    hipStream_t copy = nullptr;
+    const size_t xb = (size_t)rep->model->in_elems * rep->model->batch * sizeof(float);
+    const size_t yb = (size_t)rep->model->out_elems * rep->model->batch * sizeof(float);
+    hipError_t e = hipSetDevice(rep->ctx->device);
+    for (int i = 0; i < 2 && e == hipSuccess; ++i) {
+      e = hipMalloc((void**)&sx[i], xb);
+      if (e == hipSuccess) e = hipMalloc((void**)&sy[i], yb);
+      if (e == hipSuccess) e = hipEventCreateWithFlags(&filled[i], hipEventDisableTiming);
+      if (e == hipSuccess) e = hipEventCreateWithFlags(&consumed[i], hipEventDisableTiming);
     }
-    SN_HIP(hipStreamCreateWithFlags(&rep->copy_stream, hipStreamNonBlocking));
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&copy, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+      for (int i = 0; i < 2; ++i) {
+        if (sx[i]) (void)hipFree(sx[i]);
+        if (sy[i]) (void)hipFree(sy[i]);
+        if (filled[i]) (void)hipEventDestroy(filled[i]);
+        if (consumed[i]) (void)hipEventDestroy(consumed[i]);
+      }
+      return fail(e == hipErrorOutOfMemory ? SN_E_OOM : SN_E_HIP, "sn_train_epoch_host: setting up the staging slots failed: %s",
+                  hipGetErrorString(e));
+    }
+    for (int i = 0; i < 2; ++i) {
+      rep->stage_x[i] = sx[i];
+      rep->stage_y[i] = sy[i];
+      rep->owned.push_back(sx[i]);
+      rep->owned.push_back(sy[i]);
+      rep->ev_filled[i] = filled[i];
+      rep->ev_consumed[i] = consumed[i];
+    }
+    rep->copy_stream = copy;
   }
   const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
   auto fill = [&](int64_t i, int slot) -> int {

@@ -125,6 +125,8 @@ int sn_ctx_create(int device, void* stream, sn_ctx** out) {
 
 int sn_ctx_destroy(sn_ctx* ctx) {
   SN_TRY(check_ctx(ctx));
+  // models (and through them replicas) keep a pointer to the context and its stream
+  if (ctx->live_models != 0) return fail(SN_E_STATE, "context still has %d live models: destroy replicas and models first", ctx->live_models);
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->stream);
   for (auto& p : ctx->pending) {

@@ -1134,6 +1134,12 @@ def test_error_paths(S, ctx):
         cm.close()                                          # replicas still alive
     rep.close()
     cm.close()
+    other = S.Context(0)                                    # a context cannot go away under its models
+    held = S.CompiledModel(other, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3,), 8)
+    with pytest.raises(S.ScanetError, match="live models"):
+        other.close()
+    held.close()
+    other.close()
     with pytest.raises(S.ScanetError):                      # Dense straight on an image
         S.CompiledModel(ctx, [l.desc() for l in spec_layers], S.MeanSquaredError.kind, (3, 3, 1), 8)
     with pytest.raises(S.ScanetError):                      # kernel larger than the input
