@@ -318,6 +318,14 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev
 int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const float* wpack, float* dh_parts, int64_t part_stride,
                         int gates = 4);
+// One launch per reverse LSTM step: gate gradients (g: gates, c, c_prev, dh parts, dy_seq, dz as for launch_lstm_gates_bwd;
+// dc_in null = zeros, dc_out another buffer) and, unless wpack is null, the lstm_bwd_parts(H) partial products whose sum
+// is dh_{t-1}, written out_part_stride elements apart.  wpack: launch_lstm_pack_bwd (at most lstm_pack_elems floats).
+bool lstm_step_bwd_fused_ok(int H, const LstmWeights& w);
+int lstm_bwd_parts(int H);
+int launch_lstm_pack_bwd(sn_ctx* ctx, const LstmWeights& w, int H, float* pack);
+int launch_lstm_step_bwd(sn_ctx* ctx, const LstmGateBwdArgs& g, const float* dc_in, float* dc_out, const float* wpack, float* dh_out,
+                         int64_t out_part_stride, int rows, int H);
 // simple cell: r_t[rows, H] = [x[:, t, :], r_prev] * [Wk; Wr] from the one-gate pack (r_prev null at t == 0)
 int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* r_prev, int rows, int H, const float* wpack, float* out);
 

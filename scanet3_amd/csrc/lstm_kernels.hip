@@ -290,6 +290,171 @@ __global__ __launch_bounds__(256) void step_product_kernel(StepMulArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------- backward step, fused
+// One launch per reverse time step: the gate gradients of step t (element-wise) and the product that carries the
+// hidden gradient back, dh_{t-1} = sum over gates of dz_gate * Wr_gate^T.  A workgroup owns BR batch rows x BU hidden
+// units: it turns those cells' dh, dc and saved gates into dz (written out for the weight-gradient GEMM and kept in
+// LDS as the product's A operand, k = gate * BU + unit), and multiplies by the matching K slice of the recurrent
+// weights, which travels to LDS with LDS-direct loads while the element-wise part runs.  Every workgroup so
+// contributes one K slice of dh_{t-1} for its rows: the H / BU partial results are written side by side and the next
+// (earlier) step adds them in slice order.  Every cell belongs to exactly one workgroup per column chunk.
+//   do = dh * tanh(c);  dc += (1 - tanh(c)^2) * (dh * o)
+//   df = dc * c_prev;   di = dc * g;   dg = dc * i;   dc_prev = dc * f
+//   dz_gate = act'(z_gate) * d_gate  (sigmoid: s(1-s), tanh: 1 - g^2)
+constexpr int BR = 16, BU = 32, BK4 = 4 * BU, BKP = BK4 + 4, BN_MAX = 128;
+
+struct StepBwdArgs {
+  const float* gates;    // [rows, 4H] activated f, i, g, o of this step
+  const float* c;        // c_t
+  const float* c_prev;   // c_{t-1} or null (zeros)
+  const float* dh;       // dh_parts arrays, dh_part_stride elements apart, added in order; may be null with dh_parts == 0
+  int dh_parts;
+  int64_t dh_part_stride;
+  const float* dy_seq;   // optional: this step's slice of the gradient of a returned sequence, row r at dy_seq + r * dy_seq_ld
+  int64_t dy_seq_ld;
+  const float* dc_in;    // dc carried from step t+1, or null (zeros)
+  float* dc_out;         // dc for step t-1 (a different buffer than dc_in: other workgroups still read that one)
+  float* dz;             // [rows, 4H]
+  const float* wpack;    // recurrent weights in LDS order (pack_bwd_kernel), null: no product (first time step)
+  float* dh_out;         // [H / BU][part_stride] partial dh_{t-1}
+  int64_t out_part_stride;
+  int rows, H;
+};
+
+// [slice of BU units][column block of 16 inputs n][k quad q of the slice's 4*BU k][16 columns][4 consecutive k]:
+// k = gate * BU + unit, value Wr_gate[n][slice * BU + unit]
+__global__ __launch_bounds__(256) void pack_bwd_kernel(LstmWeights w, int H, float* __restrict__ out) {
+  const int64_t cells = (int64_t)(H / BU) * (H / 16) * (BK4 / 4) * 16;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < cells; e += (int64_t)gridDim.x * 256) {
+    const int col = (int)(e & 15);
+    int64_t t = e >> 4;
+    const int q = (int)(t % (BK4 / 4)); t /= (BK4 / 4);
+    const int cb = (int)(t % (H / 16));
+    const int slice = (int)(t / (H / 16));
+    const int gate = (4 * q) / BU, ul = (4 * q) % BU;
+    *(f4v*)(out + e * 4) = *(const f4v*)(w.wr[gate] + (int64_t)(cb * 16 + col) * H + slice * BU + ul);
+  }
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+__global__ __launch_bounds__(256) void lstm_step_bwd_kernel(StepBwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* As = lds;              // [BR][BKP]
+  float* Bs = lds + BR * BKP;   // [column blocks of this chunk][BK4 / 4][16][4]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int slice = blockIdx.x, r0 = blockIdx.y * BR, n0 = blockIdx.z * BN_MAX;
+  const int ncols = min(BN_MAX, a.H - n0), ncb = ncols / 16;  // H % 16 == 0
+  const bool product = a.wpack != nullptr;
+
+  // ---- everything the workgroup's cells need is requested first (two cells per thread, every load in flight at once),
+  // the weight slab right behind it, so the element-wise arithmetic runs while the slab is still on its way
+  constexpr int CELLS = BR * BU / 256, MAX_PARTS = 8;
+  float f[CELLS], in[CELLS], gg[CELLS], o[CELLS], cc[CELLS], cp[CELLS], dcv[CELLS], dyv[CELLS], dhp[CELLS][MAX_PARTS];
+  bool live[CELLS];
+#pragma unroll
+  for (int ci = 0; ci < CELLS; ++ci) {
+    const int e = tid + ci * 256, row = e / BU, ul = e % BU;
+    live[ci] = r0 + row < a.rows;
+    const int64_t i = (int64_t)(live[ci] ? r0 + row : 0) * a.H + slice * BU + ul;
+    const int64_t zb = (int64_t)(live[ci] ? r0 + row : 0) * 4 * a.H + slice * BU + ul;
+    f[ci] = a.gates[zb];
+    in[ci] = a.gates[zb + a.H];
+    gg[ci] = a.gates[zb + 2 * a.H];
+    o[ci] = a.gates[zb + 3 * a.H];
+    cc[ci] = a.c[i];
+    cp[ci] = a.c_prev ? a.c_prev[i] : 0.f;
+    dcv[ci] = a.dc_in ? a.dc_in[i] : 0.f;
+    dyv[ci] = a.dy_seq ? a.dy_seq[(int64_t)(live[ci] ? r0 + row : 0) * a.dy_seq_ld + slice * BU + ul] : 0.f;
+#pragma unroll
+    for (int p = 0; p < MAX_PARTS; ++p) dhp[ci][p] = p < a.dh_parts ? a.dh[i + p * a.dh_part_stride] : 0.f;
+  }
+  // the weight slab for this slice and column chunk: one contiguous run in the pack, copied 1 KiB per issue
+  if (product) {
+    const float* slab = a.wpack + ((int64_t)slice * (a.H / 16) + n0 / 16) * (BK4 / 4) * 64;
+    const uint32_t bytes = (uint32_t)ncb * (BK4 / 4) * 64 * 4;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(slab), 0, (int)bytes, 0x00020000);
+    for (uint32_t off = (uint32_t)wave * 1024u; off < bytes; off += 4096u)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)((char*)Bs + off), 16, (int)(off + lane * 16), 0, 0, 0);
+  }
+
+  // ---- gate gradients of this workgroup's cells (only column chunk 0 writes them out: the chunks share the cells)
+  const bool writer = blockIdx.z == 0;
+#pragma unroll
+  for (int ci = 0; ci < CELLS; ++ci) {
+    const int e = tid + ci * 256, row = e / BU, ul = e % BU;
+    float dzf = 0.f, dzi = 0.f, dzg = 0.f, dzo = 0.f;
+    if (live[ci]) {
+      const int u = slice * BU + ul;
+      const int64_t i = (int64_t)(r0 + row) * a.H + u;
+      const int64_t zb = (int64_t)(r0 + row) * 4 * a.H + u;
+      const float tc = tanhf(cc[ci]);
+      float dh = dhp[ci][0];
+#pragma unroll
+      for (int p = 1; p < MAX_PARTS; ++p)
+        if (p < a.dh_parts) dh += dhp[ci][p];
+      for (int p = MAX_PARTS; p < a.dh_parts; ++p) dh += a.dh[i + p * a.dh_part_stride];  // more slices than registers hold
+      if (a.dy_seq) dh = dh + dyv[ci];
+      const float d_o = dh * tc;
+      float dc = dcv[ci] + (1.0f - tc * tc) * (dh * o[ci]);
+      const float df = dc * cp[ci], di = dc * gg[ci], dg = dc * in[ci];
+      dzf = (f[ci] * (1.0f - f[ci])) * df;
+      dzi = (in[ci] * (1.0f - in[ci])) * di;
+      dzg = (1.0f - gg[ci] * gg[ci]) * dg;
+      dzo = (o[ci] * (1.0f - o[ci])) * d_o;
+      if (writer) {
+        a.dc_out[i] = dc * f[ci];
+        a.dz[zb] = dzf;
+        a.dz[zb + a.H] = dzi;
+        a.dz[zb + 2 * a.H] = dzg;
+        a.dz[zb + 3 * a.H] = dzo;
+      }
+    }
+    float* arow = As + row * BKP + ul;
+    arow[0] = dzf;
+    arow[BU] = dzi;
+    arow[2 * BU] = dzg;
+    arow[3 * BU] = dzo;
+  }
+  if (!product) return;
+  __builtin_amdgcn_s_waitcnt(0);  // this wavefront's LDS-direct loads have landed
+  __syncthreads();
+
+  // ---- dh partial [BR x ncols] = As [BR x BK4] * Bs: wavefront w takes column blocks w, w + 4, ...
+  const int c16 = lane & 15, g = lane >> 4;
+  f4v acc[BN_MAX / 64];
+#pragma unroll
+  for (int j = 0; j < BN_MAX / 64; ++j) acc[j] = f4v{0.f, 0.f, 0.f, 0.f};
+  const float* ap = As + c16 * BKP + 4 * g;
+#pragma unroll 2
+  for (int kb = 0; kb < BK4 / 16; ++kb) {
+    const f4v av = *(const f4v*)(ap + 16 * kb);
+    f4v bv[BN_MAX / 64];
+#pragma unroll
+    for (int j = 0; j < BN_MAX / 64; ++j) {
+      const int cb = wave + 4 * j;
+      bv[j] = cb < ncb ? *(const f4v*)(Bs + (((int64_t)cb * (BK4 / 4) + kb * 4 + g) * 16 + c16) * 4) : f4v{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+      for (int j = 0; j < BN_MAX / 64; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bv[j][v], acc[j], 0, 0, 0);
+  }
+  float* out = a.dh_out + (int64_t)slice * a.out_part_stride;
+#pragma unroll
+  for (int j = 0; j < BN_MAX / 64; ++j) {
+    const int cb = wave + 4 * j;
+    if (cb >= ncb) continue;
+    const int col = n0 + cb * 16 + c16;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int row = r0 + 4 * g + v;
+      if (row < a.rows) out[(int64_t)row * a.H + col] = acc[j][v];
+    }
+  }
+}
+
 size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 or 32)
   const int K16 = round16(K);
   const size_t slabs = (size_t)RB * (K16 + 4) + (size_t)cols * K16, exchange = 4 * RB * ZP;
@@ -367,6 +532,39 @@ int launch_lstm_step_dh(sn_ctx* ctx, const float* dz, int rows, int H, const flo
   StepMulArgs a{dz, (int64_t)gates * H, H, nullptr, 0, 0, H, wpack, kq, (int64_t)(H / 16) * kq * 64, dh_parts, H, part_stride, rows, H};
   LaunchScope scope(ctx, "lstm_step_hidden_gradient", rows, H, gates * H);
   return launch_step_product(ctx, a, gates);
+}
+
+bool lstm_step_bwd_fused_ok(int H, const LstmWeights& w) {
+  if (H % BU != 0) return false;
+  for (int g = 0; g < 4; ++g)
+    if (!aligned16(w.wr[g])) return false;
+  return true;
+}
+
+int lstm_bwd_parts(int H) { return H / BU; }
+
+int launch_lstm_pack_bwd(sn_ctx* ctx, const LstmWeights& w, int H, float* pack) {
+  const int64_t cells = (int64_t)(H / BU) * (H / 16) * (BK4 / 4) * 16;
+  LaunchScope scope(ctx, "lstm_pack_weights");
+  hipLaunchKernelGGL(pack_bwd_kernel, dim3((unsigned)std::min<int64_t>(ceil_div(cells, 256), 2048)), dim3(256), 0, ctx->stream, w, H, pack);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_lstm_step_bwd(sn_ctx* ctx, const LstmGateBwdArgs& g, const float* dc_in, float* dc_out, const float* wpack, float* dh_out,
+                         int64_t out_part_stride, int rows, int H) {
+  if (rows <= 0) return SN_OK;
+  SN_REQUIRE(H % BU == 0 && (!wpack || aligned16(wpack)), "lstm_step_backward: H=%d outside what the fused kernel handles", H);
+  SN_REQUIRE(dc_in != dc_out, "lstm_step_backward: the cell gradient needs two buffers");
+  StepBwdArgs a{g.gates, g.c, g.c_prev, g.dh, g.dh_parts, g.dh_part_stride, g.dy_seq, g.dy_seq_ld, dc_in, dc_out, g.dz, wpack, dh_out,
+                out_part_stride, rows, H};
+  const int chunks = wpack ? (int)ceil_div(H, BN_MAX) : 1;
+  const size_t smem = ((size_t)BR * BKP + (size_t)std::min(H, BN_MAX) * BK4) * sizeof(float);
+  LaunchScope scope(ctx, "lstm_step_backward", rows, H, 4 * H);
+  SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_bwd_kernel, ((size_t)BR * BKP + (size_t)BN_MAX * BK4) * sizeof(float)));
+  hipLaunchKernelGGL(lstm_step_bwd_kernel, dim3((unsigned)(H / BU), (unsigned)ceil_div(rows, BR), (unsigned)chunks), dim3(256), smem, ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
 }
 
 // r_t[rows, H] = [x_t, r_prev] * [Wk; Wr]: the simple cell's step (pack from launch_lstm_pack(.., gates = 1))

@@ -97,6 +97,7 @@ struct sn_replica {
   std::vector<float*> lstm_pk_fwd, lstm_pk_dh;              // per op: weights in the step kernels' LDS order
   float* lstm_dh[2] = {nullptr, nullptr};
   float* lstm_dc = nullptr;
+  float* lstm_dc2 = nullptr;  // the fused backward step reads the carried cell gradient from one buffer and writes the other
   // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
   std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
   std::vector<float*> bn_buf;  // per batch-norm op: mean, var, 1/sqrt(var+eps), scale, two gradient vectors
@@ -440,7 +441,7 @@ static int alloc_replica(sn_replica* r) {
   r->bn_buf.assign(n_ops, nullptr);
   r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
   r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
-  int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0;
+  int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0, lstm_parts = 4;
   for (size_t i = 0; i < n_ops; ++i) {
     const Op& op = m->ops[i];
     if (op.kind == OP_FLATTEN) continue;  // a view of its input
@@ -455,6 +456,7 @@ static int alloc_replica(sn_replica* r) {
       SN_TRY(launch_fill(r->ctx, r->lstm_h[i], 0.f, bh));
       lstm_z = std::max(lstm_z, bh * 4);
       lstm_h = std::max(lstm_h, bh);
+      lstm_parts = std::max<int64_t>(lstm_parts, lstm_bwd_parts(op.H));
       if (op.ret_seq) SN_TRY(dev_alloc(r, &r->act[i], B * op.out_elems));
       continue;  // output = last slice of lstm_h unless the whole sequence is returned
     }
@@ -481,9 +483,10 @@ static int alloc_replica(sn_replica* r) {
   }
   SN_TRY(dev_alloc(r, &r->bf_colp, bf_colp));
   SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
-  SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h * 4));  // four per-gate partial sums each
-  SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h * 4));
+  SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h * lstm_parts));  // partial sums of the hidden gradient: per gate, or per slice of units
+  SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h * lstm_parts));
   SN_TRY(dev_alloc(r, &r->lstm_dc, lstm_h));
+  SN_TRY(dev_alloc(r, &r->lstm_dc2, lstm_h));
   SN_TRY(dev_alloc(r, &r->grad_buf[0], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->grad_buf[1], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->ws, m->workspace_elems));
@@ -811,7 +814,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         const float* dh = op.ret_seq ? nullptr : dy;  // gradient of the last hidden state (a returned sequence adds its own per step)
         int hb = 0, dh_parts = op.ret_seq ? 0 : 1;
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
-        if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
+        // one launch per step (gate gradients + the product that carries dh back) where the layer's shape allows it
+        const bool fused_bwd = fused && lstm_step_bwd_fused_ok(op.H, w);
+        if (fused_bwd && op.T > 1) SN_TRY(launch_lstm_pack_bwd(ctx, w, op.H, r->lstm_pk_dh[i]));
+        else if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
+        float* dcbuf[2] = {r->lstm_dc, r->lstm_dc2};
+        int db = 0;
         for (int t = op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                             t == 0 ? param_ptr(r, r->w, op.state_p[0]) : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
@@ -819,6 +827,16 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           if (op.ret_seq) {  // this step's own output gradient joins what the later steps carried back
             a.dy_seq = dy + (int64_t)t * op.H;
             a.dy_seq_ld = (int64_t)op.T * op.H;
+          }
+          if (fused_bwd) {
+            SN_TRY(launch_lstm_step_bwd(ctx, a, t == op.T - 1 ? nullptr : dcbuf[db], dcbuf[db ^ 1], t > 0 ? r->lstm_pk_dh[i] : nullptr,
+                                        r->lstm_dh[hb], bh, rows, op.H));
+            db ^= 1;
+            if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
+            dh = r->lstm_dh[hb];
+            dh_parts = lstm_bwd_parts(op.H);
+            hb ^= 1;
+            continue;
           }
           SN_TRY(launch_lstm_gates_bwd(ctx, a, rows, op.H));
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, a.dz, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
