@@ -279,6 +279,12 @@ int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float*
 int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems);
 int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems);
 
+// the same two products with LDS-direct loads into a three-stage ring (conv_ring_kernels.hip), for the shapes *_ok accepts
+bool conv_ring_fwd_ok(const ConvGeom& g, const float* x, const float* w, const Epilogue& e);
+int launch_conv_ring_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& e);
+bool conv_ring_dgrad_ok(const ConvGeom& g, const float* dy, const float* w);
+int launch_conv_ring_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx);
+
 struct LstmWeights {
   const float* wk[4];  // [F,H] forget,input,gate,output
   const float* wr[4];  // [H,H]

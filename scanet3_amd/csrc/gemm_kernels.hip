@@ -1436,6 +1436,7 @@ int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float*
     SN_HIP(hipGetLastError());
     return SN_OK;
   }
+  if (conv_ring_fwd_ok(g, x, w, e)) return launch_conv_ring_fwd(ctx, g, x, w, e);
   StdEpilogue ep{e};
   if (TapLoader::ok(x, g.n, g.h, g.w, g.cin, g.kh, g.kw) && FlatLoader<false>::ok(w, 1, g.cout, N, K)) {
     TapLoader al{x, M, g.ho, g.wo, g.sh, g.sw, -g.pt, -g.pl, 1, 1, g.h, g.w, g.cin, g.kh, g.kw};
@@ -1452,6 +1453,7 @@ int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const flo
   Epilogue e;
   e.out = dx;
   e.ldo = g.cin;
+  if (conv_ring_dgrad_ok(g, dy, w)) return launch_conv_ring_dgrad(ctx, g, dy, w, dx);
   StdEpilogue ep{e};
   if (g.sh == 1 && g.sw == 1 && TapLoader::ok(dy, g.n, g.ho, g.wo, g.cout, g.kh, g.kw) && aligned16(w) &&
       (int64_t)K * g.cin * 4 < FAST_SPAN) {
