@@ -358,6 +358,23 @@ def bench_optim(S, ctx, steps, warmup, n=100_000_000, k=8, n_avg=25_000_000):
         out[name] = {"bytes_per_elem": OPT_BYTES[name], "ms_per_step": 1e3 * dt / steps, "kernel_avg_us": avg_s * 1e6,
                      "GBps": OPT_BYTES[name] * n / avg_s / 1e9, "frac_of_peak": OPT_BYTES[name] * n / avg_s / 1e9 / PEAK_HBM_GBS,
                      "elems_per_s": n / avg_s}
+    # a plain copy of the same 100 M elements (the mean of ONE input: n floats in, n out) is what this box's memory
+    # system gives a streaming kernel; the update kernels are to be read against it as well as against the 8 TB/s peak
+    for _ in range(warmup):
+        ctx.average([wb], states[0])
+    ctx.sync()
+    ctx.profile_reset()
+    ctx.profile(True)
+    for _ in range(steps):
+        ctx.average([wb], states[0])
+    ctx.profile(False)
+    kern = ctx.profile_report()["average_replicas"]
+    avg_s = kern[0] / kern[1] * 1e-3
+    out["copy_100M"] = {"n": n, "bytes_per_elem": 8, "kernel_avg_us": avg_s * 1e6, "GBps": 8 * n / avg_s / 1e9,
+                        "frac_of_peak": 8 * n / avg_s / 1e9 / PEAK_HBM_GBS}
+    for name, _ in algs:
+        out[name]["frac_of_copy"] = out[name]["GBps"] / out["copy_100M"]["GBps"]
+    ctx.profile_reset()
     for b in states + [wb, gb]:
         b.free()
     # averaging

@@ -101,35 +101,36 @@ constexpr int n_states() {
   return (KIND == SN_OPT_SGD || KIND == SN_OPT_ADAGRAD || KIND == SN_OPT_RMSPROP) ? 1 : (KIND == SN_OPT_AMSGRAD ? 3 : 2);
 }
 
-// A block owns 256*U consecutive float4 of every array and touches ONE ARRAY AT A TIME: U loads of w,
-// then U of g, ... then the stores array by array.  Each wavefront so issues U back-to-back 1 KiB rows of
-// the same stream; measured on MI355X this keeps 4 read + 3 write streams at about 6.1 TB/s where the
-// element-interleaved order reaches 5.6 TB/s.  U = 4 is the sweet spot (8 spills registers).
-template <int KIND, int U>
-__global__ __launch_bounds__(256) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
+// A block owns T*U consecutive float4 of every array and touches ONE ARRAY AT A TIME: U loads of w,
+// then U of g, ... then the stores array by array (measured on MI355X: 6.1 TB/s for Adam's 4 read + 3 write
+// streams where the element-interleaved order reaches 5.6 TB/s).
+template <int KIND, int U, int T>
+__global__ __launch_bounds__(T) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
                                                             f4* __restrict__ s1, f4* __restrict__ s2, int64_t n4,
                                                             OptScalars p) {
   constexpr int NS = n_states<KIND>();
-  const int64_t base = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
+  if (U == 1 && base >= n4) return;  // one vector per thread: one early exit instead of a check around every access
+#define SN_IN_RANGE(u) (U == 1 || base + (u) * T < n4)
   f4 vw[U], vg[U], a[U], b[U], c[U];
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    if (base + u * 256 < n4) vw[u] = __builtin_nontemporal_load(w + base + u * 256);
+    if (SN_IN_RANGE(u)) vw[u] = __builtin_nontemporal_load(w + base + u * T);
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    if (base + u * 256 < n4) vg[u] = __builtin_nontemporal_load(g + base + u * 256);
+    if (SN_IN_RANGE(u)) vg[u] = __builtin_nontemporal_load(g + base + u * T);
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    if (base + u * 256 < n4) a[u] = __builtin_nontemporal_load(s0 + base + u * 256);
+    if (SN_IN_RANGE(u)) a[u] = __builtin_nontemporal_load(s0 + base + u * T);
   if (NS > 1) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) b[u] = __builtin_nontemporal_load(s1 + base + u * 256);
+      if (SN_IN_RANGE(u)) b[u] = __builtin_nontemporal_load(s1 + base + u * T);
   }
   if (NS > 2) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) c[u] = __builtin_nontemporal_load(s2 + base + u * 256);
+      if (SN_IN_RANGE(u)) c[u] = __builtin_nontemporal_load(s2 + base + u * T);
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
@@ -145,21 +146,22 @@ __global__ __launch_bounds__(256) void optimizer_kernel_v4(f4* __restrict__ w, c
   }
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    if (base + u * 256 < n4) __builtin_nontemporal_store(vw[u], w + base + u * 256);
+    if (SN_IN_RANGE(u)) __builtin_nontemporal_store(vw[u], w + base + u * T);
 #pragma unroll
   for (int u = 0; u < U; ++u)
-    if (base + u * 256 < n4) __builtin_nontemporal_store(a[u], s0 + base + u * 256);
+    if (SN_IN_RANGE(u)) __builtin_nontemporal_store(a[u], s0 + base + u * T);
   if (NS > 1) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) __builtin_nontemporal_store(b[u], s1 + base + u * 256);
+      if (SN_IN_RANGE(u)) __builtin_nontemporal_store(b[u], s1 + base + u * T);
   }
   if (NS > 2) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) __builtin_nontemporal_store(c[u], s2 + base + u * 256);
+      if (SN_IN_RANGE(u)) __builtin_nontemporal_store(c[u], s2 + base + u * T);
   }
 }
+#undef SN_IN_RANGE
 
 // Scalar form for a misaligned buffer or the last n % 4 elements.
 template <int KIND>
@@ -183,14 +185,17 @@ static bool aligned16(const void* p) { return p == nullptr || (reinterpret_cast<
 template <int KIND>
 static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g, float* s0, float* s1, float* s2, int64_t n,
                         const OptScalars& p) {
-  constexpr int UNROLL = 4;
+  // One vector per thread; threads per block measured per number of state tensors on 100 M elements (MI355X): 128 for one or
+  // two states (SGD 308 us against 319 with 4 vectors x 256 threads, Adam 446 against 467), 64 for three (AMSGrad 596
+  // against 614).  Many small blocks keep more independent request streams in flight than few large ones.
+  constexpr int UNROLL = 1, THREADS = n_states<KIND>() <= 2 ? 128 : 64;
   const bool vec = aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2);
   const int64_t n4 = vec ? n / 4 : 0;
   if (n4 > 0) {
-    const int64_t blocks = ceil_div(n4, (int64_t)256 * UNROLL);  // one pass, no grid-stride loop
+    const int64_t blocks = ceil_div(n4, (int64_t)THREADS * UNROLL);  // one pass, no grid-stride loop
     SN_REQUIRE(blocks <= 0x7fffffff, "optimizer update over %lld elements exceeds one launch", (long long)n);
     LaunchScope scope(ctx, name);
-    hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (f4*)w,
+    hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
                        (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p);
   }
   const int64_t done = n4 * 4;
@@ -232,10 +237,18 @@ struct AvgOutputs {
   float* p[SN_MAX_AVG_INPUTS + 1];
 };
 
-// Block-contiguous like the optimizer kernel: a block owns 256*U float4, reads them input by input.
+// Block-contiguous like the optimizer kernel: a block owns AVG_T*U float4, reads them input by input.  Measured on 8 x 25 M
+// (MI355X): 128 threads x 1 vector 6.18 TB/s, 64 x 1 6.20, 256 x 2 5.98, 256 x 1 5.54, 512 x 1 5.91; a plain copy
+// kernel of the same shape reaches 6.15 TB/s on the same box.
+constexpr int AVG_T = 128;
 template <int K_STATIC, int U>
-__global__ __launch_bounds__(256) void average_kernel_v4(AvgInputs in, int k, int64_t n4, AvgOutputs out, int n_out, float kf) {
-  const int64_t base = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+__global__ __launch_bounds__(AVG_T) void average_kernel_v4(AvgInputs in, int k, int64_t n4, AvgOutputs out, int n_out, float kf) {
+  constexpr int T = AVG_T;
+  const int64_t base = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
+  // with one vector per thread the bounds check is one early exit; a check around every load made the compiler wait for
+  // each load before it issued the next
+  if (U == 1 && base >= n4) return;
+#define SN_IN_RANGE(u) (U == 1 || base + (u) * T < n4)
   f4 acc[U];
   if constexpr (K_STATIC > 0) {
     f4 v[K_STATIC][U];
@@ -243,7 +256,7 @@ __global__ __launch_bounds__(256) void average_kernel_v4(AvgInputs in, int k, in
     for (int r = 0; r < K_STATIC; ++r)
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (base + u * 256 < n4) v[r][u] = __builtin_nontemporal_load((const f4*)in.p[r] + base + u * 256);
+        if (SN_IN_RANGE(u)) v[r][u] = __builtin_nontemporal_load((const f4*)in.p[r] + base + u * T);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       acc[u] = v[0][u];
@@ -253,19 +266,20 @@ __global__ __launch_bounds__(256) void average_kernel_v4(AvgInputs in, int k, in
   } else {
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) acc[u] = __builtin_nontemporal_load((const f4*)in.p[0] + base + u * 256);
+      if (SN_IN_RANGE(u)) acc[u] = __builtin_nontemporal_load((const f4*)in.p[0] + base + u * T);
     for (int r = 1; r < k; ++r)
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (base + u * 256 < n4) acc[u] = acc[u] + __builtin_nontemporal_load((const f4*)in.p[r] + base + u * 256);
+        if (SN_IN_RANGE(u)) acc[u] = acc[u] + __builtin_nontemporal_load((const f4*)in.p[r] + base + u * T);
   }
 #pragma unroll
   for (int u = 0; u < U; ++u) acc[u] = acc[u] / kf;  // `plus(inputs) / inputs.size` (models/Aggregation.scala:16-19)
   for (int o = 0; o < n_out; ++o)
 #pragma unroll
     for (int u = 0; u < U; ++u)
-      if (base + u * 256 < n4) __builtin_nontemporal_store(acc[u], (f4*)out.p[o] + base + u * 256);
+      if (SN_IN_RANGE(u)) __builtin_nontemporal_store(acc[u], (f4*)out.p[o] + base + u * T);
 }
+#undef SN_IN_RANGE
 
 __global__ __launch_bounds__(256) void average_kernel_scalar(AvgInputs in, int k, int64_t first, int64_t n, AvgOutputs out,
                                                               int n_out, float kf) {
@@ -292,18 +306,18 @@ int launch_average(sn_ctx* ctx, const AvgInputs& in, int k, int64_t n, float* ou
   const int64_t n4 = vec ? n / 4 : 0;
   const float kf = (float)k;
   if (n4 > 0) {
-    constexpr int U = 2;
-    const int64_t blocks = ceil_div(n4, 256 * U);
+    constexpr int U = 1;
+    const int64_t blocks = ceil_div(n4, AVG_T * U);
     SN_REQUIRE(blocks <= 0x7fffffff, "average over %lld elements exceeds one launch", (long long)n);
     LaunchScope scope(ctx, "average_replicas");
     if (k == 8)
-      hipLaunchKernelGGL((average_kernel_v4<8, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<8, U>), dim3((unsigned)blocks), dim3(AVG_T), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else if (k == 4)
-      hipLaunchKernelGGL((average_kernel_v4<4, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<4, U>), dim3((unsigned)blocks), dim3(AVG_T), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else if (k == 2)
-      hipLaunchKernelGGL((average_kernel_v4<2, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<2, U>), dim3((unsigned)blocks), dim3(AVG_T), 0, ctx->stream, in, k, n4, o, n_out, kf);
     else
-      hipLaunchKernelGGL((average_kernel_v4<0, U>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, in, k, n4, o, n_out, kf);
+      hipLaunchKernelGGL((average_kernel_v4<0, U>), dim3((unsigned)blocks), dim3(AVG_T), 0, ctx->stream, in, k, n4, o, n_out, kf);
   }
   if (n4 * 4 < n) {
     LaunchScope scope(ctx, "average_replicas");
