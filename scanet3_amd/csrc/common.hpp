@@ -175,6 +175,13 @@ int launch_sequence_gather(sn_ctx* ctx, const float* slices, int64_t slice_strid
 int launch_step_slice_add(sn_ctx* ctx, float* dst, const float* src, int64_t src_ld, int rows, int H, bool accumulate);
 int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int hidden);
 
+// ---- Dense(H, act) >> Dense(C, Softmax) + CategoricalCrossentropy in two launches (mlp2_kernels.hip): forward, loss terms
+// and every gradient.  scratch_a / scratch_b: what mlp2_fused_ok asks for; row_loss: `rows` floats.
+bool mlp2_fused_ok(int rows_max, int K, int H, int C, int64_t scratch_a_elems, int64_t scratch_b_elems);
+int launch_mlp2_grad(sn_ctx* ctx, const float* x, const float* y, const float* w1, const float* b1, const float* w2, const float* b2, int rows,
+                     int K, int H, int C, int act1, float act1_param, bool stable, float* h, float* z2, float* p, float* scratch_a,
+                     float* scratch_b, float* row_loss, float* loss_dev, float* g_w1, float* g_b1, float* g_w2, float* g_b2);
+
 // ---- seeded random tensors (random_kernels.hip): scale / shift may be null
 int launch_random_fill(sn_ctx* ctx, float* out, int64_t n, int dist, uint64_t seed, const float* scale, const float* shift);
 

@@ -929,9 +929,33 @@ static int read_loss(sn_replica* r, float* loss_host) {
 
 // want_loss = false: the caller does not read this step's loss value (the steps inside an epoch, sn_step / sn_grad without a
 // loss pointer), so the kernels that only finish the scalar are not launched
+// Dense(H, act) >> Dense(C) >> Softmax under CategoricalCrossentropy, small enough for the two-launch training pass
+static bool mlp2_path(const sn_model* m) {
+  if (m->ops.size() != 3 || m->loss != SN_LOSS_CATEGORICAL_CROSSENTROPY || (m->flags & SN_FLAG_GEMM_BF16)) return false;
+  const Op& d1 = m->ops[0];
+  const Op& d2 = m->ops[1];
+  if (d1.kind != OP_DENSE || d2.kind != OP_DENSE || d2.act != SN_ACT_IDENTITY || m->ops[2].kind != OP_SOFTMAX) return false;
+  const int64_t scratch = (int64_t)m->batch * m->max_act_elems;
+  return mlp2_fused_ok(m->batch, (int)d1.in_elems, (int)d1.out_elems, (int)d2.out_elems, scratch, scratch);
+}
+
 static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss) {
   sn_model* m = r->model;
   const int last = (int)m->ops.size() - 1;
+  if (mlp2_path(m)) {
+    const Op& d1 = m->ops[0];
+    const Op& d2 = m->ops[1];
+    SN_TRY(launch_mlp2_grad(r->ctx, x, y, param_ptr(r, r->w, d1.w), param_ptr(r, r->w, d1.b), param_ptr(r, r->w, d2.w), param_ptr(r, r->w, d2.b), rows,
+                            (int)d1.in_elems, (int)d1.out_elems, (int)d2.out_elems, d1.act, d1.act_param,
+                            (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0, r->act[0], r->act[1], r->act[2], r->grad_buf[0], r->grad_buf[1],
+                            r->loss_partials, want_loss ? r->loss_dev : nullptr, param_ptr(r, r->g, d1.w), param_ptr(r, r->g, d1.b),
+                            param_ptr(r, r->g, d2.w), param_ptr(r, r->g, d2.b)));
+    if (want_loss) SN_TRY(add_penalties(r, true));
+    for (auto& p : m->params)
+      if (p.reg_kind != SN_REG_NONE)
+        SN_TRY(launch_penalty_grad(r->ctx, r->w + p.info.offset, r->g + p.info.offset, p.info.size, p.reg_kind, p.reg_lambda));
+    return SN_OK;
+  }
   if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
     // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
     SN_TRY(forward(r, x, rows, true, true));

@@ -448,6 +448,12 @@ MODELS = {
     "batchnorm_200_channels": ([("dense", 200, "tanh"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
     "batchnorm_256_channels": ([("dense", 256, "relu"), ("batchnorm", 0.9, 1e-3), ("dense", 5, "softmax")], "cce", (31,), 300, "normal_onehot"),
     "dense_identity_mse": ([("dense", 6, "identity")], "mse", (4,), 8, "normal_regression"),
+    # Dense >> Dense(Softmax) + CategoricalCrossentropy small enough for the two-launch training pass: a reduction length
+    # that is no multiple of 16, rows that are no multiple of 16, all 64 hidden units / 16 classes, penalties on top
+    "mlp2_odd_sizes_tanh": ([("dense", 37, "tanh"), ("dense", 16, "softmax")], "cce", (36,), 33, "normal_onehot"),
+    "mlp2_64_hidden_relu": ([("dense", 64, "relu"), ("dense", 3, "softmax")], "cce", (1024,), 100, "normal_onehot"),
+    "mlp2_identity_one_class": ([("dense", 5, "identity"), ("dense", 1, "softmax")], "cce", (8,), 16, "normal_onehot"),
+    "mlp2_regularized": ([("dense", 20, "sigmoid", "l2", 0.05), ("dense", 4, "softmax", "l1", 0.01)], "cce", (8,), 17, "uniform_onehot"),
 }
 
 
@@ -500,7 +506,7 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     h.close()
 
 
-@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
+@pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("mlp2_odd_sizes_tanh", 15), ("mlp2_regularized", 15), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
                                         ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("cnn_batchnorm_fused", 12), ("mlp_bce_l2", 25),
                                         ("lstm_regularized", 15), ("batchnorm_regularized", 15)])
 @pytest.mark.parametrize("alg", ["adam", "sgd_momentum", "amsgrad"])
