@@ -437,6 +437,12 @@ MODELS = {
                                             ("dense", 3, "softmax")], "cce", (21, 19, 2), 40, "uniform_onehot"),
     "conv_first_layer_four_filters": ([("conv", 4, (2, 2), (1, 1), "valid", "relu", False), ("flatten",), ("dense", 3, "softmax")],
                                       "cce", (30, 30, 3), 8, "uniform_onehot"),
+    # second-layer filter gradient in its row form (32 or 64 input channels): an odd row length (one padding position per row), Same
+    # padding on all four sides, a stride in each direction, a bias; and 64 input channels under a 5 x 3 kernel onto 32 filters
+    "conv_rows_same_stride_bias": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 64, (3, 3), (2, 1), "same", "tanh", True),
+                                    ("flatten",), ("dense", 3, "softmax")], "cce", (14, 13, 1), 80, "uniform_onehot"),
+    "conv_rows_64_channels_5x3": ([("conv", 64, (3, 3), (1, 1), "valid", "tanh", False), ("conv", 32, (5, 3), (1, 2), "same", "relu", False),
+                                   ("flatten",), ("dense", 3, "softmax")], "cce", (12, 12, 1), 90, "uniform_onehot"),
     # Dense from thousands of features onto a few units: gradients as row streams (2048+ features, at most 16 units); a feature count
     # that leaves a partial block of 64, 7 rows over 4 wavefronts, 16 and 5 units, an L2 penalty on the streamed weights
     "dense_many_features_few_units": ([("dense", 2050, "tanh"), ("dense", 5, "softmax", "l2", 0.01)], "cce", (33,), 7, "normal_onehot"),
