@@ -126,6 +126,7 @@ def model_work(layers, in_shape, batch):
             fwd, dh, wg, dx = 2.0 * batch * G * H * (F + H), 2.0 * batch * H * G * H, 2.0 * (F + H) * G * H * T * batch, 2.0 * batch * F * G * H
             total += T * fwd + (T - 1) * dh + wg + (0 if first else T * dx)
             labels[f"[{batch}x{G * H}x{F + H}]"] = fwd
+            labels[f"[{batch * T}x{G * H}x{F + H}]"] = T * fwd             # every forward step in one launch
             labels[f"[{batch}x{G * H}x{H}]"] = 2.0 * batch * G * H * H       # the recurrent half alone (input half hoisted)
             labels[f"[{batch * T}x{G * H}x{F}]"] = 2.0 * batch * T * G * H * F
             labels[f"[{batch}x{H}x{G * H}]"] = dh

@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -58,6 +59,14 @@ struct sn_ctx {
   bool owns_stream;
   int compute_units;
   int live_models = 0;  // models created from this context and not yet destroyed
+  // Recurrent sequence kernels (one launch for all time steps): arrival counters of their row groups in device memory,
+  // a word in pinned host memory that such a kernel sets when it gives up waiting for its neighbours, and how many
+  // polls it waits before it does.  Allocated by the first launch that needs them.
+  unsigned* seq_arrived = nullptr;
+  int* seq_gave_up = nullptr;      // host address
+  int* seq_gave_up_dev = nullptr;  // the same word as the device sees it
+  unsigned seq_spin_limit = 0;
+  int seq_force_coherent = 0;      // hand over as if every row group were spread over several XCDs
   // timing
   bool profiling;
   std::vector<sn::PendingEvent> pending;
@@ -85,6 +94,11 @@ struct LaunchScope {
   ~LaunchScope();
 };
 int profile_drain(sn_ctx* ctx);
+// Sets up the context's sequence-kernel words on first use.
+int seq_sync_init(sn_ctx* ctx);
+constexpr int SEQ_COUNTERS = 1024;
+// After a stream synchronisation: SN_E_STATE (once) if a sequence kernel gave up waiting since the last check.
+int check_async(sn_ctx* ctx);
 // looks up this device's address of the library's static scratch array (model.hip); `device` must be current
 int static_scratch_init(int device);
 
@@ -326,6 +340,13 @@ bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w, int 
 // (Wr of the 4 gates), lstm_pack_elems(F, H) floats each at most; rebuilt once per pass over the sequence.
 int64_t lstm_pack_elems(int F, int H);
 int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh, int gates = 4);
+// All T forward steps of an LSTM layer in one launch: the workgroups keep their weight slab in LDS and hand h_t to each
+// other through memory, one arrival counter per group of 32 batch rows.  h: T + 1 slices of `slice` floats, slice 0 the
+// initial hidden state (read only if h0_valid); gates / c: T slices.  lstm_sequence_fwd_ok says whether the launch fits
+// the device whole, which the hand-over needs.
+bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w);
+int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
+                             const float* wpack, float* gates, float* c, float* h, int64_t slice);
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h);
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev

@@ -197,6 +197,203 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------- all forward steps in one launch
+// The same decomposition as the step kernel (32 batch rows x 16 hidden units per workgroup), but the workgroup stays for
+// the whole sequence: its weight slab is copied to LDS once, its cell states live in registers, and only [x_t, h_{t-1}]
+// is fetched per step.  h_t is handed from the unit groups of a row group to each other through memory: after its
+// stores of step t have been acknowledged a workgroup adds 1 to the row group's arrival counter; before step t + 1 it
+// waits until the counter shows every workgroup of the group.  That needs all workgroups of the launch on the device at
+// once, which the host checks against the device's occupancy before it picks this kernel.  The wait is bounded all the
+// same: a workgroup that polls `spin_limit` times in vain (or sees that another one did) raises the abort word, reports
+// through `gave_up` and leaves, and so does every other workgroup at its next wait.
+//
+// The hand-over avoids device-scope fences, which on this hardware write back and invalidate a whole L2 and cost tens
+// of microseconds per step here.  Two forms instead, chosen per row group:
+//   within one XCD   plain stores and loads.  The XCD's L2 is the one cache between its CUs: a store acknowledged
+//                    (s_waitcnt vmcnt(0)) is in L2, and a load of an address this CU has not touched in this launch
+//                    (every h slice is read once) misses L1 and finds it there.  7.1 us per step at 512 x 256.
+//   across XCDs      every access is itself coherent at device scope: h_t is written with device-scope atomic stores
+//                    (write-through), read with loads that carry the same coherence bit (sc1).  14.3 us per step.
+// Workgroup ids are mapped to (row group, unit group) so that a row group's workgroups have ids congruent mod 8, which
+// the dispatcher places on one XCD.  That is not taken on trust: each workgroup reads the XCD it runs on from the
+// hardware register, the members of a row group compare theirs in a first arrival round before any hand-over, and one
+// mismatch switches the whole row group to the second form.  The counter itself is only touched with device-scope atomics.
+__device__ __forceinline__ f4v load_coherent(const float* p) {
+  f4v v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+template <int N>
+__device__ __forceinline__ void wait_coherent_loads(f4v (&v)[N]) {  // ties the wait to the registers the loads fill
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i]));
+}
+
+struct SeqFwdArgs {
+  const float* x;        // [rows, T, F]
+  const float* c0;       // [rows, H] or null: zeros
+  const float* wpack;    // pack_fwd_kernel's order
+  const float* bias[4];
+  float* gates;          // T slices of 4 * slice floats: activated forget, input, gate, output of [rows, 4H]
+  float* c;              // T slices
+  float* h;              // T + 1 slices, slice t + 1 = h_t; slice 0 is read only if h0_valid
+  int64_t slice;
+  int h0_valid;
+  int rows, T, F, H;
+  int row_groups, unit_groups;
+  unsigned* sync;        // zero at launch: [row groups] arrival counters, [row groups] XCD words, [row groups] spread flags, abort word
+  unsigned spin_limit;
+  int* gave_up;          // host-visible
+  int force_coherent;    // take the across-XCD form everywhere
+};
+
+// Waits (thread 0 polls) until *count >= target.  Returns nonzero in every thread if the wait was given up.
+__device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, unsigned* abort_word, unsigned spin_limit, int* gave_up, int* stop) {
+  if (threadIdx.x == 0) {
+    unsigned spins = 0;
+    int bad = 0;
+    while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (__hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u || ++spins > spin_limit) {
+        bad = 1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (bad) {
+      __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    *stop = bad;
+  }
+  __syncthreads();
+  return *stop;
+}
+
+__global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
+  constexpr int UB = 16, NCB = 4, NRB = 2;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ int stop;
+  const int K = a.F + a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
+  float* As = lds;  // [RB][KP]
+  float* Zx = lds;  // [4 gates][RB][ZP] over As once every wavefront has finished multiplying
+  float* Bs = lds + (RB * KP > 4 * RB * ZP ? RB * KP : 4 * RB * ZP);  // [NCB][kq][16 columns][4], kept for the whole sequence
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // id -> (row group, unit group): ids congruent mod 8 share an XCD, so XCD x takes the row groups x, x + 8, ...
+  const int slot = blockIdx.x >> 3;
+  const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
+  if (rg >= a.row_groups) return;  // the grid is rounded up to whole rounds of 8 row groups
+  const int r0 = rg * RB, u0 = ug * UB;
+  unsigned* my_count = a.sync + rg;
+  unsigned* my_xcd = a.sync + a.row_groups + rg;
+  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
+  unsigned* abort_word = a.sync + 3 * a.row_groups;
+
+  // ---- arrival round 0: do the members of this row group share an XCD?
+  if (tid == 0) {
+    const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
+    unsigned seen = 0u;
+    __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((seen != 0u && seen != mine) || a.force_coherent) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the flag is acknowledged before this workgroup counts itself in, so whoever has seen the full count sees the flag
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+    __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  {  // the slab of this unit group: 4 gates x kq quads x 16 units, already in LDS cell order
+    const f4v* slab = reinterpret_cast<const f4v*>(a.wpack) + (int64_t)ug * NCB * kq * 16;
+    for (int e = tid; e < NCB * kq * 16; e += 256) reinterpret_cast<f4v*>(Bs)[e] = slab[e];
+  }
+  // the two cells this thread finishes per step: row e / 16, unit e % 16 for e = tid, tid + 256
+  float c_reg[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int e = tid + 256 * j, row = e / UB, u = e % UB;
+    c_reg[j] = a.c0 && r0 + row < a.rows ? a.c0[(int64_t)(r0 + row) * a.H + u0 + u] : 0.f;
+  }
+  const int cb = wave % NCB, rb0 = (wave / NCB) * NRB;
+  float bias;
+  {
+    const int col = cb * 16 + (lane & 15);
+    bias = a.bias[col / UB] ? a.bias[col / UB][u0 + col % UB] : 0.f;
+  }
+
+  constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
+  const int arow = tid >> 3;
+  bool spread = true;  // until round 0 is complete (the first wait below), write as if the row group were spread out
+  for (int t = 0; t < a.T; ++t) {
+    const bool with_h = t > 0 || a.h0_valid;
+    if (t > 0) {  // h_{t-1} is complete once every unit group of this row group has arrived t + 1 times (round 0 included)
+      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(t + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+      if (t == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    }
+    // ---- [x_t, h_{t-1}] of the 32 rows: every load is issued before the first LDS write
+    {
+      f4v va[NA];
+      const float* hp = a.h + (int64_t)t * a.slice;
+      const bool coherent = spread && t > 0;  // slice 0 was written before this launch
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int q = i * 8 + (tid & 7), k = q * 4;
+        va[i] = f4v{0.f, 0.f, 0.f, 0.f};
+        if (q < kq && r0 + arow < a.rows && k < K) {
+          if (k < a.F) va[i] = *(const f4v*)(a.x + ((int64_t)(r0 + arow) * a.T + t) * a.F + k);
+          else if (!with_h) continue;
+          else if (coherent) va[i] = load_coherent(hp + (int64_t)(r0 + arow) * a.H + (k - a.F));
+          else va[i] = *(const f4v*)(hp + (int64_t)(r0 + arow) * a.H + (k - a.F));
+        }
+      }
+      if (coherent) wait_coherent_loads(va);
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int q = i * 8 + (tid & 7);
+        if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
+      }
+    }
+    __syncthreads();
+    f4v acc[NRB];
+#pragma unroll
+    for (int r = 0; r < NRB; ++r) acc[r] = f4v{0.f, 0.f, 0.f, 0.f};
+    multiply_blocks<NRB>(As, Bs, K16, cb, rb0, lane, acc);
+    __syncthreads();
+    {  // pre-activations to the exchange area: element v of a lane is row 4*(l/16) + v of its block, column l%16
+      const int col = cb * 16 + (lane & 15), gate = col / UB, u = col % UB, g = lane >> 4;
+#pragma unroll
+      for (int r = 0; r < NRB; ++r)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) Zx[(gate * RB + (rb0 + r) * 16 + 4 * g + v) * ZP + u] = acc[r][v] + bias;
+    }
+    __syncthreads();
+    // ---- c = c_prev * f + i * g ; h = o * tanh(c)   (layer/RNN.scala:336-337)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = tid + 256 * j, row = e / UB, u = e % UB;
+      if (r0 + row >= a.rows) continue;
+      const float f = sigmoidf_(Zx[(0 * RB + row) * ZP + u]);
+      const float in = sigmoidf_(Zx[(1 * RB + row) * ZP + u]);
+      const float g = tanhf(Zx[(2 * RB + row) * ZP + u]);
+      const float o = sigmoidf_(Zx[(3 * RB + row) * ZP + u]);
+      const int64_t i = (int64_t)(r0 + row) * a.H + u0 + u;
+      float* gt = a.gates + (int64_t)t * 4 * a.slice + (int64_t)(r0 + row) * 4 * a.H + u0 + u;
+      const float c = c_reg[j] * f + in * g;
+      c_reg[j] = c;
+      gt[0] = f;
+      gt[a.H] = in;
+      gt[2 * a.H] = g;
+      gt[3 * a.H] = o;
+      a.c[(int64_t)t * a.slice + i] = c;
+      float* hout = a.h + (int64_t)(t + 1) * a.slice + i;
+      if (spread) __hip_atomic_store(hout, o * tanhf(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else *hout = o * tanhf(c);
+    }
+    // ---- hand h_t over: every wavefront waits until its stores have been acknowledged, then one thread counts the
+    // workgroup in
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
+    __syncthreads();  // (also: Zx is free again)
+    if (tid == 0 && t + 1 < a.T) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // ---------------------------------------------------------------------------- one product per step, whole K in LDS
 // out_z[m, u] = sum_k A[m, k] * W_z[u, k] for z = blockIdx.z, where a row of A is [a0 row (k0 values), a1 row (k1 values)]
 // and W_z comes packed as [unit block of 16][k/4][16 units][4 consecutive k] with `kq_pack` quads per unit block.
@@ -521,6 +718,39 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
   LaunchScope scope(ctx, "lstm_step_forward", rows, 4 * H, K);
   SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_fwd_kernel, lds_bytes(MAX_K, 64)));
   hipLaunchKernelGGL(lstm_step_fwd_kernel, dim3((unsigned)(H / 16), (unsigned)ceil_div(rows, RB)), dim3(256), lds_bytes(K, 64), ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+namespace {
+size_t sequence_lds_bytes(int K) {  // the weight slab lies behind both the operand rows and the exchange area
+  const int K16 = round16(K);
+  return ((size_t)std::max(RB * (K16 + 4), 4 * RB * ZP) + (size_t)64 * K16) * sizeof(float);
+}
+}  // namespace
+
+bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) {
+  if (rows <= 0 || !lstm_step_fused_ok(F, H, x, w)) return false;
+  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+  if (3 * groups + 1 > SEQ_COUNTERS) return false;
+  if (allow_dynamic_lds(ctx, (const void*)lstm_sequence_fwd_kernel, sequence_lds_bytes(MAX_K)) != SN_OK) return false;
+  int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_sequence_fwd_kernel, 256, sequence_lds_bytes(F + H)) != hipSuccess) return false;
+  return blocks <= (int64_t)per_cu * ctx->compute_units;
+}
+
+int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
+                             const float* wpack, float* gates, float* c, float* h, int64_t slice) {
+  if (rows <= 0 || T <= 0) return SN_OK;
+  SN_REQUIRE(lstm_sequence_fwd_ok(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SN_TRY(seq_sync_init(ctx));
+  const int groups = (int)ceil_div(rows, RB);
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * groups + 1));  // all-zero bits
+  SeqFwdArgs a{x, c0, wpack, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
+               ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+  LaunchScope scope(ctx, "lstm_sequence_forward", rows * T, 4 * H, F + H);  // T steps of rows x 4H x (F + H)
+  hipLaunchKernelGGL(lstm_sequence_fwd_kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_lds_bytes(F + H),
+                     ctx->stream, a);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

@@ -601,6 +601,12 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         if (carried)
           SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[1]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
                                 ctx->stream));
+        if (fused && op.T > 1 && lstm_sequence_fwd_ok(ctx, rows, op.F, op.H, in, w)) {  // every step in one launch
+          SN_TRY(launch_lstm_sequence_fwd(ctx, in, op.T, op.F, carried ? 1 : 0, carried ? param_ptr(r, r->w, op.state_p[0]) : nullptr, rows, op.H,
+                                          w, r->lstm_pk_fwd[i], r->lstm_gates[i], r->lstm_c[i], r->lstm_h[i], bh));
+          if (op.ret_seq) SN_TRY(launch_sequence_gather(ctx, r->lstm_h[i], bh, 1, r->act[i], rows, op.T, op.H));
+          break;
+        }
         for (int t = 0; t < op.T; ++t) {
           const float* h_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
           const float* c_prev = t == 0 ? (carried ? param_ptr(r, r->w, op.state_p[0]) : nullptr) : r->lstm_c[i] + (int64_t)(t - 1) * bh;
@@ -924,7 +930,7 @@ static int read_loss(sn_replica* r, float* loss_host) {
   if (!loss_host) return SN_OK;
   SN_HIP(hipMemcpyAsync(loss_host, r->loss_dev, sizeof(float), hipMemcpyDeviceToHost, r->ctx->stream));
   SN_HIP(hipStreamSynchronize(r->ctx->stream));
-  return SN_OK;
+  return check_async(r->ctx);
 }
 
 // want_loss = false: the caller does not read this step's loss value (the steps inside an epoch, sn_step / sn_grad without a

@@ -78,6 +78,40 @@ int profile_drain(sn_ctx* ctx) {
   return SN_OK;
 }
 
+int seq_sync_init(sn_ctx* ctx) {
+  if (ctx->seq_arrived) return SN_OK;
+  unsigned* arrived = nullptr;
+  int* word = nullptr;
+  void* word_dev = nullptr;
+  SN_HIP(hipSetDevice(ctx->device));
+  hipError_t e = hipMalloc(&arrived, SEQ_COUNTERS * sizeof(unsigned));
+  if (e == hipSuccess) e = hipHostMalloc(&word, sizeof(int), hipHostMallocMapped);
+  if (e == hipSuccess) {
+    *word = 0;
+    e = hipHostGetDevicePointer(&word_dev, word, 0);
+  }
+  if (e != hipSuccess) {
+    if (arrived) (void)hipFree(arrived);
+    if (word) (void)hipHostFree(word);
+    return fail(SN_E_HIP, "setting up the sequence kernels' counters failed: %s", hipGetErrorString(e));
+  }
+  ctx->seq_arrived = arrived;
+  ctx->seq_gave_up = word;
+  ctx->seq_gave_up_dev = static_cast<int*>(word_dev);
+  // about a microsecond per poll: two seconds before a kernel whose neighbours never arrive gives up
+  ctx->seq_spin_limit = 2000000u;
+  if (const char* v = getenv("SCANET_SEQUENCE_SPIN_LIMIT")) ctx->seq_spin_limit = (unsigned)strtoul(v, nullptr, 10);
+  if (const char* v = getenv("SCANET_SEQUENCE_COHERENT")) ctx->seq_force_coherent = atoi(v) != 0;
+  return SN_OK;
+}
+
+int check_async(sn_ctx* ctx) {
+  if (!ctx->seq_gave_up || *(volatile int*)ctx->seq_gave_up == 0) return SN_OK;
+  *(volatile int*)ctx->seq_gave_up = 0;
+  return fail(SN_E_STATE, "a recurrent sequence kernel gave up waiting for its neighbour workgroups (are other processes using this GPU?): "
+                          "the results of the calls since the last synchronisation are invalid");
+}
+
 static int check_ctx(sn_ctx* ctx) {
   if (!ctx || ctx->magic != CTX_MAGIC) return fail(SN_E_STATE, "invalid or destroyed context handle");
   return SN_OK;
@@ -134,6 +168,8 @@ int sn_ctx_destroy(sn_ctx* ctx) {
     (void)hipEventDestroy(p.stop);
   }
   for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+  if (ctx->seq_arrived) (void)hipFree(ctx->seq_arrived);
+  if (ctx->seq_gave_up) (void)hipHostFree(ctx->seq_gave_up);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   ctx->magic = 0;
   delete ctx;
@@ -143,7 +179,7 @@ int sn_ctx_destroy(sn_ctx* ctx) {
 int sn_sync(sn_ctx* ctx) {
   SN_TRY(check_ctx(ctx));
   SN_HIP(hipStreamSynchronize(ctx->stream));
-  return SN_OK;
+  return check_async(ctx);
 }
 
 int sn_device_info(sn_ctx* ctx, char* name, int name_cap, int64_t* hbm_bytes, int32_t* compute_units) {
@@ -206,7 +242,7 @@ int sn_copy_d2h(sn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes) 
   SN_REQUIRE(dst_host && src_dev, "sn_copy_d2h: null pointer");
   SN_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
   SN_HIP(hipStreamSynchronize(ctx->stream));
-  return SN_OK;
+  return check_async(ctx);
 }
 
 int sn_fill(sn_ctx* ctx, float* dst_dev, float value, int64_t n) {

@@ -1013,6 +1013,65 @@ def test_stateful_rnn_steps_match_oracle(S, ctx, kind, units, features, batch):
     Yb.free()
 
 
+@pytest.mark.parametrize("coherent", ["0", "1"])
+def test_lstm_sequence_kernel_hands_over_within_and_across_xcds(S, monkeypatch, coherent):
+    """The one-launch LSTM forward picks per row group how h_t travels between workgroups: plain accesses when the row group
+    sits on one XCD, device-coherent ones otherwise.  SCANET_SEQUENCE_COHERENT=1 (read when a context first launches the
+    kernel) forces the second form everywhere; both must give the oracle's numbers, here with several row groups, a partial
+    last one, 4 unit groups and a carried state."""
+    monkeypatch.setenv("SCANET_SEQUENCE_COHERENT", coherent)
+    c = S.Context(0)
+    try:
+        units, T, features, batch = 64, 9, 12, 150
+        om = O.Model([O.LSTM(units, stateful=True), O.Dense(2, O.ACT_IDENTITY)], O.LOSS_MSE)
+        layers = S.LSTM(units, stateful=True) >> S.Dense(2, S.Identity)
+        cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+        rep = cm.replica(None)
+        rng = np.random.default_rng(77)
+        params = glorot_params(om, (batch, T, features), rng)
+        for p in params:
+            if O.is_unaggregated_path(p):
+                params[p] = rng.uniform(-0.5, 0.5, params[p].shape).astype(f32)
+        x = rng.standard_normal((batch, T, features)).astype(f32)
+        y = rng.uniform(-1, 1, (batch, 2)).astype(f32)
+        rep.set_params(params)
+        xb, yb = c.to_device(x), c.to_device(y)
+        assert rel_err(rep.forward(xb), om.forward(x, params)) <= TOL_GEMM
+        oloss, ograds = om.grad(x, y, params)
+        assert abs(rep.grad(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+        ggrads = rep.get_grads()
+        for p in ograds:
+            assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        for o in (rep, cm):
+            o.close()
+        xb.free()
+        yb.free()
+    finally:
+        c.close()
+
+
+def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch):
+    """A workgroup of the one-launch LSTM forward that waits for its neighbours polls a bounded number of times.  With the
+    bound forced to zero (SCANET_SEQUENCE_SPIN_LIMIT, read when a context first launches the kernel) the first workgroup
+    that has to wait gives up, every other one follows at its next wait, the kernel ends, and the next synchronising call
+    reports it once."""
+    monkeypatch.setenv("SCANET_SEQUENCE_SPIN_LIMIT", "0")
+    c = S.Context(0)
+    try:
+        layers = S.LSTM(256) >> S.Dense(1, S.Tanh)
+        cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (64, 32), 512)
+        rep = cm.replica(None)
+        xb = c.to_device(np.random.default_rng(5).standard_normal((512, 64, 32)).astype(f32))
+        with pytest.raises(S.ScanetError, match="gave up waiting"):
+            rep.forward(xb)
+        c.sync()                          # reported once: the context stays usable
+        for o in (rep, cm):
+            o.close()
+        xb.free()
+    finally:
+        c.close()
+
+
 def test_maximizing_step_adds_the_delta(S, ctx):
     """`Optimizer.maximize` (Optimizer.scala:186,326-336): w + delta, through the flat kernel and through sn_step."""
     from scanet3_amd import _lib as L
