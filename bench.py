@@ -300,6 +300,19 @@ def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
 CSRC = os.path.join(ROOT, "scanet3_amd", "csrc")
 MEASURED_TRAFFIC = {
     # kernel label (or optimizer name): (bytes per launch, source file, sha1 of the file when measured)
+    # rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (one run each), KiB per dispatch, scaled by what the same counters read
+    # for a plain copy of 400 MB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the summaries are under profiles/
+    "conv2d_forward[52900x64x288]": (22.26e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
+    "conv2d_input_gradient[62500x32x576]": (22.31e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
+    "conv2d_filter_gradient[288x64x52900]": (42.06e6, "gemm_kernels.hip", "78b4b4210fc4231c76bc9149edbb1284b66dabc5"),
+    "gemm_bf16_256[8192x4096x4096]": (539.0e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
+    "gemm_bf16_256[4096x4096x8192]": (495.3e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
+    "gemm_bf16_256_handover[8192x4096x4096]": (469.5e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
+    "lstm_sequence_forward[32768x1024x288]": (248.9e6, "lstm_kernels.hip", "47f1d2fd485afeb9f2ee37fc61587908b2151a7e"),
+    "lstm_step_backward[512x256x1024]": (15.75e6, "lstm_kernels.hip", "47f1d2fd485afeb9f2ee37fc61587908b2151a7e"),
+    "lstm_weight_gradient[289x1024x32768]": (323.0e6, "gemm_kernels.hip", "78b4b4210fc4231c76bc9149edbb1284b66dabc5"),
+    "adam": (2.800e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
+    "average": (0.900e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
 }
 
 
