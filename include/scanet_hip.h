@@ -172,7 +172,14 @@ SN_API int sn_ctx_create(int device, void* stream, sn_ctx** out);
 SN_API int sn_ctx_destroy(sn_ctx* ctx);
 /* Message of the calling thread's most recent failing call (never NULL). */
 SN_API const char* sn_last_error(void);
-/* Blocks until everything issued on the context's stream has finished. */
+/* Blocks until everything issued on the context's stream has finished.
+ * Like every call that synchronises (sn_copy_d2h, a step or gradient call that returns its loss), it returns
+ * SN_E_STATE once if a recurrent layer's one-launch forward kernel gave up waiting for its neighbour workgroups
+ * since the previous synchronisation (only possible when something else occupies compute units of the same GPU):
+ * the results computed since then are invalid, the context stays usable.  The wait is a bounded number of polls
+ * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, read when a context first launches that
+ * kernel; SCANET_SEQUENCE_COHERENT=1 makes the kernel hand its state over with device-coherent accesses even
+ * between workgroups of one XCD). */
 SN_API int sn_sync(sn_ctx* ctx);
 /* Name, HBM bytes and compute-unit count of the context's device
  * (reference: core/Devices.scala:23-37 lists TF devices). */
