@@ -130,6 +130,7 @@ def model_work(layers, in_shape, batch):
             labels[f"[{batch}x{G * H}x{H}]"] = 2.0 * batch * G * H * H       # the recurrent half alone (input half hoisted)
             labels[f"[{batch * T}x{G * H}x{F}]"] = 2.0 * batch * T * G * H * F
             labels[f"[{batch}x{H}x{G * H}]"] = dh
+            labels[f"[{batch * (T - 1)}x{H}x{G * H}]"] = (T - 1) * dh      # every backward product in one launch
             labels[f"[{batch}x{H}x{H}]"] = dh
             labels[f"[{F + H}x{G * H}x{T * batch}]"] = wg
             labels[f"[{F + H + 1}x{G * H}x{T * batch}]"] = wg

@@ -340,6 +340,14 @@ bool lstm_step_fused_ok(int F, int H, const float* x, const LstmWeights& w, int 
 // (Wr of the 4 gates), lstm_pack_elems(F, H) floats each at most; rebuilt once per pass over the sequence.
 int64_t lstm_pack_elems(int F, int H);
 int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pack_fwd, float* pack_dh, int gates = 4);
+// The simple cell's recurrences over all time steps in one launch (the LSTM sequence kernel's structure without gates).
+// Forward: r_slices holds T + 1 slices, slice t + 1 = r_t, slice 0 read only if first_valid.  Backward: dr_slices holds T
+// slices, slice T - 1 complete at launch, slice t - 1 = dr_t * Wr^T (+ dy_seq[:, t - 1, :] when given) for t = T-1 .. 1.
+bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const float* wpack);
+int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wpack, float* r_slices,
+                            int64_t slice);
+bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wpack);
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wpack, int64_t slice);
 // All T forward steps of an LSTM layer in one launch: the workgroups keep their weight slab in LDS and hand h_t to each
 // other through memory, one arrival counter per group of 32 batch rows.  h: T + 1 slices of `slice` floats, slice 0 the
 // initial hidden state (read only if h0_valid); gates / c: T slices.  lstm_sequence_fwd_ok says whether the launch fits

@@ -487,6 +487,122 @@ __global__ __launch_bounds__(256) void step_product_kernel(StepMulArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------- the simple cell's steps in one launch
+// The simple cell's two recurrences are one product per step with nothing around it:
+//   forward   r_t     = [x_t, r_{t-1}] * [Wk; Wr]                         (layer/RNN.scala:189-196), t = 0 .. T-1
+//   backward  dr_{t-1} = dr_t * Wr^T (+ the output gradient of step t-1 when the layer returns its sequence), t = T-1 .. 1
+// so one kernel runs either for all steps, built like lstm_sequence_fwd_kernel: a workgroup owns 32 batch rows x 32
+// units, keeps its weight slab in LDS, and the 32-unit groups of a row group hand the step's result to each other
+// through memory with the same arrival counter, placement check, bounded wait and two hand-over forms.  Every slice
+// is written once and read once per launch, so within an XCD plain loads find it in L2.
+struct SeqMulArgs {
+  const float* x;       // forward: [rows, T, F]; backward: null
+  float* rec;           // slices of `slice` floats; forward: slice t + 1 = r_t (slice 0 read only if first_valid),
+                        // backward: slice t = dr_t, slice T - 1 complete at launch
+  const float* dy_seq;  // backward, returned sequence: [rows, T, H] added to slice t - 1 as it is written; or null
+  const float* wpack;   // [unit block of 16][K16 / 4][16 units][4 k]
+  int64_t slice;
+  int first_valid;
+  int rows, T, F, H;    // backward: F = 0
+  int row_groups, unit_groups;
+  unsigned* sync;
+  unsigned spin_limit;
+  int* gave_up;
+  int force_coherent;
+};
+
+template <bool BACKWARD>
+__global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
+  constexpr int CBT = 32, NCB = CBT / 16, NRB = NCB / 2;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ int stop;
+  const int K = a.F + a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
+  float* As = lds;            // [RB][KP]
+  float* Bs = lds + RB * KP;  // [NCB][kq][16 units][4], kept for the whole sequence
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slot = blockIdx.x >> 3;
+  const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
+  if (rg >= a.row_groups) return;
+  const int r0 = rg * RB, u0 = ug * CBT;
+  unsigned* my_count = a.sync + rg;
+  unsigned* my_xcd = a.sync + a.row_groups + rg;
+  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
+  unsigned* abort_word = a.sync + 3 * a.row_groups;
+
+  if (tid == 0) {  // arrival round 0: do the members of this row group share an XCD?
+    const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
+    unsigned seen = 0u;
+    __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((seen != 0u && seen != mine) || a.force_coherent) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+    __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  {  // the slab of this group's two unit blocks: contiguous in the pack, already in LDS cell order
+    const f4v* slab = reinterpret_cast<const f4v*>(a.wpack) + (int64_t)(u0 >> 4) * kq * 16;
+    const int blocks = min(NCB, (a.H - u0 + 15) >> 4);
+    for (int e = tid; e < NCB * kq * 16; e += 256) reinterpret_cast<f4v*>(Bs)[e] = e < blocks * kq * 16 ? slab[e] : f4v{0.f, 0.f, 0.f, 0.f};
+  }
+  const int cb = wave % NCB, rb0 = (wave / NCB) * NRB;
+  constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
+  const int arow = tid >> 3;
+  const int steps = BACKWARD ? a.T - 1 : a.T;
+  bool spread = true;  // until round 0 is complete (the first wait below)
+  for (int s = 0; s < steps; ++s) {
+    const int t = BACKWARD ? a.T - 1 - s : s;  // the step whose operand slice is read
+    if (s > 0) {  // the slice is complete once every unit group of this row group has arrived s + 1 times (round 0 included)
+      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+      if (s == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    }
+    {
+      f4v va[NA];
+      const float* rp = a.rec + (int64_t)t * a.slice;
+      const bool with_rec = BACKWARD || s > 0 || a.first_valid;
+      const bool coherent = spread && s > 0;  // the first slice was written before this launch
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int q = i * 8 + (tid & 7), k = q * 4;
+        va[i] = f4v{0.f, 0.f, 0.f, 0.f};
+        if (q < kq && r0 + arow < a.rows && k < K) {
+          if (k < a.F) va[i] = *(const f4v*)(a.x + ((int64_t)(r0 + arow) * a.T + t) * a.F + k);
+          else if (!with_rec) continue;
+          else if (coherent) va[i] = load_coherent(rp + (int64_t)(r0 + arow) * a.H + (k - a.F));
+          else va[i] = *(const f4v*)(rp + (int64_t)(r0 + arow) * a.H + (k - a.F));
+        }
+      }
+      if (coherent) wait_coherent_loads(va);
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int q = i * 8 + (tid & 7);
+        if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
+      }
+    }
+    __syncthreads();
+    f4v acc[NRB];
+#pragma unroll
+    for (int r = 0; r < NRB; ++r) acc[r] = f4v{0.f, 0.f, 0.f, 0.f};
+    multiply_blocks<NRB>(As, Bs, K16, cb, rb0, lane, acc);
+    const int col = u0 + cb * 16 + (lane & 15), g = lane >> 4;
+    const int to = BACKWARD ? t - 1 : t + 1;
+    if (col < a.H) {
+      float* out = a.rec + (int64_t)to * a.slice;
+#pragma unroll
+      for (int r = 0; r < NRB; ++r)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int row = r0 + (rb0 + r) * 16 + 4 * g + v;
+          if (row >= a.rows) continue;
+          float val = acc[r][v];
+          if (BACKWARD && a.dy_seq) val = val + a.dy_seq[((int64_t)row * a.T + to) * a.H + col];
+          if (spread) __hip_atomic_store(out + (int64_t)row * a.H + col, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else out[(int64_t)row * a.H + col] = val;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0): the stores are acknowledged
+    __syncthreads();  // (also: As is free again)
+    if (tid == 0 && s + 1 < steps) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // ---------------------------------------------------------------------------- backward step, fused
 // One launch per reverse time step: the gate gradients of step t (element-wise) and the product that carries the
 // hidden gradient back, dh_{t-1} = sum over gates of dz_gate * Wr_gate^T.  A workgroup owns BR batch rows x BU hidden
@@ -805,6 +921,66 @@ int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const 
   StepMulArgs a{x + (int64_t)t * F, (int64_t)T * F, F, r_prev, H, H, 0, wpack, round16(F + H) / 4, 0, out, H, 0, rows, H};
   LaunchScope scope(ctx, "rnn_step_forward", rows, H, r_prev ? F + H : F);
   return launch_step_product(ctx, a, 1);
+}
+
+namespace {
+size_t rnn_sequence_lds_bytes(int K) {
+  const int K16 = round16(K);
+  return ((size_t)RB * (K16 + 4) + (size_t)32 * K16) * sizeof(float);
+}
+template <bool BACKWARD>
+bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
+  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * ceil_div(H, 32);
+  if (3 * groups + 1 > SEQ_COUNTERS) return false;
+  if (allow_dynamic_lds(ctx, (const void*)rnn_sequence_kernel<BACKWARD>, rnn_sequence_lds_bytes(MAX_K)) != SN_OK) return false;
+  int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rnn_sequence_kernel<BACKWARD>, 256, rnn_sequence_lds_bytes(K)) != hipSuccess) return false;
+  return blocks <= (int64_t)per_cu * ctx->compute_units;
+}
+template <bool BACKWARD>
+int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
+  SN_TRY(seq_sync_init(ctx));
+  a.row_groups = (int)ceil_div(a.rows, RB);
+  a.unit_groups = (int)ceil_div(a.H, 32);
+  a.sync = ctx->seq_arrived;
+  a.spin_limit = ctx->seq_spin_limit;
+  a.gave_up = ctx->seq_gave_up_dev;
+  a.force_coherent = ctx->seq_force_coherent;
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * a.row_groups + 1));  // all-zero bits
+  const int steps = BACKWARD ? a.T - 1 : a.T;
+  LaunchScope scope(ctx, name, a.rows * steps, a.H, K);  // `steps` products of rows x H x K
+  hipLaunchKernelGGL(rnn_sequence_kernel<BACKWARD>, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256),
+                     rnn_sequence_lds_bytes(K), ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+}  // namespace
+
+bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const float* wpack) {
+  return rows > 0 && F % 4 == 0 && H % 16 == 0 && F + H <= MAX_K && aligned16(x) && aligned16(wpack) && rnn_sequence_fits<false>(ctx, rows, F + H, H);
+}
+
+int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wpack, float* r_slices,
+                            int64_t slice) {
+  if (rows <= 0 || T <= 0) return SN_OK;
+  SN_REQUIRE(rnn_sequence_fwd_ok(ctx, rows, F, H, x, wpack), "rnn_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SeqMulArgs a{};
+  a.x = x; a.rec = r_slices; a.wpack = wpack; a.slice = slice; a.first_valid = first_valid;
+  a.rows = rows; a.T = T; a.F = F; a.H = H;
+  return launch_rnn_sequence<false>(ctx, a, "rnn_sequence_forward", F + H);
+}
+
+bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wpack) {
+  return rows > 0 && H % 16 == 0 && H <= MAX_K && aligned16(wpack) && rnn_sequence_fits<true>(ctx, rows, H, H);
+}
+
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wpack, int64_t slice) {
+  if (rows <= 0 || T <= 1) return SN_OK;
+  SN_REQUIRE(rnn_sequence_bwd_ok(ctx, rows, H, wpack), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
+  SeqMulArgs a{};
+  a.rec = dr_slices; a.dy_seq = dy_seq; a.wpack = wpack; a.slice = slice;
+  a.rows = rows; a.T = T; a.F = 0; a.H = H;
+  return launch_rnn_sequence<true>(ctx, a, "rnn_sequence_backward", H);
 }
 
 }  // namespace sn

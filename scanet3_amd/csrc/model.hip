@@ -642,7 +642,10 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         if (carried)
           SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[0]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
                                 ctx->stream));
-        for (int t = 0; t < op.T; ++t) {
+        const bool whole = fused && op.T > 1 && rnn_sequence_fwd_ok(ctx, rows, op.F, op.H, in, r->lstm_pk_fwd[i]);
+        if (whole)  // every step in one launch
+          SN_TRY(launch_rnn_sequence_fwd(ctx, in, op.T, op.F, carried ? 1 : 0, rows, op.H, r->lstm_pk_fwd[i], r->lstm_h[i], bh));
+        for (int t = whole ? op.T : 0; t < op.T; ++t) {
           const float* r_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
           float* r_t = r->lstm_h[i] + (int64_t)(t + 1) * bh;
           if (fused) SN_TRY(launch_rnn_step_fwd(ctx, in, t, op.T, op.F, r_prev, rows, op.H, r->lstm_pk_fwd[i], r_t));
@@ -897,7 +900,16 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         }
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
         if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));
-        for (int t = op.T - 1; t >= 0; --t) {
+        const bool whole = fused && op.T > 1 && rnn_sequence_bwd_ok(ctx, rows, op.H, r->lstm_pk_dh[i]);
+        if (whole) {  // every step in one launch (it adds a returned sequence's output gradients itself), then the input gradients
+          dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
+          if (op.ret_seq) SN_TRY(launch_step_slice_add(ctx, dr, dy + (int64_t)(op.T - 1) * op.H, (int64_t)op.T * op.H, rows, op.H, false));
+          SN_TRY(launch_rnn_sequence_bwd(ctx, r->lstm_dz[i], op.ret_seq ? dy : nullptr, op.T, rows, op.H, r->lstm_pk_dh[i], bh));
+          if (need_dx)
+            for (int t = op.T - 1; t >= 0; --t)
+              SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
+        }
+        for (int t = whole ? -1 : op.T - 1; t >= 0; --t) {
           dr = r->lstm_dz[i] + (int64_t)t * bh;
           if (op.ret_seq) SN_TRY(launch_step_slice_add(ctx, dr, dy + (int64_t)t * op.H, (int64_t)op.T * op.H, rows, op.H, t < op.T - 1));
           if (need_dx) SN_TRY(launch_lstm_dx(ctx, dr, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));

@@ -1014,6 +1014,45 @@ def test_stateful_rnn_steps_match_oracle(S, ctx, kind, units, features, batch):
 
 
 @pytest.mark.parametrize("coherent", ["0", "1"])
+@pytest.mark.parametrize("units", [64, 48])
+def test_simple_rnn_sequence_kernels_hand_over_within_and_across_xcds(S, monkeypatch, coherent, units):
+    """The simple cell's one-launch forward and backward in both hand-over forms (see the LSTM test below): a returned
+    sequence feeding a second recurrent layer (so the backward launch adds the output gradients of every step and the input
+    gradients follow from its slices), a carried state, several row groups with a partial last one, and a unit count that
+    leaves the last 32-unit group half empty."""
+    monkeypatch.setenv("SCANET_SEQUENCE_COHERENT", coherent)
+    c = S.Context(0)
+    try:
+        T, features, batch = 9, 12, 150
+        om = O.Model([O.SimpleRNN(units, O.ACT_TANH, stateful=True, return_sequence=True), O.SimpleRNN(32, O.ACT_SIGMOID),
+                      O.Dense(2, O.ACT_IDENTITY)], O.LOSS_MSE)
+        layers = S.SimpleRNN(units, S.Tanh, stateful=True, returnSequence=True) >> S.SimpleRNN(32, S.Sigmoid) >> S.Dense(2, S.Identity)
+        cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+        rep = cm.replica(None)
+        rng = np.random.default_rng(78)
+        params = glorot_params(om, (batch, T, features), rng)
+        for p in params:
+            if O.is_unaggregated_path(p):
+                params[p] = rng.uniform(-0.5, 0.5, params[p].shape).astype(f32)
+        x = rng.standard_normal((batch, T, features)).astype(f32)
+        y = rng.uniform(-1, 1, (batch, 2)).astype(f32)
+        rep.set_params(params)
+        xb, yb = c.to_device(x), c.to_device(y)
+        assert rel_err(rep.forward(xb), om.forward(x, params)) <= TOL_GEMM
+        oloss, ograds = om.grad(x, y, params)
+        assert abs(rep.grad(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+        ggrads = rep.get_grads()
+        for p in ograds:
+            assert rel_err(ggrads[p], ograds[p]) <= TOL_GEMM, p
+        for o in (rep, cm):
+            o.close()
+        xb.free()
+        yb.free()
+    finally:
+        c.close()
+
+
+@pytest.mark.parametrize("coherent", ["0", "1"])
 def test_lstm_sequence_kernel_hands_over_within_and_across_xcds(S, monkeypatch, coherent):
     """The one-launch LSTM forward picks per row group how h_t travels between workgroups: plain accesses when the row group
     sits on one XCD, device-coherent ones otherwise.  SCANET_SEQUENCE_COHERENT=1 (read when a context first launches the
