@@ -309,8 +309,15 @@ MEASURED_TRAFFIC = {
     "gemm_bf16_256[8192x4096x4096]": (539.0e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256[4096x4096x8192]": (495.3e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256_handover[8192x4096x4096]": (469.5e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
-    "lstm_sequence_forward[32768x1024x288]": (248.9e6, "lstm_kernels.hip", "47f1d2fd485afeb9f2ee37fc61587908b2151a7e"),
-    "lstm_step_backward[512x256x1024]": (15.75e6, "lstm_kernels.hip", "47f1d2fd485afeb9f2ee37fc61587908b2151a7e"),
+    "lstm_sequence_forward[32768x1024x288]": (248.9e6, "lstm_kernels.hip", "02cf5722ef270bfd13cbeaf004f2898aaad9fc8f"),
+    "lstm_step_backward[512x256x1024]": (15.75e6, "lstm_kernels.hip", "02cf5722ef270bfd13cbeaf004f2898aaad9fc8f"),
+    "rnn_sequence_forward[32768x256x288]": (73.6e6, "lstm_kernels.hip", "02cf5722ef270bfd13cbeaf004f2898aaad9fc8f"),
+    "rnn_sequence_backward[32256x256x256]": (68.6e6, "lstm_kernels.hip", "02cf5722ef270bfd13cbeaf004f2898aaad9fc8f"),
+    "conv2d_forward[121000x64x288]": (53.32e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
+    "conv2d_input_gradient[169000x32x576]": (53.72e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
+    "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "78b4b4210fc4231c76bc9149edbb1284b66dabc5"),
+    "mlp2_rows_forward_backward[1000x50x784]": (5.41e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
+    "mlp2_weight_gradients[784x50x1000]": (8.69e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
     "lstm_weight_gradient[289x1024x32768]": (323.0e6, "gemm_kernels.hip", "78b4b4210fc4231c76bc9149edbb1284b66dabc5"),
     "adam": (2.800e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
     "average": (0.900e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
