@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
 //                    (write-through), read with loads that carry the same coherence bit (sc1).  14.3 us per step.
 // Workgroup ids are mapped to (row group, unit group) so that a row group's workgroups have ids congruent mod 8, which
 // the dispatcher places on one XCD.  That is not taken on trust: each workgroup reads the XCD it runs on from the
-// hardware register, the members of a row group compare theirs in a first arrival round before any hand-over, and one
+// hardware register, the members of a row group compare theirs in a first arrival before any hand-over, and one
 // mismatch switches the whole row group to the second form.  The counter itself is only touched with device-scope atomics.
 __device__ __forceinline__ f4v load_coherent(const float* p) {
   f4v v;
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
   unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
   unsigned* abort_word = a.sync + 3 * a.row_groups;
 
-  // ---- arrival round 0: do the members of this row group share an XCD?
+  // ---- arrival 0 (the placement check): do the members of this row group share an XCD?
   if (tid == 0) {
     const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
     unsigned seen = 0u;
@@ -320,10 +320,10 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
 
   constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
   const int arow = tid >> 3;
-  bool spread = true;  // until round 0 is complete (the first wait below), write as if the row group were spread out
+  bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
   for (int t = 0; t < a.T; ++t) {
     const bool with_h = t > 0 || a.h0_valid;
-    if (t > 0) {  // h_{t-1} is complete once every unit group of this row group has arrived t + 1 times (round 0 included)
+    if (t > 0) {  // h_{t-1} is complete once every unit group of this row group has arrived t + 1 times (arrival 0 included)
       if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(t + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
       if (t == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
@@ -529,7 +529,7 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
   unsigned* abort_word = a.sync + 3 * a.row_groups;
 
-  if (tid == 0) {  // arrival round 0: do the members of this row group share an XCD?
+  if (tid == 0) {  // arrival 0 (the placement check): do the members of this row group share an XCD?
     const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
     unsigned seen = 0u;
     __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -546,10 +546,10 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
   const int arow = tid >> 3;
   const int steps = BACKWARD ? a.T - 1 : a.T;
-  bool spread = true;  // until round 0 is complete (the first wait below)
+  bool spread = true;  // until arrival 0 is complete (the first wait below)
   for (int s = 0; s < steps; ++s) {
     const int t = BACKWARD ? a.T - 1 - s : s;  // the step whose operand slice is read
-    if (s > 0) {  // the slice is complete once every unit group of this row group has arrived s + 1 times (round 0 included)
+    if (s > 0) {  // the slice is complete once every unit group of this row group has arrived s + 1 times (arrival 0 included)
       if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
       if (s == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
