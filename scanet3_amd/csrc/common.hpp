@@ -355,6 +355,12 @@ int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, 
 bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w);
 int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
                              const float* wpack, float* gates, float* c, float* h, int64_t slice);
+// All reverse steps in one launch (H a power of two from 16 to 256): dz (T slices of 4 * slice floats) from the saved gates
+// and cell states, the gradient of the last hidden state (dh_last, may be null) and of a returned sequence (dy_seq
+// [rows, T, H], may be null).  wpack: launch_lstm_pack's pack_dh.  lstm_sequence_bwd_ok: as for the forward launch.
+bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w);
+int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
+                             int rows, int H, const LstmWeights& w, const float* wpack, float* dz, int64_t slice);
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h);
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev

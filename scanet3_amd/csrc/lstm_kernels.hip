@@ -768,6 +768,181 @@ __global__ __launch_bounds__(256) void lstm_step_bwd_kernel(StepBwdArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------- all backward steps in one launch
+// The reverse recurrence, built like lstm_sequence_fwd_kernel: a workgroup owns 32 batch rows x 16 hidden units for the
+// whole sequence, keeps dc of its cells in registers and the recurrent weights of its units (all 4H k-values) in LDS.
+// What the unit groups of a row group hand to each other is dz_t itself, which has to be written anyway (the
+// weight-gradient GEMM reads it): a workgroup turns dh_t, dc and the saved gates of its cells into its 64 columns of
+// dz_t, counts itself in, waits for the others, reads the 32 complete rows of dz_t and multiplies them by its weight
+// slab, which is dh_{t-1} of its own cells and never leaves the workgroup.  Every dz slice is written once and read
+// once per launch, so the two hand-over forms of the forward kernel apply unchanged (plain accesses within an XCD,
+// device-coherent ones otherwise), and so do the placement check and the bounded wait.
+//   do = dh * tanh(c);  dc += (1 - tanh(c)^2) * (dh * o)
+//   df = dc * c_prev;   di = dc * g;   dg = dc * i;   dc_prev = dc * f
+//   dz_gate = act'(z_gate) * d_gate;   dh_{t-1}[r, u] = sum_{gate, n} dz_t[r, gate H + n] * Wr_gate[u][n]
+// The rows of dz_t go straight from memory into the MFMA operand registers (lane (row, g) of a 16-row block holds
+// k = 16 kb + 4 g .. + 3): wavefront w multiplies row block w % 2 over half w / 2 of the 4H k-values, the two halves
+// meet in LDS and are added in a fixed order.
+struct SeqBwdArgs {
+  const float* gates;    // T slices of 4 * slice floats: activated forget, input, gate, output of [rows, 4H]
+  const float* c;        // T slices
+  const float* c0;       // [rows, H] or null: zeros
+  const float* dh_last;  // [rows, H] gradient of h_{T-1}, or null
+  const float* dy_seq;   // [rows, T, H] gradient of a returned sequence (every step adds its own slice), or null
+  const float* wpack;    // pack_dh_kernel's order
+  float* dz;             // T slices of 4 * slice floats
+  int64_t slice;
+  int rows, T, H;
+  int row_groups, unit_groups;
+  unsigned* sync;        // zero at launch, as in SeqFwdArgs
+  unsigned spin_limit;
+  int* gave_up;
+  int force_coherent;
+};
+
+template <int NKB>  // 16-long k blocks per wavefront: H = 8 NKB
+__global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
+  constexpr int UB = 16, H = 8 * NKB, HQ = H / 4;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  __shared__ int stop;
+  f4v* Bs = reinterpret_cast<f4v*>(lds);  // [4H / 4][16 units]: 4 consecutive k each, kept for the whole sequence
+  float* Ps = lds + 4 * H * UB;           // [2 halves of k][RB][ZP] partial dh
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slot = blockIdx.x >> 3;
+  const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
+  if (rg >= a.row_groups) return;
+  const int r0 = rg * RB, u0 = ug * UB;
+  unsigned* my_count = a.sync + rg;
+  unsigned* my_xcd = a.sync + a.row_groups + rg;
+  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
+  unsigned* abort_word = a.sync + 3 * a.row_groups;
+
+  if (tid == 0) {  // arrival 0 (the placement check): do the members of this row group share an XCD?
+    const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
+    unsigned seen = 0u;
+    __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((seen != 0u && seen != mine) || a.force_coherent) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
+    __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  {  // this unit group's block of every gate: [gate][unit block][n / 4][16 units] in the pack -> [gate H / 4 + n / 4][16 units]
+    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
+    for (int e = tid; e < 4 * HQ * UB; e += 256) {
+      const int gate = e / (HQ * UB), rem = e % (HQ * UB);
+      Bs[e] = pack[((int64_t)(gate * a.unit_groups + ug) * HQ) * UB + rem];
+    }
+  }
+  // the two cells this thread owns: row e / 16, unit e % 16 for e = tid, tid + 256
+  bool live[2];
+  int64_t ci[2], zi[2], yi[2];
+  float f[2], in[2], gg[2], o[2], cc[2], cp[2], dyv[2], dh[2], dcv[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int e = tid + 256 * j, row = e / UB, u = e % UB;
+    live[j] = r0 + row < a.rows;
+    const int64_t r = live[j] ? r0 + row : 0;
+    ci[j] = r * H + u0 + u;
+    zi[j] = r * 4 * H + u0 + u;
+    yi[j] = r * a.T * H + u0 + u;
+    const int t = a.T - 1;
+    const float* gt = a.gates + (int64_t)t * 4 * a.slice + zi[j];
+    f[j] = gt[0];
+    in[j] = gt[H];
+    gg[j] = gt[2 * H];
+    o[j] = gt[3 * H];
+    cc[j] = a.c[(int64_t)t * a.slice + ci[j]];
+    cp[j] = t > 0 ? a.c[(int64_t)(t - 1) * a.slice + ci[j]] : (a.c0 ? a.c0[ci[j]] : 0.f);
+    dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)t * H] : 0.f;
+    dh[j] = a.dh_last ? a.dh_last[ci[j]] : 0.f;
+    dcv[j] = 0.f;
+  }
+  const int rb = wave & 1, kh = wave >> 1, row16 = lane & 15, g = lane >> 4;
+  // rows past the batch multiply the last row again: their results belong to no cell
+  const int64_t a_off = (int64_t)min(r0 + rb * 16 + row16, a.rows - 1) * 4 * H + kh * 2 * H + 4 * g;
+  const f4v* bp = Bs + (kh * (H / 2) + g) * UB + row16;
+  bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
+  for (int t = a.T - 1;; --t) {
+    // ---- gate gradients of step t
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (!live[j]) continue;
+      const float tc = tanhf(cc[j]);
+      float d = dh[j];
+      if (a.dy_seq) d = d + dyv[j];
+      const float d_o = d * tc;
+      const float dc = dcv[j] + (1.0f - tc * tc) * (d * o[j]);
+      const float df = dc * cp[j], di = dc * gg[j], dg = dc * in[j];
+      const float dzf = (f[j] * (1.0f - f[j])) * df;
+      const float dzi = (in[j] * (1.0f - in[j])) * di;
+      const float dzg = (1.0f - gg[j] * gg[j]) * dg;
+      const float dzo = (o[j] * (1.0f - o[j])) * d_o;
+      dcv[j] = dc * f[j];
+      float* zt = a.dz + (int64_t)t * 4 * a.slice + zi[j];
+      if (spread) {
+        __hip_atomic_store(zt, dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(zt + H, dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(zt + 2 * H, dzg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(zt + 3 * H, dzo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        zt[0] = dzf;
+        zt[H] = dzi;
+        zt[2 * H] = dzg;
+        zt[3 * H] = dzo;
+      }
+    }
+    if (t == 0) break;
+    // ---- hand dz_t over: stores acknowledged in every wavefront, then one thread counts the workgroup in
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
+    __syncthreads();
+    if (tid == 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // ---- what step t - 1 needs from the forward pass is requested while the others arrive
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const float* gt = a.gates + (int64_t)(t - 1) * 4 * a.slice + zi[j];
+      f[j] = gt[0];
+      in[j] = gt[H];
+      gg[j] = gt[2 * H];
+      o[j] = gt[3 * H];
+      cc[j] = cp[j];
+      cp[j] = t > 1 ? a.c[(int64_t)(t - 2) * a.slice + ci[j]] : (a.c0 ? a.c0[ci[j]] : 0.f);
+      dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)(t - 1) * H] : 0.f;
+    }
+    const int done = a.T - 1 - t;  // hand-overs before this one
+    if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+    if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    // ---- dh_{t-1} of this workgroup's cells = dz_t (32 complete rows) * the weight slab
+    {
+      const float* ap = a.dz + (int64_t)t * 4 * a.slice + a_off;
+      f4v av[NKB];
+      if (spread) {
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) av[kb] = load_coherent(ap + 16 * kb);
+        wait_coherent_loads(av);
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) av[kb] = *(const f4v*)(ap + 16 * kb);
+      }
+      f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        const f4v bv = bp[kb * 4 * UB];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kb][v], bv[v], acc[kb & 1], 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) Ps[(kh * RB + rb * 16 + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = tid + 256 * j, row = e / UB, u = e % UB;
+      dh[j] = Ps[row * ZP + u] + Ps[(RB + row) * ZP + u];
+    }
+  }
+}
+
+size_t sequence_bwd_lds_bytes(int H) { return ((size_t)4 * H * 16 + 2 * RB * ZP) * sizeof(float); }
+
 size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 or 32)
   const int K16 = round16(K);
   const size_t slabs = (size_t)RB * (K16 + 4) + (size_t)cols * K16, exchange = 4 * RB * ZP;
@@ -909,6 +1084,55 @@ int launch_lstm_step_bwd(sn_ctx* ctx, const LstmGateBwdArgs& g, const float* dc_
   LaunchScope scope(ctx, "lstm_step_backward", rows, H, 4 * H);
   SN_TRY(allow_dynamic_lds(ctx, (const void*)lstm_step_bwd_kernel, ((size_t)BR * BKP + (size_t)BN_MAX * BK4) * sizeof(float)));
   hipLaunchKernelGGL(lstm_step_bwd_kernel, dim3((unsigned)(H / BU), (unsigned)ceil_div(rows, BR), (unsigned)chunks), dim3(256), smem, ctx->stream, a);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+namespace {
+// calls f(kernel, H / 8) for the instantiation that handles H, or returns false
+template <typename F>
+bool with_sequence_bwd_kernel(int H, F&& f) {
+  switch (H) {
+    case 16: f(lstm_sequence_bwd_kernel<2>); return true;
+    case 32: f(lstm_sequence_bwd_kernel<4>); return true;
+    case 64: f(lstm_sequence_bwd_kernel<8>); return true;
+    case 128: f(lstm_sequence_bwd_kernel<16>); return true;
+    case 256: f(lstm_sequence_bwd_kernel<32>); return true;
+    default: return false;
+  }
+}
+}  // namespace
+
+bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
+  if (rows <= 0) return false;
+  for (int g = 0; g < 4; ++g)
+    if (!aligned16(w.wr[g])) return false;
+  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+  if (3 * groups + 1 > SEQ_COUNTERS) return false;
+  bool fits = false;
+  const bool known = with_sequence_bwd_kernel(H, [&](auto kernel) {
+    if (allow_dynamic_lds(ctx, (const void*)kernel, sequence_bwd_lds_bytes(H)) != SN_OK) return;
+    int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, sequence_bwd_lds_bytes(H)) != hipSuccess) return;
+    fits = blocks <= (int64_t)per_cu * ctx->compute_units;
+  });
+  return known && fits;
+}
+
+int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
+                             int rows, int H, const LstmWeights& w, const float* wpack, float* dz, int64_t slice) {
+  if (rows <= 0 || T <= 0) return SN_OK;
+  SN_REQUIRE(lstm_sequence_bwd_ok(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
+  SN_REQUIRE(aligned16(wpack) && aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
+  SN_TRY(seq_sync_init(ctx));
+  const int groups = (int)ceil_div(rows, RB);
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * groups + 1));  // all-zero bits
+  SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, wpack, dz, slice, rows, T, H, groups, H / 16,
+               ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+  LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
+  with_sequence_bwd_kernel(H, [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_bwd_lds_bytes(H), ctx->stream, a);
+  });
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

@@ -825,11 +825,20 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
         // one launch per step (gate gradients + the product that carries dh back) where the layer's shape allows it
         const bool fused_bwd = fused && lstm_step_bwd_fused_ok(op.H, w);
-        if (fused_bwd && op.T > 1) SN_TRY(launch_lstm_pack_bwd(ctx, w, op.H, r->lstm_pk_dh[i]));
+        // every reverse step in one launch where the whole grid fits the device; the input gradients follow per step
+        const bool whole = fused && op.T > 1 && lstm_sequence_bwd_ok(ctx, rows, op.H, w);
+        if (whole) {
+          SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
+          SN_TRY(launch_lstm_sequence_bwd(ctx, r->lstm_gates[i], r->lstm_c[i], param_ptr(r, r->w, op.state_p[0]), op.ret_seq ? nullptr : dy,
+                                          op.ret_seq ? dy : nullptr, op.T, rows, op.H, w, r->lstm_pk_dh[i], r->lstm_dz[i], bh));
+          if (need_dx)
+            for (int t = op.T - 1; t >= 0; --t)
+              SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh * 4, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
+        } else if (fused_bwd && op.T > 1) SN_TRY(launch_lstm_pack_bwd(ctx, w, op.H, r->lstm_pk_dh[i]));
         else if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
         float* dcbuf[2] = {r->lstm_dc, r->lstm_dc2};
         int db = 0;
-        for (int t = op.T - 1; t >= 0; --t) {
+        for (int t = whole ? -1 : op.T - 1; t >= 0; --t) {
           LstmGateBwdArgs a{r->lstm_gates[i] + (int64_t)t * bh * 4, r->lstm_c[i] + (int64_t)t * bh,
                             t == 0 ? param_ptr(r, r->w, op.state_p[0]) : r->lstm_c[i] + (int64_t)(t - 1) * bh, dh, r->lstm_dc,
                             r->lstm_dz[i] + (int64_t)t * bh * 4, t == op.T - 1 ? 1 : 0, dh_parts, bh};

@@ -1054,10 +1054,10 @@ def test_simple_rnn_sequence_kernels_hand_over_within_and_across_xcds(S, monkeyp
 
 @pytest.mark.parametrize("coherent", ["0", "1"])
 def test_lstm_sequence_kernel_hands_over_within_and_across_xcds(S, monkeypatch, coherent):
-    """The one-launch LSTM forward picks per row group how h_t travels between workgroups: plain accesses when the row group
-    sits on one XCD, device-coherent ones otherwise.  SCANET_SEQUENCE_COHERENT=1 (read when a context first launches the
-    kernel) forces the second form everywhere; both must give the oracle's numbers, here with several row groups, a partial
-    last one, 4 unit groups and a carried state."""
+    """The one-launch LSTM forward and backward pick per row group how h_t (backward: dz_t) travels between workgroups: plain
+    accesses when the row group sits on one XCD, device-coherent ones otherwise.  SCANET_SEQUENCE_COHERENT=1 (read when a
+    context first launches the kernel) forces the second form everywhere; both must give the oracle's numbers, here with
+    several row groups, a partial last one, 4 unit groups and a carried state."""
     monkeypatch.setenv("SCANET_SEQUENCE_COHERENT", coherent)
     c = S.Context(0)
     try:
