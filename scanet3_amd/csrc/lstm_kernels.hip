@@ -650,6 +650,7 @@ __global__ __launch_bounds__(256) void pack_bwd_kernel(LstmWeights w, int H, flo
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
 __global__ __launch_bounds__(256) void lstm_step_bwd_kernel(StepBwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -800,14 +801,14 @@ struct SeqBwdArgs {
   int force_coherent;
 };
 
-template <int NKB>  // 16-long k blocks per wavefront: H = 8 NKB
+template <int NKB, int KO = 0>  // 16-long k blocks per wavefront: H = 8 NKB
 __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   constexpr int UB = 16, H = 8 * NKB, HQ = H / 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
-  f4v* Bs = reinterpret_cast<f4v*>(lds);  // [4H / 4][16 units]: 4 consecutive k each, kept for the whole sequence
-  float* Ps = lds + 4 * H * UB;           // [2 halves of k][RB][ZP] partial dh
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* Ps = lds;                  // [2 halves of k][RB][ZP] partial dh
+  float* As = lds + 2 * RB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]: dz_t as the loads deliver it
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;
@@ -821,15 +822,20 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
     unsigned seen = 0u;
     __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((seen != 0u && seen != mine) || a.force_coherent) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((seen != 0u && seen != mine) || (a.force_coherent == 1)) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
     __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  {  // this unit group's block of every gate: [gate][unit block][n / 4][16 units] in the pack -> [gate H / 4 + n / 4][16 units]
+  const int rb = wave & 1, kh = wave >> 1, row16 = lane & 15, g = lane >> 4;
+  // This wavefront's half of the unit group's weights stays in registers in MFMA operand order: lane (unit, g) holds
+  // k = kh 2H + 16 kb + 4 g .. + 3 of block kb.  The pack is [gate][unit block][n / 4][16 units][4 n].
+  f4v bw[NKB];
+  {
     const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
-    for (int e = tid; e < 4 * HQ * UB; e += 256) {
-      const int gate = e / (HQ * UB), rem = e % (HQ * UB);
-      Bs[e] = pack[((int64_t)(gate * a.unit_groups + ug) * HQ) * UB + rem];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      const int kq = kh * (H / 2) + 4 * kb + g, gate = kq / HQ, q = kq % HQ;
+      bw[kb] = pack[((int64_t)(gate * a.unit_groups + ug) * HQ + q) * UB + row16];
     }
   }
   // the two cells this thread owns: row e / 16, unit e % 16 for e = tid, tid + 256
@@ -856,11 +862,16 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     dh[j] = a.dh_last ? a.dh_last[ci[j]] : 0.f;
     dcv[j] = 0.f;
   }
-  const int rb = wave & 1, kh = wave >> 1, row16 = lane & 15, g = lane >> 4;
-  // rows past the batch multiply the last row again: their results belong to no cell
-  const int64_t a_off = (int64_t)min(r0 + rb * 16 + row16, a.rows - 1) * 4 * H + kh * 2 * H + 4 * g;
-  const f4v* bp = Bs + (kh * (H / 2) + g) * UB + row16;
-  bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
+  // One load instruction brings a 16-row x 16-k block of dz_t to 1 KiB of LDS, lane p to bytes 16 p .. 16 p + 15: four
+  // neighbouring lanes fetch the 64 contiguous bytes of one row (rows past the batch: the last row again, their results
+  // belong to no cell), and chunk c of row r lands in slot c ^ (r / 4) of the row so that the 16 lanes that later read
+  // one chunk index of 16 rows hit 16 different bank groups.
+  const int64_t a_off = (int64_t)min(r0 + rb * 16 + (lane >> 2), a.rows - 1) * 4 * H + kh * 2 * H + 4 * ((lane & 3) ^ (lane >> 4));
+  float* aw = As + wave * NKB * 256;
+  const float* ar = aw + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
+  bool spread = true;
+  constexpr int ko = KO;
+  if (ko & 2) spread = false;
   for (int t = a.T - 1;; --t) {
     // ---- gate gradients of step t
 #pragma unroll
@@ -878,7 +889,8 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       const float dzo = (o[j] * (1.0f - o[j])) * d_o;
       dcv[j] = dc * f[j];
       float* zt = a.dz + (int64_t)t * 4 * a.slice + zi[j];
-      if (spread) {
+      if (ko & 32) { if (dzf == 123.f) zt[0] = dzi + dzg + dzo; }
+      else if (spread) {
         __hip_atomic_store(zt, dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(zt + H, dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(zt + 2 * H, dzg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -892,9 +904,11 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     }
     if (t == 0) break;
     // ---- hand dz_t over: stores acknowledged in every wavefront, then one thread counts the workgroup in
+    if (!(ko & 16)) {
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (tid == 0 && !(ko & 2)) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- what step t - 1 needs from the forward pass is requested while the others arrive
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -908,26 +922,32 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)(t - 1) * H] : 0.f;
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
+    if (!(ko & 2)) {
     if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, &stop)) return;
-    if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    }
+    if (done == 0 && !(ko & 2)) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     // ---- dh_{t-1} of this workgroup's cells = dz_t (32 complete rows) * the weight slab
     {
       const float* ap = a.dz + (int64_t)t * 4 * a.slice + a_off;
-      f4v av[NKB];
-      if (spread) {
+      if (!(ko & 4)) {
+        if (spread) {
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) av[kb] = load_coherent(ap + 16 * kb);
-        wait_coherent_loads(av);
-      } else {
+          for (int kb = 0; kb < NKB; ++kb)
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 16);  // sc1: coherent at device scope
+        } else {
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) av[kb] = *(const f4v*)(ap + 16 * kb);
+          for (int kb = 0; kb < NKB; ++kb) __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 0);
+        }
       }
+      // the blocks are this wavefront's own: its loads have landed, no barrier needed (the compiler does not order LDS reads
+      // behind these loads by itself)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        const f4v bv = bp[kb * 4 * UB];
+        const f4v av = *(const f4v*)(ar + kb * 256);
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[kb][v], bv[v], acc[kb & 1], 0, 0, 0);
+        for (int v = 0; v < 4; ++v) { if (ko & 8) acc[kb & 1][v] += av[v] * bw[kb][v]; else acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0); }
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) Ps[(kh * RB + rb * 16 + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
@@ -941,7 +961,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   }
 }
 
-size_t sequence_bwd_lds_bytes(int H) { return ((size_t)4 * H * 16 + 2 * RB * ZP) * sizeof(float); }
+size_t sequence_bwd_lds_bytes(int H) { return ((size_t)2 * RB * ZP + (size_t)RB * 4 * H) * sizeof(float); }
 
 size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 or 32)
   const int K16 = round16(K);
@@ -1097,7 +1117,21 @@ bool with_sequence_bwd_kernel(int H, F&& f) {
     case 32: f(lstm_sequence_bwd_kernel<4>); return true;
     case 64: f(lstm_sequence_bwd_kernel<8>); return true;
     case 128: f(lstm_sequence_bwd_kernel<16>); return true;
-    case 256: f(lstm_sequence_bwd_kernel<32>); return true;
+    case 256: {
+      const char* v = getenv("SN_KO");
+      switch (v ? atoi(v) : 0) {
+        case 2: f(lstm_sequence_bwd_kernel<32, 2>); break;
+        case 6: f(lstm_sequence_bwd_kernel<32, 6>); break;
+        case 10: f(lstm_sequence_bwd_kernel<32, 10>); break;
+        case 14: f(lstm_sequence_bwd_kernel<32, 14>); break;
+        case 18: f(lstm_sequence_bwd_kernel<32, 18>); break;
+        case 34: f(lstm_sequence_bwd_kernel<32, 34>); break;
+        case 50: f(lstm_sequence_bwd_kernel<32, 50>); break;
+        case 62: f(lstm_sequence_bwd_kernel<32, 62>); break;
+        default: f(lstm_sequence_bwd_kernel<32>); break;
+      }
+      return true;
+    }
     default: return false;
   }
 }
