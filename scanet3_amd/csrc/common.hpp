@@ -96,7 +96,10 @@ struct LaunchScope {
 int profile_drain(sn_ctx* ctx);
 // Sets up the context's sequence-kernel words on first use.
 int seq_sync_init(sn_ctx* ctx);
-constexpr int SEQ_COUNTERS = 1024;
+// Words of a context's sequence-kernel area: one block of SEQ_GROUP_WORDS per row group (arrival counter, XCD word,
+// spread flag; a block of its own so that the pollers of different row groups do not meet on one cache line), then the
+// abort word's block.
+constexpr int SEQ_GROUP_WORDS = 64, SEQ_MAX_GROUPS = 1023, SEQ_COUNTERS = (SEQ_MAX_GROUPS + 1) * SEQ_GROUP_WORDS;
 // After a stream synchronisation: SN_E_STATE (once) if a sequence kernel gave up waiting since the last check.
 int check_async(sn_ctx* ctx);
 // looks up this device's address of the library's static scratch array (model.hip); `device` must be current

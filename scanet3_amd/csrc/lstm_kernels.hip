@@ -242,7 +242,7 @@ struct SeqFwdArgs {
   int h0_valid;
   int rows, T, F, H;
   int row_groups, unit_groups;
-  unsigned* sync;        // zero at launch: [row groups] arrival counters, [row groups] XCD words, [row groups] spread flags, abort word
+  unsigned* sync;        // zero at launch: per row group a block of SEQ_GROUP_WORDS (arrival counter, XCD word, spread flag), then the abort word
   unsigned spin_limit;
   int* gave_up;          // host-visible
   int force_coherent;    // take the across-XCD form everywhere
@@ -254,7 +254,8 @@ __device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, u
     unsigned spins = 0;
     int bad = 0;
     while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      if (__hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u || ++spins > spin_limit) {
+      // (every workgroup of the launch watches the one abort word: a look every 16th round keeps them off each other)
+      if (++spins > spin_limit || ((spins & 15u) == 0u && __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
         bad = 1;
         break;
       }
@@ -270,24 +271,36 @@ __device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, u
   return *stop;
 }
 
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+__device__ __align__(16) const float seq_zero_chunk[4] = {0.f, 0.f, 0.f, 0.f};  // what the k padding and an absent h_{-1} read
+
+// Shape of the kernel: a workgroup owns 16 batch rows x 16 hidden units, so that two or more workgroups share a CU and one
+// of them multiplies while another waits for its hand-over.  Wavefront w owns gate w: its [K x 16] weights stay in
+// registers in MFMA operand order.  The 16 rows of [x_t, h_{t-1}] arrive through LDS-direct loads (one load = 16 rows x
+// 16 k = 1 KiB of LDS, lane p to bytes 16 p .. 16 p + 15: four neighbouring lanes fetch 64 contiguous bytes of a row, and
+// chunk c of row r lands in slot c ^ (r / 4) so that the reads of one chunk index over 16 rows hit 16 different bank
+// groups); the wavefronts share the blocks, each requests every fourth one.
+constexpr int SRB = 16;  // batch rows per workgroup of the one-launch kernels
+
+template <int NKB>  // 16-long blocks of k over [x_t, h_{t-1}], padded with zeros
 __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
-  constexpr int UB = 16, NCB = 4, NRB = 2;
+  constexpr int UB = 16;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
-  const int K = a.F + a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
-  float* As = lds;  // [RB][KP]
-  float* Zx = lds;  // [4 gates][RB][ZP] over As once every wavefront has finished multiplying
-  float* Bs = lds + (RB * KP > 4 * RB * ZP ? RB * KP : 4 * RB * ZP);  // [NCB][kq][16 columns][4], kept for the whole sequence
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* As = lds;              // [NKB][16 rows x 16 k]
+  float* Zx = lds + NKB * 256;  // [4 gates][16 rows][ZP]
+  const int K = a.F + a.H, kq = round16(K) / 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // id -> (row group, unit group): ids congruent mod 8 share an XCD, so XCD x takes the row groups x, x + 8, ...
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;  // the grid is rounded up to whole rounds of 8 row groups
-  const int r0 = rg * RB, u0 = ug * UB;
-  unsigned* my_count = a.sync + rg;
-  unsigned* my_xcd = a.sync + a.row_groups + rg;
-  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
-  unsigned* abort_word = a.sync + 3 * a.row_groups;
+  const int r0 = rg * SRB, u0 = ug * UB;
+  unsigned* my_count = a.sync + rg * SEQ_GROUP_WORDS;
+  unsigned* my_xcd = my_count + 1;
+  unsigned* my_spread = my_count + 2;
+  unsigned* abort_word = a.sync + a.row_groups * SEQ_GROUP_WORDS;
 
   // ---- arrival 0 (the placement check): do the members of this row group share an XCD?
   if (tid == 0) {
@@ -300,26 +313,31 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
     __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  {  // the slab of this unit group: 4 gates x kq quads x 16 units, already in LDS cell order
-    const f4v* slab = reinterpret_cast<const f4v*>(a.wpack) + (int64_t)ug * NCB * kq * 16;
-    for (int e = tid; e < NCB * kq * 16; e += 256) reinterpret_cast<f4v*>(Bs)[e] = slab[e];
-  }
-  // the two cells this thread finishes per step: row e / 16, unit e % 16 for e = tid, tid + 256
-  float c_reg[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int e = tid + 256 * j, row = e / UB, u = e % UB;
-    c_reg[j] = a.c0 && r0 + row < a.rows ? a.c0[(int64_t)(r0 + row) * a.H + u0 + u] : 0.f;
-  }
-  const int cb = wave % NCB, rb0 = (wave / NCB) * NRB;
-  float bias;
+  const int row16 = lane & 15, g = lane >> 4;
+  // weights of gate `wave`: lane (unit = row16, g) holds k = 16 kb + 4 g .. + 3 for every kb
+  f4v bw[NKB];
   {
-    const int col = cb * 16 + (lane & 15);
-    bias = a.bias[col / UB] ? a.bias[col / UB][u0 + col % UB] : 0.f;
+    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);  // [unit group][gate][kq][16 units]: 4 consecutive k each
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      const int q = 4 * kb + g;
+      bw[kb] = q < kq ? pack[((int64_t)(ug * 4 + wave) * kq + q) * UB + row16] : f4v{0.f, 0.f, 0.f, 0.f};
+    }
   }
+  // the cell this thread finishes per step: row tid / 16, unit tid % 16
+  const int crow = tid >> 4, cu = tid & 15;
+  const bool live = r0 + crow < a.rows;
+  const int64_t ci = (int64_t)(live ? r0 + crow : 0) * a.H + u0 + cu, zi = (int64_t)(live ? r0 + crow : 0) * 4 * a.H + u0 + cu;
+  float c_reg = a.c0 ? a.c0[ci] : 0.f;
+  float bias[4];
+#pragma unroll
+  for (int gate = 0; gate < 4; ++gate) bias[gate] = a.bias[gate] ? a.bias[gate][u0 + cu] : 0.f;
+  // operand loads: lane p fetches chunk (p % 4) ^ (p / 16) of row p / 4 (rows past the batch: the last row again)
+  const int chunk = (lane & 3) ^ (lane >> 4);
+  const int64_t arow = min(r0 + (lane >> 2), a.rows - 1);
+  const float* xrow = a.x + arow * a.T * a.F;
+  const float* ar = As + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
 
-  constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
-  const int arow = tid >> 3;
   bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
   for (int t = 0; t < a.T; ++t) {
     const bool with_h = t > 0 || a.h0_valid;
@@ -327,62 +345,46 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
       if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(t + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
       if (t == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
-    // ---- [x_t, h_{t-1}] of the 32 rows: every load is issued before the first LDS write
-    {
-      f4v va[NA];
-      const float* hp = a.h + (int64_t)t * a.slice;
-      const bool coherent = spread && t > 0;  // slice 0 was written before this launch
+    const float* xt = xrow + (int64_t)t * a.F;
+    const float* ht = a.h + (int64_t)t * a.slice + arow * a.H - a.F;  // indexed by k
+    const bool coherent = spread && t > 0;  // slice 0 was written before this launch
 #pragma unroll
-      for (int i = 0; i < NA; ++i) {
-        const int q = i * 8 + (tid & 7), k = q * 4;
-        va[i] = f4v{0.f, 0.f, 0.f, 0.f};
-        if (q < kq && r0 + arow < a.rows && k < K) {
-          if (k < a.F) va[i] = *(const f4v*)(a.x + ((int64_t)(r0 + arow) * a.T + t) * a.F + k);
-          else if (!with_h) continue;
-          else if (coherent) va[i] = load_coherent(hp + (int64_t)(r0 + arow) * a.H + (k - a.F));
-          else va[i] = *(const f4v*)(hp + (int64_t)(r0 + arow) * a.H + (k - a.F));
-        }
-      }
-      if (coherent) wait_coherent_loads(va);
-#pragma unroll
-      for (int i = 0; i < NA; ++i) {
-        const int q = i * 8 + (tid & 7);
-        if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
-      }
+    for (int i = 0; i < (NKB + 3) / 4; ++i) {
+      const int kb = wave + 4 * i;  // uniform in the wavefront
+      if (kb >= NKB) break;
+      const int k0 = 16 * kb + 4 * chunk;
+      const float* src = k0 < a.F ? xt + k0 : (k0 < K && with_h ? ht + k0 : seq_zero_chunk);
+      if (coherent) __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(As + kb * 256), 16, 0, 16);  // sc1: coherent at device scope
+      else __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(As + kb * 256), 16, 0, 0);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the compiler does not order LDS reads behind these loads by itself)
     __syncthreads();
-    f4v acc[NRB];
+    f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-    for (int r = 0; r < NRB; ++r) acc[r] = f4v{0.f, 0.f, 0.f, 0.f};
-    multiply_blocks<NRB>(As, Bs, K16, cb, rb0, lane, acc);
-    __syncthreads();
-    {  // pre-activations to the exchange area: element v of a lane is row 4*(l/16) + v of its block, column l%16
-      const int col = cb * 16 + (lane & 15), gate = col / UB, u = col % UB, g = lane >> 4;
+    for (int kb = 0; kb < NKB; ++kb) {
+      const f4v av = *(const f4v*)(ar + kb * 256);
 #pragma unroll
-      for (int r = 0; r < NRB; ++r)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) Zx[(gate * RB + (rb0 + r) * 16 + 4 * g + v) * ZP + u] = acc[r][v] + bias;
+      for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0);
     }
-    __syncthreads();
+    // pre-activations to the exchange area: element v of a lane is row 4 g + v, unit row16 of gate `wave`
+#pragma unroll
+    for (int v = 0; v < 4; ++v) Zx[(wave * SRB + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
+    __syncthreads();  // (also: every wavefront has read As)
     // ---- c = c_prev * f + i * g ; h = o * tanh(c)   (layer/RNN.scala:336-337)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int e = tid + 256 * j, row = e / UB, u = e % UB;
-      if (r0 + row >= a.rows) continue;
-      const float f = sigmoidf_(Zx[(0 * RB + row) * ZP + u]);
-      const float in = sigmoidf_(Zx[(1 * RB + row) * ZP + u]);
-      const float g = tanhf(Zx[(2 * RB + row) * ZP + u]);
-      const float o = sigmoidf_(Zx[(3 * RB + row) * ZP + u]);
-      const int64_t i = (int64_t)(r0 + row) * a.H + u0 + u;
-      float* gt = a.gates + (int64_t)t * 4 * a.slice + (int64_t)(r0 + row) * 4 * a.H + u0 + u;
-      const float c = c_reg[j] * f + in * g;
-      c_reg[j] = c;
+    if (live) {
+      const float f = sigmoidf_(Zx[(0 * SRB + crow) * ZP + cu] + bias[0]);
+      const float in = sigmoidf_(Zx[(1 * SRB + crow) * ZP + cu] + bias[1]);
+      const float gg = tanhf(Zx[(2 * SRB + crow) * ZP + cu] + bias[2]);
+      const float o = sigmoidf_(Zx[(3 * SRB + crow) * ZP + cu] + bias[3]);
+      float* gt = a.gates + (int64_t)t * 4 * a.slice + zi;
+      const float c = c_reg * f + in * gg;
+      c_reg = c;
       gt[0] = f;
       gt[a.H] = in;
-      gt[2 * a.H] = g;
+      gt[2 * a.H] = gg;
       gt[3 * a.H] = o;
-      a.c[(int64_t)t * a.slice + i] = c;
-      float* hout = a.h + (int64_t)(t + 1) * a.slice + i;
+      a.c[(int64_t)t * a.slice + ci] = c;
+      float* hout = a.h + (int64_t)(t + 1) * a.slice + ci;
       if (spread) __hip_atomic_store(hout, o * tanhf(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else *hout = o * tanhf(c);
     }
@@ -524,10 +526,10 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;
   const int r0 = rg * RB, u0 = ug * CBT;
-  unsigned* my_count = a.sync + rg;
-  unsigned* my_xcd = a.sync + a.row_groups + rg;
-  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
-  unsigned* abort_word = a.sync + 3 * a.row_groups;
+  unsigned* my_count = a.sync + rg * SEQ_GROUP_WORDS;
+  unsigned* my_xcd = my_count + 1;
+  unsigned* my_spread = my_count + 2;
+  unsigned* abort_word = a.sync + a.row_groups * SEQ_GROUP_WORDS;
 
   if (tid == 0) {  // arrival 0 (the placement check): do the members of this row group share an XCD?
     const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
@@ -648,9 +650,6 @@ __global__ __launch_bounds__(256) void pack_bwd_kernel(LstmWeights w, int H, flo
     *(f4v*)(out + e * 4) = *(const f4v*)(w.wr[gate] + (int64_t)(cb * 16 + col) * H + slice * BU + ul);
   }
 }
-
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* global_ptr_t;
 
 __global__ __launch_bounds__(256) void lstm_step_bwd_kernel(StepBwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -801,7 +800,7 @@ struct SeqBwdArgs {
   int force_coherent;
 };
 
-template <int NKB, int KO = 0>  // 16-long k blocks per wavefront: H = 8 NKB
+template <int NKB>  // 16-long k blocks per wavefront: H = 8 NKB
 __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   constexpr int UB = 16, H = 8 * NKB, HQ = H / 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -813,16 +812,16 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;
   const int r0 = rg * RB, u0 = ug * UB;
-  unsigned* my_count = a.sync + rg;
-  unsigned* my_xcd = a.sync + a.row_groups + rg;
-  unsigned* my_spread = a.sync + 2 * a.row_groups + rg;
-  unsigned* abort_word = a.sync + 3 * a.row_groups;
+  unsigned* my_count = a.sync + rg * SEQ_GROUP_WORDS;
+  unsigned* my_xcd = my_count + 1;
+  unsigned* my_spread = my_count + 2;
+  unsigned* abort_word = a.sync + a.row_groups * SEQ_GROUP_WORDS;
 
   if (tid == 0) {  // arrival 0 (the placement check): do the members of this row group share an XCD?
     const unsigned mine = 1u + (__builtin_amdgcn_s_getreg((3 << 11) | 20) & 15u);  // HW_REG_XCC_ID, 4 bits
     unsigned seen = 0u;
     __hip_atomic_compare_exchange_strong(my_xcd, &seen, mine, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((seen != 0u && seen != mine) || (a.force_coherent == 1)) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((seen != 0u && seen != mine) || a.force_coherent) __hip_atomic_store(my_spread, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
     __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
@@ -869,9 +868,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   const int64_t a_off = (int64_t)min(r0 + rb * 16 + (lane >> 2), a.rows - 1) * 4 * H + kh * 2 * H + 4 * ((lane & 3) ^ (lane >> 4));
   float* aw = As + wave * NKB * 256;
   const float* ar = aw + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
-  bool spread = true;
-  constexpr int ko = KO;
-  if (ko & 2) spread = false;
+  bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
   for (int t = a.T - 1;; --t) {
     // ---- gate gradients of step t
 #pragma unroll
@@ -889,8 +886,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       const float dzo = (o[j] * (1.0f - o[j])) * d_o;
       dcv[j] = dc * f[j];
       float* zt = a.dz + (int64_t)t * 4 * a.slice + zi[j];
-      if (ko & 32) { if (dzf == 123.f) zt[0] = dzi + dzg + dzo; }
-      else if (spread) {
+      if (spread) {
         __hip_atomic_store(zt, dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(zt + H, dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(zt + 2 * H, dzg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -904,11 +900,9 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     }
     if (t == 0) break;
     // ---- hand dz_t over: stores acknowledged in every wavefront, then one thread counts the workgroup in
-    if (!(ko & 16)) {
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
     __syncthreads();
-    }
-    if (tid == 0 && !(ko & 2)) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- what step t - 1 needs from the forward pass is requested while the others arrive
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -922,32 +916,28 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)(t - 1) * H] : 0.f;
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
-    if (!(ko & 2)) {
     if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, &stop)) return;
-    }
-    if (done == 0 && !(ko & 2)) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     // ---- dh_{t-1} of this workgroup's cells = dz_t (32 complete rows) * the weight slab
     {
       const float* ap = a.dz + (int64_t)t * 4 * a.slice + a_off;
-      if (!(ko & 4)) {
-        if (spread) {
+      if (spread) {
 #pragma unroll
-          for (int kb = 0; kb < NKB; ++kb)
-            __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 16);  // sc1: coherent at device scope
-        } else {
+        for (int kb = 0; kb < NKB; ++kb)
+          __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 16);  // sc1: coherent at device scope
+      } else {
 #pragma unroll
-          for (int kb = 0; kb < NKB; ++kb) __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 0);
-        }
+        for (int kb = 0; kb < NKB; ++kb) __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 0);
       }
-      // the blocks are this wavefront's own: its loads have landed, no barrier needed (the compiler does not order LDS reads
-      // behind these loads by itself)
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The blocks are this wavefront's own, so no barrier: block kb is multiplied as soon as all but the NKB - 1 - kb loads
+      // behind it have landed (loads return in order; the compiler does not order LDS reads behind these loads by itself).
       f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKB - 1 - kb) : "memory");
         const f4v av = *(const f4v*)(ar + kb * 256);
 #pragma unroll
-        for (int v = 0; v < 4; ++v) { if (ko & 8) acc[kb & 1][v] += av[v] * bw[kb][v]; else acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0); }
+        for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0);
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) Ps[(kh * RB + rb * 16 + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
@@ -1034,34 +1024,52 @@ int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const
 }
 
 namespace {
-size_t sequence_lds_bytes(int K) {  // the weight slab lies behind both the operand rows and the exchange area
-  const int K16 = round16(K);
-  return ((size_t)std::max(RB * (K16 + 4), 4 * RB * ZP) + (size_t)64 * K16) * sizeof(float);
+size_t sequence_lds_bytes(int nkb) { return (size_t)(nkb * 256 + 4 * SRB * ZP) * sizeof(float); }  // operand blocks + exchange area
+
+// calls f(kernel, blocks of 16 k) for the smallest instantiation that covers K, or returns false
+template <typename F>
+bool with_sequence_fwd_kernel(int K, F&& f) {
+  const int need = (K + 15) / 16;
+  if (need <= 2) f(lstm_sequence_fwd_kernel<2>, 2);
+  else if (need <= 3) f(lstm_sequence_fwd_kernel<3>, 3);
+  else if (need <= 5) f(lstm_sequence_fwd_kernel<5>, 5);
+  else if (need <= 8) f(lstm_sequence_fwd_kernel<8>, 8);
+  else if (need <= 12) f(lstm_sequence_fwd_kernel<12>, 12);
+  else if (need <= 18) f(lstm_sequence_fwd_kernel<18>, 18);
+  else if (need <= 25) f(lstm_sequence_fwd_kernel<25>, 25);
+  else return false;
+  return true;
 }
 }  // namespace
 
 bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) {
   if (rows <= 0 || !lstm_step_fused_ok(F, H, x, w)) return false;
-  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
-  if (3 * groups + 1 > SEQ_COUNTERS) return false;
-  if (allow_dynamic_lds(ctx, (const void*)lstm_sequence_fwd_kernel, sequence_lds_bytes(MAX_K)) != SN_OK) return false;
-  int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, lstm_sequence_fwd_kernel, 256, sequence_lds_bytes(F + H)) != hipSuccess) return false;
-  return blocks <= (int64_t)per_cu * ctx->compute_units;
+  const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+  if (groups > SEQ_MAX_GROUPS) return false;
+  bool fits = false;
+  const bool known = with_sequence_fwd_kernel(F + H, [&](auto kernel, int nkb) {
+    if (allow_dynamic_lds(ctx, (const void*)kernel, sequence_lds_bytes(nkb)) != SN_OK) return;
+    int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, sequence_lds_bytes(nkb)) != hipSuccess) return;
+    fits = blocks <= (int64_t)per_cu * ctx->compute_units;
+  });
+  return known && fits;
 }
 
 int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
                              const float* wpack, float* gates, float* c, float* h, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_fwd_ok(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SN_REQUIRE(aligned16(wpack) && aligned16(h), "lstm_sequence_forward: operands must start on 16-byte boundaries");
   SN_TRY(seq_sync_init(ctx));
-  const int groups = (int)ceil_div(rows, RB);
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * groups + 1));  // all-zero bits
+  const int groups = (int)ceil_div(rows, SRB);
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
   SeqFwdArgs a{x, c0, wpack, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
                ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_forward", rows * T, 4 * H, F + H);  // T steps of rows x 4H x (F + H)
-  hipLaunchKernelGGL(lstm_sequence_fwd_kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_lds_bytes(F + H),
-                     ctx->stream, a);
+  with_sequence_fwd_kernel(F + H, [&](auto kernel, int nkb) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_lds_bytes(nkb), ctx->stream, a);
+  });
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
@@ -1117,21 +1125,7 @@ bool with_sequence_bwd_kernel(int H, F&& f) {
     case 32: f(lstm_sequence_bwd_kernel<4>); return true;
     case 64: f(lstm_sequence_bwd_kernel<8>); return true;
     case 128: f(lstm_sequence_bwd_kernel<16>); return true;
-    case 256: {
-      const char* v = getenv("SN_KO");
-      switch (v ? atoi(v) : 0) {
-        case 2: f(lstm_sequence_bwd_kernel<32, 2>); break;
-        case 6: f(lstm_sequence_bwd_kernel<32, 6>); break;
-        case 10: f(lstm_sequence_bwd_kernel<32, 10>); break;
-        case 14: f(lstm_sequence_bwd_kernel<32, 14>); break;
-        case 18: f(lstm_sequence_bwd_kernel<32, 18>); break;
-        case 34: f(lstm_sequence_bwd_kernel<32, 34>); break;
-        case 50: f(lstm_sequence_bwd_kernel<32, 50>); break;
-        case 62: f(lstm_sequence_bwd_kernel<32, 62>); break;
-        default: f(lstm_sequence_bwd_kernel<32>); break;
-      }
-      return true;
-    }
+    case 256: f(lstm_sequence_bwd_kernel<32>); return true;
     default: return false;
   }
 }
@@ -1142,7 +1136,7 @@ bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
   for (int g = 0; g < 4; ++g)
     if (!aligned16(w.wr[g])) return false;
   const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
-  if (3 * groups + 1 > SEQ_COUNTERS) return false;
+  if (groups > SEQ_MAX_GROUPS) return false;
   bool fits = false;
   const bool known = with_sequence_bwd_kernel(H, [&](auto kernel) {
     if (allow_dynamic_lds(ctx, (const void*)kernel, sequence_bwd_lds_bytes(H)) != SN_OK) return;
@@ -1160,7 +1154,7 @@ int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, co
   SN_REQUIRE(aligned16(wpack) && aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
   SN_TRY(seq_sync_init(ctx));
   const int groups = (int)ceil_div(rows, RB);
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * groups + 1));  // all-zero bits
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
   SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, wpack, dz, slice, rows, T, H, groups, H / 16,
                ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
@@ -1189,7 +1183,7 @@ size_t rnn_sequence_lds_bytes(int K) {
 template <bool BACKWARD>
 bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
   const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * ceil_div(H, 32);
-  if (3 * groups + 1 > SEQ_COUNTERS) return false;
+  if (groups > SEQ_MAX_GROUPS) return false;
   if (allow_dynamic_lds(ctx, (const void*)rnn_sequence_kernel<BACKWARD>, rnn_sequence_lds_bytes(MAX_K)) != SN_OK) return false;
   int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rnn_sequence_kernel<BACKWARD>, 256, rnn_sequence_lds_bytes(K)) != hipSuccess) return false;
@@ -1204,7 +1198,7 @@ int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
   a.spin_limit = ctx->seq_spin_limit;
   a.gave_up = ctx->seq_gave_up_dev;
   a.force_coherent = ctx->seq_force_coherent;
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, 3 * a.row_groups + 1));  // all-zero bits
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(a.row_groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
   const int steps = BACKWARD ? a.T - 1 : a.T;
   LaunchScope scope(ctx, name, a.rows * steps, a.H, K);  // `steps` products of rows x H x K
   hipLaunchKernelGGL(rnn_sequence_kernel<BACKWARD>, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256),
