@@ -769,20 +769,19 @@ __global__ __launch_bounds__(256) void lstm_step_bwd_kernel(StepBwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------- all backward steps in one launch
-// The reverse recurrence, built like lstm_sequence_fwd_kernel: a workgroup owns 32 batch rows x 16 hidden units for the
-// whole sequence, keeps dc of its cells in registers and the recurrent weights of its units (all 4H k-values) in LDS.
+// The reverse recurrence, built like lstm_sequence_fwd_kernel: a workgroup owns 16 batch rows x 16 hidden units for the
+// whole sequence, keeps dc of its cells and the recurrent weights of its units (all 4H k-values) in registers.
 // What the unit groups of a row group hand to each other is dz_t itself, which has to be written anyway (the
 // weight-gradient GEMM reads it): a workgroup turns dh_t, dc and the saved gates of its cells into its 64 columns of
-// dz_t, counts itself in, waits for the others, reads the 32 complete rows of dz_t and multiplies them by its weight
+// dz_t, counts itself in, waits for the others, reads the 16 complete rows of dz_t and multiplies them by its weight
 // slab, which is dh_{t-1} of its own cells and never leaves the workgroup.  Every dz slice is written once and read
 // once per launch, so the two hand-over forms of the forward kernel apply unchanged (plain accesses within an XCD,
 // device-coherent ones otherwise), and so do the placement check and the bounded wait.
 //   do = dh * tanh(c);  dc += (1 - tanh(c)^2) * (dh * o)
 //   df = dc * c_prev;   di = dc * g;   dg = dc * i;   dc_prev = dc * f
 //   dz_gate = act'(z_gate) * d_gate;   dh_{t-1}[r, u] = sum_{gate, n} dz_t[r, gate H + n] * Wr_gate[u][n]
-// The rows of dz_t go straight from memory into the MFMA operand registers (lane (row, g) of a 16-row block holds
-// k = 16 kb + 4 g .. + 3): wavefront w multiplies row block w % 2 over half w / 2 of the 4H k-values, the two halves
-// meet in LDS and are added in a fixed order.
+// Wavefront w multiplies the rows by gate w's quarter of the 4H k-values; the four partial sums meet in LDS and are
+// added in a fixed order.
 struct SeqBwdArgs {
   const float* gates;    // T slices of 4 * slice floats: activated forget, input, gate, output of [rows, 4H]
   const float* c;        // T slices
@@ -800,18 +799,18 @@ struct SeqBwdArgs {
   int force_coherent;
 };
 
-template <int NKB>  // 16-long k blocks per wavefront: H = 8 NKB
+template <int NKB>  // 16-long k blocks per wavefront: H = 16 NKB
 __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
-  constexpr int UB = 16, H = 8 * NKB, HQ = H / 4;
+  constexpr int UB = 16, H = 16 * NKB, HQ = H / 4;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
-  float* Ps = lds;                  // [2 halves of k][RB][ZP] partial dh
-  float* As = lds + 2 * RB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]: dz_t as the loads deliver it
+  float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial dh
+  float* As = lds + 4 * SRB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]: dz_t as the loads deliver it
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;
-  const int r0 = rg * RB, u0 = ug * UB;
+  const int r0 = rg * SRB, u0 = ug * UB;
   unsigned* my_count = a.sync + rg * SEQ_GROUP_WORDS;
   unsigned* my_xcd = my_count + 1;
   unsigned* my_spread = my_count + 2;
@@ -825,67 +824,57 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
     __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  const int rb = wave & 1, kh = wave >> 1, row16 = lane & 15, g = lane >> 4;
-  // This wavefront's half of the unit group's weights stays in registers in MFMA operand order: lane (unit, g) holds
-  // k = kh 2H + 16 kb + 4 g .. + 3 of block kb.  The pack is [gate][unit block][n / 4][16 units][4 n].
+  const int row16 = lane & 15, g = lane >> 4;
+  // Wavefront w multiplies the k-values of gate w (k = w H .. w H + H - 1).  Its part of the unit group's weights stays in
+  // registers in MFMA operand order: lane (unit, g) holds n = 16 kb + 4 g .. + 3 of block kb.  The pack is
+  // [gate][unit block][n / 4][16 units][4 n].
   f4v bw[NKB];
   {
     const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-      const int kq = kh * (H / 2) + 4 * kb + g, gate = kq / HQ, q = kq % HQ;
-      bw[kb] = pack[((int64_t)(gate * a.unit_groups + ug) * HQ + q) * UB + row16];
-    }
+    for (int kb = 0; kb < NKB; ++kb) bw[kb] = pack[((int64_t)(wave * a.unit_groups + ug) * HQ + 4 * kb + g) * UB + row16];
   }
-  // the two cells this thread owns: row e / 16, unit e % 16 for e = tid, tid + 256
-  bool live[2];
-  int64_t ci[2], zi[2], yi[2];
-  float f[2], in[2], gg[2], o[2], cc[2], cp[2], dyv[2], dh[2], dcv[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int e = tid + 256 * j, row = e / UB, u = e % UB;
-    live[j] = r0 + row < a.rows;
-    const int64_t r = live[j] ? r0 + row : 0;
-    ci[j] = r * H + u0 + u;
-    zi[j] = r * 4 * H + u0 + u;
-    yi[j] = r * a.T * H + u0 + u;
+  // the cell this thread owns: row tid / 16, unit tid % 16
+  const int crow = tid >> 4, cu = tid & 15;
+  const bool live = r0 + crow < a.rows;
+  const int64_t cr = live ? r0 + crow : 0;
+  const int64_t ci = cr * H + u0 + cu, zi = cr * 4 * H + u0 + cu, yi = cr * a.T * H + u0 + cu;
+  float f, in, gg, o, cc, cp, dyv, dh, dcv = 0.f;
+  {
     const int t = a.T - 1;
-    const float* gt = a.gates + (int64_t)t * 4 * a.slice + zi[j];
-    f[j] = gt[0];
-    in[j] = gt[H];
-    gg[j] = gt[2 * H];
-    o[j] = gt[3 * H];
-    cc[j] = a.c[(int64_t)t * a.slice + ci[j]];
-    cp[j] = t > 0 ? a.c[(int64_t)(t - 1) * a.slice + ci[j]] : (a.c0 ? a.c0[ci[j]] : 0.f);
-    dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)t * H] : 0.f;
-    dh[j] = a.dh_last ? a.dh_last[ci[j]] : 0.f;
-    dcv[j] = 0.f;
+    const float* gt = a.gates + (int64_t)t * 4 * a.slice + zi;
+    f = gt[0];
+    in = gt[H];
+    gg = gt[2 * H];
+    o = gt[3 * H];
+    cc = a.c[(int64_t)t * a.slice + ci];
+    cp = t > 0 ? a.c[(int64_t)(t - 1) * a.slice + ci] : (a.c0 ? a.c0[ci] : 0.f);
+    dyv = a.dy_seq ? a.dy_seq[yi + (int64_t)t * H] : 0.f;
+    dh = a.dh_last ? a.dh_last[ci] : 0.f;
   }
   // One load instruction brings a 16-row x 16-k block of dz_t to 1 KiB of LDS, lane p to bytes 16 p .. 16 p + 15: four
   // neighbouring lanes fetch the 64 contiguous bytes of one row (rows past the batch: the last row again, their results
   // belong to no cell), and chunk c of row r lands in slot c ^ (r / 4) of the row so that the 16 lanes that later read
   // one chunk index of 16 rows hit 16 different bank groups.
-  const int64_t a_off = (int64_t)min(r0 + rb * 16 + (lane >> 2), a.rows - 1) * 4 * H + kh * 2 * H + 4 * ((lane & 3) ^ (lane >> 4));
+  const int64_t a_off = (int64_t)min(r0 + (lane >> 2), a.rows - 1) * 4 * H + wave * H + 4 * ((lane & 3) ^ (lane >> 4));
   float* aw = As + wave * NKB * 256;
   const float* ar = aw + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
   bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
   for (int t = a.T - 1;; --t) {
     // ---- gate gradients of step t
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (!live[j]) continue;
-      const float tc = tanhf(cc[j]);
-      float d = dh[j];
-      if (a.dy_seq) d = d + dyv[j];
+    if (live) {
+      const float tc = tanhf(cc);
+      float d = dh;
+      if (a.dy_seq) d = d + dyv;
       const float d_o = d * tc;
-      const float dc = dcv[j] + (1.0f - tc * tc) * (d * o[j]);
-      const float df = dc * cp[j], di = dc * gg[j], dg = dc * in[j];
-      const float dzf = (f[j] * (1.0f - f[j])) * df;
-      const float dzi = (in[j] * (1.0f - in[j])) * di;
-      const float dzg = (1.0f - gg[j] * gg[j]) * dg;
-      const float dzo = (o[j] * (1.0f - o[j])) * d_o;
-      dcv[j] = dc * f[j];
-      float* zt = a.dz + (int64_t)t * 4 * a.slice + zi[j];
+      const float dc = dcv + (1.0f - tc * tc) * (d * o);
+      const float df = dc * cp, di = dc * gg, dg = dc * in;
+      const float dzf = (f * (1.0f - f)) * df;
+      const float dzi = (in * (1.0f - in)) * di;
+      const float dzg = (1.0f - gg * gg) * dg;
+      const float dzo = (o * (1.0f - o)) * d_o;
+      dcv = dc * f;
+      float* zt = a.dz + (int64_t)t * 4 * a.slice + zi;
       if (spread) {
         __hip_atomic_store(zt, dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(zt + H, dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -904,21 +893,20 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     __syncthreads();
     if (tid == 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- what step t - 1 needs from the forward pass is requested while the others arrive
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const float* gt = a.gates + (int64_t)(t - 1) * 4 * a.slice + zi[j];
-      f[j] = gt[0];
-      in[j] = gt[H];
-      gg[j] = gt[2 * H];
-      o[j] = gt[3 * H];
-      cc[j] = cp[j];
-      cp[j] = t > 1 ? a.c[(int64_t)(t - 2) * a.slice + ci[j]] : (a.c0 ? a.c0[ci[j]] : 0.f);
-      dyv[j] = a.dy_seq ? a.dy_seq[yi[j] + (int64_t)(t - 1) * H] : 0.f;
+    {
+      const float* gt = a.gates + (int64_t)(t - 1) * 4 * a.slice + zi;
+      f = gt[0];
+      in = gt[H];
+      gg = gt[2 * H];
+      o = gt[3 * H];
+      cc = cp;
+      cp = t > 1 ? a.c[(int64_t)(t - 2) * a.slice + ci] : (a.c0 ? a.c0[ci] : 0.f);
+      dyv = a.dy_seq ? a.dy_seq[yi + (int64_t)(t - 1) * H] : 0.f;
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
     if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, &stop)) return;
     if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-    // ---- dh_{t-1} of this workgroup's cells = dz_t (32 complete rows) * the weight slab
+    // ---- dh_{t-1} of this workgroup's cells = dz_t (16 complete rows) * the weight slab
     {
       const float* ap = a.dz + (int64_t)t * 4 * a.slice + a_off;
       if (spread) {
@@ -940,18 +928,14 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
         for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0);
       }
 #pragma unroll
-      for (int v = 0; v < 4; ++v) Ps[(kh * RB + rb * 16 + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
+      for (int v = 0; v < 4; ++v) Ps[(wave * SRB + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
     }
     __syncthreads();
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int e = tid + 256 * j, row = e / UB, u = e % UB;
-      dh[j] = Ps[row * ZP + u] + Ps[(RB + row) * ZP + u];
-    }
+    dh = (Ps[crow * ZP + cu] + Ps[(SRB + crow) * ZP + cu]) + (Ps[(2 * SRB + crow) * ZP + cu] + Ps[(3 * SRB + crow) * ZP + cu]);
   }
 }
 
-size_t sequence_bwd_lds_bytes(int H) { return ((size_t)2 * RB * ZP + (size_t)RB * 4 * H) * sizeof(float); }
+size_t sequence_bwd_lds_bytes(int H) { return ((size_t)4 * SRB * ZP + (size_t)SRB * 4 * H) * sizeof(float); }
 
 size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 or 32)
   const int K16 = round16(K);
@@ -1117,15 +1101,15 @@ int launch_lstm_step_bwd(sn_ctx* ctx, const LstmGateBwdArgs& g, const float* dc_
 }
 
 namespace {
-// calls f(kernel, H / 8) for the instantiation that handles H, or returns false
+// calls f(kernel) for the instantiation that handles H, or returns false
 template <typename F>
 bool with_sequence_bwd_kernel(int H, F&& f) {
   switch (H) {
-    case 16: f(lstm_sequence_bwd_kernel<2>); return true;
-    case 32: f(lstm_sequence_bwd_kernel<4>); return true;
-    case 64: f(lstm_sequence_bwd_kernel<8>); return true;
-    case 128: f(lstm_sequence_bwd_kernel<16>); return true;
-    case 256: f(lstm_sequence_bwd_kernel<32>); return true;
+    case 16: f(lstm_sequence_bwd_kernel<1>); return true;
+    case 32: f(lstm_sequence_bwd_kernel<2>); return true;
+    case 64: f(lstm_sequence_bwd_kernel<4>); return true;
+    case 128: f(lstm_sequence_bwd_kernel<8>); return true;
+    case 256: f(lstm_sequence_bwd_kernel<16>); return true;
     default: return false;
   }
 }
@@ -1135,7 +1119,7 @@ bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
   if (rows <= 0) return false;
   for (int g = 0; g < 4; ++g)
     if (!aligned16(w.wr[g])) return false;
-  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+  const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
   bool fits = false;
   const bool known = with_sequence_bwd_kernel(H, [&](auto kernel) {
@@ -1153,7 +1137,7 @@ int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, co
   SN_REQUIRE(lstm_sequence_bwd_ok(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SN_REQUIRE(aligned16(wpack) && aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
   SN_TRY(seq_sync_init(ctx));
-  const int groups = (int)ceil_div(rows, RB);
+  const int groups = (int)ceil_div(rows, SRB);
   SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
   SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, wpack, dz, slice, rows, T, H, groups, H / 16,
                ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
