@@ -63,6 +63,7 @@ struct sn_ctx {
   // a word in pinned host memory that such a kernel sets when it gives up waiting for its neighbours, and how many
   // polls it waits before it does.  Allocated by the first launch that needs them.
   unsigned* seq_arrived = nullptr;
+  int64_t seq_next = 0;            // first word of the area no launch has used since it was last cleared
   int* seq_gave_up = nullptr;      // host address
   int* seq_gave_up_dev = nullptr;  // the same word as the device sees it
   unsigned seq_spin_limit = 0;
@@ -94,8 +95,9 @@ struct LaunchScope {
   ~LaunchScope();
 };
 int profile_drain(sn_ctx* ctx);
-// Sets up the context's sequence-kernel words on first use.
-int seq_sync_init(sn_ctx* ctx);
+// Hands a sequence-kernel launch its own all-zero block for `groups` row groups out of the context's area (set up on
+// first use).  The area is cleared in one go whenever it has been used up, so a launch costs no fill of its own.
+int seq_sync_take(sn_ctx* ctx, int groups, unsigned** block);
 // Words of a context's sequence-kernel area: one block of SEQ_GROUP_WORDS per row group (arrival counter, XCD word,
 // spread flag; a block of its own so that the pollers of different row groups do not meet on one cache line), then the
 // abort word's block.

@@ -1045,11 +1045,11 @@ int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_v
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_fwd_ok(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
   SN_REQUIRE(aligned16(wpack) && aligned16(h), "lstm_sequence_forward: operands must start on 16-byte boundaries");
-  SN_TRY(seq_sync_init(ctx));
   const int groups = (int)ceil_div(rows, SRB);
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
+  unsigned* sync = nullptr;
+  SN_TRY(seq_sync_take(ctx, groups, &sync));
   SeqFwdArgs a{x, c0, wpack, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
-               ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_forward", rows * T, 4 * H, F + H);  // T steps of rows x 4H x (F + H)
   with_sequence_fwd_kernel(F + H, [&](auto kernel, int nkb) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_lds_bytes(nkb), ctx->stream, a);
@@ -1136,11 +1136,11 @@ int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, co
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_bwd_ok(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SN_REQUIRE(aligned16(wpack) && aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
-  SN_TRY(seq_sync_init(ctx));
   const int groups = (int)ceil_div(rows, SRB);
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
+  unsigned* sync = nullptr;
+  SN_TRY(seq_sync_take(ctx, groups, &sync));
   SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, wpack, dz, slice, rows, T, H, groups, H / 16,
-               ctx->seq_arrived, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
   with_sequence_bwd_kernel(H, [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_bwd_lds_bytes(H), ctx->stream, a);
@@ -1175,14 +1175,12 @@ bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
 }
 template <bool BACKWARD>
 int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
-  SN_TRY(seq_sync_init(ctx));
   a.row_groups = (int)ceil_div(a.rows, RB);
   a.unit_groups = (int)ceil_div(a.H, 32);
-  a.sync = ctx->seq_arrived;
+  SN_TRY(seq_sync_take(ctx, a.row_groups, &a.sync));
   a.spin_limit = ctx->seq_spin_limit;
   a.gave_up = ctx->seq_gave_up_dev;
   a.force_coherent = ctx->seq_force_coherent;
-  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, (int64_t)(a.row_groups + 1) * SEQ_GROUP_WORDS));  // all-zero bits
   const int steps = BACKWARD ? a.T - 1 : a.T;
   LaunchScope scope(ctx, name, a.rows * steps, a.H, K);  // `steps` products of rows x H x K
   hipLaunchKernelGGL(rnn_sequence_kernel<BACKWARD>, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256),

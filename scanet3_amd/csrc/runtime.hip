@@ -78,7 +78,7 @@ int profile_drain(sn_ctx* ctx) {
   return SN_OK;
 }
 
-int seq_sync_init(sn_ctx* ctx) {
+static int seq_sync_init(sn_ctx* ctx) {
   if (ctx->seq_arrived) return SN_OK;
   unsigned* arrived = nullptr;
   int* word = nullptr;
@@ -96,12 +96,26 @@ int seq_sync_init(sn_ctx* ctx) {
     return fail(SN_E_HIP, "setting up the sequence kernels' counters failed: %s", hipGetErrorString(e));
   }
   ctx->seq_arrived = arrived;
+  ctx->seq_next = SEQ_COUNTERS;  // nothing cleared yet
   ctx->seq_gave_up = word;
   ctx->seq_gave_up_dev = static_cast<int*>(word_dev);
   // about a microsecond per poll: two seconds before a kernel whose neighbours never arrive gives up
   ctx->seq_spin_limit = 2000000u;
   if (const char* v = getenv("SCANET_SEQUENCE_SPIN_LIMIT")) ctx->seq_spin_limit = (unsigned)strtoul(v, nullptr, 10);
   if (const char* v = getenv("SCANET_SEQUENCE_COHERENT")) ctx->seq_force_coherent = atoi(v) != 0;
+  return SN_OK;
+}
+
+int seq_sync_take(sn_ctx* ctx, int groups, unsigned** block) {
+  SN_TRY(seq_sync_init(ctx));
+  const int64_t need = (int64_t)(groups + 1) * SEQ_GROUP_WORDS;
+  SN_REQUIRE(groups >= 1 && need <= SEQ_COUNTERS, "sequence kernel: %d row groups are more than the counter area holds", groups);
+  if (ctx->seq_next + need > SEQ_COUNTERS) {  // used up: the launches that used it are ahead of this fill on the stream
+    SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_arrived), 0.f, SEQ_COUNTERS));  // all-zero bits
+    ctx->seq_next = 0;
+  }
+  *block = ctx->seq_arrived + ctx->seq_next;
+  ctx->seq_next += need;
   return SN_OK;
 }
 
