@@ -174,7 +174,7 @@ SN_API int sn_ctx_destroy(sn_ctx* ctx);
 SN_API const char* sn_last_error(void);
 /* Blocks until everything issued on the context's stream has finished.
  * Like every call that synchronises (sn_copy_d2h, a step or gradient call that returns its loss), it returns
- * SN_E_STATE once if a recurrent layer's one-launch forward kernel gave up waiting for its neighbour workgroups
+ * SN_E_STATE once if a recurrent layer's one-launch forward or backward kernel gave up waiting for its neighbour workgroups
  * since the previous synchronisation (only possible when something else occupies compute units of the same GPU):
  * the results computed since then are invalid, the context stays usable.  The wait is a bounded number of polls
  * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, read when a context first launches that
