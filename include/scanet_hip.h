@@ -279,7 +279,8 @@ SN_API int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_de
                    int32_t global_iter, int32_t* iterations_host, float* loss_host);
 
 /* The same epoch over a partition in HOST memory (best allocated with sn_host_alloc: pinned memory makes the copies
- * asynchronous): batch i+1 is copied to the device on a second stream while batch i trains.  Replaces the
+ * asynchronous): runs of consecutive batches (1, 2, 4, ... up to 32 MiB or 64 batches) are copied to the device on a
+ * second stream while the run before trains.  Replaces the
  * TensorIterator -> feed path of optimizeOnPartition (optimizers/Iterators.scala:39-83, Optimizer.scala:136-157).
  * Results are those of sn_train_epoch on a device-resident copy of the same partition. */
 SN_API int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_host, int64_t total_rows, int32_t batch,

@@ -106,6 +106,7 @@ struct sn_replica {
   // host-fed epochs: two device slots per tensor, a copy stream, "slot filled" / "slot consumed" events
   float* stage_x[2] = {nullptr, nullptr};
   float* stage_y[2] = {nullptr, nullptr};
+  int64_t stage_group = 1;  // full batches a staging slot holds
   hipStream_t copy_stream = nullptr;
   hipEvent_t ev_filled[2] = {nullptr, nullptr}, ev_consumed[2] = {nullptr, nullptr};
   std::vector<void*> owned;
@@ -1403,8 +1404,12 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
     float* sy[2] = {nullptr, nullptr};
     hipEvent_t filled[2] = {nullptr, nullptr}, consumed[2] = {nullptr, nullptr};
     hipStream_t copy = nullptr;
-    const size_t xb = (size_t)rep->model->in_elems * rep->model->batch * sizeof(float);
-    const size_t yb = (size_t)rep->model->out_elems * rep->model->batch * sizeof(float);
+    // A slot holds a run of consecutive batches (up to 32 MiB or 64 batches): one copy and one pair of events per run
+    // instead of per step, which is what a small model's step would otherwise wait for.
+    const size_t one = (size_t)(rep->model->in_elems + rep->model->out_elems) * rep->model->batch * sizeof(float);
+    const int64_t group = std::max<int64_t>(1, std::min<int64_t>(64, (int64_t)(((size_t)32 << 20) / one)));
+    const size_t xb = (size_t)rep->model->in_elems * rep->model->batch * sizeof(float) * group;
+    const size_t yb = (size_t)rep->model->out_elems * rep->model->batch * sizeof(float) * group;
     hipError_t e = hipSetDevice(rep->ctx->device);
     for (int i = 0; i < 2 && e == hipSuccess; ++i) {
       e = hipMalloc((void**)&sx[i], xb);
@@ -1432,35 +1437,48 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
       rep->ev_consumed[i] = consumed[i];
     }
     rep->copy_stream = copy;
+    rep->stage_group = group;
   }
   const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
-  auto fill = [&](int64_t i, int slot) -> int {
-    SN_HIP(hipMemcpyAsync(rep->stage_x[slot], x_host + i * xs, (size_t)xs * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
-    SN_HIP(hipMemcpyAsync(rep->stage_y[slot], y_host + i * ys, (size_t)ys * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
+  // Runs of 1, 2, 4, ... up to stage_group batches: the first step waits for one batch only, later copies are long
+  const int64_t G = rep->stage_group;
+  auto fill = [&](int64_t first, int64_t nb, int slot) -> int {
+    SN_HIP(hipMemcpyAsync(rep->stage_x[slot], x_host + first * xs, (size_t)(nb * xs) * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
+    SN_HIP(hipMemcpyAsync(rep->stage_y[slot], y_host + first * ys, (size_t)(nb * ys) * sizeof(float), hipMemcpyHostToDevice, rep->copy_stream));
     SN_HIP(hipEventRecord(rep->ev_filled[slot], rep->copy_stream));
     return SN_OK;
   };
   // earlier work on the compute stream may still read the slots (a previous epoch's last loss)
   SN_HIP(hipEventRecord(rep->ev_consumed[0], compute));
   SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[0], 0));
-  SN_TRY(fill(0, 0));
-  for (int64_t i = 0; i < n_batches; ++i) {
-    const int slot = (int)(i & 1);
-    if (i + 1 < n_batches) {  // the other slot was last read by step i-1, already queued on the compute stream
-      if (i >= 1) SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[slot ^ 1], 0));
-      SN_TRY(fill(i + 1, slot ^ 1));
+  int64_t first = 0, nb = 1, last_first = 0;
+  int slot = 0;
+  SN_TRY(fill(first, nb, slot));
+  for (int64_t run = 0; first < n_batches; ++run) {
+    const int64_t next_first = first + nb, next_nb = std::min(std::min(G, 2 * nb), n_batches - next_first);
+    if (next_nb > 0) {  // the other slot was last read by the steps of run - 1, already queued on the compute stream
+      if (run >= 1) SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[slot ^ 1], 0));
+      SN_TRY(fill(next_first, next_nb, slot ^ 1));
     }
     SN_HIP(hipStreamWaitEvent(compute, rep->ev_filled[slot], 0));
-    SN_TRY(grad_pass(rep, rep->stage_x[slot], rep->stage_y[slot], batch, false));
-    SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
+    for (int64_t j = 0; j < nb; ++j) {
+      SN_TRY(grad_pass(rep, rep->stage_x[slot] + j * xs, rep->stage_y[slot] + j * ys, batch, false));
+      SN_TRY(update(rep, global_iter + (int)(first + j) + 1));  // optimizers/Optimizer.scala:143
+    }
     SN_HIP(hipEventRecord(rep->ev_consumed[slot], compute));
+    last_first = first;
+    first = next_first;
+    nb = next_nb;
+    slot ^= 1;
   }
+  const int last_slot = slot ^ 1;  // the slot of the run that held the last batch
   if (iterations_host) *iterations_host = (int32_t)n_batches;
-  const int last = (int)((n_batches - 1) & 1);
+  const float* last_x = rep->stage_x[last_slot] + (n_batches - 1 - last_first) * xs;
+  const float* last_y = rep->stage_y[last_slot] + (n_batches - 1 - last_first) * ys;
   if (loss_host) {  // optimizers/Optimizer.scala:148: loss of the last batch under the updated weights
-    SN_TRY(forward(rep, rep->stage_x[last], batch, false, true));
-    const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, rep->stage_x[last], batch);
-    SN_TRY(loss_of(rep, pred, rep->stage_y[last], batch, nullptr, true));
+    SN_TRY(forward(rep, last_x, batch, false, true));
+    const float* pred = op_output(rep, (int)rep->model->ops.size() - 1, last_x, batch);
+    SN_TRY(loss_of(rep, pred, last_y, batch, nullptr, true));
     SN_TRY(read_loss(rep, loss_host));
   } else {
     SN_HIP(hipStreamSynchronize(compute));  // the host buffers may be reused once this returns

@@ -856,10 +856,11 @@ def test_train_epoch_with_layer_state_and_its_average(S, ctx):
     cm.close()
 
 
-@pytest.mark.parametrize("n_batches", [1, 2, 7])
+@pytest.mark.parametrize("n_batches", [1, 2, 7, 127, 128, 300])
 def test_train_epoch_from_host_memory_equals_resident_epoch(S, ctx, n_batches):
-    """`sn_train_epoch_host` (batches copied on a second stream while the previous one trains) must leave exactly the
-    weights, optimizer state and loss of `sn_train_epoch` on a device-resident copy: same kernels, same order."""
+    """`sn_train_epoch_host` (runs of 1, 2, 4, ... batches, at most the 64 a staging slot of this small model holds, copied on a second
+    stream while the run before trains) must leave exactly the weights,
+    optimizer state and loss of `sn_train_epoch` on a device-resident copy: same kernels, same order."""
     spec = [("dense", 24, "tanh"), ("dense", 3, "softmax")]
     om, layers, sloss = build_pair(spec, "cce")
     batch, rows = 32, 32 * n_batches + 5               # 5 rows of a partial batch that both paths skip
