@@ -1090,6 +1090,39 @@ def test_lstm_sequence_kernel_hands_over_within_and_across_xcds(S, monkeypatch, 
         c.close()
 
 
+@pytest.mark.parametrize("units,features,batch,T", [(16, 4, 37, 5), (32, 8, 16, 3), (64, 12, 50, 4), (64, 64, 17, 2), (128, 52, 37, 5),
+                                                    (256, 32, 40, 3), (256, 144, 33, 4), (48, 16, 20, 3)])
+def test_lstm_sequence_kernels_over_their_instantiations(S, ctx, units, features, batch, T):
+    """The one-launch LSTM kernels are compiled per operand length: the forward one for 2, 3, 5, 8, 12, 18 and 25 blocks of
+    16 k-values over [x_t, h_{t-1}] (shorter operands are padded with zeros), the backward one for 16, 32, 64, 128 and 256
+    hidden units (48 units: forward in one launch, backward one launch per step).  Each against the oracle, with a last row
+    group that is not full, a bias and a second LSTM layer above that consumes the returned sequence."""
+    om = O.Model([O.LSTM(units, return_sequence=True), O.LSTM(16), O.Dense(2, O.ACT_IDENTITY)], O.LOSS_MSE)
+    layers = S.LSTM(units, returnSequence=True) >> S.LSTM(16) >> S.Dense(2, S.Identity)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+    rep = cm.replica(None)
+    rng = np.random.default_rng(4000 + units + features)
+    params = glorot_params(om, (batch, T, features), rng)
+    for p in params:
+        if params[p].ndim == 1:
+            params[p] = params[p] + rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
+    x = rng.standard_normal((batch, T, features)).astype(f32)
+    y = rng.uniform(-1, 1, (batch, 2)).astype(f32)
+    rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    assert rel_err(rep.forward(xb), om.forward(x, params)) <= TOL_GEMM
+    oloss, ograds = om.grad(x, y, params)
+    assert abs(rep.grad(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ggrads = rep.get_grads()
+    _, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_GEMM, 3.0 * rel_err(ograds[p], grads64[p])), p
+    for o in (rep, cm):
+        o.close()
+    xb.free()
+    yb.free()
+
+
 def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch):
     """A workgroup of the one-launch LSTM forward that waits for its neighbours polls a bounded number of times.  With the
     bound forced to zero (SCANET_SEQUENCE_SPIN_LIMIT, read when a context first launches the kernel) the first workgroup
