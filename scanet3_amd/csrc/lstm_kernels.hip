@@ -493,10 +493,11 @@ __global__ __launch_bounds__(256) void step_product_kernel(StepMulArgs a) {
 // The simple cell's two recurrences are one product per step with nothing around it:
 //   forward   r_t     = [x_t, r_{t-1}] * [Wk; Wr]                         (layer/RNN.scala:189-196), t = 0 .. T-1
 //   backward  dr_{t-1} = dr_t * Wr^T (+ the output gradient of step t-1 when the layer returns its sequence), t = T-1 .. 1
-// so one kernel runs either for all steps, built like lstm_sequence_fwd_kernel: a workgroup owns 32 batch rows x 32
-// units, keeps its weight slab in LDS, and the 32-unit groups of a row group hand the step's result to each other
-// through memory with the same arrival counter, placement check, bounded wait and two hand-over forms.  Every slice
-// is written once and read once per launch, so within an XCD plain loads find it in L2.
+// so one kernel runs either for all steps, built like the LSTM's one-launch kernels: a workgroup owns 16 batch rows x 16
+// units, each of its wavefronts multiplies a quarter of k (weights in registers, its blocks of the operand rows through
+// LDS-direct loads into LDS of its own), the four partial sums meet in LDS, and the unit groups of a row group hand the
+// step's result to each other through memory with the same arrival counter, placement check, bounded wait and two
+// hand-over forms.  Every slice is written once and read once per launch, so within an XCD plain loads find it in L2.
 struct SeqMulArgs {
   const float* x;       // forward: [rows, T, F]; backward: null
   float* rec;           // slices of `slice` floats; forward: slice t + 1 = r_t (slice 0 read only if first_valid),
@@ -513,19 +514,19 @@ struct SeqMulArgs {
   int force_coherent;
 };
 
-template <bool BACKWARD>
+template <bool BACKWARD, int NKBW>  // NKBW: 16-long blocks of k per wavefront (4 NKBW blocks cover K, padded with zeros)
 __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
-  constexpr int CBT = 32, NCB = CBT / 16, NRB = NCB / 2;
+  constexpr int UB = 16;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
-  const int K = a.F + a.H, K16 = round16(K), KP = K16 + 4, kq = K16 / 4;
-  float* As = lds;            // [RB][KP]
-  float* Bs = lds + RB * KP;  // [NCB][kq][16 units][4], kept for the whole sequence
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial sums
+  float* As = lds + 4 * SRB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]
+  const int K = a.F + a.H, kq = round16(K) / 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
   if (rg >= a.row_groups) return;
-  const int r0 = rg * RB, u0 = ug * CBT;
+  const int r0 = rg * SRB, u0 = ug * UB;
   unsigned* my_count = a.sync + rg * SEQ_GROUP_WORDS;
   unsigned* my_xcd = my_count + 1;
   unsigned* my_spread = my_count + 2;
@@ -539,14 +540,29 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
     __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
-  {  // the slab of this group's two unit blocks: contiguous in the pack, already in LDS cell order
-    const f4v* slab = reinterpret_cast<const f4v*>(a.wpack) + (int64_t)(u0 >> 4) * kq * 16;
-    const int blocks = min(NCB, (a.H - u0 + 15) >> 4);
-    for (int e = tid; e < NCB * kq * 16; e += 256) reinterpret_cast<f4v*>(Bs)[e] = e < blocks * kq * 16 ? slab[e] : f4v{0.f, 0.f, 0.f, 0.f};
+  const int row16 = lane & 15, g = lane >> 4;
+  // wavefront w multiplies k blocks w NKBW .. w NKBW + NKBW - 1; its part of the unit block's weights stays in registers in
+  // MFMA operand order (the pack is [unit block][K16 / 4][16 units][4 consecutive k])
+  f4v bw[NKBW];
+  {
+    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
+#pragma unroll
+    for (int i = 0; i < NKBW; ++i) {
+      const int q = 4 * (wave * NKBW + i) + g;
+      bw[i] = q < kq ? pack[((int64_t)ug * kq + q) * UB + row16] : f4v{0.f, 0.f, 0.f, 0.f};
+    }
   }
-  const int cb = wave % NCB, rb0 = (wave / NCB) * NRB;
-  constexpr int NA = 12;  // 8 * NA quads per operand row cover MAX_K
-  const int arow = tid >> 3;
+  // the element this thread finishes per step: row tid / 16, unit tid % 16
+  const int crow = tid >> 4, cu = tid & 15;
+  const bool live = r0 + crow < a.rows;
+  const int64_t ci = (int64_t)(live ? r0 + crow : 0) * a.H + u0 + cu;
+  // operand loads (see lstm_sequence_fwd_kernel): lane p fetches chunk (p % 4) ^ (p / 16) of row p / 4
+  const int chunk = (lane & 3) ^ (lane >> 4);
+  const int64_t arow = min(r0 + (lane >> 2), a.rows - 1);
+  const float* xrow = BACKWARD ? nullptr : a.x + arow * a.T * a.F;
+  float* aw = As + wave * NKBW * 256;
+  const float* ar = aw + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
+
   const int steps = BACKWARD ? a.T - 1 : a.T;
   bool spread = true;  // until arrival 0 is complete (the first wait below)
   for (int s = 0; s < steps; ++s) {
@@ -555,52 +571,39 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
       if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
       if (s == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
-    {
-      f4v va[NA];
-      const float* rp = a.rec + (int64_t)t * a.slice;
-      const bool with_rec = BACKWARD || s > 0 || a.first_valid;
-      const bool coherent = spread && s > 0;  // the first slice was written before this launch
+    const bool with_rec = BACKWARD || s > 0 || a.first_valid;
+    const bool coherent = spread && s > 0;  // the first slice was written before this launch
+    const float* xt = BACKWARD ? nullptr : xrow + (int64_t)t * a.F;
+    const float* rt = a.rec + (int64_t)t * a.slice + arow * a.H - a.F;  // indexed by k
 #pragma unroll
-      for (int i = 0; i < NA; ++i) {
-        const int q = i * 8 + (tid & 7), k = q * 4;
-        va[i] = f4v{0.f, 0.f, 0.f, 0.f};
-        if (q < kq && r0 + arow < a.rows && k < K) {
-          if (k < a.F) va[i] = *(const f4v*)(a.x + ((int64_t)(r0 + arow) * a.T + t) * a.F + k);
-          else if (!with_rec) continue;
-          else if (coherent) va[i] = load_coherent(rp + (int64_t)(r0 + arow) * a.H + (k - a.F));
-          else va[i] = *(const f4v*)(rp + (int64_t)(r0 + arow) * a.H + (k - a.F));
-        }
-      }
-      if (coherent) wait_coherent_loads(va);
-#pragma unroll
-      for (int i = 0; i < NA; ++i) {
-        const int q = i * 8 + (tid & 7);
-        if (q < kq) *(f4v*)(As + arow * KP + q * 4) = va[i];
-      }
+    for (int i = 0; i < NKBW; ++i) {
+      const int k0 = 16 * (wave * NKBW + i) + 4 * chunk;
+      const float* src = k0 < a.F ? xt + k0 : (k0 < K && with_rec ? rt + k0 : seq_zero_chunk);
+      if (coherent) __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(aw + i * 256), 16, 0, 16);  // sc1: coherent at device scope
+      else __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(aw + i * 256), 16, 0, 0);
     }
+    // the blocks are this wavefront's own: no barrier, block i is multiplied once all but the loads behind it have landed
+    f4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NKBW; ++i) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKBW - 1 - i) : "memory");
+      const f4v av = *(const f4v*)(ar + i * 256);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[i][v], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) Ps[(wave * SRB + 4 * g + v) * ZP + row16] = acc[v];
     __syncthreads();
-    f4v acc[NRB];
-#pragma unroll
-    for (int r = 0; r < NRB; ++r) acc[r] = f4v{0.f, 0.f, 0.f, 0.f};
-    multiply_blocks<NRB>(As, Bs, K16, cb, rb0, lane, acc);
-    const int col = u0 + cb * 16 + (lane & 15), g = lane >> 4;
     const int to = BACKWARD ? t - 1 : t + 1;
-    if (col < a.H) {
-      float* out = a.rec + (int64_t)to * a.slice;
-#pragma unroll
-      for (int r = 0; r < NRB; ++r)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          const int row = r0 + (rb0 + r) * 16 + 4 * g + v;
-          if (row >= a.rows) continue;
-          float val = acc[r][v];
-          if (BACKWARD && a.dy_seq) val = val + a.dy_seq[((int64_t)row * a.T + to) * a.H + col];
-          if (spread) __hip_atomic_store(out + (int64_t)row * a.H + col, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          else out[(int64_t)row * a.H + col] = val;
-        }
+    if (live) {
+      float val = (Ps[crow * ZP + cu] + Ps[(SRB + crow) * ZP + cu]) + (Ps[(2 * SRB + crow) * ZP + cu] + Ps[(3 * SRB + crow) * ZP + cu]);
+      if (BACKWARD && a.dy_seq) val = val + a.dy_seq[((int64_t)(r0 + crow) * a.T + to) * a.H + u0 + cu];
+      float* out = a.rec + (int64_t)to * a.slice + ci;
+      if (spread) __hip_atomic_store(out, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else *out = val;
     }
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0): the stores are acknowledged
-    __syncthreads();  // (also: As is free again)
+    __syncthreads();  // (also: Ps is free again)
     if (tid == 0 && s + 1 < steps) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
@@ -1160,31 +1163,48 @@ int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const 
 }
 
 namespace {
-size_t rnn_sequence_lds_bytes(int K) {
-  const int K16 = round16(K);
-  return ((size_t)RB * (K16 + 4) + (size_t)32 * K16) * sizeof(float);
+size_t rnn_sequence_lds_bytes(int nkbw) { return ((size_t)4 * SRB * ZP + (size_t)4 * nkbw * 256) * sizeof(float); }
+
+// calls f(kernel, blocks per wavefront) for the smallest instantiation that covers K, or returns false
+template <bool BACKWARD, typename F>
+bool with_rnn_sequence_kernel(int K, F&& f) {
+  const int need = (int)ceil_div(ceil_div(K, 16), 4);
+  if (need <= 1) f(rnn_sequence_kernel<BACKWARD, 1>, 1);
+  else if (need <= 2) f(rnn_sequence_kernel<BACKWARD, 2>, 2);
+  else if (need <= 3) f(rnn_sequence_kernel<BACKWARD, 3>, 3);
+  else if (need <= 4) f(rnn_sequence_kernel<BACKWARD, 4>, 4);
+  else if (need <= 5) f(rnn_sequence_kernel<BACKWARD, 5>, 5);
+  else if (need <= 7) f(rnn_sequence_kernel<BACKWARD, 7>, 7);
+  else return false;
+  return true;
 }
 template <bool BACKWARD>
 bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
-  const int64_t groups = ceil_div(rows, RB), blocks = 8 * ceil_div(groups, 8) * ceil_div(H, 32);
+  const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
-  if (allow_dynamic_lds(ctx, (const void*)rnn_sequence_kernel<BACKWARD>, rnn_sequence_lds_bytes(MAX_K)) != SN_OK) return false;
-  int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, rnn_sequence_kernel<BACKWARD>, 256, rnn_sequence_lds_bytes(K)) != hipSuccess) return false;
-  return blocks <= (int64_t)per_cu * ctx->compute_units;
+  bool fits = false;
+  const bool known = with_rnn_sequence_kernel<BACKWARD>(K, [&](auto kernel, int nkbw) {
+    if (allow_dynamic_lds(ctx, (const void*)kernel, rnn_sequence_lds_bytes(nkbw)) != SN_OK) return;
+    int per_cu = 0;  // the hand-over between workgroups needs the whole grid resident at once
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, rnn_sequence_lds_bytes(nkbw)) != hipSuccess) return;
+    fits = blocks <= (int64_t)per_cu * ctx->compute_units;
+  });
+  return known && fits;
 }
 template <bool BACKWARD>
 int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
-  a.row_groups = (int)ceil_div(a.rows, RB);
-  a.unit_groups = (int)ceil_div(a.H, 32);
+  a.row_groups = (int)ceil_div(a.rows, SRB);
+  a.unit_groups = a.H / 16;
   SN_TRY(seq_sync_take(ctx, a.row_groups, &a.sync));
   a.spin_limit = ctx->seq_spin_limit;
   a.gave_up = ctx->seq_gave_up_dev;
   a.force_coherent = ctx->seq_force_coherent;
   const int steps = BACKWARD ? a.T - 1 : a.T;
   LaunchScope scope(ctx, name, a.rows * steps, a.H, K);  // `steps` products of rows x H x K
-  hipLaunchKernelGGL(rnn_sequence_kernel<BACKWARD>, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256),
-                     rnn_sequence_lds_bytes(K), ctx->stream, a);
+  with_rnn_sequence_kernel<BACKWARD>(K, [&](auto kernel, int nkbw) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256), rnn_sequence_lds_bytes(nkbw),
+                       ctx->stream, a);
+  });
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
