@@ -177,7 +177,7 @@ SN_API const char* sn_last_error(void);
  * SN_E_STATE once if a recurrent layer's one-launch forward or backward kernel gave up waiting for its neighbour workgroups
  * since the previous synchronisation (only possible when something else occupies compute units of the same GPU):
  * the results computed since then are invalid, the context stays usable.  The wait is a bounded number of polls
- * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, read when a context first launches that
+ * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, 0 = give up at the first wait; read when a context first launches that
  * kernel; SCANET_SEQUENCE_COHERENT=1 makes the kernel hand its state over with device-coherent accesses even
  * between workgroups of one XCD). */
 SN_API int sn_sync(sn_ctx* ctx);

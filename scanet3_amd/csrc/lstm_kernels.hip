@@ -252,8 +252,8 @@ struct SeqFwdArgs {
 __device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, unsigned* abort_word, unsigned spin_limit, int* gave_up, int* stop) {
   if (threadIdx.x == 0) {
     unsigned spins = 0;
-    int bad = 0;
-    while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+    int bad = spin_limit == 0u;  // a limit of zero gives up at the first wait whatever the counter shows (how a test forces this path)
+    while (!bad && __hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
       // (every workgroup of the launch watches the one abort word: a look every 16th round keeps them off each other)
       if (++spins > spin_limit || ((spins & 15u) == 0u && __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)) {
         bad = 1;

@@ -1123,15 +1123,15 @@ def test_lstm_sequence_kernels_over_their_instantiations(S, ctx, units, features
     yb.free()
 
 
-def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch):
-    """A workgroup of the one-launch LSTM forward that waits for its neighbours polls a bounded number of times.  With the
-    bound forced to zero (SCANET_SEQUENCE_SPIN_LIMIT, read when a context first launches the kernel) the first workgroup
-    that has to wait gives up, every other one follows at its next wait, the kernel ends, and the next synchronising call
-    reports it once."""
+@pytest.mark.parametrize("kind", ["lstm", "simple_rnn"])
+def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
+    """A workgroup of a one-launch recurrent kernel that waits for its neighbours polls a bounded number of times.  With the
+    bound forced to zero (SCANET_SEQUENCE_SPIN_LIMIT, read when a context first launches such a kernel) every workgroup
+    gives up at its first wait, the kernel ends, and the next synchronising call reports it once."""
     monkeypatch.setenv("SCANET_SEQUENCE_SPIN_LIMIT", "0")
     c = S.Context(0)
     try:
-        layers = S.LSTM(256) >> S.Dense(1, S.Tanh)
+        layers = (S.LSTM(256) if kind == "lstm" else S.SimpleRNN(256, S.Tanh)) >> S.Dense(1, S.Tanh)
         cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (64, 32), 512)
         rep = cm.replica(None)
         xb = c.to_device(np.random.default_rng(5).standard_normal((512, 64, 32)).astype(f32))
