@@ -267,6 +267,12 @@ int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* 
 int launch_dense_skinny_dx(sn_ctx* ctx, const float* dy, const float* w, float* dx, int rows, int in_f, int out_f);
 // The same layer forward for small batches (partial sums per feature chunk in the workspace, then a fixed-order reduction
 // that applies e's bias and activation); dense_skinny_fwd_shape says whether shape and workspace are in its range.
+// A Dense layer onto at most 4 units from at most 1024 features (a regression head behind a recurrent layer): forward in one
+// launch, backward (activation gradient from the layer's output y, dX unless dx is null, dW, db unless null) in two.
+bool dense_tiny_shape(int rows, int in_f, int out_f, int64_t ws_elems);
+int launch_dense_tiny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f);
+int launch_dense_tiny_bwd(sn_ctx* ctx, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw, float* db, int rows,
+                          int in_f, int out_f, int act, float act_param, float* ws, int64_t ws_elems);
 bool dense_skinny_fwd_shape(int rows, int in_f, int out_f, int64_t ws_elems);
 int64_t dense_skinny_fwd_workspace(int rows, int in_f, int out_f);  // floats of workspace the forward form needs
 int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,

@@ -1959,4 +1959,144 @@ int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const E
   return SN_OK;
 }
 
+// ============================================================================ Dense onto a few units from a short row
+// A Dense(1..4) head behind a recurrent layer (512 x 256 -> 1): as GEMMs its three products are a split-K launch plus a
+// reduction launch each, every one of them at the floor of what a launch costs.  Here the forward pass is one launch (a
+// wavefront per row: 64 lanes walk the row, a butterfly adds them in a fixed order, lane 0 applies bias and activation)
+// and the backward pass two: a workgroup takes 16 rows, turns dY into dZ = act'(Y) dY itself, writes dX = dZ W^T
+// (AllKernels.scala:382-388) and leaves its share of dW = X^T dZ and db as one partial [in_f + 1][out_f];
+// gemm_small_reduce_kernel adds the partials in a fixed order.
+constexpr int TINY_MAX_UNITS = 4, TINY_MAX_FEATURES = 1024, TINY_MIN_FEATURES = 16, TINY_ROWS = 16, TINY_MAX_ROWS = 16384;
+
+bool dense_tiny_shape(int rows, int in_f, int out_f, int64_t ws_elems) {
+  return rows >= 1 && rows <= TINY_MAX_ROWS && out_f >= 1 && out_f <= TINY_MAX_UNITS && in_f >= TINY_MIN_FEATURES && in_f <= TINY_MAX_FEATURES &&
+         ceil_div(rows, TINY_ROWS) * (int64_t)(in_f + 1) * out_f <= ws_elems;
+}
+
+template <int N>
+__global__ __launch_bounds__(256) void dense_tiny_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, StdEpilogue ep, int rows,
+                                                             int in_f) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  float s[N];
+#pragma unroll
+  for (int n = 0; n < N; ++n) s[n] = 0.f;
+  const float* xr = x + (int64_t)row * in_f;
+  for (int i = lane; i < in_f; i += 64) {
+    const float xv = xr[i];
+#pragma unroll
+    for (int n = 0; n < N; ++n) s[n] = __builtin_fmaf(xv, w[i * N + n], s[n]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+    for (int n = 0; n < N; ++n) s[n] += __shfl_xor(s[n], off, 64);
+  if (lane == 0) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) ep.store(row, n, s[n]);
+  }
+}
+
+// the activation's gradient from its output (AllKernels.scala:297-302, 397-404, 414-420)
+__device__ __forceinline__ float tiny_act_bwd(int act, float y, float dy, float param) {
+  switch (act) {
+    case SN_ACT_SIGMOID: return (y * (1.0f - y)) * dy;
+    case SN_ACT_TANH: return (1.0f - y * y) * dy;
+    case SN_ACT_RELU: return (param < y ? 1.0f : 0.0f) * dy;
+    default: return dy;
+  }
+}
+
+template <int N>
+__global__ __launch_bounds__(256) void dense_tiny_bwd_kernel(const float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ dy,
+                                                             const float* __restrict__ w, float* __restrict__ dx, float* __restrict__ partial,
+                                                             int rows, int in_f, int act, float act_param, int with_bias) {
+  __shared__ float dzs[TINY_ROWS][N];
+  const int tid = threadIdx.x, r0 = blockIdx.x * TINY_ROWS, nr = min(TINY_ROWS, rows - r0);
+  if (tid < TINY_ROWS * N) {
+    const int r = tid / N, n = tid % N;
+    const int64_t o = (int64_t)(r0 + r) * N + n;
+    dzs[r][n] = r < nr ? tiny_act_bwd(act, y[o], dy[o], act_param) : 0.f;  // rows past the batch add nothing
+  }
+  __syncthreads();
+  float* part = partial + (int64_t)blockIdx.x * (in_f + with_bias) * N;
+  for (int i = tid; i < in_f; i += 256) {
+    float wr[N], acc[N], xv[TINY_ROWS];
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      wr[n] = w[i * N + n];
+      acc[n] = 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < TINY_ROWS; ++r) xv[r] = x[(int64_t)(r0 + (r < nr ? r : nr - 1)) * in_f + i];  // every load in flight
+#pragma unroll
+    for (int r = 0; r < TINY_ROWS; ++r) {
+      float s = 0.f;
+#pragma unroll
+      for (int n = 0; n < N; ++n) {
+        acc[n] = __builtin_fmaf(xv[r], dzs[r][n], acc[n]);
+        s = __builtin_fmaf(dzs[r][n], wr[n], s);
+      }
+      if (dx && r < nr) dx[(int64_t)(r0 + r) * in_f + i] = s;
+    }
+#pragma unroll
+    for (int n = 0; n < N; ++n) part[i * N + n] = acc[n];
+  }
+  if (with_bias && tid < N) {
+    float s = 0.f;
+    for (int r = 0; r < TINY_ROWS; ++r) s += dzs[r][tid];
+    part[in_f * N + tid] = s;
+  }
+}
+
+int launch_dense_tiny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f) {
+  SN_REQUIRE(dense_tiny_shape(rows, in_f, out_f, (int64_t)1 << 40), "dense_forward_row_dots: shape outside the kernel's range");
+  StdEpilogue ep{e};
+  LaunchScope scope(ctx, "dense_forward_row_dots", rows, out_f, in_f);
+  const unsigned blocks = (unsigned)ceil_div(rows, 4);
+#define SN_TINY_FWD(N) hipLaunchKernelGGL((dense_tiny_fwd_kernel<N>), dim3(blocks), dim3(256), 0, ctx->stream, x, w, ep, rows, in_f)
+  switch (out_f) {
+    case 1: SN_TINY_FWD(1); break;
+    case 2: SN_TINY_FWD(2); break;
+    case 3: SN_TINY_FWD(3); break;
+    default: SN_TINY_FWD(4); break;
+  }
+#undef SN_TINY_FWD
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_dense_tiny_bwd(sn_ctx* ctx, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw, float* db, int rows,
+                          int in_f, int out_f, int act, float act_param, float* ws, int64_t ws_elems) {
+  SN_REQUIRE(ws && dense_tiny_shape(rows, in_f, out_f, ws_elems), "dense_backward_rows16: shape outside the kernel's range");
+  const int parts = (int)ceil_div(rows, TINY_ROWS), with_bias = db ? 1 : 0;
+  {
+    LaunchScope scope(ctx, "dense_backward_rows16", rows, in_f, out_f);
+#define SN_TINY_BWD(N)                                                                                                                \
+  hipLaunchKernelGGL((dense_tiny_bwd_kernel<N>), dim3((unsigned)parts), dim3(256), 0, ctx->stream, x, y, dy, w, dx, ws, rows, in_f, act, \
+                     act_param, with_bias)
+    switch (out_f) {
+      case 1: SN_TINY_BWD(1); break;
+      case 2: SN_TINY_BWD(2); break;
+      case 3: SN_TINY_BWD(3); break;
+      default: SN_TINY_BWD(4); break;
+    }
+#undef SN_TINY_BWD
+  }
+  Epilogue e;
+  e.out = dw; e.ldo = out_f;
+  if (db) {
+    e.row_index = in_f;
+    e.row_out = db;
+  }
+  StdEpilogue ep{e};
+  LaunchScope scope(ctx, "small_output_reduce");
+  const int M = in_f + with_bias;
+  hipLaunchKernelGGL((gemm_small_reduce_kernel<StdEpilogue>), dim3((unsigned)ceil_div(M * out_f, 4)), dim3(256), 0, ctx->stream, (const float*)ws,
+                     parts, M, out_f, ep);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+
 }  // namespace sn

@@ -562,6 +562,8 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
             if (hidden_f32_not_needed(m, i)) eb.e.out = nullptr;  // the next layer and the backward pass read the bf16 copies
           }
           SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_x[i], in_f, r->bf_wt[i], in_f, rows, out_f, in_f, eb));
+        } else if (!bf16 && dense_tiny_shape(rows, in_f, out_f, m->workspace_elems)) {  // a few units behind a short row: one launch
+          SN_TRY(launch_dense_tiny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f));
         } else if (!bf16 && r->ws && dense_skinny_fwd_shape(rows, in_f, out_f, m->workspace_elems)) {
           SN_TRY(launch_dense_skinny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f, r->ws, m->workspace_elems));
         } else {
@@ -738,6 +740,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
             SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
             cur ^= 1;
           }
+          break;
+        }
+        if (!bf16 && r->ws && dense_tiny_shape(rows, in_f, out_f, m->workspace_elems)) {  // activation gradient, dX, dW and db in two launches
+          SN_TRY(launch_dense_tiny_bwd(ctx, in, r->act[i], dy, param_ptr(r, r->w, op.w), need_dx ? dx : nullptr, param_ptr(r, r->g, op.w),
+                                       param_ptr(r, r->g, op.b), rows, in_f, out_f, op.act, op.act_param, r->ws, m->workspace_elems));
+          if (need_dx) cur ^= 1;
           break;
         }
         if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
