@@ -305,7 +305,7 @@ MEASURED_TRAFFIC = {
     # for a plain copy of 400 MB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the summaries are under profiles/
     "conv2d_forward[52900x64x288]": (22.26e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[62500x32x576]": (22.31e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x52900]": (42.06e6, "gemm_kernels.hip", "a96c4c6b0a53b9d2759bd888da36c265d02c10e9"),
+    "conv2d_filter_gradient[288x64x52900]": (42.1e6, "gemm_kernels.hip", "06b9679400a5000eb07b58edced0c54e0b31cbe7"),
     "gemm_bf16_256[8192x4096x4096]": (539.0e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256[4096x4096x8192]": (495.3e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256_handover[8192x4096x4096]": (469.5e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
@@ -315,11 +315,11 @@ MEASURED_TRAFFIC = {
     "rnn_sequence_backward[32256x256x256]": (69.6e6, "lstm_kernels.hip", "0b1ed317af18c546ea065eb090fcdb3915d4b9bb"),
     "conv2d_forward[121000x64x288]": (53.32e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[169000x32x576]": (53.72e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x121000]": (72.19e6, "gemm_kernels.hip", "a96c4c6b0a53b9d2759bd888da36c265d02c10e9"),
+    "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "06b9679400a5000eb07b58edced0c54e0b31cbe7"),
     "mlp2_rows_forward_backward[1000x50x784]": (5.41e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
     "mlp2_weight_gradients[784x50x1000]": (8.69e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
-    "lstm_weight_gradient[289x1024x32768]": (318.5e6, "gemm_kernels.hip", "a96c4c6b0a53b9d2759bd888da36c265d02c10e9"),
-    "lstm_weight_gradient[288x256x32768]": (99.1e6, "gemm_kernels.hip", "a96c4c6b0a53b9d2759bd888da36c265d02c10e9"),
+    "lstm_weight_gradient[289x1024x32768]": (320.5e6, "gemm_kernels.hip", "06b9679400a5000eb07b58edced0c54e0b31cbe7"),
+    "lstm_weight_gradient[288x256x32768]": (99.1e6, "gemm_kernels.hip", "06b9679400a5000eb07b58edced0c54e0b31cbe7"),
     "adam": (2.800e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
     "average": (0.900e9, "optim_kernels.hip", "97cefbfb711005e251547ae97ed98d30a5e119cc"),
 }
