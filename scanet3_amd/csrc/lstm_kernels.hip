@@ -1,14 +1,17 @@
-// Fused LSTM time-step kernels for gfx950.
+// Recurrent-layer kernels for gfx950 (LSTM and the simple cell).
 //
-// One recurrent step multiplies a [rows, F+H] operand by weights that stay the same for the whole sequence
-// and is far too small to fill the chip as a tiled GEMM followed by an element-wise pass.  Here one workgroup
-// owns 32 batch rows x 64 output columns, stages the WHOLE reduction dimension of both operands in LDS with
-// every global load in flight at once, multiplies with v_mfma_f32_16x16x4_f32 (one 16-column block per
-// wavefront, two row blocks each) and finishes the step in its epilogue:
-//   forward  (layer/RNN.scala:303-340): the 64 columns are the four gates of 16 hidden units, so the
-//            workgroup applies the gate activations and writes gates, c_t and h_t itself;
-//   backward (the dz * Wr^T product of the reverse step): the reduction over 4H is cut per gate, each cut
-//            writes its own partial dh, and the gate-gradient kernel of the next (earlier) step adds the four.
+// One recurrent step multiplies a [rows, F+H] operand by weights that stay the same for the whole sequence and is far
+// too small to fill the chip as a tiled GEMM followed by an element-wise pass.  Two families live here:
+//   * one launch per direction for ALL time steps (lstm_sequence_fwd_kernel, lstm_sequence_bwd_kernel,
+//     rnn_sequence_kernel): a workgroup owns 16 batch rows x 16 hidden units for the whole sequence, keeps its weights in
+//     registers and its cell state (or cell gradient) too, fetches the step's operand rows with LDS-direct loads, and the
+//     unit groups of a row group hand h_t (backward: dz_t) to each other through the XCD's L2 with an arrival counter;
+//   * one launch per step (lstm_step_fwd_kernel, lstm_step_bwd_kernel, step_product_kernel), used where the first family
+//     does not fit the device or the shape: a workgroup owns 32 batch rows x 64 output columns, stages the WHOLE reduction
+//     dimension of both operands in LDS with every global load in flight at once, multiplies with
+//     v_mfma_f32_16x16x4_f32 and finishes the step in its epilogue (forward, layer/RNN.scala:303-340: the 64 columns are
+//     the four gates of 16 hidden units, so the workgroup applies the gate activations and writes gates, c_t and h_t
+//     itself; backward: gate gradients and the dz * Wr^T product share a kernel, cut into partial dh per unit slice).
 #include "common.hpp"
 
 namespace sn {
