@@ -354,24 +354,24 @@ int launch_lstm_pack(sn_ctx* ctx, const LstmWeights& w, int F, int H, float* pac
 // The simple cell's recurrences over all time steps in one launch (the LSTM sequence kernel's structure without gates).
 // Forward: r_slices holds T + 1 slices, slice t + 1 = r_t, slice 0 read only if first_valid.  Backward: dr_slices holds T
 // slices, slice T - 1 complete at launch, slice t - 1 = dr_t * Wr^T (+ dy_seq[:, t - 1, :] when given) for t = T-1 .. 1.
-bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const float* wpack);
-int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wpack, float* r_slices,
-                            int64_t slice);
-bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wpack);
-int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wpack, int64_t slice);
-// All T forward steps of an LSTM layer in one launch: the workgroups keep their weight slab in LDS and hand h_t to each
+bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x);
+int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wk, const float* wr,
+                            float* r_slices, int64_t slice);
+bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr);
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice);
+// All T forward steps of an LSTM layer in one launch: the workgroups keep their weights in registers and hand h_t to each
 // other through memory, one arrival counter per group of 32 batch rows.  h: T + 1 slices of `slice` floats, slice 0 the
 // initial hidden state (read only if h0_valid); gates / c: T slices.  lstm_sequence_fwd_ok says whether the launch fits
 // the device whole, which the hand-over needs.
 bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w);
 int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
-                             const float* wpack, float* gates, float* c, float* h, int64_t slice);
+                             float* gates, float* c, float* h, int64_t slice);
 // All reverse steps in one launch (H a power of two from 16 to 256): dz (T slices of 4 * slice floats) from the saved gates
 // and cell states, the gradient of the last hidden state (dh_last, may be null) and of a returned sequence (dy_seq
-// [rows, T, H], may be null).  wpack: launch_lstm_pack's pack_dh.  lstm_sequence_bwd_ok: as for the forward launch.
+// [rows, T, H], may be null).  lstm_sequence_bwd_ok: as for the forward launch.
 bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w);
 int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
-                             int rows, int H, const LstmWeights& w, const float* wpack, float* dz, int64_t slice);
+                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice);
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h);
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev

@@ -236,7 +236,8 @@ __device__ __forceinline__ void wait_coherent_loads(f4v (&v)[N]) {  // ties the 
 struct SeqFwdArgs {
   const float* x;        // [rows, T, F]
   const float* c0;       // [rows, H] or null: zeros
-  const float* wpack;    // pack_fwd_kernel's order
+  const float* wk[4];    // [F, H] forget, input, gate, output
+  const float* wr[4];    // [H, H]
   const float* bias[4];
   float* gates;          // T slices of 4 * slice floats: activated forget, input, gate, output of [rows, 4H]
   float* c;              // T slices
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
   __shared__ int stop;
   float* As = lds;              // [NKB][16 rows x 16 k]
   float* Zx = lds + NKB * 256;  // [4 gates][16 rows][ZP]
-  const int K = a.F + a.H, kq = round16(K) / 4;
+  const int K = a.F + a.H;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // id -> (row group, unit group): ids congruent mod 8 share an XCD, so XCD x takes the row groups x, x + 8, ...
   const int slot = blockIdx.x >> 3;
@@ -317,15 +318,19 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
   }
 
   const int row16 = lane & 15, g = lane >> 4;
-  // weights of gate `wave`: lane (unit = row16, g) holds k = 16 kb + 4 g .. + 3 for every kb
+  // weights of gate `wave`: lane (unit = row16, g) holds k = 16 kb + 4 g .. + 3 for every kb, k over [Wk; Wr], zeros past K
+  // (read once per launch, straight from the layer's tensors: 16 lanes fetch 64 contiguous bytes of a weight row)
   f4v bw[NKB];
   {
-    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);  // [unit group][gate][kq][16 units]: 4 consecutive k each
+    const float* wkc = a.wk[wave] + u0 + row16;
+    const float* wrc = a.wr[wave] + u0 + row16;
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-      const int q = 4 * kb + g;
-      bw[kb] = q < kq ? pack[((int64_t)(ug * 4 + wave) * kq + q) * UB + row16] : f4v{0.f, 0.f, 0.f, 0.f};
-    }
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = 16 * kb + 4 * g + j;
+        bw[kb][j] = k < a.F ? wkc[(int64_t)k * a.H] : (k < K ? wrc[(int64_t)(k - a.F) * a.H] : 0.f);
+      }
   }
   // the cell this thread finishes per step: row tid / 16, unit tid % 16
   const int crow = tid >> 4, cu = tid & 15;
@@ -506,7 +511,8 @@ struct SeqMulArgs {
   float* rec;           // slices of `slice` floats; forward: slice t + 1 = r_t (slice 0 read only if first_valid),
                         // backward: slice t = dr_t, slice T - 1 complete at launch
   const float* dy_seq;  // backward, returned sequence: [rows, T, H] added to slice t - 1 as it is written; or null
-  const float* wpack;   // [unit block of 16][K16 / 4][16 units][4 k]
+  const float* wk;      // forward: [F, H] kernel weights; backward: null
+  const float* wr;      // [H, H] recurrent weights
   int64_t slice;
   int first_valid;
   int rows, T, F, H;    // backward: F = 0
@@ -524,7 +530,7 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   __shared__ int stop;
   float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial sums
   float* As = lds + 4 * SRB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]
-  const int K = a.F + a.H, kq = round16(K) / 4;
+  const int K = a.F + a.H;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
@@ -545,14 +551,20 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   }
   const int row16 = lane & 15, g = lane >> 4;
   // wavefront w multiplies k blocks w NKBW .. w NKBW + NKBW - 1; its part of the unit block's weights stays in registers in
-  // MFMA operand order (the pack is [unit block][K16 / 4][16 units][4 consecutive k])
+  // MFMA operand order, read once per launch from the layer's own tensors: forward B[k][u] = [Wk; Wr][k][u] (16 lanes fetch
+  // 64 contiguous bytes of a weight row), backward B[k = n][u] = Wr[u][n] (a lane's 4 k-values are 16 contiguous bytes)
   f4v bw[NKBW];
-  {
-    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
 #pragma unroll
-    for (int i = 0; i < NKBW; ++i) {
-      const int q = 4 * (wave * NKBW + i) + g;
-      bw[i] = q < kq ? pack[((int64_t)ug * kq + q) * UB + row16] : f4v{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < NKBW; ++i) {
+    const int k0 = 16 * (wave * NKBW + i) + 4 * g;
+    if (BACKWARD) {
+      bw[i] = k0 < K ? *(const f4v*)(a.wr + (int64_t)(u0 + row16) * a.H + k0) : f4v{0.f, 0.f, 0.f, 0.f};
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = k0 + j;
+        bw[i][j] = k < a.F ? a.wk[(int64_t)k * a.H + u0 + row16] : (k < K ? a.wr[(int64_t)(k - a.F) * a.H + u0 + row16] : 0.f);
+      }
     }
   }
   // the element this thread finishes per step: row tid / 16, unit tid % 16
@@ -794,7 +806,7 @@ struct SeqBwdArgs {
   const float* c0;       // [rows, H] or null: zeros
   const float* dh_last;  // [rows, H] gradient of h_{T-1}, or null
   const float* dy_seq;   // [rows, T, H] gradient of a returned sequence (every step adds its own slice), or null
-  const float* wpack;    // pack_dh_kernel's order
+  const float* wr[4];    // [H, H] recurrent weights of forget, input, gate, output
   float* dz;             // T slices of 4 * slice floats
   int64_t slice;
   int rows, T, H;
@@ -807,7 +819,7 @@ struct SeqBwdArgs {
 
 template <int NKB>  // 16-long k blocks per wavefront: H = 16 NKB
 __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
-  constexpr int UB = 16, H = 16 * NKB, HQ = H / 4;
+  constexpr int UB = 16, H = 16 * NKB;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
   float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial dh
@@ -832,13 +844,13 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   }
   const int row16 = lane & 15, g = lane >> 4;
   // Wavefront w multiplies the k-values of gate w (k = w H .. w H + H - 1).  Its part of the unit group's weights stays in
-  // registers in MFMA operand order: lane (unit, g) holds n = 16 kb + 4 g .. + 3 of block kb.  The pack is
-  // [gate][unit block][n / 4][16 units][4 n].
+  // registers in MFMA operand order: lane (unit, g) holds Wr_w[unit][n = 16 kb + 4 g .. + 3] of block kb, 16 contiguous
+  // bytes of the layer's own tensor, read once per launch.
   f4v bw[NKB];
   {
-    const f4v* pack = reinterpret_cast<const f4v*>(a.wpack);
+    const float* wrow = a.wr[wave] + (int64_t)(u0 + row16) * H + 4 * g;
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) bw[kb] = pack[((int64_t)(wave * a.unit_groups + ug) * HQ + 4 * kb + g) * UB + row16];
+    for (int kb = 0; kb < NKB; ++kb) bw[kb] = *(const f4v*)(wrow + 16 * kb);
   }
   // the cell this thread owns: row tid / 16, unit tid % 16
   const int crow = tid >> 4, cu = tid & 15;
@@ -1047,14 +1059,14 @@ bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, c
 }
 
 int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
-                             const float* wpack, float* gates, float* c, float* h, int64_t slice) {
+                             float* gates, float* c, float* h, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_fwd_ok(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
-  SN_REQUIRE(aligned16(wpack) && aligned16(h), "lstm_sequence_forward: operands must start on 16-byte boundaries");
+  SN_REQUIRE(aligned16(h), "lstm_sequence_forward: operands must start on 16-byte boundaries");
   const int groups = (int)ceil_div(rows, SRB);
   unsigned* sync = nullptr;
   SN_TRY(seq_sync_take(ctx, groups, &sync));
-  SeqFwdArgs a{x, c0, wpack, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
+  SeqFwdArgs a{x, c0, {w.wk[0], w.wk[1], w.wk[2], w.wk[3]}, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
                sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_forward", rows * T, 4 * H, F + H);  // T steps of rows x 4H x (F + H)
   with_sequence_fwd_kernel(F + H, [&](auto kernel, int nkb) {
@@ -1138,14 +1150,14 @@ bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
 }
 
 int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
-                             int rows, int H, const LstmWeights& w, const float* wpack, float* dz, int64_t slice) {
+                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_bwd_ok(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
-  SN_REQUIRE(aligned16(wpack) && aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
+  SN_REQUIRE(aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
   const int groups = (int)ceil_div(rows, SRB);
   unsigned* sync = nullptr;
   SN_TRY(seq_sync_take(ctx, groups, &sync));
-  SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, wpack, dz, slice, rows, T, H, groups, H / 16,
+  SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, dz, slice, rows, T, H, groups, H / 16,
                sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
   with_sequence_bwd_kernel(H, [&](auto kernel) {
@@ -1213,29 +1225,29 @@ int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
 }
 }  // namespace
 
-bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const float* wpack) {
-  return rows > 0 && F % 4 == 0 && H % 16 == 0 && F + H <= MAX_K && aligned16(x) && aligned16(wpack) && rnn_sequence_fits<false>(ctx, rows, F + H, H);
+bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x) {
+  return rows > 0 && F % 4 == 0 && H % 16 == 0 && F + H <= MAX_K && aligned16(x) && rnn_sequence_fits<false>(ctx, rows, F + H, H);
 }
 
-int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wpack, float* r_slices,
-                            int64_t slice) {
+int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wk, const float* wr,
+                            float* r_slices, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
-  SN_REQUIRE(rnn_sequence_fwd_ok(ctx, rows, F, H, x, wpack), "rnn_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SN_REQUIRE(rnn_sequence_fwd_ok(ctx, rows, F, H, x), "rnn_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
   SeqMulArgs a{};
-  a.x = x; a.rec = r_slices; a.wpack = wpack; a.slice = slice; a.first_valid = first_valid;
+  a.x = x; a.rec = r_slices; a.wk = wk; a.wr = wr; a.slice = slice; a.first_valid = first_valid;
   a.rows = rows; a.T = T; a.F = F; a.H = H;
   return launch_rnn_sequence<false>(ctx, a, "rnn_sequence_forward", F + H);
 }
 
-bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wpack) {
-  return rows > 0 && H % 16 == 0 && H <= MAX_K && aligned16(wpack) && rnn_sequence_fits<true>(ctx, rows, H, H);
+bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr) {
+  return rows > 0 && H % 16 == 0 && H <= MAX_K && aligned16(wr) && rnn_sequence_fits<true>(ctx, rows, H, H);
 }
 
-int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wpack, int64_t slice) {
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice) {
   if (rows <= 0 || T <= 1) return SN_OK;
-  SN_REQUIRE(rnn_sequence_bwd_ok(ctx, rows, H, wpack), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
+  SN_REQUIRE(rnn_sequence_bwd_ok(ctx, rows, H, wr), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SeqMulArgs a{};
-  a.rec = dr_slices; a.dy_seq = dy_seq; a.wpack = wpack; a.slice = slice;
+  a.rec = dr_slices; a.dy_seq = dy_seq; a.wr = wr; a.slice = slice;
   a.rows = rows; a.T = T; a.F = 0; a.H = H;
   return launch_rnn_sequence<true>(ctx, a, "rnn_sequence_backward", H);
 }

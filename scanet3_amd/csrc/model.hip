@@ -598,18 +598,18 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w);
-        if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr));
         // stateful: the first step starts from the carried state (slice 0 of the hidden slices otherwise stays zero)
         const bool carried = op.state_p[0] >= 0;
         if (carried)
           SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[1]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
                                 ctx->stream));
-        if (fused && op.T > 1 && lstm_sequence_fwd_ok(ctx, rows, op.F, op.H, in, w)) {  // every step in one launch
+        if (fused && op.T > 1 && lstm_sequence_fwd_ok(ctx, rows, op.F, op.H, in, w)) {  // every step in one launch (it reads the weights as they lie)
           SN_TRY(launch_lstm_sequence_fwd(ctx, in, op.T, op.F, carried ? 1 : 0, carried ? param_ptr(r, r->w, op.state_p[0]) : nullptr, rows, op.H,
-                                          w, r->lstm_pk_fwd[i], r->lstm_gates[i], r->lstm_c[i], r->lstm_h[i], bh));
+                                          w, r->lstm_gates[i], r->lstm_c[i], r->lstm_h[i], bh));
           if (op.ret_seq) SN_TRY(launch_sequence_gather(ctx, r->lstm_h[i], bh, 1, r->act[i], rows, op.T, op.H));
           break;
         }
+        if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr));  // the step kernels' LDS order
         for (int t = 0; t < op.T; ++t) {
           const float* h_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
           const float* c_prev = t == 0 ? (carried ? param_ptr(r, r->w, op.state_p[0]) : nullptr) : r->lstm_c[i] + (int64_t)(t - 1) * bh;
@@ -640,14 +640,14 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         const int64_t bh = (int64_t)m->batch * op.H;
         const LstmWeights w = lstm_weights(r, op, r->w);  // slot 0 only, no bias inside the recurrence
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
-        if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr, 1));
         const bool carried = op.state_p[0] >= 0;  // stateful: slice 0 is the product the previous batch ended with
         if (carried)
           SN_HIP(hipMemcpyAsync(r->lstm_h[i], param_ptr(r, r->w, op.state_p[0]), (size_t)rows * op.H * sizeof(float), hipMemcpyDeviceToDevice,
                                 ctx->stream));
-        const bool whole = fused && op.T > 1 && rnn_sequence_fwd_ok(ctx, rows, op.F, op.H, in, r->lstm_pk_fwd[i]);
-        if (whole)  // every step in one launch
-          SN_TRY(launch_rnn_sequence_fwd(ctx, in, op.T, op.F, carried ? 1 : 0, rows, op.H, r->lstm_pk_fwd[i], r->lstm_h[i], bh));
+        const bool whole = fused && op.T > 1 && rnn_sequence_fwd_ok(ctx, rows, op.F, op.H, in);
+        if (whole)  // every step in one launch (it reads the weights as they lie)
+          SN_TRY(launch_rnn_sequence_fwd(ctx, in, op.T, op.F, carried ? 1 : 0, rows, op.H, w.wk[0], w.wr[0], r->lstm_h[i], bh));
+        else if (fused) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, r->lstm_pk_fwd[i], nullptr, 1));  // the step kernel's LDS order
         for (int t = whole ? op.T : 0; t < op.T; ++t) {
           const float* r_prev = t == 0 && !carried ? nullptr : r->lstm_h[i] + (int64_t)t * bh;
           float* r_t = r->lstm_h[i] + (int64_t)(t + 1) * bh;
@@ -837,9 +837,8 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         // every reverse step in one launch where the whole grid fits the device; the input gradients follow per step
         const bool whole = fused && op.T > 1 && lstm_sequence_bwd_ok(ctx, rows, op.H, w);
         if (whole) {
-          SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i]));
           SN_TRY(launch_lstm_sequence_bwd(ctx, r->lstm_gates[i], r->lstm_c[i], param_ptr(r, r->w, op.state_p[0]), op.ret_seq ? nullptr : dy,
-                                          op.ret_seq ? dy : nullptr, op.T, rows, op.H, w, r->lstm_pk_dh[i], r->lstm_dz[i], bh));
+                                          op.ret_seq ? dy : nullptr, op.T, rows, op.H, w, r->lstm_dz[i], bh));
           if (need_dx)
             for (int t = op.T - 1; t >= 0; --t)
               SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh * 4, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
@@ -917,12 +916,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dr, op.H, param_ptr(r, r->g, op.b), rows, op.H, r->ws, m->workspace_elems));
         }
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
-        if (fused && op.T > 1) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));
-        const bool whole = fused && op.T > 1 && rnn_sequence_bwd_ok(ctx, rows, op.H, r->lstm_pk_dh[i]);
+        const bool whole = fused && op.T > 1 && rnn_sequence_bwd_ok(ctx, rows, op.H, w.wr[0]);
+        if (fused && op.T > 1 && !whole) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));  // the step kernel's LDS order
         if (whole) {  // every step in one launch (it adds a returned sequence's output gradients itself), then the input gradients
           dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
           if (op.ret_seq) SN_TRY(launch_step_slice_add(ctx, dr, dy + (int64_t)(op.T - 1) * op.H, (int64_t)op.T * op.H, rows, op.H, false));
-          SN_TRY(launch_rnn_sequence_bwd(ctx, r->lstm_dz[i], op.ret_seq ? dy : nullptr, op.T, rows, op.H, r->lstm_pk_dh[i], bh));
+          SN_TRY(launch_rnn_sequence_bwd(ctx, r->lstm_dz[i], op.ret_seq ? dy : nullptr, op.T, rows, op.H, w.wr[0], bh));
           if (need_dx)
             for (int t = op.T - 1; t >= 0; --t)
               SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
