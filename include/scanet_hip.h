@@ -176,7 +176,8 @@ SN_API const char* sn_last_error(void);
  * Like every call that synchronises (sn_copy_d2h, a step or gradient call that returns its loss), it returns
  * SN_E_STATE once if a recurrent layer's one-launch forward or backward kernel gave up waiting for its neighbour workgroups
  * since the previous synchronisation (only possible when something else occupies compute units of the same GPU):
- * the results computed since then are invalid, the context stays usable.  The wait is a bounded number of polls
+ * the results computed since then are invalid, the context stays usable and from then on runs recurrent layers with one
+ * launch per time step.  The wait is a bounded number of polls
  * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, 0 = give up at the first wait; read when a context first launches that
  * kernel; SCANET_SEQUENCE_COHERENT=1 makes the kernel hand its state over with device-coherent accesses even
  * between workgroups of one XCD). */

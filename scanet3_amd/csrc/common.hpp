@@ -68,6 +68,7 @@ struct sn_ctx {
   int* seq_gave_up_dev = nullptr;  // the same word as the device sees it
   unsigned seq_spin_limit = 0;
   int seq_force_coherent = 0;      // hand over as if every row group were spread over several XCDs
+  bool seq_disabled = false;       // a one-launch kernel gave up once: from then on the per-step kernels run
   // timing
   bool profiling;
   std::vector<sn::PendingEvent> pending;

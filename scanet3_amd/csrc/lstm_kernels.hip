@@ -1045,6 +1045,7 @@ bool with_sequence_fwd_kernel(int K, F&& f) {
 }  // namespace
 
 bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) {
+  if (ctx->seq_disabled) return false;
   if (rows <= 0 || !lstm_step_fused_ok(F, H, x, w)) return false;
   const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
@@ -1134,6 +1135,7 @@ bool with_sequence_bwd_kernel(int H, F&& f) {
 }  // namespace
 
 bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
+  if (ctx->seq_disabled) return false;
   if (rows <= 0) return false;
   for (int g = 0; g < 4; ++g)
     if (!aligned16(w.wr[g])) return false;
@@ -1195,6 +1197,7 @@ bool with_rnn_sequence_kernel(int K, F&& f) {
 }
 template <bool BACKWARD>
 bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
+  if (ctx->seq_disabled) return false;
   const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
   bool fits = false;

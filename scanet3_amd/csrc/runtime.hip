@@ -122,6 +122,7 @@ int seq_sync_take(sn_ctx* ctx, int groups, unsigned** block) {
 int check_async(sn_ctx* ctx) {
   if (!ctx->seq_gave_up || *(volatile int*)ctx->seq_gave_up == 0) return SN_OK;
   *(volatile int*)ctx->seq_gave_up = 0;
+  ctx->seq_disabled = true;  // something else holds compute units of this GPU: do not count on the whole grid being resident again
   return fail(SN_E_STATE, "a recurrent sequence kernel gave up waiting for its neighbour workgroups (are other processes using this GPU?): "
                           "the results of the calls since the last synchronisation are invalid");
 }

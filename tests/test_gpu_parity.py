@@ -1127,7 +1127,8 @@ def test_lstm_sequence_kernels_over_their_instantiations(S, ctx, units, features
 def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
     """A workgroup of a one-launch recurrent kernel that waits for its neighbours polls a bounded number of times.  With the
     bound forced to zero (SCANET_SEQUENCE_SPIN_LIMIT, read when a context first launches such a kernel) every workgroup
-    gives up at its first wait, the kernel ends, and the next synchronising call reports it once."""
+    gives up at its first wait, the kernel ends, the next synchronising call reports it once, and the context falls back to
+    one launch per time step for the rest of its life."""
     monkeypatch.setenv("SCANET_SEQUENCE_SPIN_LIMIT", "0")
     c = S.Context(0)
     try:
@@ -1138,6 +1139,8 @@ def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
         with pytest.raises(S.ScanetError, match="gave up waiting"):
             rep.forward(xb)
         c.sync()                          # reported once: the context stays usable
+        again = rep.forward(xb)           # and from now on runs the layer one launch per step
+        assert np.isfinite(again).all() and np.array_equal(again, rep.forward(xb))
         for o in (rep, cm):
             o.close()
         xb.free()
