@@ -309,10 +309,10 @@ MEASURED_TRAFFIC = {
     "gemm_bf16_256[8192x4096x4096]": (539.0e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256[4096x4096x8192]": (495.3e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
     "gemm_bf16_256_handover[8192x4096x4096]": (469.5e6, "gemm_bf16.hip", "5dd97701c0b88d2bfa7ad86c07371e25b8af46be"),
-    "lstm_sequence_forward[32768x1024x288]": (249.7e6, "lstm_kernels.hip", "75bc16cd4929468ddf357f5fcab603fb9215652e"),
-    "lstm_sequence_backward[32256x256x1024]": (445.3e6, "lstm_kernels.hip", "75bc16cd4929468ddf357f5fcab603fb9215652e"),
-    "rnn_sequence_forward[32768x256x288]": (74.8e6, "lstm_kernels.hip", "75bc16cd4929468ddf357f5fcab603fb9215652e"),
-    "rnn_sequence_backward[32256x256x256]": (69.6e6, "lstm_kernels.hip", "75bc16cd4929468ddf357f5fcab603fb9215652e"),
+    "lstm_sequence_forward[32768x1024x288]": (249.7e6, "lstm_kernels.hip", "d2c6735cc068e8265d486453ebf886289f280779"),
+    "lstm_sequence_backward[32256x256x1024]": (445.3e6, "lstm_kernels.hip", "d2c6735cc068e8265d486453ebf886289f280779"),
+    "rnn_sequence_forward[32768x256x288]": (74.8e6, "lstm_kernels.hip", "d2c6735cc068e8265d486453ebf886289f280779"),
+    "rnn_sequence_backward[32256x256x256]": (69.6e6, "lstm_kernels.hip", "d2c6735cc068e8265d486453ebf886289f280779"),
     "conv2d_forward[121000x64x288]": (53.32e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[169000x32x576]": (53.72e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "06b9679400a5000eb07b58edced0c54e0b31cbe7"),
