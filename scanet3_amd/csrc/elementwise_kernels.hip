@@ -614,19 +614,35 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(const float* __restrict__
   }
 }
 
+// Division of an index below 2^31 by a divisor fixed for the launch, as a multiplication and a shift (the device has no
+// integer divider: a division by a run-time value is some twenty instructions, and these kernels take three per element).
+// d >= 1.  q = (hi32(x * mul) + x) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
+struct FastDiv {
+  uint32_t mul, shift, d;
+};
+static inline FastDiv fast_div(uint32_t d) {
+  uint32_t shift = 0;
+  while ((1ull << shift) < d) ++shift;
+  const uint64_t mul = ((1ull << 32) * ((1ull << shift) - d)) / d + 1;
+  return FastDiv{(uint32_t)mul, shift, d};
+}
+__device__ __forceinline__ uint32_t div_by(uint32_t x, const FastDiv& f) { return (__umulhi(x, f.mul) + x) >> f.shift; }
+
 // The same forward pass for 2x2 max windows, 4 channels per thread, 32-bit indices: the four window cells are requested
 // together (cells outside the input re-read the tensor's first element and never win), then compared in window order.
 __global__ __launch_bounds__(256) void pool2x2_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, uint8_t* __restrict__ arg,
-                                                           int n, int h, int w, int c, int ho, int wo, int sh, int sw, int pt, int pl) {
+                                                           int n, int h, int w, int c, int ho, int wo, int sh, int sw, int pt, int pl,
+                                                           FastDiv by_cv, FastDiv by_wo, FastDiv by_ho) {
   const uint32_t cv = (uint32_t)(c / 4);
   const uint32_t total = (uint32_t)n * ho * wo * cv;
   const uint32_t stride = (uint32_t)gridDim.x * blockDim.x;
   for (uint32_t i = (uint32_t)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const uint32_t ch = (i % cv) * 4;
-    uint32_t t = i / cv;
-    const int ow = (int)(t % wo); t /= wo;
-    const int oh = (int)(t % ho);
-    const uint32_t b = t / ho;
+    uint32_t t = div_by(i, by_cv);
+    const uint32_t ch = (i - t * cv) * 4;
+    uint32_t t2 = div_by(t, by_wo);
+    const int ow = (int)(t - t2 * (uint32_t)wo);
+    const uint32_t b = div_by(t2, by_ho);
+    const int oh = (int)(t2 - b * (uint32_t)ho);
     float4 val[4];
     bool in[4];
 #pragma unroll
@@ -668,7 +684,8 @@ int launch_pool_fwd(sn_ctx* ctx, bool avg, const float* x, float* y, uint8_t* ar
     else hipLaunchKernelGGL((pool_fwd_kernel<V, I, false>), grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, kh, kw, sh, sw, pt, pl);    \
   } while (0)
   if (v4 && small && !avg && kh == 2 && kw == 2)
-    hipLaunchKernelGGL(pool2x2_fwd_kernel, grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, sh, sw, pt, pl);
+    hipLaunchKernelGGL(pool2x2_fwd_kernel, grid, dim3(256), 0, ctx->stream, x, y, arg, n, h, w, c, ho, wo, sh, sw, pt, pl, fast_div((uint32_t)(c / 4)),
+                       fast_div((uint32_t)wo), fast_div((uint32_t)ho));
   else if (v4 && small) SN_POOL_FWD(4, uint32_t);
   else if (v4) SN_POOL_FWD(4, uint64_t);
   else if (small) SN_POOL_FWD(1, uint32_t);
@@ -759,18 +776,22 @@ __global__ __launch_bounds__(256) void pool_bwd_kernel(const float* __restrict__
 // The same backward pass for 2x2 max windows, 4 channels per thread, 32-bit indices: an input element lies in at most 2 x 2
 // windows (oh_hi - a, ow_hi - d for a, d in {0, 1}); their argmax words and gradients are requested together (windows that do
 // not exist re-read the first element and are ignored) and added in the order of the general kernel (oh, then ow, ascending).
+template <int S>  // both strides when they are equal and 1 or 2 (divisions by a constant), 0: read sh, sw
 __global__ __launch_bounds__(256) void pool2x2_bwd_kernel(const float* __restrict__ dy, const uint8_t* __restrict__ arg,
-                                                           float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo, int sh,
-                                                           int sw, int pt, int pl, const float* __restrict__ y_in, int act, float act_param) {
+                                                           float* __restrict__ dx, int n, int h, int w, int c, int ho, int wo, int sh_,
+                                                           int sw_, int pt, int pl, const float* __restrict__ y_in, int act, float act_param,
+                                                           FastDiv by_cv, FastDiv by_w, FastDiv by_h) {
+  const int sh = S ? S : sh_, sw = S ? S : sw_;
   const uint32_t cv = (uint32_t)(c / 4);
   const uint32_t total = (uint32_t)n * h * w * cv;
   const uint32_t stride = (uint32_t)gridDim.x * blockDim.x;
   for (uint32_t i = (uint32_t)xcd_contiguous_block() * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const uint32_t ch = (i % cv) * 4;
-    uint32_t t = i / cv;
-    const int ix = (int)(t % w); t /= w;
-    const int iy = (int)(t % h);
-    const uint32_t b = t / h;
+    uint32_t t = div_by(i, by_cv);
+    const uint32_t ch = (i - t * cv) * 4;
+    uint32_t t2 = div_by(t, by_w);
+    const int ix = (int)(t - t2 * (uint32_t)w);
+    const uint32_t b = div_by(t2, by_h);
+    const int iy = (int)(t2 - b * (uint32_t)h);
     int oh_lo = iy + pt - 1;
     oh_lo = oh_lo <= 0 ? 0 : (oh_lo + sh - 1) / sh;
     int oh_hi = (iy + pt) / sh;
@@ -830,7 +851,15 @@ int launch_pool_bwd(sn_ctx* ctx, bool avg, const float* dy, const uint8_t* arg, 
                          pt, pl, y_in, act, act_param);                                                                       \
   } while (0)
   if (v4 && small && !avg && kh == 2 && kw == 2)
-    hipLaunchKernelGGL(pool2x2_bwd_kernel, grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, sh, sw, pt, pl, y_in, act, act_param);
+  {
+    const FastDiv by_cv = fast_div((uint32_t)(c / 4)), by_w = fast_div((uint32_t)w), by_h = fast_div((uint32_t)h);
+    if (sh == 1 && sw == 1)
+      hipLaunchKernelGGL(pool2x2_bwd_kernel<1>, grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, sh, sw, pt, pl, y_in, act, act_param, by_cv, by_w, by_h);
+    else if (sh == 2 && sw == 2)
+      hipLaunchKernelGGL(pool2x2_bwd_kernel<2>, grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, sh, sw, pt, pl, y_in, act, act_param, by_cv, by_w, by_h);
+    else
+      hipLaunchKernelGGL(pool2x2_bwd_kernel<0>, grid, dim3(256), 0, ctx->stream, dy, arg, dx, n, h, w, c, ho, wo, sh, sw, pt, pl, y_in, act, act_param, by_cv, by_w, by_h);
+  }
   else if (v4 && small) SN_POOL_BWD(4, uint32_t);
   else if (v4) SN_POOL_BWD(4, uint64_t);
   else if (small) SN_POOL_BWD(1, uint32_t);
