@@ -60,25 +60,6 @@ def build_library(verbose: bool = True) -> str:
     return LIB_PATH
 
 
-def build_probes(verbose: bool = True) -> list:
-    """Compiles the stand-alone measurement programs under probes/ (they are not part of the library)."""
-    probes = os.path.join(HERE, "probes")
-    out_dir = os.path.join(probes, "build")
-    os.makedirs(out_dir, exist_ok=True)
-    built = []
-    for src in sorted(f for f in os.listdir(probes) if f.endswith(".hip")):
-        exe = os.path.join(out_dir, os.path.splitext(src)[0])
-        res = subprocess.run([hipcc(), "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                              "-o", exe, os.path.join(probes, src)], capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError(f"hipcc failed for probes/{src}:\n{res.stdout}\n{res.stderr}")
-        built.append(exe)
-    if verbose:
-        print(f"built {len(built)} probes under {out_dir}")
-    return built
-
-
 if __name__ == "__main__":
     build_library()
-    build_probes()
     sys.exit(0)
