@@ -283,25 +283,35 @@ int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const E
 // Besides the fp32 result (e.out, may be null) the epilogue can emit bf16 copies in both orientations,
 // which is how a Dense layer hands its output to the next one without a separate cast pass.
 struct EpilogueBf16 {
-  Epilogue e;
+  Epilogue e;                // e.out may be null when out_bf is set; e.act: identity or ReLU only
   void* out_bf = nullptr;    // bf16 [M, e.ldo]
-  void* out_bf_t = nullptr;  // bf16 [N, ld_t]
-  int64_t ld_t = 0;
-  // Gradient hand-over to the Dense layer below (dX products only; full 128-row / 128-column tiles, out_bf_t set, e.act
-  // identity): the result is multiplied by that layer's ReLU gradient, read off the sign of its output's transposed bf16
-  // copy grad_mask_t [N, ld_t] (null: identity activation, nothing to multiply), before it is cast and stored, and
-  // col_partials [M / 64, N] (optional) receives the column sums of every 64-row block of the fp32 values.
+  // Forward product that leaves as bf16 only (full 256 x 256 tiles, ReLU at 0): one bit per output value, set where
+  // the value passed the ReLU, [M * N / 32] words in the order the kernel's lanes hold the values.
+  void* signs_out = nullptr;
+  // Gradient hand-over to the Dense layer below (dX products only; full 256 x 256 tiles, out_bf set, e.out null, no
+  // bias, identity): the result is multiplied by that layer's ReLU gradient, read from the sign words its forward
+  // product wrote (null: identity activation, nothing to multiply), before it is cast and stored, and col_partials
+  // [M / 64, N] (optional) receives the column sums of every 64-row block of the fp32 values.
   bool grad_handover = false;
-  const void* grad_mask_t = nullptr;
+  const void* signs_in = nullptr;
   float* col_partials = nullptr;
 };
-int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep);
-// bf16 copies out[rows,cols] and out_t[cols,rows] of an fp32 matrix; with y != null the activation gradient
-// act'(y) * src is what gets cast (and is written to dz in fp32 when dz != null).  col_partials (optional,
-// [ceil(rows/64), cols]) receives the column sums of every 64-row block of the fp32 values.  y_bf: the layer output
-// as bf16 [rows, cols], used in place of y when y is null (enough for ReLU, whose gradient only needs the sign).
-int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
-                          int act, float act_param, float* dz, float* col_partials = nullptr, const void* y_bf = nullptr);
+// The three products of a Dense layer on bf16 copies of the tensors as they lie (no transposed copies):
+//   FORWARD  C[M,N] = a[M,K] . b[K,N]      (X . W)
+//   DX       C[M,N] = a[M,K] . b[N,K]^T    (dZ . W^T)
+//   DW       C[M,N] = a[K,M]^T . b[K,N]    (X^T . dZ)
+// lda / ldb are the row pitches of a and b as stored.
+enum { GEMM_BF16_FORWARD = 0, GEMM_BF16_DX = 1, GEMM_BF16_DW = 2 };
+int launch_gemm_bf16(sn_ctx* ctx, int product, const void* a, int64_t lda, const void* b, int64_t ldb, int M, int N, int K,
+                     const EpilogueBf16& ep);
+// true when an [M, N] forward result can leave as bf16 only and its dX counterpart can hand dZ over
+bool gemm_bf16_full_tiles(const sn_ctx* ctx, int M, int N);
+// bf16 copy out[rows,cols] of an fp32 matrix; with y or y_bf given the activation gradient act'(y) * src is what gets
+// cast (and is written to dz in fp32 when dz != null).  col_partials (optional, [ceil(rows/64), cols]) receives the
+// column sums of every 64-row block of the fp32 values.  y_bf: the layer output as bf16 [rows, cols], used in place of
+// y when y is null (enough for ReLU at 0, whose gradient only needs the sign).
+int launch_cast_bf16(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, const float* y, int act, float act_param,
+                     float* dz, float* col_partials = nullptr, const void* y_bf = nullptr);
 
 struct ConvGeom {
   int n, h, w, cin;      // input

@@ -1,65 +1,53 @@
 // bf16 matrix-core GEMM for the wide Dense layers (fp32 master data, bf16 operands, fp32 accumulate).
 //
-// Canonical form: C[M,N] = A[M,K] * Bt[N,K]^T with BOTH operands K-contiguous bf16, so every
-// global load is a 16-byte chunk of 8 consecutive k and goes to LDS unchanged.  The three Dense
-// products map onto it with bf16 copies kept in both orientations:
-//   forward  Y  = X  W      A = X   [rows,in]   Bt = W^T  [out,in]
-//   dX          = dY W^T    A = dY  [rows,out]  Bt = W    [in,out]
-//   dW          = X^T dY    A = X^T [in,rows]   Bt = dY^T [out,rows]
-// cast_transpose_kernel writes the two bf16 orientations of an fp32 matrix in one pass (optionally
-// applying the activation gradient on the way), which is all the extra traffic this path costs.
+// C[M,N] = sum_k A(m,k) B(n,k).  Each operand is either k-major (rows of its output index, k contiguous:
+// element (r,k) at p[r*ld + k]) or index-major (rows of k, the output index contiguous: element (r,k) at
+// p[k*ld + r]), so the three Dense products read the tensors as they lie and no transposed copy exists:
+//   forward  Y  = X  W      A = X  [rows,in]  k-major       B = W  [in,out]    index-major
+//   dX          = dZ W^T    A = dZ [rows,out] k-major       B = W  [in,out]    k-major
+//   dW          = X^T dZ    A = X  [rows,in]  index-major   B = dZ [rows,out]  index-major
 //
-// Kernel shape (WT = 128): 256 threads = 4 wavefronts (2x2), block tile 256x256, K step 64,
-// wavefront tile 128x128 = 4x4 v_mfma_f32_32x32x16_bf16 (256 accumulator registers per lane,
-// one wavefront per SIMD).  LDS holds two stages of A and B tiles (2 x 64 KiB of the 160 KiB);
-// rows are 128 bytes and their 16-byte chunks are XOR-swizzled so that the ds_read_b128 fragment
-// loads are conflict free.  Tiles travel HBM/L2 -> LDS with `buffer_load_dwordx4 ... lds`: no
-// staging registers, no ds_write instructions, and out-of-range rows / the k tail arrive as zeros
-// from the buffer descriptor's range check.  The loads of stage k+2 are issued right after the
-// barrier that publishes stage k+1, so they have a whole stage of MFMAs (about 2048 cycles) to land.
-// WT = 64 is the same kernel with a 128x128 block tile for outputs too small to fill 256 CUs.
+// Kernel shape: 256 threads = 4 wavefronts (2x2), wavefront tile (32 TM) x (32 TN) of v_mfma_f32_32x32x16_bf16
+// (TM = TN = 4: 256 accumulator registers per lane, one wavefront per SIMD), k stage 64, two LDS stages.  Tiles
+// travel HBM/L2 -> LDS with `buffer_load_dwordx4 ... lds` (no staging registers; rows past the matrix and the
+// k tail arrive as zeros from the buffer descriptor's range check).  A k-major tile is [rows][128 B] with
+// XOR-swizzled 16-byte chunks and feeds the matrix cores through ds_read_b128; an index-major tile is
+// [64 k][rows * 2 B] with XOR-swizzled 32-byte pairs and is read with ds_read_b64_tr_b16, which hands every
+// lane four consecutive k of its own row.  A workgroup walks several output tiles (persistent grid) and the stage
+// ring runs on across tile boundaries: the first stages of the next tile load while a tile's results leave.
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace sn {
 
 typedef __bf16 bf16;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s4v __attribute__((ext_vector_type(4)));
+typedef short s8v __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
-constexpr int GBK = 64;  // k per stage: 8 chunks of 8 bf16 = 128 bytes per tile row
+constexpr int GBK = 64;  // k per stage
 
-// Byte offset of 16-byte chunk `chunk` of tile row `row`.  The XOR pattern puts any 8 consecutive rows of one
-// logical chunk on 8 different 16-byte bank groups of a 128-byte line, and any 16 consecutive rows on 16
-// different groups of a 256-byte double line, so ds_read_b128 / ds_write_b128 stay conflict free whether the
-// LDS serves 8 or 16 lanes per cycle.
+// k-major tile: byte offset of 16-byte chunk `chunk` of tile row `row`.  Any 8 consecutive rows of one logical
+// chunk land on 8 different 16-byte bank groups of a 128-byte line, any 16 on 16 groups of a 256-byte double line.
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ ((row & 7) ^ ((row >> 3) & 1))) << 4); }
+// index-major tile: 16-byte chunk c of k-row k sits at chunk c ^ mn_xor(k) of that row.  The four k-rows a
+// transposing read touches per 16 lanes move their 32-byte pairs to four different bank groups, whether the LDS
+// serves 16 lanes (128 B) or 32 lanes (256 B) per cycle.
+__device__ __forceinline__ int mn_xor(int k) { return (0x6530 >> ((k & 3) * 4) & 7) << 1; }  // pair index ^ {0, 3, 5, 6}
 
-// Activations of the bf16 path: hardware exp2 / reciprocal (about 1e-6 relative), far inside bf16's 4e-3
-// and small enough to sit 256 times in an unrolled epilogue.
-__device__ __forceinline__ float fast_sigmoid(float v) { return __frcp_rn(1.0f + __expf(-v)); }
-__device__ __forceinline__ float fast_tanh(float v) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * v)); }
-
-__device__ __forceinline__ float bf_act(int act, float v, float param) {
-  switch (act) {
-    case SN_ACT_SIGMOID: return fast_sigmoid(v);
-    case SN_ACT_TANH: return fast_tanh(v);
-    case SN_ACT_RELU: return fmaxf(param, v);
-    default: return v;
-  }
-}
-
-// Raw buffer descriptor over [p, p + bytes): loads whose offset falls outside return zero, which is
-// how partial tiles (rows past M or N, the k tail) are handled without a branch.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
 constexpr uint32_t OOB = 0x80000000u;  // beyond any operand (operands are checked to be < 2 GiB)
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef __attribute__((address_space(3))) s4v* lds_s4p;
 
-// Epilogue modes: 0..3 = the activation (SN_ACT_*) as a compile-time constant, -1 = decide at run time (edge tiles).
 __device__ __forceinline__ float bf_act_grad(int act, float y, float dy, float param) {
   switch (act) {
     case SN_ACT_SIGMOID: return (y * (1.0f - y)) * dy;
@@ -69,325 +57,495 @@ __device__ __forceinline__ float bf_act_grad(int act, float y, float dy, float p
   }
 }
 
-// Per-wavefront LDS staging area for the transposed bf16 copy: [WT columns][WT rows + 4] bf16.
-template <int WT>
-constexpr int tr_pitch() { return WT * 2 + 8; }  // bytes per staged column
+// Epilogue modes (compile-time).
+constexpr int MODE_F32 = 0;       // fp32 result (+ bias, ReLU), optionally a bf16 copy; any shape (bounds-checked unless FULL)
+constexpr int MODE_BF16 = 1;      // bf16 result only (+ bias, ReLU at 0) and the ReLU's sign bits, full tiles
+constexpr int MODE_HANDOVER = 2;  // MODE_BF16 for a dX product that writes the dZ of the layer below (see GemmBf16Args)
 
-constexpr int MODE_HANDOVER = 8;  // EpilogueBf16::grad_handover (full tiles only)
+struct GemmBf16Args {
+  const bf16* a; const bf16* b;
+  int64_t lda, ldb;
+  int M, N, K;
+  int tiles_m, tiles_n;
+  float* out;            // fp32 [M, ldo] (MODE_F32)
+  bf16* out_bf;          // bf16 [M, ldo]
+  int64_t ldo;
+  const float* bias;     // per column, may be null
+  float relu_at;         // threshold of the ReLU (ACT = relu)
+  // MODE_BF16 with ReLU: one bit per output value, 1 where the value passed the ReLU, in the order the lanes of the
+  // 256 x 256 tiling hold them ([tile][wavefront][8 words][lane]); MODE_HANDOVER reads the same words back.
+  uint32_t* signs_out;
+  const uint32_t* signs_in;
+  float* col_partials;   // MODE_HANDOVER: [M / 64, N] column sums of every 64-row block of the fp32 values
+};
 
-template <int MODE, bool FULL, int TI>
-__device__ __forceinline__ void store_tile(const f16v (&acc)[TI][TI], const EpilogueBf16& ep, int mbase, int nbase, int lane, int M,
-                                           int N, char* stage) {
-  // mbase/nbase: origin of this wavefront's (32 TI) x (32 TI) tile.  Lane l holds column l%32 of every 32x32
-  // sub-tile and rows 8*(v/4) + 4*(l/32) + v%4 for accumulator element v.
-  constexpr int WT = 32 * TI;
-  constexpr int PITCH = tr_pitch<WT>();
-  const int l32 = lane & 31, lhi = lane >> 5;
-  const int row0 = mbase + lhi * 4, col0 = nbase + l32;
-  const int ldo = (int)ep.e.ldo;
-  const int64_t origin = (int64_t)row0 * ldo + col0;
-  float* out = ep.e.out ? ep.e.out + origin : nullptr;
-  bf16* obf = ep.out_bf ? (bf16*)ep.out_bf + origin : nullptr;
-  const bool transposed = ep.out_bf_t != nullptr;
-  // Hand-over mode: the 4 rows a lane holds per (i, vq) are 8 contiguous bytes of the transposed output copy of the layer
-  // below; a column's 4 TI masks are requested one column ahead of their use (requesting the whole tile's masks up front
-  // was measured and is slower).
-  constexpr bool HAND = MODE == MODE_HANDOVER;
-  constexpr int MT = HAND ? TI : 1;
-  const bf16* ym = (HAND && ep.grad_mask_t) ? (const bf16*)ep.grad_mask_t + (int64_t)col0 * ep.ld_t + row0 : nullptr;
-  bf16x4 mk[2][MT][4];
-  if (HAND && ym) {
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-#pragma unroll
-      for (int vq = 0; vq < 4; ++vq) mk[0][i][vq] = *(const bf16x4*)(ym + i * 32 + vq * 8);
-    }
-  }
-#pragma unroll
-  for (int j = 0; j < TI; ++j) {
-    if (!FULL && col0 + j * 32 >= N) continue;
-    const float bias = ep.e.bias ? ep.e.bias[col0 + j * 32] : 0.f;
-    if (HAND && ym && j + 1 < TI) {
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq) mk[(j + 1) & 1][i][vq] = *(const bf16x4*)(ym + (int64_t)(j + 1) * 32 * ep.ld_t + i * 32 + vq * 8);
-      }
-    }
-    float csum[(TI + 1) / 2];
-#pragma unroll
-    for (int b = 0; b < (TI + 1) / 2; ++b) csum[b] = 0.f;
-#pragma unroll
-    for (int i = 0; i < TI; ++i) {
-      // keep the scheduler from hoisting every tile's loads to the top: the accumulators fill the register file
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        bf16x4 packed;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = i * 32 + vq * 8 + e;
-          float x = acc[i][j][vq * 4 + e];
-          if (HAND) {
-            if (ym) x = (ep.e.act_param < (float)mk[j & 1][HAND ? i : 0][vq][e] ? 1.0f : 0.0f) * x;
-            csum[i / 2] += x;
-          }
-          if (FULL || row0 + r < M) {
-            if (ep.e.bias) x = x + bias;
-            if (MODE == SN_ACT_SIGMOID) x = fast_sigmoid(x);
-            else if (MODE == SN_ACT_TANH) x = fast_tanh(x);
-            else if (MODE == SN_ACT_RELU) x = fmaxf(ep.e.act_param, x);
-            else if (MODE < 0) x = bf_act(ep.e.act, x, ep.e.act_param);
-            if (out) out[r * ldo + j * 32] = x;
-            if (obf) obf[r * ldo + j * 32] = (bf16)x;
-          }
-          packed[e] = (bf16)x;
-        }
-        // 4 consecutive rows of one column are 8 contiguous bytes of the transposed tile
-        if (transposed) *(bf16x4*)(stage + (j * 32 + l32) * PITCH + (i * 32 + vq * 8 + lhi * 4) * 2) = packed;
-      }
-    }
-    if (HAND && ep.col_partials) {  // this column's sums over the wavefront's 64-row blocks: the two half-waves hold 4 rows of every 8 each
-#pragma unroll
-      for (int b = 0; b < (TI + 1) / 2; ++b) {
-        const float t = csum[b] + __shfl_xor(csum[b], 32, 64);
-        if (lhi == 0) ep.col_partials[(int64_t)(mbase / 64 + b) * N + col0 + j * 32] = t;
-      }
-    }
-  }
-  if (transposed) {
-    // C^T leaves through LDS so that every store instruction writes whole 16-byte chunks of contiguous rows:
-    // a lane takes 8 rows of one column, 64 lanes cover 64 / (WT/8) columns.
-    constexpr int CH = WT / 8;         // 16-byte chunks per staged column
-    constexpr int CPI = 64 / CH;       // columns per store instruction
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wavefront's staging writes are done (LDS is in-order per wave)
-    const int ch = lane % CH, cc = lane / CH;
-    bf16* obt = (bf16*)ep.out_bf_t;
-#pragma unroll 4
-    for (int c = 0; c < WT; c += CPI) {
-      const int col = c + cc;
-      const bf16x8 v = *(const bf16x8*)(stage + col * PITCH + ch * 16);
-      if (FULL || (nbase + col < N && mbase + ch * 8 < M))
-        *(bf16x8*)(obt + (int64_t)(nbase + col) * ep.ld_t + mbase + ch * 8) = v;
-    }
-  }
-}
-
-template <int WT, int MODE>
-__device__ __forceinline__ void gemm_bf16_tn_body(const bf16* __restrict__ A, int64_t lda, const bf16* __restrict__ Bt, int64_t ldb,
-                                                  int M, int N, int K, const EpilogueBf16& ep, int tiles_m, int tiles_n) {
-  constexpr int BT = 2 * WT;        // block tile edge
-  constexpr int TI = WT / 32;       // MFMA tiles per wavefront edge
-  constexpr int ISSUES = BT / 32;   // LDS-load issues per wavefront per operand per stage (8 rows of 128 B each)
-  constexpr int STAGE = BT * 128;   // bytes of one operand tile
+template <int TM, int TN, bool AMN, bool BMN, int MODE, int ACT, bool FULL>
+__device__ __forceinline__ void gemm_bf16_body(const GemmBf16Args& g) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;        // block tile
+  constexpr int STAGE_A = BM * 128, STAGE_B = BN * 128;  // bytes of one operand stage, either layout
+  constexpr int IA = 2 * TM, IB = 2 * TN;          // LDS-load issues per wavefront, operand and stage (1 KiB each)
+  static_assert(MODE == MODE_F32 || (TM == 4 && TN == 4 && FULL), "the bf16-only epilogues are built for full 256 x 256 tiles");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* sA = smem;                  // [2][STAGE]
-  char* sB = smem + 2 * STAGE;      // [2][STAGE]
-
-  // Tile order.  Consecutive workgroup ids land on different XCDs (8, each with its own L2), so first give
-  // every XCD a contiguous run of tile numbers, then walk the tiles in groups of 4 tile-rows, column by
-  // column: the 32 tiles an XCD works on at a time then form a 4 x 8 patch that shares 4 A panels and
-  // 8 B panels in that XCD's L2.
-  int t = blockIdx.x;
-  const int total = tiles_m * tiles_n;
-  if ((total & 7) == 0) t = (t & 7) * (total >> 3) + (t >> 3);
-  constexpr int GROUP = 4;
-  const int per_group = GROUP * tiles_n;
-  const int first_m = (t / per_group) * GROUP;
-  const int gsz = min(tiles_m - first_m, GROUP);
-  const int tm = first_m + (t % per_group) % gsz, tn = (t % per_group) / gsz;
-  const int m0 = tm * BT, n0 = tn * BT;
+  char* const sA = smem;                 // [2][STAGE_A]
+  char* const sB = smem + 2 * STAGE_A;   // [2][STAGE_B]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: LDS load targets go through M0
   const int l32 = lane & 31, lhi = lane >> 5;
-  const int wm = (wave >> 1) * WT, wn = (wave & 1) * WT;
+  const int wm = (wave >> 1) * (32 * TM), wn = (wave & 1) * (32 * TN);
+  const int M = g.M, N = g.N, K = g.K;
+  const int nk = ((K + GBK - 1) / GBK + 1) & ~1;  // stages per tile, padded to an even count (a padding stage loads zeros)
 
-  const __amdgpu_buffer_rsrc_t rsA = make_rsrc(A, (uint32_t)(((int64_t)(M - 1) * lda + K) * 2));
-  const __amdgpu_buffer_rsrc_t rsB = make_rsrc(Bt, (uint32_t)(((int64_t)(N - 1) * ldb + K) * 2));
-
-  // Staging map: issue q of wavefront w fills tile rows w*(BT/4) + 8q .. +7 (1 KiB of LDS, lane l at +16 l).
-  // LDS position (row r, physical chunk p) must hold logical chunk p ^ f(r), so that is what the lane fetches.
-  const int srow = lane >> 3, pchunk = lane & 7;
-  int lchunk[2];  // logical chunk for even / odd 8-row groups (f(r) = (r & 7) ^ ((r >> 3) & 1))
-  lchunk[0] = pchunk ^ srow;
-  lchunk[1] = pchunk ^ srow ^ 1;
-  const int r0 = wave * (BT / 4) + srow;                     // tile row of issue 0; issue q adds 8q
-  const int qa = (M - m0 - r0 + 7) >> 3, qb = (N - n0 - r0 + 7) >> 3;  // issues q >= qa / qb fall past the matrix
-  const uint32_t a0 = (uint32_t)(((int64_t)(m0 + r0) * lda) * 2), b0 = (uint32_t)(((int64_t)(n0 + r0) * ldb) * 2);
-  const uint32_t astep = (uint32_t)(lda * 16), bstep = (uint32_t)(ldb * 16);  // 8 rows in bytes
-  // One 1 KiB LDS-bound load: issue q of this wavefront for stage k0 of operand A / B.  A k0 at or past K
-  // gives out-of-range offsets, which the buffer load answers with zeros and no memory traffic.
-  // K is a multiple of 8, so a 16-byte chunk lies inside or outside its row as a whole.
-  auto issue_a = [&](int q, int k0, int buf) {
-    const int kc = k0 + lchunk[q & 1] * 8;
-    const uint32_t off = (q < qa && kc < K) ? a0 + q * astep + (uint32_t)kc * 2 : OOB;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr)(sA + buf * STAGE + wave * (BT / 4) * 128 + q * 1024), 16, (int)off, 0, 0, 0);
-  };
-  auto issue_b = [&](int q, int k0, int buf) {
-    const int kc = k0 + lchunk[q & 1] * 8;
-    const uint32_t off = (q < qb && kc < K) ? b0 + q * bstep + (uint32_t)kc * 2 : OOB;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr)(sB + buf * STAGE + wave * (BT / 4) * 128 + q * 1024), 16, (int)off, 0, 0, 0);
-  };
-
-  f16v acc[TI][TI];
-#pragma unroll
-  for (int i = 0; i < TI; ++i)
-#pragma unroll
-    for (int j = 0; j < TI; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  bf16x8 f0a[TI], f0b[TI], f1a[TI], f1b[TI];
-  // Fragment r of k sub-step s (16 k-values) of the stage in buffer `buf`, in the order the MFMAs of the next
-  // sub-step want them: A0, B0 .. B(TI-1), A1 .. A(TI-1).
-#define SN_READ_ONE(FA, FB, buf, s, r)                                                                              \
-  {                                                                                                                 \
-    if ((r) == 0) FA[0] = *(const bf16x8*)(sA + (buf) * STAGE + swz(wm + l32, (s) * 2 + lhi));                       \
-    else if ((r) <= TI) FB[(r) - 1] = *(const bf16x8*)(sB + (buf) * STAGE + swz(wn + ((r) - 1) * 32 + l32, (s) * 2 + lhi)); \
-    else FA[(r) - TI] = *(const bf16x8*)(sA + (buf) * STAGE + swz(wm + ((r) - TI) * 32 + l32, (s) * 2 + lhi));       \
-  }
-#define SN_FENCE() __builtin_amdgcn_sched_barrier(0)
-  // One k sub-step: TI*TI MFMAs in pairs; behind each pair go two fragment reads for the next sub-step
-  // (DO_READ) and this pair's share of the stage loads of operand LOAD (0 none, 1 A, 2 B), so that LDS reads
-  // and global loads are issued in the shadow of the matrix cores instead of between their bursts.
-  constexpr int NG = TI * TI / 2, PPR = TI / 2, LPG = ISSUES / NG;
-#define SN_SUBSTEP(CA, CB, NA, NB, DO_READ, rbuf, rs, LOAD, lk0, lbuf)                                               \
-  {                                                                                                                 \
-    _Pragma("unroll") for (int g = 0; g < NG; ++g) {                                                                 \
-      const int i_ = g / PPR, j_ = (g % PPR) * 2;                                                                   \
-      acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(CA[i_], CB[j_], acc[i_][j_], 0, 0, 0);                   \
-      acc[i_][j_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(CA[i_], CB[j_ + 1], acc[i_][j_ + 1], 0, 0, 0);       \
-      if (DO_READ) {                                                                                                \
-        _Pragma("unroll") for (int r_ = 2 * g; r_ < 2 * g + 2; ++r_)                                                 \
-          if (r_ < 2 * TI) SN_READ_ONE(NA, NB, rbuf, rs, r_);                                                       \
-      }                                                                                                             \
-      if ((LOAD) == 1) { _Pragma("unroll") for (int q_ = g * LPG; q_ < (g + 1) * LPG; ++q_) issue_a(q_, lk0, lbuf); } \
-      if ((LOAD) == 2) { _Pragma("unroll") for (int q_ = g * LPG; q_ < (g + 1) * LPG; ++q_) issue_b(q_, lk0, lbuf); } \
-      SN_FENCE();                                                                                                   \
-    }                                                                                                               \
-  }
-  // all of this wavefront's LDS-bound loads have landed, then everybody's
-#define SN_PUBLISH()                      \
-  {                                       \
-    __builtin_amdgcn_s_waitcnt(0);        \
-    __syncthreads();                      \
-  }
-
-  // Pipeline over k stages of 64 (4 sub-steps of 16) and two LDS buffers.  One barrier per stage, before
-  // sub-step 3: it publishes stage kt+1 and frees the current buffer.  The A half of stage kt+2 is loaded
-  // into the freed buffer during sub-step 3, the B half during sub-step 0 of the next stage, one load
-  // behind every MFMA pair; sub-step 3 also covers the first fragment reads of stage kt+1.
-  const int nk = (K + GBK - 1) / GBK;
-#pragma unroll
-  for (int q = 0; q < ISSUES; ++q) { issue_a(q, 0, 0); issue_b(q, 0, 0); }
-  SN_PUBLISH();
-#pragma unroll
-  for (int q = 0; q < ISSUES; ++q) issue_a(q, GBK, 1);
-#pragma unroll
-  for (int r = 0; r < 2 * TI; ++r) SN_READ_ONE(f0a, f0b, 0, 0, r);
-  SN_FENCE();
-  for (int kt = 0; kt + 1 < nk; ++kt) {
-    const int buf = kt & 1;
-    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 1, 2, (kt + 1) * GBK, buf ^ 1);
-    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf, 2, 0, 0, 0);
-    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 3, 0, 0, 0);
-    SN_PUBLISH();
-    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf ^ 1, 0, 1, (kt + 2) * GBK, buf);
-  }
-  {
-    const int buf = (nk - 1) & 1;
-    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 1, 0, 0, 0);
-    SN_SUBSTEP(f1a, f1b, f0a, f0b, true, buf, 2, 0, 0, 0);
-    SN_SUBSTEP(f0a, f0b, f1a, f1b, true, buf, 3, 0, 0, 0);
-    SN_SUBSTEP(f1a, f1b, f0a, f0b, false, 0, 0, 0, 0, 0);
-  }
-  __builtin_amdgcn_s_waitcnt(0);  // the zero-filling loads past the last stage have landed before LDS is reused
-#undef SN_READ_ONE
-#undef SN_SUBSTEP
-#undef SN_FENCE
-#undef SN_PUBLISH
-
-  // accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
-  char* stage = smem + wave * (WT * tr_pitch<WT>());
-  if (ep.out_bf_t) __syncthreads();  // the staging areas overlay the operand tiles other wavefronts may still be reading
-  // The epilogue mode is a template parameter of the KERNEL (the host picks it): with one full-tile and one
-  // edge-tile instantiation per kernel the accumulators stay in registers; a run-time switch over all modes
-  // inside one kernel makes the compiler demote them to scratch memory.
-  // The 256x256 kernel is only launched on outputs it tiles exactly: adding the bounds-checked variant next to
-  // the full-tile one also pushes its 256 accumulators out of the register file.
-  if (WT == 128 || (m0 + BT <= M && n0 + BT <= N)) store_tile<MODE, true, TI>(acc, ep, m0 + wm, n0 + wn, lane, M, N, stage);
-  else store_tile<-1, false, TI>(acc, ep, m0 + wm, n0 + wn, lane, M, N, stage);  // edge tiles: bounds-checked, mode picked at run time
-}
-
-// 256x256 tiles: 256 accumulator registers per lane, one wavefront per SIMD
-template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void gemm_bf16_tn_256(const bf16* __restrict__ A, int64_t lda, const bf16* __restrict__ Bt, int64_t ldb, int M, int N, int K,
-                      EpilogueBf16 ep, int tiles_m, int tiles_n) {
-  gemm_bf16_tn_body<128, MODE>(A, lda, Bt, ldb, M, N, K, ep, tiles_m, tiles_n);
-}
-// 128x128 tiles: two workgroups per CU
-template <int MODE>
-__global__ __launch_bounds__(256, 2)
-void gemm_bf16_tn_128(const bf16* __restrict__ A, int64_t lda, const bf16* __restrict__ Bt, int64_t ldb, int M, int N, int K,
-                      EpilogueBf16 ep, int tiles_m, int tiles_n) {
-  gemm_bf16_tn_body<64, MODE>(A, lda, Bt, ldb, M, N, K, ep, tiles_m, tiles_n);
-}
-
-template <int MODE>
-static int launch_mode(sn_ctx* ctx, const bf16* a, int64_t lda, const bf16* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep) {
-  const int64_t big_tiles = ceil_div(M, 256) * ceil_div(N, 256);
-  if (big_tiles >= ctx->compute_units && M % 256 == 0 && N % 256 == 0) {
-    const size_t smem = 4 * 128 * tr_pitch<128>() > 4 * 256 * 128 ? 4 * 128 * tr_pitch<128>() : 4 * 256 * 128;
-    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_256<MODE>, smem));
-    const int tm = (int)ceil_div(M, 256), tn = (int)ceil_div(N, 256);
-    LaunchScope scope(ctx, MODE == MODE_HANDOVER ? "gemm_bf16_256_handover" : "gemm_bf16_256", M, N, K);
-    hipLaunchKernelGGL(gemm_bf16_tn_256<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);
+  // ------------------------------------------------------------------ this workgroup's tiles
+  // Consecutive workgroup ids land on different XCDs (8, each with its own L2): every XCD gets a contiguous run of
+  // tile numbers, and tile numbers walk the output in groups of 4 tile-rows, column by column, so the tiles an XCD
+  // works on at a time form a patch that shares few A and B panels in its L2.
+  const int total = g.tiles_m * g.tiles_n;
+  int first, stride, count;
+  if ((gridDim.x & 7) == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+    const int base = total >> 3, rem = total & 7;
+    const int lo = xcd * base + min(xcd, rem), n_x = base + (xcd < rem ? 1 : 0);
+    first = lo + slot; stride = slots; count = slot < n_x ? (n_x - slot + slots - 1) / slots : 0;
   } else {
-    const size_t smem = 4 * 64 * tr_pitch<64>() > 4 * 128 * 128 ? 4 * 64 * tr_pitch<64>() : 4 * 128 * 128;
-    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_tn_128<MODE>, smem));
-    const int tm = (int)ceil_div(M, 128), tn = (int)ceil_div(N, 128);
-    LaunchScope scope(ctx, MODE == MODE_HANDOVER ? "gemm_bf16_128_handover" : "gemm_bf16_128", M, N, K);
-    hipLaunchKernelGGL(gemm_bf16_tn_128<MODE>, dim3((unsigned)(tm * tn)), dim3(256), smem, ctx->stream, a, lda, bt, ldb, M, N, K, ep, tm, tn);
+    first = blockIdx.x; stride = gridDim.x; count = (int)blockIdx.x < total ? (total - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+  }
+  if (count == 0) return;
+  auto tile_origin = [&](int t, int& m0, int& n0) {
+    constexpr int GROUP = 4;
+    const int per_group = GROUP * g.tiles_n;
+    const int first_m = (t / per_group) * GROUP;
+    const int gsz = min(g.tiles_m - first_m, GROUP);
+    m0 = (first_m + (t % per_group) % gsz) * BM;
+    n0 = ((t % per_group) / gsz) * BN;
+  };
+
+  // ------------------------------------------------------------------ global -> LDS
+  const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.a, (uint32_t)((AMN ? (int64_t)(K - 1) * g.lda + M : (int64_t)(M - 1) * g.lda + K) * 2));
+  const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.b, (uint32_t)((BMN ? (int64_t)(K - 1) * g.ldb + N : (int64_t)(N - 1) * g.ldb + K) * 2));
+  // A load cursor: where the next stage of this operand comes from.  base[p]: this lane's byte offset for issue 0
+  // (p = parity of the issue number) at k = 0 of the cursor's tile; issue q adds q * qstep, stage k0 adds k0 * kmul.
+  struct Cursor { uint32_t base[2]; int k0; int next_tile; };
+  // k-major: issue q of wavefront w fills tile rows w*(rows/4) + 8q .. +7; LDS position (row, physical chunk p) holds
+  // logical chunk p ^ f(row).  Rows past the matrix lie past the descriptor's range by themselves (ld >= K); a chunk
+  // past K inside a row does not, so that is checked per issue.
+  // index-major: issue q fills k-rows w*16 + kpi*q .. of the stage (kpi = 1024 / row bytes); LDS position (k, physical
+  // chunk p) holds logical chunk p ^ mn_xor(k).  k-rows past K are out of range by themselves; a chunk past the last
+  // column is not, so the lane's base is out of range then.
+  auto setup = [&](auto MN_, auto T_, Cursor& c, int origin, int64_t ld, int extent, int klane[2]) {
+    constexpr bool MN = decltype(MN_)::value;
+    constexpr int T = decltype(T_)::value;
+    if (c.next_tile >= count) { c.base[0] = c.base[1] = OOB; c.k0 = 0; return; }
+    if (!MN) {
+      const int srow = lane >> 3, pchunk = lane & 7;
+      const int row = wave * (16 * T) + srow;
+      klane[0] = (pchunk ^ srow) * 8; klane[1] = (pchunk ^ srow ^ 1) * 8;
+      const uint32_t rowoff = (uint32_t)(((int64_t)(origin + row) * ld) * 2);
+      c.base[0] = rowoff + klane[0] * 2; c.base[1] = rowoff + klane[1] * 2;
+    } else {
+      constexpr int RB = 128 * T;          // bytes per k-row of the tile
+      constexpr int CPR = RB / 16;         // chunks per k-row
+      constexpr int KPI = 1024 / RB;       // k-rows per issue
+      const int kb = wave * 16 + lane / CPR, pc = lane % CPR;
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const int k = kb + KPI * p;        // k-row of issue p within the stage; issue q is 2-periodic in k & 3 (KPI = 2) or constant (KPI = 4)
+        const int col = origin + 8 * (pc ^ mn_xor(k));
+        c.base[p] = col < extent ? (uint32_t)(((int64_t)kb * ld + col) * 2) : OOB;
+      }
+      klane[0] = klane[1] = 0;
+    }
+    c.k0 = 0;
+  };
+  int klaneA[2], klaneB[2];
+  const uint32_t qstepA = AMN ? (uint32_t)((1024 / (128 * TM)) * g.lda * 2) : (uint32_t)(g.lda * 16);
+  const uint32_t qstepB = BMN ? (uint32_t)((1024 / (128 * TN)) * g.ldb * 2) : (uint32_t)(g.ldb * 16);
+  const uint32_t kmulA = AMN ? (uint32_t)(g.lda * 2) : 2u, kmulB = BMN ? (uint32_t)(g.ldb * 2) : 2u;
+  Cursor ca, cb;
+  ca.next_tile = cb.next_tile = 0;
+  auto cursor_tile_a = [&]() {
+    int m0 = 0, n0 = 0;
+    if (ca.next_tile < count) tile_origin(first + ca.next_tile * stride, m0, n0);
+    setup(std::integral_constant<bool, AMN>{}, std::integral_constant<int, TM>{}, ca, m0, g.lda, M, klaneA);
+    ++ca.next_tile;
+  };
+  auto cursor_tile_b = [&]() {
+    int m0 = 0, n0 = 0;
+    if (cb.next_tile < count) tile_origin(first + cb.next_tile * stride, m0, n0);
+    setup(std::integral_constant<bool, BMN>{}, std::integral_constant<int, TN>{}, cb, n0, g.ldb, N, klaneB);
+    ++cb.next_tile;
+  };
+  cursor_tile_a();
+  cursor_tile_b();
+  auto issue_a = [&](int q, int buf) {
+    uint32_t off = ca.base[q & 1] + (uint32_t)q * qstepA + (uint32_t)ca.k0 * kmulA;
+    if (!AMN && ca.k0 + klaneA[q & 1] >= K) off = OOB;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsA, (lds_ptr)(sA + buf * STAGE_A + wave * (STAGE_A / 4) + q * 1024), 16, (int)off, 0, 0, 0);
+  };
+  auto issue_b = [&](int q, int buf) {
+    uint32_t off = cb.base[q & 1] + (uint32_t)q * qstepB + (uint32_t)cb.k0 * kmulB;
+    if (!BMN && cb.k0 + klaneB[q & 1] >= K) off = OOB;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsB, (lds_ptr)(sB + buf * STAGE_B + wave * (STAGE_B / 4) + q * 1024), 16, (int)off, 0, 0, 0);
+  };
+  // after the last issue of a stage the cursor moves one stage on; the pipeline below moves it to the workgroup's
+  // next tile (cursor_tile_*) between the stages where the loads cross a tile boundary
+  auto advance_a = [&]() { ca.k0 += GBK; };
+  auto advance_b = [&]() { cb.k0 += GBK; };
+
+  // ------------------------------------------------------------------ LDS -> fragments
+  // k-major fragment of sub-step s: ds_read_b128 of chunk 2s + lane/32 of row (32 i + lane%32): per-lane offsets per s.
+  // index-major fragment: two transposing reads; lane l (16-lane group gq = l/16, source role r = l%16) addresses the
+  // four rows m = 16 (gq & 1) + 4 (r & 3) .. +3 of k-row 16 s + 8 (gq >> 1) + 4 h + r / 4 (h = first / second read) and
+  // receives row 16 (gq & 1) + r of k-rows 16 s + 8 (l / 32) + 4 h .. +3: the k-values the k-major fragment of the
+  // other operand holds in the same order.
+  int fa_off[4], fb_off[4];  // k-major: per s; index-major: per i (or j)
+  {
+    const int f = (l32 & 7) ^ ((l32 >> 3) & 1);
+    const int gq = lane >> 4, r = lane & 15;
+    const int xl = mn_xor(r >> 2);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      if (!AMN) fa_off[s] = (wm + l32) * 128 + (((s * 2 + lhi) ^ f) << 4);
+      else fa_off[s] = s < TM ? ((8 * (gq >> 1) + (r >> 2)) * (128 * TM) + ((((wm >> 3) + 4 * s + 2 * (gq & 1) + ((r & 3) >> 1)) ^ xl) << 4) + (r & 1) * 8) : 0;
+      if (!BMN) fb_off[s] = (wn + l32) * 128 + (((s * 2 + lhi) ^ f) << 4);
+      else fb_off[s] = s < TN ? ((8 * (gq >> 1) + (r >> 2)) * (128 * TN) + ((((wn >> 3) + 4 * s + 2 * (gq & 1) + ((r & 3) >> 1)) ^ xl) << 4) + (r & 1) * 8) : 0;
+    }
+  }
+  auto read_tr = [&](const char* p) -> s4v { return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4p)(p)); };
+  auto read_a = [&](int buf, int s, int i) -> bf16x8 {
+    if (!AMN) return *(const bf16x8*)(sA + buf * STAGE_A + fa_off[s] + i * 4096);
+    const char* p = sA + buf * STAGE_A + fa_off[i] + s * (16 * 128 * TM);
+    const s4v lo = read_tr(p), hi = read_tr(p + 4 * 128 * TM);
+    const s8v v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
+  auto read_b = [&](int buf, int s, int j) -> bf16x8 {
+    if (!BMN) return *(const bf16x8*)(sB + buf * STAGE_B + fb_off[s] + j * 4096);
+    const char* p = sB + buf * STAGE_B + fb_off[j] + s * (16 * 128 * TN);
+    const s4v lo = read_tr(p), hi = read_tr(p + 4 * 128 * TN);
+    const s8v v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
+
+  f16v acc[TM][TN];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  };
+  zero_acc();
+
+  // the row pitch as a per-lane value the compiler cannot fold: row offsets are then made where they are used
+  // instead of as hundreds of scalars computed (and spilled) up front
+  uint32_t ldo_v = (uint32_t)g.ldo;
+  asm volatile("" : "+v"(ldo_v));
+
+  // B fragments are double-buffered; an A fragment's register is free again as soon as the last MFMA of its row of
+  // sub-tiles has been issued, so the A fragments of the next sub-step are read into the same registers.
+  bf16x8 fa[TM], fb[2][TN];
+#define SN_FENCE() __builtin_amdgcn_sched_barrier(0)
+  constexpr int NG = TM * TN / 2, PPR = TN / 2;
+  // One k sub-step: TM*TN MFMAs in pairs (row of sub-tiles by row) from A fragments fa and B fragment set CUR;
+  // behind each pair go this pair's share of the fragment reads for the next sub-step (buffer RBUF, sub-step RS:
+  // B fragment j behind pair j NG / TN, A fragment i behind the last pair of row i), of the stage loads of operand
+  // LOAD (0 none, 1 A, 2 B) into buffer LBUF.
+  auto substep = [&](auto CUR_, auto DO_READ_, auto RBUF_, auto RS_, auto LOAD_, auto LBUF_) {
+    constexpr int CUR = decltype(CUR_)::value, RBUF = decltype(RBUF_)::value, RS = decltype(RS_)::value;
+    constexpr int LOAD = decltype(LOAD_)::value, LBUF = decltype(LBUF_)::value;
+    constexpr bool DO_READ = decltype(DO_READ_)::value;
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi) {
+      const int i_ = gi / PPR, j_ = (gi % PPR) * 2;
+      acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i_], fb[CUR][j_], acc[i_][j_], 0, 0, 0);
+      acc[i_][j_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i_], fb[CUR][j_ + 1], acc[i_][j_ + 1], 0, 0, 0);
+      if constexpr (DO_READ) {
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+          if ((jj * NG) / TN == gi) fb[CUR ^ 1][jj] = read_b(RBUF, RS, jj);
+        if ((gi % PPR) == PPR - 1) fa[i_] = read_a(RBUF, RS, i_);
+      }
+      if constexpr (LOAD == 1) {
+#pragma unroll
+        for (int q_ = gi * (IA / NG); q_ < (gi + 1) * (IA / NG); ++q_) issue_a(q_, LBUF);
+      }
+      if constexpr (LOAD == 2) {
+#pragma unroll
+        for (int q_ = gi * (IB / NG); q_ < (gi + 1) * (IB / NG); ++q_) issue_b(q_, LBUF);
+      }
+      SN_FENCE();
+    }
+    if constexpr (LOAD == 1) advance_a();
+    if constexpr (LOAD == 2) advance_b();
+  };
+  // all of this wavefront's LDS-bound loads have landed, then everybody's
+  auto publish = [&]() {
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+  };
+  // One stage out of buffer BUF: sub-steps 0..3.  The barrier before sub-step 3 publishes the next stage (other
+  // buffer) and frees this one: the A half of the stage after next is loaded into it during sub-step 3, the B half
+  // during sub-step 0 of the next stage, one load behind every MFMA pair; sub-step 3 also reads the first fragments
+  // of the next stage.
+  auto stage = [&](auto BUF_) {
+    constexpr int BUF = decltype(BUF_)::value;
+    typedef std::integral_constant<int, 0> I0; typedef std::integral_constant<int, 1> I1; typedef std::integral_constant<int, 2> I2;
+    typedef std::integral_constant<int, 3> I3; typedef std::true_type Y;
+    typedef std::integral_constant<int, BUF> B; typedef std::integral_constant<int, BUF ^ 1> NB;
+    substep(I0{}, Y{}, B{}, I1{}, I2{}, NB{});
+    substep(I1{}, Y{}, B{}, I2{}, I0{}, I0{});
+    substep(I0{}, Y{}, B{}, I3{}, I0{}, I0{});
+    publish();
+    substep(I1{}, Y{}, NB{}, I0{}, I1{}, B{});
+  };
+
+  // ------------------------------------------------------------------ epilogues
+  // An accumulator value is fetched where it is used: left to itself the register allocator copies all 256 of them
+  // out of the accumulator file in front of the epilogue and spills everything else to make room.
+  auto acc_at = [&](int i, int j, int v) -> float {
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(acc[i][j][v]));
+    return x;
+  };
+  const float* bias = g.bias;
+  // MODE_F32: bias, activation, fp32 store (and the optional bf16 copy) straight from the accumulators
+  auto store_f32 = [&](int m0, int n0) {
+    const int row0 = m0 + wm + lhi * 4, col0 = n0 + wn + l32;
+    const uint32_t origin = (uint32_t)row0 * (uint32_t)g.ldo + (uint32_t)col0;
+    float* const out = g.out;
+    bf16* const obf = g.out_bf;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if (!FULL && col0 + j * 32 >= N) continue;
+      const float bj = bias ? bias[col0 + j * 32] : 0.f;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        __builtin_amdgcn_sched_barrier(0);  // keeps the scheduler from hoisting every sub-tile's address arithmetic to the top
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int r = i * 32 + (v >> 2) * 8 + (v & 3);
+          float x = acc_at(i, j, v);
+          if (FULL || row0 + r < M) {
+            if (bias) x = x + bj;
+            if (ACT == SN_ACT_RELU) x = fmaxf(g.relu_at, x);
+            const uint32_t at = origin + (uint32_t)r * ldo_v + j * 32;
+            if (out) out[at] = x;
+            if (obf) obf[at] = (bf16)x;
+          }
+        }
+      }
+    }
+  };
+  // MODE_BF16 / MODE_HANDOVER: bias, ReLU and its sign bits (or the ReLU gradient of the layer below and the column
+  // sums of what passes), the bf16 cast and two-byte stores, 64 contiguous bytes per row and instruction.
+  uint32_t sw[8];  // MODE_HANDOVER: the tile's sign words, requested one stage ahead of the epilogue
+  auto request_signs = [&](int t) {
+    if constexpr (MODE == MODE_HANDOVER) {
+      if (g.signs_in) {
+        const uint32_t* sp = g.signs_in + ((int64_t)(t * 4 + wave) * 8) * 64 + lane;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) sw[w] = sp[w * 64];
+      }
+    }
+  };
+  auto store_bf16 = [&](int t, int m0, int n0) {
+    if constexpr (MODE != MODE_F32) {
+      const uint32_t origin = (uint32_t)(m0 + wm + lhi * 4) * (uint32_t)g.ldo + (uint32_t)(n0 + wn + l32);
+      bf16* const o = g.out_bf;
+      const bool masked = MODE == MODE_HANDOVER && g.signs_in != nullptr;
+      uint32_t bits = 0;
+      float csum[TN][TM / 2];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const float bj = (MODE == MODE_BF16 && bias) ? bias[n0 + wn + l32 + j * 32] : 0.f;
+          uint32_t word = MODE == MODE_HANDOVER ? sw[(i * TN + j) >> 1] : 0u;
+          if (i % 2 == 0) csum[j][i / 2] = 0.f;
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            float x = acc_at(i, j, v);
+            if constexpr (MODE == MODE_BF16) {
+              if (bias) x = x + bj;
+              if (ACT == SN_ACT_RELU) {
+                // bits = 2 bits + (0 < x): the compare's lane mask is the add's carry-in
+                if (g.signs_out) asm volatile("v_cmp_lt_f32 vcc, 0, %1\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(bits) : "v"(x) : "vcc");
+                x = fmaxf(0.f, x);
+              }
+            } else {
+              // word += word shifts the next sign bit into the carry, which keeps or clears the value
+              if (masked) asm volatile("v_add_co_u32 %0, vcc, %0, %0\n\tv_cndmask_b32 %1, 0, %1, vcc" : "+v"(word), "+v"(x) : : "vcc");
+              csum[j][i / 2] += x;
+            }
+            o[origin + (uint32_t)(i * 32 + (v >> 2) * 8 + (v & 3)) * ldo_v + j * 32] = (bf16)x;
+          }
+          if constexpr (MODE == MODE_HANDOVER) sw[(i * TN + j) >> 1] = word;
+          if constexpr (MODE == MODE_BF16) {
+            if (ACT == SN_ACT_RELU && g.signs_out && ((i * TN + j) & 1)) {
+              g.signs_out[((int64_t)(t * 4 + wave) * 8 + ((i * TN + j) >> 1)) * 64 + lane] = bits;
+              bits = 0;
+            }
+          }
+        }
+      }
+      if constexpr (MODE == MODE_HANDOVER) {
+        if (g.col_partials) {  // the two half-waves hold 4 rows of every 8 each
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int b = 0; b < TM / 2; ++b) {
+              const float tsum = csum[j][b] + __shfl_xor(csum[j][b], 32, 64);
+              if (lhi == 0) g.col_partials[(int64_t)((m0 + wm) / 64 + b) * N + n0 + wn + l32 + j * 32] = tsum;
+            }
+        }
+      }
+    }
+  };
+
+  // ------------------------------------------------------------------ the pipeline
+  typedef std::integral_constant<int, 0> Z0;
+  typedef std::integral_constant<int, 1> Z1;
+  // first tile: stage 0 complete and the A half of stage 1 in flight, fragments of sub-step 0 read
+#pragma unroll
+  for (int q = 0; q < IA; ++q) issue_a(q, 0);
+  advance_a();
+#pragma unroll
+  for (int q = 0; q < IB; ++q) issue_b(q, 0);
+  advance_b();
+  publish();
+#pragma unroll
+  for (int q = 0; q < IA; ++q) issue_a(q, 1);
+  advance_a();
+#pragma unroll
+  for (int jj = 0; jj < TN; ++jj) fb[0][jj] = read_b(0, 0, jj);
+#pragma unroll
+  for (int ii = 0; ii < TM; ++ii) fa[ii] = read_a(0, 0, ii);
+  SN_FENCE();
+  // Stage kt loads the B half of stage kt + 1 and the A half of stage kt + 2, so in a tile's last pair of stages
+  // (nk - 2, nk - 1) every A load and the second B load belong to the next tile: the A cursor changes tile in front
+  // of that pair, the B cursor between its two stages.
+  if (nk == 2) cursor_tile_a();  // the prologue's second A load already was the next tile's
+  for (int it = 0; it < count; ++it) {
+    const int t = first + it * stride;
+    int m0, n0;
+    tile_origin(t, m0, n0);
+    for (int kp = 0; kp < nk / 2 - 1; ++kp) {
+      stage(Z0{});
+      stage(Z1{});
+    }
+    if (nk > 2) cursor_tile_a();
+    if (MODE == MODE_HANDOVER) request_signs(t);
+    stage(Z0{});
+    cursor_tile_b();
+    stage(Z1{});
+    if (nk == 2) cursor_tile_a();
+    // the first loads of the next tile are in flight while this one's results leave
+    if constexpr (MODE == MODE_F32) store_f32(m0, n0);
+    else store_bf16(t, m0, n0);
+    zero_acc();
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // the zero-filling loads past the last stage have landed before the workgroup leaves
+#undef SN_FENCE
+}
+
+template <int TM, int TN, bool AMN, bool BMN, int MODE, int ACT, bool FULL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_bf16_one(GemmBf16Args g) {  // one workgroup per CU: up to 512 registers per lane
+  gemm_bf16_body<TM, TN, AMN, BMN, MODE, ACT, FULL>(g);
+}
+template <int TM, int TN, bool AMN, bool BMN, int MODE, int ACT, bool FULL>
+__global__ __launch_bounds__(256, 2)
+void gemm_bf16_two(GemmBf16Args g) {  // two workgroups per CU (128 x 128 tiles)
+  gemm_bf16_body<TM, TN, AMN, BMN, MODE, ACT, FULL>(g);
+}
+
+template <int TM, int TN, bool AMN, bool BMN, int MODE, int ACT, bool FULL>
+static int launch_shape(sn_ctx* ctx, const GemmBf16Args& g0, const char* label) {
+  GemmBf16Args g = g0;
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  g.tiles_m = (int)ceil_div(g.M, BM);
+  g.tiles_n = (int)ceil_div(g.N, BN);
+  const int total = g.tiles_m * g.tiles_n;
+  const size_t smem = 2 * 128 * (BM + BN);
+  constexpr bool TWO = TM == 2 && TN == 2;
+  const int slots = ctx->compute_units * (TWO ? 2 : 1);
+  const int grid = total < slots ? total : slots;
+  if constexpr (TWO) {
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_two<TM, TN, AMN, BMN, MODE, ACT, FULL>, smem));
+    LaunchScope scope(ctx, label, g.M, g.N, g.K);
+    hipLaunchKernelGGL((gemm_bf16_two<TM, TN, AMN, BMN, MODE, ACT, FULL>), dim3((unsigned)grid), dim3(256), smem, ctx->stream, g);
+  } else {
+    SN_TRY(allow_dynamic_lds(ctx, (const void*)gemm_bf16_one<TM, TN, AMN, BMN, MODE, ACT, FULL>, smem));
+    LaunchScope scope(ctx, label, g.M, g.N, g.K);
+    hipLaunchKernelGGL((gemm_bf16_one<TM, TN, AMN, BMN, MODE, ACT, FULL>), dim3((unsigned)grid), dim3(256), smem, ctx->stream, g);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
 
-int launch_gemm_bf16_tn(sn_ctx* ctx, const void* a, int64_t lda, const void* bt, int64_t ldb, int M, int N, int K, const EpilogueBf16& ep) {
-  SN_REQUIRE(a && bt && (ep.e.out || ep.out_bf || ep.out_bf_t), "gemm_bf16: null operand");
-  SN_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0, "gemm_bf16: K and the row pitches must be multiples of 8 (got K=%d)", K);
-  SN_REQUIRE(((int64_t)M * lda + K) * 2 < (int64_t)1 << 31 && ((int64_t)N * ldb + K) * 2 < (int64_t)1 << 31,
-             "gemm_bf16: an operand of %d x %d / %d x %d bf16 exceeds the 2 GiB a buffer descriptor may span", M, K, N, K);
-  SN_REQUIRE((int64_t)M * ep.e.ldo < (int64_t)1 << 31 && (int64_t)N * ep.ld_t < (int64_t)1 << 31,
-             "gemm_bf16: output of %d rows x pitch %lld exceeds 2^31 elements", M, (long long)ep.e.ldo);
-  if (M <= 0 || N <= 0) return SN_OK;
-  const bf16* A = (const bf16*)a;
-  const bf16* B = (const bf16*)bt;
-  if (ep.grad_handover) {
-    SN_REQUIRE(M % 128 == 0 && N % 128 == 0 && ep.out_bf_t && ep.e.act == SN_ACT_IDENTITY && !ep.e.bias && ep.ld_t % 4 == 0,
-               "gemm_bf16: the gradient hand-over needs full 128 x 128 tiles, a transposed output and a plain product (got %d x %d)", M, N);
-    return launch_mode<MODE_HANDOVER>(ctx, A, lda, B, ldb, M, N, K, ep);
+// MODE_F32 for any shape: the largest tile that still gives every CU one, bounds-checked unless the 256 x 256 tiling is exact.
+template <bool AMN, bool BMN, int ACT>
+static int launch_f32(sn_ctx* ctx, const GemmBf16Args& g) {
+  const int cus = ctx->compute_units;
+  const int64_t t44 = ceil_div(g.M, 256) * ceil_div(g.N, 256), t24 = ceil_div(g.M, 128) * ceil_div(g.N, 256);
+  if (t44 >= cus) {
+    if (g.M % 256 == 0 && g.N % 256 == 0) return launch_shape<4, 4, AMN, BMN, MODE_F32, ACT, true>(ctx, g, "gemm_bf16_256x256");
+    return launch_shape<4, 4, AMN, BMN, MODE_F32, ACT, false>(ctx, g, "gemm_bf16_256x256");
   }
-  switch (ep.e.act) {
-    case SN_ACT_SIGMOID: return launch_mode<SN_ACT_SIGMOID>(ctx, A, lda, B, ldb, M, N, K, ep);
-    case SN_ACT_TANH: return launch_mode<SN_ACT_TANH>(ctx, A, lda, B, ldb, M, N, K, ep);
-    case SN_ACT_RELU: return launch_mode<SN_ACT_RELU>(ctx, A, lda, B, ldb, M, N, K, ep);
-    default: return launch_mode<SN_ACT_IDENTITY>(ctx, A, lda, B, ldb, M, N, K, ep);
-  }
+  if (t24 >= cus) return launch_shape<2, 4, AMN, BMN, MODE_F32, ACT, false>(ctx, g, "gemm_bf16_128x256");
+  return launch_shape<2, 2, AMN, BMN, MODE_F32, ACT, false>(ctx, g, "gemm_bf16_128x128");
 }
 
-// ---------------------------------------------------------------------------- fp32 -> bf16 in both orientations
-// out[r][c] and out_t[c][r] (either may be null) from src[r*ld + c]; when y != null the value cast is
-// the activation gradient act'(y) * src, which is also written back to dz (fp32) when dz != null.
-__global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __restrict__ src, int64_t ld, int rows, int cols,
-                                                              bf16* __restrict__ out, bf16* __restrict__ out_t,
-                                                              const float* __restrict__ y, const bf16* __restrict__ y_bf, int act,
-                                                              float act_param, float* __restrict__ dz, float* __restrict__ col_partials) {
-  // 64x64 tile; a thread handles 4 consecutive columns of 4 rows (float4 in, 8-byte bf16x4 out), and on the
-  // transposed side 4 consecutive rows of one column.  cols and rows are multiples of 4 (checked by the caller).
-  __shared__ bf16 tile[64][68];
+int launch_gemm_bf16(sn_ctx* ctx, int product, const void* a, int64_t lda, const void* b, int64_t ldb, int M, int N, int K,
+                     const EpilogueBf16& ep) {
+  SN_REQUIRE(a && b && (ep.e.out || ep.out_bf), "gemm_bf16: null operand");
+  SN_REQUIRE(product == GEMM_BF16_FORWARD || product == GEMM_BF16_DX || product == GEMM_BF16_DW, "gemm_bf16: unknown product %d", product);
+  const bool amn = product == GEMM_BF16_DW, bmn = product != GEMM_BF16_DX;
+  SN_REQUIRE(M % 8 == 0 && N % 8 == 0 && K % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0,
+             "gemm_bf16: M, N, K and the row pitches must be multiples of 8 (got %d x %d x %d)", M, N, K);
+  SN_REQUIRE(((amn ? (int64_t)K : (int64_t)M) * lda + 512) * 2 < (int64_t)1 << 31 && ((bmn ? (int64_t)K : (int64_t)N) * ldb + 512) * 2 < (int64_t)1 << 31,
+             "gemm_bf16: an operand of %d x %d x %d exceeds the 2 GiB a buffer descriptor may span", M, N, K);
+  SN_REQUIRE((int64_t)M * ep.e.ldo < (int64_t)1 << 31, "gemm_bf16: output of %d rows x pitch %lld exceeds 2^31 elements", M, (long long)ep.e.ldo);
+  SN_REQUIRE(ep.e.act == SN_ACT_IDENTITY || ep.e.act == SN_ACT_RELU, "gemm_bf16: only ReLU rides in the epilogue (got activation %d)", ep.e.act);
+  if (M <= 0 || N <= 0) return SN_OK;
+  GemmBf16Args g;
+  g.a = (const bf16*)a; g.b = (const bf16*)b; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N; g.K = K; g.tiles_m = g.tiles_n = 0;
+  g.out = ep.e.out; g.out_bf = (bf16*)ep.out_bf; g.ldo = ep.e.ldo; g.bias = ep.e.bias; g.relu_at = ep.e.act_param;
+  g.signs_out = (uint32_t*)ep.signs_out; g.signs_in = (const uint32_t*)ep.signs_in; g.col_partials = ep.col_partials;
+  const bool relu = ep.e.act == SN_ACT_RELU;
+  const bool tiles_256 = M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= ctx->compute_units;
+  if (ep.grad_handover) {
+    SN_REQUIRE(product == GEMM_BF16_DX && tiles_256 && g.out_bf && !g.out && !relu && !g.bias,
+               "gemm_bf16: the gradient hand-over needs a plain dX product on full 256 x 256 tiles (got %d x %d)", M, N);
+    return launch_shape<4, 4, false, false, MODE_HANDOVER, SN_ACT_IDENTITY, true>(ctx, g, "gemm_bf16_256x256_handover");
+  }
+  if (product == GEMM_BF16_FORWARD && !g.out && tiles_256 && (!relu || g.relu_at == 0.f)) {  // a hidden layer whose output lives as bf16 only
+    if (relu) return launch_shape<4, 4, false, true, MODE_BF16, SN_ACT_RELU, true>(ctx, g, "gemm_bf16_256x256_bf16out");
+    return launch_shape<4, 4, false, true, MODE_BF16, SN_ACT_IDENTITY, true>(ctx, g, "gemm_bf16_256x256_bf16out");
+  }
+  SN_REQUIRE(g.out != nullptr, "gemm_bf16: this shape needs an fp32 output (bf16-only results are for full 256 x 256 tiles)");
+  if (product == GEMM_BF16_FORWARD) return relu ? launch_f32<false, true, SN_ACT_RELU>(ctx, g) : launch_f32<false, true, SN_ACT_IDENTITY>(ctx, g);
+  SN_REQUIRE(!relu && !g.bias, "gemm_bf16: gradient products take no bias and no activation");
+  if (product == GEMM_BF16_DX) return launch_f32<false, false, SN_ACT_IDENTITY>(ctx, g);
+  return launch_f32<true, true, SN_ACT_IDENTITY>(ctx, g);
+}
+
+// true when a forward product of this shape can leave as bf16 only (and its dX counterpart can hand dZ over)
+bool gemm_bf16_full_tiles(const sn_ctx* ctx, int M, int N) {
+  return M % 256 == 0 && N % 256 == 0 && (int64_t)(M / 256) * (N / 256) >= ctx->compute_units;
+}
+
+// ---------------------------------------------------------------------------- fp32 -> bf16
+// out[r][c] from src[r*ld + c]; when y or y_bf is given the value cast is the activation gradient act'(y) * src
+// (also written back to dz in fp32 when dz != null); col_partials (optional, [ceil(rows/64), cols]) receives the
+// column sums of every 64-row block of the fp32 values.
+__global__ __launch_bounds__(256) void cast_bf16_kernel(const float* __restrict__ src, int64_t ld, int rows, int cols, bf16* __restrict__ out,
+                                                         const float* __restrict__ y, const bf16* __restrict__ y_bf, int act, float act_param,
+                                                         float* __restrict__ dz, float* __restrict__ col_partials) {
+  // 64x64 tile; a thread handles 4 consecutive columns of 4 rows (float4 in, 8-byte bf16x4 out).
   __shared__ float colp[16][64];
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const int tc = (threadIdx.x & 15) * 4, tr = threadIdx.x >> 4;
@@ -410,47 +568,33 @@ __global__ __launch_bounds__(256) void cast_transpose_kernel(const float* __rest
         for (int e = 0; e < 4; ++e) v[e] = bf_act_grad(act, yy[e], v[e], act_param);
         if (dz) *(f4*)(dz + (int64_t)r * ld + c) = v;
       }
-      bf16x4 b;
+      bf16x4 bq;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) b[e] = (bf16)v[e];
-      if (out) *(bf16x4*)(out + (int64_t)r * cols + c) = b;
+      for (int e = 0; e < 4; ++e) bq[e] = (bf16)v[e];
+      *(bf16x4*)(out + (int64_t)r * cols + c) = bq;
     }
     csum += v;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) tile[tr + 16 * i][tc + e] = (bf16)v[e];
   }
-  if (!out_t) return;
-  if (col_partials) {
+  if (!col_partials) return;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) colp[tr][tc + e] = csum[e];
-  }
+  for (int e = 0; e < 4; ++e) colp[tr][tc + e] = csum[e];
   __syncthreads();
-  if (col_partials && threadIdx.x < 64 && c0 + threadIdx.x < cols) {  // column sums of this 64-row block, rows in a fixed order
+  if (threadIdx.x < 64 && c0 + threadIdx.x < cols) {  // column sums of this 64-row block, rows in a fixed order
     float t = 0.f;
 #pragma unroll
     for (int j = 0; j < 16; ++j) t += colp[j][threadIdx.x];
     col_partials[(int64_t)blockIdx.y * cols + c0 + threadIdx.x] = t;
   }
-  if (!out_t) return;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = c0 + tr + 16 * i, r = r0 + tc;  // column c of the source, rows r..r+3
-    if (c < cols && r < rows) {
-      bf16x4 b;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) b[e] = tile[tc + e][tr + 16 * i];
-      *(bf16x4*)(out_t + (int64_t)c * rows + r) = b;
-    }
-  }
 }
 
-int launch_cast_transpose(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, void* out_t, const float* y,
-                          int act, float act_param, float* dz, float* col_partials, const void* y_bf) {
+int launch_cast_bf16(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, const float* y, int act, float act_param,
+                     float* dz, float* col_partials, const void* y_bf) {
   if (rows <= 0 || cols <= 0) return SN_OK;
+  SN_REQUIRE(out != nullptr, "cast_bf16: null output");
   SN_REQUIRE(rows % 4 == 0 && cols % 4 == 0 && ld % 4 == 0, "cast_bf16: rows, cols and pitch must be multiples of 4");
   LaunchScope scope(ctx, (y || y_bf) ? "activation_backward_cast_bf16" : "cast_bf16");
-  hipLaunchKernelGGL(cast_transpose_kernel, dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256), 0, ctx->stream,
-                     src, ld, rows, cols, (bf16*)out, (bf16*)out_t, y, (const bf16*)y_bf, act, act_param, dz, col_partials);
+  hipLaunchKernelGGL(cast_bf16_kernel, dim3((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(rows, 64)), dim3(256), 0, ctx->stream,
+                     src, ld, rows, cols, (bf16*)out, y, (const bf16*)y_bf, act, act_param, dz, col_partials);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

@@ -98,8 +98,10 @@ struct sn_replica {
   float* lstm_dh[2] = {nullptr, nullptr};
   float* lstm_dc = nullptr;
   float* lstm_dc2 = nullptr;  // the fused backward step reads the carried cell gradient from one buffer and writes the other
-  // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op, both orientations
-  std::vector<uint16_t*> bf_x, bf_xt, bf_dz, bf_dzt, bf_w, bf_wt;
+  // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op its input, its dZ and its weights as they lie,
+  // and one bit per output value where a hidden ReLU layer's output lives as bf16 only (the sign its gradient needs)
+  std::vector<uint16_t*> bf_x, bf_dz, bf_w;
+  std::vector<uint32_t*> bf_signs;
   std::vector<float*> bn_buf;  // per batch-norm op: mean, var, 1/sqrt(var+eps), scale, two gradient vectors
   float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
   bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
@@ -411,7 +413,13 @@ static bool hidden_f32_not_needed(const sn_model* m, size_t i) {
   return dense_bf16_fast(m, op) && dense_bf16_fast(m, m->ops[i + 1]) && sign_is_enough && m->batch % 8 == 0;
 }
 
-// The 256x256 bf16 kernel needs 16-byte chunks of 8 k-values in every operand row.
+// ... and does so for a pass over `rows` rows when the [rows, out] result tiles exactly into the 256 x 256 tiles whose
+// stores the bf16 kernel can park; the backward pass of the same rows then finds the layer's dZ handed over.
+static bool hidden_bf16_only(const sn_replica* r, size_t i, int rows) {
+  return hidden_f32_not_needed(r->model, i) && gemm_bf16_full_tiles(r->ctx, rows, (int)r->model->ops[i].out_elems);
+}
+
+// The bf16 kernel moves 16-byte chunks of 8 values along every operand row.
 static bool dense_bf16_fast(const sn_model* m, const Op& op) {
   return (m->flags & SN_FLAG_GEMM_BF16) && op.kind == OP_DENSE && op.in_elems % 8 == 0 && op.out_elems % 8 == 0 && m->batch % 8 == 0;
 }
@@ -440,8 +448,7 @@ static int alloc_replica(sn_replica* r) {
   r->lstm_pk_fwd.assign(n_ops, nullptr);
   r->lstm_pk_dh.assign(n_ops, nullptr);
   r->bn_buf.assign(n_ops, nullptr);
-  r->bf_x.assign(n_ops, nullptr); r->bf_xt.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr);
-  r->bf_dzt.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_wt.assign(n_ops, nullptr);
+  r->bf_x.assign(n_ops, nullptr); r->bf_dz.assign(n_ops, nullptr); r->bf_w.assign(n_ops, nullptr); r->bf_signs.assign(n_ops, nullptr);
   int64_t lstm_z = 0, lstm_h = 0, bf_colp = 0, lstm_parts = 4;
   for (size_t i = 0; i < n_ops; ++i) {
     const Op& op = m->ops[i];
@@ -474,11 +481,9 @@ static int alloc_replica(sn_replica* r) {
     if (op.kind == OP_POOL && !op.pool_avg) SN_TRY(dev_alloc(r, &r->arg[i], B * op.out_elems));
     if (dense_bf16_fast(m, op)) {
       SN_TRY(dev_alloc(r, &r->bf_x[i], B * op.in_elems));
-      SN_TRY(dev_alloc(r, &r->bf_xt[i], B * op.in_elems));
       SN_TRY(dev_alloc(r, &r->bf_dz[i], B * op.out_elems));
-      SN_TRY(dev_alloc(r, &r->bf_dzt[i], B * op.out_elems));
       SN_TRY(dev_alloc(r, &r->bf_w[i], op.in_elems * op.out_elems));
-      SN_TRY(dev_alloc(r, &r->bf_wt[i], op.in_elems * op.out_elems));
+      if (hidden_f32_not_needed(m, i) && op.act == SN_ACT_RELU) SN_TRY(dev_alloc(r, &r->bf_signs[i], ceil_div(B * op.out_elems, 32)));
       bf_colp = std::max(bf_colp, ceil_div(B, 64) * op.out_elems);
     }
   }
@@ -535,8 +540,8 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
   if (bf16 && r->bf_weights_stale) {
     for (size_t i = 0; i < m->ops.size(); ++i)
       if (dense_bf16_fast(m, m->ops[i]))
-        SN_TRY(launch_cast_transpose(ctx, param_ptr(r, r->w, m->ops[i].w), m->ops[i].out_elems, (int)m->ops[i].in_elems,
-                                     (int)m->ops[i].out_elems, r->bf_w[i], r->bf_wt[i], nullptr, 0, 0.f, nullptr));
+        SN_TRY(launch_cast_bf16(ctx, param_ptr(r, r->w, m->ops[i].w), m->ops[i].out_elems, (int)m->ops[i].in_elems,
+                                (int)m->ops[i].out_elems, r->bf_w[i], nullptr, 0, 0.f, nullptr));
     r->bf_weights_stale = false;
   }
   std::vector<char> bf_ready(m->ops.size() + 1, 0);  // op i's bf16 input copies were written by op i-1's epilogue
@@ -549,19 +554,22 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         Epilogue ep;
         ep.out = r->act[i]; ep.ldo = out_f; ep.bias = param_ptr(r, r->w, op.b); ep.act = op.act; ep.act_param = op.act_param;
         if (dense_bf16_fast(m, op) && rows % 8 == 0) {
-          // X in both orientations (X^T feeds dW later) unless the layer below already wrote them from its
-          // epilogue, then Y = X . (W^T)^T on the matrix cores
-          if (!bf_ready[i]) SN_TRY(launch_cast_transpose(ctx, in, in_f, rows, in_f, r->bf_x[i], r->bf_xt[i], nullptr, 0, 0.f, nullptr));
+          // the bf16 copy of X unless the layer below already wrote it from its epilogue, then Y = X . W on the matrix cores
+          if (!bf_ready[i]) SN_TRY(launch_cast_bf16(ctx, in, in_f, rows, in_f, r->bf_x[i], nullptr, 0, 0.f, nullptr));
           EpilogueBf16 eb;
           eb.e = ep;
-          if (i + 1 < m->ops.size() && dense_bf16_fast(m, m->ops[i + 1])) {
+          const bool in_kernel_act = op.act == SN_ACT_IDENTITY || op.act == SN_ACT_RELU;
+          if (!in_kernel_act) { eb.e.bias = nullptr; eb.e.act = SN_ACT_IDENTITY; }  // sigmoid / tanh: a pass of their own below
+          if (in_kernel_act && i + 1 < m->ops.size() && dense_bf16_fast(m, m->ops[i + 1])) {
             eb.out_bf = r->bf_x[i + 1];
-            eb.out_bf_t = r->bf_xt[i + 1];
-            eb.ld_t = rows;
             bf_ready[i + 1] = true;
-            if (hidden_f32_not_needed(m, i)) eb.e.out = nullptr;  // the next layer and the backward pass read the bf16 copies
+            if (hidden_bf16_only(r, i, rows)) {  // the next layer and the backward pass read the bf16 copy and the sign bits
+              eb.e.out = nullptr;
+              eb.signs_out = r->bf_signs[i];
+            }
           }
-          SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_x[i], in_f, r->bf_wt[i], in_f, rows, out_f, in_f, eb));
+          SN_TRY(launch_gemm_bf16(ctx, GEMM_BF16_FORWARD, r->bf_x[i], in_f, r->bf_w[i], out_f, rows, out_f, in_f, eb));
+          if (!in_kernel_act) SN_TRY(launch_bias_act(ctx, r->act[i], ep.bias, r->act[i], rows, out_f, op.act, op.act_param));
         } else if (!bf16 && dense_tiny_shape(rows, in_f, out_f, m->workspace_elems)) {  // a few units behind a short row: one launch
           SN_TRY(launch_dense_tiny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f));
         } else if (!bf16 && r->ws && dense_skinny_fwd_shape(rows, in_f, out_f, m->workspace_elems)) {
@@ -705,39 +713,36 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
       case OP_DENSE: {
         const int in_f = (int)op.in_elems, out_f = (int)op.out_elems;
         if (dense_bf16_fast(m, op) && rows % 8 == 0) {
-          // one pass: dZ = act'(Y) * dY in fp32 (bias gradient) and as bf16 in both orientations
-          // (the fp32 dZ itself is not kept: its only other reader would be the bias gradient, summed here per 64-row block)
-          const bool y_from_bf = hidden_f32_not_needed(m, (size_t)i);
+          // one pass: dZ = act'(Y) * dY as bf16 (the fp32 dZ itself is not kept: its only other reader would be the bias
+          // gradient, summed here per 64-row block from the fp32 values)
+          const bool y_from_bf = hidden_bf16_only(r, (size_t)i, rows);
           if (!dz_handed_over)
-            SN_TRY(launch_cast_transpose(ctx, dy, out_f, rows, out_f, r->bf_dz[i], r->bf_dzt[i],
-                                         op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
-                                         op.b >= 0 ? r->bf_colp : nullptr,
-                                         op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
+            SN_TRY(launch_cast_bf16(ctx, dy, out_f, rows, out_f, r->bf_dz[i],
+                                    op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
+                                    op.b >= 0 ? r->bf_colp : nullptr,
+                                    op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
           dz_handed_over = false;
           if (op.b >= 0)
             SN_TRY(launch_col_sum(ctx, r->bf_colp, out_f, param_ptr(r, r->g, op.b), ceil_div(rows, 64), out_f, r->ws, m->workspace_elems));
           EpilogueBf16 ew;
           ew.e.out = param_ptr(r, r->g, op.w); ew.e.ldo = out_f;
-          SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_xt[i], rows, r->bf_dzt[i], rows, in_f, out_f, rows, ew));  // dW = X^T . dZ
+          SN_TRY(launch_gemm_bf16(ctx, GEMM_BF16_DW, r->bf_x[i], in_f, r->bf_dz[i], out_f, in_f, out_f, rows, ew));  // dW = X^T . dZ
           if (need_dx) {
             EpilogueBf16 ex;
             ex.e.out = dx; ex.e.ldo = in_f;
-            // A bf16 Dense layer below whose output only lives as bf16 copies (ReLU or no activation) takes its dZ straight
-            // from this product's epilogue: activation gradient, both bf16 orientations and the bias gradient's block sums,
-            // instead of an fp32 dX that a second kernel would read back, mask and cast.
-            if (hidden_f32_not_needed(m, (size_t)i - 1) && rows % 128 == 0 && in_f % 128 == 0) {
+            // A bf16 Dense layer below whose output only lives as a bf16 copy (ReLU at 0 or no activation) takes its dZ
+            // straight from this product's epilogue: activation gradient, the bf16 cast and the bias gradient's block
+            // sums, instead of an fp32 dX that a second kernel would read back, mask and cast.
+            if (i > 0 && hidden_bf16_only(r, (size_t)i - 1, rows)) {
               const Op& below = m->ops[i - 1];
               ex.e.out = nullptr;
               ex.out_bf = r->bf_dz[i - 1];
-              ex.out_bf_t = r->bf_dzt[i - 1];
-              ex.ld_t = rows;
               ex.grad_handover = true;
-              ex.grad_mask_t = below.act == SN_ACT_RELU ? r->bf_xt[i] : nullptr;
-              ex.e.act_param = below.act_param;
+              ex.signs_in = below.act == SN_ACT_RELU ? r->bf_signs[i - 1] : nullptr;
               ex.col_partials = below.b >= 0 ? r->bf_colp : nullptr;
               dz_handed_over = true;
             }
-            SN_TRY(launch_gemm_bf16_tn(ctx, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
+            SN_TRY(launch_gemm_bf16(ctx, GEMM_BF16_DX, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
             cur ^= 1;
           }
           break;
@@ -1050,6 +1055,7 @@ static int tensor_io(sn_replica* r, float* base, int index, float* host, const f
   } else {
     SN_HIP(hipMemcpyAsync(host, base + p.offset, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, r->ctx->stream));
     SN_HIP(hipStreamSynchronize(r->ctx->stream));
+    return check_async(r->ctx);  // what was read may come from a pass whose one-launch recurrent kernel gave up
   }
   return SN_OK;
 }
@@ -1349,6 +1355,7 @@ int sn_count_correct(sn_replica* rep, const float* x_dev, const float* y_dev, in
   unsigned long long c = 0;
   SN_HIP(hipMemcpyAsync(&c, rep->count_dev, sizeof(c), hipMemcpyDeviceToHost, rep->ctx->stream));
   SN_HIP(hipStreamSynchronize(rep->ctx->stream));
+  SN_TRY(check_async(rep->ctx));
   *count_host = (int64_t)c;
   return SN_OK;
 }
