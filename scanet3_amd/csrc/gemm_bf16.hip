@@ -57,6 +57,85 @@ __device__ __forceinline__ float bf_act_grad(int act, float y, float dy, float p
   }
 }
 
+// One transposing read, written as assembly: the compiler puts `s_waitcnt vmcnt(0)` in front of the builtin form
+// whenever an LDS-bound global load is in flight (it cannot tell which one the read depends on), which would end the
+// overlap of loads and matrix work.  The result is valid only after the `s_waitcnt lgkmcnt` the kernel issues itself.
+// offset = BUF * STAGE + S * 16 * RB + H * 4 * RB must be an immediate: one case per (buffer, sub-step, half).
+template <int RB, int STAGE>
+__device__ __forceinline__ s4v tr_read(uint32_t addr, int buf, int s, int h) {
+  s4v v;
+#define SN_TR_CASE(B, S, H) \
+  case ((B) * 8 + (S) * 2 + (H)): asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"((B) * STAGE + (S) * 16 * RB + (H) * 4 * RB)); break;
+  switch (buf * 8 + s * 2 + h) {
+    SN_TR_CASE(0, 0, 0) SN_TR_CASE(0, 0, 1) SN_TR_CASE(0, 1, 0) SN_TR_CASE(0, 1, 1) SN_TR_CASE(0, 2, 0) SN_TR_CASE(0, 2, 1) SN_TR_CASE(0, 3, 0) SN_TR_CASE(0, 3, 1)
+    SN_TR_CASE(1, 0, 0) SN_TR_CASE(1, 0, 1) SN_TR_CASE(1, 1, 0) SN_TR_CASE(1, 1, 1) SN_TR_CASE(1, 2, 0) SN_TR_CASE(1, 2, 1) SN_TR_CASE(1, 3, 0) SN_TR_CASE(1, 3, 1)
+    default: __builtin_unreachable();
+  }
+#undef SN_TR_CASE
+  return v;
+}
+// s_waitcnt lgkmcnt(N) that the fragment halves named as operands are ordered behind
+template <int N> __device__ __forceinline__ void wait_lgkm(s4v& a, s4v& b) {
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void wait_lgkm(s4v& a, s4v& b, s4v& c, s4v& d) {
+  asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) : "n"(N));
+}
+template <int N> __device__ __forceinline__ void wait_lgkm(s4v& a, s4v& b, s4v& c, s4v& d, s4v& e, s4v& f) {
+  asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f) : "n"(N));
+}
+template <typename... T>
+__device__ __forceinline__ void wait_lgkm_n(int n, T&... h) {
+  switch (n) {
+    case 0: wait_lgkm<0>(h...); break;   case 1: wait_lgkm<1>(h...); break;   case 2: wait_lgkm<2>(h...); break;
+    case 3: wait_lgkm<3>(h...); break;   case 4: wait_lgkm<4>(h...); break;   case 5: wait_lgkm<5>(h...); break;
+    case 6: wait_lgkm<6>(h...); break;   case 7: wait_lgkm<7>(h...); break;   case 8: wait_lgkm<8>(h...); break;
+    case 9: wait_lgkm<9>(h...); break;   case 10: wait_lgkm<10>(h...); break; case 11: wait_lgkm<11>(h...); break;
+    case 12: wait_lgkm<12>(h...); break; case 13: wait_lgkm<13>(h...); break; case 14: wait_lgkm<14>(h...); break;
+    default: wait_lgkm<15>(h...); break;
+  }
+}
+
+// The fragment reads of a sub-step, in issue order: behind MFMA pair g first the B fragments j with j NG / TN == g,
+// then A fragment i if g is the last pair of row i.  wait_before(g) = how many transposing reads (two per
+// index-major fragment; the compiler keeps its own count for k-major ones) may still be in flight when pair g of the
+// NEXT sub-step starts, such that the index-major fragments that pair multiplies have landed; -1: nothing to wait
+// for, or an earlier pair of the sub-step already waited for as much.
+template <int TM, int TN, bool AMN, bool BMN>
+struct FragSchedule {
+  static constexpr int NG = TM * TN / 2, PPR = TN / 2;
+  // position in issue order of A fragment i / B fragment j, and the number of transposing reads issued up to and
+  // including each position
+  static constexpr int pos_a(int i) { int p = 0; for (int g = 0; g < NG; ++g) { for (int j = 0; j < TN; ++j) if ((j * NG) / TN == g) ++p; if (g % PPR == PPR - 1) { if (g / PPR == i) return p; ++p; } } return -1; }
+  static constexpr int pos_b(int jq) { int p = 0; for (int g = 0; g < NG; ++g) { for (int j = 0; j < TN; ++j) if ((j * NG) / TN == g) { if (j == jq) return p; ++p; } if (g % PPR == PPR - 1) ++p; } return -1; }
+  static constexpr int reads_through(int pos) {  // transposing reads issued at positions 0 .. pos
+    int p = 0, n = 0;
+    for (int g = 0; g < NG; ++g) { for (int j = 0; j < TN; ++j) if ((j * NG) / TN == g) { if (p <= pos && BMN) n += 2; ++p; } if (g % PPR == PPR - 1) { if (p <= pos && AMN) n += 2; ++p; } }
+    return n;
+  }
+  static constexpr int reads_in_groups_before(int gi) {  // transposing reads issued behind pairs 0 .. gi-1
+    int n = 0;
+    for (int g = 0; g < gi; ++g) { for (int j = 0; j < TN; ++j) if ((j * NG) / TN == g && BMN) n += 2; if (g % PPR == PPR - 1 && AMN) n += 2; }
+    return n;
+  }
+  static constexpr int latest_needed(int gi) {  // last position among the index-major fragments pair gi multiplies, -1 if none
+    const int i = gi / PPR, j = (gi % PPR) * 2;
+    int latest = -1;
+    if (AMN && pos_a(i) > latest) latest = pos_a(i);
+    if (BMN && pos_b(j) > latest) latest = pos_b(j);
+    if (BMN && pos_b(j + 1) > latest) latest = pos_b(j + 1);
+    return latest;
+  }
+  static constexpr int wait_before(int gi) {
+    const int latest = latest_needed(gi);
+    if (latest < 0) return -1;
+    for (int g = 0; g < gi; ++g) if (latest_needed(g) >= latest) return -1;
+    const int total = reads_through(TM + TN - 1);
+    const int n = (total - reads_through(latest)) + reads_in_groups_before(gi);
+    return n > 15 ? 15 : n;
+  }
+};
+
 // Epilogue modes (compile-time).
 constexpr int MODE_F32 = 0;       // fp32 result (+ bias, ReLU), optionally a bf16 copy; any shape (bounds-checked unless FULL)
 constexpr int MODE_BF16 = 1;      // bf16 result only (+ bias, ReLU at 0) and the ReLU's sign bits, full tiles
@@ -211,21 +290,11 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmBf16Args& g) {
       else fb_off[s] = s < TN ? ((8 * (gq >> 1) + (r >> 2)) * (128 * TN) + ((((wn >> 3) + 4 * s + 2 * (gq & 1) + ((r & 3) >> 1)) ^ xl) << 4) + (r & 1) * 8) : 0;
     }
   }
-  auto read_tr = [&](const char* p) -> s4v { return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4p)(p)); };
-  auto read_a = [&](int buf, int s, int i) -> bf16x8 {
-    if (!AMN) return *(const bf16x8*)(sA + buf * STAGE_A + fa_off[s] + i * 4096);
-    const char* p = sA + buf * STAGE_A + fa_off[i] + s * (16 * 128 * TM);
-    const s4v lo = read_tr(p), hi = read_tr(p + 4 * 128 * TM);
-    const s8v v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, v);
-  };
-  auto read_b = [&](int buf, int s, int j) -> bf16x8 {
-    if (!BMN) return *(const bf16x8*)(sB + buf * STAGE_B + fb_off[s] + j * 4096);
-    const char* p = sB + buf * STAGE_B + fb_off[j] + s * (16 * 128 * TN);
-    const s4v lo = read_tr(p), hi = read_tr(p + 4 * 128 * TN);
-    const s8v v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, v);
-  };
+  const uint32_t lds_a = (uint32_t)(size_t)(lds_ptr)sA, lds_b = (uint32_t)(size_t)(lds_ptr)sB;
+  auto read_a_km = [&](int buf, int s, int i) -> bf16x8 { return *(const bf16x8*)(sA + buf * STAGE_A + fa_off[s] + i * 4096); };
+  auto read_b_km = [&](int buf, int s, int j) -> bf16x8 { return *(const bf16x8*)(sB + buf * STAGE_B + fb_off[s] + j * 4096); };
+  auto read_a_mn = [&](int buf, int s, int i, int h) -> s4v { return tr_read<128 * TM, STAGE_A>(lds_a + fa_off[i], buf, s, h); };
+  auto read_b_mn = [&](int buf, int s, int j, int h) -> s4v { return tr_read<128 * TN, STAGE_B>(lds_b + fb_off[j], buf, s, h); };
 
   f16v acc[TM][TN];
   auto zero_acc = [&]() {
@@ -245,12 +314,19 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmBf16Args& g) {
 
   // B fragments are double-buffered; an A fragment's register is free again as soon as the last MFMA of its row of
   // sub-tiles has been issued, so the A fragments of the next sub-step are read into the same registers.
-  bf16x8 fa[TM], fb[2][TN];
+  // k-major fragments as the compiler's own loads; index-major ones as the two halves the transposing reads deliver
+  bf16x8 fa[AMN ? 1 : TM], fb[2][BMN ? 1 : TN];
+  s4v fa_lo[AMN ? TM : 1], fa_hi[AMN ? TM : 1], fb_lo[2][BMN ? TN : 1], fb_hi[2][BMN ? TN : 1];
+  auto frag_of = [&](const s4v& lo, const s4v& hi) -> bf16x8 {
+    const s8v v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+  };
 #define SN_FENCE() __builtin_amdgcn_sched_barrier(0)
   constexpr int NG = TM * TN / 2, PPR = TN / 2;
-  // One k sub-step: TM*TN MFMAs in pairs (row of sub-tiles by row) from A fragments fa and B fragment set CUR;
+  typedef FragSchedule<TM, TN, AMN, BMN> Sched;
+  // One k sub-step: TM*TN MFMAs in pairs (row of sub-tiles by row) from the A fragments and B fragment set CUR;
   // behind each pair go this pair's share of the fragment reads for the next sub-step (buffer RBUF, sub-step RS:
-  // B fragment j behind pair j NG / TN, A fragment i behind the last pair of row i), of the stage loads of operand
+  // B fragment j behind pair j NG / TN, A fragment i behind the last pair of row i) and of the stage loads of operand
   // LOAD (0 none, 1 A, 2 B) into buffer LBUF.
   auto substep = [&](auto CUR_, auto DO_READ_, auto RBUF_, auto RS_, auto LOAD_, auto LBUF_) {
     constexpr int CUR = decltype(CUR_)::value, RBUF = decltype(RBUF_)::value, RS = decltype(RS_)::value;
@@ -259,13 +335,30 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmBf16Args& g) {
 #pragma unroll
     for (int gi = 0; gi < NG; ++gi) {
       const int i_ = gi / PPR, j_ = (gi % PPR) * 2;
-      acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i_], fb[CUR][j_], acc[i_][j_], 0, 0, 0);
-      acc[i_][j_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i_], fb[CUR][j_ + 1], acc[i_][j_ + 1], 0, 0, 0);
+      if constexpr (AMN || BMN) {
+        const int w = Sched::wait_before(gi);
+        if (w >= 0) {
+          if constexpr (AMN && BMN) wait_lgkm_n(w, fa_lo[i_], fa_hi[i_], fb_lo[CUR][j_], fb_hi[CUR][j_], fb_lo[CUR][j_ + 1], fb_hi[CUR][j_ + 1]);
+          else if constexpr (AMN) wait_lgkm_n(w, fa_lo[i_], fa_hi[i_]);
+          else wait_lgkm_n(w, fb_lo[CUR][j_], fb_hi[CUR][j_], fb_lo[CUR][j_ + 1], fb_hi[CUR][j_ + 1]);
+        }
+      }
+      const bf16x8 av = AMN ? frag_of(fa_lo[AMN ? i_ : 0], fa_hi[AMN ? i_ : 0]) : fa[AMN ? 0 : i_];
+      const bf16x8 bv0 = BMN ? frag_of(fb_lo[CUR][BMN ? j_ : 0], fb_hi[CUR][BMN ? j_ : 0]) : fb[CUR][BMN ? 0 : j_];
+      const bf16x8 bv1 = BMN ? frag_of(fb_lo[CUR][BMN ? j_ + 1 : 0], fb_hi[CUR][BMN ? j_ + 1 : 0]) : fb[CUR][BMN ? 0 : j_ + 1];
+      acc[i_][j_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv0, acc[i_][j_], 0, 0, 0);
+      acc[i_][j_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv1, acc[i_][j_ + 1], 0, 0, 0);
       if constexpr (DO_READ) {
 #pragma unroll
         for (int jj = 0; jj < TN; ++jj)
-          if ((jj * NG) / TN == gi) fb[CUR ^ 1][jj] = read_b(RBUF, RS, jj);
-        if ((gi % PPR) == PPR - 1) fa[i_] = read_a(RBUF, RS, i_);
+          if ((jj * NG) / TN == gi) {
+            if constexpr (BMN) { fb_lo[CUR ^ 1][jj] = read_b_mn(RBUF, RS, jj, 0); fb_hi[CUR ^ 1][jj] = read_b_mn(RBUF, RS, jj, 1); }
+            else fb[CUR ^ 1][jj] = read_b_km(RBUF, RS, jj);
+          }
+        if ((gi % PPR) == PPR - 1) {
+          if constexpr (AMN) { fa_lo[i_] = read_a_mn(RBUF, RS, i_, 0); fa_hi[i_] = read_a_mn(RBUF, RS, i_, 1); }
+          else fa[i_] = read_a_km(RBUF, RS, i_);
+        }
       }
       if constexpr (LOAD == 1) {
 #pragma unroll
@@ -420,9 +513,16 @@ __device__ __forceinline__ void gemm_bf16_body(const GemmBf16Args& g) {
   for (int q = 0; q < IA; ++q) issue_a(q, 1);
   advance_a();
 #pragma unroll
-  for (int jj = 0; jj < TN; ++jj) fb[0][jj] = read_b(0, 0, jj);
+  for (int jj = 0; jj < TN; ++jj) {
+    if constexpr (BMN) { fb_lo[0][jj] = read_b_mn(0, 0, jj, 0); fb_hi[0][jj] = read_b_mn(0, 0, jj, 1); }
+    else fb[0][jj] = read_b_km(0, 0, jj);
+  }
 #pragma unroll
-  for (int ii = 0; ii < TM; ++ii) fa[ii] = read_a(0, 0, ii);
+  for (int ii = 0; ii < TM; ++ii) {
+    if constexpr (AMN) { fa_lo[ii] = read_a_mn(0, 0, ii, 0); fa_hi[ii] = read_a_mn(0, 0, ii, 1); }
+    else fa[ii] = read_a_km(0, 0, ii);
+  }
+  if constexpr (AMN || BMN) __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the steady-state waits count from a full sub-step of reads
   SN_FENCE();
   // Stage kt loads the B half of stage kt + 1 and the A half of stage kt + 2, so in a tile's last pair of stages
   // (nk - 2, nk - 1) every A load and the second B load belong to the next tile: the A cursor changes tile in front
