@@ -290,7 +290,7 @@ def bench_wide_mlp(S, ctx, steps, warmup, bf16=True):
         S, ctx, "MLP 4096->4096 relu->4096 relu->1000 softmax, batch 8192, Adam 1e-3, " + ("bf16 MFMA / fp32 acc" if bf16 else "fp32"),
         S.Dense(4096, S.ReLU()) >> S.Dense(4096, S.ReLU()) >> S.Dense(1000, S.Softmax),
         S.CategoricalCrossentropy, (4096,), 8192, S.Adam(1e-3),
-        lambda rng, n: (rng.standard_normal((n, 4096)).astype(np.float32), one_hot(rng, n, 1000)), 1, steps, warmup,
+        lambda rng, n: (rng.standard_normal((n, 4096)).astype(np.float32), one_hot(rng, n, 1000)), 4, steps, warmup,
         flags=L.FLAG_GEMM_BF16 if bf16 else 0)
 
 

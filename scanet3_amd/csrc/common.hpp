@@ -131,8 +131,9 @@ struct OptScalars {
 };
 OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter);
 int opt_state_count(int kind);
+// wbf (optional): the updated weights are also written as bf16, element for element
 int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
-                     int64_t n, int iter);
+                     int64_t n, int iter, void* wbf = nullptr);
 struct AvgInputs {
   const float* p[SN_MAX_AVG_INPUTS];
 };

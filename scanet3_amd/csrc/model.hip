@@ -100,7 +100,8 @@ struct sn_replica {
   float* lstm_dc2 = nullptr;  // the fused backward step reads the carried cell gradient from one buffer and writes the other
   // bf16 operand copies of the Dense layers (SN_FLAG_GEMM_BF16): per op its input, its dZ and its weights as they lie,
   // and one bit per output value where a hidden ReLU layer's output lives as bf16 only (the sign its gradient needs)
-  std::vector<uint16_t*> bf_x, bf_dz, bf_w;
+  std::vector<uint16_t*> bf_x, bf_dz, bf_w;  // bf_w[i] points into bf_wflat
+  uint16_t* bf_wflat = nullptr;              // bf16 copy of the flat parameter buffer (same offsets), written by the optimizer
   std::vector<uint32_t*> bf_signs;
   std::vector<float*> bn_buf;  // per batch-norm op: mean, var, 1/sqrt(var+eps), scale, two gradient vectors
   float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
@@ -482,12 +483,16 @@ static int alloc_replica(sn_replica* r) {
     if (dense_bf16_fast(m, op)) {
       SN_TRY(dev_alloc(r, &r->bf_x[i], B * op.in_elems));
       SN_TRY(dev_alloc(r, &r->bf_dz[i], B * op.out_elems));
-      SN_TRY(dev_alloc(r, &r->bf_w[i], op.in_elems * op.out_elems));
       if (hidden_f32_not_needed(m, i) && op.act == SN_ACT_RELU) SN_TRY(dev_alloc(r, &r->bf_signs[i], ceil_div(B * op.out_elems, 32)));
       bf_colp = std::max(bf_colp, ceil_div(B, 64) * op.out_elems);
     }
   }
   SN_TRY(dev_alloc(r, &r->bf_colp, bf_colp));
+  if (m->flags & SN_FLAG_GEMM_BF16) {
+    SN_TRY(dev_alloc(r, &r->bf_wflat, m->flat_elems));
+    for (size_t i = 0; i < n_ops; ++i)
+      if (dense_bf16_fast(m, m->ops[i])) r->bf_w[i] = r->bf_wflat + m->params[m->ops[i].w].info.offset;
+  }
   SN_TRY(dev_alloc(r, &r->lstm_z, lstm_z));
   SN_TRY(dev_alloc(r, &r->lstm_dh[0], lstm_h * lstm_parts));  // partial sums of the hidden gradient: per gate, or per slice of units
   SN_TRY(dev_alloc(r, &r->lstm_dh[1], lstm_h * lstm_parts));
@@ -1013,13 +1018,14 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bo
 
 static int update(sn_replica* r, int iter) {
   SN_REQUIRE(r->has_opt, "replica was created without an optimizer");
-  r->bf_weights_stale = true;
   sn_model* m = r->model;
   // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
-  // the statistics are those of the gradient pass that has just run
+  // the statistics are those of the gradient pass that has just run.  In bf16 mode the optimizer writes the bf16 copy of
+  // what it updates in the same pass (every Dense weight is trainable), so the copies stay current.
   for (const auto& run : m->trainable_runs)
     SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,
-                            r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter));
+                            r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter,
+                            r->bf_wflat ? r->bf_wflat + run.first : nullptr));
   for (size_t i = 0; i < m->ops.size(); ++i) {
     const Op& op = m->ops[i];
     if (op.kind == OP_BATCHNORM)

@@ -104,10 +104,12 @@ constexpr int n_states() {
 // A block owns T*U consecutive float4 of every array and touches ONE ARRAY AT A TIME: U loads of w,
 // then U of g, ... then the stores array by array (measured on MI355X: 6.1 TB/s for Adam's 4 read + 3 write
 // streams where the element-interleaved order reaches 5.6 TB/s).
-template <int KIND, int U, int T>
+// WBF: the updated weights also leave as bf16 (wbf, same element order), for the bf16 matrix products of the next pass.
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+template <int KIND, int U, int T, bool WBF>
 __global__ __launch_bounds__(T) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
                                                             f4* __restrict__ s1, f4* __restrict__ s2, int64_t n4,
-                                                            OptScalars p) {
+                                                            OptScalars p, bf16x4_t* __restrict__ wbf) {
   constexpr int NS = n_states<KIND>();
   const int64_t base = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
   if (U == 1 && base >= n4) return;  // one vector per thread: one early exit instead of a check around every access
@@ -147,6 +149,16 @@ __global__ __launch_bounds__(T) void optimizer_kernel_v4(f4* __restrict__ w, con
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (SN_IN_RANGE(u)) __builtin_nontemporal_store(vw[u], w + base + u * T);
+  if (WBF) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (SN_IN_RANGE(u)) {
+        bf16x4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = (__bf16)vw[u][e];
+        wbf[base + u * T] = h;
+      }
+  }
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (SN_IN_RANGE(u)) __builtin_nontemporal_store(a[u], s0 + base + u * T);
@@ -167,13 +179,15 @@ __global__ __launch_bounds__(T) void optimizer_kernel_v4(f4* __restrict__ w, con
 template <int KIND>
 __global__ __launch_bounds__(256) void optimizer_kernel_scalar(float* __restrict__ w, const float* __restrict__ g,
                                                                 float* __restrict__ s0, float* __restrict__ s1,
-                                                                float* __restrict__ s2, int64_t n, OptScalars p) {
+                                                                float* __restrict__ s2, int64_t n, OptScalars p,
+                                                                __bf16* __restrict__ wbf) {
   constexpr int NS = n_states<KIND>();
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     float ww = w[i], aa = s0[i], bb = NS > 1 ? s1[i] : 0.f, cc = NS > 2 ? s2[i] : 0.f;
     update_one<KIND>(ww, g[i], aa, bb, cc, p);
     w[i] = ww;
+    if (wbf) wbf[i] = (__bf16)ww;
     s0[i] = aa;
     if (NS > 1) s1[i] = bb;
     if (NS > 2) s2[i] = cc;
@@ -184,19 +198,23 @@ static bool aligned16(const void* p) { return p == nullptr || (reinterpret_cast<
 
 template <int KIND>
 static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g, float* s0, float* s1, float* s2, int64_t n,
-                        const OptScalars& p) {
+                        const OptScalars& p, void* wbf) {
   // One vector per thread; threads per block measured per number of state tensors on 100 M elements (MI355X): 128 for one or
   // two states (SGD 308 us against 319 with 4 vectors x 256 threads, Adam 446 against 467), 64 for three (AMSGrad 596
   // against 614).  Many small blocks keep more independent request streams in flight than few large ones.
   constexpr int UNROLL = 1, THREADS = n_states<KIND>() <= 2 ? 128 : 64;
-  const bool vec = aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2);
+  const bool vec = aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2) && (reinterpret_cast<uintptr_t>(wbf) & 7u) == 0;
   const int64_t n4 = vec ? n / 4 : 0;
   if (n4 > 0) {
     const int64_t blocks = ceil_div(n4, (int64_t)THREADS * UNROLL);  // one pass, no grid-stride loop
     SN_REQUIRE(blocks <= 0x7fffffff, "optimizer update over %lld elements exceeds one launch", (long long)n);
     LaunchScope scope(ctx, name);
-    hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
-                       (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p);
+    if (wbf)
+      hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS, true>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
+                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)wbf);
+    else
+      hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS, false>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
+                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)nullptr);
   }
   const int64_t done = n4 * 4;
   if (done < n) {
@@ -206,14 +224,14 @@ static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g,
     if (blocks > cap) blocks = cap;
     LaunchScope scope(ctx, name);
     hipLaunchKernelGGL((optimizer_kernel_scalar<KIND>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w + done, g + done,
-                       s0 + done, s1 ? s1 + done : nullptr, s2 ? s2 + done : nullptr, rest, p);
+                       s0 + done, s1 ? s1 + done : nullptr, s2 ? s2 + done : nullptr, rest, p, wbf ? (__bf16*)wbf + done : nullptr);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
 
 int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
-                     int64_t n, int iter) {
+                     int64_t n, int iter, void* wbf) {
   const int ns = opt_state_count(d.kind);
   SN_REQUIRE(ns > 0, "unknown optimizer kind %d", d.kind);
   SN_REQUIRE(w && g && s0 && (ns < 2 || s1) && (ns < 3 || s2), "optimizer kind %d needs %d state buffers", d.kind, ns);
@@ -221,14 +239,14 @@ int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const fl
   if (n <= 0) return SN_OK;
   const OptScalars p = make_opt_scalars(d, iter);
   switch (d.kind) {
-    case SN_OPT_SGD: return launch_opt_t<SN_OPT_SGD>(ctx, "optimizer_sgd", w, g, s0, s1, s2, n, p);
-    case SN_OPT_ADAGRAD: return launch_opt_t<SN_OPT_ADAGRAD>(ctx, "optimizer_adagrad", w, g, s0, s1, s2, n, p);
-    case SN_OPT_ADADELTA: return launch_opt_t<SN_OPT_ADADELTA>(ctx, "optimizer_adadelta", w, g, s0, s1, s2, n, p);
-    case SN_OPT_RMSPROP: return launch_opt_t<SN_OPT_RMSPROP>(ctx, "optimizer_rmsprop", w, g, s0, s1, s2, n, p);
-    case SN_OPT_ADAM: return launch_opt_t<SN_OPT_ADAM>(ctx, "optimizer_adam", w, g, s0, s1, s2, n, p);
-    case SN_OPT_NADAM: return launch_opt_t<SN_OPT_NADAM>(ctx, "optimizer_nadam", w, g, s0, s1, s2, n, p);
-    case SN_OPT_ADAMAX: return launch_opt_t<SN_OPT_ADAMAX>(ctx, "optimizer_adamax", w, g, s0, s1, s2, n, p);
-    default: return launch_opt_t<SN_OPT_AMSGRAD>(ctx, "optimizer_amsgrad", w, g, s0, s1, s2, n, p);
+    case SN_OPT_SGD: return launch_opt_t<SN_OPT_SGD>(ctx, "optimizer_sgd", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_ADAGRAD: return launch_opt_t<SN_OPT_ADAGRAD>(ctx, "optimizer_adagrad", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_ADADELTA: return launch_opt_t<SN_OPT_ADADELTA>(ctx, "optimizer_adadelta", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_RMSPROP: return launch_opt_t<SN_OPT_RMSPROP>(ctx, "optimizer_rmsprop", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_ADAM: return launch_opt_t<SN_OPT_ADAM>(ctx, "optimizer_adam", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_NADAM: return launch_opt_t<SN_OPT_NADAM>(ctx, "optimizer_nadam", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_ADAMAX: return launch_opt_t<SN_OPT_ADAMAX>(ctx, "optimizer_adamax", w, g, s0, s1, s2, n, p, wbf);
+    default: return launch_opt_t<SN_OPT_AMSGRAD>(ctx, "optimizer_amsgrad", w, g, s0, s1, s2, n, p, wbf);
   }
 }
 
