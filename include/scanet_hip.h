@@ -173,11 +173,14 @@ SN_API int sn_ctx_destroy(sn_ctx* ctx);
 /* Message of the calling thread's most recent failing call (never NULL). */
 SN_API const char* sn_last_error(void);
 /* Blocks until everything issued on the context's stream has finished.
- * Like every call that synchronises (sn_copy_d2h, a step or gradient call that returns its loss), it returns
- * SN_E_STATE once if a recurrent layer's one-launch forward or backward kernel gave up waiting for its neighbour workgroups
+ * Like every call that synchronises the compute stream and hands results back (sn_copy_d2h, sn_params_get /
+ * sn_optstate_get / sn_grads_get, sn_count_correct, sn_error_sum, sn_train_epoch_host, the profile readers, a step or
+ * gradient call that returns its loss), it returns SN_E_STATE once if a recurrent layer's one-launch forward or backward kernel gave up waiting for its neighbour workgroups
  * since the previous synchronisation (only possible when something else occupies compute units of the same GPU):
  * the results computed since then are invalid, the context stays usable and from then on runs recurrent layers with one
- * launch per time step.  The wait is a bounded number of polls
+ * launch per time step.  The optimizer update of a training step whose passes gave up does not run: weights and
+ * optimizer state keep the values they had before that step (and before every later step until the error is
+ * reported); a stateful recurrent layer's carried state is undefined after such a step.  The wait is a bounded number of polls
  * (environment variable SCANET_SEQUENCE_SPIN_LIMIT, default 2000000, 0 = give up at the first wait; read when a context first launches that
  * kernel; SCANET_SEQUENCE_COHERENT=1 makes the kernel hand its state over with device-coherent accesses even
  * between workgroups of one XCD). */

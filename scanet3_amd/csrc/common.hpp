@@ -66,6 +66,7 @@ struct sn_ctx {
   int64_t seq_next = 0;            // first word of the area no launch has used since it was last cleared
   int* seq_gave_up = nullptr;      // host address
   int* seq_gave_up_dev = nullptr;  // the same word as the device sees it
+  int* seq_failed_dev = nullptr;   // device memory: set with it, read by the optimizer launch that follows a recurrent pass
   unsigned seq_spin_limit = 0;
   int seq_force_coherent = 0;      // hand over as if every row group were spread over several XCDs
   bool seq_disabled = false;       // a one-launch kernel gave up once: from then on the per-step kernels run
@@ -132,8 +133,9 @@ struct OptScalars {
 OptScalars make_opt_scalars(const sn_optimizer_desc& d, int iter);
 int opt_state_count(int kind);
 // wbf (optional): the updated weights are also written as bf16, element for element
+// skip_if (optional, device memory): the launch leaves everything as it is when *skip_if is not zero
 int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
-                     int64_t n, int iter, void* wbf = nullptr);
+                     int64_t n, int iter, void* wbf = nullptr, const int* skip_if = nullptr);
 struct AvgInputs {
   const float* p[SN_MAX_AVG_INPUTS];
 };

@@ -249,11 +249,12 @@ struct SeqFwdArgs {
   unsigned* sync;        // zero at launch: per row group a block of SEQ_GROUP_WORDS (arrival counter, XCD word, spread flag), then the abort word
   unsigned spin_limit;
   int* gave_up;          // host-visible
+  int* failed;           // the same flag in device memory: the optimizer launch of the step looks at it
   int force_coherent;    // take the across-XCD form everywhere
 };
 
 // Waits (thread 0 polls) until *count >= target.  Returns nonzero in every thread if the wait was given up.
-__device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, unsigned* abort_word, unsigned spin_limit, int* gave_up, int* stop) {
+__device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, unsigned* abort_word, unsigned spin_limit, int* gave_up, int* failed, int* stop) {
   if (threadIdx.x == 0) {
     unsigned spins = 0;
     int bad = spin_limit == 0u;  // a limit of zero gives up at the first wait whatever the counter shows (how a test forces this path)
@@ -267,6 +268,7 @@ __device__ __forceinline__ int wait_arrivals(unsigned* count, unsigned target, u
     }
     if (bad) {
       __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(failed, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     *stop = bad;
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_fwd_kernel(SeqFwdArgs a) {
   for (int t = 0; t < a.T; ++t) {
     const bool with_h = t > 0 || a.h0_valid;
     if (t > 0) {  // h_{t-1} is complete once every unit group of this row group has arrived t + 1 times (arrival 0 included)
-      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(t + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(t + 1), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
       if (t == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
     const float* xt = xrow + (int64_t)t * a.F;
@@ -520,6 +522,7 @@ struct SeqMulArgs {
   unsigned* sync;
   unsigned spin_limit;
   int* gave_up;
+  int* failed;
   int force_coherent;
 };
 
@@ -583,7 +586,7 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   for (int s = 0; s < steps; ++s) {
     const int t = BACKWARD ? a.T - 1 - s : s;  // the step whose operand slice is read
     if (s > 0) {  // the slice is complete once every unit group of this row group has arrived s + 1 times (arrival 0 included)
-      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+      if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
       if (s == 1) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     }
     const bool with_rec = BACKWARD || s > 0 || a.first_valid;
@@ -814,6 +817,7 @@ struct SeqBwdArgs {
   unsigned* sync;        // zero at launch, as in SeqFwdArgs
   unsigned spin_limit;
   int* gave_up;
+  int* failed;
   int force_coherent;
 };
 
@@ -922,7 +926,7 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       dyv = a.dy_seq ? a.dy_seq[yi + (int64_t)(t - 1) * H] : 0.f;
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
-    if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, &stop)) return;
+    if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
     if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     // ---- dh_{t-1} of this workgroup's cells = dz_t (16 complete rows) * the weight slab
     {
@@ -1044,8 +1048,12 @@ bool with_sequence_fwd_kernel(int K, F&& f) {
 }
 }  // namespace
 
-bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) {
-  if (ctx->seq_disabled) return false;
+// true once a one-launch kernel of this context has given up waiting, reported to the caller or not yet (the flag sits
+// in pinned host memory, so looking needs no synchronisation): from then on the per-step kernels run
+static bool sequence_kernels_off(const sn_ctx* ctx) {
+  return ctx->seq_disabled || (ctx->seq_gave_up && *(volatile int*)ctx->seq_gave_up != 0);
+}
+static bool lstm_sequence_fwd_fits(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) {
   if (rows <= 0 || !lstm_step_fused_ok(F, H, x, w)) return false;
   const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
@@ -1058,17 +1066,18 @@ bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, c
   });
   return known && fits;
 }
+bool lstm_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x, const LstmWeights& w) { return !sequence_kernels_off(ctx) && lstm_sequence_fwd_fits(ctx, rows, F, H, x, w); }
 
 int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_valid, const float* c0, int rows, int H, const LstmWeights& w,
                              float* gates, float* c, float* h, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
-  SN_REQUIRE(lstm_sequence_fwd_ok(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SN_REQUIRE(lstm_sequence_fwd_fits(ctx, rows, F, H, x, w), "lstm_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
   SN_REQUIRE(aligned16(h), "lstm_sequence_forward: operands must start on 16-byte boundaries");
   const int groups = (int)ceil_div(rows, SRB);
   unsigned* sync = nullptr;
   SN_TRY(seq_sync_take(ctx, groups, &sync));
   SeqFwdArgs a{x, c0, {w.wk[0], w.wk[1], w.wk[2], w.wk[3]}, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, {w.b[0], w.b[1], w.b[2], w.b[3]}, gates, c, h, slice, h0_valid, rows, T, F, H, groups, H / 16,
-               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_failed_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_forward", rows * T, 4 * H, F + H);  // T steps of rows x 4H x (F + H)
   with_sequence_fwd_kernel(F + H, [&](auto kernel, int nkb) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_lds_bytes(nkb), ctx->stream, a);
@@ -1134,8 +1143,7 @@ bool with_sequence_bwd_kernel(int H, F&& f) {
 }
 }  // namespace
 
-bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
-  if (ctx->seq_disabled) return false;
+static bool lstm_sequence_bwd_fits(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
   if (rows <= 0) return false;
   for (int g = 0; g < 4; ++g)
     if (!aligned16(w.wr[g])) return false;
@@ -1150,17 +1158,18 @@ bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) {
   });
   return known && fits;
 }
+bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) { return !sequence_kernels_off(ctx) && lstm_sequence_bwd_fits(ctx, rows, H, w); }
 
 int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
                              int rows, int H, const LstmWeights& w, float* dz, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
-  SN_REQUIRE(lstm_sequence_bwd_ok(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
+  SN_REQUIRE(lstm_sequence_bwd_fits(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SN_REQUIRE(aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
   const int groups = (int)ceil_div(rows, SRB);
   unsigned* sync = nullptr;
   SN_TRY(seq_sync_take(ctx, groups, &sync));
   SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, dz, slice, rows, T, H, groups, H / 16,
-               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_force_coherent};
+               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_failed_dev, ctx->seq_force_coherent};
   LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
   with_sequence_bwd_kernel(H, [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_bwd_lds_bytes(H), ctx->stream, a);
@@ -1197,7 +1206,6 @@ bool with_rnn_sequence_kernel(int K, F&& f) {
 }
 template <bool BACKWARD>
 bool rnn_sequence_fits(sn_ctx* ctx, int rows, int K, int H) {
-  if (ctx->seq_disabled) return false;
   const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
   if (groups > SEQ_MAX_GROUPS) return false;
   bool fits = false;
@@ -1216,6 +1224,7 @@ int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
   SN_TRY(seq_sync_take(ctx, a.row_groups, &a.sync));
   a.spin_limit = ctx->seq_spin_limit;
   a.gave_up = ctx->seq_gave_up_dev;
+  a.failed = ctx->seq_failed_dev;
   a.force_coherent = ctx->seq_force_coherent;
   const int steps = BACKWARD ? a.T - 1 : a.T;
   LaunchScope scope(ctx, name, a.rows * steps, a.H, K);  // `steps` products of rows x H x K
@@ -1228,27 +1237,29 @@ int launch_rnn_sequence(sn_ctx* ctx, SeqMulArgs a, const char* name, int K) {
 }
 }  // namespace
 
-bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x) {
+static bool rnn_sequence_fwd_fits(sn_ctx* ctx, int rows, int F, int H, const float* x) {
   return rows > 0 && F % 4 == 0 && H % 16 == 0 && F + H <= MAX_K && aligned16(x) && rnn_sequence_fits<false>(ctx, rows, F + H, H);
 }
+bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x) { return !sequence_kernels_off(ctx) && rnn_sequence_fwd_fits(ctx, rows, F, H, x); }
 
 int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wk, const float* wr,
                             float* r_slices, int64_t slice) {
   if (rows <= 0 || T <= 0) return SN_OK;
-  SN_REQUIRE(rnn_sequence_fwd_ok(ctx, rows, F, H, x), "rnn_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
+  SN_REQUIRE(rnn_sequence_fwd_fits(ctx, rows, F, H, x), "rnn_sequence_forward: rows=%d F=%d H=%d do not fit the device in one launch", rows, F, H);
   SeqMulArgs a{};
   a.x = x; a.rec = r_slices; a.wk = wk; a.wr = wr; a.slice = slice; a.first_valid = first_valid;
   a.rows = rows; a.T = T; a.F = F; a.H = H;
   return launch_rnn_sequence<false>(ctx, a, "rnn_sequence_forward", F + H);
 }
 
-bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr) {
+static bool rnn_sequence_bwd_fits(sn_ctx* ctx, int rows, int H, const float* wr) {
   return rows > 0 && H % 16 == 0 && H <= MAX_K && aligned16(wr) && rnn_sequence_fits<true>(ctx, rows, H, H);
 }
+bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr) { return !sequence_kernels_off(ctx) && rnn_sequence_bwd_fits(ctx, rows, H, wr); }
 
 int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice) {
   if (rows <= 0 || T <= 1) return SN_OK;
-  SN_REQUIRE(rnn_sequence_bwd_ok(ctx, rows, H, wr), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
+  SN_REQUIRE(rnn_sequence_bwd_fits(ctx, rows, H, wr), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SeqMulArgs a{};
   a.rec = dr_slices; a.dy_seq = dy_seq; a.wr = wr; a.slice = slice;
   a.rows = rows; a.T = T; a.F = 0; a.H = H;

@@ -1019,13 +1019,17 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bo
 static int update(sn_replica* r, int iter) {
   SN_REQUIRE(r->has_opt, "replica was created without an optimizer");
   sn_model* m = r->model;
+  // A one-launch recurrent kernel of an earlier pass that gave up is reported before anything moves (the flag sits in
+  // pinned host memory: no synchronisation needed to look); one of THIS step's passes that gives up, which the host
+  // cannot know yet, makes the optimizer launch below leave weights and optimizer state as they are.
+  if (r->ctx->seq_gave_up && *(volatile int*)r->ctx->seq_gave_up != 0) return check_async(r->ctx);
   // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
   // the statistics are those of the gradient pass that has just run.  In bf16 mode the optimizer writes the bf16 copy of
   // what it updates in the same pass (every Dense weight is trainable), so the copies stay current.
   for (const auto& run : m->trainable_runs)
     SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,
                             r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter,
-                            r->bf_wflat ? r->bf_wflat + run.first : nullptr));
+                            r->bf_wflat ? r->bf_wflat + run.first : nullptr, r->ctx->seq_failed_dev));
   for (size_t i = 0; i < m->ops.size(); ++i) {
     const Op& op = m->ops[i];
     if (op.kind == OP_BATCHNORM)
@@ -1473,6 +1477,15 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
   SN_HIP(hipStreamWaitEvent(rep->copy_stream, rep->ev_consumed[0], 0));
   int64_t first = 0, nb = 1, last_first = 0;
   int slot = 0;
+  // The caller may reuse its host buffers as soon as this function returns, also when it returns an error: whatever
+  // path leaves it, the copies queued so far (and the steps they feed) have finished first.
+  struct DrainOnExit {
+    hipStream_t copy, compute;
+    ~DrainOnExit() {
+      (void)hipStreamSynchronize(compute);
+      (void)hipStreamSynchronize(copy);
+    }
+  } drain{rep->copy_stream, compute};
   SN_TRY(fill(first, nb, slot));
   for (int64_t run = 0; first < n_batches; ++run) {
     const int64_t next_first = first + nb, next_nb = std::min(std::min(G, 2 * nb), n_batches - next_first);
@@ -1501,7 +1514,8 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
     SN_TRY(loss_of(rep, pred, last_y, batch, nullptr, true));
     SN_TRY(read_loss(rep, loss_host));
   } else {
-    SN_HIP(hipStreamSynchronize(compute));  // the host buffers may be reused once this returns
+    SN_HIP(hipStreamSynchronize(compute));
+    SN_TRY(check_async(rep->ctx));
   }
   SN_HIP(hipStreamSynchronize(rep->copy_stream));
   return SN_OK;

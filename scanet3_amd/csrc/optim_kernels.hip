@@ -109,8 +109,9 @@ typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 template <int KIND, int U, int T, bool WBF>
 __global__ __launch_bounds__(T) void optimizer_kernel_v4(f4* __restrict__ w, const f4* __restrict__ g, f4* __restrict__ s0,
                                                             f4* __restrict__ s1, f4* __restrict__ s2, int64_t n4,
-                                                            OptScalars p, bf16x4_t* __restrict__ wbf) {
+                                                            OptScalars p, bf16x4_t* __restrict__ wbf, const int* __restrict__ skip_if) {
   constexpr int NS = n_states<KIND>();
+  if (skip_if && *skip_if) return;  // the gradient pass in front of this update failed: nothing moves
   const int64_t base = (int64_t)blockIdx.x * (T * U) + threadIdx.x;
   if (U == 1 && base >= n4) return;  // one vector per thread: one early exit instead of a check around every access
 #define SN_IN_RANGE(u) (U == 1 || base + (u) * T < n4)
@@ -180,8 +181,9 @@ template <int KIND>
 __global__ __launch_bounds__(256) void optimizer_kernel_scalar(float* __restrict__ w, const float* __restrict__ g,
                                                                 float* __restrict__ s0, float* __restrict__ s1,
                                                                 float* __restrict__ s2, int64_t n, OptScalars p,
-                                                                __bf16* __restrict__ wbf) {
+                                                                __bf16* __restrict__ wbf, const int* __restrict__ skip_if) {
   constexpr int NS = n_states<KIND>();
+  if (skip_if && *skip_if) return;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     float ww = w[i], aa = s0[i], bb = NS > 1 ? s1[i] : 0.f, cc = NS > 2 ? s2[i] : 0.f;
@@ -198,7 +200,7 @@ static bool aligned16(const void* p) { return p == nullptr || (reinterpret_cast<
 
 template <int KIND>
 static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g, float* s0, float* s1, float* s2, int64_t n,
-                        const OptScalars& p, void* wbf) {
+                        const OptScalars& p, void* wbf, const int* skip_if) {
   // One vector per thread; threads per block measured per number of state tensors on 100 M elements (MI355X): 128 for one or
   // two states (SGD 308 us against 319 with 4 vectors x 256 threads, Adam 446 against 467), 64 for three (AMSGrad 596
   // against 614).  Many small blocks keep more independent request streams in flight than few large ones.
@@ -211,10 +213,10 @@ static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g,
     LaunchScope scope(ctx, name);
     if (wbf)
       hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS, true>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
-                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)wbf);
+                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)wbf, skip_if);
     else
       hipLaunchKernelGGL((optimizer_kernel_v4<KIND, UNROLL, THREADS, false>), dim3((unsigned)blocks), dim3(THREADS), 0, ctx->stream, (f4*)w,
-                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)nullptr);
+                         (const f4*)g, (f4*)s0, (f4*)s1, (f4*)s2, n4, p, (bf16x4_t*)nullptr, skip_if);
   }
   const int64_t done = n4 * 4;
   if (done < n) {
@@ -224,14 +226,14 @@ static int launch_opt_t(sn_ctx* ctx, const char* name, float* w, const float* g,
     if (blocks > cap) blocks = cap;
     LaunchScope scope(ctx, name);
     hipLaunchKernelGGL((optimizer_kernel_scalar<KIND>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w + done, g + done,
-                       s0 + done, s1 ? s1 + done : nullptr, s2 ? s2 + done : nullptr, rest, p, wbf ? (__bf16*)wbf + done : nullptr);
+                       s0 + done, s1 ? s1 + done : nullptr, s2 ? s2 + done : nullptr, rest, p, wbf ? (__bf16*)wbf + done : nullptr, skip_if);
   }
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
 
 int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
-                     int64_t n, int iter, void* wbf) {
+                     int64_t n, int iter, void* wbf, const int* skip_if) {
   const int ns = opt_state_count(d.kind);
   SN_REQUIRE(ns > 0, "unknown optimizer kind %d", d.kind);
   SN_REQUIRE(w && g && s0 && (ns < 2 || s1) && (ns < 3 || s2), "optimizer kind %d needs %d state buffers", d.kind, ns);
@@ -239,14 +241,14 @@ int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const fl
   if (n <= 0) return SN_OK;
   const OptScalars p = make_opt_scalars(d, iter);
   switch (d.kind) {
-    case SN_OPT_SGD: return launch_opt_t<SN_OPT_SGD>(ctx, "optimizer_sgd", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_ADAGRAD: return launch_opt_t<SN_OPT_ADAGRAD>(ctx, "optimizer_adagrad", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_ADADELTA: return launch_opt_t<SN_OPT_ADADELTA>(ctx, "optimizer_adadelta", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_RMSPROP: return launch_opt_t<SN_OPT_RMSPROP>(ctx, "optimizer_rmsprop", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_ADAM: return launch_opt_t<SN_OPT_ADAM>(ctx, "optimizer_adam", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_NADAM: return launch_opt_t<SN_OPT_NADAM>(ctx, "optimizer_nadam", w, g, s0, s1, s2, n, p, wbf);
-    case SN_OPT_ADAMAX: return launch_opt_t<SN_OPT_ADAMAX>(ctx, "optimizer_adamax", w, g, s0, s1, s2, n, p, wbf);
-    default: return launch_opt_t<SN_OPT_AMSGRAD>(ctx, "optimizer_amsgrad", w, g, s0, s1, s2, n, p, wbf);
+    case SN_OPT_SGD: return launch_opt_t<SN_OPT_SGD>(ctx, "optimizer_sgd", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_ADAGRAD: return launch_opt_t<SN_OPT_ADAGRAD>(ctx, "optimizer_adagrad", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_ADADELTA: return launch_opt_t<SN_OPT_ADADELTA>(ctx, "optimizer_adadelta", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_RMSPROP: return launch_opt_t<SN_OPT_RMSPROP>(ctx, "optimizer_rmsprop", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_ADAM: return launch_opt_t<SN_OPT_ADAM>(ctx, "optimizer_adam", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_NADAM: return launch_opt_t<SN_OPT_NADAM>(ctx, "optimizer_nadam", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    case SN_OPT_ADAMAX: return launch_opt_t<SN_OPT_ADAMAX>(ctx, "optimizer_adamax", w, g, s0, s1, s2, n, p, wbf, skip_if);
+    default: return launch_opt_t<SN_OPT_AMSGRAD>(ctx, "optimizer_amsgrad", w, g, s0, s1, s2, n, p, wbf, skip_if);
   }
 }
 

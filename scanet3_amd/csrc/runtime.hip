@@ -83,8 +83,10 @@ static int seq_sync_init(sn_ctx* ctx) {
   unsigned* arrived = nullptr;
   int* word = nullptr;
   void* word_dev = nullptr;
+  int* failed = nullptr;
   SN_HIP(hipSetDevice(ctx->device));
   hipError_t e = hipMalloc(&arrived, SEQ_COUNTERS * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMalloc(&failed, 256);
   if (e == hipSuccess) e = hipHostMalloc(&word, sizeof(int), hipHostMallocMapped);
   if (e == hipSuccess) {
     *word = 0;
@@ -92,12 +94,15 @@ static int seq_sync_init(sn_ctx* ctx) {
   }
   if (e != hipSuccess) {
     if (arrived) (void)hipFree(arrived);
+    if (failed) (void)hipFree(failed);
     if (word) (void)hipHostFree(word);
     return fail(SN_E_HIP, "setting up the sequence kernels' counters failed: %s", hipGetErrorString(e));
   }
   ctx->seq_arrived = arrived;
   ctx->seq_next = SEQ_COUNTERS;  // nothing cleared yet
   ctx->seq_gave_up = word;
+  ctx->seq_failed_dev = failed;
+  SN_TRY(launch_fill(ctx, reinterpret_cast<float*>(failed), 0.f, 64));  // all-zero bits; a kernel, not a memset node
   ctx->seq_gave_up_dev = static_cast<int*>(word_dev);
   // about a microsecond per poll: two seconds before a kernel whose neighbours never arrive gives up
   ctx->seq_spin_limit = 2000000u;
@@ -122,6 +127,8 @@ int seq_sync_take(sn_ctx* ctx, int groups, unsigned** block) {
 int check_async(sn_ctx* ctx) {
   if (!ctx->seq_gave_up || *(volatile int*)ctx->seq_gave_up == 0) return SN_OK;
   *(volatile int*)ctx->seq_gave_up = 0;
+  // the device's copy of the flag is cleared behind everything queued so far (a kernel, not a memset node)
+  if (ctx->seq_failed_dev) (void)launch_fill(ctx, reinterpret_cast<float*>(ctx->seq_failed_dev), 0.f, 1);
   ctx->seq_disabled = true;  // something else holds compute units of this GPU: do not count on the whole grid being resident again
   return fail(SN_E_STATE, "a recurrent sequence kernel gave up waiting for its neighbour workgroups (are other processes using this GPU?): "
                           "the results of the calls since the last synchronisation are invalid");
@@ -185,6 +192,7 @@ int sn_ctx_destroy(sn_ctx* ctx) {
   for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
   if (ctx->seq_arrived) (void)hipFree(ctx->seq_arrived);
   if (ctx->seq_gave_up) (void)hipHostFree(ctx->seq_gave_up);
+  if (ctx->seq_failed_dev) (void)hipFree(ctx->seq_failed_dev);
   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
   ctx->magic = 0;
   delete ctx;
@@ -296,7 +304,10 @@ int sn_random_fill(sn_ctx* ctx, float* dst_dev, int64_t n, int32_t dist, uint64_
 
 int sn_profile_enable(sn_ctx* ctx, int32_t on) {
   SN_TRY(check_ctx(ctx));
-  if (!on) SN_TRY(profile_drain(ctx));
+  if (!on) {
+    SN_TRY(profile_drain(ctx));
+    SN_TRY(check_async(ctx));
+  }
   ctx->profiling = on != 0;
   return SN_OK;
 }
@@ -304,6 +315,7 @@ int sn_profile_enable(sn_ctx* ctx, int32_t on) {
 int sn_profile_reset(sn_ctx* ctx) {
   SN_TRY(check_ctx(ctx));
   SN_TRY(profile_drain(ctx));
+  SN_TRY(check_async(ctx));  // the drain synchronised the stream
   ctx->profile.clear();
   ctx->profile_names.clear();
   return SN_OK;
@@ -313,6 +325,7 @@ int sn_profile_count(sn_ctx* ctx, int32_t* n) {
   SN_TRY(check_ctx(ctx));
   SN_REQUIRE(n != nullptr, "sn_profile_count: out is NULL");
   SN_TRY(profile_drain(ctx));
+  SN_TRY(check_async(ctx));  // the drain synchronised the stream
   *n = (int32_t)ctx->profile_names.size();
   return SN_OK;
 }

@@ -1146,6 +1146,54 @@ def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
         xb.free()
     finally:
         c.close()
+    # A training step whose passes give up: every call that hands results back reports it, and the optimizer update of
+    # that step did not run (weights and both Adam slots are what they were).
+    c = S.Context(0)
+    try:
+        cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (64, 32), 512)
+        rep = cm.replica(S.Adam(0.01))
+        rng = np.random.default_rng(6)
+        xb = c.to_device(rng.standard_normal((512, 64, 32)).astype(f32))
+        yb = c.to_device(rng.uniform(-1, 1, (512, 1)).astype(f32))
+        before, slots = rep.get_params(), [rep.get_opt_state(0), rep.get_opt_state(1)]
+        # the forward kernel gives up; the step itself reports it if the host sees the flag before it queues the update
+        # (then the update is never launched), otherwise the first call that hands results back does (and the update
+        # that was launched found the device's copy of the flag and left everything alone)
+        with pytest.raises(S.ScanetError, match="gave up waiting"):
+            rep.step(xb, yb, 1, want_loss=False)
+            rep.get_params()
+        after, slots_after = rep.get_params(), [rep.get_opt_state(0), rep.get_opt_state(1)]
+        for p in before:
+            assert np.array_equal(before[p], after[p]), p
+        for a_, b_ in zip(slots, slots_after):
+            for p in a_:
+                assert np.array_equal(a_[p], b_[p]), p
+        rep.step(xb, yb, 1, want_loss=False)       # the same step through the per-step kernels now moves the weights
+        moved = rep.get_params()
+        assert any(not np.array_equal(before[p], moved[p]) for p in before)
+        for o in (rep, cm):
+            o.close()
+        xb.free()
+        yb.free()
+    finally:
+        c.close()
+    # ... and so does the accuracy count
+    c = S.Context(0)
+    try:
+        cm = S.CompiledModel(c, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (64, 32), 512)
+        rep = cm.replica(None)
+        rng = np.random.default_rng(7)
+        xb = c.to_device(rng.standard_normal((512, 64, 32)).astype(f32))
+        yb = c.to_device(rng.uniform(-1, 1, (512, 1)).astype(f32))
+        with pytest.raises(S.ScanetError, match="gave up waiting"):
+            rep.count_correct(xb, yb)
+        assert rep.count_correct(xb, yb) >= 0
+        for o in (rep, cm):
+            o.close()
+        xb.free()
+        yb.free()
+    finally:
+        c.close()
 
 
 def test_maximizing_step_adds_the_delta(S, ctx):
