@@ -259,7 +259,8 @@ SN_API int sn_forward(sn_replica* rep, const float* x_dev, int32_t rows, float* 
  * only sn_step and the epoch calls move layer state. */
 SN_API int sn_forward_training(sn_replica* rep, const float* x_dev, int32_t rows, float* out_dev);
 /* sn_forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same result as sn_forward, but every
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  What is tested is that the call leaves
+ * the device's free memory unchanged; recording it into a graph is not.  Same result as sn_forward, but every
  * intermediate of the pass (layer outputs, pooling offsets, BatchNorm vectors, the GEMM workspace) lives in one
  * 64 MiB device array that is part of the library image (each GPU the library runs on holds its copy until the
  * process ends), and the call makes no hipMalloc / hipFree.  Fails with SN_E_INVALID when `rows` of this model need

@@ -201,26 +201,37 @@ __global__ __launch_bounds__(256) void lstm_step_fwd_kernel(StepFwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------- all forward steps in one launch
-// The same decomposition as the step kernel (32 batch rows x 16 hidden units per workgroup), but the workgroup stays for
-// the whole sequence: its weight slab is copied to LDS once, its cell states live in registers, and only [x_t, h_{t-1}]
-// is fetched per step.  h_t is handed from the unit groups of a row group to each other through memory: after its
-// stores of step t have been acknowledged a workgroup adds 1 to the row group's arrival counter; before step t + 1 it
-// waits until the counter shows every workgroup of the group.  That needs all workgroups of the launch on the device at
-// once, which the host checks against the device's occupancy before it picks this kernel.  The wait is bounded all the
-// same: a workgroup that polls `spin_limit` times in vain (or sees that another one did) raises the abort word, reports
-// through `gave_up` and leaves, and so does every other workgroup at its next wait.
+// A workgroup owns 16 batch rows x 16 hidden units for the whole sequence (512 x 256 gives 512 workgroups, two or more
+// per CU, so one multiplies while its neighbour on the CU waits).  Wavefront w owns gate w: its [K x 16] weights are read
+// once per launch, as they lie, into registers in MFMA operand order; the cell states of the workgroup's cells live in
+// registers; per step only the 16 rows of [x_t, h_{t-1}] are fetched, straight into LDS (LDS-direct loads), multiplied on
+// v_mfma_f32_16x16x4_f32, and the four gates meet in LDS.  h_t is handed from the unit groups of a row group to each
+// other through memory: after its stores of step t have been acknowledged a workgroup adds 1 to the row group's arrival
+// counter; before step t + 1 it waits until the counter shows every workgroup of the group.  That needs all workgroups
+// of the launch on the device at once, which the host checks against the device's occupancy before it picks this
+// kernel.  The wait is bounded all the same: a workgroup that polls `spin_limit` times in vain (or sees that another
+// one did) raises the abort word, reports through `gave_up` / `failed` and leaves, and so does every other workgroup at
+// its next wait.  About 4.4 us per step at 512 x 256 x 288 (one launch per step: 11.2 us).
 //
 // The hand-over avoids device-scope fences, which on this hardware write back and invalidate a whole L2 and cost tens
 // of microseconds per step here.  Two forms instead, chosen per row group:
 //   within one XCD   plain stores and loads.  The XCD's L2 is the one cache between its CUs: a store acknowledged
-//                    (s_waitcnt vmcnt(0)) is in L2, and a load of an address this CU has not touched in this launch
-//                    (every h slice is read once) misses L1 and finds it there.  7.1 us per step at 512 x 256.
+//                    (s_waitcnt vmcnt(0)) is in L2, and a load of a line this CU's vector L1 does not hold finds it
+//                    there.  That the L1 does not hold it rests on two things: every h (dz, r) slice is written once
+//                    and read once per launch, at addresses nobody has read before in this launch; and the vector L1
+//                    is write-through WITHOUT write-allocate, so the 64 bytes a workgroup itself stored into a
+//                    128-byte line of the slice did not bring that line into its L1 (the other half of the line comes
+//                    from a neighbour workgroup and must be read from L2).  The second premise is a property of this
+//                    hardware that the kernel relies on and cannot check; the parity tests (both forms, several
+//                    steps with different data per step) are what pins it.
 //   across XCDs      every access is itself coherent at device scope: h_t is written with device-scope atomic stores
-//                    (write-through), read with loads that carry the same coherence bit (sc1).  14.3 us per step.
+//                    (write-through), read with loads that carry the same coherence bit (sc1).  About twice the time.
 // Workgroup ids are mapped to (row group, unit group) so that a row group's workgroups have ids congruent mod 8, which
 // the dispatcher places on one XCD.  That is not taken on trust: each workgroup reads the XCD it runs on from the
 // hardware register, the members of a row group compare theirs in a first arrival before any hand-over, and one
-// mismatch switches the whole row group to the second form.  The counter itself is only touched with device-scope atomics.
+// mismatch switches the whole row group to the second form.  Each row group's counter, XCD word and flag have 256 bytes
+// of their own (all counters in one line made every polling workgroup of the launch meet on that line), and the counter
+// itself is only touched with device-scope atomics.
 __device__ __forceinline__ f4v load_coherent(const float* p) {
   f4v v;
   asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");

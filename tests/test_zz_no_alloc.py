@@ -4,6 +4,8 @@ Both run the same kernels on the same weights, one with its intermediates in the
 with them in the library's static device array, so the outputs must be bit-identical.  Two calls in a row, the second
 with fewer rows: the static array still holds the first call's contents.  Needs an MI355X: run with `-m gpu`.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -35,10 +37,21 @@ def test_static_forward_matches_forward_on_two_calls_in_a_row():
         x = rng.random((batch,) + in_shape, f32)
         xb = ctx.to_device(x)
         out = ctx.alloc(batch * cm.out_elems)
+        hip = ctypes.CDLL("libamdhip64.so")
+
+        def free_device_bytes():
+            free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+            assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+            return free.value
+
         for rows in (96, 40):                # the second call is smaller and finds the first one's data in the array
             want = rep.forward(xb, rows)
             out.fill(-1.0)
+            ctx.sync()
+            before = free_device_bytes()
             rep.forward_static(xb, out, rows)
+            ctx.sync()
+            assert free_device_bytes() == before, "the call allocated or freed device memory"
             got = out.numpy()[: rows * cm.out_elems].reshape(want.shape)
             assert np.array_equal(got, want), rows
             assert np.all(out.numpy()[rows * cm.out_elems:] == -1.0)      # nothing written past `rows`
