@@ -23,6 +23,7 @@ int fail(int code, const char* fmt, ...);
 #define SN_HIP(expr)                                                                         \
   do {                                                                                       \
     hipError_t e__ = (expr);                                                                 \
+    if (e__ != hipSuccess) (void)hipGetLastError(); /* or the next launch check finds it */  \
     if (e__ != hipSuccess)                                                                   \
       return sn::fail(e__ == hipErrorOutOfMemory ? SN_E_OOM : SN_E_HIP, "%s failed: %s (%s:%d)", #expr, \
                       hipGetErrorString(e__), __FILE__, __LINE__);                           \

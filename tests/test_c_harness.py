@@ -1,5 +1,7 @@
-"""The C ABI from a caller that is not Python: include/scanet_hip.h compiled as strict C99, and (on a GPU) a C program
-that drives three training steps, compared with the CPU oracle on the same numbers."""
+"""The C ABI from a caller that is not Python: include/scanet_hip.h compiled as strict C99, and (on a GPU) two C
+programs, one that drives three training steps and one that runs an epoch the way a JVM binding would (host partitions,
+two replicas, their average, predictions, accuracy count, optimizer state), compared with the CPU oracle on the same
+numbers."""
 import importlib.util
 import os
 import subprocess
@@ -68,3 +70,56 @@ def test_c_program_trains_three_steps_like_the_oracle():
         assert abs(losses[t] - float(loss)) <= 1e-5 * max(1.0, abs(float(loss))), t
     for path in params:
         np.testing.assert_allclose(params_c[path].reshape(params[path].shape), params[path], rtol=1e-4, atol=1e-6, err_msg=path)
+
+
+@pytest.mark.gpu
+def test_c_program_runs_an_epoch_on_two_replicas_like_the_oracle():
+    """epoch_harness.c: sn_host_alloc -> sn_train_epoch_host on two replicas -> sn_replicas_average -> sn_params_get /
+    sn_optstate_get / sn_forward / sn_count_correct, against `O.optimize_on_partition`, `O.average_uniform`,
+    `Model.forward` and `O.count_correct`."""
+    binary = os.path.join(HARNESS_DIR, "epoch_harness")
+    assert os.path.exists(binary), "build the harness first: python tests/c_harness/build.py (build() of __graft_entry__ does)"
+    batch, batches, tail, features, hidden, classes, replicas = 16, 4, 5, 6, 8, 3, 2
+    part_rows = batch * batches + tail
+    out = subprocess.run([binary], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    epochs, vectors, correct = {}, {}, None
+    for line in out.stdout.splitlines():
+        parts = line.split()
+        if parts[0] == "epoch":
+            epochs[int(parts[1])] = (int(parts[2]), float(parts[3]))
+        elif parts[0] == "correct":
+            correct = int(parts[1])
+        else:
+            vectors[(parts[0], parts[1])] = np.asarray([float(v) for v in parts[2:]], f32)
+    om = O.Model([O.Dense(hidden, O.ACT_TANH), O.Dense(classes, O.ACT_SOFTMAX)], O.LOSS_CCE)
+    gen = Lcg()
+    params = {}
+    for path, shape in om.param_defs((batch, features)):
+        n = int(np.prod(shape))
+        params[path] = np.asarray([(gen.unit() - f32(0.5)) * f32(0.5) for _ in range(n)], f32).reshape(shape)
+    partitions = []
+    for _ in range(replicas):
+        x = np.asarray([gen.unit() for _ in range(part_rows * features)], f32).reshape(part_rows, features)
+        y = np.zeros((part_rows, classes), f32)
+        for r in range(part_rows):
+            y[r, int(gen.unit() * f32(classes))] = 1.0
+        partitions.append((x, y))
+    alg = O.Adam(0.05)
+    results = []
+    for r, (x, y) in enumerate(partitions):
+        iters, p, st, loss = O.optimize_on_partition(om, alg, x, y, batch, 0, params, O.init_opt_state(alg, params))
+        assert epochs[r][0] == iters == batches                       # the 5-row tail is skipped
+        assert abs(epochs[r][1] - float(loss)) <= 1e-5 * max(1.0, abs(float(loss))), r
+        results.append((p, st))
+    mean = {p: O.average_uniform([res[0][p] for res in results]) for p in params}
+    first = next(iter(params))
+    slots = [O.average_uniform([res[1][first][s] for res in results]) for s in range(2)]
+    for r in range(replicas):                                          # both replicas hold the average afterwards
+        for path in params:
+            np.testing.assert_allclose(vectors[(f"param{r}", path)].reshape(mean[path].shape), mean[path], rtol=1e-4, atol=1e-6, err_msg=path)
+        for s in range(2):
+            np.testing.assert_allclose(vectors[(f"slot{s}_{r}", first)].reshape(slots[s].shape), slots[s], rtol=1e-4, atol=1e-7)
+    x0, y0 = partitions[0][0][:batch], partitions[0][1][:batch]
+    np.testing.assert_allclose(vectors[("pred", "batch0")].reshape(batch, classes), om.forward(x0, mean), rtol=1e-4, atol=1e-6)
+    assert correct == O.count_correct(om, x0, y0, mean)

@@ -9,6 +9,7 @@ the largest magnitude of the reference tensor, helpers.norm_err):
   loss trajectories ............................ 1e-3
   accuracy counts .............................. exact
 """
+import ctypes
 import zlib
 
 import numpy as np
@@ -1619,3 +1620,101 @@ def test_zero_length_calls_are_no_ops(S, ctx):
     ctx.sync()
     np.testing.assert_array_equal(buf.numpy(), np.full(4, 7.0, f32))
     buf.free()
+
+
+# ----------------------------------------------------------------------------- resuming a run, and calls that must fail cleanly
+
+
+def test_resumed_run_continues_bit_for_bit(S, ctx):
+    """Checkpoint / resume through the boundary: parameters, both Adam slots and the iteration number moved to a
+    fresh replica after 4 of 9 steps; the continuation must equal the uninterrupted run bit for bit (the step is a
+    pure function of those and the batch)."""
+    om, layers, sloss = build_pair([("conv", 8, (3, 3), (1, 1), "same", "relu", True), ("pool", (2, 2), (2, 2), "valid"), ("flatten",),
+                                    ("dense", 16, "tanh"), ("dense", 5, "softmax")], "cce")
+    batch, in_shape, steps, cut = 32, (12, 12, 2), 9, 4
+    rng = np.random.default_rng(20251125 + 21)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, in_shape, batch)
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    X = rng.random((3 * batch,) + in_shape, f32)
+    Y = one_hot(rng, 3 * batch, 5)
+    Xb, Yb = ctx.to_device(X), ctx.to_device(Y)
+    xs, ys = batch * int(np.prod(in_shape)), batch * 5
+
+    def run(rep, first, last):
+        return [rep.step(Xb.offset(((t - 1) % 3) * xs), Yb.offset(((t - 1) % 3) * ys), t, want_loss=True) for t in range(first, last + 1)]
+
+    whole = cm.replica(S.Adam(0.01))
+    whole.set_params(params)
+    losses = run(whole, 1, steps)
+    head = cm.replica(S.Adam(0.01))
+    head.set_params(params)
+    head_losses = run(head, 1, cut)
+    saved = (head.get_params(), head.get_opt_state(0), head.get_opt_state(1))
+    head.close()
+    tail = cm.replica(S.Adam(0.01))
+    tail.set_params(saved[0])
+    tail.set_opt_state(0, saved[1])
+    tail.set_opt_state(1, saved[2])
+    tail_losses = run(tail, cut + 1, steps)
+    assert head_losses + tail_losses == losses
+    for got, want in zip((tail.get_params(), tail.get_opt_state(0), tail.get_opt_state(1)),
+                         (whole.get_params(), whole.get_opt_state(0), whole.get_opt_state(1))):
+        for p in want:
+            assert np.array_equal(got[p], want[p]), p
+    for o in (tail, whole, cm):
+        o.close()
+    Xb.free()
+    Yb.free()
+
+
+def test_impossible_allocation_fails_cleanly(S, ctx):
+    """A buffer no device holds: SN_E_OOM (-3), and the context goes on working."""
+    from scanet3_amd import _lib as L
+    p = ctypes.c_void_p()
+    rc = L.lib.sn_buffer_alloc(ctx.handle, ctypes.c_size_t(1 << 50), ctypes.byref(p))
+    assert rc == -3 and not p.value, (rc, L.lib.sn_last_error())
+    host = ctypes.c_void_p()
+    rc = L.lib.sn_host_alloc(ctx.handle, ctypes.c_size_t(1 << 50), ctypes.byref(host))
+    assert rc in (-3, -5) and not host.value, (rc, L.lib.sn_last_error())
+    a = np.arange(1000, dtype=f32)
+    b = ctx.to_device(a)
+    b.fill(2.0)                       # a kernel launch right behind the failures: no stale error left behind
+    ctx.sync()
+    assert np.array_equal(b.numpy(), np.full(1000, 2.0, f32))
+    b.free()
+
+
+def test_nan_input_propagates_and_returns(S, ctx):
+    """A NaN in the batch: the step returns (no wait depends on the data), its loss is NaN, and so is every weight the
+    NaN reaches, as the same arithmetic gives on the CPU."""
+    om, layers, sloss = build_pair([("dense", 12, "sigmoid"), ("dense", 4, "softmax")], "cce")
+    batch, features = 24, 7
+    rng = np.random.default_rng(20251125 + 22)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], sloss.kind, (features,), batch)
+    rep = cm.replica(S.Adam(0.01))
+    params = glorot_params(om, (batch, features), rng)
+    rep.set_params(params)
+    x = rng.random((batch, features), f32)
+    x[3, 2] = np.nan
+    y = one_hot(rng, batch, 4)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    loss = rep.step(xb, yb, 1, want_loss=True)
+    assert np.isnan(loss)
+    with np.errstate(all="ignore"):
+        oparams, _, oloss, _ = O.train_step(om, O.Adam(0.01), x, y, params, O.init_opt_state(O.Adam(0.01), params), 1)
+    assert np.isnan(float(oloss))
+    got = rep.get_params()
+    for p in oparams:
+        assert np.array_equal(np.isnan(got[p]), np.isnan(oparams[p])), p
+    # the LSTM's one-launch kernels wait on counters, never on values: a NaN sequence ends like any other
+    _, rlayers, rloss = build_pair([("lstm", 32), ("dense", 1, "tanh")], "mse")
+    rcm = S.CompiledModel(ctx, [l.desc() for l in rlayers.layers], rloss.kind, (6, 8), 64)
+    rrep = rcm.replica(S.Adam(0.01))
+    xr = rng.standard_normal((64, 6, 8)).astype(f32)
+    xr[0, 0, 0] = np.nan
+    xrb, yrb = ctx.to_device(xr), ctx.to_device(rng.uniform(-1, 1, (64, 1)).astype(f32))
+    assert np.isnan(rrep.step(xrb, yrb, 1, want_loss=True))
+    for o in (rrep, rcm, rep, cm):
+        o.close()
+    for b in (xb, yb, xrb, yrb):
+        b.free()

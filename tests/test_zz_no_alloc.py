@@ -37,7 +37,10 @@ def test_static_forward_matches_forward_on_two_calls_in_a_row():
         x = rng.random((batch,) + in_shape, f32)
         xb = ctx.to_device(x)
         out = ctx.alloc(batch * cm.out_elems)
-        hip = ctypes.CDLL("libamdhip64.so")
+        # the HIP runtime instance the library itself is linked to (a second copy of the runtime would know no device)
+        with open("/proc/self/maps") as maps:
+            hip_path = next(line.split()[-1] for line in maps if "libamdhip64" in line and "/torch/" not in line)
+        hip = ctypes.CDLL(hip_path)
 
         def free_device_bytes():
             free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
