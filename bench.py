@@ -481,8 +481,54 @@ def cpu_baseline_lenet(pool_stride=1, budget_s=15.0):
         if time.perf_counter() - t0 > budget_s or n >= 200:
             break
     dt = time.perf_counter() - t0
-    return {"value": batch * n / dt, "unit": "samples/s", "cores": int(threads), "kind": "port",
-            "sample": f"{n} LeNet training steps of batch {batch} (numpy oracle, BLAS threads = {threads})"}
+    out = {"value": batch * n / dt, "unit": "samples/s", "cores": int(threads), "kind": "port",
+           "sample": f"{n} LeNet training steps of batch {batch} (numpy oracle, BLAS threads = {threads})"}
+    out["torch_cpu"] = torch_cpu_lenet(pool_stride, budget_s=10.0)
+    return out
+
+
+def torch_cpu_lenet(pool_stride=1, budget_s=10.0):
+    """The same LeNet training step through torch on the host cores (oneDNN convolutions, autograd, torch's Adam): a
+    framework-grade CPU figure beside the numpy port.  NOT the reference (that is TensorFlow-Java, which this image
+    does not hold) and not op-order faithful; torch is imported here and nowhere else.  None if torch cannot be imported."""
+    try:
+        import torch
+        import torch.nn.functional as F
+    except Exception:
+        return None
+    torch.manual_seed(SEED)
+    batch = 100
+    w1 = torch.nn.Parameter(torch.empty(32, 1, 3, 3).uniform_(-0.1, 0.1))
+    w2 = torch.nn.Parameter(torch.empty(64, 32, 3, 3).uniform_(-0.05, 0.05))
+    side = 28 - 2
+    side = (side - 2) // pool_stride + 1
+    side = side - 2
+    side = (side - 2) // pool_stride + 1
+    w3 = torch.nn.Parameter(torch.empty(side * side * 64, 10).uniform_(-0.01, 0.01))
+    b3 = torch.nn.Parameter(torch.zeros(10))
+    opt = torch.optim.Adam([w1, w2, w3, b3], lr=1e-3, eps=1e-7)
+    x = torch.rand(batch, 1, 28, 28)
+    y = torch.randint(0, 10, (batch,))
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        h = F.max_pool2d(F.relu(F.conv2d(x, w1)), 2, pool_stride)
+        h = F.max_pool2d(F.relu(F.conv2d(h, w2)), 2, pool_stride)
+        loss = F.cross_entropy(h.flatten(1) @ w3 + b3, y)
+        loss.backward()
+        opt.step()
+
+    for _ in range(3):
+        step()
+    n, t0 = 0, time.perf_counter()
+    while True:
+        n += 1
+        step()
+        if time.perf_counter() - t0 > budget_s or n >= 2000:
+            break
+    dt = time.perf_counter() - t0
+    return {"value": batch * n / dt, "unit": "samples/s", "cores": int(torch.get_num_threads()), "kind": "torch-cpu, not the reference",
+            "sample": f"{n} LeNet training steps of batch {batch} (torch {torch.__version__} on CPU: conv2d / max_pool2d / autograd / Adam)"}
 
 
 def main():
