@@ -53,6 +53,19 @@ struct PendingEvent {
 
 }  // namespace sn
 
+// The reduction of partial sums that a launcher left to its caller because sn_ctx::defer asked for it:
+// dst[o] = sum over `parts` partial results partial[p * outs + o] (o < outs), added in the order of the kernel that would
+// otherwise have run right away: kind 1 = splitk_reduce4_kernel's (eight interleaved chains, then a pairwise tree),
+// kind 2 = gemm_small_reduce_kernel's (64 interleaved chains, then a chain).  The training step hands these to the
+// launch that also applies the optimizer (launch_finish), so a filter gradient is summed and used in one pass.
+struct DeferredReduce {
+  int kind = 0;
+  const float* partial = nullptr;
+  int parts = 0, outs = 0;
+  float* dst = nullptr;
+};
+constexpr int MAX_DEFERRED = 4;
+
 struct sn_ctx {
   uint32_t magic;
   int device;
@@ -67,6 +80,7 @@ struct sn_ctx {
   int64_t seq_next = 0;            // first word of the area no launch has used since it was last cleared
   int* seq_gave_up = nullptr;      // host address
   int* seq_gave_up_dev = nullptr;  // the same word as the device sees it
+  DeferredReduce* defer = nullptr;   // set by a caller that takes the next partial-sum reduction on itself (cleared by the launcher that fills it)
   int* seq_failed_dev = nullptr;   // device memory: set with it, read by the optimizer launch that follows a recurrent pass
   unsigned seq_spin_limit = 0;
   int seq_force_coherent = 0;      // hand over as if every row group were spread over several XCDs
@@ -137,6 +151,13 @@ int opt_state_count(int kind);
 // skip_if (optional, device memory): the launch leaves everything as it is when *skip_if is not zero
 int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const float* g, float* s0, float* s1, float* s2,
                      int64_t n, int iter, void* wbf = nullptr, const int* skip_if = nullptr);
+// One launch that finishes a training step: the deferred reductions d[0..n_d) land in the gradient buffer g (their
+// targets lie inside it), and every element of the flat buffers [0, n) gets its optimizer update, the reduced ones from
+// the sums just made.  Same arithmetic and order as the reduction kernels followed by launch_optimizer.
+int launch_finish(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, float* g, float* s0, float* s1, float* s2, int64_t n, int iter,
+                  const DeferredReduce* defs, int n_defs, const int* skip_if);
+// Runs a deferred reduction on its own (when no optimizer launch follows that could take it).
+int launch_deferred_reduce(sn_ctx* ctx, const DeferredReduce& d);
 struct AvgInputs {
   const float* p[SN_MAX_AVG_INPUTS];
 };

@@ -106,6 +106,13 @@ struct sn_replica {
   std::vector<float*> bn_buf;  // per batch-norm op: mean, var, 1/sqrt(var+eps), scale, two gradient vectors
   float* bf_colp = nullptr;  // per-64-row-block column sums of dZ (bias gradient of the bf16 Dense path)
   bool bf_weights_stale = true;  // weights changed since their bf16 copies were made
+  // Training steps of a model whose whole flat buffer is one optimizer launch: the sums of the convolutions' partial
+  // filter gradients wait for that launch (launch_finish) instead of running as launches of their own.  Every such
+  // convolution has a workspace of its own (the shared one is overwritten by the next product).
+  bool fuse_finish = false, defer_now = false;
+  std::vector<float*> ws_defer;
+  DeferredReduce deferred[MAX_DEFERRED];
+  int n_deferred = 0;
   // host-fed epochs: two device slots per tensor, a copy stream, "slot filled" / "slot consumed" events
   float* stage_x[2] = {nullptr, nullptr};
   float* stage_y[2] = {nullptr, nullptr};
@@ -427,6 +434,7 @@ static bool dense_bf16_fast(const sn_model* m, const Op& op) {
 
 static float* param_ptr(sn_replica* r, float* base, int idx) { return idx < 0 ? nullptr : base + r->model->params[idx].info.offset; }
 
+static bool mlp2_path(const sn_model* m);
 static int alloc_replica(sn_replica* r) {
   sn_model* m = r->model;
   const int64_t B = m->batch;
@@ -501,6 +509,20 @@ static int alloc_replica(sn_replica* r) {
   SN_TRY(dev_alloc(r, &r->grad_buf[0], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->grad_buf[1], B * m->max_act_elems));
   SN_TRY(dev_alloc(r, &r->ws, m->workspace_elems));
+  r->ws_defer.assign(n_ops, nullptr);
+  bool penalties = false;
+  for (const auto& p : m->params) penalties = penalties || p.reg_kind != SN_REG_NONE;
+  r->fuse_finish = r->has_opt && !(m->flags & SN_FLAG_GEMM_BF16) && !penalties && !mlp2_path(m) && m->trainable_runs.size() == 1 &&
+                   m->trainable_runs[0].first == 0 && m->workspace_elems > 0 && m->workspace_elems <= ((int64_t)64 << 20);
+  if (r->fuse_finish) {
+    int n_conv = 0;
+    for (size_t i = 0; i < n_ops; ++i)
+      if (m->ops[i].kind == OP_CONV && n_conv < MAX_DEFERRED) {
+        SN_TRY(dev_alloc(r, &r->ws_defer[i], m->workspace_elems));
+        ++n_conv;
+      }
+    r->fuse_finish = n_conv > 0;
+  }
   SN_TRY(dev_alloc(r, &r->loss_dev, 1));
   SN_TRY(dev_alloc(r, &r->loss_partials, std::max<int64_t>(1024, m->batch)));
   SN_TRY(dev_alloc(r, &r->count_dev, 1));
@@ -802,7 +824,18 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         act_grad_done = false;
         if (op.b >= 0)
           SN_TRY(launch_col_sum(ctx, dy, g.cout, param_ptr(r, r->g, op.b), (int64_t)rows * g.ho * g.wo, g.cout, r->ws, m->workspace_elems));
-        SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems));
+        if (r->defer_now && r->ws_defer[i] && r->n_deferred < MAX_DEFERRED) {
+          // the sum of this product's partial results waits for the optimizer launch of the step
+          DeferredReduce& slot = r->deferred[r->n_deferred];
+          slot = DeferredReduce{};
+          ctx->defer = &slot;
+          const int rc = launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws_defer[i], m->workspace_elems);
+          ctx->defer = nullptr;
+          SN_TRY(rc);
+          if (slot.kind != 0) ++r->n_deferred;
+        } else {
+          SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems));
+        }
         if (need_dx) {
           SN_TRY(launch_conv_dgrad(ctx, g, dy, param_ptr(r, r->w, op.w), dx, r->ws, m->workspace_elems));
           cur ^= 1;
@@ -984,7 +1017,18 @@ static bool mlp2_path(const sn_model* m) {
   return mlp2_fused_ok(m->batch, (int)d1.in_elems, (int)d1.out_elems, (int)d2.out_elems, scratch, scratch);
 }
 
-static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss) {
+// for_update: the optimizer update of the same step follows (update()), which may then take over reductions this pass
+// leaves open; without it (sn_grad) every gradient is complete when the pass returns.
+static int grad_pass_body(sn_replica* r, const float* x, const float* y, int rows, bool want_loss);
+static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss, bool for_update = false) {
+  r->n_deferred = 0;
+  r->defer_now = for_update && r->fuse_finish;
+  const int rc = grad_pass_body(r, x, y, rows, want_loss);
+  r->defer_now = false;
+  if (rc != SN_OK) r->n_deferred = 0;
+  return rc;
+}
+static int grad_pass_body(sn_replica* r, const float* x, const float* y, int rows, bool want_loss) {
   sn_model* m = r->model;
   const int last = (int)m->ops.size() - 1;
   if (mlp2_path(m)) {
@@ -1026,6 +1070,12 @@ static int update(sn_replica* r, int iter) {
   // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
   // the statistics are those of the gradient pass that has just run.  In bf16 mode the optimizer writes the bf16 copy of
   // what it updates in the same pass (every Dense weight is trainable), so the copies stay current.
+  if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer (fuse_finish: one run from 0)
+    const auto& run = m->trainable_runs[0];
+    const int nd = r->n_deferred;
+    r->n_deferred = 0;
+    SN_TRY(launch_finish(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], run.second, iter, r->deferred, nd, r->ctx->seq_failed_dev));
+  } else
   for (const auto& run : m->trainable_runs)
     SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,
                             r->s[2] ? r->s[2] + run.first : nullptr, run.second - run.first, iter,
@@ -1262,7 +1312,7 @@ int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   SN_TRY(check_rows(rep, rows));
   SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
   SN_REQUIRE(rep->has_opt, "replica was created without an optimizer");
-  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr));
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr, true));
   SN_TRY(update(rep, iter));
   return read_loss(rep, loss_host);
 }
@@ -1393,7 +1443,7 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
              (long long)total_rows, batch);
   const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
   for (int64_t i = 0; i < n_batches; ++i) {
-    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch, false));  // the epoch's loss is evaluated after its last update
+    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch, false, true));  // the epoch's loss is evaluated after its last update
     SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
   }
   if (iterations_host) *iterations_host = (int32_t)n_batches;
@@ -1495,7 +1545,7 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
     }
     SN_HIP(hipStreamWaitEvent(compute, rep->ev_filled[slot], 0));
     for (int64_t j = 0; j < nb; ++j) {
-      SN_TRY(grad_pass(rep, rep->stage_x[slot] + j * xs, rep->stage_y[slot] + j * ys, batch, false));
+      SN_TRY(grad_pass(rep, rep->stage_x[slot] + j * xs, rep->stage_y[slot] + j * ys, batch, false, true));
       SN_TRY(update(rep, global_iter + (int)(first + j) + 1));  // optimizers/Optimizer.scala:143
     }
     SN_HIP(hipEventRecord(rep->ev_consumed[slot], compute));

@@ -252,6 +252,238 @@ int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const fl
   }
 }
 
+// ---- the launch that finishes a training step ------------------------------------------------
+// Sections of one grid: first the plain update of every float4 of the flat buffers that no deferred reduction owns
+// (128 threads, one vector each, as optimizer_kernel_v4), then per deferred reduction the blocks that add its partial
+// sums, in the order of the stand-alone reduction kernels, store the sums to the gradient buffer and update the
+// parameters they belong to right away.
+struct FinishPlan {
+  DeferredReduce r[MAX_DEFERRED];
+  int64_t first[MAX_DEFERRED];  // index in the flat buffers of r[i].dst[0]
+  int block0[MAX_DEFERRED + 1]; // first block of reduction i; block0[0] = number of plain blocks
+  int n;
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void finish_kernel(float* __restrict__ w, float* __restrict__ g, float* __restrict__ s0, float* __restrict__ s1,
+                                                      float* __restrict__ s2, int64_t n, OptScalars p, FinishPlan plan,
+                                                      const int* __restrict__ skip_if) {
+  constexpr int NS = n_states<KIND>();
+  __shared__ f4 part4[8][32];
+  __shared__ float part1[64][4];
+  const bool skip = skip_if && *skip_if;  // a failed pass: gradients are still summed, nothing is updated
+  const int b = blockIdx.x;
+  if (b < plan.block0[0]) {
+    if (skip || threadIdx.x >= 128) return;
+    const int64_t i4 = (int64_t)b * 128 + threadIdx.x, e = i4 * 4;
+    if (e >= n) return;
+    for (int k = 0; k < plan.n; ++k)
+      if (e >= plan.first[k] && e < plan.first[k] + plan.r[k].outs) return;  // a reduction block updates these
+    if (e + 4 <= n) {
+      f4 vw = *(const f4*)(w + e), vg = *(const f4*)(g + e), a = *(const f4*)(s0 + e), bb = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+      if (NS > 1) bb = *(const f4*)(s1 + e);
+      if (NS > 2) c = *(const f4*)(s2 + e);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float ww = vw[q], aa = a[q], b2 = bb[q], cc = c[q];
+        update_one<KIND>(ww, vg[q], aa, b2, cc, p);
+        vw[q] = ww; a[q] = aa; bb[q] = b2; c[q] = cc;
+      }
+      *(f4*)(w + e) = vw;
+      *(f4*)(s0 + e) = a;
+      if (NS > 1) *(f4*)(s1 + e) = bb;
+      if (NS > 2) *(f4*)(s2 + e) = c;
+    } else {
+      for (int64_t q = e; q < n; ++q) {
+        float ww = w[q], aa = s0[q], b2 = NS > 1 ? s1[q] : 0.f, cc = NS > 2 ? s2[q] : 0.f;
+        update_one<KIND>(ww, g[q], aa, b2, cc, p);
+        w[q] = ww; s0[q] = aa;
+        if (NS > 1) s1[q] = b2;
+        if (NS > 2) s2[q] = cc;
+      }
+    }
+    return;
+  }
+  int k = 0;
+  while (k + 1 < plan.n && b >= plan.block0[k + 1]) ++k;
+  const DeferredReduce& r = plan.r[k];
+  const int lb = b - plan.block0[k];
+  const int64_t flat0 = plan.first[k];
+  if (r.kind == 1) {
+    // splitk_reduce4_kernel's order: 8 groups of 32 lanes x 4 consecutive outputs; group q adds partials q, q + 8, ...
+    const int64_t total4 = r.outs / 4;
+    const int q = threadIdx.x >> 5, j = threadIdx.x & 31;
+    const int64_t i = (int64_t)lb * 32 + j;
+    f4 s = {0.f, 0.f, 0.f, 0.f};
+    if (i < total4) {
+      const f4* w4 = reinterpret_cast<const f4*>(r.partial) + i;
+      int z = q;
+      for (; z + 56 < r.parts; z += 64) {  // 8 loads of 16 bytes in flight, added in split order
+        f4 a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = w4[(int64_t)(z + 8 * u) * total4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += a[u];
+      }
+      for (; z < r.parts; z += 8) s += w4[(int64_t)z * total4];
+    }
+    part4[q][j] = s;
+    __syncthreads();
+    if (q == 0 && i < total4) {
+      const f4 t = ((part4[0][j] + part4[1][j]) + (part4[2][j] + part4[3][j])) + ((part4[4][j] + part4[5][j]) + (part4[6][j] + part4[7][j]));
+      const int64_t e = flat0 + i * 4;
+      *(f4*)(g + e) = t;
+      if (!skip) {
+        f4 vw = *(const f4*)(w + e), a = *(const f4*)(s0 + e), bb = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+        if (NS > 1) bb = *(const f4*)(s1 + e);
+        if (NS > 2) c = *(const f4*)(s2 + e);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          float ww = vw[x], aa = a[x], b2 = bb[x], cc = c[x];
+          update_one<KIND>(ww, t[x], aa, b2, cc, p);
+          vw[x] = ww; a[x] = aa; bb[x] = b2; c[x] = cc;
+        }
+        *(f4*)(w + e) = vw;
+        *(f4*)(s0 + e) = a;
+        if (NS > 1) *(f4*)(s1 + e) = bb;
+        if (NS > 2) *(f4*)(s2 + e) = c;
+      }
+    }
+  } else {
+    // gemm_small_reduce_kernel's order: a block owns 4 outputs, 64 lanes each walk every 64th partial
+    const int ol = threadIdx.x & 3, pl = threadIdx.x >> 2;
+    const int o = lb * 4 + ol;
+    float s = 0.f;
+    if (o < r.outs) {
+      for (int i = pl; i < r.parts; i += 64 * 8) {  // 8 loads in flight, added in part order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = i + 64 * u < r.parts ? r.partial[(int64_t)(i + 64 * u) * r.outs + o] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+      }
+    }
+    part1[pl][ol] = s;
+    __syncthreads();
+    if (threadIdx.x < 4 && o < r.outs) {
+      float t = 0.f;
+#pragma unroll 8
+      for (int j = 0; j < 64; ++j) t += part1[j][ol];
+      const int64_t e = flat0 + o;
+      g[e] = t;
+      if (!skip) {
+        float ww = w[e], aa = s0[e], b2 = NS > 1 ? s1[e] : 0.f, cc = NS > 2 ? s2[e] : 0.f;
+        update_one<KIND>(ww, t, aa, b2, cc, p);
+        w[e] = ww; s0[e] = aa;
+        if (NS > 1) s1[e] = b2;
+        if (NS > 2) s2[e] = cc;
+      }
+    }
+  }
+}
+
+template <int KIND>
+static int launch_finish_t(sn_ctx* ctx, float* w, float* g, float* s0, float* s1, float* s2, int64_t n, const OptScalars& p, const FinishPlan& plan,
+                           int blocks, const int* skip_if) {
+  LaunchScope scope(ctx, "gradient_sums_and_optimizer");
+  hipLaunchKernelGGL((finish_kernel<KIND>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w, g, s0, s1, s2, n, p, plan, skip_if);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
+int launch_finish(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, float* g, float* s0, float* s1, float* s2, int64_t n, int iter,
+                  const DeferredReduce* defs, int n_defs, const int* skip_if) {
+  const int ns = opt_state_count(d.kind);
+  SN_REQUIRE(ns > 0, "unknown optimizer kind %d", d.kind);
+  SN_REQUIRE(w && g && s0 && (ns < 2 || s1) && (ns < 3 || s2), "optimizer kind %d needs %d state buffers", d.kind, ns);
+  SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
+  SN_REQUIRE(n_defs >= 1 && n_defs <= MAX_DEFERRED, "launch_finish takes 1..%d deferred reductions, got %d", MAX_DEFERRED, n_defs);
+  SN_REQUIRE(aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2), "launch_finish: buffers must be 16-byte aligned");
+  FinishPlan plan;
+  plan.n = n_defs;
+  int64_t blocks = ceil_div(ceil_div(n, 4), 128);
+  plan.block0[0] = (int)blocks;
+  for (int i = 0; i < n_defs; ++i) {
+    const DeferredReduce& r = defs[i];
+    SN_REQUIRE((r.kind == 1 || r.kind == 2) && r.partial && r.dst && r.parts >= 1 && r.outs >= 4 && r.outs % 4 == 0, "launch_finish: malformed reduction %d", i);
+    SN_REQUIRE(r.dst >= g && r.dst + r.outs <= g + n && (r.dst - g) % 4 == 0, "launch_finish: reduction %d does not write into the gradient buffer", i);
+    plan.r[i] = r;
+    plan.first[i] = r.dst - g;
+    blocks += r.kind == 1 ? ceil_div(r.outs / 4, 32) : ceil_div(r.outs, 4);
+    plan.block0[i + 1] = (int)blocks;
+  }
+  SN_REQUIRE(blocks <= 0x7fffffff, "launch_finish: %lld elements exceed one launch", (long long)n);
+  const OptScalars p = make_opt_scalars(d, iter);
+  switch (d.kind) {
+    case SN_OPT_SGD: return launch_finish_t<SN_OPT_SGD>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_ADAGRAD: return launch_finish_t<SN_OPT_ADAGRAD>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_ADADELTA: return launch_finish_t<SN_OPT_ADADELTA>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_RMSPROP: return launch_finish_t<SN_OPT_RMSPROP>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_ADAM: return launch_finish_t<SN_OPT_ADAM>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_NADAM: return launch_finish_t<SN_OPT_NADAM>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    case SN_OPT_ADAMAX: return launch_finish_t<SN_OPT_ADAMAX>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+    default: return launch_finish_t<SN_OPT_AMSGRAD>(ctx, w, g, s0, s1, s2, n, p, plan, (int)blocks, skip_if);
+  }
+}
+
+// the sums alone, when no optimizer launch follows
+__global__ __launch_bounds__(256) void deferred_reduce_kernel(DeferredReduce r) {
+  __shared__ f4 part4[8][32];
+  __shared__ float part1[64][4];
+  if (r.kind == 1) {
+    const int64_t total4 = r.outs / 4;
+    const int q = threadIdx.x >> 5, j = threadIdx.x & 31;
+    const int64_t i = (int64_t)blockIdx.x * 32 + j;
+    f4 s = {0.f, 0.f, 0.f, 0.f};
+    if (i < total4) {
+      const f4* w4 = reinterpret_cast<const f4*>(r.partial) + i;
+      int z = q;
+      for (; z + 56 < r.parts; z += 64) {
+        f4 a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = w4[(int64_t)(z + 8 * u) * total4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += a[u];
+      }
+      for (; z < r.parts; z += 8) s += w4[(int64_t)z * total4];
+    }
+    part4[q][j] = s;
+    __syncthreads();
+    if (q == 0 && i < total4)
+      reinterpret_cast<f4*>(r.dst)[i] = ((part4[0][j] + part4[1][j]) + (part4[2][j] + part4[3][j])) + ((part4[4][j] + part4[5][j]) + (part4[6][j] + part4[7][j]));
+  } else {
+    const int ol = threadIdx.x & 3, pl = threadIdx.x >> 2;
+    const int o = blockIdx.x * 4 + ol;
+    float s = 0.f;
+    if (o < r.outs) {
+      for (int i = pl; i < r.parts; i += 64 * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = i + 64 * u < r.parts ? r.partial[(int64_t)(i + 64 * u) * r.outs + o] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+      }
+    }
+    part1[pl][ol] = s;
+    __syncthreads();
+    if (threadIdx.x < 4 && o < r.outs) {
+      float t = 0.f;
+#pragma unroll 8
+      for (int j = 0; j < 64; ++j) t += part1[j][ol];
+      r.dst[o] = t;
+    }
+  }
+}
+
+int launch_deferred_reduce(sn_ctx* ctx, const DeferredReduce& d) {
+  SN_REQUIRE((d.kind == 1 || d.kind == 2) && d.partial && d.dst && d.outs % 4 == 0, "malformed deferred reduction");
+  LaunchScope scope(ctx, d.kind == 1 ? "splitk_reduce" : "small_output_reduce");
+  const int64_t blocks = d.kind == 1 ? ceil_div(d.outs / 4, 32) : ceil_div(d.outs, 4);
+  hipLaunchKernelGGL(deferred_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, d);
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
 // ---- K-replica average --------------------------------------------------------------------
 struct AvgOutputs {
   float* p[SN_MAX_AVG_INPUTS + 1];
