@@ -373,6 +373,13 @@ int launch_lstm_dh(sn_ctx* ctx, const float* dz, int rows, int H, const LstmWeig
 int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, int T, const LstmWeights& w, float* dx, float* ws,
                    int64_t ws_elems, int gates = 4);
 // dWk = X^T dZ, dWr = Hprev^T dZ over all steps (dz_all, h_all time-major [T,rows,*]; h_all[t] = h_{t-1})
+// The same gradient with all F + H rows x 128 columns per workgroup and one k range each (F <= 32, H in {64, 128, 256},
+// gates * H a multiple of 128): `ranges_out` partial results [F + H + 1, gates * H] (last row: column sums of dz, the
+// bias gradient) land in ws for the caller to add.  lstm_wgrad_rows_workspace: floats of ws it needs (0: shape not taken).
+bool lstm_wgrad_rows_ok(const sn_ctx* ctx, const float* x, const float* h, const float* dz, int rows, int T, int F, int H, int gates);
+int64_t lstm_wgrad_rows_workspace(const sn_ctx* ctx, int rows, int T, int F, int H, int gates);
+int launch_lstm_wgrad_rows(sn_ctx* ctx, const float* x, const float* h, const float* dz, int rows, int T, int F, int H, int gates, float* ws,
+                           int64_t ws_elems, int* ranges_out);
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
                       const LstmGrads& g, float* ws, int64_t ws_elems, int gates = 4);
 // The simple recurrent cell is the same four products with one gate (gates = 1): its weights sit in slot 0.

@@ -1662,6 +1662,25 @@ int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, 
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
                       const LstmGrads& g, float* ws, int64_t ws_elems, int gates) {
   const bool has_bias = g.b[0] != nullptr;
+  if (ws && lstm_wgrad_rows_ok(ctx, x, h_prev_all, dz_all, rows, T, F, H, gates) &&
+      lstm_wgrad_rows_workspace(ctx, rows, T, F, H, gates) <= ws_elems && aligned16(ws)) {
+    // all F + H rows x 128 columns per workgroup, one k range each; then the ranges are added into the layer's tensors
+    int ranges = 0;
+    SN_TRY(launch_lstm_wgrad_rows(ctx, x, h_prev_all, dz_all, rows, T, F, H, gates, ws, ws_elems, &ranges));
+    LstmWgradEpilogue ep{g, F, H};
+    const int Mo = F + H + 1, No = gates * H;
+    const int64_t total = (int64_t)Mo * No;
+    LaunchScope scope(ctx, "splitk_reduce");
+    if (total % 4 == 0) {
+      const int64_t blocks = std::min<int64_t>(ceil_div(total / 4, 32), (int64_t)ctx->compute_units * 16);
+      hipLaunchKernelGGL((splitk_reduce4_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, ranges, Mo, No, ep);
+    } else {
+      const int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
+      hipLaunchKernelGGL((splitk_reduce_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, ranges, Mo, No, ep);
+    }
+    SN_HIP(hipGetLastError());
+    return SN_OK;
+  }
   const int M = F + H + (has_bias ? 1 : 0);
   LstmWgradA al{x, h_prev_all, rows, T, F, H, M};
   StridedLoader<false> bl{dz_all, 1, (int64_t)gates * H, gates * H};

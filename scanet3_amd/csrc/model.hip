@@ -324,6 +324,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ws = std::max(ws, gemm_workspace_elems(B, op.H, 4 * op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.F, 4 * op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(op.F + op.H + 1, 4 * op.H, op.T * B, cu));
+        ws = std::max(ws, lstm_wgrad_rows_workspace(m->ctx, B, op.T, op.F, op.H, 4));
         ++i;
         break;
       }
@@ -370,6 +371,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ws = std::max(ws, gemm_workspace_elems(B, op.H, op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(B, op.F, op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(op.F + op.H, op.H, op.T * B, cu));
+        ws = std::max(ws, lstm_wgrad_rows_workspace(m->ctx, B, op.T, op.F, op.H, 1));
         ++i;
         break;
       }
@@ -1066,7 +1068,11 @@ static int update(sn_replica* r, int iter) {
   // A one-launch recurrent kernel of an earlier pass that gave up is reported before anything moves (the flag sits in
   // pinned host memory: no synchronisation needed to look); one of THIS step's passes that gives up, which the host
   // cannot know yet, makes the optimizer launch below leave weights and optimizer state as they are.
-  if (r->ctx->seq_gave_up && *(volatile int*)r->ctx->seq_gave_up != 0) return check_async(r->ctx);
+  if (r->ctx->seq_gave_up && *(volatile int*)r->ctx->seq_gave_up != 0) {
+    // kernels queued behind the one that gave up may do the same: let them end, so that this is reported once
+    SN_HIP(hipStreamSynchronize(r->ctx->stream));
+    return check_async(r->ctx);
+  }
   // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
   // the statistics are those of the gradient pass that has just run.  In bf16 mode the optimizer writes the bf16 copy of
   // what it updates in the same pass (every Dense weight is trainable), so the copies stay current.
