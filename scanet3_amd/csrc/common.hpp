@@ -380,6 +380,8 @@ bool lstm_wgrad_rows_ok(const sn_ctx* ctx, const float* x, const float* h, const
 int64_t lstm_wgrad_rows_workspace(const sn_ctx* ctx, int rows, int T, int F, int H, int gates);
 int launch_lstm_wgrad_rows(sn_ctx* ctx, const float* x, const float* h, const float* dz, int rows, int T, int F, int H, int gates, float* ws,
                            int64_t ws_elems, int* ranges_out);
+// adds `parts` partial sums [F + H + 1][gates * H] (rows: x features, h features, column sums of dz) into the layer's tensors
+int launch_lstm_wgrad_reduce(sn_ctx* ctx, const float* ws, int parts, int F, int H, int gates, const LstmGrads& g);
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
                       const LstmGrads& g, float* ws, int64_t ws_elems, int gates = 4);
 // The simple recurrent cell is the same four products with one gate (gates = 1): its weights sit in slot 0.
@@ -413,8 +415,14 @@ int launch_lstm_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int h0_v
 // and cell states, the gradient of the last hidden state (dh_last, may be null) and of a returned sequence (dy_seq
 // [rows, T, H], may be null).  lstm_sequence_bwd_ok: as for the forward launch.
 bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w);
+// With x [rows, T, F], h (T + 1 slices, slice t = h_{t-1}) and a workspace the same launch also accumulates the weight
+// gradient where the shape allows it (H 64, 128 or 256; F even up to 32 or a multiple of 4 up to 64): *wgrad_parts partial
+// sums [F + H + 1][4H] are left in ws for launch_lstm_wgrad_reduce, or *wgrad_parts = 0 and the caller runs
+// launch_lstm_wgrad.  lstm_sequence_bwd_wgrad_workspace: floats of ws that takes (0: the shape cannot).
+int64_t lstm_sequence_bwd_wgrad_workspace(int rows, int T, int F, int H);
 int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
-                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice);
+                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice, const float* x = nullptr, const float* h = nullptr,
+                             int F = 0, float* ws = nullptr, int64_t ws_elems = 0, int* wgrad_parts = nullptr);
 int launch_lstm_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const float* h_prev, const float* c_prev, int rows, int H,
                          const LstmWeights& w, const float* wpack, float* gates, float* c, float* h);
 // dh_parts[g] (g = 0..3, part_stride elements apart) = dz[:, g*H:(g+1)*H] * Wr_g^T; their sum is dh_prev

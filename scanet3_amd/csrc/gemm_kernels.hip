@@ -1659,6 +1659,22 @@ int launch_lstm_dx(sn_ctx* ctx, const float* dz, int rows, int H, int F, int t, 
   return launch_any<false>(ctx, "lstm_input_gradient", rows, F, gates * H, al, bl, ep, ws, ws_elems);
 }
 
+int launch_lstm_wgrad_reduce(sn_ctx* ctx, const float* ws, int parts, int F, int H, int gates, const LstmGrads& g) {
+  LstmWgradEpilogue ep{g, F, H};
+  const int Mo = F + H + 1, No = gates * H;
+  const int64_t total = (int64_t)Mo * No;
+  LaunchScope scope(ctx, "splitk_reduce");
+  if (total % 4 == 0) {
+    const int64_t blocks = std::min<int64_t>(ceil_div(total / 4, 32), (int64_t)ctx->compute_units * 16);
+    hipLaunchKernelGGL((splitk_reduce4_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, ws, parts, Mo, No, ep);
+  } else {
+    const int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
+    hipLaunchKernelGGL((splitk_reduce_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, ws, parts, Mo, No, ep);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
 int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, const float* dz_all, int rows, int T, int F, int H,
                       const LstmGrads& g, float* ws, int64_t ws_elems, int gates) {
   const bool has_bias = g.b[0] != nullptr;
@@ -1667,19 +1683,7 @@ int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, cons
     // all F + H rows x 128 columns per workgroup, one k range each; then the ranges are added into the layer's tensors
     int ranges = 0;
     SN_TRY(launch_lstm_wgrad_rows(ctx, x, h_prev_all, dz_all, rows, T, F, H, gates, ws, ws_elems, &ranges));
-    LstmWgradEpilogue ep{g, F, H};
-    const int Mo = F + H + 1, No = gates * H;
-    const int64_t total = (int64_t)Mo * No;
-    LaunchScope scope(ctx, "splitk_reduce");
-    if (total % 4 == 0) {
-      const int64_t blocks = std::min<int64_t>(ceil_div(total / 4, 32), (int64_t)ctx->compute_units * 16);
-      hipLaunchKernelGGL((splitk_reduce4_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, ranges, Mo, No, ep);
-    } else {
-      const int64_t blocks = std::min<int64_t>(ceil_div(total, 32), (int64_t)ctx->compute_units * 16);
-      hipLaunchKernelGGL((splitk_reduce_kernel<LstmWgradEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, ranges, Mo, No, ep);
-    }
-    SN_HIP(hipGetLastError());
-    return SN_OK;
+    return launch_lstm_wgrad_reduce(ctx, ws, ranges, F, H, gates, g);
   }
   const int M = F + H + (has_bias ? 1 : 0);
   LstmWgradA al{x, h_prev_all, rows, T, F, H, M};

@@ -830,15 +830,54 @@ struct SeqBwdArgs {
   int* gave_up;
   int* failed;
   int force_coherent;
+  // the weight gradient riding along (XW > 0 instantiations only)
+  const float* x;        // [rows, T, F]
+  const float* h;        // T + 1 slices, slice t = h_{t-1}
+  float* wpartial;       // [row_groups][F + H + 1][4H]: every row group's own sum over its rows and all steps
+  int F;
 };
 
-template <int NKB>  // 16-long k blocks per wavefront: H = 16 NKB
-__global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
+// The weight gradient can ride along (XW > 0: x features per lane, 2 or 4; H a multiple of 64).  dW[m, n] = sum over
+// (t, row) of [x_t | h_{t-1}][row, m] * dz_t[row, n], and a workgroup holds its 16 rows x 64 columns of dz_t the moment it
+// has computed them: it keeps the [F + H, 64] block of the sum that belongs to its rows and columns in accumulator
+// registers for the whole launch.  Per step the dz tile goes to LDS (the B operand: lane (n, g) reads row g + 4 i), the
+// operand rows come straight from memory a step ahead (lane (m, g) holds 4 consecutive features of row g + 4 i, so MFMA
+// (j, i) multiplies features {4 m + j} by rows {g + 4 i}: accumulator tile j collects every fourth feature), and the
+// multiplications run between the workgroup's arrival and its wait for the others, where its wavefronts would idle.
+// Wavefront w owns a 64-feature run of h (all its gate tiles, or a share of them when H < 256) and the x features of gate
+// tile w.  The bias gradient is each thread's running sum of its own four dz values, added over the 16 rows at the end.
+// What leaves is one partial [F + H + 1, 4H] per row group, which splitk_reduce adds in a fixed order.
+constexpr int DZP = 80;  // row pitch of the dz tile in LDS: rows g and g + 1 land in different halves of the banks
+
+// LDS-direct loads of blocks KB .. NKB - 1 of a 16-row operand: block kb = 64 bytes of every row, 1 KiB of LDS
+template <int KB, int NKB, int AUX>
+__device__ __forceinline__ void load_row_blocks(global_ptr_t ap, float* aw) {
+  if constexpr (KB < NKB) {
+    __builtin_amdgcn_global_load_lds(ap, (lds_ptr_t)(aw + KB * (256 - 16)), 16, 64 * KB, AUX);
+    load_row_blocks<KB + 1, NKB, AUX>(ap, aw);
+  }
+}
+
+// base + a per-lane BYTE offset of 32 bits: the form the compiler turns into "scalar base + one offset register" accesses
+template <typename T>
+__device__ __forceinline__ T* at_bytes(T* uniform_base, unsigned byte_offset) {
+  return (T*)((char*)uniform_base + byte_offset);
+}
+template <typename T>
+__device__ __forceinline__ const T* at_bytes(const T* uniform_base, unsigned byte_offset) {
+  return (const T*)((const char*)uniform_base + byte_offset);
+}
+
+template <int NKB, int XW>  // 16-long k blocks per wavefront: H = 16 NKB
+__device__ __forceinline__ void lstm_sequence_bwd_body(const SeqBwdArgs& a) {
   constexpr int UB = 16, H = 16 * NKB;
+  constexpr bool WG = XW > 0;
+  constexpr int S = WG ? NKB / 4 : 1;  // 64-feature runs of h = gate tiles per wavefront
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
   float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial dh
   float* As = lds + 4 * SRB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]: dz_t as the loads deliver it
+  float* Dzs = As + SRB * 4 * H;   // [SRB][DZP]: this workgroup's own 64 columns of dz_t (weight gradient only)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
   const int rg = (blockIdx.x & 7) + 8 * (slot / a.unit_groups), ug = slot % a.unit_groups;
@@ -870,31 +909,91 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
   // the cell this thread owns: row tid / 16, unit tid % 16
   const int crow = tid >> 4, cu = tid & 15;
   const bool live = r0 + crow < a.rows;
-  const int64_t cr = live ? r0 + crow : 0;
-  const int64_t ci = cr * H + u0 + cu, zi = cr * 4 * H + u0 + cu, yi = cr * a.T * H + u0 + cu;
+  // per-lane offsets are unsigned 32-bit byte counts (the launch checks the sizes): with a uniform base per access they
+  // travel as one register and the base in scalar registers
+  const unsigned cr = live ? r0 + crow : 0;
+  unsigned ci = 4u * (cr * H + u0 + cu), zi = 4u * (cr * 4 * H + u0 + cu);
+  const int64_t yi = (int64_t)cr * a.T * H + u0 + cu;
   float f, in, gg, o, cc, cp, dyv, dh, dcv = 0.f;
   {
     const int t = a.T - 1;
-    const float* gt = a.gates + (int64_t)t * 4 * a.slice + zi;
-    f = gt[0];
-    in = gt[H];
-    gg = gt[2 * H];
-    o = gt[3 * H];
-    cc = a.c[(int64_t)t * a.slice + ci];
-    cp = t > 0 ? a.c[(int64_t)(t - 1) * a.slice + ci] : (a.c0 ? a.c0[ci] : 0.f);
+    const float* gt = a.gates + (int64_t)t * 4 * a.slice;
+    f = *at_bytes(gt, zi);
+    in = *at_bytes(gt + H, zi);
+    gg = *at_bytes(gt + 2 * H, zi);
+    o = *at_bytes(gt + 3 * H, zi);
+    cc = *at_bytes(a.c + (int64_t)t * a.slice, ci);
+    cp = t > 0 ? *at_bytes(a.c + (int64_t)(t - 1) * a.slice, ci) : (a.c0 ? *at_bytes(a.c0, ci) : 0.f);
     dyv = a.dy_seq ? a.dy_seq[yi + (int64_t)t * H] : 0.f;
-    dh = a.dh_last ? a.dh_last[ci] : 0.f;
+    dh = a.dh_last ? *at_bytes(a.dh_last, ci) : 0.f;
   }
   // One load instruction brings a 16-row x 16-k block of dz_t to 1 KiB of LDS, lane p to bytes 16 p .. 16 p + 15: four
   // neighbouring lanes fetch the 64 contiguous bytes of one row (rows past the batch: the last row again, their results
   // belong to no cell), and chunk c of row r lands in slot c ^ (r / 4) of the row so that the 16 lanes that later read
   // one chunk index of 16 rows hit 16 different bank groups.
-  const int64_t a_off = (int64_t)min(r0 + (lane >> 2), a.rows - 1) * 4 * H + wave * H + 4 * ((lane & 3) ^ (lane >> 4));
+  unsigned a_off = 4u * ((unsigned)min(r0 + (lane >> 2), a.rows - 1) * 4 * H + 4 * ((lane & 3) ^ (lane >> 4)));
   float* aw = As + wave * NKB * 256;
   const float* ar = aw + (row16 * 4 + (g ^ (row16 >> 2))) * 4;
   bool spread = true;  // until arrival 0 is complete (the first wait below), write as if the row group were spread out
+  // ---- weight gradient: accumulators, operand addresses and the operand rows of the first step
+  const int sw = wave / (4 / S), nt0 = (wave % (4 / S)) * S;  // this wavefront's run of h features and its first gate tile
+  f4v acch[WG ? 4 : 1][S], accx[WG ? XW : 1];
+  typedef float xwv __attribute__((ext_vector_type(WG ? XW : 2)));
+  f4v ah[4];
+  xwv ax[4];
+  float bsum[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool x_lane = XW * row16 < a.F;  // lanes past the last feature load the row's first ones and multiply zeros
+  // (the batch is a multiple of 16 rows here: row g + 4 i is a uniform distance from row g, one per-lane offset serves all four)
+  unsigned hoff = 4u * (g * H + 4 * row16), xoff = 4u * (g * a.T * a.F + (x_lane ? XW * row16 : 0));
+  auto request_operands = [&](int t) {  // [x_t | h_{t-1}] of rows g + 4 i: 16 bytes of h and XW floats of x per lane and row
+    const float* hs = a.h + (int64_t)t * a.slice + r0 * H + 64 * sw;
+    const float* xs = a.x + ((int64_t)r0 * a.T + t) * a.F;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ah[i] = *(const f4v*)at_bytes(hs + 4 * i * H, hoff);
+      ax[i] = *(const xwv*)at_bytes(xs + (int64_t)4 * i * a.T * a.F, xoff);
+    }
+  };
+  if constexpr (WG) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int n = 0; n < S; ++n) acch[j][n] = f4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < XW; ++j) accx[j] = f4v{0.f, 0.f, 0.f, 0.f};
+    request_operands(a.T - 1);
+  }
+  // These multiplications are off the chain the next step waits for; the other workgroup of the CU may be on its chain, so
+  // they run at the lower of two wavefront priorities.
+  auto weight_gradient_step = [&]() {  // += [x_t | h_{t-1}]^T (16 rows) * dz_t (the tile in LDS)
+    const float* dzr = Dzs + g * DZP + row16;
+    __builtin_amdgcn_s_setprio(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float bx = dzr[4 * i * DZP + 16 * wave];
+#pragma unroll
+      for (int j = 0; j < XW; ++j) accx[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(x_lane ? ax[i][j] : 0.f, bx, accx[j], 0, 0, 0);
+#pragma unroll
+      for (int n = 0; n < S; ++n) {
+        const float bh = dzr[4 * i * DZP + 16 * (nt0 + n)];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acch[j][n] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[i][j], bh, acch[j][n], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_setprio(1);
+  };
+  if constexpr (WG) __builtin_amdgcn_s_setprio(1);
   for (int t = a.T - 1;; --t) {
+    // (opaque per step: otherwise the compiler folds each offset into a 64-bit per-lane pointer of its own that it carries
+    // through the loop, two registers per access instead of one for all)
+    asm volatile("" : "+v"(ci), "+v"(zi), "+v"(a_off), "+v"(hoff), "+v"(xoff));
     // ---- gate gradients of step t
+    if constexpr (WG) {
+      if (!live) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) Dzs[crow * DZP + 16 * q + cu] = 0.f;
+      }
+    }
     if (live) {
       const float tc = tanhf(cc);
       float d = dh;
@@ -907,49 +1006,64 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
       const float dzg = (1.0f - gg * gg) * dg;
       const float dzo = (o * (1.0f - o)) * d_o;
       dcv = dc * f;
-      float* zt = a.dz + (int64_t)t * 4 * a.slice + zi;
+      float* zt = a.dz + (int64_t)t * 4 * a.slice;
       if (spread) {
-        __hip_atomic_store(zt, dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(zt + H, dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(zt + 2 * H, dzg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(zt + 3 * H, dzo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(at_bytes(zt, zi), dzf, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(at_bytes(zt + H, zi), dzi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(at_bytes(zt + 2 * H, zi), dzg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(at_bytes(zt + 3 * H, zi), dzo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
-        zt[0] = dzf;
-        zt[H] = dzi;
-        zt[2 * H] = dzg;
-        zt[3 * H] = dzo;
+        *at_bytes(zt, zi) = dzf;
+        *at_bytes(zt + H, zi) = dzi;
+        *at_bytes(zt + 2 * H, zi) = dzg;
+        *at_bytes(zt + 3 * H, zi) = dzo;
+      }
+      if constexpr (WG) {
+        float* dl = Dzs + crow * DZP + cu;
+        dl[0] = dzf;
+        dl[16] = dzi;
+        dl[32] = dzg;
+        dl[48] = dzo;
+        bsum[0] += dzf;
+        bsum[1] += dzi;
+        bsum[2] += dzg;
+        bsum[3] += dzo;
       }
     }
-    if (t == 0) break;
+    if (!WG && t == 0) break;
     // ---- hand dz_t over: stores acknowledged in every wavefront, then one thread counts the workgroup in
+    //      (with the weight gradient the last step comes this far too: the barrier publishes its dz tile)
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0)
     __syncthreads();
-    if (tid == 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0 && t > 0) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- what step t - 1 needs from the forward pass is requested while the others arrive
-    {
-      const float* gt = a.gates + (int64_t)(t - 1) * 4 * a.slice + zi;
-      f = gt[0];
-      in = gt[H];
-      gg = gt[2 * H];
-      o = gt[3 * H];
+    if (t > 0) {
+      const float* gt = a.gates + (int64_t)(t - 1) * 4 * a.slice;
+      f = *at_bytes(gt, zi);
+      in = *at_bytes(gt + H, zi);
+      gg = *at_bytes(gt + 2 * H, zi);
+      o = *at_bytes(gt + 3 * H, zi);
       cc = cp;
-      cp = t > 1 ? a.c[(int64_t)(t - 2) * a.slice + ci] : (a.c0 ? a.c0[ci] : 0.f);
+      cp = t > 1 ? *at_bytes(a.c + (int64_t)(t - 2) * a.slice, ci) : (a.c0 ? *at_bytes(a.c0, ci) : 0.f);
       dyv = a.dy_seq ? a.dy_seq[yi + (int64_t)(t - 1) * H] : 0.f;
+    }
+    // ---- this step's share of the weight gradient while the others arrive (the tile was published by the barrier above),
+    //      then the operand rows of step t - 1, which have a whole step to land
+    if constexpr (WG) {
+      weight_gradient_step();
+      if (t == 0) break;
+      request_operands(t - 1);
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
     if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
     if (done == 0) spread = __hip_atomic_load(my_spread, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     // ---- dh_{t-1} of this workgroup's cells = dz_t (16 complete rows) * the weight slab
     {
-      const float* ap = a.dz + (int64_t)t * 4 * a.slice + a_off;
-      if (spread) {
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-          __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 16);  // sc1: coherent at device scope
-      } else {
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) __builtin_amdgcn_global_load_lds((global_ptr_t)(ap + 16 * kb), (lds_ptr_t)(aw + kb * 256), 16, 0, 0);
-      }
+      // Block kb lies 64 kb bytes further along the row and 1024 kb bytes further in LDS.  The instruction's immediate offset
+      // moves both addresses, so one per-lane address serves all blocks: the LDS base handed over is 64 kb bytes short.
+      const global_ptr_t ap = (global_ptr_t)at_bytes(a.dz + (int64_t)t * 4 * a.slice + wave * H, a_off);
+      if (spread) load_row_blocks<0, NKB, 16>(ap, aw);  // sc1: coherent at device scope
+      else load_row_blocks<0, NKB, 0>(ap, aw);
       // The blocks are this wavefront's own, so no barrier: block kb is multiplied as soon as all but the NKB - 1 - kb loads
       // behind it have landed (loads return in order; the compiler does not order LDS reads behind these loads by itself).
       f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
@@ -966,9 +1080,50 @@ __global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
     __syncthreads();
     dh = (Ps[crow * ZP + cu] + Ps[(SRB + crow) * ZP + cu]) + (Ps[(2 * SRB + crow) * ZP + cu] + Ps[(3 * SRB + crow) * ZP + cu]);
   }
+  if constexpr (WG) {
+    // ---- this row group's partial: rows 0..F-1 (x), F..F+H-1 (h), F+H (column sums of dz)
+    const int N = 4 * H;
+    float* out = a.wpartial + (int64_t)rg * (a.F + H + 1) * N + u0 + row16;
+#pragma unroll
+    for (int j = 0; j < XW; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int m = XW * (4 * g + v) + j;
+        if (m < a.F) out[(int64_t)m * N + wave * H] = accx[j][v];
+      }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int n = 0; n < S; ++n)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) out[(int64_t)(a.F + 64 * sw + 4 * (4 * g + v) + j) * N + (nt0 + n) * H] = acch[j][n][v];
+    __syncthreads();  // every wavefront has read the tile: it now carries the per-thread column sums
+#pragma unroll
+    for (int q = 0; q < 4; ++q) Dzs[crow * DZP + 16 * q + cu] = bsum[q];
+    __syncthreads();
+    if (tid < 64) {
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < SRB; ++r) sum += Dzs[r * DZP + tid];
+      a.wpartial[((int64_t)rg * (a.F + H + 1) + a.F + H) * N + (tid >> 4) * H + u0 + (tid & 15)] = sum;
+    }
+  }
 }
 
-size_t sequence_bwd_lds_bytes(int H) { return ((size_t)4 * SRB * ZP + (size_t)SRB * 4 * H) * sizeof(float); }
+template <int NKB>
+__global__ __launch_bounds__(256) void lstm_sequence_bwd_kernel(SeqBwdArgs a) {
+  lstm_sequence_bwd_body<NKB, 0>(a);
+}
+
+// two workgroups per CU = two wavefronts per SIMD: 256 registers each
+template <int NKB, int XW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void lstm_sequence_bwd_wgrad_kernel(SeqBwdArgs a) {
+  lstm_sequence_bwd_body<NKB, XW>(a);
+}
+
+size_t sequence_bwd_lds_bytes(int H, bool with_wgrad = false) {
+  return ((size_t)4 * SRB * ZP + (size_t)SRB * 4 * H + (with_wgrad ? (size_t)SRB * DZP : 0)) * sizeof(float);
+}
 
 size_t lds_bytes(int K, int cols) {  // cols: output columns per workgroup (64 or 32)
   const int K16 = round16(K);
@@ -1159,7 +1314,7 @@ static bool lstm_sequence_bwd_fits(sn_ctx* ctx, int rows, int H, const LstmWeigh
   for (int g = 0; g < 4; ++g)
     if (!aligned16(w.wr[g])) return false;
   const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
-  if (groups > SEQ_MAX_GROUPS) return false;
+  if (groups > SEQ_MAX_GROUPS || (int64_t)rows * 4 * H >= ((int64_t)1 << 30)) return false;  // (the kernel's per-lane byte offsets are 32-bit)
   bool fits = false;
   const bool known = with_sequence_bwd_kernel(H, [&](auto kernel) {
     if (allow_dynamic_lds(ctx, (const void*)kernel, sequence_bwd_lds_bytes(H)) != SN_OK) return;
@@ -1171,19 +1326,80 @@ static bool lstm_sequence_bwd_fits(sn_ctx* ctx, int rows, int H, const LstmWeigh
 }
 bool lstm_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const LstmWeights& w) { return !sequence_kernels_off(ctx) && lstm_sequence_bwd_fits(ctx, rows, H, w); }
 
+namespace {
+// calls f(kernel) for the instantiation that also accumulates the weight gradient, or returns false
+template <typename Fn>
+bool with_sequence_bwd_wgrad_kernel(int H, int F, Fn&& f) {
+  const int xw = F % 2 == 0 && F <= 32 ? 2 : (F % 4 == 0 && F <= 64 ? 4 : 0);
+  if (xw == 0) return false;
+  switch (H * 8 + xw) {
+    case 64 * 8 + 2: f(lstm_sequence_bwd_wgrad_kernel<4, 2>); return true;
+    case 64 * 8 + 4: f(lstm_sequence_bwd_wgrad_kernel<4, 4>); return true;
+    case 128 * 8 + 2: f(lstm_sequence_bwd_wgrad_kernel<8, 2>); return true;
+    case 128 * 8 + 4: f(lstm_sequence_bwd_wgrad_kernel<8, 4>); return true;
+    case 256 * 8 + 2: f(lstm_sequence_bwd_wgrad_kernel<16, 2>); return true;
+    case 256 * 8 + 4: f(lstm_sequence_bwd_wgrad_kernel<16, 4>); return true;
+    default: return false;
+  }
+}
+
+bool sequence_wgrad_wanted() {  // SCANET_SEQUENCE_WGRAD=0 keeps the weight gradient in its own launch
+  const char* e = getenv("SCANET_SEQUENCE_WGRAD");
+  return !(e && e[0] == '0');
+}
+}  // namespace
+
+// Floats of workspace the backward launch needs to carry the weight gradient along (one partial per 16-row group), or 0
+// where it cannot (shape).
+int64_t lstm_sequence_bwd_wgrad_workspace(int rows, int T, int F, int H) {
+  if (rows <= 0 || rows % SRB != 0 || T <= 0 || (int64_t)rows * T * F >= ((int64_t)1 << 30)) return 0;
+  if (!with_sequence_bwd_wgrad_kernel(H, F, [](auto) {})) return 0;
+  return ceil_div(rows, SRB) * (int64_t)(F + H + 1) * 4 * H;
+}
+
+static bool lstm_sequence_bwd_wgrad_fits(sn_ctx* ctx, int rows, int T, int F, int H, const float* x, const float* h, const float* ws, int64_t ws_elems) {
+  const int64_t need = lstm_sequence_bwd_wgrad_workspace(rows, T, F, H);
+  if (!sequence_wgrad_wanted() || need == 0 || !ws || need > ws_elems || !aligned16(x) || !aligned16(h)) return false;
+  const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+  bool fits = false;
+  with_sequence_bwd_wgrad_kernel(H, F, [&](auto kernel) {
+    if (allow_dynamic_lds(ctx, (const void*)kernel, sequence_bwd_lds_bytes(H, true)) != SN_OK) return;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, sequence_bwd_lds_bytes(H, true)) != hipSuccess) return;
+    fits = blocks <= (int64_t)per_cu * ctx->compute_units;
+  });
+  return fits;
+}
+
+// With x, h (T + 1 slices, slice t = h_{t-1}) and a workspace the launch also leaves the weight gradient's partial sums
+// [*wgrad_parts][F + H + 1][4H] in ws where the shape allows it (*wgrad_parts = 0 otherwise: the caller runs the product).
 int launch_lstm_sequence_bwd(sn_ctx* ctx, const float* gates, const float* c, const float* c0, const float* dh_last, const float* dy_seq, int T,
-                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice) {
+                             int rows, int H, const LstmWeights& w, float* dz, int64_t slice, const float* x, const float* h, int F, float* ws,
+                             int64_t ws_elems, int* wgrad_parts) {
+  if (wgrad_parts) *wgrad_parts = 0;
   if (rows <= 0 || T <= 0) return SN_OK;
   SN_REQUIRE(lstm_sequence_bwd_fits(ctx, rows, H, w), "lstm_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SN_REQUIRE(aligned16(dz), "lstm_sequence_backward: operands must start on 16-byte boundaries");
   const int groups = (int)ceil_div(rows, SRB);
+  const bool with_wgrad = wgrad_parts && x && h && lstm_sequence_bwd_wgrad_fits(ctx, rows, T, F, H, x, h, ws, ws_elems);
   unsigned* sync = nullptr;
   SN_TRY(seq_sync_take(ctx, groups, &sync));
   SeqBwdArgs a{gates, c, c0, dh_last, dy_seq, {w.wr[0], w.wr[1], w.wr[2], w.wr[3]}, dz, slice, rows, T, H, groups, H / 16,
-               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_failed_dev, ctx->seq_force_coherent};
+               sync, ctx->seq_spin_limit, ctx->seq_gave_up_dev, ctx->seq_failed_dev, ctx->seq_force_coherent, x, h, ws, F};
+  const dim3 grid((unsigned)(8 * ceil_div(groups, 8) * (H / 16)));
+  if (with_wgrad) {
+    // T - 1 products of rows x H x 4H and T of (F + H) x 4H x rows: as one shape, rows x 4H x ((T - 1) H + T (F + H)) / T per step
+    LaunchScope scope(ctx, "lstm_sequence_backward_and_weight_gradient", rows, 4 * H, (T - 1) * H + T * (F + H));
+    with_sequence_bwd_wgrad_kernel(H, F, [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, grid, dim3(256), sequence_bwd_lds_bytes(H, true), ctx->stream, a);
+    });
+    SN_HIP(hipGetLastError());
+    *wgrad_parts = groups;
+    return SN_OK;
+  }
   LaunchScope scope(ctx, "lstm_sequence_backward", rows * (T - 1), H, 4 * H);  // T - 1 products of rows x H x 4H
   with_sequence_bwd_kernel(H, [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(groups, 8) * (H / 16))), dim3(256), sequence_bwd_lds_bytes(H), ctx->stream, a);
+    hipLaunchKernelGGL(kernel, grid, dim3(256), sequence_bwd_lds_bytes(H), ctx->stream, a);
   });
   SN_HIP(hipGetLastError());
   return SN_OK;

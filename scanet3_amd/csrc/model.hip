@@ -325,6 +325,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ws = std::max(ws, gemm_workspace_elems(B, op.F, 4 * op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(op.F + op.H + 1, 4 * op.H, op.T * B, cu));
         ws = std::max(ws, lstm_wgrad_rows_workspace(m->ctx, B, op.T, op.F, op.H, 4));
+        if (B <= 1024) ws = std::max(ws, lstm_sequence_bwd_wgrad_workspace(B, op.T, op.F, op.H));  // one partial per 16 rows: up to 64 of them
         ++i;
         break;
       }
@@ -881,9 +882,18 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         const bool fused_bwd = fused && lstm_step_bwd_fused_ok(op.H, w);
         // every reverse step in one launch where the whole grid fits the device; the input gradients follow per step
         const bool whole = fused && op.T > 1 && lstm_sequence_bwd_ok(ctx, rows, op.H, w);
+        LstmGrads gr;
+        for (int gi = 0; gi < 4; ++gi) {
+          gr.wk[gi] = param_ptr(r, r->g, op.lstm_p[gi][0]);
+          gr.wr[gi] = param_ptr(r, r->g, op.lstm_p[gi][1]);
+          gr.b[gi] = param_ptr(r, r->g, op.lstm_p[gi][2]);
+        }
+        int wgrad_parts = 0;  // > 0: the backward launch has left the weight gradient's partial sums in the workspace
         if (whole) {
           SN_TRY(launch_lstm_sequence_bwd(ctx, r->lstm_gates[i], r->lstm_c[i], param_ptr(r, r->w, op.state_p[0]), op.ret_seq ? nullptr : dy,
-                                          op.ret_seq ? dy : nullptr, op.T, rows, op.H, w, r->lstm_dz[i], bh));
+                                          op.ret_seq ? dy : nullptr, op.T, rows, op.H, w, r->lstm_dz[i], bh, in, r->lstm_h[i], op.F, r->ws,
+                                          m->workspace_elems, &wgrad_parts));
+          if (wgrad_parts > 0) SN_TRY(launch_lstm_wgrad_reduce(ctx, r->ws, wgrad_parts, op.F, op.H, 4, gr));  // before the workspace's next user
           if (need_dx)
             for (int t = op.T - 1; t >= 0; --t)
               SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh * 4, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems));
@@ -923,13 +933,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
             hb ^= 1;
           }
         }
-        LstmGrads gr;
-        for (int gi = 0; gi < 4; ++gi) {
-          gr.wk[gi] = param_ptr(r, r->g, op.lstm_p[gi][0]);
-          gr.wr[gi] = param_ptr(r, r->g, op.lstm_p[gi][1]);
-          gr.b[gi] = param_ptr(r, r->g, op.lstm_p[gi][2]);
-        }
-        SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems));
+        if (wgrad_parts == 0) SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems));
         if (need_dx) cur ^= 1;
         break;
       }

@@ -1162,6 +1162,55 @@ def test_lstm_sequence_kernels_over_their_instantiations(S, ctx, units, features
     yb.free()
 
 
+@pytest.mark.parametrize("units,features,batch,T,second", [(64, 12, 48, 4, 16), (64, 64, 32, 3, 16), (128, 52, 32, 5, 16), (128, 28, 16, 2, 16),
+                                                           (256, 32, 48, 3, 16), (256, 36, 32, 4, 16), (64, 8, 32, 6, 64), (256, 32, 16, 1, 16)])
+def test_lstm_backward_launch_that_carries_the_weight_gradient(S, ctx, monkeypatch, units, features, batch, T, second):
+    """With 64, 128 or 256 units, a batch that is a multiple of 16 rows and at most 64 features the one-launch backward pass also accumulates the layer's weight gradient (a partial sum per 16-row group,
+    added by the reduction kernel).  Each instantiation against the oracle and against the separate product
+    (SCANET_SEQUENCE_WGRAD=0), with a second LSTM above; `second` = 64 makes that one take the same path with an input
+    gradient to deliver (its workspace is shared with the per-step input-gradient products), T = 1 has no hand-over."""
+    om = O.Model([O.LSTM(units, return_sequence=True), O.LSTM(second), O.Dense(2, O.ACT_IDENTITY)], O.LOSS_MSE)
+    layers = S.LSTM(units, returnSequence=True) >> S.LSTM(second) >> S.Dense(2, S.Identity)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+    rep = cm.replica(None)
+    rng = np.random.default_rng(5000 + units + features)
+    params = glorot_params(om, (batch, T, features), rng)
+    for p in params:
+        if params[p].ndim == 1:
+            params[p] = params[p] + rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
+    x = rng.standard_normal((batch, T, features)).astype(f32)
+    y = rng.uniform(-1, 1, (batch, 2)).astype(f32)
+    rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    oloss, ograds = om.grad(x, y, params)
+    ctx.profile_reset()
+    ctx.profile(True)
+    assert abs(rep.grad(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ctx.sync()
+    ctx.profile(False)
+    labels = list(ctx.profile_report())
+    if T > 1:
+        assert any(l.startswith("lstm_sequence_backward_and_weight_gradient") for l in labels), labels
+    ggrads = rep.get_grads()
+    _, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_GEMM, 3.0 * rel_err(ograds[p], grads64[p])), p
+    monkeypatch.setenv("SCANET_SEQUENCE_WGRAD", "0")
+    ctx.profile_reset()
+    ctx.profile(True)
+    rep.grad(xb, yb)
+    ctx.sync()
+    ctx.profile(False)
+    assert not any(l.startswith("lstm_sequence_backward_and_weight_gradient") for l in ctx.profile_report())
+    separate = rep.get_grads()
+    for p in ograds:
+        assert rel_err(ggrads[p], separate[p]) <= TOL_GEMM, p
+    for o in (rep, cm):
+        o.close()
+    xb.free()
+    yb.free()
+
+
 @pytest.mark.parametrize("kind", ["lstm", "simple_rnn"])
 def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
     """A workgroup of a one-launch recurrent kernel that waits for its neighbours polls a bounded number of times.  With the
