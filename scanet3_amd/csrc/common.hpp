@@ -304,9 +304,9 @@ int64_t dense_skinny_fwd_workspace(int rows, int in_f, int out_f);  // floats of
 int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,
                             int64_t ws_elems);
 
-// bf16 fast path (gemm_bf16.hip): C[M,N] = A[M,K] * Bt[N,K]^T, operands bf16 with k contiguous.
-// Besides the fp32 result (e.out, may be null) the epilogue can emit bf16 copies in both orientations,
-// which is how a Dense layer hands its output to the next one without a separate cast pass.
+// bf16 fast path (gemm_bf16.hip): the three products of a Dense layer on bf16 operands read as the tensors lie (no
+// transposed copies), fp32 accumulation.  Besides or instead of the fp32 result (e.out, may be null) the epilogue can
+// emit the result as bf16, which is how a Dense layer hands its output to the next one without a separate cast pass.
 struct EpilogueBf16 {
   Epilogue e;                // e.out may be null when out_bf is set; e.act: identity or ReLU only
   void* out_bf = nullptr;    // bf16 [M, e.ldo]
