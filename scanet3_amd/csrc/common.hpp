@@ -403,7 +403,12 @@ bool rnn_sequence_fwd_ok(sn_ctx* ctx, int rows, int F, int H, const float* x);
 int launch_rnn_sequence_fwd(sn_ctx* ctx, const float* x, int T, int F, int first_valid, int rows, int H, const float* wk, const float* wr,
                             float* r_slices, int64_t slice);
 bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr);
-int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice);
+// (with x, the forward slices r and a workspace the launch can carry the weight gradient, as launch_lstm_sequence_bwd does:
+// H 64, 128, 192 or 256, the batch a multiple of 16, F a multiple of 4 up to 64)
+int64_t rnn_sequence_bwd_wgrad_workspace(int rows, int T, int F, int H);
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice,
+                            const float* x = nullptr, const float* r_slices = nullptr, int F = 0, float* ws = nullptr, int64_t ws_elems = 0,
+                            int* wgrad_parts = nullptr);
 // All T forward steps of an LSTM layer in one launch: the workgroups keep their weights in registers and hand h_t to each
 // other through memory, one arrival counter per group of 32 batch rows.  h: T + 1 slices of `slice` floats, slice 0 the
 // initial hidden state (read only if h0_valid); gates / c: T slices.  lstm_sequence_fwd_ok says whether the launch fits

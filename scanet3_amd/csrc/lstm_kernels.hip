@@ -292,6 +292,26 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 __device__ __align__(16) const float seq_zero_chunk[4] = {0.f, 0.f, 0.f, 0.f};  // what the k padding and an absent h_{-1} read
 
+// LDS-direct loads of blocks KB .. NKB - 1 of a 16-row operand: block kb = 64 bytes of every row, 1 KiB of LDS
+template <int KB, int NKB, int AUX>
+__device__ __forceinline__ void load_row_blocks(global_ptr_t ap, float* aw) {
+  if constexpr (KB < NKB) {
+    __builtin_amdgcn_global_load_lds(ap, (lds_ptr_t)(aw + KB * (256 - 16)), 16, 64 * KB, AUX);
+    load_row_blocks<KB + 1, NKB, AUX>(ap, aw);
+  }
+}
+
+// base + a per-lane BYTE offset of 32 bits: the form the compiler turns into "scalar base + one offset register" accesses
+template <typename T>
+__device__ __forceinline__ T* at_bytes(T* uniform_base, unsigned byte_offset) {
+  return (T*)((char*)uniform_base + byte_offset);
+}
+template <typename T>
+__device__ __forceinline__ const T* at_bytes(const T* uniform_base, unsigned byte_offset) {
+  return (const T*)((const char*)uniform_base + byte_offset);
+}
+
+
 // Shape of the kernel: a workgroup owns 16 batch rows x 16 hidden units, so that two or more workgroups share a CU and one
 // of them multiplies while another waits for its hand-over.  Wavefront w owns gate w: its [K x 16] weights stay in
 // registers in MFMA operand order.  The 16 rows of [x_t, h_{t-1}] arrive through LDS-direct loads (one load = 16 rows x
@@ -535,15 +555,29 @@ struct SeqMulArgs {
   int* gave_up;
   int* failed;
   int force_coherent;
+  // backward with the weight gradient riding along (XW > 0 instantiations)
+  const float* wg_x;    // [rows, T, wg_F]
+  const float* wg_r;    // the forward pass's slices: slice t = r_{t-1}
+  float* wpartial;      // [row_groups][wg_F + H + 1][H]
+  int wg_F;
 };
 
-template <bool BACKWARD, int NKBW>  // NKBW: 16-long blocks of k per wavefront (4 NKBW blocks cover K, padded with zeros)
+// XW > 0 (backward only; H a multiple of 64, the batch a multiple of 16 rows): the launch also accumulates the layer's weight
+// gradient dW[m, n] = sum over (t, row) of [x_t | r_{t-1}][row, m] * dr_t[row, n], as lstm_sequence_bwd_body does for the
+// LSTM: the workgroup keeps the [F + H, 16] block that belongs to its rows and units in accumulator registers (wavefront w
+// the 64-feature run w of r, one wavefront the x features), takes dr_t of its own cells from LDS the moment it has
+// computed them (slice T - 1, which is complete at launch, from memory), the operand rows straight from memory a step
+// ahead, and multiplies right behind its arrival signal.  One partial [F + H + 1, H] per row group leaves at the end (its
+// last row, the place of a bias gradient, is not written: the simple cell's bias acts on the last step only).
+template <bool BACKWARD, int NKBW, int XW = 0>  // NKBW: 16-long blocks of k per wavefront (4 NKBW blocks cover K, padded with zeros)
 __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
   constexpr int UB = 16;
+  constexpr bool WG = BACKWARD && XW > 0;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   __shared__ int stop;
   float* Ps = lds;                 // [4 quarters of k][SRB][ZP] partial sums
   float* As = lds + 4 * SRB * ZP;  // (16-byte aligned) [wavefront][k block][16 rows x 16 k]
+  float* Dzs = As + 4 * NKBW * 256;  // [SRB][16]: dr of this workgroup's cells (weight gradient only)
   const int K = a.F + a.H;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int slot = blockIdx.x >> 3;
@@ -594,7 +628,50 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
 
   const int steps = BACKWARD ? a.T - 1 : a.T;
   bool spread = true;  // until arrival 0 is complete (the first wait below)
+  // ---- weight gradient: accumulators, operand rows, the step of slice T - 1
+  typedef float xwv __attribute__((ext_vector_type(WG ? XW : 2)));
+  constexpr int XWAVE = NKBW % 4;  // the wavefront that takes the x features: the first one without a run of r, if there is one
+  f4v accr[4], accx[WG ? XW : 1], ah[4];
+  xwv ax[4];
+  const bool x_lane = XW * row16 < a.wg_F;
+  unsigned hoff = 4u * (g * a.H + 4 * row16), xoff = 4u * (g * a.T * a.wg_F + (x_lane ? XW * row16 : 0));
+  auto request_operands = [&](int tt) {  // [x_tt | r_{tt-1}] of rows g + 4 i
+    const float* hs = a.wg_r + (int64_t)tt * a.slice + r0 * a.H + 64 * min(wave, NKBW - 1);
+    const float* xs = a.wg_x + ((int64_t)r0 * a.T + tt) * a.wg_F;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ah[i] = *(const f4v*)at_bytes(hs + 4 * i * a.H, hoff);
+      ax[i] = *(const xwv*)at_bytes(xs + (int64_t)4 * i * a.T * a.wg_F, xoff);
+    }
+  };
+  auto weight_gradient_step = [&]() {  // += [x | r]^T (16 rows) * dr (the tile in LDS)
+    const float* dzr = Dzs + g * 16 + row16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float b = dzr[4 * i * 16];
+      if (wave < NKBW) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) accr[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ah[i][j], b, accr[j], 0, 0, 0);
+      }
+      if (wave == XWAVE) {
+#pragma unroll
+        for (int j = 0; j < XW; ++j) accx[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(x_lane ? ax[i][j] : 0.f, b, accx[j], 0, 0, 0);
+      }
+    }
+  };
+  if constexpr (WG) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) accr[j] = f4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < XW; ++j) accx[j] = f4v{0.f, 0.f, 0.f, 0.f};
+    request_operands(a.T - 1);
+    Dzs[crow * 16 + cu] = live ? a.rec[(int64_t)(a.T - 1) * a.slice + ci] : 0.f;
+    __syncthreads();
+    weight_gradient_step();
+    request_operands(a.T - 2);
+  }
   for (int s = 0; s < steps; ++s) {
+    if constexpr (WG) asm volatile("" : "+v"(hoff), "+v"(xoff));  // (keeps the offsets one register each: see lstm_sequence_bwd_body)
     const int t = BACKWARD ? a.T - 1 - s : s;  // the step whose operand slice is read
     if (s > 0) {  // the slice is complete once every unit group of this row group has arrived s + 1 times (arrival 0 included)
       if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(s + 1), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
@@ -630,10 +707,36 @@ __global__ __launch_bounds__(256) void rnn_sequence_kernel(SeqMulArgs a) {
       float* out = a.rec + (int64_t)to * a.slice + ci;
       if (spread) __hip_atomic_store(out, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else *out = val;
+      if constexpr (WG) Dzs[crow * 16 + cu] = val;
+    } else if constexpr (WG) {
+      Dzs[crow * 16 + cu] = 0.f;
     }
     __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));  // vmcnt(0): the stores are acknowledged
-    __syncthreads();  // (also: Ps is free again)
+    __syncthreads();  // (also: Ps is free again, the dr tile is published)
     if (tid == 0 && s + 1 < steps) __hip_atomic_fetch_add(my_count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if constexpr (WG) {  // slice `to` is this workgroup's own: its share of the weight gradient while the others arrive
+      weight_gradient_step();
+      if (to > 0) request_operands(to - 1);
+    }
+  }
+  if constexpr (WG) {  // this row group's partial: rows 0..F-1 (x), F..F+H-1 (r)
+    const int N = a.H;
+    float* out = a.wpartial + (int64_t)rg * (a.wg_F + a.H + 1) * N + u0 + row16;
+    if (wave == XWAVE) {
+#pragma unroll
+      for (int j = 0; j < XW; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int m = XW * (4 * g + v) + j;
+          if (m < a.wg_F) out[(int64_t)m * N] = accx[j][v];
+        }
+    }
+    if (wave < NKBW) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) out[(int64_t)(a.wg_F + 64 * wave + 4 * (4 * g + v) + j) * N] = accr[j][v];
+    }
   }
 }
 
@@ -848,25 +951,6 @@ struct SeqBwdArgs {
 // tile w.  The bias gradient is each thread's running sum of its own four dz values, added over the 16 rows at the end.
 // What leaves is one partial [F + H + 1, 4H] per row group, which splitk_reduce adds in a fixed order.
 constexpr int DZP = 80;  // row pitch of the dz tile in LDS: rows g and g + 1 land in different halves of the banks
-
-// LDS-direct loads of blocks KB .. NKB - 1 of a 16-row operand: block kb = 64 bytes of every row, 1 KiB of LDS
-template <int KB, int NKB, int AUX>
-__device__ __forceinline__ void load_row_blocks(global_ptr_t ap, float* aw) {
-  if constexpr (KB < NKB) {
-    __builtin_amdgcn_global_load_lds(ap, (lds_ptr_t)(aw + KB * (256 - 16)), 16, 64 * KB, AUX);
-    load_row_blocks<KB + 1, NKB, AUX>(ap, aw);
-  }
-}
-
-// base + a per-lane BYTE offset of 32 bits: the form the compiler turns into "scalar base + one offset register" accesses
-template <typename T>
-__device__ __forceinline__ T* at_bytes(T* uniform_base, unsigned byte_offset) {
-  return (T*)((char*)uniform_base + byte_offset);
-}
-template <typename T>
-__device__ __forceinline__ const T* at_bytes(const T* uniform_base, unsigned byte_offset) {
-  return (const T*)((const char*)uniform_base + byte_offset);
-}
 
 template <int NKB, int XW>  // 16-long k blocks per wavefront: H = 16 NKB
 __device__ __forceinline__ void lstm_sequence_bwd_body(const SeqBwdArgs& a) {
@@ -1416,7 +1500,23 @@ int launch_rnn_step_fwd(sn_ctx* ctx, const float* x, int t, int T, int F, const 
 }
 
 namespace {
-size_t rnn_sequence_lds_bytes(int nkbw) { return ((size_t)4 * SRB * ZP + (size_t)4 * nkbw * 256) * sizeof(float); }
+size_t rnn_sequence_lds_bytes(int nkbw, bool with_wgrad = false) {
+  return ((size_t)4 * SRB * ZP + (size_t)4 * nkbw * 256 + (with_wgrad ? SRB * 16 : 0)) * sizeof(float);
+}
+
+// calls f(kernel, blocks per wavefront) for the backward instantiation that also accumulates the weight gradient, or returns false
+template <typename Fn>
+bool with_rnn_sequence_wgrad_kernel(int H, int F, Fn&& f) {
+  if (F % 4 != 0 || F > 64) return false;
+  const bool two = F <= 32;
+  switch (H) {
+    case 64: two ? f(rnn_sequence_kernel<true, 1, 2>, 1) : f(rnn_sequence_kernel<true, 1, 4>, 1); return true;
+    case 128: two ? f(rnn_sequence_kernel<true, 2, 2>, 2) : f(rnn_sequence_kernel<true, 2, 4>, 2); return true;
+    case 192: two ? f(rnn_sequence_kernel<true, 3, 2>, 3) : f(rnn_sequence_kernel<true, 3, 4>, 3); return true;
+    case 256: two ? f(rnn_sequence_kernel<true, 4, 2>, 4) : f(rnn_sequence_kernel<true, 4, 4>, 4); return true;
+    default: return false;
+  }
+}
 
 // calls f(kernel, blocks per wavefront) for the smallest instantiation that covers K, or returns false
 template <bool BACKWARD, typename F>
@@ -1484,13 +1584,54 @@ static bool rnn_sequence_bwd_fits(sn_ctx* ctx, int rows, int H, const float* wr)
 }
 bool rnn_sequence_bwd_ok(sn_ctx* ctx, int rows, int H, const float* wr) { return !sequence_kernels_off(ctx) && rnn_sequence_bwd_fits(ctx, rows, H, wr); }
 
-int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice) {
+// Floats of workspace the backward launch needs to carry the weight gradient along (one partial per 16-row group), or 0
+// where it cannot (shape).
+int64_t rnn_sequence_bwd_wgrad_workspace(int rows, int T, int F, int H) {
+  if (rows <= 0 || rows % SRB != 0 || T <= 1 || (int64_t)rows * T * F >= ((int64_t)1 << 30) || (int64_t)rows * H >= ((int64_t)1 << 30)) return 0;
+  if (!with_rnn_sequence_wgrad_kernel(H, F, [](auto, int) {})) return 0;
+  return ceil_div(rows, SRB) * (int64_t)(F + H + 1) * H;
+}
+
+// With x [rows, T, F], the forward pass's slices r (slice t = r_{t-1}) and a workspace the launch also leaves the weight
+// gradient's partial sums [*wgrad_parts][F + H + 1][H] in ws where the shape allows it (*wgrad_parts = 0 otherwise).
+int launch_rnn_sequence_bwd(sn_ctx* ctx, float* dr_slices, const float* dy_seq, int T, int rows, int H, const float* wr, int64_t slice,
+                            const float* x, const float* r_slices, int F, float* ws, int64_t ws_elems, int* wgrad_parts) {
+  if (wgrad_parts) *wgrad_parts = 0;
   if (rows <= 0 || T <= 1) return SN_OK;
   SN_REQUIRE(rnn_sequence_bwd_fits(ctx, rows, H, wr), "rnn_sequence_backward: rows=%d H=%d do not fit the device in one launch", rows, H);
   SeqMulArgs a{};
   a.rec = dr_slices; a.dy_seq = dy_seq; a.wr = wr; a.slice = slice;
   a.rows = rows; a.T = T; a.F = 0; a.H = H;
-  return launch_rnn_sequence<true>(ctx, a, "rnn_sequence_backward", H);
+  const int64_t need = rnn_sequence_bwd_wgrad_workspace(rows, T, F, H);
+  bool with_wgrad = wgrad_parts && x && r_slices && sequence_wgrad_wanted() && need > 0 && ws && need <= ws_elems && aligned16(x) && aligned16(r_slices);
+  if (with_wgrad) {  // the grid must still be resident at once with this instantiation's registers and LDS
+    const int64_t groups = ceil_div(rows, SRB), blocks = 8 * ceil_div(groups, 8) * (H / 16);
+    bool fits = false;
+    with_rnn_sequence_wgrad_kernel(H, F, [&](auto kernel, int nkbw) {
+      if (allow_dynamic_lds(ctx, (const void*)kernel, rnn_sequence_lds_bytes(nkbw, true)) != SN_OK) return;
+      int per_cu = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, rnn_sequence_lds_bytes(nkbw, true)) != hipSuccess) return;
+      fits = blocks <= (int64_t)per_cu * ctx->compute_units;
+    });
+    with_wgrad = fits;
+  }
+  if (!with_wgrad) return launch_rnn_sequence<true>(ctx, a, "rnn_sequence_backward", H);
+  a.wg_x = x; a.wg_r = r_slices; a.wpartial = ws; a.wg_F = F;
+  a.row_groups = (int)ceil_div(a.rows, SRB);
+  a.unit_groups = a.H / 16;
+  SN_TRY(seq_sync_take(ctx, a.row_groups, &a.sync));
+  a.spin_limit = ctx->seq_spin_limit;
+  a.gave_up = ctx->seq_gave_up_dev;
+  a.failed = ctx->seq_failed_dev;
+  a.force_coherent = ctx->seq_force_coherent;
+  // T - 1 products of rows x H x H and T of (F + H) x H x rows: as one shape, rows x H x ((T - 1) H + T (F + H))
+  LaunchScope scope(ctx, "rnn_sequence_backward_and_weight_gradient", rows, H, (T - 1) * H + T * (F + H));
+  with_rnn_sequence_wgrad_kernel(H, F, [&](auto kernel, int nkbw) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(8 * ceil_div(a.row_groups, 8) * a.unit_groups)), dim3(256), rnn_sequence_lds_bytes(nkbw, true), ctx->stream, a);
+  });
+  SN_HIP(hipGetLastError());
+  *wgrad_parts = a.row_groups;
+  return SN_OK;
 }
 
 }  // namespace sn

@@ -373,6 +373,7 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ws = std::max(ws, gemm_workspace_elems(B, op.F, op.H, cu));
         ws = std::max(ws, gemm_workspace_elems(op.F + op.H, op.H, op.T * B, cu));
         ws = std::max(ws, lstm_wgrad_rows_workspace(m->ctx, B, op.T, op.F, op.H, 1));
+        if (B <= 1024) ws = std::max(ws, rnn_sequence_bwd_wgrad_workspace(B, op.T, op.F, op.H));
         ++i;
         break;
       }
@@ -967,10 +968,16 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         const bool fused = lstm_step_fused_ok(op.F, op.H, in, w, 1);
         const bool whole = fused && op.T > 1 && rnn_sequence_bwd_ok(ctx, rows, op.H, w.wr[0]);
         if (fused && op.T > 1 && !whole) SN_TRY(launch_lstm_pack(ctx, w, op.F, op.H, nullptr, r->lstm_pk_dh[i], 1));  // the step kernel's LDS order
+        LstmGrads gr{};
+        gr.wk[0] = param_ptr(r, r->g, op.lstm_p[0][0]);
+        gr.wr[0] = param_ptr(r, r->g, op.lstm_p[0][1]);
+        int wgrad_parts = 0;  // > 0: the backward launch has left the weight gradient's partial sums in the workspace
         if (whole) {  // every step in one launch (it adds a returned sequence's output gradients itself), then the input gradients
           dr = r->lstm_dz[i] + (int64_t)(op.T - 1) * bh;
           if (op.ret_seq) SN_TRY(launch_step_slice_add(ctx, dr, dy + (int64_t)(op.T - 1) * op.H, (int64_t)op.T * op.H, rows, op.H, false));
-          SN_TRY(launch_rnn_sequence_bwd(ctx, r->lstm_dz[i], op.ret_seq ? dy : nullptr, op.T, rows, op.H, w.wr[0], bh));
+          SN_TRY(launch_rnn_sequence_bwd(ctx, r->lstm_dz[i], op.ret_seq ? dy : nullptr, op.T, rows, op.H, w.wr[0], bh, in, r->lstm_h[i], op.F,
+                                         r->ws, m->workspace_elems, &wgrad_parts));
+          if (wgrad_parts > 0) SN_TRY(launch_lstm_wgrad_reduce(ctx, r->ws, wgrad_parts, op.F, op.H, 1, gr));  // before the workspace's next user
           if (need_dx)
             for (int t = op.T - 1; t >= 0; --t)
               SN_TRY(launch_lstm_dx(ctx, r->lstm_dz[i] + (int64_t)t * bh, rows, op.H, op.F, t, op.T, w, dx, r->ws, m->workspace_elems, 1));
@@ -984,10 +991,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
             else SN_TRY(launch_lstm_dh(ctx, dr, rows, op.H, w, dr - bh, r->ws, m->workspace_elems, 1));
           }
         }
-        LstmGrads gr{};
-        gr.wk[0] = param_ptr(r, r->g, op.lstm_p[0][0]);
-        gr.wr[0] = param_ptr(r, r->g, op.lstm_p[0][1]);
-        SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems, 1));
+        if (wgrad_parts == 0) SN_TRY(launch_lstm_wgrad(ctx, in, r->lstm_h[i], r->lstm_dz[i], rows, op.T, op.F, op.H, gr, r->ws, m->workspace_elems, 1));
         if (need_dx) cur ^= 1;
         break;
       }

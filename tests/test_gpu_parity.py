@@ -1211,6 +1211,54 @@ def test_lstm_backward_launch_that_carries_the_weight_gradient(S, ctx, monkeypat
     yb.free()
 
 
+@pytest.mark.parametrize("units,features,batch,T,ret_seq", [(64, 12, 48, 4, False), (64, 64, 32, 3, True), (128, 52, 32, 5, False),
+                                                            (192, 8, 16, 2, True), (256, 32, 48, 6, True), (256, 36, 32, 4, False)])
+def test_simple_rnn_backward_launch_that_carries_the_weight_gradient(S, ctx, monkeypatch, units, features, batch, T, ret_seq):
+    """The simple cell's one-launch backward pass accumulates the weight gradient too (64, 128, 192 or 256 units, a batch
+    that is a multiple of 16 rows, at most 64 features): each instantiation against the oracle and against the separate
+    product (SCANET_SEQUENCE_WGRAD=0), as the only recurrent layer and under a second one that consumes its sequence."""
+    second = [O.SimpleRNN(16)] if ret_seq else []
+    om = O.Model([O.SimpleRNN(units, return_sequence=ret_seq)] + second + [O.Dense(2, O.ACT_IDENTITY)], O.LOSS_MSE)
+    layers = S.SimpleRNN(units, returnSequence=ret_seq)
+    if ret_seq:
+        layers = layers >> S.SimpleRNN(16)
+    layers = layers >> S.Dense(2, S.Identity)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.MeanSquaredError.kind, (T, features), batch)
+    rep = cm.replica(None)
+    rng = np.random.default_rng(6000 + units + features)
+    params = glorot_params(om, (batch, T, features), rng)
+    x = rng.standard_normal((batch, T, features)).astype(f32)
+    y = rng.uniform(-1, 1, (batch, 2)).astype(f32)
+    rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    oloss, ograds = om.grad(x, y, params)
+    ctx.profile_reset()
+    ctx.profile(True)
+    assert abs(rep.grad(xb, yb) - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ctx.sync()
+    ctx.profile(False)
+    labels = list(ctx.profile_report())
+    assert any(l.startswith("rnn_sequence_backward_and_weight_gradient") for l in labels), labels
+    ggrads = rep.get_grads()
+    _, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_GEMM, 3.0 * rel_err(ograds[p], grads64[p])), p
+    monkeypatch.setenv("SCANET_SEQUENCE_WGRAD", "0")
+    ctx.profile_reset()
+    ctx.profile(True)
+    rep.grad(xb, yb)
+    ctx.sync()
+    ctx.profile(False)
+    assert not any(l.startswith("rnn_sequence_backward_and_weight_gradient") for l in ctx.profile_report())
+    separate = rep.get_grads()
+    for p in ograds:
+        assert rel_err(ggrads[p], separate[p]) <= TOL_GEMM, p
+    for o in (rep, cm):
+        o.close()
+    xb.free()
+    yb.free()
+
+
 @pytest.mark.parametrize("kind", ["lstm", "simple_rnn"])
 def test_lstm_sequence_kernel_gives_up_instead_of_hanging(S, monkeypatch, kind):
     """A workgroup of a one-launch recurrent kernel that waits for its neighbours polls a bounded number of times.  With the
