@@ -994,7 +994,8 @@ def test_k_replica_training_matches_oracle(S, linear_function):
         assert rel_err(trained.params[p], oparams[p]) <= 1e-4
 
 
-@pytest.mark.parametrize("kind,units,features,batch", [("lstm", 32, 8, 64), ("lstm", 6, 3, 10), ("simple_rnn", 32, 8, 64), ("simple_rnn", 5, 3, 9)])
+@pytest.mark.parametrize("kind,units,features,batch", [("lstm", 32, 8, 64), ("lstm", 6, 3, 10), ("simple_rnn", 32, 8, 64), ("simple_rnn", 5, 3, 9),
+                                                      ("lstm", 64, 8, 32), ("simple_rnn", 64, 8, 32)])  # the last two: backward launches that carry the weight gradient
 def test_stateful_rnn_steps_match_oracle(S, ctx, kind, units, features, batch):
     """`RNN(cell, stateful = true)` (RNN.scala:27,34,66-72) through the fused step kernels (32 units) and the tiled path:
     every step starts from the state the one before left, which sits in the parameter table as a non-trainable,
