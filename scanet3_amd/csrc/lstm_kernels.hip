@@ -1136,7 +1136,6 @@ __device__ __forceinline__ void lstm_sequence_bwd_body(const SeqBwdArgs& a) {
     if constexpr (WG) {
       weight_gradient_step();
       if (t == 0) break;
-      request_operands(t - 1);
     }
     const int done = a.T - 1 - t;  // hand-overs before this one
     if (wait_arrivals(my_count, (unsigned)a.unit_groups * (unsigned)(done + 2), abort_word, a.spin_limit, a.gave_up, a.failed, &stop)) return;
@@ -1148,12 +1147,18 @@ __device__ __forceinline__ void lstm_sequence_bwd_body(const SeqBwdArgs& a) {
       const global_ptr_t ap = (global_ptr_t)at_bytes(a.dz + (int64_t)t * 4 * a.slice + wave * H, a_off);
       if (spread) load_row_blocks<0, NKB, 16>(ap, aw);  // sc1: coherent at device scope
       else load_row_blocks<0, NKB, 0>(ap, aw);
+      // The weight gradient's operand rows of step t - 1 are requested behind these loads (8 load instructions): in front
+      // of them they would have to land before the first block could be multiplied, in front of the wait before the poll
+      // could return.  They have a whole step to land.
+      constexpr int YOUNGER = WG ? 8 : 0;
+      if constexpr (WG) request_operands(t - 1);
       // The blocks are this wavefront's own, so no barrier: block kb is multiplied as soon as all but the NKB - 1 - kb loads
-      // behind it have landed (loads return in order; the compiler does not order LDS reads behind these loads by itself).
+      // behind it (and the YOUNGER ones behind those) have landed (loads return in order; the compiler does not order LDS
+      // reads behind these loads by itself).
       f4v acc[2] = {f4v{0.f, 0.f, 0.f, 0.f}, f4v{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKB - 1 - kb) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NKB - 1 - kb + YOUNGER) : "memory");
         const f4v av = *(const f4v*)(ar + kb * 256);
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[kb & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[v], bw[kb][v], acc[kb & 1], 0, 0, 0);
@@ -1161,7 +1166,12 @@ __device__ __forceinline__ void lstm_sequence_bwd_body(const SeqBwdArgs& a) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) Ps[(wave * SRB + 4 * g + v) * ZP + row16] = acc[0][v] + acc[1][v];
     }
-    __syncthreads();
+    if constexpr (WG) {  // (not __syncthreads: its fence would wait for the operand rows requested above)
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the partial sums are in LDS
+      __builtin_amdgcn_s_barrier();
+    } else {
+      __syncthreads();
+    }
     dh = (Ps[crow * ZP + cu] + Ps[(SRB + crow) * ZP + cu]) + (Ps[(2 * SRB + crow) * ZP + cu] + Ps[(3 * SRB + crow) * ZP + cu]);
   }
   if constexpr (WG) {
