@@ -345,7 +345,19 @@ struct ConvGeom {
 };
 int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& ep, float* ws, int64_t ws_elems);
 int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems);
-int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems);
+// A 2 x 2 max pooling right above a first-layer convolution, for launch_conv_wgrad's direct kernel: the pooling's output
+// gradient dy [n, ho, wo, cout], its recorded first-maximum offsets (one byte per output value) and the convolution's saved
+// output y with its activation; the kernel then forms the convolution's output gradient itself (no launch_pool_bwd).
+struct PoolGrad {
+  const float* dy = nullptr;
+  const uint8_t* arg = nullptr;
+  const float* y = nullptr;
+  int ho = 0, wo = 0, sh = 1, sw = 1, pt = 0, pl = 0, act = 0;
+  float act_param = 0.f;
+};
+bool conv_wgrad_is_direct(const sn_ctx* ctx, const ConvGeom& g, const float* ws, int64_t ws_elems, bool with_pool = false);
+int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems,
+                      const PoolGrad* pool = nullptr);
 
 // the same two products with LDS-direct loads into a three-stage ring (conv_ring_kernels.hip), for the shapes *_ok accepts
 bool conv_ring_fwd_ok(const ConvGeom& g, const float* x, const float* w, const Epilogue& e);

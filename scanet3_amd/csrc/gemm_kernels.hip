@@ -1489,10 +1489,24 @@ int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const flo
 // leave as one partial [M][cout] per workgroup; gemm_small_reduce_kernel adds the partials in a fixed order.
 constexpr int WGRAD_DIRECT_MAX_TAPS = 36;
 
-template <int MT>  // upper bound of kh*kw*cin
+// POOL: the convolution's output gradient is not in memory yet.  A 2 x 2 max pooling sits right above the layer and the
+// kernel computes dy[position, filter] itself from the pooling's output gradient, the recorded first-maximum offsets and
+// the convolution's saved output (for its activation gradient), exactly as pool2x2_bwd_kernel does: an element lies in at
+// most 2 x 2 windows, whose contributions are added in (oh, ow) order, then act'(y) multiplies.  One launch and one pass
+// over the tensor less for a first layer, whose input gradient nobody needs.
+__device__ __forceinline__ float pool_grad_act_bwd(int act, float y, float dy, float param) {  // elementwise_kernels.hip: act_bwd
+  switch (act) {
+    case SN_ACT_SIGMOID: return (y * (1.0f - y)) * dy;
+    case SN_ACT_TANH: return (1.0f - y * y) * dy;
+    case SN_ACT_RELU: return (param < y ? 1.0f : 0.0f) * dy;
+    default: return dy;
+  }
+}
+
+template <int MT, bool POOL>  // MT: upper bound of kh*kw*cin
 __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ dy,
                                                                  float* __restrict__ partial, int rows_per_band, int bands_per_image,
-                                                                 int items, int lw, int cshift, int staged_full) {
+                                                                 int items, int lw, int cshift, int staged_full, PoolGrad pg) {
   extern __shared__ float wg_lds[];
   const int tid = threadIdx.x;
   const int M = g.kh * g.kw * g.cin;
@@ -1522,6 +1536,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
     const float* dyb = dy + ((int64_t)b * g.ho + oh0) * g.wo * g.cout;
     constexpr int U = 16;  // positions per lane whose dy loads are in flight together
     int* origin = reinterpret_cast<int*>(wg_lds + staged_full);  // per position of the band: LDS offset of its top-left input element
+    float* dcv = wg_lds + staged_full + rows_per_band * g.wo;    // POOL: the band's output gradient [P][cout]
     __syncthreads();  // the previous item's readers are done with the staged rows
     for (int e = tid; e < staged; e += 256) {
       const int row = e / row_elems, rem = e % row_elems;
@@ -1529,6 +1544,47 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
       wg_lds[e] = ((unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w) ? x[(((int64_t)b * g.h + iy) * g.w + ix) * g.cin + ci] : 0.f;
     }
     for (int p = tid; p < P; p += 256) origin[p] = (p / g.wo) * g.sh * row_elems + (p % g.wo) * g.sw * g.cin;  // one division per position, not per lane
+    if constexpr (POOL) {
+      // the band's output gradient [P][cout], four filters per thread: position (iy, ix) of the convolution's output = of the
+      // pooling's input lies in the windows oh_lo + {0, 1} x ow_lo + {0, 1} (those that exist)
+      const int cv = g.cout >> 2;
+      for (int e = tid; e < P * cv; e += 256) {
+        const int p = e / cv, ch = (e - p * cv) * 4;
+        const int iy = oh0 + p / g.wo, ix = p % g.wo;
+        int oh_lo = iy + pg.pt - 1;
+        oh_lo = oh_lo <= 0 ? 0 : (oh_lo + pg.sh - 1) / pg.sh;
+        int oh_hi = (iy + pg.pt) / pg.sh;
+        if (oh_hi > pg.ho - 1) oh_hi = pg.ho - 1;
+        int ow_lo = ix + pg.pl - 1;
+        ow_lo = ow_lo <= 0 ? 0 : (ow_lo + pg.sw - 1) / pg.sw;
+        int ow_hi = (ix + pg.pl) / pg.sw;
+        if (ow_hi > pg.wo - 1) ow_hi = pg.wo - 1;
+        const f4v yv = *(const f4v*)(pg.y + ((((int64_t)b * g.ho + iy) * g.wo + ix) * g.cout + ch));
+        uint32_t a4[4], want[4];
+        f4v gk[4];
+        bool on[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {  // windows that do not exist re-read the first element and are ignored
+          const int oh = oh_lo + (k >> 1), ow = ow_lo + (k & 1);
+          on[k] = oh <= oh_hi && ow <= ow_hi;
+          const int64_t o = on[k] ? (((int64_t)b * pg.ho + oh) * pg.wo + ow) * g.cout + ch : ch;
+          want[k] = (uint32_t)((iy - (oh * pg.sh - pg.pt)) * 2 + (ix - (ow * pg.sw - pg.pl)));
+          a4[k] = *(const uint32_t*)(pg.arg + o);
+          gk[k] = *(const f4v*)(pg.dy + o);
+        }
+        f4v sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (!on[k]) continue;
+          if ((a4[k] & 255u) == want[k]) sum[0] += gk[k][0];
+          if (((a4[k] >> 8) & 255u) == want[k]) sum[1] += gk[k][1];
+          if (((a4[k] >> 16) & 255u) == want[k]) sum[2] += gk[k][2];
+          if ((a4[k] >> 24) == want[k]) sum[3] += gk[k][3];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dcv[p * g.cout + ch + q] = pool_grad_act_bwd(pg.act, yv[q], sum[q], pg.act_param);
+      }
+    }
     __syncthreads();
     for (int p0 = slot; p0 < P; p0 += slots * U) {
       float d[U];
@@ -1538,7 +1594,9 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
         const int p = p0 + u * slots;
         const bool in = p < P;
         const int pp = in ? p : 0;
-        const float v = dyb[(int64_t)pp * g.cout + cc];  // always a valid address: no branch around the load
+        float v;
+        if constexpr (POOL) v = dcv[pp * g.cout + cc];  // formed below, once per band
+        else v = dyb[(int64_t)pp * g.cout + cc];  // always a valid address: no branch around the load
         d[u] = (in && live) ? v : 0.f;
         base[u] = origin[pp];
       }
@@ -1565,7 +1623,24 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
   }
 }
 
-static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems, int* rc) {
+// true when launch_conv_wgrad takes the direct kernel for this layer (which can also stand in for a max pooling's backward
+// pass above it: launch_conv_wgrad's `pool` argument)
+bool conv_wgrad_is_direct(const sn_ctx* ctx, const ConvGeom& g, const float* ws, int64_t ws_elems, bool with_pool) {
+  const int M = g.kh * g.kw * g.cin, N = g.cout;
+  const int64_t K = (int64_t)g.n * g.ho * g.wo;
+  if (!ws || g.cin > 4 || M > WGRAD_DIRECT_MAX_TAPS || N > 64 || K < SMALL_MIN_K) return false;
+  const int64_t room = std::min<int64_t>((int64_t)4 * ctx->compute_units, ws_elems / ((int64_t)M * N));
+  if (room < 32) return false;
+  const int lw = (g.wo - 1) * g.sw + g.kw;
+  const int rows_per_band = (int)std::min<int64_t>(g.ho, std::max<int64_t>(1, ceil_div((int64_t)g.n * g.ho, room)));
+  const int bands = (int)ceil_div((int64_t)g.ho, (int64_t)rows_per_band);
+  const int64_t staged = (int64_t)((rows_per_band - 1) * g.sh + g.kh) * lw * g.cin;
+  const int64_t lds_floats = std::max<int64_t>(staged + (int64_t)rows_per_band * g.wo * (with_pool ? 1 + N : 1), (int64_t)256 * M);
+  return lds_floats * 4 <= 48 * 1024 && (int64_t)g.n * bands < (int64_t)1 << 30 && (!with_pool || N % 4 == 0);
+}
+
+static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems, int* rc,
+                              const PoolGrad* pool) {
   const int M = g.kh * g.kw * g.cin, N = g.cout;
   const int64_t K = (int64_t)g.n * g.ho * g.wo;
   if (!ws || g.cin > 4 || M > WGRAD_DIRECT_MAX_TAPS || N > 64 || K < SMALL_MIN_K) return false;
@@ -1578,14 +1653,21 @@ static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, co
   const int bands = (int)ceil_div((int64_t)g.ho, (int64_t)rows_per_band);
   const int64_t items = (int64_t)g.n * bands;
   const int64_t staged = (int64_t)((rows_per_band - 1) * g.sh + g.kh) * lw * g.cin;
-  const int64_t lds_floats = std::max<int64_t>(staged + (int64_t)rows_per_band * g.wo, (int64_t)256 * M);
+  const int64_t lds_floats = std::max<int64_t>(staged + (int64_t)rows_per_band * g.wo * (pool ? 1 + N : 1), (int64_t)256 * M);
   if (lds_floats * 4 > 48 * 1024 || items >= (int64_t)1 << 30) return false;
   const int parts = (int)std::min<int64_t>(items, room);
   {
-    LaunchScope scope(ctx, "conv2d_filter_gradient_direct", M, N, (int)K);
-#define SN_WGRAD_DIRECT(MT)                                                                                                        \
-  hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float), ctx->stream, g, \
-                     x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged)
+    LaunchScope scope(ctx, pool ? "maxpool_backward_and_conv2d_filter_gradient_direct" : "conv2d_filter_gradient_direct", M, N, (int)K);
+    const PoolGrad pg = pool ? *pool : PoolGrad{};
+#define SN_WGRAD_DIRECT(MT)                                                                                                             \
+  do {                                                                                                                                  \
+    if (pool)                                                                                                                           \
+      hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT, true>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float),    \
+                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg);                     \
+    else                                                                                                                                \
+      hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT, false>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float),   \
+                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg);                     \
+  } while (0)
     if (M <= 9) SN_WGRAD_DIRECT(9);
     else if (M <= 18) SN_WGRAD_DIRECT(18);
     else SN_WGRAD_DIRECT(36);
@@ -1608,10 +1690,12 @@ static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, co
   return true;
 }
 
-int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems) {
+int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems,
+                      const PoolGrad* pool) {
   const int M = g.kh * g.kw * g.cin, N = g.cout, K = g.n * g.ho * g.wo;
   int rc = SN_OK;
-  if (conv_wgrad_direct(ctx, g, x, dy, dw, ws, ws_elems, &rc)) return rc;
+  if (conv_wgrad_direct(ctx, g, x, dy, dw, ws, ws_elems, &rc, pool)) return rc;
+  SN_REQUIRE(pool == nullptr, "conv2d_filter_gradient: only the direct kernel takes a pooling's gradient (ask conv_wgrad_is_direct first)");
   if (!(ws && small_parts(M, N, K, ctx->compute_units, ws_elems)) && WgradXLoader::ok(x, g) && FlatLoader<false>::ok(dy, 1, g.cout, N, K)) {
     const int interior = g.pt == 0 && g.pl == 0 && (g.ho - 1) * g.sh + g.kh <= g.h && (g.wo - 1) * g.sw + g.kw <= g.w;
     WgradXLoader al{x, g, M, interior};

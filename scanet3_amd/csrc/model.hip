@@ -733,6 +733,8 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
   if (first < 0) first = (int)m->ops.size() - 1;
   bool act_grad_done = false;  // the op above already applied this op's activation gradient
+  bool pool_pending = false;   // the max pooling above a first-layer convolution left its backward pass to the filter gradient
+  PoolGrad pool_grad;
   bool dz_handed_over = false;  // the bf16 Dense op above already wrote this op's dZ copies and bias-gradient block sums
   for (int i = first; i >= 0; --i) {  // grad_buf[cur] holds d loss / d (output of op i)
     const Op& op = m->ops[i];
@@ -824,7 +826,9 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         ConvGeom g{rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2], (int)op.out_dims[0], (int)op.out_dims[1],
                    (int)op.out_dims[2], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl};
         const int64_t n_out = (int64_t)rows * op.out_elems;
-        if (op.act != SN_ACT_IDENTITY && !act_grad_done) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
+        const PoolGrad* pool = pool_pending ? &pool_grad : nullptr;  // the pooling above left its backward pass to this product
+        pool_pending = false;
+        if (op.act != SN_ACT_IDENTITY && !act_grad_done && !pool) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, n_out, op.act, op.act_param));
         act_grad_done = false;
         if (op.b >= 0)
           SN_TRY(launch_col_sum(ctx, dy, g.cout, param_ptr(r, r->g, op.b), (int64_t)rows * g.ho * g.wo, g.cout, r->ws, m->workspace_elems));
@@ -833,12 +837,12 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           DeferredReduce& slot = r->deferred[r->n_deferred];
           slot = DeferredReduce{};
           ctx->defer = &slot;
-          const int rc = launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws_defer[i], m->workspace_elems);
+          const int rc = launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws_defer[i], m->workspace_elems, pool);
           ctx->defer = nullptr;
           SN_TRY(rc);
           if (slot.kind != 0) ++r->n_deferred;
         } else {
-          SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems));
+          SN_TRY(launch_conv_wgrad(ctx, g, in, dy, param_ptr(r, r->g, op.w), r->ws, m->workspace_elems, pool));
         }
         if (need_dx) {
           SN_TRY(launch_conv_dgrad(ctx, g, dy, param_ptr(r, r->w, op.w), dx, r->ws, m->workspace_elems));
@@ -851,6 +855,23 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           // a convolution with an activation right below: its activation gradient rides along (one pass less over the tensor)
           const Op& below = m->ops[i - 1];
           const bool fuse = below.kind == OP_CONV && below.act != SN_ACT_IDENTITY;
+          // The first layer's convolution needs its output gradient for the filter gradient only (and has no bias to sum it
+          // for): where that product runs as the direct kernel, the kernel forms the gradient itself from what this pooling
+          // would have read, and the pooling's backward launch and the tensor it writes are not needed.
+          if (i == 1 && below.kind == OP_CONV && below.b < 0 && !op.pool_avg && op.kh == 2 && op.kw == 2 && rows > 0) {
+            const ConvGeom cg{rows, (int)below.in_dims[0], (int)below.in_dims[1], (int)below.in_dims[2], (int)below.out_dims[0],
+                              (int)below.out_dims[1], (int)below.out_dims[2], below.kh, below.kw, below.sh, below.sw, below.pt, below.pl};
+            const bool deferred = r->defer_now && r->ws_defer[0] && r->n_deferred < MAX_DEFERRED;
+            const bool aligned = ((reinterpret_cast<uintptr_t>(dy) | reinterpret_cast<uintptr_t>(r->arg[i]) | reinterpret_cast<uintptr_t>(r->act[i - 1])) & 15u) == 0;
+            if (aligned && conv_wgrad_is_direct(ctx, cg, deferred ? r->ws_defer[0] : r->ws, m->workspace_elems, true)) {
+              pool_grad.dy = dy; pool_grad.arg = r->arg[i]; pool_grad.y = r->act[i - 1];
+              pool_grad.ho = (int)op.out_dims[0]; pool_grad.wo = (int)op.out_dims[1];
+              pool_grad.sh = op.sh; pool_grad.sw = op.sw; pool_grad.pt = op.pt; pool_grad.pl = op.pl;
+              pool_grad.act = below.act; pool_grad.act_param = below.act_param;
+              pool_pending = true;
+              break;
+            }
+          }
           SN_TRY(launch_pool_bwd(ctx, op.pool_avg, dy, r->arg[i], dx, rows, (int)op.in_dims[0], (int)op.in_dims[1], (int)op.in_dims[2],
                                     (int)op.out_dims[0], (int)op.out_dims[1], op.kh, op.kw, op.sh, op.sw, op.pt, op.pl,
                                     fuse ? r->act[i - 1] : nullptr, below.act, below.act_param));

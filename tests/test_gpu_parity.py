@@ -454,6 +454,15 @@ MODELS = {
                                 "cce", (18, 17, 3), 30, "uniform_onehot"),
     "conv_first_layer_5x5": ([("conv", 6, (5, 5), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 2), "valid"), ("flatten",), ("dense", 4, "softmax")],
                              "cce", (16, 16, 1), 40, "uniform_onehot"),
+    # a max pooling right above a first-layer convolution without bias: the filter-gradient kernel forms the convolution's
+    # output gradient itself (no pooling backward launch).  Same padding at stride 1 and 2 (windows that hang over the
+    # edge), an odd image under a strided convolution, tanh / identity / ReLU, 1 and 3 input channels
+    "conv_pool_first_layer_same_s1": ([("conv", 8, (3, 3), (1, 1), "valid", "tanh", False), ("pool", (2, 2), (1, 1), "same"), ("flatten",),
+                                       ("dense", 3, "softmax")], "cce", (12, 11, 3), 30, "uniform_onehot"),
+    "conv_pool_first_layer_same_s2": ([("conv", 6, (3, 2), (2, 1), "same", "identity", False), ("pool", (2, 2), (2, 2), "same"), ("flatten",),
+                                       ("dense", 3, "softmax")], "cce", (17, 15, 3), 40, "uniform_onehot"),
+    "conv_pool_first_layer_valid_s2_1": ([("conv", 16, (2, 2), (1, 1), "valid", "relu", False), ("pool", (2, 2), (2, 1), "valid"), ("flatten",),
+                                          ("dense", 4, "softmax")], "cce", (15, 14, 1), 24, "uniform_onehot"),
     # first-layer forward in its row-band form (at most 18 taps, 4 << j filters, >= 2048 output pixels): several bands per image with
     # Same padding above and below, strides and a bias; and 4 filters (one lane per pixel) over 3 channels
     "conv_first_layer_bands_same_stride": ([("conv", 64, (3, 3), (2, 1), "same", "tanh", True), ("pool", (2, 2), (2, 2), "valid"), ("flatten",),
