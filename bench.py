@@ -305,7 +305,7 @@ MEASURED_TRAFFIC = {
     # for a plain copy of 400 MB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the summaries are under profiles/
     "conv2d_forward[52900x64x288]": (22.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[62500x32x576]": (22.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x52900]": (42.1e6, "gemm_kernels.hip", "6ab2817374a05140b3c8ecff9ee239c30578043e"),
+    "conv2d_filter_gradient[288x64x52900]": (42.1e6, "gemm_kernels.hip", "30efc35fc3f57cefda7a62af3133e72495ea8d20"),
     "gemm_bf16_256x256_bf16out[8192x4096x4096]": (474.9e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_256x256[4096x4096x8192]": (491.1e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_256x256_handover[8192x4096x4096]": (486.2e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
@@ -318,7 +318,7 @@ MEASURED_TRAFFIC = {
     "rnn_sequence_backward_and_weight_gradient[512x256x34560]": (116.8e6, "lstm_kernels.hip", "a4185c13417e2c3aa00b48e9ee68b94c3d12c124"),
     "conv2d_forward[121000x64x288]": (53.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[169000x32x576]": (53.7e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "6ab2817374a05140b3c8ecff9ee239c30578043e"),
+    "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "30efc35fc3f57cefda7a62af3133e72495ea8d20"),
     "mlp2_rows_forward_backward[1000x50x784]": (5.41e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
     "mlp2_weight_gradients[784x50x1000]": (8.69e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
     "lstm_weight_gradient_rows[289x1024x32768]": (474.3e6, "lstm_wgrad_kernels.hip", "070ad64002f0fb967fbd759a0aabe0851ddfb7e3"),
