@@ -225,7 +225,20 @@ int launch_lstm_gates_bwd(sn_ctx* ctx, const LstmGateBwdArgs& a, int rows, int h
 bool mlp2_fused_ok(int rows_max, int K, int H, int C, int64_t scratch_a_elems, int64_t scratch_b_elems);
 int launch_mlp2_grad(sn_ctx* ctx, const float* x, const float* y, const float* w1, const float* b1, const float* w2, const float* b2, int rows,
                      int K, int H, int C, int act1, float act1_param, bool stable, float* h, float* z2, float* p, float* scratch_a,
-                     float* scratch_b, float* row_loss, float* loss_dev, float* g_w1, float* g_b1, float* g_w2, float* g_b2);
+                     float* scratch_b, float* row_loss, float* loss_dev, float* g_w1, float* g_b1, float* g_w2, float* g_b2,
+                     const struct Mlp2Update* update = nullptr);
+// The optimizer update riding in the second launch: every thread that finishes a gradient value applies it to its
+// parameter on the spot (same arithmetic as the streaming optimizer kernels), so a training step is two launches.  w, g
+// and the state buffers are the replica's flat buffers; the gradient pointers above must point into g.
+struct Mlp2Update {
+  int kind = -1, n_states = 0;
+  OptScalars p;
+  float* w = nullptr;
+  const float* g = nullptr;
+  float* s0 = nullptr;
+  float* s1 = nullptr;
+  float* s2 = nullptr;
+};
 
 // ---- seeded random tensors (random_kernels.hip): scale / shift may be null
 int launch_random_fill(sn_ctx* ctx, float* out, int64_t n, int dist, uint64_t seed, const float* scale, const float* shift);

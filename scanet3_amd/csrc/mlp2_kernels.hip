@@ -13,6 +13,7 @@
 //     in LDS, dz1 fragments as 16-byte loads), and the sums of the row blocks' partial dW2 / db1 / db2 in block order.
 // Every sum has a fixed order, so results do not depend on the launch.
 #include "common.hpp"
+#include "optim_update.hpp"
 
 namespace sn {
 namespace {
@@ -40,7 +41,19 @@ struct Mlp2Args {
   float* g_w1; float* g_b1; float* g_w2; float* g_b2;   // gradients (b may be null)
   int rows, K, H, C, act1, stable;
   float act1_param, neg_inv_rows;
+  Mlp2Update upd;    // kind >= 0: kernel 2 applies every gradient value it finishes to its parameter
 };
+
+// the optimizer update of the parameter whose gradient g_at[0] has just been stored
+__device__ __forceinline__ void apply_update(const Mlp2Update& u, const float* g_at, float grad) {
+  const int64_t off = g_at - u.g;
+  float w = u.w[off], s0 = u.s0[off], s1 = u.n_states > 1 ? u.s1[off] : 0.f, s2 = u.n_states > 2 ? u.s2[off] : 0.f;
+  update_any(u.kind, w, grad, s0, s1, s2, u.p);
+  u.w[off] = w;
+  u.s0[off] = s0;
+  if (u.n_states > 1) u.s1[off] = s1;
+  if (u.n_states > 2) u.s2[off] = s2;
+}
 
 __device__ __forceinline__ float act_fwd1(int act, float v, float param) {
   switch (act) {
@@ -242,9 +255,14 @@ __global__ __launch_bounds__(256) void mlp2_weights_kernel(Mlp2Args a, int nblk,
         for (int u = 0; u < 8; ++u) s += v[u];
       }
       for (; b < nblk; ++b) s += a.part[(int64_t)b * np + e];
-      if (e < a.H * a.C) a.g_w2[e] = s;
-      else if (e < a.H * a.C + a.H) { if (a.g_b1) a.g_b1[e - a.H * a.C] = s; }
-      else if (a.g_b2) a.g_b2[e - a.H * a.C - a.H] = s;
+      float* at = nullptr;
+      if (e < a.H * a.C) at = a.g_w2 + e;
+      else if (e < a.H * a.C + a.H) at = a.g_b1 ? a.g_b1 + (e - a.H * a.C) : nullptr;
+      else at = a.g_b2 ? a.g_b2 + (e - a.H * a.C - a.H) : nullptr;
+      if (at) {
+        *at = s;
+        if (a.upd.kind >= 0) apply_update(a.upd, at, s);
+      }
     }
     return;
   }
@@ -312,7 +330,11 @@ __global__ __launch_bounds__(256) void mlp2_weights_kernel(Mlp2Args a, int nblk,
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const int f = f0 + 4 * g + v;
-      if (f < a.K) a.g_w1[(int64_t)f * a.H + col] = acc[v];
+      if (f < a.K) {
+        float* at = a.g_w1 + (int64_t)f * a.H + col;
+        *at = acc[v];
+        if (a.upd.kind >= 0) apply_update(a.upd, at, acc[v]);
+      }
     }
   }
 }
@@ -344,11 +366,12 @@ bool mlp2_fused_ok(int rows_max, int K, int H, int C, int64_t scratch_a_elems, i
 
 int launch_mlp2_grad(sn_ctx* ctx, const float* x, const float* y, const float* w1, const float* b1, const float* w2, const float* b2, int rows,
                      int K, int H, int C, int act1, float act1_param, bool stable, float* h, float* z2, float* p, float* scratch_a,
-                     float* scratch_b, float* row_loss, float* loss_dev, float* g_w1, float* g_b1, float* g_w2, float* g_b2) {
+                     float* scratch_b, float* row_loss, float* loss_dev, float* g_w1, float* g_b1, float* g_w2, float* g_b2,
+                     const Mlp2Update* update) {
   SN_REQUIRE(rows > 0, "loss over an empty batch");
   SN_REQUIRE(aligned16(x) && aligned16(scratch_a), "mlp2: x and the scratch buffers must be 16-byte aligned");
   Mlp2Args a{x, y, w1, b1, w2, b2, h, z2, p, scratch_a, row_loss, scratch_b, g_w1, g_b1, g_w2, g_b2,
-             rows, K, H, C, act1, stable ? 1 : 0, act1_param, -(1.0f / (float)rows)};
+             rows, K, H, C, act1, stable ? 1 : 0, act1_param, -(1.0f / (float)rows), update ? *update : Mlp2Update{}};
   const int nblk = (int)ceil_div(rows, MR), nslab = (int)ceil_div(K, 16);
   {
     LaunchScope scope(ctx, "mlp2_rows_forward_backward", rows, H, K);
@@ -356,7 +379,7 @@ int launch_mlp2_grad(sn_ctx* ctx, const float* x, const float* y, const float* w
     hipLaunchKernelGGL(mlp2_rows_kernel, dim3((unsigned)nblk), dim3(256), rows_lds(K), ctx->stream, a);
   }
   {
-    LaunchScope scope(ctx, "mlp2_weight_gradients", K, H, rows);
+    LaunchScope scope(ctx, update ? "mlp2_weight_gradients_and_optimizer" : "mlp2_weight_gradients", K, H, rows);
     SN_TRY(allow_dynamic_lds(ctx, (const void*)mlp2_weights_kernel, weights_lds(1792)));
     hipLaunchKernelGGL(mlp2_weights_kernel, dim3((unsigned)(nslab + 1)), dim3(256), weights_lds(rows), ctx->stream, a, nblk, nslab);
   }

@@ -109,6 +109,8 @@ struct sn_replica {
   // Training steps of a model whose whole flat buffer is one optimizer launch: the sums of the convolutions' partial
   // filter gradients wait for that launch (launch_finish) instead of running as launches of their own.  Every such
   // convolution has a workspace of its own (the shared one is overwritten by the next product).
+  bool updated_in_pass = false;  // the gradient pass of this step has applied the optimizer itself
+  int pass_iter = 0;             // iteration number of the update that follows the running gradient pass (0: none follows)
   bool fuse_finish = false, defer_now = false;
   std::vector<float*> ws_defer;
   DeferredReduce deferred[MAX_DEFERRED];
@@ -1051,12 +1053,17 @@ static bool mlp2_path(const sn_model* m) {
 // for_update: the optimizer update of the same step follows (update()), which may then take over reductions this pass
 // leaves open; without it (sn_grad) every gradient is complete when the pass returns.
 static int grad_pass_body(sn_replica* r, const float* x, const float* y, int rows, bool want_loss);
-static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss, bool for_update = false) {
+// update_iter > 0: the optimizer update with that iteration number follows (update()), and may be taken over by this pass
+static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss, int update_iter = 0) {
+  const bool for_update = update_iter > 0;
   r->n_deferred = 0;
+  r->updated_in_pass = false;
+  r->pass_iter = update_iter;
   r->defer_now = for_update && r->fuse_finish;
   const int rc = grad_pass_body(r, x, y, rows, want_loss);
   r->defer_now = false;
   if (rc != SN_OK) r->n_deferred = 0;
+  r->pass_iter = update_iter;  // (kept for update()'s check)
   return rc;
 }
 static int grad_pass_body(sn_replica* r, const float* x, const float* y, int rows, bool want_loss) {
@@ -1065,11 +1072,25 @@ static int grad_pass_body(sn_replica* r, const float* x, const float* y, int row
   if (mlp2_path(m)) {
     const Op& d1 = m->ops[0];
     const Op& d2 = m->ops[1];
+    // A training step of a model without penalties: the second launch applies the optimizer to every gradient value it
+    // finishes (the pass touches every parameter of the model exactly once), and update() has nothing left to launch.
+    Mlp2Update u;
+    const Mlp2Update* upd = nullptr;
+    bool penalties = false;
+    for (const auto& p : m->params) penalties = penalties || p.reg_kind != SN_REG_NONE;
+    if (r->pass_iter > 0 && r->has_opt && !penalties) {
+      u.kind = r->opt.kind;
+      u.n_states = opt_state_count(r->opt.kind);
+      u.p = make_opt_scalars(r->opt, r->pass_iter);
+      u.w = r->w; u.g = r->g; u.s0 = r->s[0]; u.s1 = r->s[1]; u.s2 = r->s[2];
+      upd = &u;
+      r->updated_in_pass = true;
+    }
     SN_TRY(launch_mlp2_grad(r->ctx, x, y, param_ptr(r, r->w, d1.w), param_ptr(r, r->w, d1.b), param_ptr(r, r->w, d2.w), param_ptr(r, r->w, d2.b), rows,
                             (int)d1.in_elems, (int)d1.out_elems, (int)d2.out_elems, d1.act, d1.act_param,
                             (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0, r->act[0], r->act[1], r->act[2], r->grad_buf[0], r->grad_buf[1],
                             r->loss_partials, want_loss ? r->loss_dev : nullptr, param_ptr(r, r->g, d1.w), param_ptr(r, r->g, d1.b),
-                            param_ptr(r, r->g, d2.w), param_ptr(r, r->g, d2.b)));
+                            param_ptr(r, r->g, d2.w), param_ptr(r, r->g, d2.b), upd));
     if (want_loss) SN_TRY(add_penalties(r, true));
     for (auto& p : m->params)
       if (p.reg_kind != SN_REG_NONE)
@@ -1105,7 +1126,10 @@ static int update(sn_replica* r, int iter) {
   // weights move by the algorithm, layer state by the layer's own rule (`nextWeights ++ nextState`, Optimizer.scala:142-144);
   // the statistics are those of the gradient pass that has just run.  In bf16 mode the optimizer writes the bf16 copy of
   // what it updates in the same pass (every Dense weight is trainable), so the copies stay current.
-  if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer (fuse_finish: one run from 0)
+  if (r->updated_in_pass) {  // the gradient pass has applied the update itself (with this iteration number)
+    SN_REQUIRE(r->pass_iter == iter, "update(%d) behind a gradient pass that was run for iteration %d", iter, r->pass_iter);
+    r->updated_in_pass = false;
+  } else if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer (fuse_finish: one run from 0)
     const auto& run = m->trainable_runs[0];
     const int nd = r->n_deferred;
     r->n_deferred = 0;
@@ -1347,7 +1371,7 @@ int sn_step(sn_replica* rep, const float* x_dev, const float* y_dev, int32_t row
   SN_TRY(check_rows(rep, rows));
   SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
   SN_REQUIRE(rep->has_opt, "replica was created without an optimizer");
-  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr, true));
+  SN_TRY(grad_pass(rep, x_dev, y_dev, rows, loss_host != nullptr, iter));
   SN_TRY(update(rep, iter));
   return read_loss(rep, loss_host);
 }
@@ -1478,7 +1502,7 @@ int sn_train_epoch(sn_replica* rep, const float* x_dev, const float* y_dev, int6
              (long long)total_rows, batch);
   const int64_t xs = rep->model->in_elems * batch, ys = rep->model->out_elems * batch;
   for (int64_t i = 0; i < n_batches; ++i) {
-    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch, false, true));  // the epoch's loss is evaluated after its last update
+    SN_TRY(grad_pass(rep, x_dev + i * xs, y_dev + i * ys, batch, false, global_iter + (int)i + 1));  // the epoch's loss is evaluated after its last update
     SN_TRY(update(rep, global_iter + (int)i + 1));  // optimizers/Optimizer.scala:143
   }
   if (iterations_host) *iterations_host = (int32_t)n_batches;
@@ -1580,7 +1604,7 @@ int sn_train_epoch_host(sn_replica* rep, const float* x_host, const float* y_hos
     }
     SN_HIP(hipStreamWaitEvent(compute, rep->ev_filled[slot], 0));
     for (int64_t j = 0; j < nb; ++j) {
-      SN_TRY(grad_pass(rep, rep->stage_x[slot] + j * xs, rep->stage_y[slot] + j * ys, batch, false, true));
+      SN_TRY(grad_pass(rep, rep->stage_x[slot] + j * xs, rep->stage_y[slot] + j * ys, batch, false, global_iter + (int)(first + j) + 1));
       SN_TRY(update(rep, global_iter + (int)(first + j) + 1));  // optimizers/Optimizer.scala:143
     }
     SN_HIP(hipEventRecord(rep->ev_consumed[slot], compute));
