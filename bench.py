@@ -319,13 +319,13 @@ MEASURED_TRAFFIC = {
     "conv2d_forward[121000x64x288]": (53.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[169000x32x576]": (53.7e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "30efc35fc3f57cefda7a62af3133e72495ea8d20"),
-    "mlp2_rows_forward_backward[1000x50x784]": (5.41e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
-    "mlp2_weight_gradients[784x50x1000]": (8.69e6, "mlp2_kernels.hip", "e04a506fff012dcd9aaca59bc39e3803e793af96"),
+    "mlp2_rows_forward_backward[1000x50x784]": (5.4e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),
+    "mlp2_weight_gradients_and_optimizer[784x50x1000]": (9.8e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),
     "lstm_weight_gradient_rows[289x1024x32768]": (474.3e6, "lstm_wgrad_kernels.hip", "070ad64002f0fb967fbd759a0aabe0851ddfb7e3"),
     "lstm_weight_gradient_rows[289x256x32768]": (147.1e6, "lstm_wgrad_kernels.hip", "070ad64002f0fb967fbd759a0aabe0851ddfb7e3"),
-    "gradient_sums_and_optimizer": (36.5e6, "optim_kernels.hip", "506ae1fc6d64e8a6c4163ab08e75d09c679ff875"),
-    "adam": (2.800e9, "optim_kernels.hip", "506ae1fc6d64e8a6c4163ab08e75d09c679ff875"),
-    "average": (0.900e9, "optim_kernels.hip", "506ae1fc6d64e8a6c4163ab08e75d09c679ff875"),
+    "gradient_sums_and_optimizer": (36.5e6, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
+    "adam": (2.800e9, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
+    "average": (0.900e9, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
 }
 
 
