@@ -64,7 +64,7 @@ struct DeferredReduce {
   int parts = 0, outs = 0;
   float* dst = nullptr;
 };
-constexpr int MAX_DEFERRED = 4;
+constexpr int MAX_DEFERRED = 4, MAX_FINISH_HOLES = 4;
 
 struct sn_ctx {
   uint32_t magic;
@@ -154,8 +154,9 @@ int launch_optimizer(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, const fl
 // One launch that finishes a training step: the deferred reductions d[0..n_d) land in the gradient buffer g (their
 // targets lie inside it), and every element of the flat buffers [0, n) gets its optimizer update, the reduced ones from
 // the sums just made.  Same arithmetic and order as the reduction kernels followed by launch_optimizer.
+// holes: n_holes pairs [first, end) of elements the update leaves alone (tensors that are not trainable)
 int launch_finish(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, float* g, float* s0, float* s1, float* s2, int64_t n, int iter,
-                  const DeferredReduce* defs, int n_defs, const int* skip_if);
+                  const DeferredReduce* defs, int n_defs, const int* skip_if, const int64_t* holes = nullptr, int n_holes = 0);
 // Runs a deferred reduction on its own (when no optimizer launch follows that could take it).
 int launch_deferred_reduce(sn_ctx* ctx, const DeferredReduce& d);
 struct AvgInputs {

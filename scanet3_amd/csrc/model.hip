@@ -518,8 +518,9 @@ static int alloc_replica(sn_replica* r) {
   r->ws_defer.assign(n_ops, nullptr);
   bool penalties = false;
   for (const auto& p : m->params) penalties = penalties || p.reg_kind != SN_REG_NONE;
-  r->fuse_finish = r->has_opt && !(m->flags & SN_FLAG_GEMM_BF16) && !penalties && !mlp2_path(m) && m->trainable_runs.size() == 1 &&
-                   m->trainable_runs[0].first == 0 && m->workspace_elems > 0 && m->workspace_elems <= ((int64_t)64 << 20);
+  // (several runs of trainable tensors, i.e. a BatchNorm's moving statistics in between: the launch skips the gaps)
+  r->fuse_finish = r->has_opt && !(m->flags & SN_FLAG_GEMM_BF16) && !penalties && !mlp2_path(m) && !m->trainable_runs.empty() &&
+                   m->trainable_runs.size() <= (size_t)MAX_FINISH_HOLES && m->workspace_elems > 0 && m->workspace_elems <= ((int64_t)64 << 20);
   if (r->fuse_finish) {
     int n_conv = 0;
     for (size_t i = 0; i < n_ops; ++i)
@@ -1130,10 +1131,16 @@ static int update(sn_replica* r, int iter) {
     SN_REQUIRE(r->pass_iter == iter, "update(%d) behind a gradient pass that was run for iteration %d", iter, r->pass_iter);
     r->updated_in_pass = false;
   } else if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer (fuse_finish: one run from 0)
-    const auto& run = m->trainable_runs[0];
     const int nd = r->n_deferred;
     r->n_deferred = 0;
-    SN_TRY(launch_finish(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], run.second, iter, r->deferred, nd, r->ctx->seq_failed_dev));
+    int64_t holes[2 * MAX_FINISH_HOLES];
+    int n_holes = 0;
+    int64_t at = 0;
+    for (const auto& run : m->trainable_runs) {  // what lies between the runs is not the optimizer's
+      if (run.first > at) { holes[2 * n_holes] = at; holes[2 * n_holes + 1] = run.first; ++n_holes; }
+      at = run.second;
+    }
+    SN_TRY(launch_finish(r->ctx, r->opt, r->w, r->g, r->s[0], r->s[1], r->s[2], at, iter, r->deferred, nd, r->ctx->seq_failed_dev, holes, n_holes));
   } else
   for (const auto& run : m->trainable_runs)
     SN_TRY(launch_optimizer(r->ctx, r->opt, r->w + run.first, r->g + run.first, r->s[0] + run.first, r->s[1] ? r->s[1] + run.first : nullptr,

@@ -201,6 +201,10 @@ struct FinishPlan {
   int64_t first[MAX_DEFERRED];  // index in the flat buffers of r[i].dst[0]
   int block0[MAX_DEFERRED + 1]; // first block of reduction i; block0[0] = number of plain blocks
   int n;
+  // ranges of the flat buffers the optimizer must leave alone (tensors that are not trainable: a BatchNorm's moving
+  // statistics); tensors start on 256-byte boundaries, so no float4 straddles an end
+  int64_t hole_first[MAX_FINISH_HOLES], hole_end[MAX_FINISH_HOLES];
+  int n_holes;
 };
 
 template <int KIND>
@@ -218,6 +222,8 @@ __global__ __launch_bounds__(256) void finish_kernel(float* __restrict__ w, floa
     if (e >= n) return;
     for (int k = 0; k < plan.n; ++k)
       if (e >= plan.first[k] && e < plan.first[k] + plan.r[k].outs) return;  // a reduction block updates these
+    for (int k = 0; k < plan.n_holes; ++k)
+      if (e >= plan.hole_first[k] && e < plan.hole_end[k]) return;           // not trainable
     if (e + 4 <= n) {
       f4 vw = *(const f4*)(w + e), vg = *(const f4*)(g + e), a = *(const f4*)(s0 + e), bb = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
       if (NS > 1) bb = *(const f4*)(s1 + e);
@@ -331,15 +337,23 @@ static int launch_finish_t(sn_ctx* ctx, float* w, float* g, float* s0, float* s1
 }
 
 int launch_finish(sn_ctx* ctx, const sn_optimizer_desc& d, float* w, float* g, float* s0, float* s1, float* s2, int64_t n, int iter,
-                  const DeferredReduce* defs, int n_defs, const int* skip_if) {
+                  const DeferredReduce* defs, int n_defs, const int* skip_if, const int64_t* holes, int n_holes) {
   const int ns = opt_state_count(d.kind);
   SN_REQUIRE(ns > 0, "unknown optimizer kind %d", d.kind);
   SN_REQUIRE(w && g && s0 && (ns < 2 || s1) && (ns < 3 || s2), "optimizer kind %d needs %d state buffers", d.kind, ns);
   SN_REQUIRE(iter >= 1, "iteration numbers start at 1, got %d", iter);
   SN_REQUIRE(n_defs >= 1 && n_defs <= MAX_DEFERRED, "launch_finish takes 1..%d deferred reductions, got %d", MAX_DEFERRED, n_defs);
   SN_REQUIRE(aligned16(w) && aligned16(g) && aligned16(s0) && aligned16(s1) && aligned16(s2), "launch_finish: buffers must be 16-byte aligned");
+  SN_REQUIRE(n_holes >= 0 && n_holes <= MAX_FINISH_HOLES && (n_holes == 0 || holes), "launch_finish takes up to %d untouched ranges, got %d", MAX_FINISH_HOLES, n_holes);
   FinishPlan plan;
   plan.n = n_defs;
+  plan.n_holes = n_holes;
+  for (int i = 0; i < n_holes; ++i) {
+    SN_REQUIRE(holes[2 * i] % 4 == 0 && holes[2 * i + 1] % 4 == 0 && holes[2 * i] <= holes[2 * i + 1] && holes[2 * i + 1] <= n,
+               "launch_finish: untouched range %d is not made of whole float4s of the buffer", i);
+    plan.hole_first[i] = holes[2 * i];
+    plan.hole_end[i] = holes[2 * i + 1];
+  }
   int64_t blocks = ceil_div(ceil_div(n, 4), 128);
   plan.block0[0] = (int)blocks;
   for (int i = 0; i < n_defs; ++i) {
