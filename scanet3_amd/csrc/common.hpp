@@ -180,6 +180,12 @@ int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp
 // (row_loss: `rows` floats of scratch; loss_dev == nullptr: the loss value is not wanted, its final reduction is skipped)
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
                        int cols, bool stable);
+// The same when the logits still lie as `parts` partial sums [part][rows * cols] of a Dense layer's forward product (at most
+// SOFTMAX_PARTIALS_MAX_COLS columns): the kernel adds them in the order of that product's own reduction, adds the bias
+// (may be null), writes the logits to z_out and goes on as launch_softmax_cce.
+constexpr int SOFTMAX_PARTIALS_MAX_COLS = 16;
+int launch_softmax_cce_partials(sn_ctx* ctx, const float* partial, int parts, const float* bias, float* z_out, const float* y, float* p,
+                                float* dz, float* loss_dev, float* row_loss, int rows, int cols, bool stable);
 // out[c] = sum over rows of dy[r*ld + c]; `ws` (optional) lets many rows be summed in parallel slices
 int launch_col_sum(sn_ctx* ctx, const float* dy, int64_t ld, float* out, int64_t rows, int cols, float* ws, int64_t ws_elems);
 // partials: at least 1024 floats of scratch
@@ -303,8 +309,9 @@ int launch_gemm(sn_ctx* ctx, const GemmDesc& g, const Epilogue& ep, float* works
 // Gradients of a Dense layer from many features onto at most 16 units, as row streams over X (fp32, contiguous
 // [rows, in_f] / [in_f, out_f] / [rows, out_f] tensors); dense_skinny_shape says whether a shape is in their range.
 bool dense_skinny_shape(int rows, int in_f, int out_f);
-int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f);
-int launch_dense_skinny_dx(sn_ctx* ctx, const float* dy, const float* w, float* dx, int rows, int in_f, int out_f);
+// (w and dx, both or neither: the same launch also writes the input gradient dx = dy . w^T)
+int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f,
+                           const float* w = nullptr, float* dx = nullptr);
 // The same layer forward for small batches (partial sums per feature chunk in the workspace, then a fixed-order reduction
 // that applies e's bias and activation); dense_skinny_fwd_shape says whether shape and workspace are in its range.
 // A Dense layer onto at most 4 units from at most 1024 features (a regression head behind a recurrent layer): forward in one
@@ -315,8 +322,10 @@ int launch_dense_tiny_bwd(sn_ctx* ctx, const float* x, const float* y, const flo
                           int in_f, int out_f, int act, float act_param, float* ws, int64_t ws_elems);
 bool dense_skinny_fwd_shape(int rows, int in_f, int out_f, int64_t ws_elems);
 int64_t dense_skinny_fwd_workspace(int rows, int in_f, int out_f);  // floats of workspace the forward form needs
+// parts_left (optional): the reduction is not launched; *parts_left partial sums [part][rows * out_f] stay in ws for a
+// launch of the caller's that adds them in the same order (launch_softmax_cce_partials)
 int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,
-                            int64_t ws_elems);
+                            int64_t ws_elems, int* parts_left = nullptr);
 
 // bf16 fast path (gemm_bf16.hip): the three products of a Dense layer on bf16 operands read as the tensors lie (no
 // transposed copies), fp32 accumulation.  Besides or instead of the fp32 result (e.out, may be null) the epilogue can

@@ -344,6 +344,89 @@ __global__ __launch_bounds__(256) void softmax_cce_reg_kernel(const float* __res
   if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
 }
 
+// The row kernel for logits that still lie as partial sums [part][rows * cols] of the Dense product below (a product over
+// many features that left one partial result per feature chunk).  64 lanes per logit walk every 64th part, their sums
+// are added as a chain, then the bias: the order of the product's own reduction kernel.  The first wavefront then holds
+// the row's logits, one per lane, and finishes as softmax_cce_reg_kernel<1> does with 64 threads.
+__global__ __launch_bounds__(1024) void softmax_cce_partials_kernel(const float* __restrict__ partial, int parts, const float* __restrict__ bias,
+                                                                     float* __restrict__ z_out, const float* __restrict__ y,
+                                                                     float* __restrict__ p, float* __restrict__ dz, float* __restrict__ row_loss,
+                                                                     int rows, int cols, int stable, float neg_inv_rows) {
+  __shared__ float sm[64][SOFTMAX_PARTIALS_MAX_COLS];
+  const int ol = threadIdx.x % cols, pl = threadIdx.x / cols;  // blockDim.x = 64 * cols
+  const int64_t outs = (int64_t)rows * cols;
+  const int64_t base = (int64_t)blockIdx.x * cols;
+  {
+    const int64_t o = base + ol;
+    float s = 0.f;
+    for (int i = pl; i < parts; i += 64 * 8) {  // 8 loads in flight, added in part order
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = i + 64 * u < parts ? partial[(int64_t)(i + 64 * u) * outs + o] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    sm[pl][ol] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x >= 64) return;
+  const int c = threadIdx.x;
+  const bool live = c < cols;
+  float zv = 0.f, yv = 0.f;
+  if (live) {
+    float t = 0.f;
+#pragma unroll 8
+    for (int j = 0; j < 64; ++j) t += sm[j][c];
+    if (bias) t = t + bias[c];
+    z_out[base + c] = t;
+    zv = t;
+    yv = y[base + c];
+  }
+  const float eps = 1e-8f;
+  float mx = 0.f;
+  if (stable) mx = wave_max(live ? zv : -INFINITY);
+  float s = 0.f;
+  if (live) {
+    zv = expf(zv - mx);
+    s += zv;
+  }
+  const float total = 0.f + wave_sum(s);
+  float term = 0.f, dot = 0.f;
+  if (live) {
+    const float pi = zv / total;
+    zv = pi;
+    term += yv * logf(pi + eps);
+    dot += pi * ((yv * neg_inv_rows) / (pi + eps));
+  }
+  const float row_term = 0.f + wave_sum(term);
+  const float row_dot = 0.f + wave_sum(dot);
+  if (live) {
+    const float pi = zv;
+    const float dpi = (yv * neg_inv_rows) / (pi + eps);
+    p[base + c] = pi;
+    dz[base + c] = pi * dpi - pi * row_dot;
+  }
+  if (c == 0) row_loss[blockIdx.x] = row_term;
+}
+
+int launch_softmax_cce_partials(sn_ctx* ctx, const float* partial, int parts, const float* bias, float* z_out, const float* y, float* p,
+                                float* dz, float* loss_dev, float* row_loss, int rows, int cols, bool stable) {
+  SN_REQUIRE(rows > 0 && cols > 0 && cols <= SOFTMAX_PARTIALS_MAX_COLS && parts > 0, "softmax over partial sums: %d rows, %d columns, %d parts", rows, cols, parts);
+  {
+    LaunchScope scope(ctx, "small_output_reduce_softmax_crossentropy_fused");
+    const float neg_inv_rows = -(1.0f / (float)rows);
+    hipLaunchKernelGGL(softmax_cce_partials_kernel, dim3(rows), dim3(64 * cols), 0, ctx->stream, partial, parts, bias, z_out, y, p, dz, row_loss,
+                       rows, cols, stable ? 1 : 0, neg_inv_rows);
+  }
+  if (loss_dev) {
+    LaunchScope scope(ctx, "loss_stage2");
+    hipLaunchKernelGGL(loss_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, (int)SN_LOSS_CATEGORICAL_CROSSENTROPY, (const float*)row_loss,
+                       rows, loss_dev, 0.f, (float)rows);
+  }
+  SN_HIP(hipGetLastError());
+  return SN_OK;
+}
+
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
                        int cols, bool stable) {
   SN_REQUIRE(rows > 0 && cols > 0, "loss over an empty batch");

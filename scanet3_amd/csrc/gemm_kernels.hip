@@ -1784,35 +1784,44 @@ int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, cons
 // as [rows + 1][4 NQ] floats (units padded with zeros, one all-zero row for out-of-range rows) and is read as broadcasts.
 constexpr int SKINNY_MAX_UNITS = 16, SKINNY_MIN_FEATURES = 2048, SKINNY_MAX_LDS_FLOATS = 8192, SKINNY_ROWS_IN_FLIGHT = 32;
 
-template <int NQ>
+template <int NQ, int NT = 256>  // NT: threads of the workgroup
 __device__ __forceinline__ void skinny_stage_dy(f4v* dyl, const float* __restrict__ dy, int rows, int out_f) {
   float* flat = reinterpret_cast<float*>(dyl);
   constexpr int padded = NQ * 4;
   const int total = (rows + 1) * padded;
-  for (int base = 0; base < total; base += 256 * 8) {  // 8 loads per thread are issued before any of them is stored
+  for (int base = 0; base < total; base += NT * 8) {  // 8 loads per thread are issued before any of them is stored
     float v[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int e = base + u * 256 + (int)threadIdx.x;
+      const int e = base + u * NT + (int)threadIdx.x;
       const int b = e / padded, n = e % padded;
       v[u] = (b < rows && n < out_f) ? dy[(int64_t)b * out_f + n] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int e = base + u * 256 + (int)threadIdx.x;
+      const int e = base + u * NT + (int)threadIdx.x;
       if (e < total) flat[e] = v[u];
     }
   }
 }
 
 // dW[i, n] = sum_b X[b, i] dY[b, n] (math/alg/AllKernels.scala:382-388, the left operand's gradient of a matrix product
-// seen from the weights), db[n] = sum_b dY[b, n].  The four wavefronts' partial sums meet in LDS and are added in wavefront order.
-template <int NQ>
-__global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dw,
-                                                               float* __restrict__ db, int rows, int in_f, int out_f, int rows_per_wave) {
+// seen from the weights), db[n] = sum_b dY[b, n].  The wavefronts' partial sums meet in LDS and are added in wavefront order.
+// With DX the same launch also writes the layer's input gradient dX[b, i] = sum_n dY[b, n] W[i, n] (the right operand's
+// side): a lane keeps its feature's weight row in registers and walks its wavefront's rows of dY, which are in LDS
+// already, while the first rows of X are still on their way.
+constexpr int SKINNY_DW_WAVES = 4;
+template <int NQ, bool DX>
+__global__ __launch_bounds__(SKINNY_DW_WAVES * 64) void dense_skinny_dw_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dw,
+                                                               float* __restrict__ db, int rows, int in_f, int out_f, int rows_per_wave,
+                                                               const float* __restrict__ w, float* __restrict__ dx) {
   extern __shared__ f4v skinny_lds[];
   f4v* dyl = skinny_lds;                         // [rows + 1][NQ]
-  f4v* part = skinny_lds + (rows + 1) * NQ;      // [3][NQ][64]
+  f4v* part = skinny_lds + (rows + 1) * NQ;      // [SKINNY_DW_WAVES - 1][NQ][64]
+  // the workgroup's 64 rows of W, then of dW, as they lie in memory (64 * out_f values in a row): they cross between
+  // memory and LDS as one run, neighbouring threads on neighbouring values, and between LDS and the lanes row by row
+  // (a lane fetching or storing its own row would touch a cache line per lane and unit)
+  float* wrows = reinterpret_cast<float*>(part + (SKINNY_DW_WAVES - 1) * NQ * 64);  // [64][out_f]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = blockIdx.x * 64 + lane;
   const bool live = i < in_f;
@@ -1824,8 +1833,39 @@ __global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __res
   // the first batch of X is on its way while dY is staged
 #pragma unroll
   for (int u = 0; u < U; ++u) xv[u] = b0 + u < b1 ? xp[(int64_t)(b0 + u) * in_f] : 0.f;
-  skinny_stage_dy<NQ>(dyl, dy, rows, out_f);
+  const int64_t run0 = (int64_t)blockIdx.x * 64 * out_f, run_end = (int64_t)in_f * out_f;
+  if constexpr (DX) {
+    for (int f = threadIdx.x; f < 64 * out_f; f += SKINNY_DW_WAVES * 64) wrows[f] = run0 + f < run_end ? w[run0 + f] : 0.f;
+  }
+  skinny_stage_dy<NQ, SKINNY_DW_WAVES * 64>(dyl, dy, rows, out_f);
   __syncthreads();
+  f4v wr[DX ? NQ : 1];
+  if constexpr (DX) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float v = wrows[lane * out_f + (q * 4 + k < out_f ? q * 4 + k : 0)];
+        wr[q][k] = q * 4 + k < out_f ? v : 0.f;
+      }
+    }
+  }
+  if constexpr (DX) {  // while the first rows of X are on their way
+    if (live) {
+      float* o = dx + i;
+#pragma unroll 4
+      for (int b = b0; b < b1; ++b) {
+        float s = 0.f;
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const f4v d = dyl[b * NQ + q];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) s = __builtin_fmaf(d[k], wr[q][k], s);
+        }
+        o[(int64_t)b * in_f] = s;
+      }
+    }
+  }
   f4v acc[NQ];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) acc[q] = f4v{0.f, 0.f, 0.f, 0.f};
@@ -1852,7 +1892,7 @@ __global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __res
   __syncthreads();
   if (wave == 0) {
 #pragma unroll
-    for (int w = 0; w < 3; ++w) {
+    for (int w = 0; w < SKINNY_DW_WAVES - 1; ++w) {
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const f4v p = part[(w * NQ + q) * 64 + lane];
@@ -1860,15 +1900,18 @@ __global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __res
         for (int k = 0; k < 4; ++k) acc[q][k] = acc[q][k] + p[k];
       }
     }
-    if (live) {
-      float* o = dw + (int64_t)i * out_f;
+    // (every wavefront has read its rows of W long before: the block-wide barrier above lies in between)
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
+    for (int q = 0; q < NQ; ++q) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          if (q * 4 + k < out_f) o[q * 4 + k] = acc[q][k];
-      }
+      for (int k = 0; k < 4; ++k)
+        if (q * 4 + k < out_f) wrows[lane * out_f + q * 4 + k] = acc[q][k];
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int f = lane; f < 64 * out_f; f += 64)
+      if (run0 + f < run_end) dw[run0 + f] = wrows[f];
   } else if (wave == 1 && blockIdx.x == 0 && db && lane < out_f) {
     const float* flat = reinterpret_cast<const float*>(dyl);
     float s = 0.f;
@@ -1877,54 +1920,28 @@ __global__ __launch_bounds__(256) void dense_skinny_dw_kernel(const float* __res
   }
 }
 
-// dX[b, i] = sum_n dY[b, n] W[i, n] (AllKernels.scala:382-388, the right operand's side): a lane keeps its feature's
-// weight row in registers and walks its wavefront's rows.
-template <int NQ>
-__global__ __launch_bounds__(256) void dense_skinny_dx_kernel(const float* __restrict__ dy, const float* __restrict__ w, float* __restrict__ dx,
-                                                               int rows, int in_f, int out_f, int rows_per_wave) {
-  extern __shared__ f4v skinny_lds[];
-  f4v* dyl = skinny_lds;
-  skinny_stage_dy<NQ>(dyl, dy, rows, out_f);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int i = blockIdx.x * 64 + lane;
-  const bool live = i < in_f;
-  f4v wr[NQ];
-#pragma unroll
-  for (int q = 0; q < NQ; ++q) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) wr[q][k] = (live && q * 4 + k < out_f) ? w[(int64_t)i * out_f + q * 4 + k] : 0.f;
-  }
-  __syncthreads();
-  const int b0 = wave * rows_per_wave;
-  const int b1 = b0 + rows_per_wave < rows ? b0 + rows_per_wave : rows;
-  if (!live) return;
-  float* o = dx + i;
-#pragma unroll 4
-  for (int b = b0; b < b1; ++b) {
-    float s = 0.f;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-      const f4v d = dyl[b * NQ + q];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) s = __builtin_fmaf(d[k], wr[q][k], s);
-    }
-    o[(int64_t)b * in_f] = s;
-  }
-}
-
 bool dense_skinny_shape(int rows, int in_f, int out_f) {
   const int nq = (out_f + 3) / 4;
   return rows >= 4 && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES && (int64_t)(rows + 1) * nq * 4 <= SKINNY_MAX_LDS_FLOATS;
 }
 
-int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f) {
+int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f, const float* w,
+                           float* dx) {
   SN_REQUIRE(dense_skinny_shape(rows, in_f, out_f), "dense_weight_gradient_rows: shape outside the kernel's range");
-  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, 4);
+  SN_REQUIRE((w != nullptr) == (dx != nullptr), "dense_weight_gradient_rows: the input gradient needs the weights and a place to go");
+  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, SKINNY_DW_WAVES);
   const unsigned blocks = (unsigned)ceil_div(in_f, 64);
-  const size_t lds = ((size_t)(rows + 1) * nq + (size_t)3 * nq * 64) * sizeof(f4v);
-  LaunchScope scope(ctx, "dense_weight_gradient_rows", in_f, out_f, rows);
-#define SN_SKINNY_DW(NQ) \
-  hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ>), dim3(blocks), dim3(256), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f, rows_per_wave)
+  const size_t lds = ((size_t)(rows + 1) * nq + (size_t)(SKINNY_DW_WAVES - 1) * nq * 64) * sizeof(f4v) + (size_t)64 * out_f * sizeof(float);
+  LaunchScope scope(ctx, dx ? "dense_weight_and_input_gradient_rows" : "dense_weight_gradient_rows", in_f, out_f, rows);
+#define SN_SKINNY_DW(NQ)                                                                                                                     \
+  do {                                                                                                                                       \
+    if (dx)                                                                                                                                  \
+      hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ, true>), dim3(blocks), dim3(SKINNY_DW_WAVES * 64), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f,    \
+                         rows_per_wave, w, dx);                                                                                              \
+    else                                                                                                                                     \
+      hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ, false>), dim3(blocks), dim3(SKINNY_DW_WAVES * 64), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f,   \
+                         rows_per_wave, w, dx);                                                                                              \
+  } while (0)
   switch (nq) {
     case 1: SN_SKINNY_DW(1); break;
     case 2: SN_SKINNY_DW(2); break;
@@ -1936,32 +1953,13 @@ int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* 
   return SN_OK;
 }
 
-int launch_dense_skinny_dx(sn_ctx* ctx, const float* dy, const float* w, float* dx, int rows, int in_f, int out_f) {
-  SN_REQUIRE(dense_skinny_shape(rows, in_f, out_f), "dense_input_gradient_rows: shape outside the kernel's range");
-  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, 4);
-  const unsigned blocks = (unsigned)ceil_div(in_f, 64);
-  const size_t lds = (size_t)(rows + 1) * nq * sizeof(f4v);
-  LaunchScope scope(ctx, "dense_input_gradient_rows", rows, in_f, out_f);
-#define SN_SKINNY_DX(NQ) \
-  hipLaunchKernelGGL((dense_skinny_dx_kernel<NQ>), dim3(blocks), dim3(256), lds, ctx->stream, dy, w, dx, rows, in_f, out_f, rows_per_wave)
-  switch (nq) {
-    case 1: SN_SKINNY_DX(1); break;
-    case 2: SN_SKINNY_DX(2); break;
-    case 3: SN_SKINNY_DX(3); break;
-    default: SN_SKINNY_DX(4); break;
-  }
-#undef SN_SKINNY_DX
-  SN_HIP(hipGetLastError());
-  return SN_OK;
-}
-
 // The same layer forward for a batch of at most SKINNY_FWD_MAX_ROWS rows: Y = X W is 4 B of X per 2 out_f flops.  A workgroup
 // owns SKINNY_FWD_CHUNK consecutive features: its wavefronts fetch their rows of that chunk in one go (a lane takes two
 // neighbouring features, so a wavefront reads 512 contiguous bytes per row, all rows in flight), the chunk turns in
 // LDS ([row][129]: rows on different banks), then thread (row pair, unit quad) adds its 128 products per output in feature order and the
 // workgroup leaves one partial [rows][out_f]; gemm_small_reduce_kernel adds the partials in a fixed order and applies the
 // bias and the activation.
-constexpr int SKINNY_FWD_CHUNK = 128, SKINNY_FWD_MAX_ROWS = 112, SKINNY_FWD_ROWS_PER_WAVE = SKINNY_FWD_MAX_ROWS / 4;
+constexpr int SKINNY_FWD_CHUNK = 64, SKINNY_FWD_MAX_ROWS = 112, SKINNY_FWD_ROWS_PER_WAVE = SKINNY_FWD_MAX_ROWS / 4;
 
 template <int NQ>
 __global__ __launch_bounds__(256) void dense_skinny_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ partial,
@@ -1972,11 +1970,19 @@ __global__ __launch_bounds__(256) void dense_skinny_fwd_kernel(const float* __re
   f4v* wsm = reinterpret_cast<f4v*>(skinny_fwd_lds + ((rows * PITCH + 3) & ~3));  // [KC][NQ]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i0 = blockIdx.x * KC;
-  const int fa = i0 + 2 * lane;  // this lane's two features
+  constexpr int FL = KC / 64;     // features per lane: 1 or 2
+  const int fa = i0 + FL * lane;  // this lane's first feature
   // whole chunks of rows that start on 8-byte boundaries take 8-byte loads without a branch (rows past the batch re-read the last row)
-  const bool whole = i0 + KC <= in_f && (in_f & 1) == 0 && (reinterpret_cast<uintptr_t>(x) & 7) == 0;
+  const bool whole = FL == 2 && i0 + KC <= in_f && (in_f & 1) == 0 && (reinterpret_cast<uintptr_t>(x) & 7) == 0;
   float2 xv[R];
-  if (whole) {
+  if (FL == 1) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int b = wave + 4 * u < rows ? wave + 4 * u : rows - 1;
+      xv[u].x = fa < in_f ? x[(int64_t)b * in_f + fa] : 0.f;
+      xv[u].y = 0.f;
+    }
+  } else if (whole) {
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int b = wave + 4 * u < rows ? wave + 4 * u : rows - 1;
@@ -2013,8 +2019,8 @@ __global__ __launch_bounds__(256) void dense_skinny_fwd_kernel(const float* __re
   for (int u = 0; u < R; ++u) {
     const int b = wave + 4 * u;
     if (b < rows) {
-      xs[b * PITCH + 2 * lane] = xv[u].x;
-      xs[b * PITCH + 2 * lane + 1] = xv[u].y;
+      xs[b * PITCH + FL * lane] = xv[u].x;
+      if (FL == 2) xs[b * PITCH + FL * lane + 1] = xv[u].y;
     }
   }
   __syncthreads();
@@ -2059,7 +2065,7 @@ bool dense_skinny_fwd_shape(int rows, int in_f, int out_f, int64_t ws_elems) {
 }
 
 int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const Epilogue& e, int rows, int in_f, int out_f, float* ws,
-                            int64_t ws_elems) {
+                            int64_t ws_elems, int* parts_left) {
   SN_REQUIRE(ws && dense_skinny_fwd_shape(rows, in_f, out_f, ws_elems), "dense_forward_rows: shape outside the kernel's range");
   const int nq = (out_f + 3) / 4;
   const int parts = (int)ceil_div(in_f, SKINNY_FWD_CHUNK);
@@ -2075,6 +2081,11 @@ int launch_dense_skinny_fwd(sn_ctx* ctx, const float* x, const float* w, const E
       default: SN_SKINNY_FWD(4); break;
     }
 #undef SN_SKINNY_FWD
+  }
+  if (parts_left) {  // the caller's next launch adds the partial sums itself
+    *parts_left = parts;
+    SN_HIP(hipGetLastError());
+    return SN_OK;
   }
   StdEpilogue ep{e};
   LaunchScope scope(ctx, "small_output_reduce");

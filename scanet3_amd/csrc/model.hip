@@ -111,6 +111,8 @@ struct sn_replica {
   // convolution has a workspace of its own (the shared one is overwritten by the next product).
   bool updated_in_pass = false;  // the gradient pass of this step has applied the optimizer itself
   int pass_iter = 0;             // iteration number of the update that follows the running gradient pass (0: none follows)
+  bool leave_logit_parts = false;  // the running forward pass may leave the last Dense product's partial sums to the loss kernel
+  int logit_parts = 0;             // how many it left in ws (0: the logits are complete)
   bool fuse_finish = false, defer_now = false;
   std::vector<float*> ws_defer;
   DeferredReduce deferred[MAX_DEFERRED];
@@ -607,7 +609,10 @@ static int forward(sn_replica* r, const float* x, int rows, bool skip_last = fal
         } else if (!bf16 && dense_tiny_shape(rows, in_f, out_f, m->workspace_elems)) {  // a few units behind a short row: one launch
           SN_TRY(launch_dense_tiny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f));
         } else if (!bf16 && r->ws && dense_skinny_fwd_shape(rows, in_f, out_f, m->workspace_elems)) {
-          SN_TRY(launch_dense_skinny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f, r->ws, m->workspace_elems));
+          // the logits of a Softmax output under the fused loss kernel: that kernel adds the partial sums itself
+          const bool leave = r->leave_logit_parts && i + 2 == m->ops.size() && op.act == SN_ACT_IDENTITY && out_f <= SOFTMAX_PARTIALS_MAX_COLS;
+          SN_TRY(launch_dense_skinny_fwd(ctx, in, param_ptr(r, r->w, op.w), ep, rows, in_f, out_f, r->ws, m->workspace_elems,
+                                         leave ? &r->logit_parts : nullptr));
         } else {
           GemmDesc g{in, in_f, 1, param_ptr(r, r->w, op.w), out_f, 1, rows, out_f, in_f};
           SN_TRY(launch_gemm(ctx, g, ep, r->ws, m->workspace_elems, bf16));
@@ -791,11 +796,10 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
         }
         if (op.act != SN_ACT_IDENTITY) SN_TRY(launch_act_bwd(ctx, r->act[i], dy, dy, (int64_t)rows * out_f, op.act, op.act_param));
         if (!bf16 && dense_skinny_shape(rows, in_f, out_f)) {  // a few units behind many features: row streams, no matrix tiles
-          SN_TRY(launch_dense_skinny_dw(ctx, in, dy, param_ptr(r, r->g, op.w), param_ptr(r, r->g, op.b), rows, in_f, out_f));
-          if (need_dx) {
-            SN_TRY(launch_dense_skinny_dx(ctx, dy, param_ptr(r, r->w, op.w), dx, rows, in_f, out_f));
-            cur ^= 1;
-          }
+          // one launch for both gradients: the rows of dY are staged once
+          SN_TRY(launch_dense_skinny_dw(ctx, in, dy, param_ptr(r, r->g, op.w), param_ptr(r, r->g, op.b), rows, in_f, out_f,
+                                        need_dx ? param_ptr(r, r->w, op.w) : nullptr, need_dx ? dx : nullptr));
+          if (need_dx) cur ^= 1;
           break;
         }
         {  // dW = X^T . dY (math/alg/AllKernels.scala:382-388)
@@ -1100,9 +1104,20 @@ static int grad_pass_body(sn_replica* r, const float* x, const float* y, int row
   }
   if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
     // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
-    SN_TRY(forward(r, x, rows, true, true));
-    SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], want_loss ? r->loss_dev : nullptr,
-                              r->loss_partials, rows, (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+    r->logit_parts = 0;
+    r->leave_logit_parts = m->ops[last - 1].kind == OP_DENSE;
+    const int rc = forward(r, x, rows, true, true);
+    r->leave_logit_parts = false;
+    SN_TRY(rc);
+    if (r->logit_parts > 0) {
+      const Op& d = m->ops[last - 1];
+      SN_TRY(launch_softmax_cce_partials(r->ctx, r->ws, r->logit_parts, param_ptr(r, r->w, d.b), r->act[last - 1], y, r->act[last], r->grad_buf[1],
+                                         want_loss ? r->loss_dev : nullptr, r->loss_partials, rows, (int)m->ops[last].out_elems,
+                                         (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+    } else {
+      SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], want_loss ? r->loss_dev : nullptr,
+                                r->loss_partials, rows, (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+    }
     if (want_loss) SN_TRY(add_penalties(r, true));
     return backward(r, x, rows, last - 1, 1);
   }
@@ -1130,7 +1145,7 @@ static int update(sn_replica* r, int iter) {
   if (r->updated_in_pass) {  // the gradient pass has applied the update itself (with this iteration number)
     SN_REQUIRE(r->pass_iter == iter, "update(%d) behind a gradient pass that was run for iteration %d", iter, r->pass_iter);
     r->updated_in_pass = false;
-  } else if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer (fuse_finish: one run from 0)
+  } else if (r->n_deferred > 0) {  // one launch: the open gradient sums, then the update of the whole buffer
     const int nd = r->n_deferred;
     r->n_deferred = 0;
     int64_t holes[2 * MAX_FINISH_HOLES];

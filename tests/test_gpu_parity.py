@@ -544,6 +544,35 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     h.close()
 
 
+@pytest.mark.parametrize("name", ["mlp_tanh_relu", "lenet_small", "dense_many_features_few_units", "dense_odd_feature_count_9_units"])
+def test_stable_softmax_flag_changes_nothing_at_moderate_logits(S, ctx, name):
+    """SN_FLAG_STABLE_SOFTMAX subtracts the row maximum before exp: mathematically the same softmax, so loss and gradients
+    must agree with the oracle (which, like Activation.scala:63-69, does not subtract) as closely as without the flag.
+    Covers the loss kernel that reads finished logits and the one that adds a Dense product's partial sums itself."""
+    from scanet3_amd import _lib as L
+    spec, loss, in_shape, batch, kind = MODELS[name]
+    rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000 + 77)
+    h = Harness(S, ctx, spec, loss, in_shape, batch, flags=L.FLAG_STABLE_SOFTMAX)
+    om = h.omodel
+    params = glorot_params(om, (batch,) + in_shape, rng)
+    for p in params:
+        if params[p].ndim == 1:
+            params[p] = params[p] + rng.uniform(-0.1, 0.1, params[p].shape).astype(f32)
+    out_dim = om.out_shape((batch,) + in_shape)[-1]
+    x, y = make_data(kind, rng, batch, in_shape, out_dim)
+    h.rep.set_params(params)
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    oloss, ograds = om.grad(x, y, params)
+    gloss = h.rep.grad(xb, yb)
+    assert abs(gloss - float(oloss)) <= TOL_GEMM * max(1.0, abs(float(oloss)))
+    ggrads = h.rep.get_grads()
+    _, grads64 = om.grad(x.astype(np.float64), y.astype(np.float64), {k: v.astype(np.float64) for k, v in params.items()})
+    for p in ograds:
+        assert rel_err(ggrads[p], ograds[p]) <= max(TOL_GEMM, 3.0 * rel_err(ograds[p], grads64[p])), p
+    assert rel_err(h.rep.forward(xb, training=True), om.forward(x, params, training=True)) <= TOL_GEMM
+    h.close()
+
+
 @pytest.mark.parametrize("name,steps", [("mlp_cfg1", 10), ("mlp2_odd_sizes_tanh", 15), ("mlp2_regularized", 15), ("lenet_small", 30), ("lstm_small", 30), ("lstm_fused_shape", 20), ("lstm_stacked", 15), ("simple_rnn_stacked", 15), ("simple_rnn_small", 30),
                                         ("mlp_batchnorm", 20), ("cnn_batchnorm", 12), ("cnn_batchnorm_fused", 12), ("mlp_bce_l2", 25),
                                         ("lstm_regularized", 15), ("batchnorm_regularized", 15)])
