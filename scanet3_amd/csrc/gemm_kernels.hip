@@ -1778,177 +1778,109 @@ int launch_lstm_wgrad(sn_ctx* ctx, const float* x, const float* h_prev_all, cons
 
 // ============================================================================ Dense onto a few units: backward
 // A Dense layer from tens of thousands of features onto at most 16 units (a classifier head behind Flatten) with a
-// batch of a few hundred rows: its gradients are memory-bound streams over X, not matrix-core work.  A workgroup of
-// 4 wavefronts owns 64 consecutive features; wavefront w takes every row b with b / rows_per_wave == w, a lane one
-// feature, so every load or store of a wavefront is one contiguous 256-byte run of a row of X (or dX).  dY sits in LDS
-// as [rows + 1][4 NQ] floats (units padded with zeros, one all-zero row for out-of-range rows) and is read as broadcasts.
-constexpr int SKINNY_MAX_UNITS = 16, SKINNY_MIN_FEATURES = 2048, SKINNY_MAX_LDS_FLOATS = 8192, SKINNY_ROWS_IN_FLIGHT = 32;
-
-template <int NQ, int NT = 256>  // NT: threads of the workgroup
-__device__ __forceinline__ void skinny_stage_dy(f4v* dyl, const float* __restrict__ dy, int rows, int out_f) {
-  float* flat = reinterpret_cast<float*>(dyl);
-  constexpr int padded = NQ * 4;
-  const int total = (rows + 1) * padded;
-  for (int base = 0; base < total; base += NT * 8) {  // 8 loads per thread are issued before any of them is stored
-    float v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int e = base + u * NT + (int)threadIdx.x;
-      const int b = e / padded, n = e % padded;
-      v[u] = (b < rows && n < out_f) ? dy[(int64_t)b * out_f + n] : 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int e = base + u * NT + (int)threadIdx.x;
-      if (e < total) flat[e] = v[u];
-    }
-  }
-}
+// batch of a few hundred rows: its gradients are memory-bound streams over X and dX (one read and one write of a
+// [rows, features] tensor), with a launch that fills the chip along the feature axis.
+constexpr int SKINNY_MAX_UNITS = 16, SKINNY_MIN_FEATURES = 2048, SKINNY_MAX_ROWS = 2048;
 
 // dW[i, n] = sum_b X[b, i] dY[b, n] (math/alg/AllKernels.scala:382-388, the left operand's gradient of a matrix product
-// seen from the weights), db[n] = sum_b dY[b, n].  The wavefronts' partial sums meet in LDS and are added in wavefront order.
-// With DX the same launch also writes the layer's input gradient dX[b, i] = sum_n dY[b, n] W[i, n] (the right operand's
-// side): a lane keeps its feature's weight row in registers and walks its wavefront's rows of dY, which are in LDS
-// already, while the first rows of X are still on their way.
-constexpr int SKINNY_DW_WAVES = 4;
-template <int NQ, bool DX>
-__global__ __launch_bounds__(SKINNY_DW_WAVES * 64) void dense_skinny_dw_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dw,
-                                                               float* __restrict__ db, int rows, int in_f, int out_f, int rows_per_wave,
-                                                               const float* __restrict__ w, float* __restrict__ dx) {
-  extern __shared__ f4v skinny_lds[];
-  f4v* dyl = skinny_lds;                         // [rows + 1][NQ]
-  f4v* part = skinny_lds + (rows + 1) * NQ;      // [SKINNY_DW_WAVES - 1][NQ][64]
-  // the workgroup's 64 rows of W, then of dW, as they lie in memory (64 * out_f values in a row): they cross between
-  // memory and LDS as one run, neighbouring threads on neighbouring values, and between LDS and the lanes row by row
-  // (a lane fetching or storing its own row would touch a cache line per lane and unit)
-  float* wrows = reinterpret_cast<float*>(part + (SKINNY_DW_WAVES - 1) * NQ * 64);  // [64][out_f]
+// seen from the weights), db[n] = sum_b dY[b, n] and, with DX, the layer's input gradient dX[b, i] = sum_n dY[b, n] W[i, n]
+// (the right operand's side) in one launch on the matrix cores (v_mfma_f32_16x16x4_f32), without LDS: a wavefront owns
+// 16 features and walks all rows.  dW tile [16 features][16 units] += A B with A[m = feature][k = row] = X[row, feature] and
+// B[k = row][n = unit] = dY[row, unit]: lane (c = l % 16, g = l / 16) loads X[4 s + g, feature c] and dY[4 s + g, unit c]
+// for step s, 32 steps in flight.  dX tile [16 rows][16 features] = A B with A[m = row][k = unit] = dY[row, unit] and
+// B[k = unit][n = feature] = W[feature, unit], written while the rows of X are on their way.  The lanes of one
+// wavefront together hold every value of dY, so the bias gradient is their sum (workgroup 0, wavefront 0).
+// An accumulator value v of lane (c, g) is element [4 g + v][c] of its tile.
+template <bool DX>
+__global__ __launch_bounds__(256) void dense_skinny_grad_mfma_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                                      float* __restrict__ dw, float* __restrict__ db, int rows, int in_f,
+                                                                      int out_f, const float* __restrict__ w, float* __restrict__ dx) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int i = blockIdx.x * 64 + lane;
-  const bool live = i < in_f;
-  const float* xp = x + (live ? i : 0);
-  const int b0 = wave * rows_per_wave;
-  const int b1 = b0 + rows_per_wave < rows ? b0 + rows_per_wave : rows;
-  constexpr int U = SKINNY_ROWS_IN_FLIGHT;
-  float xv[U];
-  // the first batch of X is on its way while dY is staged
+  const int c = lane & 15, g = lane >> 4;
+  const int i0 = (blockIdx.x * 4 + wave) * 16;
+  if (i0 >= in_f) return;
+  const int feat = i0 + c;
+  const bool live = feat < in_f;
+  const float* xp = x + (live ? feat : 0);
+  const bool unit = c < out_f;
+  const float* dyp = dy + (unit ? c : 0);
+  constexpr int S = 32;  // steps (of 4 rows) in flight
+  const int steps = (rows + 3) >> 2;
+  float xv[S], dv[S];
 #pragma unroll
-  for (int u = 0; u < U; ++u) xv[u] = b0 + u < b1 ? xp[(int64_t)(b0 + u) * in_f] : 0.f;
-  const int64_t run0 = (int64_t)blockIdx.x * 64 * out_f, run_end = (int64_t)in_f * out_f;
-  if constexpr (DX) {
-    for (int f = threadIdx.x; f < 64 * out_f; f += SKINNY_DW_WAVES * 64) wrows[f] = run0 + f < run_end ? w[run0 + f] : 0.f;
+  for (int u = 0; u < S; ++u) {
+    const int b = 4 * u + g;
+    xv[u] = (live && b < rows) ? xp[(int64_t)b * in_f] : 0.f;
   }
-  skinny_stage_dy<NQ, SKINNY_DW_WAVES * 64>(dyl, dy, rows, out_f);
-  __syncthreads();
-  f4v wr[DX ? NQ : 1];
-  if constexpr (DX) {
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const float v = wrows[lane * out_f + (q * 4 + k < out_f ? q * 4 + k : 0)];
-        wr[q][k] = q * 4 + k < out_f ? v : 0.f;
-      }
-    }
+  for (int u = 0; u < S; ++u) {
+    const int b = 4 * u + g;
+    dv[u] = (unit && b < rows) ? dyp[(int64_t)b * out_f] : 0.f;
   }
-  if constexpr (DX) {  // while the first rows of X are on their way
-    if (live) {
-      float* o = dx + i;
-#pragma unroll 4
-      for (int b = b0; b < b1; ++b) {
-        float s = 0.f;
+  if constexpr (DX) {
+    const int nq = (out_f + 3) >> 2;
+    float wk[4];
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-          const f4v d = dyl[b * NQ + q];
+    for (int q = 0; q < 4; ++q) wk[q] = (live && 4 * q + g < out_f) ? w[(int64_t)feat * out_f + 4 * q + g] : 0.f;
+    for (int r0 = 0; r0 < rows; r0 += 16) {
+      f4v t = {0.f, 0.f, 0.f, 0.f};
+      const int row = r0 + c;
 #pragma unroll
-          for (int k = 0; k < 4; ++k) s = __builtin_fmaf(d[k], wr[q][k], s);
+      for (int q = 0; q < 4; ++q) {
+        if (q < nq) {
+          const float a = (row < rows && 4 * q + g < out_f) ? dy[(int64_t)row * out_f + 4 * q + g] : 0.f;
+          t = __builtin_amdgcn_mfma_f32_16x16x4f32(a, wk[q], t, 0, 0, 0);
         }
-        o[(int64_t)b * in_f] = s;
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int b = r0 + 4 * g + v;
+        if (live && b < rows) dx[(int64_t)b * in_f + feat] = t[v];
       }
     }
   }
-  f4v acc[NQ];
+  f4v acc = {0.f, 0.f, 0.f, 0.f};
+  float bsum = 0.f;
+  for (int s0 = 0; s0 < steps; s0 += S) {
+    if (s0 != 0) {
 #pragma unroll
-  for (int q = 0; q < NQ; ++q) acc[q] = f4v{0.f, 0.f, 0.f, 0.f};
-  for (int b = b0; b < b1; b += U) {
-    if (b != b0) {
-#pragma unroll
-      for (int u = 0; u < U; ++u) xv[u] = b + u < b1 ? xp[(int64_t)(b + u) * in_f] : 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int row = b + u < b1 ? b + u : rows;  // the all-zero row
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        const f4v d = dyl[row * NQ + q];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) acc[q][k] = __builtin_fmaf(xv[u], d[k], acc[q][k]);
+      for (int u = 0; u < S; ++u) {
+        const int b = 4 * (s0 + u) + g;
+        xv[u] = (live && b < rows) ? xp[(int64_t)b * in_f] : 0.f;
+        dv[u] = (unit && b < rows) ? dyp[(int64_t)b * out_f] : 0.f;
       }
     }
-  }
-  if (wave > 0) {
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) part[((wave - 1) * NQ + q) * 64 + lane] = acc[q];
-  }
-  __syncthreads();
-  if (wave == 0) {
-#pragma unroll
-    for (int w = 0; w < SKINNY_DW_WAVES - 1; ++w) {
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        const f4v p = part[(w * NQ + q) * 64 + lane];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) acc[q][k] = acc[q][k] + p[k];
-      }
+    for (int u = 0; u < S; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u], dv[u], acc, 0, 0, 0);
+      bsum += dv[u];
     }
-    // (every wavefront has read its rows of W long before: the block-wide barrier above lies in between)
+  }
 #pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-#pragma unroll
-      for (int k = 0; k < 4; ++k)
-        if (q * 4 + k < out_f) wrows[lane * out_f + q * 4 + k] = acc[q][k];
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    for (int f = lane; f < 64 * out_f; f += 64)
-      if (run0 + f < run_end) dw[run0 + f] = wrows[f];
-  } else if (wave == 1 && blockIdx.x == 0 && db && lane < out_f) {
-    const float* flat = reinterpret_cast<const float*>(dyl);
-    float s = 0.f;
-    for (int b = 0; b < rows; ++b) s += flat[b * NQ * 4 + lane];
-    db[lane] = s;
+  for (int v = 0; v < 4; ++v) {
+    const int f = i0 + 4 * g + v;
+    if (unit && f < in_f) dw[(int64_t)f * out_f + c] = acc[v];
+  }
+  if (db && blockIdx.x == 0 && wave == 0) {  // rows 4 s + g of unit c were this lane's: the four row groups meet by shuffles
+    const float s1 = __shfl(bsum, c + 16, 64), s2 = __shfl(bsum, c + 32, 64), s3 = __shfl(bsum, c + 48, 64);
+    if (g == 0 && unit) db[c] = ((bsum + s1) + s2) + s3;
   }
 }
 
 bool dense_skinny_shape(int rows, int in_f, int out_f) {
-  const int nq = (out_f + 3) / 4;
-  return rows >= 4 && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES && (int64_t)(rows + 1) * nq * 4 <= SKINNY_MAX_LDS_FLOATS;
+  return rows >= 4 && rows <= SKINNY_MAX_ROWS && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES;
 }
 
 int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f, const float* w,
                            float* dx) {
   SN_REQUIRE(dense_skinny_shape(rows, in_f, out_f), "dense_weight_gradient_rows: shape outside the kernel's range");
   SN_REQUIRE((w != nullptr) == (dx != nullptr), "dense_weight_gradient_rows: the input gradient needs the weights and a place to go");
-  const int nq = (out_f + 3) / 4, rows_per_wave = (int)ceil_div(rows, SKINNY_DW_WAVES);
   const unsigned blocks = (unsigned)ceil_div(in_f, 64);
-  const size_t lds = ((size_t)(rows + 1) * nq + (size_t)(SKINNY_DW_WAVES - 1) * nq * 64) * sizeof(f4v) + (size_t)64 * out_f * sizeof(float);
   LaunchScope scope(ctx, dx ? "dense_weight_and_input_gradient_rows" : "dense_weight_gradient_rows", in_f, out_f, rows);
-#define SN_SKINNY_DW(NQ)                                                                                                                     \
-  do {                                                                                                                                       \
-    if (dx)                                                                                                                                  \
-      hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ, true>), dim3(blocks), dim3(SKINNY_DW_WAVES * 64), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f,    \
-                         rows_per_wave, w, dx);                                                                                              \
-    else                                                                                                                                     \
-      hipLaunchKernelGGL((dense_skinny_dw_kernel<NQ, false>), dim3(blocks), dim3(SKINNY_DW_WAVES * 64), lds, ctx->stream, x, dy, dw, db, rows, in_f, out_f,   \
-                         rows_per_wave, w, dx);                                                                                              \
-  } while (0)
-  switch (nq) {
-    case 1: SN_SKINNY_DW(1); break;
-    case 2: SN_SKINNY_DW(2); break;
-    case 3: SN_SKINNY_DW(3); break;
-    default: SN_SKINNY_DW(4); break;
-  }
-#undef SN_SKINNY_DW
+  if (dx)
+    hipLaunchKernelGGL((dense_skinny_grad_mfma_kernel<true>), dim3(blocks), dim3(256), 0, ctx->stream, x, dy, dw, db, rows, in_f, out_f, w, dx);
+  else
+    hipLaunchKernelGGL((dense_skinny_grad_mfma_kernel<false>), dim3(blocks), dim3(256), 0, ctx->stream, x, dy, dw, db, rows, in_f, out_f, w, dx);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }

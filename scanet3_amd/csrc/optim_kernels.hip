@@ -259,16 +259,25 @@ __global__ __launch_bounds__(256) void finish_kernel(float* __restrict__ w, floa
     const int64_t total4 = r.outs / 4;
     const int q = threadIdx.x >> 5, j = threadIdx.x & 31;
     const int64_t i = (int64_t)lb * 32 + j;
+    const int64_t e = flat0 + i * 4;
+    // the parameters and their optimizer state are requested first: they are back by the time the sums are made
+    f4 vw = {0.f, 0.f, 0.f, 0.f}, a = {0.f, 0.f, 0.f, 0.f}, bb = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+    if (q == 0 && i < total4 && !skip) {
+      vw = *(const f4*)(w + e);
+      a = *(const f4*)(s0 + e);
+      if (NS > 1) bb = *(const f4*)(s1 + e);
+      if (NS > 2) c = *(const f4*)(s2 + e);
+    }
     f4 s = {0.f, 0.f, 0.f, 0.f};
     if (i < total4) {
       const f4* w4 = reinterpret_cast<const f4*>(r.partial) + i;
       int z = q;
       for (; z + 56 < r.parts; z += 64) {  // 8 loads of 16 bytes in flight, added in split order
-        f4 a[8];
+        f4 pv[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) a[u] = w4[(int64_t)(z + 8 * u) * total4];
+        for (int u = 0; u < 8; ++u) pv[u] = w4[(int64_t)(z + 8 * u) * total4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += a[u];
+        for (int u = 0; u < 8; ++u) s += pv[u];
       }
       for (; z < r.parts; z += 8) s += w4[(int64_t)z * total4];
     }
@@ -276,12 +285,8 @@ __global__ __launch_bounds__(256) void finish_kernel(float* __restrict__ w, floa
     __syncthreads();
     if (q == 0 && i < total4) {
       const f4 t = ((part4[0][j] + part4[1][j]) + (part4[2][j] + part4[3][j])) + ((part4[4][j] + part4[5][j]) + (part4[6][j] + part4[7][j]));
-      const int64_t e = flat0 + i * 4;
       *(f4*)(g + e) = t;
       if (!skip) {
-        f4 vw = *(const f4*)(w + e), a = *(const f4*)(s0 + e), bb = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
-        if (NS > 1) bb = *(const f4*)(s1 + e);
-        if (NS > 2) c = *(const f4*)(s2 + e);
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
           float ww = vw[x], aa = a[x], b2 = bb[x], cc = c[x];
@@ -298,26 +303,33 @@ __global__ __launch_bounds__(256) void finish_kernel(float* __restrict__ w, floa
     // gemm_small_reduce_kernel's order: a block owns 4 outputs, 64 lanes each walk every 64th partial
     const int ol = threadIdx.x & 3, pl = threadIdx.x >> 2;
     const int o = lb * 4 + ol;
+    const int64_t e = flat0 + o;
+    // the parameter and its optimizer state are requested first: they are back by the time the sum is made
+    const bool updates = threadIdx.x < 4 && o < r.outs;
+    float ww = 0.f, aa = 0.f, b2 = 0.f, cc = 0.f;
+    if (updates && !skip) {
+      ww = w[e]; aa = s0[e];
+      if (NS > 1) b2 = s1[e];
+      if (NS > 2) cc = s2[e];
+    }
     float s = 0.f;
     if (o < r.outs) {
-      for (int i = pl; i < r.parts; i += 64 * 8) {  // 8 loads in flight, added in part order
-        float v[8];
+      for (int i = pl; i < r.parts; i += 64 * 16) {  // 16 loads in flight, added in part order
+        float v[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = i + 64 * u < r.parts ? r.partial[(int64_t)(i + 64 * u) * r.outs + o] : 0.f;
+        for (int u = 0; u < 16; ++u) v[u] = i + 64 * u < r.parts ? r.partial[(int64_t)(i + 64 * u) * r.outs + o] : 0.f;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
+        for (int u = 0; u < 16; ++u) s += v[u];
       }
     }
     part1[pl][ol] = s;
     __syncthreads();
-    if (threadIdx.x < 4 && o < r.outs) {
+    if (updates) {
       float t = 0.f;
 #pragma unroll 8
       for (int j = 0; j < 64; ++j) t += part1[j][ol];
-      const int64_t e = flat0 + o;
       g[e] = t;
       if (!skip) {
-        float ww = w[e], aa = s0[e], b2 = NS > 1 ? s1[e] : 0.f, cc = NS > 2 ? s2[e] : 0.f;
         update_one<KIND>(ww, t, aa, b2, cc, p);
         w[e] = ww; s0[e] = aa;
         if (NS > 1) s1[e] = b2;
