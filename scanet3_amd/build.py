@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libscanet_hip.so")
 
-SOURCES = ["runtime.hip", "optim_kernels.hip", "elementwise_kernels.hip", "batchnorm_kernels.hip", "random_kernels.hip", "gemm_kernels.hip", "conv_ring_kernels.hip", "gemm_bf16.hip", "lstm_kernels.hip", "lstm_wgrad_kernels.hip", "mlp2_kernels.hip", "model.hip"]
+SOURCES = ["runtime.hip", "optim_kernels.hip", "elementwise_kernels.hip", "batchnorm_kernels.hip", "random_kernels.hip", "gemm_kernels.hip", "conv_ring_kernels.hip", "conv_wgrad_kernels.hip", "gemm_bf16.hip", "lstm_kernels.hip", "lstm_wgrad_kernels.hip", "mlp2_kernels.hip", "model.hip"]
 
 # -ffp-contract=off: one rounding per reference op (TensorFlow evaluates Mul and Add separately).
 # -packed-fp32-ops is switched off: some packed fp32 forms have produced wrong values on this hardware.

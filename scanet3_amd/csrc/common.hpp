@@ -366,6 +366,11 @@ struct ConvGeom {
   int ho, wo, cout;      // output
   int kh, kw, sh, sw, pt, pl;
 };
+// Conv2D filter gradient of a layer with 32 input channels, 32 or 64 filters and no padding as one matrix-core tile per
+// filter tap: `*parts` partial filters [part][kh*kw*cin*cout] are left in ws for the caller to add in part order.
+bool conv_wgrad_taps_shape(const sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy);
+int64_t conv_wgrad_taps_workspace(const sn_ctx* ctx, const ConvGeom& g);  // floats of workspace
+int launch_conv_wgrad_taps(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* ws, int64_t ws_elems, int* parts);
 int launch_conv_fwd(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* w, const Epilogue& ep, float* ws, int64_t ws_elems);
 int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const float* w, float* dx, float* ws, int64_t ws_elems);
 // A 2 x 2 max pooling right above a first-layer convolution, for launch_conv_wgrad's direct kernel: the pooling's output

@@ -1696,6 +1696,26 @@ int launch_conv_wgrad(sn_ctx* ctx, const ConvGeom& g, const float* x, const floa
   int rc = SN_OK;
   if (conv_wgrad_direct(ctx, g, x, dy, dw, ws, ws_elems, &rc, pool)) return rc;
   SN_REQUIRE(pool == nullptr, "conv2d_filter_gradient: only the direct kernel takes a pooling's gradient (ask conv_wgrad_is_direct first)");
+  if (ws && aligned16(ws) && conv_wgrad_taps_shape(ctx, g, x, dy) && conv_wgrad_taps_workspace(ctx, g) <= ws_elems) {
+    // a tile per filter tap: a few dozen partial filters instead of the 64 x 64 tiling's hundreds
+    int parts = 0;
+    SN_TRY(launch_conv_wgrad_taps(ctx, g, x, dy, ws, ws_elems, &parts));
+    const int64_t total = (int64_t)M * N;  // a multiple of 1024
+    if (ctx->defer && total >= 4096) {  // a caller that applies the optimizer next takes the sum into that launch
+      *ctx->defer = DeferredReduce{1, ws, parts, (int)total, dw};
+      ctx->defer = nullptr;
+      return SN_OK;
+    }
+    Epilogue e;
+    e.out = dw;
+    e.ldo = g.cout;
+    StdEpilogue ep{e};
+    LaunchScope scope(ctx, "splitk_reduce");
+    const int64_t blocks = std::min<int64_t>(ceil_div(total / 4, 32), (int64_t)ctx->compute_units * 16);
+    hipLaunchKernelGGL((splitk_reduce4_kernel<StdEpilogue>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, (const float*)ws, parts, M, N, ep);
+    SN_HIP(hipGetLastError());
+    return SN_OK;
+  }
   if (!(ws && small_parts(M, N, K, ctx->compute_units, ws_elems)) && WgradXLoader::ok(x, g) && FlatLoader<false>::ok(dy, 1, g.cout, N, K)) {
     const int interior = g.pt == 0 && g.pl == 0 && (g.ho - 1) * g.sh + g.kh <= g.h && (g.wo - 1) * g.sw + g.kw <= g.w;
     WgradXLoader al{x, g, M, interior};

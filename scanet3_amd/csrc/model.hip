@@ -250,6 +250,10 @@ static int build_plan(sn_model* m, const sn_layer_desc* layers, int n_layers) {
         ws = std::max(ws, gemm_workspace_elems(B * ho * wo, L.units, (int)K, cu));
         ws = std::max(ws, gemm_workspace_elems((int)K, L.units, B * ho * wo, cu));
         ws = std::max(ws, gemm_workspace_elems(B * (int)cur[0] * (int)cur[1], (int)cur[2], op.kh * op.kw * L.units, cu));
+        {
+          const ConvGeom cg{B, (int)cur[0], (int)cur[1], (int)cur[2], (int)ho, (int)wo, L.units, op.kh, op.kw, op.sh, op.sw, op.pt, op.pl};
+          if (cg.cin == 32) ws = std::max(ws, conv_wgrad_taps_workspace(m->ctx, cg));  // the filter gradient's tile-per-tap form
+        }
         break;
       }
       case SN_LAYER_POOL2D: {

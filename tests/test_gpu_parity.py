@@ -475,6 +475,15 @@ MODELS = {
                                     ("flatten",), ("dense", 3, "softmax")], "cce", (14, 13, 1), 80, "uniform_onehot"),
     "conv_rows_64_channels_5x3": ([("conv", 64, (3, 3), (1, 1), "valid", "tanh", False), ("conv", 32, (5, 3), (1, 2), "same", "relu", False),
                                    ("flatten",), ("dense", 3, "softmax")], "cce", (12, 12, 1), 90, "uniform_onehot"),
+    # filter gradient of a layer with 32 input channels and no padding as one matrix-core tile per tap (needs a few hundred output
+    # rows and 8192+ positions): 64 filters over an odd row length, 32 filters with a bias under a 2 x 3 kernel at stride (2, 1)
+    # and an even row length, and stride 2 along the row
+    "conv_taps_3x3_64_filters_odd_rows": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 64, (3, 3), (1, 1), "valid", "relu", False),
+                                           ("flatten",), ("dense", 3, "softmax")], "cce", (14, 13, 1), 100, "uniform_onehot"),
+    "conv_taps_2x3_32_filters_stride_bias": ([("conv", 32, (2, 2), (1, 1), "valid", "tanh", False), ("conv", 32, (2, 3), (2, 1), "valid", "identity", True),
+                                              ("flatten",), ("dense", 3, "softmax")], "cce", (16, 13, 2), 120, "uniform_onehot"),
+    "conv_taps_row_stride_2": ([("conv", 32, (3, 3), (1, 1), "valid", "tanh", False), ("conv", 64, (3, 3), (1, 2), "valid", "relu", False),
+                                ("flatten",), ("dense", 3, "softmax")], "cce", (12, 23, 1), 110, "uniform_onehot"),
     # Dense from thousands of features onto a few units: gradients as row streams (2048+ features, at most 16 units); a feature count
     # that leaves a partial block of 64, 7 rows over 4 wavefronts, 16 and 5 units, an L2 penalty on the streamed weights
     "dense_many_features_few_units": ([("dense", 2050, "tanh"), ("dense", 5, "softmax", "l2", 0.01)], "cce", (33,), 7, "normal_onehot"),
