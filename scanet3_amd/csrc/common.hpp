@@ -178,8 +178,10 @@ int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp
                 int rows, int cols);
 // training step of a Softmax output under CategoricalCrossentropy: p, loss value and dz in one kernel per row
 // (row_loss: `rows` floats of scratch; loss_dev == nullptr: the loss value is not wanted, its final reduction is skipped)
+// dz_bf (optional): bf16 [rows, cols], the same dz rounded to bf16 (what a bf16 Dense layer below would cast it to next)
+// p may be null when nobody reads the probabilities and cols <= 1024 (rows held in registers)
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
-                       int cols, bool stable);
+                       int cols, bool stable, void* dz_bf = nullptr);
 // The same when the logits still lie as `parts` partial sums [part][rows * cols] of a Dense layer's forward product (at most
 // SOFTMAX_PARTIALS_MAX_COLS columns): the kernel adds them in the order of that product's own reduction, adds the bias
 // (may be null), writes the logits to z_out and goes on as launch_softmax_cce.

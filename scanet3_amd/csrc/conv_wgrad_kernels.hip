@@ -298,9 +298,10 @@ bool conv_wgrad_taps_shape(const sn_ctx* ctx, const ConvGeom& g, const float* x,
   const int64_t x_bytes = (int64_t)g.n * g.h * g.w * g.cin * 4, dy_bytes = (int64_t)g.n * g.ho * g.wo * g.cout * 4;
   if (x_bytes >= ((int64_t)1 << 31) || dy_bytes >= ((int64_t)1 << 31)) return false;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 3u) return false;
+  if ((int64_t)g.n * g.ho * g.wo < 8192) return false;  // too few positions for partial results to be worth their sum
+  if (rowtap_shape(ctx, g)) return true;
   const int per = tap_ranges_per_xcd(ctx, g);
-  // enough rows for every wavefront of every range, and enough positions for the partial results to be worth their sum
-  return per >= 1 && (int64_t)g.n * g.ho >= (int64_t)per * 8 * 4 * 2 && (int64_t)g.n * g.ho * g.wo >= 8192;
+  return per >= 1 && (int64_t)g.n * g.ho >= (int64_t)per * 8 * 4 * 2;  // rows for every wavefront of every range
 }
 
 int64_t conv_wgrad_taps_workspace(const sn_ctx* ctx, const ConvGeom& g) {

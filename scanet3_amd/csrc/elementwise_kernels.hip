@@ -252,7 +252,7 @@ int launch_loss(sn_ctx* ctx, int kind, const float* p, const float* y, float* dp
 // loss_stage1_kernel and softmax_bwd_kernel compute one after the other, without the dp round trip.
 __global__ __launch_bounds__(256) void softmax_cce_kernel(const float* __restrict__ z, const float* __restrict__ y, float* __restrict__ p,
                                                            float* __restrict__ dz, float* __restrict__ row_loss, int cols, int stable,
-                                                           float neg_inv_rows) {
+                                                           float neg_inv_rows, __bf16* __restrict__ dz_bf) {
   __shared__ float smem[4];
   const int64_t base = (int64_t)blockIdx.x * cols;
   const float eps = 1e-8f;
@@ -281,7 +281,9 @@ __global__ __launch_bounds__(256) void softmax_cce_kernel(const float* __restric
   for (int c = threadIdx.x; c < cols; c += blockDim.x) {
     const float pi = p[base + c];
     const float dpi = (y[base + c] * neg_inv_rows) / (pi + eps);
-    dz[base + c] = pi * dpi - pi * row_dot;
+    const float d = pi * dpi - pi * row_dot;
+    dz[base + c] = d;
+    if (dz_bf) dz_bf[base + c] = (__bf16)d;
   }
   if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
 }
@@ -291,7 +293,7 @@ __global__ __launch_bounds__(256) void softmax_cce_kernel(const float* __restric
 template <int E>
 __global__ __launch_bounds__(256) void softmax_cce_reg_kernel(const float* __restrict__ z, const float* __restrict__ y, float* __restrict__ p,
                                                                float* __restrict__ dz, float* __restrict__ row_loss, int cols, int stable,
-                                                               float neg_inv_rows) {
+                                                               float neg_inv_rows, __bf16* __restrict__ dz_bf) {
   __shared__ float smem[4];
   const int64_t base = (int64_t)blockIdx.x * cols;
   const float eps = 1e-8f;
@@ -337,8 +339,10 @@ __global__ __launch_bounds__(256) void softmax_cce_reg_kernel(const float* __res
     if (c < cols) {
       const float pi = zv[k];
       const float dpi = (yv[k] * neg_inv_rows) / (pi + eps);
-      p[base + c] = pi;
-      dz[base + c] = pi * dpi - pi * row_dot;
+      const float d = pi * dpi - pi * row_dot;
+      if (p) p[base + c] = pi;
+      dz[base + c] = d;
+      if (dz_bf) dz_bf[base + c] = (__bf16)d;
     }
   }
   if (threadIdx.x == 0) row_loss[blockIdx.x] = row_term;
@@ -403,7 +407,7 @@ __global__ __launch_bounds__(1024) void softmax_cce_partials_kernel(const float*
   if (live) {
     const float pi = zv;
     const float dpi = (yv * neg_inv_rows) / (pi + eps);
-    p[base + c] = pi;
+    if (p) p[base + c] = pi;
     dz[base + c] = pi * dpi - pi * row_dot;
   }
   if (c == 0) row_loss[blockIdx.x] = row_term;
@@ -428,19 +432,22 @@ int launch_softmax_cce_partials(sn_ctx* ctx, const float* partial, int parts, co
 }
 
 int launch_softmax_cce(sn_ctx* ctx, const float* z, const float* y, float* p, float* dz, float* loss_dev, float* row_loss, int rows,
-                       int cols, bool stable) {
+                       int cols, bool stable, void* dz_bf) {
   SN_REQUIRE(rows > 0 && cols > 0, "loss over an empty batch");
   {
     LaunchScope scope(ctx, "softmax_crossentropy_fused");
     const int threads = cols <= 64 ? 64 : 256;
     const float neg_inv_rows = -(1.0f / (float)rows);
+    SN_REQUIRE(p || cols <= 4 * threads, "softmax_crossentropy_fused: rows of %d values need the probabilities' buffer", cols);
 #define SN_SOFTMAX_CCE_REG(E) \
-  hipLaunchKernelGGL((softmax_cce_reg_kernel<E>), dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows)
+  hipLaunchKernelGGL((softmax_cce_reg_kernel<E>), dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows, \
+                     (__bf16*)dz_bf)
     if (cols <= threads) SN_SOFTMAX_CCE_REG(1);
     else if (cols <= 2 * threads) SN_SOFTMAX_CCE_REG(2);
     else if (cols <= 4 * threads) SN_SOFTMAX_CCE_REG(4);
     else
-      hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows);
+      hipLaunchKernelGGL(softmax_cce_kernel, dim3(rows), dim3(threads), 0, ctx->stream, z, y, p, dz, row_loss, cols, stable ? 1 : 0, neg_inv_rows,
+                         (__bf16*)dz_bf);
 #undef SN_SOFTMAX_CCE_REG
   }
   if (loss_dev) {

@@ -739,7 +739,8 @@ static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, f
 
 // ---------------------------------------------------------------------------- backward
 // Starts at op `first` (the last op by default) whose output gradient lies in grad_buf[cur].
-static int backward(sn_replica* r, const float* x, int rows, int first = -1, int cur = 0) {
+// first_dz_cast: the loss kernel has already left the bf16 copy of op `first`'s output gradient in bf_dz[first]
+static int backward(sn_replica* r, const float* x, int rows, int first = -1, int cur = 0, bool first_dz_cast = false) {
   sn_model* m = r->model;
   sn_ctx* ctx = r->ctx;
   const bool bf16 = (m->flags & SN_FLAG_GEMM_BF16) != 0;
@@ -761,13 +762,16 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
           // one pass: dZ = act'(Y) * dY as bf16 (the fp32 dZ itself is not kept: its only other reader would be the bias
           // gradient, summed here per 64-row block from the fp32 values)
           const bool y_from_bf = hidden_bf16_only(r, (size_t)i, rows);
-          if (!dz_handed_over)
+          const bool cast_by_loss = first_dz_cast && i == first;  // (an identity activation: dZ = dY; its column sums come from the fp32 dY)
+          if (cast_by_loss) {
+            if (op.b >= 0) SN_TRY(launch_col_sum(ctx, dy, out_f, param_ptr(r, r->g, op.b), rows, out_f, r->ws, m->workspace_elems));
+          } else if (!dz_handed_over)
             SN_TRY(launch_cast_bf16(ctx, dy, out_f, rows, out_f, r->bf_dz[i],
                                     op.act != SN_ACT_IDENTITY && !y_from_bf ? r->act[i] : nullptr, op.act, op.act_param, nullptr,
                                     op.b >= 0 ? r->bf_colp : nullptr,
                                     op.act != SN_ACT_IDENTITY && y_from_bf ? r->bf_x[i + 1] : nullptr));
           dz_handed_over = false;
-          if (op.b >= 0)
+          if (op.b >= 0 && !cast_by_loss)
             SN_TRY(launch_col_sum(ctx, r->bf_colp, out_f, param_ptr(r, r->g, op.b), ceil_div(rows, 64), out_f, r->ws, m->workspace_elems));
           EpilogueBf16 ew;
           ew.e.out = param_ptr(r, r->g, op.w); ew.e.ldo = out_f;
@@ -1108,6 +1112,7 @@ static int grad_pass_body(sn_replica* r, const float* x, const float* y, int row
   }
   if (last >= 1 && m->ops[last].kind == OP_SOFTMAX && m->loss == SN_LOSS_CATEGORICAL_CROSSENTROPY) {
     // Softmax output under CategoricalCrossentropy: probabilities, loss and d loss / d logits in one kernel
+    bool cast_by_loss = false;
     r->logit_parts = 0;
     r->leave_logit_parts = m->ops[last - 1].kind == OP_DENSE;
     const int rc = forward(r, x, rows, true, true);
@@ -1115,15 +1120,21 @@ static int grad_pass_body(sn_replica* r, const float* x, const float* y, int row
     SN_TRY(rc);
     if (r->logit_parts > 0) {
       const Op& d = m->ops[last - 1];
-      SN_TRY(launch_softmax_cce_partials(r->ctx, r->ws, r->logit_parts, param_ptr(r, r->w, d.b), r->act[last - 1], y, r->act[last], r->grad_buf[1],
+      SN_TRY(launch_softmax_cce_partials(r->ctx, r->ws, r->logit_parts, param_ptr(r, r->w, d.b), r->act[last - 1], y, nullptr, r->grad_buf[1],
                                          want_loss ? r->loss_dev : nullptr, r->loss_partials, rows, (int)m->ops[last].out_elems,
                                          (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
     } else {
-      SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, r->act[last], r->grad_buf[1], want_loss ? r->loss_dev : nullptr,
-                                r->loss_partials, rows, (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0));
+      // a bf16 Dense layer without activation right below: the kernel also writes the bf16 copy of dZ that layer's products read
+      const Op& below = m->ops[last - 1];
+      cast_by_loss = below.kind == OP_DENSE && below.act == SN_ACT_IDENTITY && dense_bf16_fast(m, below) && rows % 8 == 0 && r->bf_dz[last - 1];
+      // (the probabilities have no reader in a gradient pass: rows that fit in registers do not store them)
+      SN_TRY(launch_softmax_cce(r->ctx, op_output(r, last - 1, x, rows), y, (int)m->ops[last].out_elems <= 1024 ? nullptr : r->act[last], r->grad_buf[1],
+                                want_loss ? r->loss_dev : nullptr,
+                                r->loss_partials, rows, (int)m->ops[last].out_elems, (m->flags & SN_FLAG_STABLE_SOFTMAX) != 0,
+                                cast_by_loss ? r->bf_dz[last - 1] : nullptr));
     }
     if (want_loss) SN_TRY(add_penalties(r, true));
-    return backward(r, x, rows, last - 1, 1);
+    return backward(r, x, rows, last - 1, 1, cast_by_loss);
   }
   SN_TRY(forward(r, x, rows, false, true));
   const float* pred = op_output(r, (int)r->model->ops.size() - 1, x, rows);

@@ -484,6 +484,15 @@ MODELS = {
                                               ("flatten",), ("dense", 3, "softmax")], "cce", (16, 13, 2), 120, "uniform_onehot"),
     "conv_taps_row_stride_2": ([("conv", 32, (3, 3), (1, 1), "valid", "tanh", False), ("conv", 64, (3, 3), (1, 2), "valid", "relu", False),
                                 ("flatten",), ("dense", 3, "softmax")], "cce", (12, 23, 1), 110, "uniform_onehot"),
+    # the same with the taps of a filter row in one workgroup (kernels up to 3 wide at unit stride along the row; needs
+    # 8 x 8 x 2 x 32 / kh output rows): 3 taps over an odd row length, 2 taps with 32 filters at stride 2 down the image over an even
+    # row length, 1 tap
+    "conv_tap_rows_3x3_64_filters": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 64, (3, 3), (1, 1), "valid", "tanh", False),
+                                      ("flatten",), ("dense", 3, "softmax")], "cce", (12, 11, 1), 160, "uniform_onehot"),
+    "conv_tap_rows_2x2_32_filters_stride": ([("conv", 32, (2, 2), (1, 1), "valid", "tanh", False), ("conv", 32, (2, 2), (2, 1), "valid", "relu", True),
+                                             ("flatten",), ("dense", 3, "softmax")], "cce", (17, 12, 1), 256, "uniform_onehot"),
+    "conv_tap_rows_3x1_64_filters": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 64, (3, 1), (1, 1), "valid", "identity", False),
+                                      ("flatten",), ("dense", 3, "softmax")], "cce", (12, 9, 1), 160, "uniform_onehot"),
     # Dense from thousands of features onto a few units: gradients as row streams (2048+ features, at most 16 units); a feature count
     # that leaves a partial block of 64, 7 rows over 4 wavefronts, 16 and 5 units, an L2 penalty on the streamed weights
     "dense_many_features_few_units": ([("dense", 2050, "tanh"), ("dense", 5, "softmax", "l2", 0.01)], "cce", (33,), 7, "normal_onehot"),
@@ -550,6 +559,42 @@ def test_forward_loss_and_gradients_match_oracle(S, ctx, name):
     # partial batch (the accuracy estimator feeds one): rows < batch must give the same per-row predictions
     rows = max(1, batch // 3)
     np.testing.assert_allclose(h.rep.forward(xb, rows), pred[:rows], rtol=1e-6, atol=1e-7)
+    h.close()
+
+
+# which launch a parity model above is there for: its gradient pass must contain a launch whose label starts with this
+KERNEL_OF_MODEL = {
+    "conv_tap_rows_3x3_64_filters": "conv2d_filter_gradient_tap_rows",
+    "conv_tap_rows_2x2_32_filters_stride": "conv2d_filter_gradient_tap_rows",
+    "conv_tap_rows_3x1_64_filters": "conv2d_filter_gradient_tap_rows",
+    "conv_taps_3x3_64_filters_odd_rows": "conv2d_filter_gradient_taps",
+    "conv_taps_2x3_32_filters_stride_bias": "conv2d_filter_gradient_taps",
+    "conv_taps_row_stride_2": "conv2d_filter_gradient_taps",
+    "conv_pool_first_layer_same_s1": "maxpool_backward_and_conv2d_filter_gradient_direct",
+    "conv_first_layer_uneven": "conv2d_filter_gradient_direct",
+    "dense_many_features_few_units": "dense_weight_and_input_gradient_rows",
+    "dense_many_features_16_units": "dense_weight_and_input_gradient_rows",
+    "dense_odd_feature_count_9_units": "small_output_reduce_softmax_crossentropy_fused",
+    "mlp_cfg1": "mlp2_",
+}
+
+
+@pytest.mark.parametrize("name", list(KERNEL_OF_MODEL))
+def test_parity_models_reach_the_kernels_they_are_named_for(S, ctx, name):
+    spec, loss, in_shape, batch, kind = MODELS[name]
+    rng = np.random.default_rng(3)
+    h = Harness(S, ctx, spec, loss, in_shape, batch)
+    out_dim = h.omodel.out_shape((batch,) + in_shape)[-1]
+    x, y = make_data(kind, rng, batch, in_shape, out_dim)
+    h.rep.set_params(glorot_params(h.omodel, (batch,) + in_shape, rng))
+    xb, yb = ctx.to_device(x), ctx.to_device(y)
+    ctx.profile_reset()
+    ctx.profile(True)
+    h.rep.grad(xb, yb)
+    ctx.sync()
+    ctx.profile(False)
+    labels = list(ctx.profile_report())
+    assert any(l.startswith(KERNEL_OF_MODEL[name]) for l in labels), labels
     h.close()
 
 
