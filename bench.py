@@ -305,27 +305,27 @@ MEASURED_TRAFFIC = {
     # for a plain copy of 400 MB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the summaries are under profiles/
     "conv2d_forward[52900x64x288]": (22.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[62500x32x576]": (22.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x52900]": (42.1e6, "gemm_kernels.hip", "30efc35fc3f57cefda7a62af3133e72495ea8d20"),
-    "gemm_bf16_256x256_bf16out[8192x4096x4096]": (474.9e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
-    "gemm_bf16_256x256[4096x4096x8192]": (491.1e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
+    "conv2d_filter_gradient_tap_rows[288x64x52900]": (28.2e6, "conv_wgrad_kernels.hip", "59eeff5824059f575e3fdc75dd99ac30a3a1a384"),
+    "gemm_bf16_256x256_bf16out[8192x4096x4096]": (474.8e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
+    "gemm_bf16_256x256[4096x4096x8192]": (494.7e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_256x256_handover[8192x4096x4096]": (486.2e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_256x256_handover[8192x4096x1000]": (187.9e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_128x128[4096x1000x8192]": (214.9e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_128x256[8192x1000x4096]": (171.4e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
-    "lstm_sequence_forward[32768x1024x288]": (249.9e6, "lstm_kernels.hip", "a4185c13417e2c3aa00b48e9ee68b94c3d12c124"),
-    "lstm_sequence_backward_and_weight_gradient[512x1024x34560]": (520.6e6, "lstm_kernels.hip", "a4185c13417e2c3aa00b48e9ee68b94c3d12c124"),
-    "rnn_sequence_forward[32768x256x288]": (74.8e6, "lstm_kernels.hip", "a4185c13417e2c3aa00b48e9ee68b94c3d12c124"),
-    "rnn_sequence_backward_and_weight_gradient[512x256x34560]": (116.8e6, "lstm_kernels.hip", "a4185c13417e2c3aa00b48e9ee68b94c3d12c124"),
+    "lstm_sequence_forward[32768x1024x288]": (249.9e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
+    "lstm_sequence_backward_and_weight_gradient[512x1024x34560]": (520.3e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
+    "rnn_sequence_forward[32768x256x288]": (74.8e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
+    "rnn_sequence_backward_and_weight_gradient[512x256x34560]": (116.8e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
     "conv2d_forward[121000x64x288]": (53.3e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
     "conv2d_input_gradient[169000x32x576]": (53.7e6, "conv_ring_kernels.hip", "32d315e7eae7c2a44ebcc35968efaa881bd1f71b"),
-    "conv2d_filter_gradient[288x64x121000]": (72.2e6, "gemm_kernels.hip", "30efc35fc3f57cefda7a62af3133e72495ea8d20"),
+    "conv2d_filter_gradient_tap_rows[288x64x121000]": (60.9e6, "conv_wgrad_kernels.hip", "59eeff5824059f575e3fdc75dd99ac30a3a1a384"),
     "mlp2_rows_forward_backward[1000x50x784]": (5.4e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),
     "mlp2_weight_gradients_and_optimizer[784x50x1000]": (9.8e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),
     "lstm_weight_gradient_rows[289x1024x32768]": (474.3e6, "lstm_wgrad_kernels.hip", "070ad64002f0fb967fbd759a0aabe0851ddfb7e3"),
     "lstm_weight_gradient_rows[289x256x32768]": (147.1e6, "lstm_wgrad_kernels.hip", "070ad64002f0fb967fbd759a0aabe0851ddfb7e3"),
-    "gradient_sums_and_optimizer": (36.5e6, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
-    "adam": (2.800e9, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
-    "average": (0.900e9, "optim_kernels.hip", "b466c420710f3e0c31a7335e17720b7a4dee11f8"),
+    "gradient_sums_and_optimizer": (23.6e6, "optim_kernels.hip", "6b4919f35f7d5a085e20f3257517e6a0a096a7b4"),
+    "adam": (2.800e9, "optim_kernels.hip", "6b4919f35f7d5a085e20f3257517e6a0a096a7b4"),
+    "average": (0.900e9, "optim_kernels.hip", "6b4919f35f7d5a085e20f3257517e6a0a096a7b4"),
 }
 
 
