@@ -144,13 +144,10 @@ __global__ __launch_bounds__(256) void conv_wgrad_taps_kernel(TapArgs a) {
 constexpr int ROWTAP_RING = 12;    // slots in flight per wavefront (4 loads each)
 constexpr int ROWTAP_WAVES = 8;
 constexpr int ROWTAP_PITCH = 33;
-constexpr size_t ROWTAP_LDS_BYTES = 96 * 1024;  // > half of the 160 KiB of a compute unit (the exchange itself needs 33 KiB)
 
 template <int KW, int NT>
 __global__ __launch_bounds__(ROWTAP_WAVES * 64) void conv_wgrad_tap_rows_kernel(TapArgs a) {
-  // one 32 x 32 tile per wavefront, in a request for more than half of a compute unit's LDS: the workgroups are sized to
-  // take a compute unit each, and a second one placed beside the first would halve the speed of both
-  extern __shared__ __attribute__((aligned(16))) float ex[];
+  __shared__ float ex[ROWTAP_WAVES * 32 * ROWTAP_PITCH];  // one 32 x 32 tile per wavefront
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // everything a row range depends on is scalar
   const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
@@ -324,26 +321,15 @@ int launch_conv_wgrad_taps(sn_ctx* ctx, const ConvGeom& g, const float* x, const
     a.ranges = a.ranges_per_xcd * 8;
     const unsigned blocks = (unsigned)(8 * a.ranges_per_xcd * g.kh);
     LaunchScope scope(ctx, "conv2d_filter_gradient_tap_rows", g.kh * g.kw * g.cin, g.cout, g.n * g.ho * g.wo);
-#define SN_ROWTAP_NT(KW, NT)                                                                                                   \
-  do {                                                                                                                         \
-    static bool raised = false; /* (the same answer for every device) */                                                       \
-    if (!raised) {                                                                                                             \
-      SN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_wgrad_tap_rows_kernel<KW, NT>),                           \
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)ROWTAP_LDS_BYTES));                          \
-      raised = true;                                                                                                           \
-    }                                                                                                                          \
-    hipLaunchKernelGGL((conv_wgrad_tap_rows_kernel<KW, NT>), dim3(blocks), dim3(ROWTAP_WAVES * 64), ROWTAP_LDS_BYTES, ctx->stream, a); \
-  } while (0)
-#define SN_ROWTAP(KW)                    \
-  do {                                   \
-    if (g.cout == 64) SN_ROWTAP_NT(KW, 2); \
-    else SN_ROWTAP_NT(KW, 1);            \
+#define SN_ROWTAP(KW)                                                                                                    \
+  do {                                                                                                                   \
+    if (g.cout == 64) hipLaunchKernelGGL((conv_wgrad_tap_rows_kernel<KW, 2>), dim3(blocks), dim3(ROWTAP_WAVES * 64), 0, ctx->stream, a); \
+    else hipLaunchKernelGGL((conv_wgrad_tap_rows_kernel<KW, 1>), dim3(blocks), dim3(ROWTAP_WAVES * 64), 0, ctx->stream, a);               \
   } while (0)
     if (g.kw == 3) SN_ROWTAP(3);
     else if (g.kw == 2) SN_ROWTAP(2);
     else SN_ROWTAP(1);
 #undef SN_ROWTAP
-#undef SN_ROWTAP_NT
     *parts = a.ranges;
     SN_HIP(hipGetLastError());
     return SN_OK;
