@@ -1821,21 +1821,25 @@ __global__ __launch_bounds__(256) void dense_skinny_grad_mfma_kernel(const float
   if (i0 >= in_f) return;
   const int feat = i0 + c;
   const bool live = feat < in_f;
-  const float* xp = x + (live ? feat : 0);
   const bool unit = c < out_f;
-  const float* dyp = dy + (unit ? c : 0);
+  // a lane's element of row b lies at the tensor's base (the same for all lanes) + a 32-bit byte offset: one register per
+  // address instead of two (the host has checked that the tensors are below 4 GiB)
+  const uint32_t xlane = (uint32_t)(live ? feat : 0) * 4u, dlane = (uint32_t)(unit ? c : 0) * 4u;
+  const uint32_t xrow = (uint32_t)in_f * 4u, drow = (uint32_t)out_f * 4u;
+  auto x_at = [&](int b) { return *(const float*)((const char*)x + (xlane + (uint32_t)b * xrow)); };
+  auto dy_at = [&](int b) { return *(const float*)((const char*)dy + (dlane + (uint32_t)b * drow)); };
   constexpr int S = 32;  // steps (of 4 rows) in flight
   const int steps = (rows + 3) >> 2;
   float xv[S], dv[S];
 #pragma unroll
   for (int u = 0; u < S; ++u) {
     const int b = 4 * u + g;
-    xv[u] = (live && b < rows) ? xp[(int64_t)b * in_f] : 0.f;
+    xv[u] = (live && b < rows) ? x_at(b) : 0.f;
   }
 #pragma unroll
   for (int u = 0; u < S; ++u) {
     const int b = 4 * u + g;
-    dv[u] = (unit && b < rows) ? dyp[(int64_t)b * out_f] : 0.f;
+    dv[u] = (unit && b < rows) ? dy_at(b) : 0.f;
   }
   if constexpr (DX) {
     const int nq = (out_f + 3) >> 2;
@@ -1855,7 +1859,7 @@ __global__ __launch_bounds__(256) void dense_skinny_grad_mfma_kernel(const float
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int b = r0 + 4 * g + v;
-        if (live && b < rows) dx[(int64_t)b * in_f + feat] = t[v];
+        if (live && b < rows) *(float*)((char*)dx + (xlane + (uint32_t)b * xrow)) = t[v];
       }
     }
   }
@@ -1866,8 +1870,8 @@ __global__ __launch_bounds__(256) void dense_skinny_grad_mfma_kernel(const float
 #pragma unroll
       for (int u = 0; u < S; ++u) {
         const int b = 4 * (s0 + u) + g;
-        xv[u] = (live && b < rows) ? xp[(int64_t)b * in_f] : 0.f;
-        dv[u] = (unit && b < rows) ? dyp[(int64_t)b * out_f] : 0.f;
+        xv[u] = (live && b < rows) ? x_at(b) : 0.f;
+        dv[u] = (unit && b < rows) ? dy_at(b) : 0.f;
       }
     }
 #pragma unroll
@@ -1888,7 +1892,8 @@ __global__ __launch_bounds__(256) void dense_skinny_grad_mfma_kernel(const float
 }
 
 bool dense_skinny_shape(int rows, int in_f, int out_f) {
-  return rows >= 4 && rows <= SKINNY_MAX_ROWS && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES;
+  return rows >= 4 && rows <= SKINNY_MAX_ROWS && out_f >= 1 && out_f <= SKINNY_MAX_UNITS && in_f >= SKINNY_MIN_FEATURES &&
+         (int64_t)rows * in_f < ((int64_t)1 << 30);
 }
 
 int launch_dense_skinny_dw(sn_ctx* ctx, const float* x, const float* dy, float* dw, float* db, int rows, int in_f, int out_f, const float* w,
