@@ -1,13 +1,14 @@
-// Conv2D filter gradient for 32 input channels as one fp32 matrix-core tile per filter tap (gfx950).
+// Conv2D filter gradient for 32 input channels as fp32 matrix-core tiles per filter tap (gfx950).
 //
 //   dW[r, q, ci, co] = sum over (b, oh, ow) of x[b, oh*sh + r, ow*sw + q, ci] * dy[b, oh, ow, co]
 //   (math/nn/AllKernels.scala:211-261: the filter's side of Conv2D's gradient), no padding.
 //
 // As a GEMM the product is [kh*kw*32] x [cout] over tens of thousands of positions: the output is tiny, so filling the
 // chip means many partial results.  Tiled 64 x 64 with a split of the positions, 256 partial filters leave and come back
-// for one result.  Here a workgroup owns ONE tap (a [32 channels] x [cout] tile) and a contiguous range of output rows
-// (b, oh); the taps of a range are neighbours in the grid, so a range's x and dy are read from memory once and from L2
-// by the other taps, and the number of partial filters is the number of ranges (a few dozen).
+// for one result.  Here a workgroup owns the [32 channels] x [cout] tiles of ONE tap (conv_wgrad_taps_kernel) or of the
+// up to three taps of one filter row (conv_wgrad_tap_rows_kernel, the form taken where it applies) and a contiguous range
+// of the output rows (b, oh); the workgroups of a range are neighbours on one XCD, so a range's x and dy are read from
+// memory once and from L2 by the other taps, and the number of partial filters is the number of ranges (a few dozen).
 //
 // Neither operand goes through LDS.  With the position as the k index both operands of v_mfma_f32_32x32x2_f32 are rows of
 // the tensors as they lie: lane l holds A[m = l % 32][k = l / 32] = x[position p + l / 32][channel l % 32] and
