@@ -363,6 +363,20 @@ bool gemm_bf16_full_tiles(const sn_ctx* ctx, int M, int N);
 int launch_cast_bf16(sn_ctx* ctx, const float* src, int64_t ld, int rows, int cols, void* out, const float* y, int act, float act_param,
                      float* dz, float* col_partials = nullptr, const void* y_bf = nullptr);
 
+// Division of an index below 2^31 by a divisor fixed for the launch, as a multiplication and a shift (the device has no
+// integer divider: a division by a run-time value is some twenty instructions, and these kernels take three per element).
+// d >= 1.  q = (hi32(x * mul) + x) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
+struct FastDiv {
+  uint32_t mul, shift, d;
+};
+static inline FastDiv fast_div(uint32_t d) {
+  uint32_t shift = 0;
+  while ((1ull << shift) < d) ++shift;
+  const uint64_t mul = ((1ull << 32) * ((1ull << shift) - d)) / d + 1;
+  return FastDiv{(uint32_t)mul, shift, d};
+}
+__device__ __forceinline__ uint32_t div_by(uint32_t x, const FastDiv& f) { return (__umulhi(x, f.mul) + x) >> f.shift; }
+
 struct ConvGeom {
   int n, h, w, cin;      // input
   int ho, wo, cout;      // output

@@ -704,19 +704,6 @@ __global__ __launch_bounds__(256) void pool_fwd_kernel(const float* __restrict__
   }
 }
 
-// Division of an index below 2^31 by a divisor fixed for the launch, as a multiplication and a shift (the device has no
-// integer divider: a division by a run-time value is some twenty instructions, and these kernels take three per element).
-// d >= 1.  q = (hi32(x * mul) + x) >> shift with shift = ceil(log2 d), mul = floor(2^32 (2^shift - d) / d) + 1.
-struct FastDiv {
-  uint32_t mul, shift, d;
-};
-static inline FastDiv fast_div(uint32_t d) {
-  uint32_t shift = 0;
-  while ((1ull << shift) < d) ++shift;
-  const uint64_t mul = ((1ull << 32) * ((1ull << shift) - d)) / d + 1;
-  return FastDiv{(uint32_t)mul, shift, d};
-}
-__device__ __forceinline__ uint32_t div_by(uint32_t x, const FastDiv& f) { return (__umulhi(x, f.mul) + x) >> f.shift; }
 
 // The same forward pass for 2x2 max windows, 4 channels per thread, 32-bit indices: the four window cells are requested
 // together (cells outside the input re-read the tensor's first element and never win), then compared in window order.

@@ -1503,21 +1503,25 @@ __device__ __forceinline__ float pool_grad_act_bwd(int act, float y, float dy, f
   }
 }
 
+// What the launch fixes and the device would otherwise divide out per thread: the LDS offset of tap m = (r, q, ci) from a
+// position's top-left input element (taps >= kh*kw*cin repeat tap 0), and the divisors of the index arithmetic.
+struct WgradDirectPlan {
+  int off[WGRAD_DIRECT_MAX_TAPS];
+  FastDiv by_cv, by_wo, by_row_elems, by_cin, by_cout;
+};
+
 template <int MT, bool POOL>  // MT: upper bound of kh*kw*cin
 __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ dy,
                                                                  float* __restrict__ partial, int rows_per_band, int bands_per_image,
-                                                                 int items, int lw, int cshift, int staged_full, PoolGrad pg) {
+                                                                 int items, int lw, int cshift, int staged_full, PoolGrad pg, WgradDirectPlan plan) {
   extern __shared__ float wg_lds[];
   const int tid = threadIdx.x;
   const int M = g.kh * g.kw * g.cin;
   const int row_elems = lw * g.cin;
-  int off[MT];  // LDS offset of tap m = (r, q, ci) from a position's top-left input element
+  int off[MT];
 #pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    const int mm = m < M ? m : 0;
-    const int ci = mm % g.cin, rq = mm / g.cin;
-    off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
-  }
+  for (int m = 0; m < MT; ++m) off[m] = plan.off[m];
+  const FastDiv by_cv = plan.by_cv, by_wo = plan.by_wo;
   float acc[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) acc[m] = 0.f;
@@ -1539,27 +1543,36 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
     float* dcv = wg_lds + staged_full + rows_per_band * g.wo;    // POOL: the band's output gradient [P][cout]
     __syncthreads();  // the previous item's readers are done with the staged rows
     for (int e = tid; e < staged; e += 256) {
-      const int row = e / row_elems, rem = e % row_elems;
-      const int iy = iy0 + row, ix = rem / g.cin - g.pl, ci = rem % g.cin;
+      const int row = (int)div_by((uint32_t)e, plan.by_row_elems), rem = e - row * row_elems;
+      const int px = (int)div_by((uint32_t)rem, plan.by_cin);
+      const int iy = iy0 + row, ix = px - g.pl, ci = rem - px * g.cin;
       wg_lds[e] = ((unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w) ? x[(((int64_t)b * g.h + iy) * g.w + ix) * g.cin + ci] : 0.f;
     }
-    for (int p = tid; p < P; p += 256) origin[p] = (p / g.wo) * g.sh * row_elems + (p % g.wo) * g.sw * g.cin;  // one division per position, not per lane
+    for (int p = tid; p < P; p += 256) {  // once per position, not per lane
+      const int prow = (int)div_by((uint32_t)p, by_wo);
+      origin[p] = prow * g.sh * row_elems + (p - prow * g.wo) * g.sw * g.cin;
+    }
     if constexpr (POOL) {
       // the band's output gradient [P][cout], four filters per thread: position (iy, ix) of the convolution's output = of the
       // pooling's input lies in the windows oh_lo + {0, 1} x ow_lo + {0, 1} (those that exist)
+      // (index arithmetic is what this phase costs: divisions by the launch's constants are multiplications, those by the
+      // pooling's stride shifts for strides 1 and 2, element offsets 32-bit)
       const int cv = g.cout >> 2;
+      auto by_stride = [](int v, int st) { return st == 1 ? v : (st == 2 ? v >> 1 : v / st); };  // v >= 0
+      const uint32_t img_y = (uint32_t)b * g.ho, img_p = (uint32_t)b * pg.ho;
       for (int e = tid; e < P * cv; e += 256) {
-        const int p = e / cv, ch = (e - p * cv) * 4;
-        const int iy = oh0 + p / g.wo, ix = p % g.wo;
+        const int p = (int)div_by((uint32_t)e, by_cv), ch = (e - p * cv) * 4;
+        const int prow = (int)div_by((uint32_t)p, by_wo);
+        const int iy = oh0 + prow, ix = p - prow * g.wo;
         int oh_lo = iy + pg.pt - 1;
-        oh_lo = oh_lo <= 0 ? 0 : (oh_lo + pg.sh - 1) / pg.sh;
-        int oh_hi = (iy + pg.pt) / pg.sh;
+        oh_lo = oh_lo <= 0 ? 0 : by_stride(oh_lo + pg.sh - 1, pg.sh);
+        int oh_hi = by_stride(iy + pg.pt, pg.sh);
         if (oh_hi > pg.ho - 1) oh_hi = pg.ho - 1;
         int ow_lo = ix + pg.pl - 1;
-        ow_lo = ow_lo <= 0 ? 0 : (ow_lo + pg.sw - 1) / pg.sw;
-        int ow_hi = (ix + pg.pl) / pg.sw;
+        ow_lo = ow_lo <= 0 ? 0 : by_stride(ow_lo + pg.sw - 1, pg.sw);
+        int ow_hi = by_stride(ix + pg.pl, pg.sw);
         if (ow_hi > pg.wo - 1) ow_hi = pg.wo - 1;
-        const f4v yv = *(const f4v*)(pg.y + ((((int64_t)b * g.ho + iy) * g.wo + ix) * g.cout + ch));
+        const f4v yv = *(const f4v*)(pg.y + (((img_y + iy) * g.wo + ix) * g.cout + ch));
         uint32_t a4[4], want[4];
         f4v gk[4];
         bool on[4];
@@ -1567,7 +1580,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
         for (int k = 0; k < 4; ++k) {  // windows that do not exist re-read the first element and are ignored
           const int oh = oh_lo + (k >> 1), ow = ow_lo + (k & 1);
           on[k] = oh <= oh_hi && ow <= ow_hi;
-          const int64_t o = on[k] ? (((int64_t)b * pg.ho + oh) * pg.wo + ow) * g.cout + ch : ch;
+          const uint32_t o = on[k] ? ((img_p + oh) * pg.wo + ow) * g.cout + ch : (uint32_t)ch;
           want[k] = (uint32_t)((iy - (oh * pg.sh - pg.pt)) * 2 + (ix - (ow * pg.sw - pg.pl)));
           a4[k] = *(const uint32_t*)(pg.arg + o);
           gk[k] = *(const f4v*)(pg.dy + o);
@@ -1616,7 +1629,7 @@ __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, cons
   __syncthreads();
   const int outs = M * g.cout;
   for (int o = tid; o < outs; o += 256) {
-    const int m = o / g.cout, co = o % g.cout;
+    const int m = (int)div_by((uint32_t)o, plan.by_cout), co = o - m * g.cout;
     float t = 0.f;
     for (int sl = 0; sl < slots; ++sl) t += wg_lds[(sl * M + m) * lanes + co];
     partial[(int64_t)blockIdx.x * outs + o] = t;
@@ -1636,7 +1649,7 @@ bool conv_wgrad_is_direct(const sn_ctx* ctx, const ConvGeom& g, const float* ws,
   const int bands = (int)ceil_div((int64_t)g.ho, (int64_t)rows_per_band);
   const int64_t staged = (int64_t)((rows_per_band - 1) * g.sh + g.kh) * lw * g.cin;
   const int64_t lds_floats = std::max<int64_t>(staged + (int64_t)rows_per_band * g.wo * (with_pool ? 1 + N : 1), (int64_t)256 * M);
-  return lds_floats * 4 <= 48 * 1024 && (int64_t)g.n * bands < (int64_t)1 << 30 && (!with_pool || N % 4 == 0);
+  return lds_floats * 4 <= 48 * 1024 && (int64_t)g.n * bands < (int64_t)1 << 30 && (!with_pool || (N % 4 == 0 && (int64_t)g.n * g.ho * g.wo * N < ((int64_t)1 << 32)));  // (32-bit element offsets there)
 }
 
 static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, const float* dy, float* dw, float* ws, int64_t ws_elems, int* rc,
@@ -1659,14 +1672,26 @@ static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, co
   {
     LaunchScope scope(ctx, pool ? "maxpool_backward_and_conv2d_filter_gradient_direct" : "conv2d_filter_gradient_direct", M, N, (int)K);
     const PoolGrad pg = pool ? *pool : PoolGrad{};
+    WgradDirectPlan plan;
+    const int row_elems = lw * g.cin;
+    for (int m = 0; m < WGRAD_DIRECT_MAX_TAPS; ++m) {
+      const int mm = m < M ? m : 0;
+      const int ci = mm % g.cin, rq = mm / g.cin;
+      plan.off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
+    }
+    plan.by_cv = fast_div((uint32_t)std::max(1, g.cout / 4));
+    plan.by_wo = fast_div((uint32_t)g.wo);
+    plan.by_row_elems = fast_div((uint32_t)row_elems);
+    plan.by_cin = fast_div((uint32_t)g.cin);
+    plan.by_cout = fast_div((uint32_t)g.cout);
 #define SN_WGRAD_DIRECT(MT)                                                                                                             \
   do {                                                                                                                                  \
     if (pool)                                                                                                                           \
       hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT, true>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float),    \
-                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg);                     \
+                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg, plan);               \
     else                                                                                                                                \
       hipLaunchKernelGGL((conv_wgrad_direct_kernel<MT, false>), dim3((unsigned)parts), dim3(256), (size_t)lds_floats * sizeof(float),   \
-                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg);                     \
+                         ctx->stream, g, x, dy, ws, rows_per_band, bands, (int)items, lw, cshift, (int)staged, pg, plan);               \
   } while (0)
     if (M <= 9) SN_WGRAD_DIRECT(9);
     else if (M <= 18) SN_WGRAD_DIRECT(18);
