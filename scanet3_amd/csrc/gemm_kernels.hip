@@ -1357,6 +1357,30 @@ __device__ __forceinline__ void fwd_rows_pixels(const float* lds, const int* ori
   for (int u = 0; u < U; ++u) *(f4v*)(outb + (int64_t)(p0 + u * slots) * e.ldo) = f4v{v[u * 4], v[u * 4 + 1], v[u * 4 + 2], v[u * 4 + 3]};
 }
 
+// What a launch of the two direct first-layer kernels below fixes and the device would otherwise divide out per thread
+// (the device has no integer divider): the LDS offset of tap m = (r, q, ci) from a position's top-left input element
+// (taps >= kh*kw*cin repeat tap 0), and the divisors of the index arithmetic.
+constexpr int WGRAD_DIRECT_MAX_TAPS = 36;
+struct DirectConvPlan {
+  int off[WGRAD_DIRECT_MAX_TAPS];
+  FastDiv by_cv, by_wo, by_row_elems, by_cin, by_cout;
+};
+static DirectConvPlan direct_conv_plan(const ConvGeom& g, int lw) {
+  DirectConvPlan plan;
+  const int M = g.kh * g.kw * g.cin, row_elems = lw * g.cin;
+  for (int m = 0; m < WGRAD_DIRECT_MAX_TAPS; ++m) {
+    const int mm = m < M ? m : 0;
+    const int ci = mm % g.cin, rq = mm / g.cin;
+    plan.off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
+  }
+  plan.by_cv = fast_div((uint32_t)std::max(1, g.cout / 4));
+  plan.by_wo = fast_div((uint32_t)g.wo);
+  plan.by_row_elems = fast_div((uint32_t)row_elems);
+  plan.by_cin = fast_div((uint32_t)g.cin);
+  plan.by_cout = fast_div((uint32_t)g.cout);
+  return plan;
+}
+
 // The same layer when the filter count is 4 << j (j = 0..6) and there are at most 18 taps: a workgroup takes a band of
 // output rows of one image and keeps the input rows under it in LDS, zero-padded; a lane owns 4 filters, holds their
 // weights for every tap in registers and walks pixels, so a pixel costs its taps' LDS reads (shared by the lanes of the
@@ -1365,7 +1389,7 @@ __device__ __forceinline__ void fwd_rows_pixels(const float* lds, const int* ori
 template <int MT>
 __global__ __launch_bounds__(256) void conv_direct_fwd_rows_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ w,
                                                                     Epilogue e, int rows_per_band, int bands_per_image, int items, int lw,
-                                                                    int qshift, int staged_full) {
+                                                                    int qshift, int staged_full, DirectConvPlan plan) {
   extern __shared__ float fw_lds[];
   const int tid = threadIdx.x;
   const int M = g.kh * g.kw * g.cin;
@@ -1377,9 +1401,7 @@ __global__ __launch_bounds__(256) void conv_direct_fwd_rows_kernel(ConvGeom g, c
   int off[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
-    const int mm = m < M ? m : 0;
-    const int ci = mm % g.cin, rq = mm / g.cin;
-    off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
+    off[m] = plan.off[m];
     const f4v zero = {0.f, 0.f, 0.f, 0.f};
     wr[m] = m < M ? *(const f4v*)(w + (int64_t)m * g.cout + col) : zero;
   }
@@ -1399,11 +1421,15 @@ __global__ __launch_bounds__(256) void conv_direct_fwd_rows_kernel(ConvGeom g, c
     const int P = (oh1 - oh0) * g.wo;
     __syncthreads();  // the previous item's readers are done with the staged rows
     for (int el = tid; el < staged; el += 256) {
-      const int row = el / row_elems, rem = el % row_elems;
-      const int iy = iy0 + row, ix = rem / g.cin - g.pl, ci = rem % g.cin;
+      const int row = (int)div_by((uint32_t)el, plan.by_row_elems), rem = el - row * row_elems;
+      const int px = (int)div_by((uint32_t)rem, plan.by_cin);
+      const int iy = iy0 + row, ix = px - g.pl, ci = rem - px * g.cin;
       fw_lds[el] = ((unsigned)iy < (unsigned)g.h && (unsigned)ix < (unsigned)g.w) ? x[(((int64_t)b * g.h + iy) * g.w + ix) * g.cin + ci] : 0.f;
     }
-    for (int p = tid; p < P; p += 256) origin[p] = (p / g.wo) * g.sh * row_elems + (p % g.wo) * g.sw * g.cin;
+    for (int p = tid; p < P; p += 256) {
+      const int prow = (int)div_by((uint32_t)p, plan.by_wo);
+      origin[p] = prow * g.sh * row_elems + (p - prow * g.wo) * g.sw * g.cin;
+    }
     __syncthreads();
     float* outb = e.out + (((int64_t)b * g.ho + oh0) * g.wo) * e.ldo + col;
     int p0 = slot;
@@ -1428,10 +1454,11 @@ static bool conv_fwd_rows(sn_ctx* ctx, const ConvGeom& g, const float* x, const 
   const int64_t lds_floats = staged + (int64_t)rows_per_band * g.wo;
   if (lds_floats * 4 > 48 * 1024 || items >= (int64_t)1 << 30) return false;
   const unsigned blocks = (unsigned)std::min<int64_t>(items, (int64_t)ctx->compute_units * 8);
+  const DirectConvPlan plan = direct_conv_plan(g, lw);
   LaunchScope scope(ctx, "conv2d_forward_direct", (int)pixels, N, K);
 #define SN_FWD_ROWS(MT)                                                                                                                  \
   hipLaunchKernelGGL((conv_direct_fwd_rows_kernel<MT>), dim3(blocks), dim3(256), (size_t)lds_floats * sizeof(float), ctx->stream, g, x, w, e, \
-                     rows_per_band, bands, (int)items, lw, qshift, (int)staged)
+                     rows_per_band, bands, (int)items, lw, qshift, (int)staged, plan)
   if (K <= 9) SN_FWD_ROWS(9);
   else SN_FWD_ROWS(18);
 #undef SN_FWD_ROWS
@@ -1487,7 +1514,6 @@ int launch_conv_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, const flo
 // (zero-padded, so taps need no bounds checks), a group of `1 << cshift` >= cout lanes owns one output position at a
 // time, each lane one filter, and keeps all M sums of that filter in registers.  The lanes' sums meet in LDS and
 // leave as one partial [M][cout] per workgroup; gemm_small_reduce_kernel adds the partials in a fixed order.
-constexpr int WGRAD_DIRECT_MAX_TAPS = 36;
 
 // POOL: the convolution's output gradient is not in memory yet.  A 2 x 2 max pooling sits right above the layer and the
 // kernel computes dy[position, filter] itself from the pooling's output gradient, the recorded first-maximum offsets and
@@ -1503,17 +1529,10 @@ __device__ __forceinline__ float pool_grad_act_bwd(int act, float y, float dy, f
   }
 }
 
-// What the launch fixes and the device would otherwise divide out per thread: the LDS offset of tap m = (r, q, ci) from a
-// position's top-left input element (taps >= kh*kw*cin repeat tap 0), and the divisors of the index arithmetic.
-struct WgradDirectPlan {
-  int off[WGRAD_DIRECT_MAX_TAPS];
-  FastDiv by_cv, by_wo, by_row_elems, by_cin, by_cout;
-};
-
 template <int MT, bool POOL>  // MT: upper bound of kh*kw*cin
 __global__ __launch_bounds__(256) void conv_wgrad_direct_kernel(ConvGeom g, const float* __restrict__ x, const float* __restrict__ dy,
                                                                  float* __restrict__ partial, int rows_per_band, int bands_per_image,
-                                                                 int items, int lw, int cshift, int staged_full, PoolGrad pg, WgradDirectPlan plan) {
+                                                                 int items, int lw, int cshift, int staged_full, PoolGrad pg, DirectConvPlan plan) {
   extern __shared__ float wg_lds[];
   const int tid = threadIdx.x;
   const int M = g.kh * g.kw * g.cin;
@@ -1672,18 +1691,7 @@ static bool conv_wgrad_direct(sn_ctx* ctx, const ConvGeom& g, const float* x, co
   {
     LaunchScope scope(ctx, pool ? "maxpool_backward_and_conv2d_filter_gradient_direct" : "conv2d_filter_gradient_direct", M, N, (int)K);
     const PoolGrad pg = pool ? *pool : PoolGrad{};
-    WgradDirectPlan plan;
-    const int row_elems = lw * g.cin;
-    for (int m = 0; m < WGRAD_DIRECT_MAX_TAPS; ++m) {
-      const int mm = m < M ? m : 0;
-      const int ci = mm % g.cin, rq = mm / g.cin;
-      plan.off[m] = (rq / g.kw) * row_elems + (rq % g.kw) * g.cin + ci;
-    }
-    plan.by_cv = fast_div((uint32_t)std::max(1, g.cout / 4));
-    plan.by_wo = fast_div((uint32_t)g.wo);
-    plan.by_row_elems = fast_div((uint32_t)row_elems);
-    plan.by_cin = fast_div((uint32_t)g.cin);
-    plan.by_cout = fast_div((uint32_t)g.cout);
+    const DirectConvPlan plan = direct_conv_plan(g, lw);
 #define SN_WGRAD_DIRECT(MT)                                                                                                             \
   do {                                                                                                                                  \
     if (pool)                                                                                                                           \
