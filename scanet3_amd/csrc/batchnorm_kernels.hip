@@ -182,8 +182,11 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(const float* __restrict__
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   if (V4) {
     const int64_t n4 = n / 4;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-      const int c = (int)((i * 4) % cols);
+    // the column walks with the index: one division at the start, then an addition and a wrap per trip
+    const int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int c = (int)((i0 * 4) % cols);
+    const int cstep = (int)((stride * 4) % cols);
+    for (int64_t i = i0; i < n4; i += stride, c = c + cstep >= cols ? c + cstep - cols : c + cstep) {
       const bn_f4 xv = *(const bn_f4*)(x + i * 4), iv = *(const bn_f4*)(inv + c), mv = *(const bn_f4*)(mean + c), bv = *(const bn_f4*)(beta + c);
       bn_f4 o;
 #pragma unroll
@@ -246,8 +249,10 @@ __global__ __launch_bounds__(256) void bn_dx_kernel(const float* __restrict__ x,
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   if (V4) {
     const int64_t n4 = n / 4;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-      const int c = (int)((i * 4) % cols);
+    const int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int c = (int)((i0 * 4) % cols);
+    const int cstep = (int)((stride * 4) % cols);
+    for (int64_t i = i0; i < n4; i += stride, c = c + cstep >= cols ? c + cstep - cols : c + cstep) {
       const bn_f4 xv = *(const bn_f4*)(x + i * 4), gv = *(const bn_f4*)(dy + i * 4), iv = *(const bn_f4*)(inv + c),
                   mv = *(const bn_f4*)(mean + c), a = *(const bn_f4*)(k1 + c), b = *(const bn_f4*)(k2 + c);
       bn_f4 o;
