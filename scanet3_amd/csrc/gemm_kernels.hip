@@ -987,10 +987,22 @@ __global__ __launch_bounds__(256) void splitk_reduce4_kernel(const float* __rest
     __syncthreads();
     if (g == 0 && i < total4) {
       const f4v t = ((part4[0][j] + part4[1][j]) + (part4[2][j] + part4[3][j])) + ((part4[4][j] + part4[5][j]) + (part4[6][j] + part4[7][j]));
+      // row and column of the first of the four outputs by one division (32-bit where the index allows: a 64-bit division
+      // is some hundred instructions on this device), the others by stepping
+      const int64_t o0 = i * 4;
+      int m, n;
+      if (o0 < ((int64_t)1 << 31)) {
+        const uint32_t q = (uint32_t)o0 / (uint32_t)N;
+        m = (int)q;
+        n = (int)((uint32_t)o0 - q * (uint32_t)N);
+      } else {
+        m = (int)(o0 / N);
+        n = (int)(o0 % N);
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int64_t o = i * 4 + e;
-        ep.store((int)(o / N), (int)(o % N), t[e]);
+        ep.store(m, n, t[e]);
+        if (++n == N) { n = 0; ++m; }
       }
     }
     __syncthreads();
