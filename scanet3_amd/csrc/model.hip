@@ -123,6 +123,11 @@ struct sn_replica {
   int64_t stage_group = 1;  // full batches a staging slot holds
   hipStream_t copy_stream = nullptr;
   hipEvent_t ev_filled[2] = {nullptr, nullptr}, ev_consumed[2] = {nullptr, nullptr};
+  // bf16 Dense models: a layer's optimizer launch runs on a second stream beside the gradient products of the layers
+  // below it (a stream of memory traffic beside matrix-core work)
+  hipStream_t update_stream = nullptr;
+  hipEvent_t ev_layer_ready = nullptr, ev_updates_done = nullptr;
+  bool side_updates = false;  // the running gradient pass updates each Dense layer as soon as its gradients are complete
   std::vector<void*> owned;
 };
 
@@ -738,6 +743,31 @@ static int loss_of(sn_replica* r, const float* pred, const float* y, int rows, f
 }
 
 // ---------------------------------------------------------------------------- backward
+// The optimizer update of one bf16 Dense layer, as soon as its gradients are complete.  With more layers to come
+// (`overlap`) the launch goes to the replica's second stream, behind an event that says the layer's products are done,
+// and runs beside the products of the layers below; the last layer's goes to the compute stream.  Same kernel, same
+// arithmetic as the one launch over the whole buffer: that one is a loop over elements, split here by layer.
+static int update_dense_layer(sn_replica* r, const Op& op, bool overlap) {
+  sn_model* m = r->model;
+  sn_ctx* ctx = r->ctx;
+  int64_t first = m->params[op.w].info.offset, end = first + m->params[op.w].info.size;
+  if (op.b >= 0) {
+    first = std::min<int64_t>(first, m->params[op.b].info.offset);
+    end = std::max<int64_t>(end, m->params[op.b].info.offset + m->params[op.b].info.size);
+  }
+  hipStream_t compute = ctx->stream;
+  if (overlap) {
+    SN_HIP(hipEventRecord(r->ev_layer_ready, compute));
+    SN_HIP(hipStreamWaitEvent(r->update_stream, r->ev_layer_ready, 0));
+    ctx->stream = r->update_stream;
+  }
+  const int rc = launch_optimizer(ctx, r->opt, r->w + first, r->g + first, r->s[0] + first, r->s[1] ? r->s[1] + first : nullptr,
+                                  r->s[2] ? r->s[2] + first : nullptr, end - first, r->pass_iter, r->bf_wflat ? r->bf_wflat + first : nullptr,
+                                  ctx->seq_failed_dev);
+  ctx->stream = compute;
+  return rc;
+}
+
 // Starts at op `first` (the last op by default) whose output gradient lies in grad_buf[cur].
 // first_dz_cast: the loss kernel has already left the bf16 copy of op `first`'s output gradient in bf_dz[first]
 static int backward(sn_replica* r, const float* x, int rows, int first = -1, int cur = 0, bool first_dz_cast = false) {
@@ -794,6 +824,7 @@ static int backward(sn_replica* r, const float* x, int rows, int first = -1, int
             SN_TRY(launch_gemm_bf16(ctx, GEMM_BF16_DX, r->bf_dz[i], out_f, r->bf_w[i], out_f, rows, in_f, out_f, ex));  // dX = dZ . W^T
             cur ^= 1;
           }
+          if (r->side_updates) SN_TRY(update_dense_layer(r, op, need_dx));  // (after dX: that product read the layer's bf16 weights)
           break;
         }
         if (!bf16 && r->ws && dense_tiny_shape(rows, in_f, out_f, m->workspace_elems)) {  // activation gradient, dX, dW and db in two launches
@@ -1066,6 +1097,40 @@ static bool mlp2_path(const sn_model* m) {
 // for_update: the optimizer update of the same step follows (update()), which may then take over reductions this pass
 // leaves open; without it (sn_grad) every gradient is complete when the pass returns.
 static int grad_pass_body(sn_replica* r, const float* x, const float* y, int rows, bool want_loss);
+// A training step of a model made of bf16 Dense layers only (and parameter-free ops), without penalties: every layer is
+// updated as soon as its gradients are complete, on a second stream, and update() has nothing left to launch.
+static int begin_side_updates(sn_replica* r, int rows, bool for_update) {
+  sn_model* m = r->model;
+  r->side_updates = false;
+  if (!for_update || !r->has_opt || !(m->flags & SN_FLAG_GEMM_BF16) || rows % 8 != 0 || m->trainable_runs.size() != 1) return SN_OK;
+  int dense = 0;
+  for (const Op& op : m->ops) {
+    if (op.kind == OP_DENSE) {
+      if (!dense_bf16_fast(m, op)) return SN_OK;
+      ++dense;
+    } else if (op.kind != OP_SOFTMAX && op.kind != OP_FLATTEN) {
+      return SN_OK;  // (layers with parameters or state of their own keep the one launch over the whole buffer)
+    }
+  }
+  if (dense < 2) return SN_OK;
+  for (const auto& p : m->params)
+    if (p.reg_kind != SN_REG_NONE) return SN_OK;
+  if (!r->update_stream) {
+    hipStream_t st = nullptr;
+    SN_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));  // (default priority, as the compute stream)
+    hipEvent_t a = nullptr, b = nullptr;
+    if (hipEventCreateWithFlags(&a, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&b, hipEventDisableTiming) != hipSuccess) {
+      if (a) (void)hipEventDestroy(a);
+      (void)hipStreamDestroy(st);
+      return fail(SN_E_HIP, "events for the update stream could not be created");
+    }
+    r->update_stream = st;
+    r->ev_layer_ready = a;
+    r->ev_updates_done = b;
+  }
+  r->side_updates = true;
+  return SN_OK;
+}
 // update_iter > 0: the optimizer update with that iteration number follows (update()), and may be taken over by this pass
 static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bool want_loss, int update_iter = 0) {
   const bool for_update = update_iter > 0;
@@ -1073,9 +1138,21 @@ static int grad_pass(sn_replica* r, const float* x, const float* y, int rows, bo
   r->updated_in_pass = false;
   r->pass_iter = update_iter;
   r->defer_now = for_update && r->fuse_finish;
-  const int rc = grad_pass_body(r, x, y, rows, want_loss);
+  SN_TRY(begin_side_updates(r, rows, for_update));
+  int rc = grad_pass_body(r, x, y, rows, want_loss);
   r->defer_now = false;
   if (rc != SN_OK) r->n_deferred = 0;
+  if (r->side_updates) {  // the compute stream goes on only after every layer's update (also after a failed pass: nothing is left running)
+    r->side_updates = false;
+    const hipError_t e1 = hipEventRecord(r->ev_updates_done, r->update_stream);
+    const hipError_t e2 = e1 == hipSuccess ? hipStreamWaitEvent(r->ctx->stream, r->ev_updates_done, 0) : e1;
+    if (e2 != hipSuccess) {
+      (void)hipStreamSynchronize(r->update_stream);
+      if (rc == SN_OK) rc = fail(SN_E_HIP, "joining the update stream failed: %s", hipGetErrorString(e2));
+    }
+    if (rc == SN_OK) r->updated_in_pass = true;
+    else r->bf_weights_stale = true;  // some layers may have moved: their bf16 copies are rebuilt from the fp32 weights
+  }
   r->pass_iter = update_iter;  // (kept for update()'s check)
   return rc;
 }
@@ -1355,6 +1432,12 @@ int sn_replica_destroy(sn_replica* rep) {
       (void)hipEventDestroy(rep->ev_consumed[i]);
     }
     (void)hipStreamDestroy(rep->copy_stream);
+  }
+  if (rep->update_stream) {
+    (void)hipStreamSynchronize(rep->update_stream);
+    (void)hipEventDestroy(rep->ev_layer_ready);
+    (void)hipEventDestroy(rep->ev_updates_done);
+    (void)hipStreamDestroy(rep->update_stream);
   }
   for (void* p : rep->owned) (void)hipFree(p);
   rep->model->live_replicas--;

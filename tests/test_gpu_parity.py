@@ -1625,6 +1625,57 @@ def test_bf16_dense_path_matches_bf16_rounded_oracle(S, ctx, dims, batch):
     yb.free()
 
 
+@pytest.mark.parametrize("alg", ["adam", "amsgrad", "sgd_momentum"])
+def test_bf16_layerwise_updates_equal_one_update_of_the_flat_buffer(S, ctx, alg):
+    """A training step of a model of bf16 Dense layers updates each layer as soon as its gradients are complete, on a second
+    stream beside the products of the layers below.  Five such steps must leave weights and optimizer state bit for bit
+    where five (gradient pass, then one optimizer launch over the whole flat buffer) steps leave them."""
+    import ctypes as C
+    from scanet3_amd import _lib as L
+    from scanet3_amd._lib import check, lib
+    dims, batch = (64, 256, 136, 104, 24), 128
+    make = {"adam": lambda: S.Adam(0.01), "amsgrad": lambda: S.AMSGrad(0.01), "sgd_momentum": lambda: S.SGD(0.05, momentum=0.9)}[alg]
+    layers = S.Dense(dims[1], S.ReLU()) >> S.Dense(dims[2], S.Tanh) >> S.Dense(dims[3], S.ReLU()) >> S.Dense(dims[4], S.Softmax)
+    cm = S.CompiledModel(ctx, [l.desc() for l in layers.layers], S.CategoricalCrossentropy.kind, (dims[0],), batch, L.FLAG_GEMM_BF16)
+    rng = np.random.default_rng(20251125 + 77)
+    values = {p: (rng.standard_normal(shape) * 0.1).astype(f32) for p, shape, _ in cm.params}
+    stepped, manual = cm.replica(make()), cm.replica(make())
+    desc = make()
+    for r in (stepped, manual):
+        r.set_params(values)
+    n_states = len(S.STATE_NAMES[desc.kind])
+    xs = [ctx.to_device(rng.standard_normal((batch, dims[0])).astype(f32)) for _ in range(2)]
+    ys = [ctx.to_device(one_hot(rng, batch, dims[-1])) for _ in range(2)]
+    w, n = manual.flat(-2)
+    g, _ = manual.flat(-1)
+    st = [manual.flat(slot)[0] for slot in range(n_states)] + [None] * (3 - n_states)
+    ctx.profile_reset()
+    ctx.profile(True)
+    for it in range(1, 6):
+        stepped.step(xs[it % 2], ys[it % 2], it)
+    ctx.sync()
+    ctx.profile(False)
+    launches = {k: v[1] for k, v in ctx.profile_report().items() if k.startswith("optimizer_")}
+    assert sum(launches.values()) >= 5 * 4, launches          # one launch per layer and step, not one per step
+    for it in range(1, 6):
+        manual.grad(xs[it % 2], ys[it % 2])
+        check(lib.sn_optimizer_update(ctx.handle, C.byref(desc), w, g, st[0], st[1], st[2], n, it))
+        manual.set_params(manual.get_params())                # (the bf16 copies of the weights follow the fp32 ones)
+    a, b = stepped.get_params(), manual.get_params()
+    for p in a:
+        np.testing.assert_array_equal(a[p], b[p], err_msg=p)
+    for slot in range(n_states):
+        sa, sb = stepped.get_opt_state(slot), manual.get_opt_state(slot)
+        for p in sa:
+            np.testing.assert_array_equal(sa[p], sb[p], err_msg=f"{p} state {slot}")
+    assert any(np.any(a[p] != values[p]) for p in a)
+    for r in (stepped, manual):
+        r.close()
+    cm.close()
+    for buf in xs + ys:
+        buf.free()
+
+
 def test_bf16_hidden_relu_with_threshold_masks_in_float32(S, ctx):
     """Hidden bf16 Dense layers under ReLU(0.1): clamped outputs equal the threshold exactly and bf16 rounds 0.1 upwards
     (0.10009765625), so a mask read off a bf16 copy of the output would let every clamped unit pass its gradient.  The
