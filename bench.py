@@ -208,13 +208,14 @@ def run_model_workload(S, ctx, name, layers, loss, in_shape, batch, alg, make_xy
             "flops_per_step": step_flops}
 
 
-def dominant_gemm_roofline(kernels, peak_tflops):
+def dominant_gemm_roofline(kernels, peak_tflops, shared=()):
     """Roofline entry for the matrix-core kernel that takes the most time: ALGORITHMIC flops of one launch (model_work)
-    divided by the launch's average duration (HIP events on the library's stream)."""
+    divided by the launch's average duration (HIP events on the library's stream).  `shared`: label prefixes of launches
+    that run beside another stream's kernels (their event times include that sharing): left out of the choice."""
     best = None
     for name, k in kernels.items():
         fl = k.get("flops_per_launch")
-        if fl is None:
+        if fl is None or any(name.startswith(p) for p in shared):
             continue
         if best is None or k["total_ms"] > best[1]["total_ms"]:
             best = (name, k, fl)
@@ -586,7 +587,7 @@ def main():
         line.update({"value": main_res["samples_per_s"], "ms_per_step": main_res["ms_per_step"],
                      "dtype": "bf16" if args.workload == "wide_mlp" else "f32",
                      "config": {"workload": main_res["workload"], "batch": main_res["batch"], "params": main_res["params"]},
-                     "roofline": dominant_gemm_roofline(main_res["kernels"], peak),
+                     "roofline": dominant_gemm_roofline(main_res["kernels"], peak, ("gemm_bf16_256x256[",) if args.workload == "wide_mlp" else ()),
                      "roofline_whole_step": whole_step_roofline(main_res, peak),
                      "host_fed": main_res["host_fed"],
                      "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
@@ -610,7 +611,8 @@ def main():
                 peak = PEAK_BF16_MFMA if which == "wide_mlp" else PEAK_FP32_MFMA
                 extras[which] = {"workload": r["workload"], "samples_per_s": r["samples_per_s"], "ms_per_step": r["ms_per_step"],
                                  "steps": r["steps"], "loss_after": r["loss_after"], "host_fed": r["host_fed"],
-                                 "roofline": dominant_gemm_roofline(r["kernels"], peak),
+                                 # (the bf16 MLP's weight-gradient products share the chip with the optimizer launches of the layers above)
+                                 "roofline": dominant_gemm_roofline(r["kernels"], peak, ("gemm_bf16_256x256[",) if which == "wide_mlp" else ()),
                                  "roofline_whole_step": whole_step_roofline(r, peak),
                                  "kernels_us_per_step": {k: round(v["per_step_us"], 2) for k, v in
                                                          sorted(r["kernels"].items(), key=lambda kv: -kv[1]["total_ms"])[:8]}}
