@@ -7,8 +7,8 @@
 //   forward:        src = x,  (sy, sx) = strides, (oy, ox) = -padding, (ty, tx) = (+1, +1), B = the filter as [K][N]
 //   input gradient: src = dy, unit strides, (oy, ox) = +padding, (ty, tx) = (-1, -1), B(k, n) = w[tap, n, channel]
 //
-// Workgroup = 4 wavefronts, each owning one 32 x 32 accumulator tile (v_mfma_f32_32x32x2_f32); block tile 64 x 64
-// (2 x 2 wavefronts) or 128 x 32 (4 x 1).  A stage is 32 k-values: every tile row is 128 bytes = eight 16-byte
+// Workgroup = 4 wavefronts, each owning one 32 x 32 accumulator tile (v_mfma_f32_32x32x2_f32): block tile 64 x 64
+// (2 x 2 wavefronts), or 64 x 32 with two wavefronts per tile that split every stage's k-values.  A stage is 32 k-values: every tile row is 128 bytes = eight 16-byte
 // chunks, stored at chunk position (chunk ^ (row & 7)) so that the 16-byte fragment reads are conflict free.  Lanes
 // with l/32 = 0 read chunks 0, 2, 4, 6 and lanes with l/32 = 1 chunks 1, 3, 5, 7: MFMA t of chunk pair j multiplies
 // k = 8j + t and k = 8j + 4 + t, one 16-byte LDS read per operand for four MFMAs.  An operand that is not
@@ -80,9 +80,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 // WAVES_M x WAVES_N wavefronts of one 32 x 32 tile each.  B_KC: B is K-contiguous in memory.  ACT: the epilogue's
 // activation, a compile-time constant so that the kernel carries one store sequence only.
-template <int WAVES_M, int WAVES_N, bool B_KC, int ACT>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingArgs a) {
-  constexpr int NW = WAVES_M * WAVES_N, BM = 32 * WAVES_M, BN = 32 * WAVES_N;
+// WAVES_K = 2: two wavefronts per tile, each multiplying one half of every stage's 32 k-values (chunk pairs 0-1 and
+// 2-3); the second hands its sums over through LDS at the end.  Twice the wavefronts per SIMD for the same matrix work:
+// a wavefront's chain per stage (wait, barrier, fragment reads, MFMAs) gets shorter against the matrix cores' time.
+template <int WAVES_M, int WAVES_N, bool B_KC, int ACT, int WAVES_K = 1>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void conv_ring_kernel(RingArgs a) {
+  constexpr int NT = WAVES_M * WAVES_N, NW = NT * WAVES_K, BM = 32 * WAVES_M, BN = 32 * WAVES_N, NJ = 4 / WAVES_K;
+  static_assert(WAVES_K == 1 || WAVES_K == 2, "one or two wavefronts per tile");
   constexpr int A_STAGE = BM * 128;                                  // bytes
   constexpr int B_STAGE = B_KC ? BN * 128 : (RK / 4) * BO_BLOCK;
   constexpr int A_ISSUES = BM / 8 / NW;                              // 1 KiB loads per wavefront and stage
@@ -182,7 +186,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingA
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 
-  const int wm = (wave / WAVES_N) * 32, wn = (wave % WAVES_N) * 32;  // (the barrier below is a no-op cost for one wavefront)
+  const int kgrp = wave / NT, wtile = wave - kgrp * NT;
+  const int wm = (wtile / WAVES_N) * 32, wn = (wtile % WAVES_N) * 32;  // (the barrier below is a no-op cost for one wavefront)
   const int arow = wm + l32, brow = wn + l32;
   const int aoff = arow * 128, asw = arow & 7;
   const int boff = brow * 128, bsw = brow & 7;
@@ -190,11 +195,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingA
   // LDS byte addresses of this lane's fragments inside a stage (the chunk swizzle folded in)
   typedef __attribute__((address_space(3))) char lds_char;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_char*)smem;
-  uint32_t a_at[4], b_at[4];
+  uint32_t a_at[NJ], b_at[NJ];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    a_at[j] = lds0 + (uint32_t)(aoff + (((2 * j + lhi) ^ asw) << 4));
-    b_at[j] = lds0 + (uint32_t)(STAGES * A_STAGE) + (B_KC ? (uint32_t)(boff + (((2 * j + lhi) ^ bsw) << 4)) : (uint32_t)((2 * j + lhi) * BO_BLOCK + brow * 4));
+  for (int jj = 0; jj < NJ; ++jj) {
+    const int j = kgrp * NJ + jj;
+    a_at[jj] = lds0 + (uint32_t)(aoff + (((2 * j + lhi) ^ asw) << 4));
+    b_at[jj] = lds0 + (uint32_t)(STAGES * A_STAGE) + (B_KC ? (uint32_t)(boff + (((2 * j + lhi) ^ bsw) << 4)) : (uint32_t)((2 * j + lhi) * BO_BLOCK + brow * 4));
   }
 
   // Two buffers, one barrier per stage.  The barrier at the top of stage s says two things: everybody's loads of stage s
@@ -208,15 +214,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingA
     __builtin_amdgcn_s_barrier();
     if (s + 1 < nk) issue_next((s + 1) & 1);
     const uint32_t oa = (uint32_t)((s & 1) * A_STAGE), ob = (uint32_t)((s & 1) * B_STAGE);
-    f4v af[4], bf[4];
+    f4v af[NJ], bf[NJ];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) asm volatile("ds_read_b128 %0, %1" : "=v"(af[j]) : "v"(a_at[j] + oa));
+    for (int j = 0; j < NJ; ++j) asm volatile("ds_read_b128 %0, %1" : "=v"(af[j]) : "v"(a_at[j] + oa));
     if constexpr (B_KC) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) asm volatile("ds_read_b128 %0, %1" : "=v"(bf[j]) : "v"(b_at[j] + ob));
+      for (int j = 0; j < NJ; ++j) asm volatile("ds_read_b128 %0, %1" : "=v"(bf[j]) : "v"(b_at[j] + ob));
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         float b0, b1, b2, b3;
         asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %4 offset:256\n\tds_read_b32 %2, %4 offset:512\n\tds_read_b32 %3, %4 offset:768"
                      : "=&v"(b0), "=&v"(b1), "=&v"(b2), "=&v"(b3)
@@ -224,12 +230,31 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingA
         bf[j] = f4v{b0, b1, b2, b3};
       }
     }
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(af[0]), "+v"(af[1]), "+v"(af[2]), "+v"(af[3]), "+v"(bf[0]), "+v"(bf[1]), "+v"(bf[2]), "+v"(bf[3]));
+    if constexpr (NJ == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(af[0]), "+v"(af[1]), "+v"(af[2]), "+v"(af[3]), "+v"(bf[0]), "+v"(bf[1]), "+v"(bf[2]), "+v"(bf[3]));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[0]), "+v"(af[1]), "+v"(bf[0]), "+v"(bf[1]));
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[j][t], bf[j][t], acc, 0, 0, 0);
+  }
+
+  if constexpr (WAVES_K == 2) {
+    // every wavefront has read its last fragments and no load is in flight: the stage buffers carry the hand-over,
+    // value v of lane l of tile t at float (t * 16 + v) * 64 + l
+    static_assert(NT * 16 * 64 * 4 <= STAGES * A_STAGE, "the hand-over fits the A stages");
+    __builtin_amdgcn_s_barrier();
+    float* ex = reinterpret_cast<float*>(smem) + wtile * 1024 + lane;
+    if (kgrp == 1) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) ex[v * 64] = acc[v];
+    }
+    __syncthreads();
+    if (kgrp == 1) return;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] += ex[v * 64];
   }
 
   const int col = n0 + wn + l32;
@@ -238,7 +263,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void conv_ring_kernel(RingA
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int WAVES_M, int WAVES_N, bool B_KC, int ACT>
+template <int WAVES_M, int WAVES_N, bool B_KC, int ACT, int WAVES_K = 1>
 int launch_ring_act(sn_ctx* ctx, const char* name, RingArgs& a, int K) {
   constexpr int BM = 32 * WAVES_M, BN = 32 * WAVES_N;
   a.tiles_m = (int)ceil_div(a.M, BM);
@@ -246,8 +271,8 @@ int launch_ring_act(sn_ctx* ctx, const char* name, RingArgs& a, int K) {
   const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
   const size_t smem = (size_t)STAGES * (BM * 128 + (B_KC ? BN * 128 : (RK / 4) * BO_BLOCK));
   LaunchScope scope(ctx, name, a.M, a.N, K);
-  hipLaunchKernelGGL((conv_ring_kernel<WAVES_M, WAVES_N, B_KC, ACT>), dim3((unsigned)(8 * ceil_div(tiles, 8))), dim3(64 * WAVES_M * WAVES_N), smem,
-                     ctx->stream, a);
+  hipLaunchKernelGGL((conv_ring_kernel<WAVES_M, WAVES_N, B_KC, ACT, WAVES_K>), dim3((unsigned)(8 * ceil_div(tiles, 8))),
+                     dim3(64 * WAVES_M * WAVES_N * WAVES_K), smem, ctx->stream, a);
   SN_HIP(hipGetLastError());
   return SN_OK;
 }
@@ -309,7 +334,10 @@ int launch_conv_ring_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, cons
   const int K = g.kh * g.kw * g.cout;
   // (two-wavefront workgroups, 32 x 64 and 64 x 32, were measured on LeNet's second convolution: forward 35 us against 31,
   // input gradient the same 30 us)
-  if (g.cin <= 32) return launch_ring<4, 1, true>(ctx, "conv2d_input_gradient", a, K);
+  // 32 columns: 64 x 32 tiles, two wavefronts per 32 x 32 tile (the input gradient has no activation).  On LeNet's
+  // second convolution 29.1 us against 30.2 for 128 x 32 tiles of one wavefront each (128 x 32 with two: 29.4); the same
+  // split of the forward product's 64 x 64 tiles changed its sums enough to matter to a 100-step trajectory and is not used.
+  if (g.cin <= 32) return launch_ring_act<2, 1, true, SN_ACT_IDENTITY, 2>(ctx, "conv2d_input_gradient", a, K);
   return launch_ring<2, 2, true>(ctx, "conv2d_input_gradient", a, K);
 }
 
