@@ -493,6 +493,13 @@ MODELS = {
                                              ("flatten",), ("dense", 3, "softmax")], "cce", (17, 12, 1), 256, "uniform_onehot"),
     "conv_tap_rows_3x1_64_filters": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 64, (3, 1), (1, 1), "valid", "identity", False),
                                       ("flatten",), ("dense", 3, "softmax")], "cce", (12, 9, 1), 160, "uniform_onehot"),
+    # input gradient of a layer with fewer than 32 input channels and 'same' padding through the kernel that feeds the matrix
+    # cores from LDS-direct loads (two wavefronts per tile): 16 of a tile's 32 columns exist, taps leave the image on all
+    # four sides, the last row tile is partial; and 32 input channels with a 2 x 3 kernel
+    "conv_input_gradient_16_channels_same": ([("conv", 16, (3, 3), (1, 1), "valid", "tanh", False), ("conv", 32, (3, 3), (1, 1), "same", "relu", True),
+                                              ("flatten",), ("dense", 3, "softmax")], "cce", (9, 13, 1), 11, "uniform_onehot"),
+    "conv_input_gradient_32_channels_2x3_same": ([("conv", 32, (3, 3), (1, 1), "valid", "relu", False), ("conv", 32, (2, 3), (1, 1), "same", "tanh", False),
+                                                  ("flatten",), ("dense", 3, "softmax")], "cce", (8, 9, 1), 13, "uniform_onehot"),
     # Dense from thousands of features onto a few units: gradients as row streams (2048+ features, at most 16 units); a feature count
     # that leaves a partial block of 64, 7 rows over 4 wavefronts, 16 and 5 units, an L2 penalty on the streamed weights
     "dense_many_features_few_units": ([("dense", 2050, "tanh"), ("dense", 5, "softmax", "l2", 0.01)], "cce", (33,), 7, "normal_onehot"),
@@ -570,6 +577,8 @@ KERNEL_OF_MODEL = {
     "conv_taps_3x3_64_filters_odd_rows": "conv2d_filter_gradient_taps",
     "conv_taps_2x3_32_filters_stride_bias": "conv2d_filter_gradient_taps",
     "conv_taps_row_stride_2": "conv2d_filter_gradient_taps",
+    "conv_input_gradient_16_channels_same": "conv2d_input_gradient[",
+    "conv_input_gradient_32_channels_2x3_same": "conv2d_input_gradient[",
     "conv_pool_first_layer_same_s1": "maxpool_backward_and_conv2d_filter_gradient_direct",
     "conv_first_layer_uneven": "conv2d_filter_gradient_direct",
     "dense_many_features_few_units": "dense_weight_and_input_gradient_rows",
