@@ -304,8 +304,8 @@ MEASURED_TRAFFIC = {
     # kernel label (or optimizer name): (bytes per launch, source file, sha1 of the file when measured)
     # rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (one run each), KiB per dispatch, scaled by what the same counters read
     # for a plain copy of 400 MB (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); the summaries are under profiles/
-    "conv2d_forward[52900x64x288]": (22.3e6, "conv_ring_kernels.hip", "89a44a72111a780757a3ddc6a90991162ce40a45"),
-    "conv2d_input_gradient[62500x32x576]": (22.3e6, "conv_ring_kernels.hip", "89a44a72111a780757a3ddc6a90991162ce40a45"),
+    "conv2d_forward[52900x64x288]": (22.3e6, "conv_ring_kernels.hip", "9ad35c60088e844b2f3f3f3c28cbad9fe520c83f"),
+    "conv2d_input_gradient[62500x32x576]": (22.3e6, "conv_ring_kernels.hip", "9ad35c60088e844b2f3f3f3c28cbad9fe520c83f"),
     "conv2d_filter_gradient_tap_rows[288x64x52900]": (28.2e6, "conv_wgrad_kernels.hip", "86fd829667595ab42abdb3131518e7142ff50eba"),
     "gemm_bf16_256x256_bf16out[8192x4096x4096]": (474.8e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
     "gemm_bf16_256x256[4096x4096x8192]": (494.7e6, "gemm_bf16.hip", "a403cf021cd20e0154725176d99f33018b440f94"),
@@ -317,8 +317,8 @@ MEASURED_TRAFFIC = {
     "lstm_sequence_backward_and_weight_gradient[512x1024x34560]": (520.3e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
     "rnn_sequence_forward[32768x256x288]": (74.8e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
     "rnn_sequence_backward_and_weight_gradient[512x256x34560]": (116.8e6, "lstm_kernels.hip", "6d2dbe90ac02733993f507dc6304b11f1f3acfbd"),
-    "conv2d_forward[121000x64x288]": (53.3e6, "conv_ring_kernels.hip", "89a44a72111a780757a3ddc6a90991162ce40a45"),
-    "conv2d_input_gradient[169000x32x576]": (53.3e6, "conv_ring_kernels.hip", "89a44a72111a780757a3ddc6a90991162ce40a45"),
+    "conv2d_forward[121000x64x288]": (53.3e6, "conv_ring_kernels.hip", "9ad35c60088e844b2f3f3f3c28cbad9fe520c83f"),
+    "conv2d_input_gradient[169000x32x576]": (53.3e6, "conv_ring_kernels.hip", "9ad35c60088e844b2f3f3f3c28cbad9fe520c83f"),
     "conv2d_filter_gradient_tap_rows[288x64x121000]": (60.9e6, "conv_wgrad_kernels.hip", "86fd829667595ab42abdb3131518e7142ff50eba"),
     "mlp2_rows_forward_backward[1000x50x784]": (5.4e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),
     "mlp2_weight_gradients_and_optimizer[784x50x1000]": (9.8e6, "mlp2_kernels.hip", "ebb1ef9fa9d2339b26bc579ca878dfb04138a92b"),

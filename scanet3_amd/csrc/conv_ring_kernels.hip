@@ -336,7 +336,7 @@ int launch_conv_ring_dgrad(sn_ctx* ctx, const ConvGeom& g, const float* dy, cons
   // input gradient the same 30 us)
   // 32 columns: 64 x 32 tiles, two wavefronts per 32 x 32 tile (the input gradient has no activation).  On LeNet's
   // second convolution 29.1 us against 30.2 for 128 x 32 tiles of one wavefront each (128 x 32 with two: 29.4); the same
-  // split of the forward product's 64 x 64 tiles changed its sums enough to matter to a 100-step trajectory and is not used.
+  // split of the forward product's 64 x 64 tiles gained nothing there (30.2 us either way) and is not used.
   if (g.cin <= 32) return launch_ring_act<2, 1, true, SN_ACT_IDENTITY, 2>(ctx, "conv2d_input_gradient", a, K);
   return launch_ring<2, 2, true>(ctx, "conv2d_input_gradient", a, K);
 }
